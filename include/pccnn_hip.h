@@ -1,0 +1,197 @@
+/*
+ * pccnn_hip.h -- C ABI of libpccnn_hip.so: the point-cloud operator path of
+ * pccnn_lib (cell keys, key sort, pillar grid, radius neighbor search, Gaussian
+ * KDE, Poisson-disk selection, KPConv / MCConv forward and backward) as
+ * hand-written HIP kernels for gfx950 (MI355X, CDNA4, wave64).
+ *
+ * Conventions
+ *  - Every pointer is a DEVICE pointer unless its name starts with `h_`.
+ *  - Tensors are dense, row-major, of exactly the stated element type.
+ *  - `stream` is a hipStream_t passed as void* (NULL = the null stream).  All
+ *    work is enqueued on it; no entry point synchronises or allocates device
+ *    memory.  Temporary storage comes in through `workspace` arguments whose
+ *    minimum size the matching *_workspace_bytes function reports.
+ *  - Return value: 0 on success, a negative PCCNN_ERR_* code otherwise;
+ *    pccnn_last_error() then returns a thread-local description.  Arguments
+ *    are validated on the host before any kernel is launched.
+ *  - D (point dimensionality) is 3 in this build; other values return
+ *    PCCNN_ERR_UNSUPPORTED.
+ *
+ * Each entry point cites the reference interface it replaces (paths relative
+ * to the reference repository; *.cuh lines are the host-function prototypes
+ * that pccnn_lib_ops/ops_list.cpp:26-54 exports to Python).
+ */
+#ifndef PCCNN_HIP_H
+#define PCCNN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PCCNN_OK 0
+#define PCCNN_ERR_INVALID (-1)     /* null pointer, negative size, inconsistent shapes */
+#define PCCNN_ERR_UNSUPPORTED (-2) /* valid request this build has no kernel for */
+#define PCCNN_ERR_WORKSPACE (-3)   /* workspace missing or too small */
+#define PCCNN_ERR_HIP (-4)         /* a HIP runtime call or kernel launch failed */
+
+const char *pccnn_last_error(void);
+int pccnn_version(void);
+
+/* ---- bounding box -------------------------------------------------------
+ * Replaces pccnn_lib/pc/BoundingBox.py:17-18 (torch_scatter scatter_min /
+ * scatter_max followed by -1e-6 / +1e-6 in fp32).
+ * pts f32[n,d], batch_ids i32[n] in [0,batch_size) -> aabb_min/max f32[batch_size,d]. */
+int pccnn_bounding_box(const float *pts, const int32_t *batch_ids, int64_t n, int d, int batch_size,
+                       float *aabb_min_out, float *aabb_max_out, void *stream);
+
+/* ---- cell keys ----------------------------------------------------------
+ * Replaces compute_keys (pccnn_lib_ops/compute_keys/compute_keys.cuh:26-31,
+ * compute_keys.cu:78-127).  num_cells i32[d] and cell_size f32[d] live on the
+ * device like the tensors the reference receives.  keys_out i64[n]. */
+int pccnn_compute_keys(const float *pts, const int32_t *batch_ids, const float *aabb_min,
+                       const int32_t *num_cells, const float *cell_size, int64_t n, int d,
+                       int64_t *keys_out, void *stream);
+
+/* ---- key sort -----------------------------------------------------------
+ * Replaces torch.argsort(cell_ids) and the index_select gathers that follow it
+ * (pccnn_lib/pc/Grid.py:52,68-70; pccnn_lib/pc/Neighborhood.py:27-32).
+ * Stable LSD radix sort of the low `key_bits` bits of non-negative 64-bit keys
+ * (key_bits <= 0 means 64).  Outputs: sorted_keys_out i64[n], perm_out i32[n]
+ * (perm_out[i] = original index of the i-th smallest key, ties in original
+ * order) and, when pts != NULL, sorted_pts_out f32[n,d] = pts[perm_out]. */
+size_t pccnn_sort_keys_workspace_bytes(int64_t n);
+int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int64_t *sorted_keys_out, int32_t *perm_out,
+                    const float *pts, int d, float *sorted_pts_out,
+                    void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- pillar grid --------------------------------------------------------
+ * Replaces build_grid_ds (pccnn_lib_ops/build_grid/build_grid_ds.cuh:25-28,
+ * build_grid_ds.cu:72-114).  sorted_keys i64[n] ascending; grid_ds_out
+ * i32[num_pillars,2] with num_pillars = batch_size*num_cells[0]*num_cells[1];
+ * (first, last+1) of each pillar's run, (0,0) for empty pillars. */
+int pccnn_build_grid_ds(const int64_t *sorted_keys, int64_t n, const int32_t *num_cells, int d,
+                        int64_t num_pillars, int32_t *grid_ds_out, void *stream);
+
+/* ---- radius neighbor search --------------------------------------------
+ * Replaces find_neighbors (pccnn_lib_ops/find_neighbors/find_neighbors.cuh:33-41,
+ * find_neighbors.cu:27-66) as two calls around the one size the host must learn:
+ *
+ *   pccnn_find_neighbors_count  -> ends_out i32[m]: inclusive running total of
+ *       min(count, max_neighbors or inf) per sample (the `start ids` tensor the
+ *       reference returns);  the caller copies ends_out[m-1] (= T) to the host,
+ *       allocates neigh i32[T,2], then calls
+ *   pccnn_find_neighbors_fill   -> neigh_out[t] = (point, sample).
+ *
+ * pts_sorted f32[n,d] / pt_keys_sorted i64[n]: points in key order;
+ * samples f32[m,d] / sample_keys i64[m]: queries in any order, keyed on the
+ * points' grid; grid_ds i32[num_pillars,2] from pccnn_build_grid_ds; radii f32[d] (device).
+ * sample_order i32[m] (nullable): a permutation that lists the samples in
+ * ascending key order -- tiles of consecutive entries then share their cell
+ * walk; NULL means natural order.  max_neighbors 0 = unlimited; otherwise a
+ * sample with more hits keeps max_neighbors of them, evenly spaced in its hit
+ * order (the reference keeps a time-seeded random subset there).
+ * point_remap i32[n] (nullable): when given, column 0 of neigh_out is
+ * point_remap[sorted index] (fuses pccnn_lib/pc/Neighborhood.py:47-53), else the
+ * sorted index as in the reference op.  Pairs are grouped by ascending sample
+ * index; inside a sample they are in ascending sorted-point order.
+ * Both calls take the same workspace (count leaves per-sample raw counts in it). */
+size_t pccnn_find_neighbors_workspace_bytes(int64_t m);
+int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t *pt_keys_sorted, int64_t n,
+                               const float *samples, const int64_t *sample_keys, int64_t m,
+                               const int32_t *sample_order, const int32_t *grid_ds, int64_t num_pillars,
+                               const int32_t *num_cells, const float *radii, int d, int max_neighbors,
+                               int32_t *ends_out,
+                               void *workspace, size_t workspace_bytes, void *stream);
+int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t *pt_keys_sorted, int64_t n,
+                              const float *samples, const int64_t *sample_keys, int64_t m,
+                              const int32_t *sample_order, const int32_t *grid_ds, int64_t num_pillars,
+                              const int32_t *num_cells, const float *radii, int d, int max_neighbors,
+                              const int32_t *ends,
+                              const int32_t *point_remap, int64_t t, int32_t *neigh_out,
+                              void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- Gaussian KDE -------------------------------------------------------
+ * Replaces compute_pdf / compute_pdf_grads (pccnn_lib_ops/compute_pdf/compute_pdf.cuh:28-51,
+ * compute_pdf.cu:153-257).  neigh i32[t,2] = (point, sample) in original point
+ * ids, ends i32[n]; samples are the points themselves.  pdf_out f32[n];
+ * pt_grads_out f32[n,d]. */
+int pccnn_compute_pdf(int manifold_dims, const float *bandwidth, const float *pts, int64_t n, int d,
+                      const int32_t *neigh, int64_t t, const int32_t *ends, float *pdf_out, void *stream);
+int pccnn_compute_pdf_grads(int manifold_dims, const float *bandwidth, const float *pts, int64_t n, int d,
+                            const int32_t *neigh, int64_t t, const int32_t *ends, const float *in_grads,
+                            float *pt_grads_out, void *stream);
+
+/* ---- Poisson-disk selection --------------------------------------------
+ * Replaces poisson_disk_sampling (pccnn_lib_ops/poisson_disk_sampling/poisson_disk_sampling.cuh:28-32,
+ * poisson_disk_sampling.cu:110-196).  Inputs are in sorted-index space.
+ * pccnn_poisson_disk_select writes selected_out i32[n] (0/1) and
+ * selected_scan_out i32[n] (inclusive running count; last entry = S);
+ * pccnn_compact_selected then writes the S selected indices, ascending, as i64. */
+size_t pccnn_poisson_disk_workspace_bytes(int64_t n);
+int pccnn_poisson_disk_select(const int64_t *sorted_keys, int64_t n, const int32_t *neigh, int64_t t,
+                              const int32_t *ends, const int32_t *num_cells, int d,
+                              int32_t *selected_out, int32_t *selected_scan_out,
+                              void *workspace, size_t workspace_bytes, void *stream);
+int pccnn_compact_selected(const int32_t *selected, const int32_t *selected_scan, int64_t n,
+                           int64_t *ids_out, void *stream);
+
+/* ---- convolutions -------------------------------------------------------
+ * Shapes: pts f32[n,d], feats f32[n,c_in], samples f32[m,d], neigh i32[t,2]
+ * (point, sample), ends i32[m], radii f32[d] (device), out f32[m,c_out].
+ *
+ * KPConv replaces kp_conv / kp_conv_grads (pccnn_lib_ops/pcconvs/kpconv.cuh:32-67,
+ * kpconv.cu:32-112): kernel_pts f32[k,d], weights f32[k*c_in, c_out] with row
+ * f*k + kk.  Backward outputs: d_weights f32[k*c_in,c_out], d_feats f32[n,c_in],
+ * d_kernel_pts f32[k,d], d_pts f32[n,d], d_samples f32[m,d].
+ *
+ * MCConv replaces mc_conv / mc_conv_grads (pccnn_lib_ops/pcconvs/mcconv.cuh:32-69,
+ * mcconv.cu:32-143): pdf f32[n], axis f32[d,k], bias f32[k] with k = hidden*num_mlps,
+ * weights f32[num_mlps, k*c_in/num_mlps, c_out/num_mlps].  Backward outputs:
+ * d_weights (same shape), d_feats, d_axis f32[d,k], d_bias f32[k], d_pdf f32[n],
+ * d_pts, d_samples.
+ *
+ * 1 <= k <= 64.  Backward outputs are fully overwritten. */
+size_t pccnn_conv_workspace_bytes(int64_t m, int64_t t, int c_in, int k, int c_out, int backward);
+int pccnn_kpconv_forward(const float *pts, const float *feats, const float *samples, const int32_t *neigh,
+                         const int32_t *ends, const float *radii, const float *kernel_pts, float sigma,
+                         const float *weights, int64_t n, int64_t m, int64_t t, int d, int c_in, int k, int c_out,
+                         float *out, void *workspace, size_t workspace_bytes, void *stream);
+int pccnn_kpconv_backward(const float *pts, const float *feats, const float *samples, const int32_t *neigh,
+                          const int32_t *ends, const float *radii, const float *kernel_pts, float sigma,
+                          const float *weights, const float *in_grads,
+                          int64_t n, int64_t m, int64_t t, int d, int c_in, int k, int c_out,
+                          float *d_weights, float *d_feats, float *d_kernel_pts, float *d_pts, float *d_samples,
+                          void *workspace, size_t workspace_bytes, void *stream);
+int pccnn_mcconv_forward(const float *pts, const float *pdf, const float *feats, const float *samples,
+                         const int32_t *neigh, const int32_t *ends, const float *radii, const float *axis,
+                         const float *bias, const float *weights,
+                         int64_t n, int64_t m, int64_t t, int d, int c_in, int k, int num_mlps, int c_out,
+                         float *out, void *workspace, size_t workspace_bytes, void *stream);
+int pccnn_mcconv_backward(const float *pts, const float *pdf, const float *feats, const float *samples,
+                          const int32_t *neigh, const int32_t *ends, const float *radii, const float *axis,
+                          const float *bias, const float *weights, const float *in_grads,
+                          int64_t n, int64_t m, int64_t t, int d, int c_in, int k, int num_mlps, int c_out,
+                          float *d_weights, float *d_feats, float *d_axis, float *d_bias, float *d_pdf,
+                          float *d_pts, float *d_samples,
+                          void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- dense contraction --------------------------------------------------
+ * The fp32 MFMA GEMM the convolutions use for the [M, K*Cin] x [K*Cin, Cout]
+ * contraction (torch::matmul at pccnn_lib_ops/pcconvs/kpconv.cu:56-57,90-96 and
+ * mcconv.cu:64-68,111-120), exposed for tests and benchmarks.
+ * C[batch][rows,cols] = op(A) * op(B) with inner size `inner`; row-major storage,
+ * a_trans: A stored [inner, rows]; b_trans: B stored [cols, inner]; lda/ldb/ldc are
+ * row strides in elements, stride_* batch strides in elements.  split_k > 1
+ * needs workspace of batch*split_k*rows*cols floats. */
+int pccnn_gemm_f32(const float *a, const float *b, float *c, int64_t rows, int64_t cols, int64_t inner,
+                   int a_trans, int b_trans, int64_t lda, int64_t ldb, int64_t ldc,
+                   int batch, int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                   int split_k, void *workspace, size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PCCNN_HIP_H */

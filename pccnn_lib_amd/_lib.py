@@ -1,0 +1,75 @@
+"""ctypes binding of ``libpccnn_hip.so`` (the C ABI declared in include/pccnn_hip.h).
+
+The library is the only compute path of this package: if it is missing, or an entry point
+returns an error, a RuntimeError is raised -- there is no CPU or PyTorch fallback.
+"""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libpccnn_hip.so")
+
+P = ctypes.c_void_p
+I64 = ctypes.c_int64
+I32 = ctypes.c_int
+F32 = ctypes.c_float
+SZ = ctypes.c_size_t
+
+# name -> (restype, argtypes); mirrors include/pccnn_hip.h declaration by declaration.
+SIGNATURES = {
+    "pccnn_last_error": (ctypes.c_char_p, []),
+    "pccnn_version": (I32, []),
+    "pccnn_bounding_box": (I32, [P, P, I64, I32, I32, P, P, P]),
+    "pccnn_compute_keys": (I32, [P, P, P, P, P, I64, I32, P, P]),
+    "pccnn_sort_keys_workspace_bytes": (SZ, [I64]),
+    "pccnn_sort_keys": (I32, [P, I64, I32, P, P, P, I32, P, P, SZ, P]),
+    "pccnn_build_grid_ds": (I32, [P, I64, P, I32, I64, P, P]),
+    "pccnn_find_neighbors_workspace_bytes": (SZ, [I64]),
+    "pccnn_find_neighbors_count": (I32, [P, P, I64, P, P, I64, P, P, I64, P, P, I32, I32, P, P, SZ, P]),
+    "pccnn_find_neighbors_fill": (I32, [P, P, I64, P, P, I64, P, P, I64, P, P, I32, I32, P, P, I64, P, P, SZ, P]),
+    "pccnn_compute_pdf": (I32, [I32, P, P, I64, I32, P, I64, P, P, P]),
+    "pccnn_compute_pdf_grads": (I32, [I32, P, P, I64, I32, P, I64, P, P, P, P]),
+    "pccnn_poisson_disk_workspace_bytes": (SZ, [I64]),
+    "pccnn_poisson_disk_select": (I32, [P, I64, P, I64, P, P, I32, P, P, P, SZ, P]),
+    "pccnn_compact_selected": (I32, [P, P, I64, P, P]),
+    "pccnn_conv_workspace_bytes": (SZ, [I64, I64, I32, I32, I32, I32]),
+    "pccnn_kpconv_forward": (I32, [P, P, P, P, P, P, P, F32, P, I64, I64, I64, I32, I32, I32, I32, P, P, SZ, P]),
+    "pccnn_kpconv_backward": (I32, [P, P, P, P, P, P, P, F32, P, P, I64, I64, I64, I32, I32, I32, I32,
+                                    P, P, P, P, P, P, SZ, P]),
+    "pccnn_mcconv_forward": (I32, [P, P, P, P, P, P, P, P, P, P, I64, I64, I64, I32, I32, I32, I32, I32,
+                                   P, P, SZ, P]),
+    "pccnn_mcconv_backward": (I32, [P, P, P, P, P, P, P, P, P, P, P, I64, I64, I64, I32, I32, I32, I32, I32,
+                                    P, P, P, P, P, P, P, P, SZ, P]),
+    "pccnn_gemm_f32": (I32, [P, P, P, I64, I64, I64, I32, I32, I64, I64, I64, I32, I64, I64, I64, I32, P, SZ, P]),
+}
+
+_lib = None
+
+
+def load():
+    """Load the shared library once and attach the C signatures."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "pccnn_lib_amd: %s is missing; build it with `python -m pccnn_lib_amd.build` "
+            "(needs hipcc; there is no fallback implementation)" % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc, what):
+    if rc != 0:
+        msg = load().pccnn_last_error()
+        raise RuntimeError("%s failed (%d): %s" % (what, rc, msg.decode() if msg else "?"))
+
+
+def call(name, *args):
+    """Call an int-returning entry point and raise on a non-zero status."""
+    check(getattr(load(), name)(*args), name)

@@ -1,0 +1,91 @@
+// Shared host/device helpers of libpccnn_hip (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/pccnn_hip.h"
+
+#define PCCNN_WAVE 64
+
+void pccnn_set_error(const char *fmt, ...);
+
+#define PCCNN_REQUIRE(cond, code, ...)                                                   \
+    do {                                                                                 \
+        if (!(cond)) {                                                                   \
+            pccnn_set_error(__VA_ARGS__);                                                \
+            return (code);                                                               \
+        }                                                                                \
+    } while (0)
+
+#define PCCNN_HIP_CHECK(expr)                                                            \
+    do {                                                                                 \
+        hipError_t err__ = (expr);                                                       \
+        if (err__ != hipSuccess) {                                                       \
+            pccnn_set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(err__), __FILE__, __LINE__); \
+            return PCCNN_ERR_HIP;                                                        \
+        }                                                                                \
+    } while (0)
+
+#define PCCNN_LAUNCH_CHECK() PCCNN_HIP_CHECK(hipGetLastError())
+
+static inline int64_t pccnn_ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static inline size_t pccnn_align(size_t x) { return (x + 255) & ~(size_t)255; }
+
+// Carves 256-byte aligned pieces out of a caller-provided workspace.
+struct PccnnArena {
+    char *base;
+    size_t size, used;
+    PccnnArena(void *p, size_t s) : base((char *)p), size(s), used(0) {}
+    template <typename T> T *take(size_t count)
+    {
+        size_t bytes = pccnn_align(count * sizeof(T));
+        if (base == nullptr || used + bytes > size) { used = size + 1; return nullptr; }
+        T *r = (T *)(base + used);
+        used += bytes;
+        return r;
+    }
+    bool ok() const { return used <= size; }
+};
+
+#ifdef __HIPCC__
+__device__ __forceinline__ int pccnn_lane() { return (int)__lane_id(); }
+
+__device__ __forceinline__ unsigned long long pccnn_lanemask_lt()
+{
+    return (1ull << pccnn_lane()) - 1ull;
+}
+
+// Broadcast lane `src` (wave-uniform) of a 32-bit value to the whole wave.
+__device__ __forceinline__ int pccnn_bcast_i(int v, int src)
+{
+    return __builtin_amdgcn_readlane(v, __builtin_amdgcn_readfirstlane(src));
+}
+__device__ __forceinline__ float pccnn_bcast_f(float v, int src)
+{
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), __builtin_amdgcn_readfirstlane(src)));
+}
+__device__ __forceinline__ long long pccnn_bcast_ll(long long v, int src)
+{
+    int lo = pccnn_bcast_i((int)(v & 0xffffffffll), src);
+    int hi = pccnn_bcast_i((int)(v >> 32), src);
+    return ((long long)hi << 32) | (unsigned int)lo;
+}
+
+__device__ __forceinline__ float pccnn_wave_sum(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+#endif
+
+// Device-wide inclusive scan of int32 (scan.hip).  `clamp_max` > 0 clamps each input first.
+// tmp must hold pccnn_scan_tmp_elems(n) ints.
+size_t pccnn_scan_tmp_elems(int64_t n);
+int pccnn_scan_inclusive_i32(const int32_t *in, int32_t *out, int64_t n, int clamp_max, int32_t *tmp,
+                             hipStream_t stream);
+
+// Internal sort entry used by other translation units.
+int pccnn_fill_i32(int32_t *p, int32_t value, int64_t count, hipStream_t stream);
+int pccnn_fill_f32(float *p, float value, int64_t count, hipStream_t stream);

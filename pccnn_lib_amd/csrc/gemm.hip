@@ -1,0 +1,231 @@
+// fp32 GEMM on the CDNA matrix cores (v_mfma_f32_32x32x2_f32), used for the
+// [M, K*Cin] x [K*Cin, Cout] contraction of the convolutions and its two transposes.
+//
+// Workgroup tile 128 x 128, inner step 16, 256 threads = 4 wavefronts in a 2 x 2 arrangement,
+// each wavefront owning a 64 x 64 block as 2 x 2 MFMA tiles (64 accumulator registers).
+// Both operand tiles are staged in LDS k-major ([16][128] plus padding) whatever their layout
+// in memory, so every fragment read is 32 consecutive floats; tiles are double-buffered and the
+// next tile's global loads are issued before the current tile's MFMAs (one barrier per step).
+// Split-K writes partial products to a workspace that a second kernel sums in a fixed order.
+#include "common.h"
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+#define GT_M 128
+#define GT_N 128
+#define GT_K 16
+#define GT_LD 130          // LDS row stride (floats): conflict-free transposing stores, 8-byte aligned rows
+
+struct GemmArgs {
+    const float *a, *b;
+    float *c;
+    int64_t rows, cols, inner;
+    int64_t lda, ldb, ldc;
+    int64_t stride_a, stride_b, stride_c;
+    int split_k;
+    int64_t k_chunk;       // inner elements per split (multiple of GT_K)
+    int aligned;           // pointers, leading dimensions and batch strides allow float4 loads
+};
+
+// Global -> registers for one 128 x 16 operand tile.  `KCONTIG`: the reduction index is the
+// contiguous one in memory (element (x, k) at p[x * ld + k]); otherwise element (x, k) at p[k * ld + x].
+template <bool KCONTIG>
+__device__ __forceinline__ void tile_load(const float *__restrict__ p, int64_t ld, int64_t x0, int64_t x_end,
+                                          int64_t k0, int64_t k_end, bool fast, float4 (&r)[2])
+{
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int idx = threadIdx.x + 256 * i;
+        int64_t x, k;
+        if (KCONTIG) { x = x0 + idx / 4; k = k0 + (idx % 4) * 4; }
+        else { k = k0 + idx / 32; x = x0 + (idx % 32) * 4; }
+        if (fast) {
+            r[i] = KCONTIG ? *(const float4 *)(p + x * ld + k) : *(const float4 *)(p + k * ld + x);
+        } else {
+            float v[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int64_t xx = KCONTIG ? x : x + c;
+                const int64_t kk = KCONTIG ? k + c : k;
+                v[c] = (xx < x_end && kk < k_end) ? (KCONTIG ? p[xx * ld + kk] : p[kk * ld + xx]) : 0.0f;
+            }
+            r[i] = make_float4(v[0], v[1], v[2], v[3]);
+        }
+    }
+}
+
+template <bool KCONTIG>
+__device__ __forceinline__ void tile_store(float (*lds)[GT_LD], const float4 (&r)[2])
+{
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int idx = threadIdx.x + 256 * i;
+        if (KCONTIG) {
+            const int x = idx / 4, k = (idx % 4) * 4;
+            lds[k + 0][x] = r[i].x;
+            lds[k + 1][x] = r[i].y;
+            lds[k + 2][x] = r[i].z;
+            lds[k + 3][x] = r[i].w;
+        } else {
+            const int k = idx / 32, x = (idx % 32) * 4;
+            *(float2 *)&lds[k][x] = make_float2(r[i].x, r[i].y);
+            *(float2 *)&lds[k][x + 2] = make_float2(r[i].z, r[i].w);
+        }
+    }
+}
+
+template <bool AT, bool BT>
+__global__ void __launch_bounds__(256)
+gemm_f32_mfma_kernel(GemmArgs g, float *__restrict__ partial)
+{
+    __shared__ __attribute__((aligned(16))) float As[2][GT_K][GT_LD];
+    __shared__ __attribute__((aligned(16))) float Bs[2][GT_K][GT_LD];
+
+    const int lane = pccnn_lane();
+    const int wave = threadIdx.x >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int batch = blockIdx.z / g.split_k;
+    const int split = blockIdx.z % g.split_k;
+    const int64_t bm = (int64_t)blockIdx.y * GT_M;
+    const int64_t bn = (int64_t)blockIdx.x * GT_N;
+    const float *a = g.a + (int64_t)batch * g.stride_a;
+    const float *b = g.b + (int64_t)batch * g.stride_b;
+    const int64_t k_begin = (int64_t)split * g.k_chunk;
+    const int64_t k_end = (k_begin + g.k_chunk < g.inner) ? k_begin + g.k_chunk : g.inner;
+    const bool fast = g.aligned && (bm + GT_M <= g.rows) && (bn + GT_N <= g.cols) && ((k_end - k_begin) % GT_K == 0);
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    float4 ra[2], rb[2];
+    const int64_t nk = (k_end - k_begin + GT_K - 1) / GT_K;
+    if (nk > 0) {
+        // A stored [rows, inner] (AT = false) has the reduction index contiguous; B stored
+        // [inner, cols] (BT = false) has the column index contiguous.
+        tile_load<!AT>(a, g.lda, bm, g.rows, k_begin, k_end, fast, ra);
+        tile_load<BT>(b, g.ldb, bn, g.cols, k_begin, k_end, fast, rb);
+        tile_store<!AT>(As[0], ra);
+        tile_store<BT>(Bs[0], rb);
+    }
+    __syncthreads();
+    for (int64_t kt = 0; kt < nk; ++kt) {
+        const int buf = (int)(kt & 1);
+        const bool more = kt + 1 < nk;
+        if (more) {
+            const int64_t k0 = k_begin + (kt + 1) * GT_K;
+            tile_load<!AT>(a, g.lda, bm, g.rows, k0, k_end, fast, ra);
+            tile_load<BT>(b, g.ldb, bn, g.cols, k0, k_end, fast, rb);
+        }
+#pragma unroll
+        for (int ks = 0; ks < GT_K / 2; ++ks) {
+            const int kr = 2 * ks + (lane >> 5);
+            const int c = lane & 31;
+            const float a0 = As[buf][kr][wm * 64 + c];
+            const float a1 = As[buf][kr][wm * 64 + 32 + c];
+            const float b0 = Bs[buf][kr][wn * 64 + c];
+            const float b1 = Bs[buf][kr][wn * 64 + 32 + c];
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+        }
+        if (more) {
+            tile_store<!AT>(As[buf ^ 1], ra);
+            tile_store<BT>(Bs[buf ^ 1], rb);
+        }
+        __syncthreads();
+    }
+
+    // Accumulator layout of the 32x32 MFMA: register v of lane l holds
+    // row 8*(v/4) + 4*(l/32) + v%4, column l%32 of the tile.
+    float *cbase;
+    int64_t ldc;
+    if (g.split_k > 1) {
+        cbase = partial + ((int64_t)batch * g.split_k + split) * g.rows * g.cols;
+        ldc = g.cols;
+    } else {
+        cbase = g.c + (int64_t)batch * g.stride_c;
+        ldc = g.ldc;
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int64_t col = bn + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int64_t row = bm + wm * 64 + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                if (row < g.rows && col < g.cols) cbase[row * ldc + col] = acc[i][j][v];
+            }
+        }
+}
+
+__global__ void __launch_bounds__(256)
+splitk_reduce_kernel(const float *__restrict__ partial, GemmArgs g, int batch_count)
+{
+    const int64_t per = g.rows * g.cols;
+    const int64_t total = per * batch_count;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t bi = i / per, e = i % per;
+        const float *src = partial + bi * g.split_k * per + e;
+        float s = 0.0f;
+        for (int k = 0; k < g.split_k; ++k) s += src[(int64_t)k * per];
+        g.c[bi * g.stride_c + (e / g.cols) * g.ldc + (e % g.cols)] = s;
+    }
+}
+
+extern "C" int pccnn_gemm_f32(const float *a, const float *b, float *c, int64_t rows, int64_t cols, int64_t inner,
+                              int a_trans, int b_trans, int64_t lda, int64_t ldb, int64_t ldc, int batch,
+                              int64_t stride_a, int64_t stride_b, int64_t stride_c, int split_k, void *workspace,
+                              size_t workspace_bytes, void *stream)
+{
+    PCCNN_REQUIRE(rows >= 0 && cols >= 0 && inner >= 0 && batch >= 1, PCCNN_ERR_INVALID,
+                  "pccnn_gemm_f32: rows=%lld cols=%lld inner=%lld batch=%d", (long long)rows, (long long)cols,
+                  (long long)inner, batch);
+    if (rows == 0 || cols == 0) return PCCNN_OK;
+    PCCNN_REQUIRE(a && b && c, PCCNN_ERR_INVALID, "pccnn_gemm_f32: null pointer");
+    PCCNN_REQUIRE(lda >= (a_trans ? rows : inner) && ldb >= (b_trans ? inner : cols) && ldc >= cols, PCCNN_ERR_INVALID,
+                  "pccnn_gemm_f32: leading dimension too small (lda=%lld ldb=%lld ldc=%lld)", (long long)lda,
+                  (long long)ldb, (long long)ldc);
+    if (split_k < 1) split_k = 1;
+    GemmArgs g;
+    g.a = a; g.b = b; g.c = c;
+    g.rows = rows; g.cols = cols; g.inner = inner;
+    g.lda = lda; g.ldb = ldb; g.ldc = ldc;
+    g.stride_a = stride_a; g.stride_b = stride_b; g.stride_c = stride_c;
+    int64_t chunk = pccnn_ceil_div(pccnn_ceil_div(inner > 0 ? inner : 1, split_k), GT_K) * GT_K;
+    split_k = (int)pccnn_ceil_div(inner > 0 ? inner : 1, chunk);
+    g.split_k = split_k;
+    g.k_chunk = chunk;
+    g.aligned = ((uintptr_t)a % 16 == 0) && ((uintptr_t)b % 16 == 0) && (lda % 4 == 0) && (ldb % 4 == 0) &&
+                (stride_a % 4 == 0) && (stride_b % 4 == 0);
+    float *partial = nullptr;
+    if (split_k > 1) {
+        size_t need = (size_t)batch * split_k * rows * cols * sizeof(float);
+        PCCNN_REQUIRE(workspace && workspace_bytes >= need, PCCNN_ERR_WORKSPACE,
+                      "pccnn_gemm_f32: split-k workspace of %zu bytes, need %zu", workspace_bytes, need);
+        partial = (float *)workspace;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid((unsigned)pccnn_ceil_div(cols, GT_N), (unsigned)pccnn_ceil_div(rows, GT_M), (unsigned)(batch * split_k));
+    PCCNN_REQUIRE(grid.y <= 65535u && grid.z <= 65535u, PCCNN_ERR_UNSUPPORTED,
+                  "pccnn_gemm_f32: grid too large");
+    if (!a_trans && !b_trans) gemm_f32_mfma_kernel<false, false><<<grid, 256, 0, s>>>(g, partial);
+    else if (!a_trans && b_trans) gemm_f32_mfma_kernel<false, true><<<grid, 256, 0, s>>>(g, partial);
+    else if (a_trans && !b_trans) gemm_f32_mfma_kernel<true, false><<<grid, 256, 0, s>>>(g, partial);
+    else gemm_f32_mfma_kernel<true, true><<<grid, 256, 0, s>>>(g, partial);
+    PCCNN_LAUNCH_CHECK();
+    if (split_k > 1) {
+        int64_t total = rows * cols * batch;
+        int64_t blocks = pccnn_ceil_div(total, 256);
+        if (blocks > 4096) blocks = 4096;
+        splitk_reduce_kernel<<<(unsigned)blocks, 256, 0, s>>>(partial, g, batch);
+        PCCNN_LAUNCH_CHECK();
+    }
+    return PCCNN_OK;
+}

@@ -1,0 +1,175 @@
+// Bounding box, cell keys and the pillar table.  All three are HBM-streaming kernels:
+// one thread per point, coalesced reads of the xyz / key arrays.
+#include "common.h"
+
+// fp32 expressions in this file must round exactly as written (no fused multiply-add).
+#pragma clang fp contract(off)
+
+// ----------------------------------------------------------- bounding box
+
+__device__ __forceinline__ void atomic_min_f32(float *addr, float v)
+{
+    // Order-preserving integer views of IEEE floats: non-negative values compare as signed
+    // ints, negative values compare reversed as unsigned ints.
+    if (v >= 0.0f) atomicMin((int *)addr, __float_as_int(v));
+    else atomicMax((unsigned int *)addr, __float_as_uint(v));
+}
+__device__ __forceinline__ void atomic_max_f32(float *addr, float v)
+{
+    if (v >= 0.0f) atomicMax((int *)addr, __float_as_int(v));
+    else atomicMin((unsigned int *)addr, __float_as_uint(v));
+}
+
+__global__ void bbox_init_kernel(float *mn, float *mx, int count)
+{
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) { mn[i] = __int_as_float(0x7f800000); mx[i] = __int_as_float(0xff800000); }
+}
+
+template <int D>
+__global__ void __launch_bounds__(256)
+bbox_reduce_kernel(const float *__restrict__ pts, const int32_t *__restrict__ batch_ids, int64_t n,
+                   float *mn, float *mx)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    bool valid = i < n;
+    int b = valid ? batch_ids[i] : -1;
+    float p[D];
+#pragma unroll
+    for (int k = 0; k < D; ++k) p[k] = valid ? pts[i * D + k] : 0.0f;
+    // When every active lane of the wave belongs to one cloud, reduce in registers and
+    // issue one atomic per wave and coordinate.
+    int b0 = __builtin_amdgcn_readfirstlane(b);
+    unsigned long long vmask = __ballot(valid);
+    bool uniform = (vmask != 0ull) && (__ballot(valid && b == b0) == vmask) && (b0 >= 0);
+    if (uniform) {
+#pragma unroll
+        for (int k = 0; k < D; ++k) {
+            float lo = valid ? p[k] : __int_as_float(0x7f800000);
+            float hi = valid ? p[k] : __int_as_float(0xff800000);
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                lo = fminf(lo, __shfl_xor(lo, o));
+                hi = fmaxf(hi, __shfl_xor(hi, o));
+            }
+            if (pccnn_lane() == 0) {
+                atomic_min_f32(&mn[b0 * D + k], lo);
+                atomic_max_f32(&mx[b0 * D + k], hi);
+            }
+        }
+    } else if (valid) {
+#pragma unroll
+        for (int k = 0; k < D; ++k) {
+            atomic_min_f32(&mn[b * D + k], p[k]);
+            atomic_max_f32(&mx[b * D + k], p[k]);
+        }
+    }
+}
+
+__global__ void bbox_pad_kernel(float *mn, float *mx, int count)
+{
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) { mn[i] = mn[i] - 1e-6f; mx[i] = mx[i] + 1e-6f; }
+}
+
+extern "C" int pccnn_bounding_box(const float *pts, const int32_t *batch_ids, int64_t n, int d, int batch_size,
+                                  float *aabb_min_out, float *aabb_max_out, void *stream)
+{
+    PCCNN_REQUIRE(d == 3, PCCNN_ERR_UNSUPPORTED, "pccnn_bounding_box: d=%d is not supported (d must be 3)", d);
+    PCCNN_REQUIRE(n >= 0 && batch_size > 0, PCCNN_ERR_INVALID, "pccnn_bounding_box: n=%lld batch_size=%d",
+                  (long long)n, batch_size);
+    PCCNN_REQUIRE(aabb_min_out && aabb_max_out && (n == 0 || (pts && batch_ids)), PCCNN_ERR_INVALID,
+                  "pccnn_bounding_box: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    int count = batch_size * d;
+    bbox_init_kernel<<<(unsigned)pccnn_ceil_div(count, 256), 256, 0, s>>>(aabb_min_out, aabb_max_out, count);
+    PCCNN_LAUNCH_CHECK();
+    if (n > 0) {
+        bbox_reduce_kernel<3><<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(pts, batch_ids, n, aabb_min_out,
+                                                                             aabb_max_out);
+        PCCNN_LAUNCH_CHECK();
+    }
+    bbox_pad_kernel<<<(unsigned)pccnn_ceil_div(count, 256), 256, 0, s>>>(aabb_min_out, aabb_max_out, count);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
+// ------------------------------------------------------------------- keys
+
+template <int D>
+__global__ void __launch_bounds__(256)
+compute_keys_kernel(const float *__restrict__ pts, const int32_t *__restrict__ batch_ids,
+                    const float *__restrict__ aabb_min, const int32_t *__restrict__ num_cells,
+                    const float *__restrict__ cell_size, int64_t n, int64_t *__restrict__ keys)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    int b = batch_ids[i];
+    long long key = 0, accum = 1;
+#pragma unroll
+    for (int k = D - 1; k >= 0; --k) {
+        // fp32, exactly in this order: subtract the box corner, multiply by the fp32
+        // reciprocal of the cell size, floor, clamp.
+        float inv = __fdiv_rn(1.0f, cell_size[k]);
+        float rel = (pts[i * D + k] - aabb_min[(int64_t)b * D + k]) * inv;
+        int nc = num_cells[k];
+        int c = (int)floorf(rel);
+        c = max(0, min(c, nc - 1));
+        key += (long long)c * accum;
+        accum *= nc;
+    }
+    keys[i] = key + accum * (long long)b;
+}
+
+extern "C" int pccnn_compute_keys(const float *pts, const int32_t *batch_ids, const float *aabb_min,
+                                  const int32_t *num_cells, const float *cell_size, int64_t n, int d,
+                                  int64_t *keys_out, void *stream)
+{
+    PCCNN_REQUIRE(d == 3, PCCNN_ERR_UNSUPPORTED, "pccnn_compute_keys: d=%d is not supported (d must be 3)", d);
+    PCCNN_REQUIRE(n >= 0, PCCNN_ERR_INVALID, "pccnn_compute_keys: n=%lld", (long long)n);
+    if (n == 0) return PCCNN_OK;
+    PCCNN_REQUIRE(pts && batch_ids && aabb_min && num_cells && cell_size && keys_out, PCCNN_ERR_INVALID,
+                  "pccnn_compute_keys: null pointer");
+    compute_keys_kernel<3><<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, (hipStream_t)stream>>>(
+        pts, batch_ids, aabb_min, num_cells, cell_size, n, (int64_t *)keys_out);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
+// ------------------------------------------------------------ pillar grid
+
+template <int D>
+__global__ void __launch_bounds__(256)
+build_grid_kernel(const int64_t *__restrict__ keys, int64_t n, const int32_t *__restrict__ num_cells,
+                  int64_t num_pillars, int32_t *__restrict__ ds)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    long long div = 1;
+#pragma unroll
+    for (int k = 2; k < D; ++k) div *= num_cells[k];
+    long long cur = keys[i] / div;
+    if (cur < 0 || cur >= num_pillars) return;   // a key outside the table is never written
+    long long prev = (i > 0) ? keys[i - 1] / div : -1;
+    long long next = (i + 1 < n) ? keys[i + 1] / div : -1;
+    if (i > 0 && prev != cur) ds[2 * cur] = (int32_t)i;
+    if (i + 1 == n || next != cur) ds[2 * cur + 1] = (int32_t)(i + 1);
+}
+
+extern "C" int pccnn_build_grid_ds(const int64_t *sorted_keys, int64_t n, const int32_t *num_cells, int d,
+                                   int64_t num_pillars, int32_t *grid_ds_out, void *stream)
+{
+    PCCNN_REQUIRE(d == 3, PCCNN_ERR_UNSUPPORTED, "pccnn_build_grid_ds: d=%d is not supported (d must be 3)", d);
+    PCCNN_REQUIRE(n >= 0 && num_pillars > 0 && num_pillars < (1ll << 30), PCCNN_ERR_INVALID,
+                  "pccnn_build_grid_ds: n=%lld num_pillars=%lld", (long long)n, (long long)num_pillars);
+    PCCNN_REQUIRE(grid_ds_out && num_cells && (n == 0 || sorted_keys), PCCNN_ERR_INVALID,
+                  "pccnn_build_grid_ds: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    int rc = pccnn_fill_i32(grid_ds_out, 0, num_pillars * 2, s);
+    if (rc != PCCNN_OK) return rc;
+    if (n == 0) return PCCNN_OK;
+    build_grid_kernel<3><<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(sorted_keys, n, num_cells, num_pillars,
+                                                                        grid_ds_out);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}

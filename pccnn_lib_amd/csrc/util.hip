@@ -1,0 +1,140 @@
+// Error reporting, fill kernels and the device-wide int32 scan shared by the other files.
+#include <stdarg.h>
+
+#include "common.h"
+
+static thread_local char g_err[512] = "";
+
+void pccnn_set_error(const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+extern "C" const char *pccnn_last_error(void) { return g_err; }
+extern "C" int pccnn_version(void) { return 1; }
+
+// ------------------------------------------------------------------ fills
+
+template <typename T> __global__ void fill_kernel(T *p, T v, int64_t n)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) p[i] = v;
+}
+
+template <typename T> static int fill_impl(T *p, T v, int64_t n, hipStream_t s)
+{
+    if (n <= 0) return PCCNN_OK;
+    int64_t blocks = pccnn_ceil_div(n, 256);
+    if (blocks > 8192) blocks = 8192;
+    fill_kernel<T><<<(unsigned)blocks, 256, 0, s>>>(p, v, n);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
+int pccnn_fill_i32(int32_t *p, int32_t v, int64_t n, hipStream_t s) { return fill_impl<int32_t>(p, v, n, s); }
+int pccnn_fill_f32(float *p, float v, int64_t n, hipStream_t s) { return fill_impl<float>(p, v, n, s); }
+
+// ------------------------------------------------------------------- scan
+// Three launches: per-tile inclusive scan + tile totals, scan of the totals by one
+// workgroup, add of the tile prefix.  Tiles are SCAN_TILE consecutive elements.
+
+#define SCAN_THREADS 256
+#define SCAN_ITEMS 8
+#define SCAN_TILE (SCAN_THREADS * SCAN_ITEMS)
+
+size_t pccnn_scan_tmp_elems(int64_t n) { return (size_t)pccnn_ceil_div(n > 0 ? n : 1, SCAN_TILE) + 1; }
+
+// Inclusive scan of one value per thread across a 256-thread workgroup.
+__device__ __forceinline__ int block_inclusive_scan(int v, int *lds /* >= 4 ints */, int &total)
+{
+    int lane = pccnn_lane();
+    int wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        int t = __shfl_up(v, o);
+        if (lane >= o) v += t;
+    }
+    if (lane == 63) lds[wave] = v;
+    __syncthreads();
+    int add = 0;
+    int tot = 0;
+#pragma unroll
+    for (int w = 0; w < SCAN_THREADS / 64; ++w) {
+        int x = lds[w];
+        if (w < wave) add += x;
+        tot += x;
+    }
+    total = tot;
+    __syncthreads();
+    return v + add;
+}
+
+__global__ void __launch_bounds__(SCAN_THREADS)
+scan_tiles_kernel(const int32_t *__restrict__ in, int32_t *__restrict__ out, int64_t n, int clamp_max,
+                  int32_t *__restrict__ tile_sums)
+{
+    __shared__ int lds[4];
+    int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
+    int v[SCAN_ITEMS];
+    int sum = 0;
+#pragma unroll
+    for (int i = 0; i < SCAN_ITEMS; ++i) {
+        int x = (base + i < n) ? in[base + i] : 0;
+        if (clamp_max > 0 && x > clamp_max) x = clamp_max;
+        sum += x;
+        v[i] = sum;
+    }
+    int total;
+    int incl = block_inclusive_scan(sum, lds, total);
+    int excl = incl - sum;
+#pragma unroll
+    for (int i = 0; i < SCAN_ITEMS; ++i)
+        if (base + i < n) out[base + i] = v[i] + excl;
+    if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
+}
+
+// Exclusive scan of the tile totals, in place, by a single workgroup.
+__global__ void __launch_bounds__(SCAN_THREADS)
+scan_tile_sums_kernel(int32_t *__restrict__ tile_sums, int64_t num_tiles)
+{
+    __shared__ int lds[4];
+    int carry = 0;
+    for (int64_t base = 0; base < num_tiles; base += SCAN_THREADS) {
+        int64_t i = base + threadIdx.x;
+        int x = (i < num_tiles) ? tile_sums[i] : 0;
+        int total;
+        int incl = block_inclusive_scan(x, lds, total);
+        if (i < num_tiles) tile_sums[i] = carry + incl - x;
+        carry += total;
+    }
+}
+
+__global__ void __launch_bounds__(SCAN_THREADS)
+scan_add_kernel(int32_t *__restrict__ out, int64_t n, const int32_t *__restrict__ tile_sums)
+{
+    int add = tile_sums[blockIdx.x];
+    int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
+#pragma unroll
+    for (int i = 0; i < SCAN_ITEMS; ++i)
+        if (base + i < n) out[base + i] += add;
+}
+
+int pccnn_scan_inclusive_i32(const int32_t *in, int32_t *out, int64_t n, int clamp_max, int32_t *tmp,
+                             hipStream_t stream)
+{
+    if (n <= 0) return PCCNN_OK;
+    int64_t tiles = pccnn_ceil_div(n, SCAN_TILE);
+    scan_tiles_kernel<<<(unsigned)tiles, SCAN_THREADS, 0, stream>>>(in, out, n, clamp_max, tmp);
+    PCCNN_LAUNCH_CHECK();
+    if (tiles > 1) {
+        scan_tile_sums_kernel<<<1, SCAN_THREADS, 0, stream>>>(tmp, tiles);
+        PCCNN_LAUNCH_CHECK();
+        scan_add_kernel<<<(unsigned)tiles, SCAN_THREADS, 0, stream>>>(out, n, tmp);
+        PCCNN_LAUNCH_CHECK();
+    }
+    return PCCNN_OK;
+}

@@ -1,0 +1,39 @@
+import torch
+
+from .. import pccnn_lib_ops
+
+
+class ComputeKPConv(torch.autograd.Function):
+    """apply(pts, features, samples, neighbors, start_ids, radii, kernel_pts, sigma, conv_weights) -> [M, Cout].
+    Gradients are routed to (pts, features, samples, -, -, -, kernel_pts, -, conv_weights)
+    (pccnn_lib/op_wrappers/compute_kpconv.py:14-73)."""
+
+    @staticmethod
+    def forward(ctx, p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_kernel_pts, p_sigma,
+                p_conv_weights):
+        ctx.save_for_backward(p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_kernel_pts,
+                              p_conv_weights)
+        ctx.sigma_ = p_sigma
+        return pccnn_lib_ops.kp_conv(p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_kernel_pts,
+                                     p_sigma, p_conv_weights)
+
+    @staticmethod
+    def backward(ctx, p_grads):
+        pts, features, samples, neighbors, start_ids, radii, kernel_pts, conv_weights = ctx.saved_tensors
+        weight_grads, feat_grads, kernel_pts_grads, pt_grads, sample_grads = pccnn_lib_ops.kp_conv_grads(
+            pts, features, samples, neighbors, start_ids, radii, kernel_pts, ctx.sigma_, conv_weights, p_grads)
+        return pt_grads, feat_grads, sample_grads, None, None, None, kernel_pts_grads, None, weight_grads
+
+
+class ComputeKPConvWeightVar(torch.autograd.Function):
+    """apply(pts, features, samples, neighbors, start_ids, radii, kernel_pts, sigma): the statistic behind the
+    variance-aware initialisation (pccnn_lib/op_wrappers/compute_kpconv.py:76-113).  Not built yet."""
+
+    @staticmethod
+    def forward(ctx, p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_kernel_pts, p_sigma):
+        return pccnn_lib_ops.kp_conv_weight_var(p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii,
+                                                p_kernel_pts, p_sigma)
+
+    @staticmethod
+    def backward(ctx, p_grads):
+        return None, None, None, None, None, None, None, None

@@ -1,0 +1,62 @@
+import torch
+
+from .. import pccnn_lib_ops
+from ..op_wrappers import BuildGridDS, ComputeKeys
+
+
+class Grid(object):
+    """Regular grid over a point cloud (pccnn_lib/pc/Grid.py:10-72).
+
+    Attributes as in the reference: ``cell_size_``, ``num_cells_`` (int32 [D]), ``cell_ids_`` (int64 [N]),
+    ``sorted_ids_`` (int64 [N]: the stable key-order permutation) and ``grid_ds_`` (int32 [B, nc0, nc1, 2]).
+    The argsort and the gathers of sorted keys / points are one native radix sort; its by-products
+    (``sorted_cell_ids_``, ``sorted_pts_``, ``sorted_ids_i32_``) are kept for Neighborhood and PointPooling."""
+
+    def __init__(self, p_point_cloud, p_bounding_box, p_cell_size):
+        self.pointcloud_ = p_point_cloud
+        self.bounding_box_ = p_bounding_box
+        self.cell_size_ = torch.as_tensor(p_cell_size, dtype=torch.float32, device=p_point_cloud.pts_.device)
+        if self.cell_size_.dim() == 0:
+            self.cell_size_ = self.cell_size_.repeat(p_point_cloud.pts_.shape[1])
+        with torch.no_grad():
+            # Grid.py:26-28: fp32 division, truncation, + 1, maximum over the clouds.
+            num_cells = (self.bounding_box_.max_ - self.bounding_box_.min_) / self.cell_size_
+            self.num_cells_ = torch.max(num_cells.to(torch.int32) + 1, dim=0)[0].contiguous()
+        self.num_cells_host_ = None
+        self.cell_ids_ = None
+        self.sorted_ids_ = None
+        self.sorted_ids_i32_ = None
+        self.sorted_cell_ids_ = None
+        self.sorted_pts_ = None
+        self.grid_ds_ = None
+
+    def num_cells_host(self):
+        if self.num_cells_host_ is None:
+            self.num_cells_host_ = self.num_cells_.tolist()
+        return self.num_cells_host_
+
+    def key_bits(self):
+        return pccnn_lib_ops.key_bits_for(self.num_cells_host(), int(self.pointcloud_.batch_size_))
+
+    def compute_cell_ids(self):
+        if self.cell_ids_ is None:
+            with torch.no_grad():
+                pts = self.pointcloud_.pts_.detach()
+                self.cell_ids_ = ComputeKeys.apply(pts, self.pointcloud_.batch_ids_, self.bounding_box_.min_,
+                                                   self.num_cells_, self.cell_size_)
+                self.sorted_cell_ids_, self.sorted_ids_i32_, self.sorted_pts_ = pccnn_lib_ops.sort_keys(
+                    self.cell_ids_, self.key_bits(), pts)
+                self.sorted_ids_ = self.sorted_ids_i32_.to(torch.int64)
+
+    def build_ds(self):
+        if self.cell_ids_ is None or self.sorted_ids_ is None:
+            raise RuntimeError('In order to build the data structure first the keys for each point has to be '
+                               'computed.')
+        if self.grid_ds_ is None:
+            with torch.no_grad():
+                shape = [int(self.pointcloud_.batch_size_)] + self.num_cells_host()[0:2] + [2]
+                self.grid_ds_ = pccnn_lib_ops.build_grid_ds(self.sorted_cell_ids_, self.num_cells_, shape)
+
+    def __repr__(self):
+        return "### Cell size:\n{}\n### Num cells:\n{}\n### Cell Ids:\n{}\n### Sorted Ids:\n{}\n### Grid Ds:\n{}".format(
+            self.cell_size_, self.num_cells_, self.cell_ids_, self.sorted_ids_, self.grid_ds_)

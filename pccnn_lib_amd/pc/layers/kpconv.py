@@ -1,0 +1,73 @@
+import math
+
+import numpy as np
+import torch
+
+from ...op_wrappers import ComputeKPConv, ComputeKPConvWeightVar
+from .conv_base import IConvLayer, IConvLayerFactory
+from .kernel_points import kernel_pts_dict
+
+
+def _seeded_rotation(seed):
+    """Rotation about x, then y, then z by angles drawn from RandomState(seed), as
+    pccnn_lib/py_utils/pc_utils.py:77-125 builds it (points are multiplied from the left: p @ R)."""
+    ax, ay, az = (np.random.RandomState(seed).random_sample(3) - 0.5) * 2.0 * (2.0 * np.pi)
+    rx = np.array([[1, 0, 0], [0, np.cos(ax), -np.sin(ax)], [0, np.sin(ax), np.cos(ax)]])
+    ry = np.array([[np.cos(ay), 0, np.sin(ay)], [0, 1, 0], [-np.sin(ay), 0, np.cos(ay)]])
+    rz = np.array([[np.cos(az), -np.sin(az), 0], [np.sin(az), np.cos(az), 0], [0, 0, 1]])
+    return rz @ (ry @ rx)
+
+
+class KPConv(IConvLayer):
+    """Kernel point convolution with linear correlation (pccnn_lib/pc/layers/KPConv.py:15-146).
+    Buffers ``kernel_pts_`` [K, D] and ``sigma_``, parameter ``conv_weights_`` [K*Cin, Cout] keep the
+    reference's names and shapes, so its state dicts load."""
+
+    def __init__(self, p_dims, p_in_features, p_out_features, p_num_kernel_pts, p_constant_weight_var=True,
+                 p_const_var_value=1.0):
+        super(KPConv, self).__init__(p_dims, p_in_features, p_out_features, p_constant_weight_var,
+                                     p_const_var_value)
+        self.num_kernel_pts_ = p_num_kernel_pts
+        kp = kernel_pts_dict[str(p_dims) + "_" + str(p_num_kernel_pts)].astype(np.float32)
+        dist = np.linalg.norm(kp, axis=-1).astype(np.float32)
+        max_dist = np.amax(dist)
+        dist, kp = dist / max_dist, kp / max_dist
+        min_distance = np.amin(dist[1:])
+        if kp.shape[-1] == 3:
+            kp = np.dot(kp, _seeded_rotation(15))
+        kp = kp.astype(np.float32)
+        self.register_buffer('kernel_pts_', torch.from_numpy(kp / (1.0 + min_distance)))
+        self.register_buffer('sigma_', torch.tensor((min_distance * 1.0) / (1.0 + min_distance)))
+        self.sigma_cpu_ = None
+        self.conv_weights_ = torch.nn.Parameter(
+            torch.empty(self.num_kernel_pts_ * self.feat_input_size_, self.feat_output_size_))
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        stdv = math.sqrt(2.0 / (self.feat_input_size_ * self.num_kernel_pts_))
+        self.conv_weights_.data.normal_(0.0, stdv)
+
+    def __compute_convolution__(self, p_pc_in, p_pc_out, p_in_features, p_radius, p_neighborhood):
+        if self.sigma_cpu_ is None:
+            self.sigma_cpu_ = self.sigma_.item()
+        if self.wamup_state_ and self.use_const_variance_init_:
+            variance = ComputeKPConvWeightVar.apply(
+                p_pc_in.pts_, p_in_features, p_pc_out.pts_, p_neighborhood.neighbors_, p_neighborhood.start_ids_,
+                p_radius, self.kernel_pts_, self.sigma_cpu_)
+            self.__update_weight_var__(1.0 / variance.item())
+            stdv = math.sqrt(self.out_constant_variance_ / self.accum_weight_var_)
+            self.conv_weights_.data.normal_(0.0, stdv)
+        return ComputeKPConv.apply(
+            p_pc_in.pts_, p_in_features, p_pc_out.pts_, p_neighborhood.neighbors_, p_neighborhood.start_ids_,
+            p_radius, self.kernel_pts_, self.sigma_cpu_, self.conv_weights_)
+
+
+class KPConvFactory(IConvLayerFactory):
+    def __init__(self, p_num_kernel_pts, p_const_var_w_init=False, p_const_var_value=1.0):
+        super(KPConvFactory, self).__init__(p_num_kernel_pts, p_const_var_w_init, p_const_var_value)
+
+    def create_conv_layer(self, p_dims, p_in_features, p_out_features):
+        cur_conv = KPConv(p_dims, p_in_features, p_out_features, self.num_basis_, self.conv_var_w_init_,
+                          self.const_var_value_)
+        self.conv_list_.append(cur_conv)
+        return cur_conv

@@ -1,0 +1,58 @@
+import math
+
+import torch
+
+from ...op_wrappers import ComputeMCConv, ComputeMCConvWeightVar
+from .conv_base import IConvLayer, IConvLayerFactory
+
+
+class MCConv(IConvLayer):
+    """Monte-Carlo convolution with a one-hidden-layer kernel (pccnn_lib/pc/layers/MCConv.py:11-140).
+    Parameters keep the reference's names and shapes: ``proj_axis_`` [D, H*m], ``proj_bias_`` [1, H*m],
+    ``conv_weights_`` [m, H*Cin, Cout/m].  The input cloud must carry a density (``compute_pdf``); the op
+    receives it multiplied by the product of the radii (MCConv.py:93-94)."""
+
+    def __init__(self, p_dims, p_in_features, p_out_features, p_hidden_size, p_num_mlps=1,
+                 p_constant_weight_var=True, p_const_var_value=1.0):
+        super(MCConv, self).__init__(p_dims, p_in_features, p_out_features, p_constant_weight_var,
+                                     p_const_var_value)
+        self.hidden_size_ = p_hidden_size
+        self.num_mlps_ = p_num_mlps
+        self.proj_axis_ = torch.nn.Parameter(torch.empty(self.num_dims_, self.hidden_size_ * self.num_mlps_))
+        self.proj_bias_ = torch.nn.Parameter(torch.empty(1, self.hidden_size_ * self.num_mlps_))
+        self.conv_weights_ = torch.nn.Parameter(
+            torch.empty(self.num_mlps_, self.hidden_size_ * self.feat_input_size_,
+                        self.feat_output_size_ // p_num_mlps))
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        self.conv_weights_.data.normal_(0.0, math.sqrt(1.0 / (self.feat_input_size_ * self.hidden_size_)))
+        self.proj_axis_.data.normal_(0.0, math.sqrt(1.0 / self.num_dims_))
+        self.proj_bias_.data.fill_(0.0)
+
+    def __compute_convolution__(self, p_pc_in, p_pc_out, p_in_features, p_radius, p_neighborhood):
+        if p_pc_in.pts_unnorm_pdf_ is None:
+            raise RuntimeError("MCConv: the input point cloud has no density; call compute_pdf(bandwidth) first")
+        cur_pdf = p_pc_in.pts_unnorm_pdf_ * torch.prod(p_radius)
+        if self.wamup_state_ and self.use_const_variance_init_:
+            variance = ComputeMCConvWeightVar.apply(
+                p_pc_in.pts_, cur_pdf, p_in_features, p_pc_out.pts_, p_neighborhood.neighbors_,
+                p_neighborhood.start_ids_, p_radius, self.proj_axis_, self.proj_bias_) * self.num_mlps_
+            self.__update_weight_var__(1.0 / variance.item())
+            stdv = math.sqrt(self.out_constant_variance_ / self.accum_weight_var_)
+            self.conv_weights_.data.normal_(0.0, stdv)
+        return ComputeMCConv.apply(
+            p_pc_in.pts_, cur_pdf, p_in_features, p_pc_out.pts_, p_neighborhood.neighbors_,
+            p_neighborhood.start_ids_, p_radius, self.proj_axis_, self.proj_bias_, self.conv_weights_)
+
+
+class MCConvFactory(IConvLayerFactory):
+    def __init__(self, p_num_basis, p_const_var_w_init=False, p_num_mlps=1, p_const_var_value=1.0):
+        super(MCConvFactory, self).__init__(p_num_basis, p_const_var_w_init, p_const_var_value)
+        self.num_mlps_ = p_num_mlps
+
+    def create_conv_layer(self, p_dims, p_in_features, p_out_features):
+        cur_conv = MCConv(p_dims, p_in_features, p_out_features, self.num_basis_, self.num_mlps_,
+                          self.conv_var_w_init_, self.const_var_value_)
+        self.conv_list_.append(cur_conv)
+        return cur_conv

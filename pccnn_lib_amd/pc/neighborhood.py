@@ -1,0 +1,33 @@
+import torch
+
+from .. import pccnn_lib_ops
+from ..op_wrappers import ComputeKeys
+
+
+class Neighborhood(object):
+    """Radius neighborhood of the samples in a gridded cloud (pccnn_lib/pc/Neighborhood.py:10-53).
+
+    ``neighbors_`` int32 [T, 2] = (original point index, sample index), grouped by ascending sample;
+    ``start_ids_`` int32 [M] = inclusive running totals (the END of each sample's segment).
+    The search radius is the grid's cell size (Neighborhood.py:44).  The sorted-index -> original-index
+    remap of the reference (:47-53) happens inside the native fill pass."""
+
+    def __init__(self, p_grid, p_samples, p_max_neighbors=0):
+        self.grid_ = p_grid
+        self.samples_ = p_samples
+        grid = p_grid
+        with torch.no_grad():
+            sample_pts = p_samples.pts_.detach()
+            if p_samples is grid.pointcloud_:
+                sample_keys = grid.cell_ids_
+                order = grid.sorted_ids_i32_
+            else:
+                sample_keys = ComputeKeys.apply(sample_pts, p_samples.batch_ids_, grid.bounding_box_.min_,
+                                                grid.num_cells_, grid.cell_size_)
+                _, order, _ = pccnn_lib_ops.sort_keys(sample_keys, grid.key_bits())
+            self.neighbors_, self.start_ids_ = pccnn_lib_ops.find_neighbors_ex(
+                grid.sorted_pts_, grid.sorted_cell_ids_, sample_pts, sample_keys, grid.grid_ds_, grid.num_cells_,
+                grid.cell_size_, p_max_neighbors, sample_order=order, point_remap=grid.sorted_ids_i32_)
+
+    def __repr__(self):
+        return "### Neighbors:\n{}\n### Start indices:\n{}".format(self.neighbors_, self.start_ids_)

@@ -1,0 +1,46 @@
+import torch
+
+from .. import pccnn_lib_ops
+from .bounding_box import BoundingBox
+from .grid import Grid
+
+
+class PointPooling(object):
+    """Point-cloud pooling (pccnn_lib/pc/PointPooling.py:16-102).
+
+    ``poisson_disk``: a maximal subset of points no two of which are neighbors at the pooling radius, selected
+    greedily in cell order; ``pooling_ids_`` holds the selected ORIGINAL point indices (int64).
+    ``cell_average``: points are grouped by grid cell; ``pooling_ids_`` maps a point to its group."""
+
+    def __init__(self, p_point_cloud, p_radii, p_method="poisson_disk"):
+        self.point_cloud_ = p_point_cloud
+        self.radii_ = p_radii
+        self.method_ = p_method
+        with torch.no_grad():
+            bb = BoundingBox(p_point_cloud)
+            grid = Grid(p_point_cloud, bb, p_radii)
+            grid.compute_cell_ids()
+            if p_method == "poisson_disk":
+                grid.build_ds()
+                # self-neighborhood in sorted index space (PointPooling.py:58-62); the sorted points are
+                # already in key order, so the natural sample order is the cell order.
+                neighbors, start_ids = pccnn_lib_ops.find_neighbors_ex(
+                    grid.sorted_pts_, grid.sorted_cell_ids_, grid.sorted_pts_, grid.sorted_cell_ids_, grid.grid_ds_,
+                    grid.num_cells_, grid.cell_size_, 0)
+                sampled = pccnn_lib_ops.poisson_disk_sampling(grid.sorted_cell_ids_, neighbors, start_ids,
+                                                              grid.num_cells_).reshape(-1)
+                self.pooling_ids_ = torch.index_select(grid.sorted_ids_, 0, sampled)
+            elif p_method == "cell_average":
+                unique_ids, inverse_ids = torch.unique(grid.cell_ids_, return_inverse=True)
+                self.pooling_ids_ = inverse_ids
+                self.num_pooling_pts_ = unique_ids.shape[0]
+            else:
+                raise RuntimeError("PointPooling: unknown method '%s'" % p_method)
+
+    def pool_tensor(self, p_in_tensor, max_pool=False):
+        if self.method_ == "poisson_disk":
+            return torch.index_select(p_in_tensor, 0, self.pooling_ids_)
+        index = self.pooling_ids_.to(torch.int64).reshape(-1, 1).expand(-1, p_in_tensor.shape[1])
+        out = torch.zeros((self.num_pooling_pts_, p_in_tensor.shape[1]), dtype=p_in_tensor.dtype,
+                          device=p_in_tensor.device)
+        return out.scatter_reduce(0, index, p_in_tensor, reduce="amax" if max_pool else "mean", include_self=False)

@@ -1,0 +1,393 @@
+"""Drop-in counterpart of the reference's ``pccnn_lib_ops`` extension module.
+
+The reference exports 26 host functions taking ``torch.Tensor`` arguments
+(pccnn_lib_ops/ops_list.cpp:26-54).  This module exports the same names with the same positional
+signatures and return conventions; each call validates its tensors, allocates the outputs and a
+workspace with torch (device memory and the current stream are all torch is used for) and
+forwards raw pointers to ``libpccnn_hip.so``.  Tensors must be CUDA/HIP tensors, contiguous and of
+exactly the reference's dtypes; anything else raises ``RuntimeError`` (the reference reads such
+input as raw memory).  The op families outside the KPConv / MCConv path raise
+``NotImplementedError``.
+
+Beyond the reference's names, ``bounding_box``, ``sort_keys`` and ``find_neighbors_ex`` expose the
+native replacements of the torch / torch_scatter glue the reference keeps in Python
+(pccnn_lib/pc/BoundingBox.py:17-18, pccnn_lib/pc/Grid.py:52,68-70, pccnn_lib/pc/Neighborhood.py:27-53).
+"""
+import torch
+
+from . import _lib
+
+_P = _lib.P
+
+
+def _stream():
+    return _P(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return _P(t.data_ptr())
+
+
+def _chk(t, name, dtype, ndim=None, device=None):
+    if not isinstance(t, torch.Tensor):
+        raise RuntimeError("%s: expected a torch.Tensor, got %s" % (name, type(t).__name__))
+    if not t.is_cuda:
+        raise RuntimeError("%s: expected a GPU tensor, got device %s" % (name, t.device))
+    if t.dtype != dtype:
+        raise RuntimeError("%s: expected dtype %s, got %s" % (name, dtype, t.dtype))
+    if ndim is not None and t.dim() != ndim:
+        raise RuntimeError("%s: expected %d dimensions, got shape %s" % (name, ndim, tuple(t.shape)))
+    if not t.is_contiguous():
+        raise RuntimeError("%s: expected a contiguous tensor" % name)
+    if device is not None and t.device != device:
+        raise RuntimeError("%s: on %s but other arguments are on %s" % (name, t.device, device))
+    return t
+
+
+def _workspace(nbytes, device):
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def _dims(pts, name):
+    d = pts.shape[1]
+    if d != 3:
+        raise RuntimeError("%s: %d-dimensional points are not supported (only 3)" % (name, d))
+    return d
+
+
+# ------------------------------------------------------------------ index / grid ops
+
+
+def bounding_box(pts, batch_ids, batch_size):
+    """Per-cloud (min - 1e-6, max + 1e-6) -> (f32[B,D], f32[B,D])."""
+    _chk(pts, "bounding_box: pts", torch.float32, 2)
+    _chk(batch_ids, "bounding_box: batch_ids", torch.int32, 1, pts.device)
+    d = _dims(pts, "bounding_box")
+    batch_size = int(batch_size)
+    mn = torch.empty((batch_size, d), dtype=torch.float32, device=pts.device)
+    mx = torch.empty_like(mn)
+    _lib.call("pccnn_bounding_box", _ptr(pts), _ptr(batch_ids), pts.shape[0], d, batch_size, _ptr(mn), _ptr(mx),
+              _stream())
+    return mn, mx
+
+
+def compute_keys(pts, batch_ids, aabb_min, grid_size, cell_size):
+    """compute_keys(pts f32[N,D], batch_ids i32[N], aabb_min f32[B,D], grid_size i32[D], cell_size f32[D]) -> i64[N]
+    (pccnn_lib_ops/compute_keys/compute_keys.cuh:26-31)."""
+    _chk(pts, "compute_keys: pts", torch.float32, 2)
+    dev = pts.device
+    _chk(batch_ids, "compute_keys: batch_ids", torch.int32, 1, dev)
+    _chk(aabb_min, "compute_keys: aabb_min", torch.float32, 2, dev)
+    _chk(grid_size, "compute_keys: grid_size", torch.int32, 1, dev)
+    _chk(cell_size, "compute_keys: cell_size", torch.float32, 1, dev)
+    d = _dims(pts, "compute_keys")
+    if batch_ids.shape[0] != pts.shape[0] or aabb_min.shape[1] != d or grid_size.shape[0] != d or cell_size.shape[0] != d:
+        raise RuntimeError("compute_keys: inconsistent shapes")
+    keys = torch.empty((pts.shape[0],), dtype=torch.int64, device=dev)
+    _lib.call("pccnn_compute_keys", _ptr(pts), _ptr(batch_ids), _ptr(aabb_min), _ptr(grid_size), _ptr(cell_size),
+              pts.shape[0], d, _ptr(keys), _stream())
+    return keys
+
+
+def sort_keys(keys, key_bits=0, pts=None):
+    """Stable radix sort of cell keys.  Returns (sorted_keys i64[N], perm i32[N], sorted_pts f32[N,D] or None)."""
+    _chk(keys, "sort_keys: keys", torch.int64, 1)
+    n = keys.shape[0]
+    dev = keys.device
+    skeys = torch.empty_like(keys)
+    perm = torch.empty((n,), dtype=torch.int32, device=dev)
+    spts = None
+    d = 3
+    if pts is not None:
+        _chk(pts, "sort_keys: pts", torch.float32, 2, dev)
+        d = _dims(pts, "sort_keys")
+        if pts.shape[0] != n:
+            raise RuntimeError("sort_keys: pts and keys differ in length")
+        spts = torch.empty_like(pts)
+    ws = _workspace(_lib.load().pccnn_sort_keys_workspace_bytes(n), dev)
+    _lib.call("pccnn_sort_keys", _ptr(keys), n, int(key_bits), _ptr(skeys), _ptr(perm),
+              _ptr(pts) if pts is not None else _P(0), d, _ptr(spts) if spts is not None else _P(0),
+              _ptr(ws), ws.numel(), _stream())
+    return skeys, perm, spts
+
+
+def build_grid_ds(keys, grid_size, out_shape):
+    """build_grid_ds(sorted keys i64[N], grid_size i32[D], out_shape [B, nc0, nc1, 2]) -> i32 tensor of out_shape
+    (pccnn_lib_ops/build_grid/build_grid_ds.cuh:25-28)."""
+    _chk(keys, "build_grid_ds: keys", torch.int64, 1)
+    _chk(grid_size, "build_grid_ds: grid_size", torch.int32, 1, keys.device)
+    out_shape = [int(v) for v in out_shape]
+    if grid_size.shape[0] != 3:
+        raise RuntimeError("build_grid_ds: only 3-dimensional grids are supported")
+    if len(out_shape) != 4 or out_shape[3] != 2 or min(out_shape) < 1:
+        raise RuntimeError("build_grid_ds: out_shape must be [batch, cells0, cells1, 2], got %s" % (out_shape,))
+    ds = torch.empty(out_shape, dtype=torch.int32, device=keys.device)
+    _lib.call("pccnn_build_grid_ds", _ptr(keys), keys.shape[0], _ptr(grid_size), 3,
+              out_shape[0] * out_shape[1] * out_shape[2], _ptr(ds), _stream())
+    return ds
+
+
+def key_bits_for(grid_size_host, batch_size):
+    """Number of significant key bits for a grid of the given host-side size."""
+    total = int(batch_size)
+    for v in grid_size_host:
+        total *= int(v)
+    return max(1, (max(total, 1) - 1).bit_length())
+
+
+def find_neighbors_ex(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, radii, max_neighbors,
+                      sample_order=None, point_remap=None):
+    """find_neighbors with the two native extras: ``sample_order`` (i32[M], samples listed in key order) and
+    ``point_remap`` (i32[N], written through to column 0 of the result)."""
+    name = "find_neighbors"
+    _chk(pts, name + ": pts", torch.float32, 2)
+    dev = pts.device
+    _chk(pt_keys, name + ": pt_keys", torch.int64, 1, dev)
+    _chk(samples, name + ": samples", torch.float32, 2, dev)
+    _chk(sample_keys, name + ": sample_keys", torch.int64, 1, dev)
+    _chk(grid_ds, name + ": grid_ds", torch.int32, 4, dev)
+    _chk(grid_size, name + ": grid_size", torch.int32, 1, dev)
+    _chk(radii, name + ": radii", torch.float32, 1, dev)
+    d = _dims(pts, name)
+    n, m = pts.shape[0], samples.shape[0]
+    if pt_keys.shape[0] != n or sample_keys.shape[0] != m or samples.shape[1] != d or grid_size.shape[0] != d \
+            or radii.shape[0] != d or grid_ds.shape[3] != 2:
+        raise RuntimeError(name + ": inconsistent shapes")
+    max_neighbors = int(max_neighbors)
+    if max_neighbors < 0:
+        raise RuntimeError(name + ": max_neighbors must be >= 0")
+    if sample_order is not None:
+        _chk(sample_order, name + ": sample_order", torch.int32, 1, dev)
+        if sample_order.shape[0] != m:
+            raise RuntimeError(name + ": sample_order has the wrong length")
+    if point_remap is not None:
+        _chk(point_remap, name + ": point_remap", torch.int32, 1, dev)
+        if point_remap.shape[0] != n:
+            raise RuntimeError(name + ": point_remap has the wrong length")
+    pillars = grid_ds.shape[0] * grid_ds.shape[1] * grid_ds.shape[2]
+    ends = torch.empty((m,), dtype=torch.int32, device=dev)
+    if m == 0:
+        return [torch.empty((0, 2), dtype=torch.int32, device=dev), ends]
+    ws = _workspace(_lib.load().pccnn_find_neighbors_workspace_bytes(m), dev)
+    order_p = _ptr(sample_order) if sample_order is not None else _P(0)
+    _lib.call("pccnn_find_neighbors_count", _ptr(pts), _ptr(pt_keys), n, _ptr(samples), _ptr(sample_keys), m, order_p,
+              _ptr(grid_ds), pillars, _ptr(grid_size), _ptr(radii), d, max_neighbors, _ptr(ends), _ptr(ws),
+              ws.numel(), _stream())
+    total = int(ends[-1].item())                      # the one host read-back, as in the reference
+    neigh = torch.empty((total, 2), dtype=torch.int32, device=dev)
+    _lib.call("pccnn_find_neighbors_fill", _ptr(pts), _ptr(pt_keys), n, _ptr(samples), _ptr(sample_keys), m, order_p,
+              _ptr(grid_ds), pillars, _ptr(grid_size), _ptr(radii), d, max_neighbors, _ptr(ends),
+              _ptr(point_remap) if point_remap is not None else _P(0), total, _ptr(neigh), _ptr(ws), ws.numel(),
+              _stream())
+    return [neigh, ends]
+
+
+def find_neighbors(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, radii, max_neighbors):
+    """find_neighbors(sorted pts, sorted keys, samples, sample keys, grid_ds, grid_size, radii, max_neighbors)
+    -> [neigh i32[T,2] = (sorted point index, sample index), ends i32[M]]
+    (pccnn_lib_ops/find_neighbors/find_neighbors.cuh:33-41)."""
+    order = None
+    if isinstance(sample_keys, torch.Tensor) and sample_keys.is_cuda and sample_keys.dim() == 1 \
+            and sample_keys.shape[0] > 4096 and isinstance(grid_size, torch.Tensor) and grid_ds.dim() == 4:
+        # queries are walked in cell order so that a wavefront's 64 queries share their cell walk
+        bits = key_bits_for(grid_size.tolist(), grid_ds.shape[0])
+        _, order, _ = sort_keys(sample_keys, bits)
+    return find_neighbors_ex(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, radii, max_neighbors, order)
+
+
+# ------------------------------------------------------------------------------ pdf
+
+
+def _pdf_args(name, bandwidth, pts, neigh, ends):
+    _chk(pts, name + ": pts", torch.float32, 2)
+    dev = pts.device
+    _chk(bandwidth, name + ": bandwidth", torch.float32, 1, dev)
+    _chk(neigh, name + ": neighbors", torch.int32, 2, dev)
+    _chk(ends, name + ": start_ids", torch.int32, 1, dev)
+    d = _dims(pts, name)
+    if bandwidth.shape[0] != d or neigh.shape[1] != 2 or ends.shape[0] != pts.shape[0]:
+        raise RuntimeError(name + ": inconsistent shapes (the samples of a pdf are the points themselves)")
+    return d
+
+
+def compute_pdf(manifold_dims, bandwidth, pts, neigh, ends):
+    """compute_pdf(manifold_dims, bandwidth f32[D], pts, neighbors, start_ids) -> f32[N]
+    (pccnn_lib_ops/compute_pdf/compute_pdf.cuh:28-33)."""
+    d = _pdf_args("compute_pdf", bandwidth, pts, neigh, ends)
+    out = torch.empty((pts.shape[0],), dtype=torch.float32, device=pts.device)
+    _lib.call("pccnn_compute_pdf", int(manifold_dims), _ptr(bandwidth), _ptr(pts), pts.shape[0], d, _ptr(neigh),
+              neigh.shape[0], _ptr(ends), _ptr(out), _stream())
+    return out
+
+
+def compute_pdf_grads(manifold_dims, bandwidth, pts, neigh, ends, in_grads):
+    """compute_pdf_grads(..., in_grads f32[N]) -> f32[N,D] (pccnn_lib_ops/compute_pdf/compute_pdf.cuh:45-51)."""
+    d = _pdf_args("compute_pdf_grads", bandwidth, pts, neigh, ends)
+    in_grads = _chk(in_grads.contiguous(), "compute_pdf_grads: in_grads", torch.float32, 1, pts.device)
+    if in_grads.shape[0] != pts.shape[0]:
+        raise RuntimeError("compute_pdf_grads: in_grads has the wrong length")
+    out = torch.empty_like(pts)
+    _lib.call("pccnn_compute_pdf_grads", int(manifold_dims), _ptr(bandwidth), _ptr(pts), pts.shape[0], d, _ptr(neigh),
+              neigh.shape[0], _ptr(ends), _ptr(in_grads), _ptr(out), _stream())
+    return out
+
+
+# -------------------------------------------------------------------------- pooling
+
+
+def poisson_disk_sampling(sorted_keys, neigh, ends, grid_size):
+    """poisson_disk_sampling(sorted keys i64[N], neighbors, start_ids, grid_size) -> i64[S,1], all in sorted-index
+    space (pccnn_lib_ops/poisson_disk_sampling/poisson_disk_sampling.cuh:28-32)."""
+    name = "poisson_disk_sampling"
+    _chk(sorted_keys, name + ": keys", torch.int64, 1)
+    dev = sorted_keys.device
+    _chk(neigh, name + ": neighbors", torch.int32, 2, dev)
+    _chk(ends, name + ": start_ids", torch.int32, 1, dev)
+    _chk(grid_size, name + ": grid_size", torch.int32, 1, dev)
+    n = sorted_keys.shape[0]
+    if ends.shape[0] != n or grid_size.shape[0] != 3 or neigh.shape[1] != 2:
+        raise RuntimeError(name + ": inconsistent shapes")
+    if n == 0:
+        return torch.empty((0, 1), dtype=torch.int64, device=dev)
+    sel = torch.empty((n,), dtype=torch.int32, device=dev)
+    scan = torch.empty_like(sel)
+    ws = _workspace(_lib.load().pccnn_poisson_disk_workspace_bytes(n), dev)
+    _lib.call("pccnn_poisson_disk_select", _ptr(sorted_keys), n, _ptr(neigh), neigh.shape[0], _ptr(ends),
+              _ptr(grid_size), 3, _ptr(sel), _ptr(scan), _ptr(ws), ws.numel(), _stream())
+    count = int(scan[-1].item())
+    ids = torch.empty((count, 1), dtype=torch.int64, device=dev)
+    _lib.call("pccnn_compact_selected", _ptr(sel), _ptr(scan), n, _ptr(ids), _stream())
+    return ids
+
+
+# ----------------------------------------------------------------------------- conv
+
+
+def _conv_args(name, pts, feats, samples, neigh, ends, radii):
+    _chk(pts, name + ": pts", torch.float32, 2)
+    dev = pts.device
+    _chk(feats, name + ": features", torch.float32, 2, dev)
+    _chk(samples, name + ": samples", torch.float32, 2, dev)
+    _chk(neigh, name + ": neighbors", torch.int32, 2, dev)
+    _chk(ends, name + ": start_ids", torch.int32, 1, dev)
+    _chk(radii, name + ": radii", torch.float32, 1, dev)
+    d = _dims(pts, name)
+    if feats.shape[0] != pts.shape[0] or samples.shape[1] != d or ends.shape[0] != samples.shape[0] \
+            or neigh.shape[1] != 2 or radii.shape[0] != d:
+        raise RuntimeError(name + ": inconsistent shapes")
+    return d, dev
+
+
+def kp_conv(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights):
+    """kp_conv(pts, feats, samples, neighbors, start_ids, radii, kernel_pts f32[K,D], sigma, weights f32[K*Cin,Cout])
+    -> f32[M,Cout] (pccnn_lib_ops/pcconvs/kpconv.cuh:32-41)."""
+    name = "kp_conv"
+    d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
+    _chk(kernel_pts, name + ": kernel_pts", torch.float32, 2, dev)
+    _chk(weights, name + ": weights", torch.float32, 2, dev)
+    n, m, t, c_in, k, c_out = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1], kernel_pts.shape[0], \
+        weights.shape[1]
+    if kernel_pts.shape[1] != d or weights.shape[0] != k * c_in:
+        raise RuntimeError(name + ": weights must be [K*Cin, Cout] and kernel_pts [K, D]")
+    out = torch.empty((m, c_out), dtype=torch.float32, device=dev)
+    ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 0), dev)
+    _lib.call("pccnn_kpconv_forward", _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends), _ptr(radii),
+              _ptr(kernel_pts), float(sigma), _ptr(weights), n, m, t, d, c_in, k, c_out, _ptr(out), _ptr(ws),
+              ws.numel(), _stream())
+    return out
+
+
+def kp_conv_grads(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights, in_grads):
+    """kp_conv_grads(..., in_grads f32[M,Cout]) -> [dW, dFeat, dKernelPts, dPts, dSamples]
+    (pccnn_lib_ops/pcconvs/kpconv.cuh:56-67)."""
+    name = "kp_conv_grads"
+    d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
+    _chk(kernel_pts, name + ": kernel_pts", torch.float32, 2, dev)
+    _chk(weights, name + ": weights", torch.float32, 2, dev)
+    in_grads = _chk(in_grads.contiguous(), name + ": in_grads", torch.float32, 2, dev)
+    n, m, t, c_in, k, c_out = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1], kernel_pts.shape[0], \
+        weights.shape[1]
+    if kernel_pts.shape[1] != d or weights.shape[0] != k * c_in or tuple(in_grads.shape) != (m, c_out):
+        raise RuntimeError(name + ": inconsistent shapes")
+    d_w, d_f = torch.empty_like(weights), torch.empty_like(feats)
+    d_kp, d_p, d_s = torch.empty_like(kernel_pts), torch.empty_like(pts), torch.empty_like(samples)
+    ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
+    _lib.call("pccnn_kpconv_backward", _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends), _ptr(radii),
+              _ptr(kernel_pts), float(sigma), _ptr(weights), _ptr(in_grads), n, m, t, d, c_in, k, c_out, _ptr(d_w),
+              _ptr(d_f), _ptr(d_kp), _ptr(d_p), _ptr(d_s), _ptr(ws), ws.numel(), _stream())
+    return [d_w, d_f, d_kp, d_p, d_s]
+
+
+def _mc_args(name, pts, pdf, axis, bias, weights, c_in, d, dev):
+    _chk(pdf, name + ": pdf", torch.float32, 1, dev)
+    _chk(axis, name + ": axis", torch.float32, 2, dev)
+    _chk(bias, name + ": bias", torch.float32, 2, dev)
+    _chk(weights, name + ": weights", torch.float32, 3, dev)
+    k = axis.shape[1]
+    num_mlps, c_out = weights.shape[0], weights.shape[0] * weights.shape[2]
+    if pdf.shape[0] != pts.shape[0] or axis.shape[0] != d or tuple(bias.shape) != (1, k) \
+            or weights.shape[1] * num_mlps != k * c_in:
+        raise RuntimeError(name + ": axis must be [D, H*mlps], bias [1, H*mlps], weights [mlps, H*Cin, Cout/mlps]")
+    return k, num_mlps, c_out
+
+
+def mc_conv(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights):
+    """mc_conv(pts, pdf f32[N], feats, samples, neighbors, start_ids, radii, axis f32[D,H*m], bias f32[1,H*m],
+    weights f32[m, H*Cin, Cout/m]) -> f32[M,Cout] (pccnn_lib_ops/pcconvs/mcconv.cuh:32-42)."""
+    name = "mc_conv"
+    d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
+    n, m, t, c_in = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1]
+    k, num_mlps, c_out = _mc_args(name, pts, pdf, axis, bias, weights, c_in, d, dev)
+    out = torch.empty((m, c_out), dtype=torch.float32, device=dev)
+    ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 0), dev)
+    _lib.call("pccnn_mcconv_forward", _ptr(pts), _ptr(pdf), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends),
+              _ptr(radii), _ptr(axis), _ptr(bias), _ptr(weights), n, m, t, d, c_in, k, num_mlps, c_out, _ptr(out),
+              _ptr(ws), ws.numel(), _stream())
+    return out
+
+
+def mc_conv_grads(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights, in_grads):
+    """mc_conv_grads(..., in_grads f32[M,Cout]) -> [dW, dFeat, dAxis, dBias f32[1,H*m], dPdf f32[N], dPts, dSamples]
+    (pccnn_lib_ops/pcconvs/mcconv.cuh:57-69)."""
+    name = "mc_conv_grads"
+    d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
+    n, m, t, c_in = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1]
+    k, num_mlps, c_out = _mc_args(name, pts, pdf, axis, bias, weights, c_in, d, dev)
+    in_grads = _chk(in_grads.contiguous(), name + ": in_grads", torch.float32, 2, dev)
+    if tuple(in_grads.shape) != (m, c_out):
+        raise RuntimeError(name + ": in_grads must be [M, Cout]")
+    d_w, d_f = torch.empty_like(weights), torch.empty_like(feats)
+    d_axis, d_bias, d_pdf = torch.empty_like(axis), torch.empty_like(bias), torch.empty_like(pdf)
+    d_p, d_s = torch.empty_like(pts), torch.empty_like(samples)
+    ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
+    _lib.call("pccnn_mcconv_backward", _ptr(pts), _ptr(pdf), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends),
+              _ptr(radii), _ptr(axis), _ptr(bias), _ptr(weights), _ptr(in_grads), n, m, t, d, c_in, k, num_mlps, c_out,
+              _ptr(d_w), _ptr(d_f), _ptr(d_axis), _ptr(d_bias), _ptr(d_pdf), _ptr(d_p), _ptr(d_s), _ptr(ws),
+              ws.numel(), _stream())
+    return [d_w, d_f, d_axis, d_bias, d_pdf, d_p, d_s]
+
+
+# ------------------------------------------------------------- names outside this path
+
+
+def _not_on_path(name):
+    def fn(*_args, **_kwargs):
+        raise NotImplementedError(
+            "pccnn_lib_ops.%s belongs to an operator family that this build does not implement "
+            "(only the KPConv / MCConv path is built)" % name)
+    fn.__name__ = name
+    return fn
+
+
+for _n in ("mc_conv_weight_var", "kp_conv_weight_var", "point_conv_basis", "point_conv_basis_grads", "point_conv",
+           "point_conv_grads", "point_conv_weight_var", "kp_conv_n", "kp_conv_n_grads", "kp_conv_n_weight_var",
+           "sph_conv", "sph_conv_grads", "sph_conv_weight_var", "pccnn", "pccnn_grads", "pccnn_weight_variance"):
+    globals()[_n] = _not_on_path(_n)
+del _n
+
+REFERENCE_NAMES = (
+    "build_grid_ds", "compute_keys", "find_neighbors", "compute_pdf", "compute_pdf_grads", "poisson_disk_sampling",
+    "mc_conv", "mc_conv_grads", "mc_conv_weight_var", "point_conv_basis", "point_conv_basis_grads", "point_conv",
+    "point_conv_grads", "point_conv_weight_var", "kp_conv", "kp_conv_grads", "kp_conv_weight_var", "kp_conv_n",
+    "kp_conv_n_grads", "kp_conv_n_weight_var", "sph_conv", "sph_conv_grads", "sph_conv_weight_var", "pccnn",
+    "pccnn_grads", "pccnn_weight_variance")

@@ -1,0 +1,90 @@
+"""The C-ABI library builds, loads without a GPU and exports every symbol the header declares."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    hdr = open(os.path.join(ROOT, "include", "pccnn_hip.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    out = {}
+    for m in re.finditer(r"\b(pccnn_\w+)\s*\(([^;]*?)\)\s*;", hdr, flags=re.S):
+        args = m.group(2).strip()
+        out[m.group(1)] = 0 if args == "void" else len(args.split(","))
+    return out
+
+
+@pytest.fixture(scope="module")
+def lib_path():
+    from pccnn_lib_amd import _lib, build
+    if not os.path.exists(_lib.LIB_PATH):
+        build.build(verbose=False)
+    return _lib.LIB_PATH
+
+
+def test_every_declared_symbol_is_exported(lib_path):
+    lib = ctypes.CDLL(lib_path)
+    declared = _declared()
+    assert len(declared) >= 20
+    for name in declared:
+        assert hasattr(lib, name), name
+
+
+def test_ctypes_table_matches_header(lib_path):
+    from pccnn_lib_amd import _lib
+    declared = _declared()
+    assert set(declared) == set(_lib.SIGNATURES)
+    for name, nargs in declared.items():
+        assert len(_lib.SIGNATURES[name][1]) == nargs, name
+
+
+def test_argument_validation_needs_no_gpu(lib_path):
+    # Host-side checks run before any kernel launch, so they can be exercised on a CPU-only machine.
+    from pccnn_lib_amd import _lib
+    lib = _lib.load()
+    assert lib.pccnn_version() == 1
+    rc = lib.pccnn_compute_keys(None, None, None, None, None, 10, 2, None, None)
+    assert rc == -2 and b"d=2" in lib.pccnn_last_error()
+    rc = lib.pccnn_compute_keys(None, None, None, None, None, 10, 3, None, None)
+    assert rc == -1 and b"null" in lib.pccnn_last_error()
+    assert lib.pccnn_compute_keys(None, None, None, None, None, 0, 3, None, None) == 0
+    rc = lib.pccnn_sort_keys(ctypes.c_void_p(16), 100, 20, ctypes.c_void_p(16), ctypes.c_void_p(16), None, 3, None,
+                             None, 0, None)
+    assert rc == -3 and b"workspace" in lib.pccnn_last_error()
+    rc = lib.pccnn_kpconv_forward(None, None, None, None, None, None, None, 0.5, None, 10, 10, 10, 3, 8, 65, 8, None,
+                                  None, 0, None)
+    assert rc == -2 and b"k=65" in lib.pccnn_last_error()
+    assert lib.pccnn_conv_workspace_bytes(1000, 5000, 32, 16, 64, 0) >= 1000 * 32 * 16 * 4
+    assert lib.pccnn_find_neighbors_workspace_bytes(1000) >= 4000
+
+
+def test_op_module_exports_reference_names():
+    from pccnn_lib_amd import pccnn_lib_ops
+    assert len(pccnn_lib_ops.REFERENCE_NAMES) == 26
+    for name in pccnn_lib_ops.REFERENCE_NAMES:
+        assert callable(getattr(pccnn_lib_ops, name))
+    with pytest.raises(NotImplementedError):
+        pccnn_lib_ops.sph_conv()
+
+
+def test_ops_reject_cpu_tensors():
+    import torch
+    from pccnn_lib_amd import pccnn_lib_ops
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        pccnn_lib_ops.compute_keys(torch.zeros(4, 3), torch.zeros(4, dtype=torch.int32), torch.zeros(1, 3),
+                                   torch.ones(3, dtype=torch.int32), torch.ones(3))
+
+
+def test_layers_keep_reference_parameter_names():
+    from pccnn_lib_amd.pc.layers import KPConv, MCConv
+    kp = KPConv(3, 8, 16, 15)
+    assert set(kp.state_dict()) == {"kernel_pts_", "sigma_", "conv_weights_"}
+    assert tuple(kp.conv_weights_.shape) == (15 * 8, 16) and tuple(kp.kernel_pts_.shape) == (15, 3)
+    assert abs(float(kp.kernel_pts_[0].abs().sum())) == 0.0 and 0 < float(kp.sigma_) < 1
+    mc = MCConv(3, 8, 16, 16, 2)
+    assert set(mc.state_dict()) == {"proj_axis_", "proj_bias_", "conv_weights_"}
+    assert tuple(mc.conv_weights_.shape) == (2, 16 * 8, 8) and tuple(mc.proj_axis_.shape) == (3, 32)

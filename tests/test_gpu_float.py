@@ -1,0 +1,249 @@
+"""HIP path vs the CPU oracle for the floating-point part of the path.  Tolerances: density and
+convolution outputs 1e-5 relative (to the largest magnitude of the tensor), gradients 1e-4."""
+import numpy as np
+import pytest
+import torch
+
+from pccnn_lib_amd import synthetic
+from tests.gpu_helpers import DEV, gpu_neighborhood, relerr, t
+
+pytestmark = pytest.mark.gpu
+
+FWD_TOL = 1e-5
+GRAD_TOL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from pccnn_lib_amd import pccnn_lib_ops
+    return pccnn_lib_ops
+
+
+def _cloud(models, batch, num_pts):
+    pts = np.ascontiguousarray(models[:batch, :num_pts, :].reshape(-1, 3), np.float32)
+    return pts, np.repeat(np.arange(batch, dtype=np.int32), num_pts)
+
+
+# ------------------------------------------------------------------------------------ gemm
+
+@pytest.mark.parametrize("rows,cols,inner,at,bt,split", [
+    (256, 128, 64, 0, 0, 1), (300, 70, 45, 0, 0, 1), (128, 256, 32, 0, 1, 1), (77, 130, 19, 0, 1, 1),
+    (128, 128, 4096, 1, 0, 8), (480, 40, 1000, 1, 0, 4), (129, 129, 17, 1, 1, 1), (1024, 128, 1024, 0, 0, 1)])
+def test_gemm_against_float64(rows, cols, inner, at, bt, split):
+    from pccnn_lib_amd import _lib
+    rng = np.random.default_rng(rows + cols + inner)
+    a = rng.normal(size=(inner, rows) if at else (rows, inner)).astype(np.float32)
+    b = rng.normal(size=(cols, inner) if bt else (inner, cols)).astype(np.float32)
+    ta, tb = t(a), t(b)
+    tc = torch.full((rows, cols), float("nan"), dtype=torch.float32, device=DEV)
+    ws = torch.empty(split * rows * cols * 4 + 256, dtype=torch.uint8, device=DEV)
+    _lib.call("pccnn_gemm_f32", _lib.P(ta.data_ptr()), _lib.P(tb.data_ptr()), _lib.P(tc.data_ptr()), rows, cols, inner,
+              at, bt, a.shape[1], b.shape[1], cols, 1, 0, 0, 0, split, _lib.P(ws.data_ptr()), ws.numel(),
+              _lib.P(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    exp = (a.T if at else a).astype(np.float64) @ (b.T if bt else b).astype(np.float64)
+    assert relerr(tc.cpu().numpy(), exp) < 1e-5
+
+
+def test_gemm_batched_strided():
+    from pccnn_lib_amd import _lib
+    rng = np.random.default_rng(0)
+    m, mlps, inner, co = 200, 2, 48, 24
+    a = rng.normal(size=(m, mlps * inner)).astype(np.float32)
+    b = rng.normal(size=(mlps, inner, co)).astype(np.float32)
+    ta, tb = t(a), t(b)
+    tc = torch.zeros((m, mlps * co), dtype=torch.float32, device=DEV)
+    _lib.call("pccnn_gemm_f32", _lib.P(ta.data_ptr()), _lib.P(tb.data_ptr()), _lib.P(tc.data_ptr()), m, co, inner, 0, 0,
+              mlps * inner, co, mlps * co, mlps, inner, inner * co, co, 1, _lib.P(0), 0,
+              _lib.P(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    exp = np.concatenate([a[:, i * inner:(i + 1) * inner].astype(np.float64) @ b[i] for i in range(mlps)], axis=1)
+    assert relerr(tc.cpu().numpy(), exp) < 1e-5
+
+
+# ------------------------------------------------------------------------------------- pdf
+
+@pytest.mark.parametrize("bw", [0.025, 0.01, 0.1])
+def test_pdf_matches_oracle(ops, oracle, models, bw):
+    # bw = 0.1 reaches the 300-neighbor cap (deterministic subset, same in the oracle's restatement)
+    pts, ids = _cloud(models, 4, 1000)
+    exp_unnorm, exp_norm, exp_nb = oracle.pointcloud_pdf(pts, ids, bw)
+    import pccnn_lib_amd as lib
+    pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+    pc.compute_pdf(np.full(3, bw, np.float32))
+    torch.cuda.synchronize()
+    assert relerr(pc.pts_unnorm_pdf_.cpu().numpy(), exp_unnorm) < FWD_TOL
+    assert relerr(pc.pts_pdf_.cpu().numpy(), exp_norm) < FWD_TOL
+    assert np.allclose(pc.pts_unnorm_pdf_.cpu().numpy(), exp_unnorm, rtol=1e-5, atol=0)
+
+
+def test_pdf_grads_match_oracle(ops, oracle, models):
+    pts, ids = _cloud(models, 2, 500)
+    bw = np.full(3, 0.08, np.float32)
+    _, _, nb = oracle.pointcloud_pdf(pts, ids, bw)
+    g = np.random.default_rng(0).normal(size=pts.shape[0]).astype(np.float32)
+    exp = oracle.compute_pdf_grads(3, bw, pts, nb["neighbors"], nb["ends"], g)
+    got = ops.compute_pdf_grads(3, t(bw), t(pts), t(nb["neighbors"]), t(nb["ends"]), t(g))
+    assert relerr(got.cpu().numpy(), exp) < GRAD_TOL
+    # through autograd: d mean(pdf) / d pts
+    import pccnn_lib_amd as lib
+    pc = lib.pc.Pointcloud(pts, ids, device=DEV, requires_grad=True)
+    pc.compute_pdf(bw)
+    pc.pts_unnorm_pdf_.mean().backward()
+    exp2 = oracle.compute_pdf_grads(3, bw, pts, nb["neighbors"], nb["ends"],
+                                    np.full(pts.shape[0], 1.0 / pts.shape[0], np.float32))
+    assert relerr(pc.pts_.grad.cpu().numpy(), exp2) < GRAD_TOL
+
+
+# ------------------------------------------------------------------------------------ conv
+
+def _conv_case(oracle, ops, seed, batch, num_pts, radius, distinct_samples):
+    pts, ids = synthetic.primitives(seed, batch, num_pts)
+    rng = np.random.default_rng(seed)
+    if distinct_samples:
+        pick = np.sort(rng.choice(pts.shape[0], pts.shape[0] // 3, replace=False))
+        smp, sids = pts[pick].copy(), ids[pick]
+    else:
+        smp, sids = pts, ids
+    nb = gpu_neighborhood(ops, pts, ids, smp, sids, radius, batch)
+    return pts, ids, smp, nb, rng
+
+
+@pytest.mark.parametrize("k,c_in,c_out,distinct", [(15, 32, 32, False), (16, 64, 48, True), (8, 5, 7, True),
+                                                   (33, 128, 16, False), (64, 16, 8, True)])
+def test_kpconv_forward_and_grads(ops, oracle, k, c_in, c_out, distinct):
+    pts, ids, smp, nb, rng = _conv_case(oracle, ops, 20 + k, 2, 1500, 0.12, distinct)
+    neigh, ends, radii = nb["neighbors"], nb["ends"], nb["radii"]
+    kp, sigma = synthetic.kernel_points_sphere(1, k)
+    feats = rng.normal(size=(pts.shape[0], c_in)).astype(np.float32)
+    w = rng.normal(0, np.sqrt(1.0 / (k * c_in)), (k * c_in, c_out)).astype(np.float32)
+    g = rng.normal(size=(smp.shape[0], c_out)).astype(np.float32)
+    d = nb["dev"]
+    out = ops.kp_conv(d["pts"], t(feats), d["samples"], d["neigh"], d["ends"], d["radii"], t(kp), sigma, t(w))
+    exp = oracle.kpconv(pts, feats, smp, neigh, ends, radii, kp, sigma, w)
+    assert relerr(out.cpu().numpy(), exp) < FWD_TOL
+    grads = ops.kp_conv_grads(d["pts"], t(feats), d["samples"], d["neigh"], d["ends"], d["radii"], t(kp), sigma, t(w),
+                              t(g))
+    exp_g = oracle.kpconv_grads(pts, feats, smp, neigh, ends, radii, kp, sigma, w, g)
+    for got, e, name in zip(grads, exp_g, ("dW", "dFeat", "dKernelPts", "dPts", "dSamples")):
+        assert tuple(got.shape) == e.shape, name
+        assert relerr(got.cpu().numpy(), e) < GRAD_TOL, name
+
+
+@pytest.mark.parametrize("hidden,mlps,c_in,c_out,distinct", [(16, 1, 64, 128, False), (8, 2, 32, 24, True),
+                                                             (16, 1, 3, 16, True), (4, 4, 8, 8, False)])
+def test_mcconv_forward_and_grads(ops, oracle, hidden, mlps, c_in, c_out, distinct):
+    pts, ids, smp, nb, rng = _conv_case(oracle, ops, 40 + hidden + mlps, 2, 1500, 0.12, distinct)
+    neigh, ends, radii = nb["neighbors"], nb["ends"], nb["radii"]
+    k = hidden * mlps
+    pdf = rng.uniform(0.5, 2.0, pts.shape[0]).astype(np.float32)
+    feats = rng.normal(size=(pts.shape[0], c_in)).astype(np.float32)
+    axis = rng.normal(0, np.sqrt(1 / 3), (3, k)).astype(np.float32)
+    bias = rng.normal(0, 0.1, (1, k)).astype(np.float32)
+    w = rng.normal(0, np.sqrt(1.0 / (c_in * hidden)), (mlps, hidden * c_in, c_out // mlps)).astype(np.float32)
+    g = rng.normal(size=(smp.shape[0], c_out)).astype(np.float32)
+    d = nb["dev"]
+    args = (d["pts"], t(pdf), t(feats), d["samples"], d["neigh"], d["ends"], d["radii"], t(axis), t(bias), t(w))
+    out = ops.mc_conv(*args)
+    exp = oracle.mcconv(pts, pdf, feats, smp, neigh, ends, radii, axis, bias, w)
+    assert relerr(out.cpu().numpy(), exp) < FWD_TOL
+    grads = ops.mc_conv_grads(*args, t(g))
+    exp_g = oracle.mcconv_grads(pts, pdf, feats, smp, neigh, ends, radii, axis, bias, w, g)
+    for got, e, name in zip(grads, exp_g, ("dW", "dFeat", "dAxis", "dBias", "dPdf", "dPts", "dSamples")):
+        assert tuple(got.shape) == e.shape, name
+        assert relerr(got.cpu().numpy(), e) < GRAD_TOL, name
+
+
+def test_config1_plumbing_kpconv_layer(oracle):
+    # 2 x 1024 sphere points, radius 0.1, K = 15, sigma 0.05, 32 -> 32: through the layer API
+    import pccnn_lib_amd as lib
+    pts = np.concatenate([synthetic.sphere_surface(np.random.default_rng(s), 1024) for s in (0, 1)])
+    ids = np.repeat(np.arange(2, dtype=np.int32), 1024)
+    rng = np.random.default_rng(2)
+    feats = rng.normal(size=(2048, 32)).astype(np.float32)
+    w = rng.normal(0, np.sqrt(1.0 / (15 * 32)), (15 * 32, 32)).astype(np.float32)
+    for sigma in (0.05, None):
+        torch.manual_seed(0)
+        layer = lib.pc.layers.KPConv(3, 32, 32, 15).to(DEV)
+        layer.conv_weights_.data.copy_(t(w))
+        if sigma is not None:
+            layer.sigma_.fill_(sigma)
+        pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+        out, nbh = layer(pc, pc, t(feats), 0.1)
+        exp_nb = oracle.neighborhood(pts, ids, pts, ids, 0.1)
+        assert np.array_equal(oracle.canonical_pairs(nbh.neighbors_.cpu().numpy()),
+                              oracle.canonical_pairs(exp_nb["neighbors"]))
+        exp = oracle.kpconv(pts, feats, pts, exp_nb["neighbors"], exp_nb["ends"], exp_nb["radii"],
+                            layer.kernel_pts_.cpu().numpy(), float(layer.sigma_.item()), w)
+        assert relerr(out.detach().cpu().numpy(), exp) < FWD_TOL
+
+
+def test_mcconv_layer_autograd_routing(oracle):
+    import pccnn_lib_amd as lib
+    pts, ids = synthetic.primitives(9, 2, 1200)
+    rng = np.random.default_rng(3)
+    feats = rng.normal(size=(pts.shape[0], 16)).astype(np.float32)
+    torch.manual_seed(1)
+    layer = lib.pc.layers.MCConv(3, 16, 32, 16).to(DEV)
+    layer.proj_bias_.data.normal_(0, 0.1)
+    pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+    pc.compute_pdf(np.full(3, 0.02, np.float32))
+    tf = t(feats).requires_grad_(True)
+    out, nbh = layer(pc, pc, tf, 0.1)
+    g = rng.normal(size=tuple(out.shape)).astype(np.float32)
+    out.backward(t(g))
+    nb = dict(neighbors=nbh.neighbors_.cpu().numpy(), ends=nbh.start_ids_.cpu().numpy())
+    radii = np.full(3, 0.1, np.float32)
+    pdf = (pc.pts_unnorm_pdf_ * torch.prod(t(radii))).cpu().numpy()
+    p = lambda x: x.detach().cpu().numpy()
+    exp_g = oracle.mcconv_grads(pts, pdf, feats, pts, nb["neighbors"], nb["ends"], radii, p(layer.proj_axis_),
+                                p(layer.proj_bias_), p(layer.conv_weights_), g)
+    assert relerr(p(layer.conv_weights_.grad), exp_g[0]) < GRAD_TOL
+    assert relerr(p(tf.grad), exp_g[1]) < GRAD_TOL
+    assert relerr(p(layer.proj_axis_.grad), exp_g[2]) < GRAD_TOL
+    assert relerr(p(layer.proj_bias_.grad), exp_g[3]) < GRAD_TOL
+
+
+def test_hierarchy_level_with_pooling(oracle):
+    # one level of a hierarchical encoder: Poisson-disk pooling, then an MCConv from the fine cloud to the pooled one
+    import pccnn_lib_amd as lib
+    pts, ids = synthetic.primitives(13, 2, 3000)
+    pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+    pool = lib.pc.PointPooling(pc, torch.full((3,), 0.05, device=DEV))
+    sel = pool.pooling_ids_.cpu().numpy()
+    pooled_pts, pooled_ids = pts[sel], ids[sel]
+    for b in range(2):
+        q = pooled_pts[pooled_ids == b].astype(np.float64)
+        dist = np.linalg.norm(q[:, None] - q[None], axis=-1) + np.eye(q.shape[0]) * 1e9
+        assert dist.min() >= 0.05 * (1 - 1e-6)
+    pc_out = lib.pc.Pointcloud(pool.pool_tensor(pc.pts_), pool.pool_tensor(pc.batch_ids_))
+    pc.compute_pdf(np.full(3, 0.01, np.float32))
+    rng = np.random.default_rng(5)
+    feats = rng.normal(size=(pts.shape[0], 8)).astype(np.float32)
+    torch.manual_seed(2)
+    layer = lib.pc.layers.MCConv(3, 8, 16, 16).to(DEV)
+    out, nbh = layer(pc, pc_out, t(feats), 0.1)
+    exp_nb = oracle.neighborhood(pts, ids, pooled_pts, pooled_ids, 0.1)
+    assert np.array_equal(oracle.canonical_pairs(nbh.neighbors_.cpu().numpy()),
+                          oracle.canonical_pairs(exp_nb["neighbors"]))
+    p = lambda x: x.detach().cpu().numpy()
+    pdf = p(pc.pts_unnorm_pdf_ * 0.1 ** 3)
+    exp = oracle.mcconv(pts, pdf, feats, pooled_pts, exp_nb["neighbors"], exp_nb["ends"], exp_nb["radii"],
+                        p(layer.proj_axis_), p(layer.proj_bias_), p(layer.conv_weights_))
+    assert relerr(p(out), exp) < 2e-5
+
+
+def test_error_paths(ops):
+    pts, ids = synthetic.primitives(1, 1, 128)
+    tp, ti = t(pts), t(ids)
+    with pytest.raises(RuntimeError, match="dtype"):
+        ops.compute_keys(tp, ti.to(torch.int64), tp[:1], torch.ones(3, dtype=torch.int32, device=DEV), tp[0])
+    with pytest.raises(RuntimeError, match="not supported"):
+        ops.bounding_box(tp[:, :2].contiguous(), ti, 1)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        ops.bounding_box(tp.t().contiguous().t(), ti, 1)
+    nb = gpu_neighborhood(ops, pts, ids, pts, ids, 0.2, 1)["dev"]
+    feats = torch.zeros((128, 4), device=DEV)
+    with pytest.raises(RuntimeError, match="k=65"):
+        ops.kp_conv(tp, feats, tp, nb["neigh"], nb["ends"], nb["radii"], torch.zeros((65, 3), device=DEV), 0.3,
+                    torch.zeros((65 * 4, 2), device=DEV))

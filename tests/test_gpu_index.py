@@ -1,0 +1,157 @@
+"""HIP path vs the CPU oracle for the integer part of the path: bit-exact keys, permutation, pillar
+table and neighbor lists (compared after sorting pairs by (sample, neighbor id)), Poisson-disk selection."""
+import numpy as np
+import pytest
+import torch
+
+from pccnn_lib_amd import synthetic
+from tests.gpu_helpers import DEV, gpu_neighborhood, t
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from pccnn_lib_amd import pccnn_lib_ops
+    return pccnn_lib_ops
+
+
+def _cloud(models, batch, num_pts):
+    pts = np.ascontiguousarray(models[:batch, :num_pts, :].reshape(-1, 3), np.float32)
+    return pts, np.repeat(np.arange(batch, dtype=np.int32), num_pts)
+
+
+def _compare_neighborhoods(oracle, got, exp):
+    for key in ("aabb_min", "aabb_max", "num_cells", "keys", "perm", "sorted_keys", "sorted_pts", "grid_ds",
+                "sample_keys", "ends"):
+        assert np.array_equal(got[key], exp[key]), key
+    assert np.array_equal(oracle.canonical_pairs(got["neigh_sorted"]), oracle.canonical_pairs(exp["neigh_sorted"]))
+    assert np.array_equal(oracle.canonical_pairs(got["neighbors"]), oracle.canonical_pairs(exp["neighbors"]))
+    # this build's own order: ascending sorted-point index inside each sample, same as the oracle's
+    assert np.array_equal(got["neigh_sorted"], exp["neigh_sorted"])
+
+
+@pytest.mark.parametrize("batch,num_pts,radius", [(4, 1000, 0.2), (4, 100, 1.0), (2, 1024, 0.05), (1, 37, 0.3)])
+@pytest.mark.parametrize("use_order", [True, False])
+def test_reference_clouds_bit_exact(ops, oracle, models, batch, num_pts, radius, use_order):
+    pts, ids = _cloud(models, batch, num_pts)
+    exp = oracle.neighborhood(pts, ids, pts, ids, radius)
+    got = gpu_neighborhood(ops, pts, ids, pts, ids, radius, batch, use_order=use_order)
+    _compare_neighborhoods(oracle, got, exp)
+
+
+def test_config1_sphere_clouds(ops, oracle):
+    # 2 x 1024 points on the unit sphere, cell = radius = 0.1
+    pts = np.concatenate([synthetic.sphere_surface(np.random.default_rng(s), 1024) for s in (0, 1)])
+    ids = np.repeat(np.arange(2, dtype=np.int32), 1024)
+    exp = oracle.neighborhood(pts, ids, pts, ids, 0.1)
+    got = gpu_neighborhood(ops, pts, ids, pts, ids, 0.1, 2)
+    _compare_neighborhoods(oracle, got, exp)
+    bf, bf_ends = oracle.brute_force_neighbors(pts, ids, pts, ids, exp["radii"])
+    assert np.array_equal(got["ends"], bf_ends)
+    assert np.array_equal(oracle.canonical_pairs(got["neighbors"]), oracle.canonical_pairs(bf))
+
+
+def test_primitive_clouds_medium(ops, oracle):
+    pts, ids = synthetic.primitives(3, 4, 4096)
+    exp = oracle.neighborhood(pts, ids, pts, ids, 0.05)
+    got = gpu_neighborhood(ops, pts, ids, pts, ids, 0.05, 4)
+    _compare_neighborhoods(oracle, got, exp)
+
+
+def test_samples_differ_from_points(ops, oracle):
+    pts, ids = synthetic.primitives(5, 3, 2000)
+    rng = np.random.default_rng(1)
+    pick = np.sort(rng.choice(pts.shape[0], 700, replace=False))
+    smp = (pts[pick] + rng.normal(0, 0.004, (700, 3))).astype(np.float32)   # some fall outside the box: clamped
+    sids = ids[pick]
+    exp = oracle.neighborhood(pts, ids, smp, sids, 0.08)
+    got = gpu_neighborhood(ops, pts, ids, smp, sids, 0.08, 3)
+    _compare_neighborhoods(oracle, got, exp)
+
+
+@pytest.mark.parametrize("cap", [4, 16])
+def test_capped_neighbors(ops, oracle, models, cap):
+    pts, ids = _cloud(models, 4, 1000)
+    exp = oracle.neighborhood(pts, ids, pts, ids, 0.2, max_neighbors=cap)
+    got = gpu_neighborhood(ops, pts, ids, pts, ids, 0.2, 4, max_neighbors=cap)
+    assert np.array_equal(got["ends"], exp["ends"])
+    assert np.diff(got["ends"], prepend=0).max() == cap
+    # same deterministic even-spaced subset as the oracle's restatement
+    assert np.array_equal(got["neigh_sorted"], exp["neigh_sorted"])
+
+
+def test_degenerate_inputs(ops, oracle):
+    # all points in one cell; a single point; duplicate points
+    pts = np.tile(np.array([[0.5, 0.5, 0.5]], np.float32), (130, 1))
+    pts[:65] += np.random.default_rng(0).normal(0, 1e-3, (65, 3)).astype(np.float32)
+    ids = np.zeros(130, np.int32)
+    exp = oracle.neighborhood(pts, ids, pts, ids, 0.5)
+    got = gpu_neighborhood(ops, pts, ids, pts, ids, 0.5, 1)
+    _compare_neighborhoods(oracle, got, exp)
+    assert got["ends"][-1] == 130 * 130
+    one = np.array([[1.0, 2.0, 3.0]], np.float32)
+    got = gpu_neighborhood(ops, one, np.zeros(1, np.int32), one, np.zeros(1, np.int32), 0.1, 1)
+    assert got["neighbors"].tolist() == [[0, 0]] and got["ends"].tolist() == [1]
+
+
+def test_empty_sample_set(ops):
+    pts, ids = synthetic.primitives(1, 1, 256)
+    g = gpu_neighborhood(ops, pts, ids, pts, ids, 0.1, 1)["dev"]
+    neigh, ends = ops.find_neighbors_ex(g["spts"], g["skeys"], torch.empty((0, 3), device=DEV),
+                                        torch.empty((0,), dtype=torch.int64, device=DEV), g["ds"], g["nc"],
+                                        g["radii"], 0)
+    assert tuple(neigh.shape) == (0, 2) and tuple(ends.shape) == (0,)
+
+
+def test_sort_is_stable_and_handles_many_passes(ops):
+    rng = np.random.default_rng(7)
+    for n, bits in ((1, 8), (2049, 3), (100000, 20), (70001, 40), (5000, 63)):
+        keys = rng.integers(0, 2 ** min(bits, 62), n, dtype=np.int64)
+        pts = rng.normal(size=(n, 3)).astype(np.float32)
+        skeys, perm, spts = ops.sort_keys(t(keys), bits, t(pts))
+        order = np.argsort(keys, kind="stable")
+        assert np.array_equal(perm.cpu().numpy(), order.astype(np.int32)), (n, bits)
+        assert np.array_equal(skeys.cpu().numpy(), keys[order])
+        assert np.array_equal(spts.cpu().numpy(), pts[order])
+
+
+def test_poisson_disk_matches_oracle(ops, oracle, models):
+    for num_pts, radius in ((1000, 0.1), (100, 3.0)):
+        pts, ids = _cloud(models, 4, num_pts)
+        exp = oracle.neighborhood(pts, ids, pts, ids, radius)
+        e_neigh, e_ends = oracle.find_neighbors(exp["sorted_pts"], exp["sorted_keys"], exp["sorted_pts"],
+                                                exp["sorted_keys"], exp["grid_ds"], exp["num_cells"], exp["radii"])
+        e_sel = oracle.poisson_disk_sampling(exp["sorted_keys"], e_neigh, e_ends, exp["num_cells"])
+        g = gpu_neighborhood(ops, pts, ids, pts, ids, radius, 4)["dev"]
+        neigh, ends = ops.find_neighbors_ex(g["spts"], g["skeys"], g["spts"], g["skeys"], g["ds"], g["nc"],
+                                            g["radii"], 0)
+        sel = ops.poisson_disk_sampling(g["skeys"], neigh, ends, g["nc"])
+        assert sel.dtype == torch.int64 and sel.shape[1] == 1
+        assert np.array_equal(sel.cpu().numpy(), e_sel)
+
+
+def test_run_twice_is_bitwise_identical(ops):
+    pts, ids = synthetic.primitives(11, 2, 3000)
+    a = gpu_neighborhood(ops, pts, ids, pts, ids, 0.06, 2)
+    b = gpu_neighborhood(ops, pts, ids, pts, ids, 0.06, 2)
+    assert np.array_equal(a["neighbors"], b["neighbors"]) and np.array_equal(a["ends"], b["ends"])
+
+
+def test_scene_scale_properties(ops):
+    # 200k-point room (the generator of the million-point configuration) checked through size-independent
+    # properties: sorted keys, permutation, self-membership, symmetry, monotone ends.
+    pts = synthetic.room(4, 200000)
+    ids = np.zeros(pts.shape[0], np.int32)
+    g = gpu_neighborhood(ops, pts, ids, pts, ids, 0.05, 1)
+    assert np.all(np.diff(g["sorted_keys"]) >= 0)
+    assert np.array_equal(np.sort(g["perm"]), np.arange(pts.shape[0]))
+    ends, neigh = g["ends"], g["neighbors"]
+    assert ends[-1] == neigh.shape[0] and np.all(np.diff(ends, prepend=0) >= 1)
+    assert np.array_equal(neigh[:, 1], np.repeat(np.arange(pts.shape[0]), np.diff(ends, prepend=0)))
+    d = np.linalg.norm(pts[neigh[:, 0]].astype(np.float64) - pts[neigh[:, 1]].astype(np.float64), axis=1)
+    assert d.max() < 0.05 * (1 + 1e-5)
+    fwd = neigh[:, 0].astype(np.int64) * pts.shape[0] + neigh[:, 1]
+    bwd = neigh[:, 1].astype(np.int64) * pts.shape[0] + neigh[:, 0]
+    assert np.array_equal(np.sort(fwd), np.sort(bwd))
+    assert np.count_nonzero(neigh[:, 0] == neigh[:, 1]) == pts.shape[0]
