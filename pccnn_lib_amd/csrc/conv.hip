@@ -249,6 +249,11 @@ __global__ void __launch_bounds__(256)
 conv_basis_bwd_kernel(ConvGeom g, const float *__restrict__ basis_grads, float *__restrict__ d_pts,
                       float *__restrict__ d_samples, float *__restrict__ d_pdf, float *__restrict__ param_grads)
 {
+    // The KPConv correlation has a kink where a pair sits exactly one sigma away from a kernel
+    // point, and every self pair (offset 0) does so for the kernel points closest to the centre.
+    // Which side of the kink such a pair falls on is decided by the last bit of the fp32
+    // distance, so the distance is evaluated exactly as written: no fused multiply-add.
+#pragma clang fp contract(off)
     extern __shared__ float lds_param[];                            // 4*K floats
     const int nparam = (BASIS == BASIS_KP ? 3 : 4) * g.k;
     for (int i = threadIdx.x; i < nparam; i += blockDim.x) lds_param[i] = 0.0f;
