@@ -1,0 +1,225 @@
+#!/usr/bin/env python3
+"""Benchmark of the point-cloud operator path on one MI355X.
+
+Workload (config 2 of the baseline: "object-scale MCConv fwd+bwd"): 16 clouds x 4096 points sampled
+on random primitives and scaled into the unit cube; radius 0.05; density by Gaussian KDE with bandwidth
+0.2 * radius; MCConv with a 3 -> 16 hidden kernel, 64 -> 128 channels, fp32.  Inputs are synthetic
+(seeded) and resident in HBM before anything is timed.
+
+One step = one MCConv forward plus one backward (all gradients the op returns) over the batch, the
+neighborhood and the densities being built beforehand.  `value` = points / second = M / step time.
+In the same run the neighbor pipeline (box, keys, radix sort, pillar table, count, scan, fill) and the
+density pipeline are timed as well and reported as extra keys of the same JSON line, next to
+
+  roofline      the dominant kernel of the step (the fp32 MFMA contraction): algorithmic flops per launch
+                divided by its mean launch duration, taken live with HIP events on the launch stream;
+  roofline_neighbors   the same for the neighbor fill kernel against HBM bandwidth;
+  cpu_baseline  the CPU oracle (scalar C + numpy, one thread) on a bounded sample of the same workload.
+
+Exactly one JSON line goes to stdout; progress goes to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+MFMA_FP32_PEAK_TFLOPS = 157.3     # MI355X dense fp32 matrix peak
+HBM_PEAK_GBPS = 8000.0            # MI355X HBM3E peak
+
+# HBM bytes per launch of the dominant kernels, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# command (see profiles/); None until measured for the current kernels.
+TRAFFIC_GEMM_BYTES = None
+TRAFFIC_NB_FILL_BYTES = None
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def make_workload(seed=2, batch=16, num_pts=4096, c_in=64, c_out=128, hidden=16):
+    from pccnn_lib_amd import synthetic
+    pts, ids = synthetic.primitives(seed, batch, num_pts)
+    rng = np.random.default_rng(seed)
+    n = pts.shape[0]
+    return dict(
+        pts=pts, ids=ids, batch=batch, num_pts=num_pts, radius=0.05, bandwidth=0.2 * 0.05,
+        feats=rng.normal(size=(n, c_in)).astype(np.float32),
+        axis=rng.normal(0, np.sqrt(1.0 / 3.0), (3, hidden)).astype(np.float32),
+        bias=np.zeros((1, hidden), np.float32),
+        weights=rng.normal(0, np.sqrt(1.0 / (hidden * c_in)), (1, hidden * c_in, c_out)).astype(np.float32),
+        out_grads=rng.normal(size=(n, c_out)).astype(np.float32),
+        c_in=c_in, c_out=c_out, hidden=hidden)
+
+
+def cpu_baseline(wl, clouds=2):
+    """The oracle's MCConv forward + backward on the first `clouds` clouds, one thread."""
+    from oracle import oracle
+    try:
+        from threadpoolctl import threadpool_limits
+    except ImportError:                                           # pragma: no cover
+        threadpool_limits = None
+    n = clouds * wl["num_pts"]
+    pts, ids, feats = wl["pts"][:n], wl["ids"][:n], wl["feats"][:n]
+    unnorm, _, _ = oracle.pointcloud_pdf(pts, ids, wl["bandwidth"])
+    nb = oracle.neighborhood(pts, ids, pts, ids, wl["radius"])
+    pdf = (unnorm * np.prod(nb["radii"])).astype(np.float32)
+    args = (pts, pdf, feats, pts, nb["neighbors"], nb["ends"], nb["radii"], wl["axis"], wl["bias"], wl["weights"])
+
+    def run():
+        oracle.mcconv(*args)
+        oracle.mcconv_grads(*args, wl["out_grads"][:n])
+
+    ctx = threadpool_limits(limits=1) if threadpool_limits else None
+    try:
+        run()                                                     # warm-up
+        t0 = time.perf_counter()
+        reps = 0
+        while reps < 3 and (reps == 0 or time.perf_counter() - t0 < 20.0):
+            run()
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+    finally:
+        if ctx is not None:
+            ctx.unregister() if hasattr(ctx, "unregister") else ctx.restore_original_limits()
+    return {"value": n / dt, "unit": "points/s", "cores": 1, "kind": "port",
+            "sample": "oracle mcconv + mcconv_grads on %d of %d clouds (%d points, %d pairs), %d repetition(s), "
+                      "neighbor search and density excluded like in `value`" % (clouds, wl["batch"], n,
+                                                                               nb["neighbors"].shape[0], reps)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this build runs on one GPU only; --gpus %d is not supported "
+            "(no collectives or sharding are part of it)" % args.gpus)
+        return 2
+
+    import torch
+    from pccnn_lib_amd import _lib, build
+    if not os.path.exists(_lib.LIB_PATH):
+        log("libpccnn_hip.so not found, building it")
+        build.build(verbose=False)
+    if not torch.cuda.is_available():
+        log("bench.py needs a GPU (torch.cuda.is_available() is False)")
+        return 3
+    import pccnn_lib_amd as lib
+    ops = lib.pccnn_lib_ops
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    wl = make_workload()
+    t = lambda a: torch.as_tensor(a, device=dev)
+    pts, ids, feats = t(wl["pts"]), t(wl["ids"]), t(wl["feats"])
+    axis, bias, weights, out_grads = t(wl["axis"]), t(wl["bias"]), t(wl["weights"]), t(wl["out_grads"])
+    radii = torch.full((3,), wl["radius"], dtype=torch.float32, device=dev)
+    bw = torch.full((3,), wl["bandwidth"], dtype=torch.float32, device=dev)
+    m = pts.shape[0]
+
+    # ---- untimed set-up: density and neighborhood (they are inputs of the timed step)
+    pc = lib.pc.Pointcloud(pts, ids)
+    pc.compute_pdf(bw)
+    nbh = lib.pc.layers.conv_base.build_neighborhood(pc, pc, radii, 0)
+    neigh, ends = nbh.neighbors_, nbh.start_ids_
+    pdf = (pc.pts_unnorm_pdf_ * torch.prod(radii)).contiguous()
+    total_pairs = int(neigh.shape[0])
+    torch.cuda.synchronize()
+    log("workload: M=N=%d, T=%d pairs (%.1f per point)" % (m, total_pairs, total_pairs / m))
+
+    conv_args = (pts, pdf, feats, pts, neigh, ends, radii, axis, bias, weights)
+
+    def conv_step():
+        out = ops.mc_conv(*conv_args)
+        grads = ops.mc_conv_grads(*conv_args, out_grads)
+        return out, grads
+
+    def pc_fresh():
+        p = lib.pc.Pointcloud.__new__(lib.pc.Pointcloud)         # same tensors, no cached grid
+        p.__dict__.update(pc.__dict__)
+        return p
+
+    def neighbor_step():
+        p = pc_fresh()
+        return lib.pc.layers.conv_base.build_neighborhood(p, p, radii, 0)
+
+    def pdf_step():
+        p = pc_fresh()
+        p.compute_pdf(bw)
+        return p
+
+    def timed(fn, steps, warmup):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        _lib.timing(enable=True, reset=True)
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        kernels = _lib.timing(enable=False)
+        return dt / steps * 1e3, kernels
+
+    conv_ms, conv_kernels = timed(conv_step, args.steps, args.warmup)
+    nb_ms, nb_kernels = timed(neighbor_step, args.steps, args.warmup)
+    pdf_ms, pdf_kernels = timed(pdf_step, args.steps, args.warmup)
+    log("conv fwd+bwd %.3f ms | neighborhood %.3f ms | density %.3f ms" % (conv_ms, nb_ms, pdf_ms))
+    for name, ks in (("conv", conv_kernels), ("neighbors", nb_kernels), ("pdf", pdf_kernels)):
+        log(name, {k: "%d x %.1f us" % (v[0], 1e3 * v[1] / v[0]) for k, v in ks.items()})
+
+    # ---- roofline of the dominant kernel: the contraction (three launches per step, equal flops)
+    kdim = wl["hidden"] * wl["c_in"]
+    gemm_flops = 2.0 * m * kdim * wl["c_out"]
+    gemm_n, gemm_total_ms = conv_kernels.get("gemm", (0, 0.0))
+    gemm_avg_ms = gemm_total_ms / max(gemm_n, 1)
+    gemm_tflops = gemm_flops / (gemm_avg_ms * 1e-3) / 1e12 if gemm_n else 0.0
+    roofline = {"kernel": "gemm_f32_mfma_kernel", "bound": "mfma", "achieved": gemm_tflops,
+                "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": gemm_tflops / MFMA_FP32_PEAK_TFLOPS,
+                "traffic": TRAFFIC_GEMM_BYTES, "flops_per_launch": gemm_flops, "avg_launch_ms": gemm_avg_ms,
+                "launches": gemm_n}
+
+    # ---- neighbor fill kernel against HBM: 8T out + 24M (sample xyz, key, order, offsets) + 20N (point xyz, key)
+    grid_bytes = 8 * wl["batch"] * int(np.prod(nbh.grid_.num_cells_host()[0:2]))
+    nb_bytes = 8.0 * total_pairs + 24.0 * m + 20.0 * m + grid_bytes
+    fill_n, fill_total_ms = nb_kernels.get("nb_fill", (0, 0.0))
+    fill_avg_ms = fill_total_ms / max(fill_n, 1)
+    fill_gbps = nb_bytes / (fill_avg_ms * 1e-3) / 1e9 if fill_n else 0.0
+    roofline_nb = {"kernel": "neighbors_kernel<fill>", "bound": "hbm", "achieved": fill_gbps, "peak": HBM_PEAK_GBPS,
+                   "unit": "GB/s", "frac": fill_gbps / HBM_PEAK_GBPS, "traffic": TRAFFIC_NB_FILL_BYTES,
+                   "bytes_per_launch": nb_bytes, "avg_launch_ms": fill_avg_ms, "launches": fill_n}
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        log("timing the CPU oracle on a sample ...")
+        cpu = cpu_baseline(wl)
+        log("cpu baseline: %.0f points/s" % cpu["value"])
+
+    result = {
+        "metric": "mcconv_fwd_bwd_points_per_sec", "value": m / (conv_ms * 1e-3), "unit": "points/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": conv_ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "config 2: MCConv fwd+bwd, 16 x 4096 points on random primitives, radius 0.05, "
+                               "KDE bandwidth 0.01, hidden 16, Cin 64 -> Cout 128, fp32",
+                   "points": m, "pairs": total_pairs, "seed": 2},
+        "neighbor_pairs_per_sec": total_pairs / (nb_ms * 1e-3), "neighborhood_ms": nb_ms,
+        "density_ms": pdf_ms,
+        "kernels_us": {leg: {k: round(1e3 * v[1] / v[0], 2) for k, v in ks.items()}
+                       for leg, ks in (("conv", conv_kernels), ("neighborhood", nb_kernels), ("density", pdf_kernels))},
+        "roofline": roofline, "roofline_neighbors": roofline_nb, "cpu_baseline": cpu,
+    }
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

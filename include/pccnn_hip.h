@@ -191,6 +191,18 @@ int pccnn_gemm_f32(const float *a, const float *b, float *c, int64_t rows, int64
                    int batch, int64_t stride_a, int64_t stride_b, int64_t stride_c,
                    int split_k, void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- per-kernel timing ---------------------------------------------------
+ * Measurement hooks with no counterpart in the reference (it has no profiler hooks).  While
+ * enabled, the entry points above bracket their main kernels with HIP events on the launch
+ * stream; pccnn_timing_read waits for the recorded events and returns, for timer `id` in
+ * [0, pccnn_timing_count()), the number of bracketed launches and their summed duration in ms
+ * since the last reset.  Timer names: pccnn_timing_name(id).  Off by default. */
+int pccnn_timing_enable(int on);
+int pccnn_timing_reset(void);
+int pccnn_timing_count(void);
+const char *pccnn_timing_name(int id);
+int pccnn_timing_read(int id, int64_t *h_launches, double *h_total_ms);
+
 #ifdef __cplusplus
 }
 #endif

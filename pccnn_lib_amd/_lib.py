@@ -40,6 +40,11 @@ SIGNATURES = {
                                    P, P, SZ, P]),
     "pccnn_mcconv_backward": (I32, [P, P, P, P, P, P, P, P, P, P, P, I64, I64, I64, I32, I32, I32, I32, I32,
                                     P, P, P, P, P, P, P, P, SZ, P]),
+    "pccnn_timing_enable": (I32, [I32]),
+    "pccnn_timing_reset": (I32, []),
+    "pccnn_timing_count": (I32, []),
+    "pccnn_timing_name": (ctypes.c_char_p, [I32]),
+    "pccnn_timing_read": (I32, [I32, P, P]),
     "pccnn_gemm_f32": (I32, [P, P, P, I64, I64, I64, I32, I32, I64, I64, I64, I32, I64, I64, I64, I32, P, SZ, P]),
 }
 
@@ -73,3 +78,20 @@ def check(rc, what):
 def call(name, *args):
     """Call an int-returning entry point and raise on a non-zero status."""
     check(getattr(load(), name)(*args), name)
+
+
+def timing(enable=None, reset=False):
+    """Switch the per-kernel timers on/off, optionally reset them, and return
+    {name: (launches, total_ms)} for the timers that fired."""
+    lib = load()
+    if reset:
+        lib.pccnn_timing_reset()
+    if enable is not None:
+        lib.pccnn_timing_enable(1 if enable else 0)
+    out = {}
+    for i in range(lib.pccnn_timing_count()):
+        n, ms = ctypes.c_int64(0), ctypes.c_double(0.0)
+        check(lib.pccnn_timing_read(i, ctypes.byref(n), ctypes.byref(ms)), "pccnn_timing_read")
+        if n.value:
+            out[lib.pccnn_timing_name(i).decode()] = (n.value, ms.value)
+    return out

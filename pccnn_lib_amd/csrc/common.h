@@ -80,6 +80,21 @@ __device__ __forceinline__ float pccnn_wave_sum(float v)
 }
 #endif
 
+// Optional per-kernel timing (off by default): a PccnnTimed object brackets the launches made
+// during its lifetime with two events on the launch stream; pccnn_timing_read sums them up.
+enum PccnnTimerId {
+    PCCNN_T_GEMM = 0, PCCNN_T_PROJ_FWD, PCCNN_T_PROJ_BWD, PCCNN_T_BASIS_BWD, PCCNN_T_NB_COUNT, PCCNN_T_NB_FILL,
+    PCCNN_T_SORT, PCCNN_T_KEYS, PCCNN_T_GRID, PCCNN_T_PDF, PCCNN_T_SCAN, PCCNN_T_COUNT
+};
+struct PccnnTimed {
+    int id;
+    hipStream_t stream;
+    hipEvent_t stop;
+    bool on;
+    PccnnTimed(int id, hipStream_t s);
+    ~PccnnTimed();
+};
+
 // Device-wide inclusive scan of int32 (scan.hip).  `clamp_max` > 0 clamps each input first.
 // tmp must hold pccnn_scan_tmp_elems(n) ints.
 size_t pccnn_scan_tmp_elems(int64_t n);

@@ -328,6 +328,7 @@ template <int BASIS>
 static int launch_proj_fwd(const ConvGeom &g, const float *feats, float *proj, hipStream_t s)
 {
     dim3 grid((unsigned)pccnn_ceil_div(g.m, 4), (unsigned)((g.c_in + 63) / 64));
+    PccnnTimed timed(PCCNN_T_PROJ_FWD, s);
     switch (kpad_of(g.k)) {
     case 8: conv_proj_fwd_kernel<BASIS, 8><<<grid, 256, 0, s>>>(g, feats, proj); break;
     case 16: conv_proj_fwd_kernel<BASIS, 16><<<grid, 256, 0, s>>>(g, feats, proj); break;
@@ -343,6 +344,7 @@ static int launch_proj_bwd(const ConvGeom &g, const float *feats, const float *p
                            float *basis_grads, hipStream_t s)
 {
     dim3 grid((unsigned)pccnn_ceil_div(g.m, 4));
+    PccnnTimed timed(PCCNN_T_PROJ_BWD, s);
     switch (kpad_of(g.k)) {
     case 8: conv_proj_bwd_kernel<BASIS, 8><<<grid, 256, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads); break;
     case 16: conv_proj_bwd_kernel<BASIS, 16><<<grid, 256, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads); break;
@@ -459,8 +461,11 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     if ((rc = launch_proj_bwd<BASIS>(g, feats, d_proj, d_feats, basis_g, s)) != PCCNN_OK) return rc;
     int64_t blocks = pccnn_ceil_div(g.t, 256);
     if (blocks > 2048) blocks = 2048;
-    conv_basis_bwd_kernel<BASIS><<<(unsigned)blocks, 256, 4 * g.k * sizeof(float), s>>>(g, basis_g, d_pts, d_samples,
-                                                                                        d_pdf, d_param);
+    {
+        PccnnTimed timed(PCCNN_T_BASIS_BWD, s);
+        conv_basis_bwd_kernel<BASIS><<<(unsigned)blocks, 256, 4 * g.k * sizeof(float), s>>>(g, basis_g, d_pts, d_samples,
+                                                                                            d_pdf, d_param);
+    }
     PCCNN_LAUNCH_CHECK();
     copy_params_kernel<<<1, 256, 0, s>>>(d_param, d_param_a, count_a, d_param_b, count_b);
     PCCNN_LAUNCH_CHECK();

@@ -215,10 +215,13 @@ extern "C" int pccnn_gemm_f32(const float *a, const float *b, float *c, int64_t 
     dim3 grid((unsigned)pccnn_ceil_div(cols, GT_N), (unsigned)pccnn_ceil_div(rows, GT_M), (unsigned)(batch * split_k));
     PCCNN_REQUIRE(grid.y <= 65535u && grid.z <= 65535u, PCCNN_ERR_UNSUPPORTED,
                   "pccnn_gemm_f32: grid too large");
-    if (!a_trans && !b_trans) gemm_f32_mfma_kernel<false, false><<<grid, 256, 0, s>>>(g, partial);
-    else if (!a_trans && b_trans) gemm_f32_mfma_kernel<false, true><<<grid, 256, 0, s>>>(g, partial);
-    else if (a_trans && !b_trans) gemm_f32_mfma_kernel<true, false><<<grid, 256, 0, s>>>(g, partial);
-    else gemm_f32_mfma_kernel<true, true><<<grid, 256, 0, s>>>(g, partial);
+    {
+        PccnnTimed timed(PCCNN_T_GEMM, s);
+        if (!a_trans && !b_trans) gemm_f32_mfma_kernel<false, false><<<grid, 256, 0, s>>>(g, partial);
+        else if (!a_trans && b_trans) gemm_f32_mfma_kernel<false, true><<<grid, 256, 0, s>>>(g, partial);
+        else if (a_trans && !b_trans) gemm_f32_mfma_kernel<true, false><<<grid, 256, 0, s>>>(g, partial);
+        else gemm_f32_mfma_kernel<true, true><<<grid, 256, 0, s>>>(g, partial);
+    }
     PCCNN_LAUNCH_CHECK();
     if (split_k > 1) {
         int64_t total = rows * cols * batch;

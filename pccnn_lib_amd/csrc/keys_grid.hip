@@ -130,6 +130,7 @@ extern "C" int pccnn_compute_keys(const float *pts, const int32_t *batch_ids, co
     if (n == 0) return PCCNN_OK;
     PCCNN_REQUIRE(pts && batch_ids && aabb_min && num_cells && cell_size && keys_out, PCCNN_ERR_INVALID,
                   "pccnn_compute_keys: null pointer");
+    PccnnTimed timed(PCCNN_T_KEYS, (hipStream_t)stream);
     compute_keys_kernel<3><<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, (hipStream_t)stream>>>(
         pts, batch_ids, aabb_min, num_cells, cell_size, n, (int64_t *)keys_out);
     PCCNN_LAUNCH_CHECK();
@@ -165,6 +166,7 @@ extern "C" int pccnn_build_grid_ds(const int64_t *sorted_keys, int64_t n, const 
     PCCNN_REQUIRE(grid_ds_out && num_cells && (n == 0 || sorted_keys), PCCNN_ERR_INVALID,
                   "pccnn_build_grid_ds: null pointer");
     hipStream_t s = (hipStream_t)stream;
+    PccnnTimed timed(PCCNN_T_GRID, s);
     int rc = pccnn_fill_i32(grid_ds_out, 0, num_pillars * 2, s);
     if (rc != PCCNN_OK) return rc;
     if (n == 0) return PCCNN_OK;

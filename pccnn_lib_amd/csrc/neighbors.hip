@@ -238,8 +238,12 @@ extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t
     a.num_cells = num_cells; a.radii = radii; a.max_neighbors = max_neighbors;
     a.counts = counts; a.ends = nullptr; a.remap = nullptr; a.t = 0; a.neigh = nullptr;
     int64_t waves = pccnn_ceil_div(m, 64);
-    neighbors_kernel<false><<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
+    {
+        PccnnTimed timed(PCCNN_T_NB_COUNT, s);
+        neighbors_kernel<false><<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
+    }
     PCCNN_LAUNCH_CHECK();
+    PccnnTimed timed(PCCNN_T_SCAN, s);
     return pccnn_scan_inclusive_i32(counts, ends_out, m, max_neighbors, scan_tmp, s);
 }
 
@@ -267,7 +271,10 @@ extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t 
     a.num_cells = num_cells; a.radii = radii; a.max_neighbors = max_neighbors;
     a.counts = counts; a.ends = ends; a.remap = point_remap; a.t = t; a.neigh = neigh_out;
     int64_t waves = pccnn_ceil_div(m, 64);
-    neighbors_kernel<true><<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
+    {
+        PccnnTimed timed(PCCNN_T_NB_FILL, s);
+        neighbors_kernel<true><<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
+    }
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
 }

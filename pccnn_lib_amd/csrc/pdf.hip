@@ -80,6 +80,7 @@ static int pdf_launch(int manifold_dims, const float *bandwidth, const float *pt
     const double norm_const = 1.0 / pow(2.0 * 3.1415, (double)(float)manifold_dims / 2.0);
     const int64_t avg = n > 0 ? t / n : 0;
     const int2 *nb = (const int2 *)neigh;
+    PccnnTimed timed(PCCNN_T_PDF, s);
 #define PDF_GO(G)                                                                                         \
     pdf_kernel<G, GRADS><<<(unsigned)pccnn_ceil_div(n * G, 256), 256, 0, s>>>(norm_const, bandwidth, pts, n, nb, \
                                                                               ends, in_grads, out)

@@ -166,6 +166,7 @@ extern "C" int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int
     int32_t *hist = arena.take<int32_t>((size_t)tiles * 256);
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "pccnn_sort_keys: workspace too small");
 
+    PccnnTimed timed(PCCNN_T_SORT, s);
     const int64_t *src_k = keys;
     const int32_t *src_v = nullptr;
     for (int p = 0; p < passes; ++p) {

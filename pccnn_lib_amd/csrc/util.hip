@@ -16,6 +16,82 @@ void pccnn_set_error(const char *fmt, ...)
 extern "C" const char *pccnn_last_error(void) { return g_err; }
 extern "C" int pccnn_version(void) { return 1; }
 
+// ----------------------------------------------------------------- timing
+
+#include <mutex>
+#include <vector>
+
+static bool g_timing_on = false;
+static std::mutex g_timing_mu;
+struct TimedPair { hipEvent_t start, stop; };
+static std::vector<TimedPair> g_timing_pending[PCCNN_T_COUNT];
+static double g_timing_ms[PCCNN_T_COUNT];
+static long long g_timing_n[PCCNN_T_COUNT];
+static const char *g_timing_names[PCCNN_T_COUNT] = {"gemm", "proj_fwd", "proj_bwd", "basis_bwd", "nb_count",
+                                                    "nb_fill",  "sort",     "keys",     "grid",      "pdf", "scan"};
+
+PccnnTimed::PccnnTimed(int id_, hipStream_t s) : id(id_), stream(s), stop(nullptr), on(g_timing_on)
+{
+    if (!on) return;
+    hipEvent_t start;
+    if (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess) { on = false; return; }
+    hipEventRecord(start, stream);
+    std::lock_guard<std::mutex> lk(g_timing_mu);
+    g_timing_pending[id].push_back({start, stop});
+}
+
+PccnnTimed::~PccnnTimed()
+{
+    if (on) hipEventRecord(stop, stream);
+}
+
+static void timing_drain()
+{
+    for (int i = 0; i < PCCNN_T_COUNT; ++i) {
+        for (auto &pr : g_timing_pending[i]) {
+            float ms = 0.0f;
+            if (hipEventSynchronize(pr.stop) == hipSuccess && hipEventElapsedTime(&ms, pr.start, pr.stop) == hipSuccess) {
+                g_timing_ms[i] += ms;
+                g_timing_n[i] += 1;
+            }
+            hipEventDestroy(pr.start);
+            hipEventDestroy(pr.stop);
+        }
+        g_timing_pending[i].clear();
+    }
+}
+
+extern "C" int pccnn_timing_enable(int on)
+{
+    std::lock_guard<std::mutex> lk(g_timing_mu);
+    timing_drain();
+    g_timing_on = on != 0;
+    return PCCNN_OK;
+}
+
+extern "C" int pccnn_timing_reset(void)
+{
+    std::lock_guard<std::mutex> lk(g_timing_mu);
+    timing_drain();
+    for (int i = 0; i < PCCNN_T_COUNT; ++i) { g_timing_ms[i] = 0.0; g_timing_n[i] = 0; }
+    return PCCNN_OK;
+}
+
+extern "C" int pccnn_timing_count(void) { return PCCNN_T_COUNT; }
+
+extern "C" const char *pccnn_timing_name(int id) { return (id >= 0 && id < PCCNN_T_COUNT) ? g_timing_names[id] : ""; }
+
+extern "C" int pccnn_timing_read(int id, int64_t *h_launches, double *h_total_ms)
+{
+    PCCNN_REQUIRE(id >= 0 && id < PCCNN_T_COUNT && h_launches && h_total_ms, PCCNN_ERR_INVALID,
+                  "pccnn_timing_read: bad timer id %d or null output", id);
+    std::lock_guard<std::mutex> lk(g_timing_mu);
+    timing_drain();
+    *h_launches = g_timing_n[id];
+    *h_total_ms = g_timing_ms[id];
+    return PCCNN_OK;
+}
+
 // ------------------------------------------------------------------ fills
 
 template <typename T> __global__ void fill_kernel(T *p, T v, int64_t n)
