@@ -99,15 +99,24 @@ int pccnn_build_grid_ds(const int64_t *sorted_keys, int64_t n, const int32_t *nu
  * index; inside a sample they are in ascending sorted-point order.
  * Both calls take the same workspace (count leaves per-sample raw counts in it). */
 size_t pccnn_find_neighbors_workspace_bytes(int64_t m);
+/* Optional accelerator for the search (no counterpart in the reference, which binary-searches the sorted
+ * keys inside each pillar, find_ranges_grid_ds.cu:111-163): cell_table_out i32[total_cells + 1], entry c =
+ * index of the first sorted point with key >= c, total_cells = batch_size * prod(num_cells).  When passed to
+ * the two calls below, the range of the three cells a pillar contributes is two table reads; with NULL the
+ * pillar table and a binary search are used.  Same results either way. */
+int pccnn_build_cell_table(const int64_t *sorted_keys, int64_t n, int64_t total_cells, int32_t *cell_table_out,
+                           void *stream);
 int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t *pt_keys_sorted, int64_t n,
                                const float *samples, const int64_t *sample_keys, int64_t m,
                                const int32_t *sample_order, const int32_t *grid_ds, int64_t num_pillars,
+                               const int32_t *cell_table, int64_t total_cells,
                                const int32_t *num_cells, const float *radii, int d, int max_neighbors,
                                int32_t *ends_out,
                                void *workspace, size_t workspace_bytes, void *stream);
 int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t *pt_keys_sorted, int64_t n,
                               const float *samples, const int64_t *sample_keys, int64_t m,
                               const int32_t *sample_order, const int32_t *grid_ds, int64_t num_pillars,
+                              const int32_t *cell_table, int64_t total_cells,
                               const int32_t *num_cells, const float *radii, int d, int max_neighbors,
                               const int32_t *ends,
                               const int32_t *point_remap, int64_t t, int32_t *neigh_out,

@@ -7,7 +7,8 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libpccnn_hip.so")
+# PCCNN_HIP_LIB points at another build of the same library (e.g. an experimental one).
+LIB_PATH = os.environ.get("PCCNN_HIP_LIB") or os.path.join(HERE, "libpccnn_hip.so")
 
 P = ctypes.c_void_p
 I64 = ctypes.c_int64
@@ -25,8 +26,10 @@ SIGNATURES = {
     "pccnn_sort_keys": (I32, [P, I64, I32, P, P, P, I32, P, P, SZ, P]),
     "pccnn_build_grid_ds": (I32, [P, I64, P, I32, I64, P, P]),
     "pccnn_find_neighbors_workspace_bytes": (SZ, [I64]),
-    "pccnn_find_neighbors_count": (I32, [P, P, I64, P, P, I64, P, P, I64, P, P, I32, I32, P, P, SZ, P]),
-    "pccnn_find_neighbors_fill": (I32, [P, P, I64, P, P, I64, P, P, I64, P, P, I32, I32, P, P, I64, P, P, SZ, P]),
+    "pccnn_build_cell_table": (I32, [P, I64, I64, P, P]),
+    "pccnn_find_neighbors_count": (I32, [P, P, I64, P, P, I64, P, P, I64, P, I64, P, P, I32, I32, P, P, SZ, P]),
+    "pccnn_find_neighbors_fill": (I32, [P, P, I64, P, P, I64, P, P, I64, P, I64, P, P, I32, I32, P, P, I64, P, P, SZ,
+                                        P]),
     "pccnn_compute_pdf": (I32, [I32, P, P, I64, I32, P, I64, P, P, P]),
     "pccnn_compute_pdf_grads": (I32, [I32, P, P, I64, I32, P, I64, P, P, P, P]),
     "pccnn_poisson_disk_workspace_bytes": (SZ, [I64]),

@@ -138,186 +138,286 @@ conv_proj_fwd_kernel(ConvGeom g, const float *__restrict__ feats, float *__restr
 
 // ------------------------------------------------------------------------------ backward
 
-// Sum p[k] over the 64 lanes for every k with log-step exchanges that halve the number of
-// live values per lane at each step.  Returns, in every lane, the total for k = *k_out.
-template <int KPAD>
-__device__ __forceinline__ float reduce_scatter(float (&p)[KPAD], int lane, int &k_out)
-{
-    int kidx = 0;
-    int mask = 32;
-#pragma unroll
-    for (int width = KPAD; width > 1; width >>= 1) {
-        const int half = width >> 1;
-        const bool upper = (lane & mask) != 0;
-#pragma unroll
-        for (int j = 0; j < half; ++j) {
-            const float send = upper ? p[j] : p[j + half];
-            const float keep = upper ? p[j + half] : p[j];
-            p[j] = keep + __shfl_xor(send, mask);
-        }
-        if (upper) kidx += half;
-        mask >>= 1;
-    }
-    float v = p[0];
-    for (; mask > 0; mask >>= 1) v += __shfl_xor(v, mask);
-    k_out = kidx;
-    return v;
-}
-
-template <int KPAD> __host__ __device__ constexpr int reduce_scatter_owner_mask()
-{
-    // lanes whose low bits (those not consumed by the halving steps) are zero own the result
-    return KPAD >= 64 ? 0 : (64 / KPAD) - 1;
-}
-
+// Backward of the gather-aggregate for one sample per single-wavefront workgroup.
+//   dF[n_t][f]  += sum_k dP[s][f][k] * w[t][k]        (lane = feature f, dP row in registers)
+//   dw[t][k]     = sum_f dP[s][f][k] * F[n_t][f]      (lane = (k, group of KPAD features), dP column in registers)
+// The basis values of up to 64 pairs are evaluated once (KPAD lanes per pair) and parked in LDS, from where
+// the dF stage reads them as broadcasts; the neighbor's feature row is read coalesced from memory, used by
+// the dF stage from registers and handed to the dw stage through LDS, so that each stage runs KPAD
+// multiply-adds per pair and lane.  dw is accumulated in LDS over the feature blocks and stored coalesced.
 template <int BASIS, int KPAD>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(64)
 conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *__restrict__ proj_grads,
                      float *__restrict__ feat_grads, float *__restrict__ basis_grads)
 {
-    const int lane = pccnn_lane();
-    const int64_t s = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (s >= g.m) return;                                           // wave-uniform
+    constexpr int PARTS = 64 / KPAD;                                // feature groups of the dw stage
+    constexpr int ROWS = 4;                                         // feature rows in flight
+    __shared__ __attribute__((aligned(16))) float w_lds[64][KPAD];
+    __shared__ __attribute__((aligned(16))) float db_lds[64][KPAD];
+    __shared__ __attribute__((aligned(16))) float row_lds[ROWS][64];
+    const int lane = threadIdx.x;
+    const int64_t s = blockIdx.x;
+    const int k = lane % KPAD, part = lane / KPAD;
     const int lo = s > 0 ? g.ends[s - 1] : 0;
     const int hi = g.ends[s];
     const float sx = g.samples[s * 3 + 0], sy = g.samples[s * 3 + 1], sz = g.samples[s * 3 + 2];
     const float ir0 = 1.0f / g.radii[0], ir1 = 1.0f / g.radii[1], ir2 = 1.0f / g.radii[2];
     LaneBasis<BASIS> lb;
-    lb.load(g, lane % KPAD);
+    lb.load(g, k);
     const int fblocks = (g.c_in + 63) / 64;
 
-    for (int fb = 0; fb < fblocks; ++fb) {
-        const int f = fb * 64 + lane;
-        const bool fvalid = f < g.c_in;
-        float gp[KPAD];
+    for (int cb = lo; cb < hi; cb += 64) {
+        const int cnt = (hi - cb) < 64 ? (hi - cb) : 64;
+        int nidx = 0;
+        float dx = 0.f, dy = 0.f, dz = 0.f, pd = 1.0f;
+        if (lane < cnt) {
+            nidx = g.neigh[cb + lane].x;
+            dx = (g.pts[(int64_t)nidx * 3 + 0] - sx) * ir0;
+            dy = (g.pts[(int64_t)nidx * 3 + 1] - sy) * ir1;
+            dz = (g.pts[(int64_t)nidx * 3 + 2] - sz) * ir2;
+            if (BASIS == BASIS_MLP) pd = g.pdf[nidx];
+        }
+        // basis values of the chunk: pass p evaluates pairs p*PARTS .. p*PARTS + PARTS - 1
+        for (int p = 0; p * PARTS < cnt; ++p) {
+            const int j = p * PARTS + part;
+            const float w = lb.eval(__shfl(dx, j), __shfl(dy, j), __shfl(dz, j), __shfl(pd, j), g.sigma);
+            w_lds[j][k] = (j < cnt) ? w : 0.0f;
+            db_lds[j][k] = 0.0f;
+        }
+        __syncthreads();
+        for (int fb = 0; fb < fblocks; ++fb) {
+            const int f = fb * 64 + lane;
+            const bool fvalid = f < g.c_in;
+            float gp[KPAD], gt[KPAD];
 #pragma unroll
-        for (int k = 0; k < KPAD; ++k) gp[k] = 0.0f;
-        if (fvalid) {
-            const float *src = proj_grads + ((int64_t)s * g.c_in + f) * g.k;
-            if (g.k == KPAD && (KPAD % 4) == 0) {
+            for (int q = 0; q < KPAD; ++q) { gp[q] = 0.0f; gt[q] = 0.0f; }
+            if (fvalid) {
+                const float *src = proj_grads + ((int64_t)s * g.c_in + f) * g.k;
+                if (g.k == KPAD && (KPAD % 4) == 0) {
 #pragma unroll
-                for (int k = 0; k < KPAD; k += 4) {
-                    const float4 v = *(const float4 *)(src + k);
-                    gp[k] = v.x; gp[k + 1] = v.y; gp[k + 2] = v.z; gp[k + 3] = v.w;
+                    for (int q = 0; q < KPAD; q += 4) {
+                        const float4 v = *(const float4 *)(src + q);
+                        gp[q] = v.x; gp[q + 1] = v.y; gp[q + 2] = v.z; gp[q + 3] = v.w;
+                    }
+                } else {
+#pragma unroll
+                    for (int q = 0; q < KPAD; ++q)
+                        if (q < g.k) gp[q] = src[q];
                 }
-            } else {
+            }
+            if (k < g.k) {
 #pragma unroll
-                for (int k = 0; k < KPAD; ++k)
-                    if (k < g.k) gp[k] = src[k];
+                for (int q = 0; q < KPAD; ++q) {
+                    const int ft = fb * 64 + part * KPAD + q;
+                    if (ft < g.c_in) gt[q] = proj_grads[((int64_t)s * g.c_in + ft) * g.k + k];
+                }
+            }
+            for (int j0 = 0; j0 < cnt; j0 += ROWS) {
+                float row[ROWS];
+                int bn[ROWS];
+#pragma unroll
+                for (int u = 0; u < ROWS; ++u) {
+                    bn[u] = pccnn_bcast_i(nidx, (j0 + u) < cnt ? (j0 + u) : 0);
+                    row[u] = (fvalid && (j0 + u) < cnt) ? feats[(int64_t)bn[u] * g.c_in + f] : 0.0f;
+                }
+#pragma unroll
+                for (int u = 0; u < ROWS; ++u) row_lds[u][lane] = row[u];
+                __syncthreads();
+#pragma unroll
+                for (int u = 0; u < ROWS; ++u) {
+                    const int j = j0 + u;
+                    if (j < cnt) {                                  // uniform
+                        float gf = 0.0f, acc = 0.0f;
+#pragma unroll
+                        for (int q = 0; q < KPAD; q += 4) {
+                            const float4 wv = *(const float4 *)&w_lds[j][q];
+                            gf += gp[q] * wv.x + gp[q + 1] * wv.y + gp[q + 2] * wv.z + gp[q + 3] * wv.w;
+                            const float4 rv = *(const float4 *)&row_lds[u][part * KPAD + q];
+                            acc += gt[q] * rv.x + gt[q + 1] * rv.y + gt[q + 2] * rv.z + gt[q + 3] * rv.w;
+                        }
+                        if (fvalid) unsafeAtomicAdd(&feat_grads[(int64_t)bn[u] * g.c_in + f], gf);
+#pragma unroll
+                        for (int o = KPAD; o < 64; o <<= 1) acc += __shfl_xor(acc, o);
+                        if (part == 0) db_lds[j][k] += acc;
+                    }
+                }
+                __syncthreads();
             }
         }
-        for (int cb = lo; cb < hi; cb += 64) {
-            const int t = cb + lane;
-            int nidx = 0;
-            float dx = 0.f, dy = 0.f, dz = 0.f, pd = 1.0f;
-            if (t < hi) {
-                nidx = g.neigh[t].x;
-                dx = (g.pts[(int64_t)nidx * 3 + 0] - sx) * ir0;
-                dy = (g.pts[(int64_t)nidx * 3 + 1] - sy) * ir1;
-                dz = (g.pts[(int64_t)nidx * 3 + 2] - sz) * ir2;
-                if (BASIS == BASIS_MLP) pd = g.pdf[nidx];
-            }
-            const int cnt = (hi - cb) < 64 ? (hi - cb) : 64;
-            for (int j = 0; j < cnt; ++j) {
-                const int bn = pccnn_bcast_i(nidx, j);
-                const float row = fvalid ? feats[(int64_t)bn * g.c_in + f] : 0.0f;
-                const float wv = lb.eval(pccnn_bcast_f(dx, j), pccnn_bcast_f(dy, j), pccnn_bcast_f(dz, j),
-                                         pccnn_bcast_f(pd, j), g.sigma);
-                float gf = 0.0f;
-                float pk[KPAD];
-#pragma unroll
-                for (int k = 0; k < KPAD; ++k) {
-                    gf += gp[k] * __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wv), k));
-                    pk[k] = gp[k] * row;
-                }
-                if (fvalid) unsafeAtomicAdd(&feat_grads[(int64_t)bn * g.c_in + f], gf);
-                int kk;
-                const float tot = reduce_scatter<KPAD>(pk, lane, kk);
-                if ((lane & reduce_scatter_owner_mask<KPAD>()) == 0 && kk < g.k) {
-                    float *dst = basis_grads + (int64_t)(cb + j) * g.k + kk;
-                    *dst = (fb == 0) ? tot : (*dst + tot);
-                }
-            }
+        __syncthreads();
+        for (int idx = lane; idx < cnt * KPAD; idx += 64) {
+            const int j = idx / KPAD, kk = idx % KPAD;
+            if (kk < g.k) basis_grads[(int64_t)(cb + j) * g.k + kk] = db_lds[j][kk];
         }
+        __syncthreads();
     }
 }
 
-// One thread per pair: derivative of the basis w.r.t. its inputs and parameters.
-// param_grads: KP -> d_kernel_pts [K,3];  MLP -> d_axis [3,K] followed by d_bias [K].
-template <int BASIS>
+// Derivative of the basis w.r.t. its inputs and parameters, one wavefront per sample.
+// KPAD lanes own one pair (lane = basis index k), so 64 / KPAD pairs are handled per step and BB_UNROLL
+// steps are in flight at once (their loads are independent).  Per-pair basis gradients are one coalesced
+// read; the offset / density gradients are reduced across the KPAD lanes with shuffles; the point and
+// density gradients are scattered with one float atomic per pair and coordinate, the sample's own gradient
+// is accumulated in registers and stored once.  Every lane keeps the parameter gradients of its own k in
+// registers; a workgroup reduces them in LDS and stores one partial row that conv_param_reduce_kernel sums
+// in a fixed order.  param layout: KP -> d_kernel_pts [K,3];  MLP -> d_axis [3,K] followed by d_bias [K].
+#define BB_UNROLL 4
+
+template <int BASIS, int KPAD>
 __global__ void __launch_bounds__(256)
 conv_basis_bwd_kernel(ConvGeom g, const float *__restrict__ basis_grads, float *__restrict__ d_pts,
-                      float *__restrict__ d_samples, float *__restrict__ d_pdf, float *__restrict__ param_grads)
+                      float *__restrict__ d_samples, float *__restrict__ d_pdf, float *__restrict__ param_partials)
 {
     // The KPConv correlation has a kink where a pair sits exactly one sigma away from a kernel
     // point, and every self pair (offset 0) does so for the kernel points closest to the centre.
     // Which side of the kink such a pair falls on is decided by the last bit of the fp32
     // distance, so the distance is evaluated exactly as written: no fused multiply-add.
 #pragma clang fp contract(off)
-    extern __shared__ float lds_param[];                            // 4*K floats
-    const int nparam = (BASIS == BASIS_KP ? 3 : 4) * g.k;
-    for (int i = threadIdx.x; i < nparam; i += blockDim.x) lds_param[i] = 0.0f;
-    __syncthreads();
+    __shared__ float lds_param[4][4 * 64];
+    constexpr int PAIRS = 64 / KPAD;                                // pairs per step
+    const int lane = pccnn_lane();
+    const int wave = threadIdx.x >> 6;
+    const int k = lane % KPAD;
+    const int sub = lane / KPAD;
+    const bool kvalid = k < g.k;
+    const int64_t s = (int64_t)blockIdx.x * 4 + wave;
+    const bool svalid = s < g.m;
     const float ir0 = 1.0f / g.radii[0], ir1 = 1.0f / g.radii[1], ir2 = 1.0f / g.radii[2];
-    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < g.t; t += (int64_t)gridDim.x * blockDim.x) {
-        const int2 pr = g.neigh[t];
-        const float dx = (g.pts[(int64_t)pr.x * 3 + 0] - g.samples[(int64_t)pr.y * 3 + 0]) * ir0;
-        const float dy = (g.pts[(int64_t)pr.x * 3 + 1] - g.samples[(int64_t)pr.y * 3 + 1]) * ir1;
-        const float dz = (g.pts[(int64_t)pr.x * 3 + 2] - g.samples[(int64_t)pr.y * 3 + 2]) * ir2;
-        float gx = 0.f, gy = 0.f, gz = 0.f, gpdf = 0.f;
-        const float *gb = basis_grads + t * g.k;
+    float c0 = 0.f, c1 = 0.f, c2 = 0.f, c3 = 0.f;                   // this lane's basis parameters
+    if (kvalid) {
         if (BASIS == BASIS_KP) {
-            for (int k = 0; k < g.k; ++k) {
-                const float vx = g.basis_a[k * 3 + 0] - dx, vy = g.basis_a[k * 3 + 1] - dy,
-                            vz = g.basis_a[k * 3 + 2] - dz;
-                const float dist = sqrtf(fmaxf(vx * vx + vy * vy + vz * vz, 0.0f));
-                const float res = 1.0f - dist / g.sigma;
-                if (res >= 0.0f) {
-                    const float c = -(gb[k] / g.sigma) * (1.0f / (dist + 1e-6f));
-                    const float cx = c * vx, cy = c * vy, cz = c * vz;
-                    gx -= cx; gy -= cy; gz -= cz;
-                    atomicAdd(&lds_param[k * 3 + 0], cx);
-                    atomicAdd(&lds_param[k * 3 + 1], cy);
-                    atomicAdd(&lds_param[k * 3 + 2], cz);
+            c0 = g.basis_a[k * 3 + 0]; c1 = g.basis_a[k * 3 + 1]; c2 = g.basis_a[k * 3 + 2];
+        } else {
+            c0 = g.basis_a[k]; c1 = g.basis_a[g.k + k]; c2 = g.basis_a[2 * g.k + k]; c3 = g.basis_b[k];
+        }
+    }
+    float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;                   // parameter gradient sums of this lane's k
+    float sgx = 0.f, sgy = 0.f, sgz = 0.f;                          // the sample's own gradient (before the sign)
+    int lo = 0, hi = 0;
+    float sx = 0.f, sy = 0.f, sz = 0.f;
+    if (svalid) {
+        lo = s > 0 ? g.ends[s - 1] : 0;
+        hi = g.ends[s];
+        sx = g.samples[s * 3 + 0]; sy = g.samples[s * 3 + 1]; sz = g.samples[s * 3 + 2];
+    }
+    for (int base = lo; base < hi; base += PAIRS * BB_UNROLL) {
+        int nidx[BB_UNROLL];
+        float px[BB_UNROLL], py[BB_UNROLL], pz[BB_UNROLL], pdv[BB_UNROLL], gk[BB_UNROLL];
+        bool tv[BB_UNROLL];
+#pragma unroll
+        for (int u = 0; u < BB_UNROLL; ++u) {
+            const int t = base + u * PAIRS + sub;
+            tv[u] = t < hi;
+            nidx[u] = tv[u] ? g.neigh[t].x : 0;
+            gk[u] = (tv[u] && kvalid) ? basis_grads[(int64_t)t * g.k + k] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < BB_UNROLL; ++u) {
+            px[u] = g.pts[(int64_t)nidx[u] * 3 + 0];
+            py[u] = g.pts[(int64_t)nidx[u] * 3 + 1];
+            pz[u] = g.pts[(int64_t)nidx[u] * 3 + 2];
+            pdv[u] = (BASIS == BASIS_MLP) ? g.pdf[nidx[u]] : 1.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < BB_UNROLL; ++u) {
+            float gx = 0.f, gy = 0.f, gz = 0.f, gpdf = 0.f;
+            if (tv[u] && kvalid) {
+                const float dx = (px[u] - sx) * ir0, dy = (py[u] - sy) * ir1, dz = (pz[u] - sz) * ir2;
+                if (BASIS == BASIS_KP) {
+                    const float vx = c0 - dx, vy = c1 - dy, vz = c2 - dz;
+                    const float dist = sqrtf(fmaxf(vx * vx + vy * vy + vz * vz, 0.0f));
+                    const float res = 1.0f - dist / g.sigma;
+                    if (res >= 0.0f) {
+                        const float c = -(gk[u] / g.sigma) * (1.0f / (dist + 1e-6f));
+                        const float cx = c * vx, cy = c * vy, cz = c * vz;
+                        gx = -cx; gy = -cy; gz = -cz;
+                        p0 += cx; p1 += cy; p2 += cz;
+                    }
+                } else {
+                    const float inv_pd = 1.0f / pdv[u];
+                    float act = dx * c0 + dy * c1 + dz * c2 + c3;
+                    const bool pos = act > 0.0f;
+                    act = pos ? act : act * 0.2f;
+                    gpdf = -(act * gk[u] * inv_pd * inv_pd);
+                    const float c = gk[u] * inv_pd * (pos ? 1.0f : 0.2f);
+                    gx = c * c0; gy = c * c1; gz = c * c2;
+                    p0 += dx * c; p1 += dy * c; p2 += dz * c; p3 += c;
                 }
             }
-        } else {
-            const float pd = g.pdf[pr.x];
-            const float inv_pd = 1.0f / pd;
-            for (int k = 0; k < g.k; ++k) {
-                const float a0 = g.basis_a[k], a1 = g.basis_a[g.k + k], a2 = g.basis_a[2 * g.k + k];
-                float act = dx * a0 + dy * a1 + dz * a2 + g.basis_b[k];
-                const bool pos = act > 0.0f;
-                act = pos ? act : act * 0.2f;
-                const float gk = gb[k];
-                gpdf -= act * gk * inv_pd * inv_pd;
-                const float c = gk * inv_pd * (pos ? 1.0f : 0.2f);
-                gx += c * a0; gy += c * a1; gz += c * a2;
-                atomicAdd(&lds_param[k], dx * c);
-                atomicAdd(&lds_param[g.k + k], dy * c);
-                atomicAdd(&lds_param[2 * g.k + k], dz * c);
-                atomicAdd(&lds_param[3 * g.k + k], c);
+#pragma unroll
+            for (int o = KPAD / 2; o > 0; o >>= 1) {
+                gx += __shfl_xor(gx, o);
+                gy += __shfl_xor(gy, o);
+                gz += __shfl_xor(gz, o);
+                if (BASIS == BASIS_MLP) gpdf += __shfl_xor(gpdf, o);
             }
-            unsafeAtomicAdd(&d_pdf[pr.x], gpdf);
+            if (tv[u] && k == 0) {
+                gx *= ir0; gy *= ir1; gz *= ir2;
+                unsafeAtomicAdd(&d_pts[(int64_t)nidx[u] * 3 + 0], gx);
+                unsafeAtomicAdd(&d_pts[(int64_t)nidx[u] * 3 + 1], gy);
+                unsafeAtomicAdd(&d_pts[(int64_t)nidx[u] * 3 + 2], gz);
+                if (BASIS == BASIS_MLP) unsafeAtomicAdd(&d_pdf[nidx[u]], gpdf);
+                sgx += gx; sgy += gy; sgz += gz;
+            }
         }
-        gx *= ir0; gy *= ir1; gz *= ir2;
-        unsafeAtomicAdd(&d_pts[(int64_t)pr.x * 3 + 0], gx);
-        unsafeAtomicAdd(&d_pts[(int64_t)pr.x * 3 + 1], gy);
-        unsafeAtomicAdd(&d_pts[(int64_t)pr.x * 3 + 2], gz);
-        unsafeAtomicAdd(&d_samples[(int64_t)pr.y * 3 + 0], -gx);
-        unsafeAtomicAdd(&d_samples[(int64_t)pr.y * 3 + 1], -gy);
-        unsafeAtomicAdd(&d_samples[(int64_t)pr.y * 3 + 2], -gz);
+    }
+    // the sample's gradient: sum over the lanes that own a pair (k == 0 of every sub-group)
+#pragma unroll
+    for (int o = KPAD; o < 64; o <<= 1) {
+        sgx += __shfl_xor(sgx, o);
+        sgy += __shfl_xor(sgy, o);
+        sgz += __shfl_xor(sgz, o);
+        p0 += __shfl_xor(p0, o);
+        p1 += __shfl_xor(p1, o);
+        p2 += __shfl_xor(p2, o);
+        p3 += __shfl_xor(p3, o);
+    }
+    if (svalid && lane == 0) {
+        d_samples[s * 3 + 0] = -sgx;
+        d_samples[s * 3 + 1] = -sgy;
+        d_samples[s * 3 + 2] = -sgz;
+    }
+    if (sub == 0) {
+        lds_param[wave][k] = p0;
+        lds_param[wave][64 + k] = p1;
+        lds_param[wave][128 + k] = p2;
+        lds_param[wave][192 + k] = p3;
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < nparam; i += blockDim.x) unsafeAtomicAdd(&param_grads[i], lds_param[i]);
+    // one partial row of 4 * 64 floats per workgroup: [component][k]
+    const int i = threadIdx.x;
+    const int comp = i >> 6, kk = i & 63;
+    float v = 0.0f;
+    if (kk < KPAD) v = lds_param[0][comp * 64 + kk] + lds_param[1][comp * 64 + kk] + lds_param[2][comp * 64 + kk] +
+                       lds_param[3][comp * 64 + kk];
+    param_partials[(int64_t)blockIdx.x * 256 + i] = v;
 }
 
-__global__ void copy_params_kernel(const float *__restrict__ src, float *__restrict__ dst_a, int count_a,
-                                   float *__restrict__ dst_b, int count_b)
+// Sums the per-workgroup partial rows ([rows][4][64]) in a fixed order; block b handles component b / 64,
+// basis index b % 64 and writes it to its place in the parameter gradient tensors.
+template <int BASIS>
+__global__ void __launch_bounds__(256)
+conv_param_reduce_kernel(const float *__restrict__ partials, int64_t rows, int k_basis, float *__restrict__ dst_a,
+                         float *__restrict__ dst_b)
 {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < count_a) dst_a[i] = src[i];
-    else if (i < count_a + count_b) dst_b[i - count_a] = src[i];
+    __shared__ float red[256];
+    const int comp = blockIdx.x >> 6, kk = blockIdx.x & 63;
+    float acc = 0.0f;
+    for (int64_t r = threadIdx.x; r < rows; r += 256) acc += partials[r * 256 + blockIdx.x];
+    red[threadIdx.x] = acc;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if (threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0 && kk < k_basis) {
+        if (BASIS == BASIS_KP) {
+            if (comp < 3) dst_a[kk * 3 + comp] = red[0];            // d_kernel_pts [K,3]
+        } else {
+            if (comp < 3) dst_a[comp * k_basis + kk] = red[0];      // d_axis [3,K]
+            else dst_b[kk] = red[0];                                // d_bias [K]
+        }
+    }
 }
 
 // ------------------------------------------------------------------------------- host side
@@ -343,13 +443,13 @@ template <int BASIS>
 static int launch_proj_bwd(const ConvGeom &g, const float *feats, const float *proj_grads, float *feat_grads,
                            float *basis_grads, hipStream_t s)
 {
-    dim3 grid((unsigned)pccnn_ceil_div(g.m, 4));
+    dim3 grid((unsigned)g.m);
     PccnnTimed timed(PCCNN_T_PROJ_BWD, s);
     switch (kpad_of(g.k)) {
-    case 8: conv_proj_bwd_kernel<BASIS, 8><<<grid, 256, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads); break;
-    case 16: conv_proj_bwd_kernel<BASIS, 16><<<grid, 256, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads); break;
-    case 32: conv_proj_bwd_kernel<BASIS, 32><<<grid, 256, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads); break;
-    default: conv_proj_bwd_kernel<BASIS, 64><<<grid, 256, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads); break;
+    case 8: conv_proj_bwd_kernel<BASIS, 8><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads); break;
+    case 16: conv_proj_bwd_kernel<BASIS, 16><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads); break;
+    case 32: conv_proj_bwd_kernel<BASIS, 32><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads); break;
+    default: conv_proj_bwd_kernel<BASIS, 64><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads); break;
     }
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
@@ -379,7 +479,8 @@ extern "C" size_t pccnn_conv_workspace_bytes(int64_t m, int64_t t, int c_in, int
     if (!backward) return proj + 256;
     size_t basis_g = pccnn_align((size_t)t * k * sizeof(float));
     size_t splitk = pccnn_align((size_t)CONV_SPLIT_K * c_in * k * c_out * sizeof(float));
-    return 2 * proj + basis_g + splitk + pccnn_align(4 * 64 * sizeof(float)) + 256;
+    size_t partials = pccnn_align((size_t)pccnn_ceil_div(m, 4) * 256 * sizeof(float));
+    return 2 * proj + basis_g + splitk + partials + 256;
 }
 
 // out[m, c_out] = P[m, c_in*k] x W, with the feature axis split over num_mlps independent
@@ -430,18 +531,17 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
 {
     // d_param_a: d_kernel_pts [K,3] (KP) or d_axis [3,K] (MLP); d_param_b: d_bias [K] (MLP only)
     const int count_a = 3 * g.k, count_b = (BASIS == BASIS_KP ? 0 : g.k);
-    const int nparam = count_a + count_b;
     int rc;
     PccnnArena arena(workspace, workspace_bytes);
-    float *d_param = arena.take<float>(4 * 64);
+    const int64_t partial_rows = pccnn_ceil_div(g.m > 0 ? g.m : 1, 4);
+    float *partials = arena.take<float>((size_t)partial_rows * 256);
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv backward: workspace of %zu bytes, need %zu", workspace_bytes,
                   pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 1));
     if ((rc = pccnn_fill_f32(d_feats, 0.0f, g.n * g.c_in, s)) != PCCNN_OK) return rc;
     if ((rc = pccnn_fill_f32(d_pts, 0.0f, g.n * 3, s)) != PCCNN_OK) return rc;
-    if ((rc = pccnn_fill_f32(d_samples, 0.0f, g.m * 3, s)) != PCCNN_OK) return rc;
-    if ((rc = pccnn_fill_f32(d_param, 0.0f, nparam, s)) != PCCNN_OK) return rc;
     if (d_pdf && (rc = pccnn_fill_f32(d_pdf, 0.0f, g.n, s)) != PCCNN_OK) return rc;
     if (g.m == 0 || g.t == 0) {
+        if ((rc = pccnn_fill_f32(d_samples, 0.0f, g.m * 3, s)) != PCCNN_OK) return rc;
         if ((rc = pccnn_fill_f32(d_param_a, 0.0f, count_a, s)) != PCCNN_OK) return rc;
         if (count_b && (rc = pccnn_fill_f32(d_param_b, 0.0f, count_b, s)) != PCCNN_OK) return rc;
         return pccnn_fill_f32(d_weights, 0.0f, (int64_t)g.c_in * g.k * c_out / num_mlps, s);
@@ -459,15 +559,18 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
                               splitk_elems * sizeof(float), s)) != PCCNN_OK)
         return rc;
     if ((rc = launch_proj_bwd<BASIS>(g, feats, d_proj, d_feats, basis_g, s)) != PCCNN_OK) return rc;
-    int64_t blocks = pccnn_ceil_div(g.t, 256);
-    if (blocks > 2048) blocks = 2048;
+    const unsigned blocks = (unsigned)partial_rows;
     {
         PccnnTimed timed(PCCNN_T_BASIS_BWD, s);
-        conv_basis_bwd_kernel<BASIS><<<(unsigned)blocks, 256, 4 * g.k * sizeof(float), s>>>(g, basis_g, d_pts, d_samples,
-                                                                                            d_pdf, d_param);
+        switch (kpad_of(g.k)) {
+        case 8: conv_basis_bwd_kernel<BASIS, 8><<<blocks, 256, 0, s>>>(g, basis_g, d_pts, d_samples, d_pdf, partials); break;
+        case 16: conv_basis_bwd_kernel<BASIS, 16><<<blocks, 256, 0, s>>>(g, basis_g, d_pts, d_samples, d_pdf, partials); break;
+        case 32: conv_basis_bwd_kernel<BASIS, 32><<<blocks, 256, 0, s>>>(g, basis_g, d_pts, d_samples, d_pdf, partials); break;
+        default: conv_basis_bwd_kernel<BASIS, 64><<<blocks, 256, 0, s>>>(g, basis_g, d_pts, d_samples, d_pdf, partials); break;
+        }
     }
     PCCNN_LAUNCH_CHECK();
-    copy_params_kernel<<<1, 256, 0, s>>>(d_param, d_param_a, count_a, d_param_b, count_b);
+    conv_param_reduce_kernel<BASIS><<<256, 256, 0, s>>>(partials, partial_rows, g.k, d_param_a, d_param_b);
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
 }

@@ -26,42 +26,88 @@ __global__ void bbox_init_kernel(float *mn, float *mx, int count)
     if (i < count) { mn[i] = __int_as_float(0x7f800000); mx[i] = __int_as_float(0xff800000); }
 }
 
+// Grid-stride reduction.  Every thread keeps a running box for the cloud it is currently in and flushes it
+// with atomics only when the cloud id changes (clouds are normally stored one after the other); at the end a
+// wavefront whose lanes all hold the same cloud reduces with shuffles, and a workgroup whose four wavefronts
+// agree combines them in LDS, so a launch issues a few hundred atomics per box corner at most.
 template <int D>
 __global__ void __launch_bounds__(256)
-bbox_reduce_kernel(const float *__restrict__ pts, const int32_t *__restrict__ batch_ids, int64_t n,
+bbox_reduce_kernel(const float *__restrict__ pts, const int32_t *__restrict__ batch_ids, int64_t n, int batch_size,
                    float *mn, float *mx)
 {
-    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    bool valid = i < n;
-    int b = valid ? batch_ids[i] : -1;
-    float p[D];
+    __shared__ float lds_lo[4][D], lds_hi[4][D];
+    __shared__ int lds_b[4];
+    const float inf = __int_as_float(0x7f800000);
+    int cur = -1;
+    float lo[D], hi[D];
 #pragma unroll
-    for (int k = 0; k < D; ++k) p[k] = valid ? pts[i * D + k] : 0.0f;
-    // When every active lane of the wave belongs to one cloud, reduce in registers and
-    // issue one atomic per wave and coordinate.
-    int b0 = __builtin_amdgcn_readfirstlane(b);
-    unsigned long long vmask = __ballot(valid);
-    bool uniform = (vmask != 0ull) && (__ballot(valid && b == b0) == vmask) && (b0 >= 0);
-    if (uniform) {
+    for (int k = 0; k < D; ++k) { lo[k] = inf; hi[k] = -inf; }
+    // a workgroup owns one contiguous chunk of the point list, so it rarely sees more than one cloud
+    const int64_t chunk = (n + gridDim.x - 1) / gridDim.x;
+    const int64_t chunk_end = ((int64_t)blockIdx.x + 1) * chunk < n ? ((int64_t)blockIdx.x + 1) * chunk : n;
+    for (int64_t i = (int64_t)blockIdx.x * chunk + threadIdx.x; i < chunk_end; i += blockDim.x) {
+        const int b = batch_ids[i];
+        if (b < 0 || b >= batch_size) continue;                       // ids outside the table are ignored
+        if (b != cur) {
+            if (cur >= 0) {
+#pragma unroll
+                for (int k = 0; k < D; ++k) {
+                    atomic_min_f32(&mn[cur * D + k], lo[k]);
+                    atomic_max_f32(&mx[cur * D + k], hi[k]);
+                    lo[k] = inf; hi[k] = -inf;
+                }
+            }
+            cur = b;
+        }
 #pragma unroll
         for (int k = 0; k < D; ++k) {
-            float lo = valid ? p[k] : __int_as_float(0x7f800000);
-            float hi = valid ? p[k] : __int_as_float(0xff800000);
+            const float v = pts[i * D + k];
+            lo[k] = fminf(lo[k], v);
+            hi[k] = fmaxf(hi[k], v);
+        }
+    }
+    const int lane = pccnn_lane(), wave = threadIdx.x >> 6;
+    const unsigned long long have = __ballot(cur >= 0);
+    const int b0 = have ? pccnn_bcast_i(cur, __builtin_ctzll(have)) : -1;
+    const bool wave_uniform = __ballot(cur >= 0 && cur != b0) == 0ull;     // idle lanes hold the neutral box
+    if (wave_uniform) {
+#pragma unroll
+        for (int k = 0; k < D; ++k) {
 #pragma unroll
             for (int o = 32; o > 0; o >>= 1) {
-                lo = fminf(lo, __shfl_xor(lo, o));
-                hi = fmaxf(hi, __shfl_xor(hi, o));
-            }
-            if (pccnn_lane() == 0) {
-                atomic_min_f32(&mn[b0 * D + k], lo);
-                atomic_max_f32(&mx[b0 * D + k], hi);
+                lo[k] = fminf(lo[k], __shfl_xor(lo[k], o));
+                hi[k] = fmaxf(hi[k], __shfl_xor(hi[k], o));
             }
         }
-    } else if (valid) {
+        if (lane == 0) {
+            lds_b[wave] = b0;
 #pragma unroll
-        for (int k = 0; k < D; ++k) {
-            atomic_min_f32(&mn[b * D + k], p[k]);
-            atomic_max_f32(&mx[b * D + k], p[k]);
+            for (int k = 0; k < D; ++k) { lds_lo[wave][k] = lo[k]; lds_hi[wave][k] = hi[k]; }
+        }
+    } else {
+        if (lane == 0) lds_b[wave] = -2;                              // handled below, per lane
+        if (cur >= 0) {
+#pragma unroll
+            for (int k = 0; k < D; ++k) {
+                atomic_min_f32(&mn[cur * D + k], lo[k]);
+                atomic_max_f32(&mx[cur * D + k], hi[k]);
+            }
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const bool same = lds_b[0] == lds_b[1] && lds_b[0] == lds_b[2] && lds_b[0] == lds_b[3];
+        for (int w = 0; w < 4; ++w) {
+            const int b = lds_b[w];
+            if (b < 0) continue;
+            if (same && w > 0) break;
+            for (int k = 0; k < D; ++k) {
+                float l = lds_lo[w][k], h = lds_hi[w][k];
+                if (same)
+                    for (int w2 = 1; w2 < 4; ++w2) { l = fminf(l, lds_lo[w2][k]); h = fmaxf(h, lds_hi[w2][k]); }
+                atomic_min_f32(&mn[b * D + k], l);
+                atomic_max_f32(&mx[b * D + k], h);
+            }
         }
     }
 }
@@ -85,8 +131,10 @@ extern "C" int pccnn_bounding_box(const float *pts, const int32_t *batch_ids, in
     bbox_init_kernel<<<(unsigned)pccnn_ceil_div(count, 256), 256, 0, s>>>(aabb_min_out, aabb_max_out, count);
     PCCNN_LAUNCH_CHECK();
     if (n > 0) {
-        bbox_reduce_kernel<3><<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(pts, batch_ids, n, aabb_min_out,
-                                                                             aabb_max_out);
+        int64_t blocks = pccnn_ceil_div(n, 256 * 8);
+        if (blocks > 256) blocks = 256;
+        bbox_reduce_kernel<3><<<(unsigned)blocks, 256, 0, s>>>(pts, batch_ids, n, batch_size, aabb_min_out,
+                                                               aabb_max_out);
         PCCNN_LAUNCH_CHECK();
     }
     bbox_pad_kernel<<<(unsigned)pccnn_ceil_div(count, 256), 256, 0, s>>>(aabb_min_out, aabb_max_out, count);

@@ -24,6 +24,8 @@ struct NbArgs {
     const int32_t *order;      // nullable
     const int32_t *grid_ds;    // [num_pillars,2]
     int64_t num_pillars;
+    const int32_t *cell_table; // nullable: [total_cells + 1] first sorted index of every cell
+    int64_t total_cells;
     const int32_t *num_cells;  // [3]
     const float *radii;        // [3]
     int max_neighbors;
@@ -100,15 +102,24 @@ neighbors_kernel(NbArgs a)
             const int x = c0 + dx, y = c1 + dy;
             if (x >= 0 && x < nc0 && y >= 0 && y < nc1) {
                 const long long pillar = pil + (long long)dx * nc1 + dy;
-                if (pillar >= 0 && pillar < a.num_pillars) {
+                const int cmin = c2 > 0 ? c2 - 1 : 0, cmax = c2 + 1 < nc2 ? c2 + 1 : nc2 - 1;
+                if (a.cell_table) {
+                    // cells cmin..cmax of the pillar are consecutive keys: two table reads give their range
+                    const long long kbase = pillar * nc2;
+                    if (pillar >= 0 && kbase + cmax + 1 <= a.total_cells) {
+                        first = a.cell_table[kbase + cmin];
+                        len = a.cell_table[kbase + cmax + 1] - first;
+                        if (first < 0 || len < 0 || (int64_t)first + len > a.n) len = 0;
+                    }
+                } else if (pillar >= 0 && pillar < a.num_pillars) {
                     int lo = a.grid_ds[2 * pillar], hi = a.grid_ds[2 * pillar + 1];
                     lo = lo < 0 ? 0 : lo;
                     hi = hi > a.n ? (int)a.n : hi;
                     if (hi > lo) {
                         // keys of the cells c2-1 .. c2+1 of this pillar
                         const long long kbase = pillar * nc2;
-                        const long long kmin = kbase + (c2 > 0 ? c2 - 1 : 0);
-                        const long long kmax = kbase + (c2 + 1 < nc2 ? c2 + 1 : nc2 - 1);
+                        const long long kmin = kbase + cmin;
+                        const long long kmax = kbase + cmax;
                         int lb = lo, ub = hi;
                         while (lb < ub) {
                             int mid = (lb + ub) >> 1;
@@ -153,12 +164,14 @@ neighbors_kernel(NbArgs a)
 
             for (int q = h; q < e; ++q) {
                 const float qx = pccnn_bcast_f(sx, q), qy = pccnn_bcast_f(sy, q), qz = pccnn_bcast_f(sz, q);
-                // fp32, no contraction: ((s - p) * (1/r)) squared, summed x, y, z, sqrt, < 1
+                // fp32, no contraction: ((s - p) * (1/r)) squared, summed x, y, z; the reference tests
+                // sqrt(acc) < 1, which for a correctly rounded fp32 sqrt holds exactly when acc < 1
+                // (the largest float below 1 has a root below the midpoint to 1, so it rounds down).
                 const float vx = (qx - px) * ir0;
                 const float vy = (qy - py) * ir1;
                 const float vz = (qz - pz) * ir2;
                 const float acc = ((0.0f + vx * vx) + vy * vy) + vz * vz;
-                const bool hit = cvalid && (__fsqrt_rn(acc) < 1.0f);
+                const bool hit = cvalid && (acc < 1.0f);
                 const unsigned long long bal = __ballot(hit);
                 const int c = __popcll(bal);
                 if (FILL) {
@@ -190,6 +203,42 @@ neighbors_kernel(NbArgs a)
     if (!FILL && valid) a.counts[s] = my_cnt;
 }
 
+// table[c] = index of the first sorted point whose key is >= c, for c in [0, total_cells]; the thread of
+// every point that starts a new key fills the entries between the previous key and its own.
+__global__ void __launch_bounds__(256)
+cell_table_kernel(const int64_t *__restrict__ keys, int64_t n, int64_t total_cells, int32_t *__restrict__ table)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i > n) return;
+    long long from, to;                                             // table[from..to] = i
+    if (i == n) {
+        from = (n > 0 ? keys[n - 1] + 1 : 0);
+        to = total_cells;
+    } else {
+        const long long key = keys[i];
+        const long long prev = i > 0 ? keys[i - 1] : -1;
+        if (key == prev) return;
+        from = prev + 1;
+        to = key;
+    }
+    if (from < 0) from = 0;
+    if (to > total_cells) to = total_cells;
+    for (long long c = from; c <= to; ++c) table[c] = (int32_t)i;
+}
+
+extern "C" int pccnn_build_cell_table(const int64_t *sorted_keys, int64_t n, int64_t total_cells,
+                                      int32_t *cell_table_out, void *stream)
+{
+    PCCNN_REQUIRE(n >= 0 && n < (1ll << 31) && total_cells > 0 && total_cells < (1ll << 40), PCCNN_ERR_INVALID,
+                  "pccnn_build_cell_table: n=%lld total_cells=%lld", (long long)n, (long long)total_cells);
+    PCCNN_REQUIRE(cell_table_out && (n == 0 || sorted_keys), PCCNN_ERR_INVALID, "pccnn_build_cell_table: null pointer");
+    PccnnTimed timed(PCCNN_T_GRID, (hipStream_t)stream);
+    cell_table_kernel<<<(unsigned)pccnn_ceil_div(n + 1, 256), 256, 0, (hipStream_t)stream>>>(sorted_keys, n, total_cells,
+                                                                                          cell_table_out);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
 extern "C" size_t pccnn_find_neighbors_workspace_bytes(int64_t m)
 {
     if (m < 1) m = 1;
@@ -198,7 +247,7 @@ extern "C" size_t pccnn_find_neighbors_workspace_bytes(int64_t m)
 
 static int nb_validate(const char *who, const float *pts_sorted, const int64_t *pt_keys_sorted, int64_t n,
                        const float *samples, const int64_t *sample_keys, int64_t m, const int32_t *grid_ds,
-                       int64_t num_pillars, const int32_t *num_cells, const float *radii, int d, int max_neighbors, void *workspace,
+                       int64_t num_pillars, const int32_t *cell_table, int64_t total_cells, const int32_t *num_cells, const float *radii, int d, int max_neighbors, void *workspace,
                        size_t workspace_bytes)
 {
     PCCNN_REQUIRE(d == 3, PCCNN_ERR_UNSUPPORTED, "%s: d=%d is not supported (d must be 3)", who, d);
@@ -206,6 +255,8 @@ static int nb_validate(const char *who, const float *pts_sorted, const int64_t *
                   who, (long long)n, (long long)m);
     PCCNN_REQUIRE(max_neighbors >= 0, PCCNN_ERR_INVALID, "%s: max_neighbors=%d", who, max_neighbors);
     PCCNN_REQUIRE(num_pillars > 0, PCCNN_ERR_INVALID, "%s: num_pillars=%lld", who, (long long)num_pillars);
+    PCCNN_REQUIRE(cell_table == nullptr || total_cells > 0, PCCNN_ERR_INVALID, "%s: cell_table with total_cells=%lld",
+                  who, (long long)total_cells);
     PCCNN_REQUIRE(grid_ds && num_cells && radii, PCCNN_ERR_INVALID, "%s: null grid pointer", who);
     PCCNN_REQUIRE(n == 0 || (pts_sorted && pt_keys_sorted), PCCNN_ERR_INVALID, "%s: null point pointer", who);
     PCCNN_REQUIRE(m == 0 || (samples && sample_keys), PCCNN_ERR_INVALID, "%s: null sample pointer", who);
@@ -218,11 +269,13 @@ static int nb_validate(const char *who, const float *pts_sorted, const int64_t *
 extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t *pt_keys_sorted, int64_t n,
                                           const float *samples, const int64_t *sample_keys, int64_t m,
                                           const int32_t *sample_order, const int32_t *grid_ds,
-                                          int64_t num_pillars, const int32_t *num_cells, const float *radii, int d, int max_neighbors,
+                                          int64_t num_pillars, const int32_t *cell_table, int64_t total_cells,
+                                          const int32_t *num_cells, const float *radii, int d, int max_neighbors,
                                           int32_t *ends_out, void *workspace, size_t workspace_bytes, void *stream)
 {
     int rc = nb_validate("pccnn_find_neighbors_count", pts_sorted, pt_keys_sorted, n, samples, sample_keys, m, grid_ds,
-                         num_pillars, num_cells, radii, d, max_neighbors, workspace, workspace_bytes);
+                         num_pillars, cell_table, total_cells, num_cells, radii, d, max_neighbors, workspace,
+                         workspace_bytes);
     if (rc != PCCNN_OK) return rc;
     if (m == 0) return PCCNN_OK;
     PCCNN_REQUIRE(ends_out, PCCNN_ERR_INVALID, "pccnn_find_neighbors_count: null ends_out");
@@ -235,6 +288,7 @@ extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t
     a.pts = pts_sorted; a.pt_keys = pt_keys_sorted; a.n = n;
     a.samples = samples; a.sample_keys = sample_keys; a.m = m;
     a.order = sample_order; a.grid_ds = grid_ds; a.num_pillars = num_pillars;
+    a.cell_table = cell_table; a.total_cells = total_cells;
     a.num_cells = num_cells; a.radii = radii; a.max_neighbors = max_neighbors;
     a.counts = counts; a.ends = nullptr; a.remap = nullptr; a.t = 0; a.neigh = nullptr;
     int64_t waves = pccnn_ceil_div(m, 64);
@@ -250,12 +304,14 @@ extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t
 extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t *pt_keys_sorted, int64_t n,
                                          const float *samples, const int64_t *sample_keys, int64_t m,
                                          const int32_t *sample_order, const int32_t *grid_ds,
-                                         int64_t num_pillars, const int32_t *num_cells, const float *radii, int d, int max_neighbors,
+                                         int64_t num_pillars, const int32_t *cell_table, int64_t total_cells,
+                                          const int32_t *num_cells, const float *radii, int d, int max_neighbors,
                                          const int32_t *ends, const int32_t *point_remap, int64_t t,
                                          int32_t *neigh_out, void *workspace, size_t workspace_bytes, void *stream)
 {
     int rc = nb_validate("pccnn_find_neighbors_fill", pts_sorted, pt_keys_sorted, n, samples, sample_keys, m, grid_ds,
-                         num_pillars, num_cells, radii, d, max_neighbors, workspace, workspace_bytes);
+                         num_pillars, cell_table, total_cells, num_cells, radii, d, max_neighbors, workspace,
+                         workspace_bytes);
     if (rc != PCCNN_OK) return rc;
     PCCNN_REQUIRE(t >= 0 && t < (1ll << 31), PCCNN_ERR_INVALID, "pccnn_find_neighbors_fill: t=%lld", (long long)t);
     if (m == 0 || t == 0) return PCCNN_OK;
@@ -268,6 +324,7 @@ extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t 
     a.pts = pts_sorted; a.pt_keys = pt_keys_sorted; a.n = n;
     a.samples = samples; a.sample_keys = sample_keys; a.m = m;
     a.order = sample_order; a.grid_ds = grid_ds; a.num_pillars = num_pillars;
+    a.cell_table = cell_table; a.total_cells = total_cells;
     a.num_cells = num_cells; a.radii = radii; a.max_neighbors = max_neighbors;
     a.counts = counts; a.ends = ends; a.remap = point_remap; a.t = t; a.neigh = neigh_out;
     int64_t waves = pccnn_ceil_div(m, 64);

@@ -1,7 +1,7 @@
 // Stable LSD radix sort of (64-bit cell key, 32-bit index) pairs, 8 bits per pass, only over
 // the significant key bits.  Per pass:
 //   1. radix_hist_kernel    : per-tile digit histogram staged in LDS, stored digit-major
-//   2. radix_scan_kernel    : one workgroup turns the [256][tiles] table into exclusive offsets
+//   2. radix_scan_kernel    : one workgroup per digit scans that digit's per-tile counts
 //   3. radix_scatter_kernel : every tile re-reads its keys, ranks them with wave ballots
 //                             (match-any on the digit bits), and scatters keys and indices;
 //                             the last pass also gathers the xyz row of every point.
@@ -30,65 +30,69 @@ radix_hist_kernel(const int64_t *__restrict__ keys, int64_t n, int shift, int32_
     tile_hist[(int64_t)threadIdx.x * num_tiles + blockIdx.x] = hist[threadIdx.x];
 }
 
-// Exclusive scan over `count` ints in place, single workgroup of 1024 threads.
-__global__ void __launch_bounds__(1024)
-radix_scan_kernel(int32_t *__restrict__ data, int64_t count)
+// One workgroup per digit: exclusive scan of that digit's per-tile counts (contiguous in the digit-major
+// table), in place; the digit's total goes to digit_totals[digit].
+__global__ void __launch_bounds__(256)
+radix_scan_kernel(int32_t *__restrict__ tile_hist, int64_t num_tiles, int32_t *__restrict__ digit_totals)
 {
-    __shared__ int wave_tot[16];
-    __shared__ int carry_s;
-    int lane = pccnn_lane();
-    int wave = threadIdx.x >> 6;
-    if (threadIdx.x == 0) carry_s = 0;
-    __syncthreads();
-    const int CH = 8;                                  // consecutive elements per thread
-    for (int64_t base = 0; base < count; base += 1024 * CH) {
-        int64_t i0 = base + (int64_t)threadIdx.x * CH;
-        int v[CH];
-        int sum = 0;
-#pragma unroll
-        for (int j = 0; j < CH; ++j) {
-            v[j] = (i0 + j < count) ? data[i0 + j] : 0;
-            sum += v[j];
-        }
-        int incl = sum;
+    __shared__ int wave_tot[4];
+    const int lane = pccnn_lane(), wave = threadIdx.x >> 6;
+    int32_t *row = tile_hist + (int64_t)blockIdx.x * num_tiles;
+    int carry = 0;
+    for (int64_t base = 0; base < num_tiles; base += 256) {
+        const int64_t i = base + threadIdx.x;
+        const int x = i < num_tiles ? row[i] : 0;
+        int incl = x;
 #pragma unroll
         for (int o = 1; o < 64; o <<= 1) {
-            int t = __shfl_up(incl, o);
+            const int t = __shfl_up(incl, o);
             if (lane >= o) incl += t;
         }
         if (lane == 63) wave_tot[wave] = incl;
         __syncthreads();
-        int add = carry_s, tot = 0;
+        int add = carry, tot = 0;
 #pragma unroll
-        for (int w = 0; w < 16; ++w) {
-            int x = wave_tot[w];
-            if (w < wave) add += x;
-            tot += x;
+        for (int w = 0; w < 4; ++w) {
+            const int v = wave_tot[w];
+            if (w < wave) add += v;
+            tot += v;
         }
-        int run = add + incl - sum;
-#pragma unroll
-        for (int j = 0; j < CH; ++j) {
-            if (i0 + j < count) data[i0 + j] = run;
-            run += v[j];
-        }
-        __syncthreads();
-        if (threadIdx.x == 0) carry_s += tot;
+        if (i < num_tiles) row[i] = add + incl - x;
+        carry += tot;
         __syncthreads();
     }
+    if (threadIdx.x == 0) digit_totals[blockIdx.x] = carry;
 }
 
 template <bool FIRST, bool GATHER>
 __global__ void __launch_bounds__(RS_THREADS)
 radix_scatter_kernel(const int64_t *__restrict__ keys_in, const int32_t *__restrict__ vals_in, int64_t n, int shift,
                      const int32_t *__restrict__ tile_offsets, int64_t num_tiles,
-                     int64_t *__restrict__ keys_out, int32_t *__restrict__ vals_out,
+                     const int32_t *__restrict__ digit_totals, int64_t *__restrict__ keys_out, int32_t *__restrict__ vals_out,
                      const float *__restrict__ pts, float *__restrict__ pts_out)
 {
     __shared__ int running[256];                       // next free output slot per digit
     __shared__ int wave_cnt[RS_WAVES][256];
     int lane = pccnn_lane();
     int wave = threadIdx.x >> 6;
-    running[threadIdx.x] = tile_offsets[(int64_t)threadIdx.x * num_tiles + blockIdx.x];
+    // first output slot of digit d for this tile = (keys with a smaller digit) + (same digit in earlier tiles)
+    {
+        const int tot = digit_totals[threadIdx.x];
+        int incl = tot;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int t = __shfl_up(incl, o);
+            if (lane >= o) incl += t;
+        }
+        if (lane == 63) wave_cnt[0][wave] = incl;
+        __syncthreads();
+        int add = 0;
+#pragma unroll
+        for (int w = 0; w < RS_WAVES; ++w)
+            if (w < wave) add += wave_cnt[0][w];
+        running[threadIdx.x] = add + incl - tot + tile_offsets[(int64_t)threadIdx.x * num_tiles + blockIdx.x];
+        __syncthreads();
+    }
 #pragma unroll
     for (int w = 0; w < RS_WAVES; ++w) wave_cnt[w][threadIdx.x] = 0;
     __syncthreads();
@@ -139,7 +143,7 @@ extern "C" size_t pccnn_sort_keys_workspace_bytes(int64_t n)
     if (n < 0) n = 0;
     int64_t tiles = pccnn_ceil_div(n > 0 ? n : 1, RS_TILE);
     return pccnn_align((size_t)n * sizeof(int64_t)) + pccnn_align((size_t)n * sizeof(int32_t)) +
-           pccnn_align((size_t)tiles * 256 * sizeof(int32_t)) + 256;
+           pccnn_align((size_t)tiles * 256 * sizeof(int32_t)) + pccnn_align(256 * sizeof(int32_t)) + 256;
 }
 
 extern "C" int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int64_t *sorted_keys_out,
@@ -164,6 +168,7 @@ extern "C" int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int
     int64_t *tmp_keys = arena.take<int64_t>((size_t)n);
     int32_t *tmp_vals = arena.take<int32_t>((size_t)n);
     int32_t *hist = arena.take<int32_t>((size_t)tiles * 256);
+    int32_t *totals = arena.take<int32_t>(256);
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "pccnn_sort_keys: workspace too small");
 
     PccnnTimed timed(PCCNN_T_SORT, s);
@@ -177,23 +182,23 @@ extern "C" int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int
         bool last = (p == passes - 1);
         radix_hist_kernel<<<(unsigned)tiles, RS_THREADS, 0, s>>>(src_k, n, shift, hist, tiles);
         PCCNN_LAUNCH_CHECK();
-        radix_scan_kernel<<<1, 1024, 0, s>>>(hist, tiles * 256);
+        radix_scan_kernel<<<256, 256, 0, s>>>(hist, tiles, totals);
         PCCNN_LAUNCH_CHECK();
         bool gather = last && pts != nullptr;
         if (p == 0) {
             if (gather)
                 radix_scatter_kernel<true, true><<<(unsigned)tiles, RS_THREADS, 0, s>>>(
-                    src_k, src_v, n, shift, hist, tiles, dst_k, dst_v, pts, sorted_pts_out);
+                    src_k, src_v, n, shift, hist, tiles, totals, dst_k, dst_v, pts, sorted_pts_out);
             else
                 radix_scatter_kernel<true, false><<<(unsigned)tiles, RS_THREADS, 0, s>>>(
-                    src_k, src_v, n, shift, hist, tiles, dst_k, dst_v, nullptr, nullptr);
+                    src_k, src_v, n, shift, hist, tiles, totals, dst_k, dst_v, nullptr, nullptr);
         } else {
             if (gather)
                 radix_scatter_kernel<false, true><<<(unsigned)tiles, RS_THREADS, 0, s>>>(
-                    src_k, src_v, n, shift, hist, tiles, dst_k, dst_v, pts, sorted_pts_out);
+                    src_k, src_v, n, shift, hist, tiles, totals, dst_k, dst_v, pts, sorted_pts_out);
             else
                 radix_scatter_kernel<false, false><<<(unsigned)tiles, RS_THREADS, 0, s>>>(
-                    src_k, src_v, n, shift, hist, tiles, dst_k, dst_v, nullptr, nullptr);
+                    src_k, src_v, n, shift, hist, tiles, totals, dst_k, dst_v, nullptr, nullptr);
         }
         PCCNN_LAUNCH_CHECK();
         src_k = dst_k;

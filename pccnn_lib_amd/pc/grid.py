@@ -10,7 +10,8 @@ class Grid(object):
     Attributes as in the reference: ``cell_size_``, ``num_cells_`` (int32 [D]), ``cell_ids_`` (int64 [N]),
     ``sorted_ids_`` (int64 [N]: the stable key-order permutation) and ``grid_ds_`` (int32 [B, nc0, nc1, 2]).
     The argsort and the gathers of sorted keys / points are one native radix sort; its by-products
-    (``sorted_cell_ids_``, ``sorted_pts_``, ``sorted_ids_i32_``) are kept for Neighborhood and PointPooling."""
+    (``sorted_cell_ids_``, ``sorted_pts_``, ``sorted_ids_i32_``) are kept for Neighborhood and PointPooling, and
+    for grids of up to 2^26 cells ``build_ds`` also builds ``cell_table_`` (first sorted index of every cell)."""
 
     def __init__(self, p_point_cloud, p_bounding_box, p_cell_size):
         self.pointcloud_ = p_point_cloud
@@ -29,6 +30,7 @@ class Grid(object):
         self.sorted_cell_ids_ = None
         self.sorted_pts_ = None
         self.grid_ds_ = None
+        self.cell_table_ = None
 
     def num_cells_host(self):
         if self.num_cells_host_ is None:
@@ -56,6 +58,11 @@ class Grid(object):
             with torch.no_grad():
                 shape = [int(self.pointcloud_.batch_size_)] + self.num_cells_host()[0:2] + [2]
                 self.grid_ds_ = pccnn_lib_ops.build_grid_ds(self.sorted_cell_ids_, self.num_cells_, shape)
+                cells = self.num_cells_host()
+                total = int(self.pointcloud_.batch_size_) * cells[0] * cells[1] * cells[2]
+                if total <= pccnn_lib_ops.CELL_TABLE_MAX_CELLS:
+                    # per-cell start offsets: the search then needs no binary search inside a pillar
+                    self.cell_table_ = pccnn_lib_ops.build_cell_table(self.sorted_cell_ids_, total)
 
     def __repr__(self):
         return "### Cell size:\n{}\n### Num cells:\n{}\n### Cell Ids:\n{}\n### Sorted Ids:\n{}\n### Grid Ds:\n{}".format(

@@ -27,7 +27,8 @@ class Neighborhood(object):
                 _, order, _ = pccnn_lib_ops.sort_keys(sample_keys, grid.key_bits())
             self.neighbors_, self.start_ids_ = pccnn_lib_ops.find_neighbors_ex(
                 grid.sorted_pts_, grid.sorted_cell_ids_, sample_pts, sample_keys, grid.grid_ds_, grid.num_cells_,
-                grid.cell_size_, p_max_neighbors, sample_order=order, point_remap=grid.sorted_ids_i32_)
+                grid.cell_size_, p_max_neighbors, sample_order=order, point_remap=grid.sorted_ids_i32_,
+                cell_table=grid.cell_table_)
 
     def __repr__(self):
         return "### Neighbors:\n{}\n### Start indices:\n{}".format(self.neighbors_, self.start_ids_)

@@ -26,7 +26,7 @@ class PointPooling(object):
                 # already in key order, so the natural sample order is the cell order.
                 neighbors, start_ids = pccnn_lib_ops.find_neighbors_ex(
                     grid.sorted_pts_, grid.sorted_cell_ids_, grid.sorted_pts_, grid.sorted_cell_ids_, grid.grid_ds_,
-                    grid.num_cells_, grid.cell_size_, 0)
+                    grid.num_cells_, grid.cell_size_, 0, cell_table=grid.cell_table_)
                 sampled = pccnn_lib_ops.poisson_disk_sampling(grid.sorted_cell_ids_, neighbors, start_ids,
                                                               grid.num_cells_).reshape(-1)
                 self.pooling_ids_ = torch.index_select(grid.sorted_ids_, 0, sampled)

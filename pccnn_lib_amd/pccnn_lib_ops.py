@@ -135,10 +135,24 @@ def key_bits_for(grid_size_host, batch_size):
     return max(1, (max(total, 1) - 1).bit_length())
 
 
+# Largest grid (in cells) for which the per-cell start table is built: 2^26 cells = 256 MiB of int32.
+CELL_TABLE_MAX_CELLS = 1 << 26
+
+
+def build_cell_table(sorted_keys, total_cells):
+    """i32[total_cells + 1]: index of the first sorted point with key >= c, for every cell c."""
+    _chk(sorted_keys, "build_cell_table: keys", torch.int64, 1)
+    table = torch.empty((int(total_cells) + 1,), dtype=torch.int32, device=sorted_keys.device)
+    _lib.call("pccnn_build_cell_table", _ptr(sorted_keys), sorted_keys.shape[0], int(total_cells), _ptr(table),
+              _stream())
+    return table
+
+
 def find_neighbors_ex(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, radii, max_neighbors,
-                      sample_order=None, point_remap=None):
-    """find_neighbors with the two native extras: ``sample_order`` (i32[M], samples listed in key order) and
-    ``point_remap`` (i32[N], written through to column 0 of the result)."""
+                      sample_order=None, point_remap=None, cell_table=None):
+    """find_neighbors with the native extras: ``sample_order`` (i32[M], samples listed in key order),
+    ``point_remap`` (i32[N], written through to column 0 of the result) and ``cell_table`` (from
+    build_cell_table: replaces the per-pillar binary searches by two table reads)."""
     name = "find_neighbors"
     _chk(pts, name + ": pts", torch.float32, 2)
     dev = pts.device
@@ -165,18 +179,22 @@ def find_neighbors_ex(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, ra
         if point_remap.shape[0] != n:
             raise RuntimeError(name + ": point_remap has the wrong length")
     pillars = grid_ds.shape[0] * grid_ds.shape[1] * grid_ds.shape[2]
+    table_p, total_cells = _P(0), 0
+    if cell_table is not None:
+        _chk(cell_table, name + ": cell_table", torch.int32, 1, dev)
+        table_p, total_cells = _ptr(cell_table), cell_table.shape[0] - 1
     ends = torch.empty((m,), dtype=torch.int32, device=dev)
     if m == 0:
         return [torch.empty((0, 2), dtype=torch.int32, device=dev), ends]
     ws = _workspace(_lib.load().pccnn_find_neighbors_workspace_bytes(m), dev)
     order_p = _ptr(sample_order) if sample_order is not None else _P(0)
     _lib.call("pccnn_find_neighbors_count", _ptr(pts), _ptr(pt_keys), n, _ptr(samples), _ptr(sample_keys), m, order_p,
-              _ptr(grid_ds), pillars, _ptr(grid_size), _ptr(radii), d, max_neighbors, _ptr(ends), _ptr(ws),
-              ws.numel(), _stream())
+              _ptr(grid_ds), pillars, table_p, total_cells, _ptr(grid_size), _ptr(radii), d, max_neighbors, _ptr(ends),
+              _ptr(ws), ws.numel(), _stream())
     total = int(ends[-1].item())                      # the one host read-back, as in the reference
     neigh = torch.empty((total, 2), dtype=torch.int32, device=dev)
     _lib.call("pccnn_find_neighbors_fill", _ptr(pts), _ptr(pt_keys), n, _ptr(samples), _ptr(sample_keys), m, order_p,
-              _ptr(grid_ds), pillars, _ptr(grid_size), _ptr(radii), d, max_neighbors, _ptr(ends),
+              _ptr(grid_ds), pillars, table_p, total_cells, _ptr(grid_size), _ptr(radii), d, max_neighbors, _ptr(ends),
               _ptr(point_remap) if point_remap is not None else _P(0), total, _ptr(neigh), _ptr(ws), ws.numel(),
               _stream())
     return [neigh, ends]
@@ -186,13 +204,19 @@ def find_neighbors(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, radii
     """find_neighbors(sorted pts, sorted keys, samples, sample keys, grid_ds, grid_size, radii, max_neighbors)
     -> [neigh i32[T,2] = (sorted point index, sample index), ends i32[M]]
     (pccnn_lib_ops/find_neighbors/find_neighbors.cuh:33-41)."""
-    order = None
+    order, table = None, None
     if isinstance(sample_keys, torch.Tensor) and sample_keys.is_cuda and sample_keys.dim() == 1 \
-            and sample_keys.shape[0] > 4096 and isinstance(grid_size, torch.Tensor) and grid_ds.dim() == 4:
+            and sample_keys.shape[0] > 4096 and isinstance(grid_size, torch.Tensor) and grid_ds.dim() == 4 \
+            and isinstance(pt_keys, torch.Tensor) and pt_keys.dtype == torch.int64:
         # queries are walked in cell order so that a wavefront's 64 queries share their cell walk
-        bits = key_bits_for(grid_size.tolist(), grid_ds.shape[0])
+        cells = grid_size.tolist()
+        bits = key_bits_for(cells, grid_ds.shape[0])
         _, order, _ = sort_keys(sample_keys, bits)
-    return find_neighbors_ex(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, radii, max_neighbors, order)
+        total = grid_ds.shape[0] * cells[0] * cells[1] * cells[2]
+        if total <= CELL_TABLE_MAX_CELLS:
+            table = build_cell_table(pt_keys, total)
+    return find_neighbors_ex(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, radii, max_neighbors, order,
+                             cell_table=table)
 
 
 # ------------------------------------------------------------------------------ pdf

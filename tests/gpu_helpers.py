@@ -11,7 +11,8 @@ def t(a, dtype=None):
     return out if dtype is None else out.to(dtype)
 
 
-def gpu_neighborhood(ops, pts, ids, samples, sample_ids, radius, batch_size, max_neighbors=0, use_order=True):
+def gpu_neighborhood(ops, pts, ids, samples, sample_ids, radius, batch_size, max_neighbors=0, use_order=True,
+                     use_table=False):
     """keys -> sort -> grid -> find_neighbors through the op module; returns host arrays keyed like
     oracle.neighborhood()."""
     tp, ti = t(pts), t(ids)
@@ -25,8 +26,11 @@ def gpu_neighborhood(ops, pts, ids, samples, sample_ids, radius, batch_size, max
     ds = ops.build_grid_ds(skeys, nc, [batch_size] + nc.tolist()[0:2] + [2])
     skey = ops.compute_keys(ts, tsi, mn, nc, radii)
     order = ops.sort_keys(skey, bits)[1] if use_order else None
-    neigh_sorted, ends = ops.find_neighbors_ex(spts, skeys, ts, skey, ds, nc, radii, max_neighbors, order)
-    neigh, ends2 = ops.find_neighbors_ex(spts, skeys, ts, skey, ds, nc, radii, max_neighbors, order, perm)
+    table = ops.build_cell_table(skeys, batch_size * int(np.prod(nc.tolist()))) if use_table else None
+    neigh_sorted, ends = ops.find_neighbors_ex(spts, skeys, ts, skey, ds, nc, radii, max_neighbors, order,
+                                               cell_table=table)
+    neigh, ends2 = ops.find_neighbors_ex(spts, skeys, ts, skey, ds, nc, radii, max_neighbors, order, perm,
+                                         cell_table=table)
     torch.cuda.synchronize()
     assert torch.equal(ends, ends2)
     c = lambda x: x.cpu().numpy()

@@ -32,11 +32,12 @@ def _compare_neighborhoods(oracle, got, exp):
 
 
 @pytest.mark.parametrize("batch,num_pts,radius", [(4, 1000, 0.2), (4, 100, 1.0), (2, 1024, 0.05), (1, 37, 0.3)])
-@pytest.mark.parametrize("use_order", [True, False])
-def test_reference_clouds_bit_exact(ops, oracle, models, batch, num_pts, radius, use_order):
+@pytest.mark.parametrize("use_order,use_table", [(True, False), (False, False), (True, True), (False, True)])
+def test_reference_clouds_bit_exact(ops, oracle, models, batch, num_pts, radius, use_order, use_table):
+    # every combination of the two search accelerators (key-ordered queries, per-cell start table)
     pts, ids = _cloud(models, batch, num_pts)
     exp = oracle.neighborhood(pts, ids, pts, ids, radius)
-    got = gpu_neighborhood(ops, pts, ids, pts, ids, radius, batch, use_order=use_order)
+    got = gpu_neighborhood(ops, pts, ids, pts, ids, radius, batch, use_order=use_order, use_table=use_table)
     _compare_neighborhoods(oracle, got, exp)
 
 
@@ -66,8 +67,9 @@ def test_samples_differ_from_points(ops, oracle):
     smp = (pts[pick] + rng.normal(0, 0.004, (700, 3))).astype(np.float32)   # some fall outside the box: clamped
     sids = ids[pick]
     exp = oracle.neighborhood(pts, ids, smp, sids, 0.08)
-    got = gpu_neighborhood(ops, pts, ids, smp, sids, 0.08, 3)
-    _compare_neighborhoods(oracle, got, exp)
+    for use_table in (False, True):
+        got = gpu_neighborhood(ops, pts, ids, smp, sids, 0.08, 3, use_table=use_table)
+        _compare_neighborhoods(oracle, got, exp)
 
 
 @pytest.mark.parametrize("cap", [4, 16])
@@ -138,12 +140,35 @@ def test_run_twice_is_bitwise_identical(ops):
     assert np.array_equal(a["neighbors"], b["neighbors"]) and np.array_equal(a["ends"], b["ends"])
 
 
+def test_drop_in_find_neighbors_and_object_api_agree(ops, oracle):
+    # the reference-signature op (sorts the queries and builds the cell table by itself above 4096 samples)
+    # and the Pointcloud / Grid / Neighborhood objects give the oracle's lists
+    import pccnn_lib_amd as lib
+    pts, ids = synthetic.primitives(21, 3, 2500)
+    exp = oracle.neighborhood(pts, ids, pts, ids, 0.07)
+    g = gpu_neighborhood(ops, pts, ids, pts, ids, 0.07, 3)
+    d = g["dev"]
+    neigh, ends = ops.find_neighbors(d["spts"], d["skeys"], d["samples"], t(g["sample_keys"]), d["ds"], d["nc"],
+                                     d["radii"], 0)
+    assert np.array_equal(neigh.cpu().numpy(), exp["neigh_sorted"]) and np.array_equal(ends.cpu().numpy(), exp["ends"])
+    pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+    nbh = lib.pc.layers.conv_base.build_neighborhood(pc, pc, torch.full((3,), 0.07, device=DEV), 0)
+    assert nbh.grid_.cell_table_ is not None
+    assert np.array_equal(nbh.neighbors_.cpu().numpy(), exp["neighbors"])
+    assert np.array_equal(nbh.start_ids_.cpu().numpy(), exp["ends"])
+    assert np.array_equal(nbh.grid_.cell_ids_.cpu().numpy(), exp["keys"])
+    assert np.array_equal(nbh.grid_.sorted_ids_.cpu().numpy(), exp["perm"].astype(np.int64))
+    assert np.array_equal(nbh.grid_.grid_ds_.cpu().numpy(), exp["grid_ds"])
+
+
 def test_scene_scale_properties(ops):
     # 200k-point room (the generator of the million-point configuration) checked through size-independent
     # properties: sorted keys, permutation, self-membership, symmetry, monotone ends.
     pts = synthetic.room(4, 200000)
     ids = np.zeros(pts.shape[0], np.int32)
-    g = gpu_neighborhood(ops, pts, ids, pts, ids, 0.05, 1)
+    g = gpu_neighborhood(ops, pts, ids, pts, ids, 0.05, 1, use_table=True)
+    g2 = gpu_neighborhood(ops, pts, ids, pts, ids, 0.05, 1, use_table=False, use_order=False)
+    assert np.array_equal(g["neighbors"], g2["neighbors"]) and np.array_equal(g["ends"], g2["ends"])
     assert np.all(np.diff(g["sorted_keys"]) >= 0)
     assert np.array_equal(np.sort(g["perm"]), np.arange(pts.shape[0]))
     ends, neigh = g["ends"], g["neighbors"]
