@@ -187,6 +187,21 @@ int pccnn_mcconv_backward(const float *pts, const float *pdf, const float *feats
                           float *d_pts, float *d_samples,
                           void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- variance statistic of the weight initialisation -----------------------
+ * Replaces kp_conv_weight_var / mc_conv_weight_var (pccnn_lib_ops/pcconvs/kpconv.cuh:82-90, mcconv.cuh:83-92;
+ * kernel pccnn_lib_ops/pcconvs/shared/compute_variance_weights.cu:24-170): out[0] (one float, device) =
+ * 1 / mean over the samples of sum_{i,j in N(s)} (w_i . w_j)(F_i . F_j), evaluated as the squared norm of the
+ * sample's projection tile.  Same tensor arguments as the forward calls, without the weights. */
+size_t pccnn_conv_weight_var_workspace_bytes(int64_t m, int c_in, int k);
+int pccnn_kpconv_weight_var(const float *pts, const float *feats, const float *samples, const int32_t *neigh,
+                            const int32_t *ends, const float *radii, const float *kernel_pts, float sigma,
+                            int64_t n, int64_t m, int64_t t, int d, int c_in, int k, float *out,
+                            void *workspace, size_t workspace_bytes, void *stream);
+int pccnn_mcconv_weight_var(const float *pts, const float *pdf, const float *feats, const float *samples,
+                            const int32_t *neigh, const int32_t *ends, const float *radii, const float *axis,
+                            const float *bias, int64_t n, int64_t m, int64_t t, int d, int c_in, int k, float *out,
+                            void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- dense contraction --------------------------------------------------
  * The fp32 MFMA GEMM the convolutions use for the [M, K*Cin] x [K*Cin, Cout]
  * contraction (torch::matmul at pccnn_lib_ops/pcconvs/kpconv.cu:56-57,90-96 and

@@ -35,6 +35,7 @@ def lib():
         _lib.orc_store_neighbors.restype = ctypes.c_int64
         _lib.orc_brute_force_neighbors.restype = ctypes.c_int64
         _lib.orc_poisson_disk.restype = ctypes.c_int64
+        _lib.orc_variance_weights.restype = ctypes.c_double
     return _lib
 
 
@@ -379,3 +380,25 @@ def mcconv_grads(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weigh
     np.add.at(dpdf, neigh[:, 0], dpdf_pair)
     dpts, dsamples = _pt_diff_grads(pts.shape[0], samples.shape[0], neigh, radii, ddiff)
     return [dw, dfeat, daxis, dbias, dpdf.astype(np.float32), dpts, dsamples]
+
+
+def variance_weights(basis, feats, neigh, ends):
+    """compute_variance_weights.cu:114-170 (no division by the neighbor count).  Returns (1 / mean, per-sample sums)."""
+    basis, feats, neigh, ends = _f32(basis), _f32(feats), _i32(neigh), _i32(ends)
+    m = ends.shape[0]
+    per = np.empty(m, np.float64)
+    val = lib().orc_variance_weights(_p(basis), _p(feats), _p(neigh), _p(ends), I64(m), I32(feats.shape[1]),
+                                     I32(basis.shape[1]), _p(per))
+    return np.float32(val), per
+
+
+def kpconv_weight_var(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma):
+    """pccnn_lib_ops/pcconvs/kpconv.cu:115-136."""
+    basis, _ = conv_basis(KP, pts, samples, neigh, radii, kernel_pts, sigma=sigma)
+    return variance_weights(basis, feats, neigh, ends)[0]
+
+
+def mcconv_weight_var(pts, pdf, feats, samples, neigh, ends, radii, axis, bias):
+    """pccnn_lib_ops/pcconvs/mcconv.cu:145-172."""
+    basis, _ = conv_basis(MLP, pts, samples, neigh, radii, axis, bias=bias, pdf=pdf)
+    return variance_weights(basis, feats, neigh, ends)[0]

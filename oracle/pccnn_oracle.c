@@ -499,3 +499,32 @@ int orc_feat_basis_proj_grads(const float *basis, const float *feats, const int3
     free(facc);
     return 0;
 }
+
+/* pccnn_lib_ops/pcconvs/shared/compute_variance_weights.cu:38-108 with pDivideNumNeighs = false (the KPConv
+ * and MCConv callers, kpconv.cu:133-135, mcconv.cu:169-171): per sample the double sum over ordered pairs
+ * (i, j) of its neighbors of (w_i . w_j) * (F_i . F_j); then :168-169, the reciprocal of the mean over the
+ * samples.  Written as the literal O(n^2) loops, accumulated in double.  per_sample_out may be NULL. */
+double orc_variance_weights(const float *basis, const float *feats, const int32_t *neigh, const int32_t *ends,
+                            int64_t m, int c_in, int k_basis, double *per_sample_out)
+{
+    double total = 0.0;
+    for (int64_t s = 0; s < m; ++s) {
+        int32_t lo = s > 0 ? ends[s - 1] : 0, hi = ends[s];
+        double acc = 0.0;
+        for (int32_t i = lo; i < hi; ++i) {
+            const float *wi = basis + (int64_t)i * k_basis;
+            const float *fi = feats + (int64_t)neigh[2 * i] * c_in;
+            for (int32_t j = lo; j < hi; ++j) {
+                const float *wj = basis + (int64_t)j * k_basis;
+                const float *fj = feats + (int64_t)neigh[2 * j] * c_in;
+                double sw = 0.0, sf = 0.0;
+                for (int k = 0; k < k_basis; ++k) sw += (double)wi[k] * (double)wj[k];
+                for (int c = 0; c < c_in; ++c) sf += (double)fi[c] * (double)fj[c];
+                acc += sw * sf;
+            }
+        }
+        if (per_sample_out) per_sample_out[s] = acc;
+        total += acc;
+    }
+    return 1.0 / (total / (double)m);
+}

@@ -420,6 +420,36 @@ conv_param_reduce_kernel(const float *__restrict__ partials, int64_t rows, int k
     }
 }
 
+// Variance statistic of the initialisation: per sample, sum over ordered neighbor pairs (i, j) of
+// (w_i . w_j)(F_i . F_j) = the squared Frobenius norm of the sample's projection tile P[s].  One wavefront
+// per row of P sums the squares; one workgroup then forms 1 / mean over the samples in double, fixed order.
+__global__ void __launch_bounds__(256)
+row_sumsq_kernel(const float *__restrict__ proj, int64_t rows, int64_t row_len, float *__restrict__ out)
+{
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= rows) return;
+    const float *src = proj + r * row_len;
+    float acc = 0.0f;
+    for (int64_t i = pccnn_lane(); i < row_len; i += 64) acc += src[i] * src[i];
+    acc = pccnn_wave_sum(acc);
+    if (pccnn_lane() == 0) out[r] = acc;
+}
+
+__global__ void __launch_bounds__(256)
+mean_reciprocal_kernel(const float *__restrict__ vals, int64_t count, float *__restrict__ out)
+{
+    __shared__ double red[256];
+    double acc = 0.0;
+    for (int64_t i = threadIdx.x; i < count; i += 256) acc += (double)vals[i];
+    red[threadIdx.x] = acc;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if (threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[0] = (float)(1.0 / (red[0] / (double)count));
+}
+
 // ------------------------------------------------------------------------------- host side
 
 static int kpad_of(int k) { return k <= 8 ? 8 : (k <= 16 ? 16 : (k <= 32 ? 32 : 64)); }
@@ -573,6 +603,60 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     conv_param_reduce_kernel<BASIS><<<256, 256, 0, s>>>(partials, partial_rows, g.k, d_param_a, d_param_b);
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
+}
+
+template <int BASIS>
+static int conv_weight_var(ConvGeom g, const float *feats, float *out, void *workspace, size_t workspace_bytes,
+                           hipStream_t s)
+{
+    PCCNN_REQUIRE(g.m > 0, PCCNN_ERR_INVALID, "conv weight variance: no samples");
+    PccnnArena arena(workspace, workspace_bytes);
+    float *proj = arena.take<float>((size_t)g.m * g.c_in * g.k);
+    float *rows = arena.take<float>((size_t)g.m);
+    PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv weight variance: workspace of %zu bytes, need %zu",
+                  workspace_bytes, pccnn_conv_weight_var_workspace_bytes(g.m, g.c_in, g.k));
+    int rc = launch_proj_fwd<BASIS>(g, feats, proj, s);
+    if (rc != PCCNN_OK) return rc;
+    row_sumsq_kernel<<<(unsigned)pccnn_ceil_div(g.m, 4), 256, 0, s>>>(proj, g.m, (int64_t)g.c_in * g.k, rows);
+    PCCNN_LAUNCH_CHECK();
+    mean_reciprocal_kernel<<<1, 256, 0, s>>>(rows, g.m, out);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
+extern "C" size_t pccnn_conv_weight_var_workspace_bytes(int64_t m, int c_in, int k)
+{
+    if (m < 1) m = 1;
+    return pccnn_align((size_t)m * c_in * k * sizeof(float)) + pccnn_align((size_t)m * sizeof(float)) + 256;
+}
+
+extern "C" int pccnn_kpconv_weight_var(const float *pts, const float *feats, const float *samples,
+                                       const int32_t *neigh, const int32_t *ends, const float *radii,
+                                       const float *kernel_pts, float sigma, int64_t n, int64_t m, int64_t t, int d,
+                                       int c_in, int k, float *out, void *workspace, size_t workspace_bytes,
+                                       void *stream)
+{
+    int rc = conv_validate("pccnn_kpconv_weight_var", n, m, t, d, c_in, k, 1, 1);
+    if (rc != PCCNN_OK) return rc;
+    PCCNN_REQUIRE(sigma > 0.0f, PCCNN_ERR_INVALID, "pccnn_kpconv_weight_var: sigma=%g", sigma);
+    PCCNN_REQUIRE(pts && feats && samples && ends && radii && kernel_pts && out && (t == 0 || neigh), PCCNN_ERR_INVALID,
+                  "pccnn_kpconv_weight_var: null pointer");
+    ConvGeom g = {pts, samples, (const int2 *)neigh, ends, radii, nullptr, kernel_pts, nullptr, sigma, n, m, t, c_in, k};
+    return conv_weight_var<BASIS_KP>(g, feats, out, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" int pccnn_mcconv_weight_var(const float *pts, const float *pdf, const float *feats, const float *samples,
+                                       const int32_t *neigh, const int32_t *ends, const float *radii,
+                                       const float *axis, const float *bias, int64_t n, int64_t m, int64_t t, int d,
+                                       int c_in, int k, float *out, void *workspace, size_t workspace_bytes,
+                                       void *stream)
+{
+    int rc = conv_validate("pccnn_mcconv_weight_var", n, m, t, d, c_in, k, 1, 1);
+    if (rc != PCCNN_OK) return rc;
+    PCCNN_REQUIRE(pts && pdf && feats && samples && ends && radii && axis && bias && out && (t == 0 || neigh),
+                  PCCNN_ERR_INVALID, "pccnn_mcconv_weight_var: null pointer");
+    ConvGeom g = {pts, samples, (const int2 *)neigh, ends, radii, pdf, axis, bias, 1.0f, n, m, t, c_in, k};
+    return conv_weight_var<BASIS_MLP>(g, feats, out, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 extern "C" int pccnn_kpconv_forward(const float *pts, const float *feats, const float *samples, const int32_t *neigh,

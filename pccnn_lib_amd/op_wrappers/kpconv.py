@@ -27,7 +27,7 @@ class ComputeKPConv(torch.autograd.Function):
 
 class ComputeKPConvWeightVar(torch.autograd.Function):
     """apply(pts, features, samples, neighbors, start_ids, radii, kernel_pts, sigma): the statistic behind the
-    variance-aware initialisation (pccnn_lib/op_wrappers/compute_kpconv.py:76-113).  Not built yet."""
+    variance-aware initialisation (pccnn_lib/op_wrappers/compute_kpconv.py:76-113)."""
 
     @staticmethod
     def forward(ctx, p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_kernel_pts, p_sigma):

@@ -27,7 +27,7 @@ class ComputeMCConv(torch.autograd.Function):
 
 class ComputeMCConvWeightVar(torch.autograd.Function):
     """apply(pts, pdf, features, samples, neighbors, start_ids, radii, proj_axis, proj_bias): the statistic behind
-    the variance-aware initialisation (pccnn_lib/op_wrappers/compute_mcconv.py:78-117).  Not built yet."""
+    the variance-aware initialisation (pccnn_lib/op_wrappers/compute_mcconv.py:78-117)."""
 
     @staticmethod
     def forward(ctx, p_pts, p_pdf, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_proj_axis,

@@ -391,6 +391,40 @@ def mc_conv_grads(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weig
     return [d_w, d_f, d_axis, d_bias, d_pdf, d_p, d_s]
 
 
+def kp_conv_weight_var(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma):
+    """kp_conv_weight_var(pts, feats, samples, neighbors, start_ids, radii, kernel_pts, sigma) -> 0-d float tensor
+    (pccnn_lib_ops/pcconvs/kpconv.cuh:82-90)."""
+    name = "kp_conv_weight_var"
+    d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
+    _chk(kernel_pts, name + ": kernel_pts", torch.float32, 2, dev)
+    n, m, t, c_in, k = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1], kernel_pts.shape[0]
+    if kernel_pts.shape[1] != d:
+        raise RuntimeError(name + ": kernel_pts must be [K, D]")
+    out = torch.empty((1,), dtype=torch.float32, device=dev)
+    ws = _workspace(_lib.load().pccnn_conv_weight_var_workspace_bytes(m, c_in, k), dev)
+    _lib.call("pccnn_kpconv_weight_var", _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends), _ptr(radii),
+              _ptr(kernel_pts), float(sigma), n, m, t, d, c_in, k, _ptr(out), _ptr(ws), ws.numel(), _stream())
+    return out.reshape(())
+
+
+def mc_conv_weight_var(pts, pdf, feats, samples, neigh, ends, radii, axis, bias):
+    """mc_conv_weight_var(pts, pdf, feats, samples, neighbors, start_ids, radii, axis, bias) -> 0-d float tensor
+    (pccnn_lib_ops/pcconvs/mcconv.cuh:83-92)."""
+    name = "mc_conv_weight_var"
+    d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
+    _chk(pdf, name + ": pdf", torch.float32, 1, dev)
+    _chk(axis, name + ": axis", torch.float32, 2, dev)
+    _chk(bias, name + ": bias", torch.float32, 2, dev)
+    n, m, t, c_in, k = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1], axis.shape[1]
+    if pdf.shape[0] != n or axis.shape[0] != d or tuple(bias.shape) != (1, k):
+        raise RuntimeError(name + ": axis must be [D, H*mlps], bias [1, H*mlps], pdf [N]")
+    out = torch.empty((1,), dtype=torch.float32, device=dev)
+    ws = _workspace(_lib.load().pccnn_conv_weight_var_workspace_bytes(m, c_in, k), dev)
+    _lib.call("pccnn_mcconv_weight_var", _ptr(pts), _ptr(pdf), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends),
+              _ptr(radii), _ptr(axis), _ptr(bias), n, m, t, d, c_in, k, _ptr(out), _ptr(ws), ws.numel(), _stream())
+    return out.reshape(())
+
+
 # ------------------------------------------------------------- names outside this path
 
 
@@ -403,7 +437,7 @@ def _not_on_path(name):
     return fn
 
 
-for _n in ("mc_conv_weight_var", "kp_conv_weight_var", "point_conv_basis", "point_conv_basis_grads", "point_conv",
+for _n in ("point_conv_basis", "point_conv_basis_grads", "point_conv",
            "point_conv_grads", "point_conv_weight_var", "kp_conv_n", "kp_conv_n_grads", "kp_conv_n_weight_var",
            "sph_conv", "sph_conv_grads", "sph_conv_weight_var", "pccnn", "pccnn_grads", "pccnn_weight_variance"):
     globals()[_n] = _not_on_path(_n)

@@ -233,6 +233,37 @@ def test_hierarchy_level_with_pooling(oracle):
     assert relerr(p(out), exp) < 2e-5
 
 
+def test_weight_variance_ops_and_layer_warmup(ops, oracle):
+    import pccnn_lib_amd as lib
+    pts, ids, smp, nb, rng = _conv_case(oracle, ops, 77, 2, 1500, 0.12, True)
+    neigh, ends, radii = nb["neighbors"], nb["ends"], nb["radii"]
+    d = nb["dev"]
+    feats = rng.normal(size=(pts.shape[0], 24)).astype(np.float32)
+    kp, sigma = synthetic.kernel_points_sphere(1, 15)
+    got = ops.kp_conv_weight_var(d["pts"], t(feats), d["samples"], d["neigh"], d["ends"], d["radii"], t(kp), sigma)
+    assert got.dim() == 0
+    exp = oracle.kpconv_weight_var(pts, feats, smp, neigh, ends, radii, kp, sigma)
+    assert abs(float(got) - float(exp)) < 1e-5 * abs(float(exp))
+    pdf = rng.uniform(0.5, 2.0, pts.shape[0]).astype(np.float32)
+    axis = rng.normal(0, 0.6, (3, 16)).astype(np.float32)
+    bias = rng.normal(0, 0.1, (1, 16)).astype(np.float32)
+    got = ops.mc_conv_weight_var(d["pts"], t(pdf), t(feats), d["samples"], d["neigh"], d["ends"], d["radii"], t(axis),
+                                 t(bias))
+    exp = oracle.mcconv_weight_var(pts, pdf, feats, smp, neigh, ends, radii, axis, bias)
+    assert abs(float(got) - float(exp)) < 1e-5 * abs(float(exp))
+    # the layers' warm-up path (KPConv.py:103-116): weights are redrawn with the variance the statistic asks for
+    torch.manual_seed(3)
+    layer = lib.pc.layers.KPConv(3, 24, 8, 15, True, 1.0).to(DEV)
+    layer.set_init_warmup_state(True)
+    pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+    out, nbh = layer(pc, pc, t(feats), 0.12)
+    var = oracle.kpconv_weight_var(pts, feats, pts, nbh.neighbors_.cpu().numpy(), nbh.start_ids_.cpu().numpy(),
+                                   np.full(3, 0.12, np.float32), layer.kernel_pts_.cpu().numpy(), layer.sigma_cpu_)
+    assert abs(layer.accum_weight_var_ - 1.0 / float(var)) < 1e-4 * abs(1.0 / float(var))
+    # with weights of that variance the output variance is about the requested constant
+    assert 0.5 < float(out.var()) < 2.0
+
+
 def test_error_paths(ops):
     pts, ids = synthetic.primitives(1, 1, 128)
     tp, ti = t(pts), t(ids)

@@ -221,3 +221,22 @@ def test_mcconv_grads_match_autograd(oracle, models, num_mlps):
     for mine, ref, name in zip(got, (tw, tf, ta, tb, tpdf, tp, ts), names):
         assert mine.shape == tuple(ref.shape), name
         assert _relerr(mine, ref.grad.numpy()) < 1e-4, name
+
+
+def test_weight_variance_equals_projection_norm(oracle, models):
+    # The double sum over neighbor pairs of (w_i . w_j)(F_i . F_j) (compute_variance_weights.cu:38-108) is the
+    # squared Frobenius norm of the sample's projection tile; the literal O(n^2) restatement must agree with it.
+    pts, ids, nb, feats, rng = _setup(oracle, models, 0.2, 12, 3)
+    kp, sigma = synthetic.kernel_points_sphere(4, 16)
+    neigh, ends, radii = nb["neighbors"], nb["ends"], nb["radii"]
+    basis, _ = oracle.conv_basis(oracle.KP, pts, pts, neigh, radii, kp, sigma=sigma)
+    val, per = oracle.variance_weights(basis, feats, neigh, ends)
+    proj = oracle.feat_basis_proj(basis, feats, neigh, ends).astype(np.float64)
+    norms = (proj ** 2).sum(axis=(1, 2))
+    assert np.allclose(per, norms, rtol=1e-5)
+    assert np.isclose(val, 1.0 / norms.mean(), rtol=1e-5)
+    assert np.isclose(oracle.kpconv_weight_var(pts, feats, pts, neigh, ends, radii, kp, sigma), val, rtol=1e-6)
+    # one sample with a single neighbor: (w . w)(F . F)
+    one = oracle.variance_weights(basis[:1], feats, neigh[:1], np.array([1], np.int32))[0]
+    f0 = feats[neigh[0, 0]].astype(np.float64)
+    assert np.isclose(1.0 / one, (basis[0].astype(np.float64) ** 2).sum() * (f0 ** 2).sum(), rtol=1e-6)
