@@ -162,15 +162,28 @@ int pccnn_compact_selected(const int32_t *selected, const int32_t *selected_scan
  * d_weights (same shape), d_feats, d_axis f32[d,k], d_bias f32[k], d_pdf f32[n],
  * d_pts, d_samples.
  *
- * 1 <= k <= 64.  Backward outputs are fully overwritten. */
+ * 1 <= k <= 64.
+ *
+ * Two arguments go beyond the reference's interface.  `proj_out` / `proj` (nullable): the projection
+ * P f32[m, c_in, k] (k fastest) that the forward call builds on its way to `out`; a caller that keeps it
+ * (proj_out != NULL) can hand it to the backward call, which otherwise rebuilds it like the reference does
+ * (kpconv.cu:78-87).  `grad_mask`: which gradients to produce (PCCNN_GRAD_* bits; PCCNN_GRAD_ALL is the
+ * reference's behaviour).  Requested outputs are fully overwritten; outputs not requested may be NULL and are
+ * not touched. */
+#define PCCNN_GRAD_WEIGHTS 1
+#define PCCNN_GRAD_FEATS 2
+#define PCCNN_GRAD_BASIS_PARAMS 4 /* d_kernel_pts, or d_axis and d_bias */
+#define PCCNN_GRAD_PDF 8
+#define PCCNN_GRAD_PTS 16         /* d_pts and d_samples */
+#define PCCNN_GRAD_ALL 31
 size_t pccnn_conv_workspace_bytes(int64_t m, int64_t t, int c_in, int k, int c_out, int backward);
 int pccnn_kpconv_forward(const float *pts, const float *feats, const float *samples, const int32_t *neigh,
                          const int32_t *ends, const float *radii, const float *kernel_pts, float sigma,
                          const float *weights, int64_t n, int64_t m, int64_t t, int d, int c_in, int k, int c_out,
-                         float *out, void *workspace, size_t workspace_bytes, void *stream);
+                         float *out, float *proj_out, void *workspace, size_t workspace_bytes, void *stream);
 int pccnn_kpconv_backward(const float *pts, const float *feats, const float *samples, const int32_t *neigh,
                           const int32_t *ends, const float *radii, const float *kernel_pts, float sigma,
-                          const float *weights, const float *in_grads,
+                          const float *weights, const float *in_grads, const float *proj, int grad_mask,
                           int64_t n, int64_t m, int64_t t, int d, int c_in, int k, int c_out,
                           float *d_weights, float *d_feats, float *d_kernel_pts, float *d_pts, float *d_samples,
                           void *workspace, size_t workspace_bytes, void *stream);
@@ -178,10 +191,11 @@ int pccnn_mcconv_forward(const float *pts, const float *pdf, const float *feats,
                          const int32_t *neigh, const int32_t *ends, const float *radii, const float *axis,
                          const float *bias, const float *weights,
                          int64_t n, int64_t m, int64_t t, int d, int c_in, int k, int num_mlps, int c_out,
-                         float *out, void *workspace, size_t workspace_bytes, void *stream);
+                         float *out, float *proj_out, void *workspace, size_t workspace_bytes, void *stream);
 int pccnn_mcconv_backward(const float *pts, const float *pdf, const float *feats, const float *samples,
                           const int32_t *neigh, const int32_t *ends, const float *radii, const float *axis,
-                          const float *bias, const float *weights, const float *in_grads,
+                          const float *bias, const float *weights, const float *in_grads, const float *proj,
+                          int grad_mask,
                           int64_t n, int64_t m, int64_t t, int d, int c_in, int k, int num_mlps, int c_out,
                           float *d_weights, float *d_feats, float *d_axis, float *d_bias, float *d_pdf,
                           float *d_pts, float *d_samples,

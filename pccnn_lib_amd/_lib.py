@@ -36,12 +36,12 @@ SIGNATURES = {
     "pccnn_poisson_disk_select": (I32, [P, I64, P, I64, P, P, I32, P, P, P, SZ, P]),
     "pccnn_compact_selected": (I32, [P, P, I64, P, P]),
     "pccnn_conv_workspace_bytes": (SZ, [I64, I64, I32, I32, I32, I32]),
-    "pccnn_kpconv_forward": (I32, [P, P, P, P, P, P, P, F32, P, I64, I64, I64, I32, I32, I32, I32, P, P, SZ, P]),
-    "pccnn_kpconv_backward": (I32, [P, P, P, P, P, P, P, F32, P, P, I64, I64, I64, I32, I32, I32, I32,
+    "pccnn_kpconv_forward": (I32, [P, P, P, P, P, P, P, F32, P, I64, I64, I64, I32, I32, I32, I32, P, P, P, SZ, P]),
+    "pccnn_kpconv_backward": (I32, [P, P, P, P, P, P, P, F32, P, P, P, I32, I64, I64, I64, I32, I32, I32, I32,
                                     P, P, P, P, P, P, SZ, P]),
     "pccnn_mcconv_forward": (I32, [P, P, P, P, P, P, P, P, P, P, I64, I64, I64, I32, I32, I32, I32, I32,
-                                   P, P, SZ, P]),
-    "pccnn_mcconv_backward": (I32, [P, P, P, P, P, P, P, P, P, P, P, I64, I64, I64, I32, I32, I32, I32, I32,
+                                   P, P, P, SZ, P]),
+    "pccnn_mcconv_backward": (I32, [P, P, P, P, P, P, P, P, P, P, P, P, I32, I64, I64, I64, I32, I32, I32, I32, I32,
                                     P, P, P, P, P, P, P, P, SZ, P]),
     "pccnn_conv_weight_var_workspace_bytes": (SZ, [I64, I32, I32]),
     "pccnn_kpconv_weight_var": (I32, [P, P, P, P, P, P, P, F32, I64, I64, I64, I32, I32, I32, P, P, SZ, P]),

@@ -5,13 +5,13 @@
 //   * one wavefront per (sample, block of 64 input features): lane l owns feature f = 64*fb + l
 //     and keeps the K partial sums of its feature in registers;
 //   * the pair geometry (neighbor id, normalised offset, density) of up to 64 pairs is loaded
-//     lane-parallel, then pair by pair the basis values w[t][0..K) are evaluated by lanes 0..K-1
-//     and handed to every lane as scalars (readlane), while the feature row of the neighbor is
-//     one coalesced read;
+//     lane-parallel; the basis values w[t][0..K) of the chunk are evaluated once, K lanes per pair,
+//     and staged in LDS, from where every lane reads them as broadcasts, while the feature row of
+//     each neighbor is one coalesced read;
 //   * P is stored k-fastest, i.e. row f*K + k of the contraction, then out = P x W on MFMA.
 // Backward: dP = dOut x W^T and dW = P^T x dOut on MFMA; a second per-sample walk turns dP into
 // feature gradients (coalesced float atomics per neighbor row) and per-pair basis gradients
-// (butterfly reduce-scatter across the lanes); a pair-parallel kernel then applies the basis
+// (feature rows staged in LDS, K-lane partial sums); a per-sample kernel then applies the basis
 // derivative and accumulates point, sample, density and basis-parameter gradients.
 #include "common.h"
 
@@ -67,71 +67,83 @@ template <int BASIS> struct LaneBasis {
 // ------------------------------------------------------------------------------- forward
 
 template <int BASIS, int KPAD>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(64)
 conv_proj_fwd_kernel(ConvGeom g, const float *__restrict__ feats, float *__restrict__ proj)
 {
-    const int lane = pccnn_lane();
-    const int64_t s = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (s >= g.m) return;                                           // wave-uniform
+    // One single-wavefront workgroup per (sample, block of 64 features).  The basis values of up to 64 pairs
+    // are evaluated once, KPAD lanes per pair, and parked in LDS; every lane then reads them back as
+    // broadcasts (four values per read) while it streams the feature rows of the neighbors.
+    constexpr int PARTS = 64 / KPAD;
+    constexpr int ROWS = 4;
+    __shared__ __attribute__((aligned(16))) float w_lds[64][KPAD];
+    const int lane = threadIdx.x;
+    const int64_t s = blockIdx.x;
     const int f = blockIdx.y * 64 + lane;
     const bool fvalid = f < g.c_in;
+    const int k = lane % KPAD, part = lane / KPAD;
     const int lo = s > 0 ? g.ends[s - 1] : 0;
     const int hi = g.ends[s];
     const float sx = g.samples[s * 3 + 0], sy = g.samples[s * 3 + 1], sz = g.samples[s * 3 + 2];
     const float ir0 = 1.0f / g.radii[0], ir1 = 1.0f / g.radii[1], ir2 = 1.0f / g.radii[2];
     LaneBasis<BASIS> lb;
-    lb.load(g, lane % KPAD);
+    lb.load(g, k);
 
     float acc[KPAD];
 #pragma unroll
-    for (int k = 0; k < KPAD; ++k) acc[k] = 0.0f;
+    for (int q = 0; q < KPAD; ++q) acc[q] = 0.0f;
 
     for (int cb = lo; cb < hi; cb += 64) {
-        const int t = cb + lane;
+        const int cnt = (hi - cb) < 64 ? (hi - cb) : 64;
         int nidx = 0;
         float dx = 0.f, dy = 0.f, dz = 0.f, pd = 1.0f;
-        if (t < hi) {
-            nidx = g.neigh[t].x;
+        if (lane < cnt) {
+            nidx = g.neigh[cb + lane].x;
             dx = (g.pts[(int64_t)nidx * 3 + 0] - sx) * ir0;
             dy = (g.pts[(int64_t)nidx * 3 + 1] - sy) * ir1;
             dz = (g.pts[(int64_t)nidx * 3 + 2] - sz) * ir2;
             if (BASIS == BASIS_MLP) pd = g.pdf[nidx];
         }
-        const int cnt = (hi - cb) < 64 ? (hi - cb) : 64;
-        for (int j0 = 0; j0 < cnt; j0 += 4) {
-            float row[4], wv[4];
+        for (int p = 0; p * PARTS < cnt; ++p) {
+            const int j = p * PARTS + part;
+            const float w = lb.eval(__shfl(dx, j), __shfl(dy, j), __shfl(dz, j), __shfl(pd, j), g.sigma);
+            w_lds[j][k] = (j < cnt) ? w : 0.0f;
+        }
+        __syncthreads();
+        for (int j0 = 0; j0 < cnt; j0 += ROWS) {
+            float row[ROWS];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int j = j0 + u;
-                row[u] = 0.0f;
-                wv[u] = 0.0f;
-                if (j < cnt) {                                      // uniform
-                    const int bn = pccnn_bcast_i(nidx, j);
-                    if (fvalid) row[u] = feats[(int64_t)bn * g.c_in + f];
-                    wv[u] = lb.eval(pccnn_bcast_f(dx, j), pccnn_bcast_f(dy, j), pccnn_bcast_f(dz, j),
-                                    pccnn_bcast_f(pd, j), g.sigma);
+            for (int u = 0; u < ROWS; ++u) {
+                const int bn = pccnn_bcast_i(nidx, (j0 + u) < cnt ? (j0 + u) : 0);
+                row[u] = (fvalid && (j0 + u) < cnt) ? feats[(int64_t)bn * g.c_in + f] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < ROWS; ++u) {
+                if (j0 + u < cnt) {                                 // uniform
+#pragma unroll
+                    for (int q = 0; q < KPAD; q += 4) {
+                        const float4 wv = *(const float4 *)&w_lds[j0 + u][q];
+                        acc[q] += row[u] * wv.x;
+                        acc[q + 1] += row[u] * wv.y;
+                        acc[q + 2] += row[u] * wv.z;
+                        acc[q + 3] += row[u] * wv.w;
+                    }
                 }
             }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-#pragma unroll
-                for (int k = 0; k < KPAD; ++k)
-                    acc[k] += row[u] * __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wv[u]), k));
-            }
         }
+        __syncthreads();
     }
     if (fvalid) {
         float *dst = proj + ((int64_t)s * g.c_in + f) * g.k;
         if (g.k == KPAD && (KPAD % 4) == 0) {
 #pragma unroll
-            for (int k = 0; k < KPAD; k += 4) {
-                float4 v = make_float4(acc[k], acc[k + 1], acc[k + 2], acc[k + 3]);
-                *(float4 *)(dst + k) = v;
+            for (int q = 0; q < KPAD; q += 4) {
+                float4 v = make_float4(acc[q], acc[q + 1], acc[q + 2], acc[q + 3]);
+                *(float4 *)(dst + q) = v;
             }
         } else {
 #pragma unroll
-            for (int k = 0; k < KPAD; ++k)
-                if (k < g.k) dst[k] = acc[k];
+            for (int q = 0; q < KPAD; ++q)
+                if (q < g.k) dst[q] = acc[q];
         }
     }
 }
@@ -145,11 +157,12 @@ conv_proj_fwd_kernel(ConvGeom g, const float *__restrict__ feats, float *__restr
 // the dF stage reads them as broadcasts; the neighbor's feature row is read coalesced from memory, used by
 // the dF stage from registers and handed to the dw stage through LDS, so that each stage runs KPAD
 // multiply-adds per pair and lane.  dw is accumulated in LDS over the feature blocks and stored coalesced.
-template <int BASIS, int KPAD>
+template <int BASIS, int KPAD, bool want_df, bool want_db>
 __global__ void __launch_bounds__(64)
 conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *__restrict__ proj_grads,
                      float *__restrict__ feat_grads, float *__restrict__ basis_grads)
 {
+    // want_df / want_db: which of the two stages this instantiation runs
     constexpr int PARTS = 64 / KPAD;                                // feature groups of the dw stage
     constexpr int ROWS = 4;                                         // feature rows in flight
     __shared__ __attribute__((aligned(16))) float w_lds[64][KPAD];
@@ -205,7 +218,7 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
                         if (q < g.k) gp[q] = src[q];
                 }
             }
-            if (k < g.k) {
+            if (want_db && k < g.k) {
 #pragma unroll
                 for (int q = 0; q < KPAD; ++q) {
                     const int ft = fb * 64 + part * KPAD + q;
@@ -220,34 +233,46 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
                     bn[u] = pccnn_bcast_i(nidx, (j0 + u) < cnt ? (j0 + u) : 0);
                     row[u] = (fvalid && (j0 + u) < cnt) ? feats[(int64_t)bn[u] * g.c_in + f] : 0.0f;
                 }
+                if (want_db) {
 #pragma unroll
-                for (int u = 0; u < ROWS; ++u) row_lds[u][lane] = row[u];
+                    for (int u = 0; u < ROWS; ++u) row_lds[u][lane] = row[u];
+                }
                 __syncthreads();
 #pragma unroll
                 for (int u = 0; u < ROWS; ++u) {
                     const int j = j0 + u;
                     if (j < cnt) {                                  // uniform
-                        float gf = 0.0f, acc = 0.0f;
+                        if (want_df) {
+                            float gf = 0.0f;
 #pragma unroll
-                        for (int q = 0; q < KPAD; q += 4) {
-                            const float4 wv = *(const float4 *)&w_lds[j][q];
-                            gf += gp[q] * wv.x + gp[q + 1] * wv.y + gp[q + 2] * wv.z + gp[q + 3] * wv.w;
-                            const float4 rv = *(const float4 *)&row_lds[u][part * KPAD + q];
-                            acc += gt[q] * rv.x + gt[q + 1] * rv.y + gt[q + 2] * rv.z + gt[q + 3] * rv.w;
+                            for (int q = 0; q < KPAD; q += 4) {
+                                const float4 wv = *(const float4 *)&w_lds[j][q];
+                                gf += gp[q] * wv.x + gp[q + 1] * wv.y + gp[q + 2] * wv.z + gp[q + 3] * wv.w;
+                            }
+                            if (fvalid) unsafeAtomicAdd(&feat_grads[(int64_t)bn[u] * g.c_in + f], gf);
                         }
-                        if (fvalid) unsafeAtomicAdd(&feat_grads[(int64_t)bn[u] * g.c_in + f], gf);
+                        if (want_db) {
+                            float acc = 0.0f;
 #pragma unroll
-                        for (int o = KPAD; o < 64; o <<= 1) acc += __shfl_xor(acc, o);
-                        if (part == 0) db_lds[j][k] += acc;
+                            for (int q = 0; q < KPAD; q += 4) {
+                                const float4 rv = *(const float4 *)&row_lds[u][part * KPAD + q];
+                                acc += gt[q] * rv.x + gt[q + 1] * rv.y + gt[q + 2] * rv.z + gt[q + 3] * rv.w;
+                            }
+#pragma unroll
+                            for (int o = KPAD; o < 64; o <<= 1) acc += __shfl_xor(acc, o);
+                            if (part == 0) db_lds[j][k] += acc;
+                        }
                     }
                 }
                 __syncthreads();
             }
         }
         __syncthreads();
-        for (int idx = lane; idx < cnt * KPAD; idx += 64) {
-            const int j = idx / KPAD, kk = idx % KPAD;
-            if (kk < g.k) basis_grads[(int64_t)(cb + j) * g.k + kk] = db_lds[j][kk];
+        if (want_db) {
+            for (int idx = lane; idx < cnt * KPAD; idx += 64) {
+                const int j = idx / KPAD, kk = idx % KPAD;
+                if (kk < g.k) basis_grads[(int64_t)(cb + j) * g.k + kk] = db_lds[j][kk];
+            }
         }
         __syncthreads();
     }
@@ -353,10 +378,12 @@ conv_basis_bwd_kernel(ConvGeom g, const float *__restrict__ basis_grads, float *
             }
             if (tv[u] && k == 0) {
                 gx *= ir0; gy *= ir1; gz *= ir2;
-                unsafeAtomicAdd(&d_pts[(int64_t)nidx[u] * 3 + 0], gx);
-                unsafeAtomicAdd(&d_pts[(int64_t)nidx[u] * 3 + 1], gy);
-                unsafeAtomicAdd(&d_pts[(int64_t)nidx[u] * 3 + 2], gz);
-                if (BASIS == BASIS_MLP) unsafeAtomicAdd(&d_pdf[nidx[u]], gpdf);
+                if (d_pts) {
+                    unsafeAtomicAdd(&d_pts[(int64_t)nidx[u] * 3 + 0], gx);
+                    unsafeAtomicAdd(&d_pts[(int64_t)nidx[u] * 3 + 1], gy);
+                    unsafeAtomicAdd(&d_pts[(int64_t)nidx[u] * 3 + 2], gz);
+                }
+                if (BASIS == BASIS_MLP && d_pdf) unsafeAtomicAdd(&d_pdf[nidx[u]], gpdf);
                 sgx += gx; sgy += gy; sgz += gz;
             }
         }
@@ -372,7 +399,7 @@ conv_basis_bwd_kernel(ConvGeom g, const float *__restrict__ basis_grads, float *
         p2 += __shfl_xor(p2, o);
         p3 += __shfl_xor(p3, o);
     }
-    if (svalid && lane == 0) {
+    if (svalid && lane == 0 && d_samples) {
         d_samples[s * 3 + 0] = -sgx;
         d_samples[s * 3 + 1] = -sgy;
         d_samples[s * 3 + 2] = -sgz;
@@ -410,7 +437,7 @@ conv_param_reduce_kernel(const float *__restrict__ partials, int64_t rows, int k
         if (threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
         __syncthreads();
     }
-    if (threadIdx.x == 0 && kk < k_basis) {
+    if (threadIdx.x == 0 && kk < k_basis && dst_a) {
         if (BASIS == BASIS_KP) {
             if (comp < 3) dst_a[kk * 3 + comp] = red[0];            // d_kernel_pts [K,3]
         } else {
@@ -457,29 +484,42 @@ static int kpad_of(int k) { return k <= 8 ? 8 : (k <= 16 ? 16 : (k <= 32 ? 32 : 
 template <int BASIS>
 static int launch_proj_fwd(const ConvGeom &g, const float *feats, float *proj, hipStream_t s)
 {
-    dim3 grid((unsigned)pccnn_ceil_div(g.m, 4), (unsigned)((g.c_in + 63) / 64));
+    dim3 grid((unsigned)g.m, (unsigned)((g.c_in + 63) / 64));
     PccnnTimed timed(PCCNN_T_PROJ_FWD, s);
     switch (kpad_of(g.k)) {
-    case 8: conv_proj_fwd_kernel<BASIS, 8><<<grid, 256, 0, s>>>(g, feats, proj); break;
-    case 16: conv_proj_fwd_kernel<BASIS, 16><<<grid, 256, 0, s>>>(g, feats, proj); break;
-    case 32: conv_proj_fwd_kernel<BASIS, 32><<<grid, 256, 0, s>>>(g, feats, proj); break;
-    default: conv_proj_fwd_kernel<BASIS, 64><<<grid, 256, 0, s>>>(g, feats, proj); break;
+    case 8: conv_proj_fwd_kernel<BASIS, 8><<<grid, 64, 0, s>>>(g, feats, proj); break;
+    case 16: conv_proj_fwd_kernel<BASIS, 16><<<grid, 64, 0, s>>>(g, feats, proj); break;
+    case 32: conv_proj_fwd_kernel<BASIS, 32><<<grid, 64, 0, s>>>(g, feats, proj); break;
+    default: conv_proj_fwd_kernel<BASIS, 64><<<grid, 64, 0, s>>>(g, feats, proj); break;
     }
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
+}
+
+template <int BASIS, int KPAD>
+static void launch_proj_bwd_k(const ConvGeom &g, const float *feats, const float *proj_grads, float *feat_grads,
+                              float *basis_grads, hipStream_t s)
+{
+    dim3 grid((unsigned)g.m);
+    if (feat_grads && basis_grads)
+        conv_proj_bwd_kernel<BASIS, KPAD, true, true><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads);
+    else if (feat_grads)
+        conv_proj_bwd_kernel<BASIS, KPAD, true, false><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads);
+    else
+        conv_proj_bwd_kernel<BASIS, KPAD, false, true><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads);
 }
 
 template <int BASIS>
 static int launch_proj_bwd(const ConvGeom &g, const float *feats, const float *proj_grads, float *feat_grads,
                            float *basis_grads, hipStream_t s)
 {
-    dim3 grid((unsigned)g.m);
+    if (!feat_grads && !basis_grads) return PCCNN_OK;
     PccnnTimed timed(PCCNN_T_PROJ_BWD, s);
     switch (kpad_of(g.k)) {
-    case 8: conv_proj_bwd_kernel<BASIS, 8><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads); break;
-    case 16: conv_proj_bwd_kernel<BASIS, 16><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads); break;
-    case 32: conv_proj_bwd_kernel<BASIS, 32><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads); break;
-    default: conv_proj_bwd_kernel<BASIS, 64><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads); break;
+    case 8: launch_proj_bwd_k<BASIS, 8>(g, feats, proj_grads, feat_grads, basis_grads, s); break;
+    case 16: launch_proj_bwd_k<BASIS, 16>(g, feats, proj_grads, feat_grads, basis_grads, s); break;
+    case 32: launch_proj_bwd_k<BASIS, 32>(g, feats, proj_grads, feat_grads, basis_grads, s); break;
+    default: launch_proj_bwd_k<BASIS, 64>(g, feats, proj_grads, feat_grads, basis_grads, s); break;
     }
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
@@ -524,84 +564,101 @@ static int contraction_fwd(const float *proj, const float *weights, float *out, 
                           inner * co, co, 1, nullptr, 0, s);
 }
 
-// d_proj[m, c_in*k] = dOut x W^T and d_weights = P^T x dOut.
-static int contraction_bwd(const float *proj, const float *weights, const float *in_grads, float *d_proj,
-                           float *d_weights, int64_t m, int c_in, int k, int num_mlps, int c_out, float *splitk_ws,
-                           size_t splitk_bytes, hipStream_t s)
-{
-    const int64_t inner = (int64_t)c_in * k / num_mlps;
-    const int64_t co = c_out / num_mlps;
-    int rc = pccnn_gemm_f32(in_grads, weights, d_proj, m, inner, co, 0, 1, c_out, co, (int64_t)c_in * k, num_mlps,
-                            co, inner * co, inner, 1, nullptr, 0, s);
-    if (rc != PCCNN_OK) return rc;
-    int split = (int)(m >= 4096 ? CONV_SPLIT_K : 1);
-    return pccnn_gemm_f32(proj, in_grads, d_weights, inner, co, m, 1, 0, (int64_t)c_in * k, c_out, co, num_mlps,
-                          inner, co, inner * co, split, splitk_ws, splitk_bytes, s);
-}
-
 template <int BASIS>
 static int conv_forward(ConvGeom g, const float *feats, const float *weights, int num_mlps, int c_out, float *out,
-                        void *workspace, size_t workspace_bytes, hipStream_t s)
+                        float *proj_out, void *workspace, size_t workspace_bytes, hipStream_t s)
 {
     if (g.m == 0) return PCCNN_OK;
-    PccnnArena arena(workspace, workspace_bytes);
-    float *proj = arena.take<float>((size_t)g.m * g.c_in * g.k);
-    PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv forward: workspace of %zu bytes, need %zu", workspace_bytes,
-                  pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 0));
+    float *proj = proj_out;
+    if (proj == nullptr) {
+        PccnnArena arena(workspace, workspace_bytes);
+        proj = arena.take<float>((size_t)g.m * g.c_in * g.k);
+        PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv forward: workspace of %zu bytes, need %zu",
+                      workspace_bytes, pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 0));
+    }
     int rc = launch_proj_fwd<BASIS>(g, feats, proj, s);
     if (rc != PCCNN_OK) return rc;
     return contraction_fwd(proj, weights, out, g.m, g.c_in, g.k, num_mlps, c_out, s);
 }
 
+// Gradients are produced only for the groups named in `mask`; pointers of groups not requested may be null.
 template <int BASIS>
 static int conv_backward(ConvGeom g, const float *feats, const float *weights, const float *in_grads, int num_mlps,
-                         int c_out, float *d_weights, float *d_feats, float *d_param_a, float *d_param_b,
-                         float *d_pdf, float *d_pts, float *d_samples, void *workspace, size_t workspace_bytes,
-                         hipStream_t s)
+                         int c_out, const float *proj_in, int mask, float *d_weights, float *d_feats,
+                         float *d_param_a, float *d_param_b, float *d_pdf, float *d_pts, float *d_samples,
+                         void *workspace, size_t workspace_bytes, hipStream_t s)
 {
     // d_param_a: d_kernel_pts [K,3] (KP) or d_axis [3,K] (MLP); d_param_b: d_bias [K] (MLP only)
     const int count_a = 3 * g.k, count_b = (BASIS == BASIS_KP ? 0 : g.k);
+    const bool want_w = mask & PCCNN_GRAD_WEIGHTS, want_f = mask & PCCNN_GRAD_FEATS;
+    const bool want_par = mask & PCCNN_GRAD_BASIS_PARAMS, want_pts = mask & PCCNN_GRAD_PTS;
+    const bool want_pdf = (mask & PCCNN_GRAD_PDF) && BASIS == BASIS_MLP;
+    const bool want_basis = want_par || want_pts || want_pdf;
     int rc;
     PccnnArena arena(workspace, workspace_bytes);
     const int64_t partial_rows = pccnn_ceil_div(g.m > 0 ? g.m : 1, 4);
     float *partials = arena.take<float>((size_t)partial_rows * 256);
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv backward: workspace of %zu bytes, need %zu", workspace_bytes,
                   pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 1));
-    if ((rc = pccnn_fill_f32(d_feats, 0.0f, g.n * g.c_in, s)) != PCCNN_OK) return rc;
-    if ((rc = pccnn_fill_f32(d_pts, 0.0f, g.n * 3, s)) != PCCNN_OK) return rc;
-    if (d_pdf && (rc = pccnn_fill_f32(d_pdf, 0.0f, g.n, s)) != PCCNN_OK) return rc;
+    if (want_f && (rc = pccnn_fill_f32(d_feats, 0.0f, g.n * g.c_in, s)) != PCCNN_OK) return rc;
+    if (want_pts && (rc = pccnn_fill_f32(d_pts, 0.0f, g.n * 3, s)) != PCCNN_OK) return rc;
+    if (want_pdf && (rc = pccnn_fill_f32(d_pdf, 0.0f, g.n, s)) != PCCNN_OK) return rc;
     if (g.m == 0 || g.t == 0) {
-        if ((rc = pccnn_fill_f32(d_samples, 0.0f, g.m * 3, s)) != PCCNN_OK) return rc;
-        if ((rc = pccnn_fill_f32(d_param_a, 0.0f, count_a, s)) != PCCNN_OK) return rc;
-        if (count_b && (rc = pccnn_fill_f32(d_param_b, 0.0f, count_b, s)) != PCCNN_OK) return rc;
-        return pccnn_fill_f32(d_weights, 0.0f, (int64_t)g.c_in * g.k * c_out / num_mlps, s);
+        if (want_pts && (rc = pccnn_fill_f32(d_samples, 0.0f, g.m * 3, s)) != PCCNN_OK) return rc;
+        if (want_par && (rc = pccnn_fill_f32(d_param_a, 0.0f, count_a, s)) != PCCNN_OK) return rc;
+        if (want_par && count_b && (rc = pccnn_fill_f32(d_param_b, 0.0f, count_b, s)) != PCCNN_OK) return rc;
+        if (want_w) return pccnn_fill_f32(d_weights, 0.0f, (int64_t)g.c_in * g.k * c_out / num_mlps, s);
+        return PCCNN_OK;
     }
 
-    float *proj = arena.take<float>((size_t)g.m * g.c_in * g.k);
-    float *d_proj = arena.take<float>((size_t)g.m * g.c_in * g.k);
+    const size_t proj_elems = (size_t)g.m * g.c_in * g.k;
+    float *proj_ws = arena.take<float>(proj_elems);
+    float *d_proj = arena.take<float>(proj_elems);
     float *basis_g = arena.take<float>((size_t)g.t * g.k);
     size_t splitk_elems = (size_t)CONV_SPLIT_K * g.c_in * g.k * c_out;
     float *splitk = arena.take<float>(splitk_elems);
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv backward: workspace of %zu bytes, need %zu", workspace_bytes,
                   pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 1));
-    if ((rc = launch_proj_fwd<BASIS>(g, feats, proj, s)) != PCCNN_OK) return rc;
-    if ((rc = contraction_bwd(proj, weights, in_grads, d_proj, d_weights, g.m, g.c_in, g.k, num_mlps, c_out, splitk,
-                              splitk_elems * sizeof(float), s)) != PCCNN_OK)
+    const int64_t inner = (int64_t)g.c_in * g.k / num_mlps;
+    const int64_t co = c_out / num_mlps;
+    if (want_w) {
+        // d_weights = P^T x dOut; P comes from the caller (kept from the forward call) or is rebuilt here
+        const float *proj = proj_in;
+        if (proj == nullptr) {
+            if ((rc = launch_proj_fwd<BASIS>(g, feats, proj_ws, s)) != PCCNN_OK) return rc;
+            proj = proj_ws;
+        }
+        const int split = (int)(g.m >= 4096 ? CONV_SPLIT_K : 1);
+        rc = pccnn_gemm_f32(proj, in_grads, d_weights, inner, co, g.m, 1, 0, (int64_t)g.c_in * g.k, c_out, co, num_mlps,
+                            inner, co, inner * co, split, splitk, splitk_elems * sizeof(float), s);
+        if (rc != PCCNN_OK) return rc;
+    }
+    if (!want_f && !want_basis) return PCCNN_OK;
+    // d_proj = dOut x W^T
+    rc = pccnn_gemm_f32(in_grads, weights, d_proj, g.m, inner, co, 0, 1, c_out, co, (int64_t)g.c_in * g.k, num_mlps, co,
+                        inner * co, inner, 1, nullptr, 0, s);
+    if (rc != PCCNN_OK) return rc;
+    if ((rc = launch_proj_bwd<BASIS>(g, feats, d_proj, want_f ? d_feats : nullptr, want_basis ? basis_g : nullptr,
+                                     s)) != PCCNN_OK)
         return rc;
-    if ((rc = launch_proj_bwd<BASIS>(g, feats, d_proj, d_feats, basis_g, s)) != PCCNN_OK) return rc;
+    if (!want_basis) return PCCNN_OK;
     const unsigned blocks = (unsigned)partial_rows;
+    float *o_pts = want_pts ? d_pts : nullptr, *o_smp = want_pts ? d_samples : nullptr;
+    float *o_pdf = want_pdf ? d_pdf : nullptr;
     {
         PccnnTimed timed(PCCNN_T_BASIS_BWD, s);
         switch (kpad_of(g.k)) {
-        case 8: conv_basis_bwd_kernel<BASIS, 8><<<blocks, 256, 0, s>>>(g, basis_g, d_pts, d_samples, d_pdf, partials); break;
-        case 16: conv_basis_bwd_kernel<BASIS, 16><<<blocks, 256, 0, s>>>(g, basis_g, d_pts, d_samples, d_pdf, partials); break;
-        case 32: conv_basis_bwd_kernel<BASIS, 32><<<blocks, 256, 0, s>>>(g, basis_g, d_pts, d_samples, d_pdf, partials); break;
-        default: conv_basis_bwd_kernel<BASIS, 64><<<blocks, 256, 0, s>>>(g, basis_g, d_pts, d_samples, d_pdf, partials); break;
+        case 8: conv_basis_bwd_kernel<BASIS, 8><<<blocks, 256, 0, s>>>(g, basis_g, o_pts, o_smp, o_pdf, partials); break;
+        case 16: conv_basis_bwd_kernel<BASIS, 16><<<blocks, 256, 0, s>>>(g, basis_g, o_pts, o_smp, o_pdf, partials); break;
+        case 32: conv_basis_bwd_kernel<BASIS, 32><<<blocks, 256, 0, s>>>(g, basis_g, o_pts, o_smp, o_pdf, partials); break;
+        default: conv_basis_bwd_kernel<BASIS, 64><<<blocks, 256, 0, s>>>(g, basis_g, o_pts, o_smp, o_pdf, partials); break;
         }
     }
     PCCNN_LAUNCH_CHECK();
-    conv_param_reduce_kernel<BASIS><<<256, 256, 0, s>>>(partials, partial_rows, g.k, d_param_a, d_param_b);
-    PCCNN_LAUNCH_CHECK();
+    if (want_par) {
+        conv_param_reduce_kernel<BASIS><<<256, 256, 0, s>>>(partials, partial_rows, g.k, d_param_a, d_param_b);
+        PCCNN_LAUNCH_CHECK();
+    }
     return PCCNN_OK;
 }
 
@@ -662,7 +719,8 @@ extern "C" int pccnn_mcconv_weight_var(const float *pts, const float *pdf, const
 extern "C" int pccnn_kpconv_forward(const float *pts, const float *feats, const float *samples, const int32_t *neigh,
                                     const int32_t *ends, const float *radii, const float *kernel_pts, float sigma,
                                     const float *weights, int64_t n, int64_t m, int64_t t, int d, int c_in, int k,
-                                    int c_out, float *out, void *workspace, size_t workspace_bytes, void *stream)
+                                    int c_out, float *out, float *proj_out, void *workspace, size_t workspace_bytes,
+                                    void *stream)
 {
     int rc = conv_validate("pccnn_kpconv_forward", n, m, t, d, c_in, k, 1, c_out);
     if (rc != PCCNN_OK) return rc;
@@ -670,32 +728,39 @@ extern "C" int pccnn_kpconv_forward(const float *pts, const float *feats, const 
     PCCNN_REQUIRE(m == 0 || (pts && feats && samples && ends && radii && kernel_pts && weights && out && (t == 0 || neigh)),
                   PCCNN_ERR_INVALID, "pccnn_kpconv_forward: null pointer");
     ConvGeom g = {pts, samples, (const int2 *)neigh, ends, radii, nullptr, kernel_pts, nullptr, sigma, n, m, t, c_in, k};
-    return conv_forward<BASIS_KP>(g, feats, weights, 1, c_out, out, workspace, workspace_bytes, (hipStream_t)stream);
+    return conv_forward<BASIS_KP>(g, feats, weights, 1, c_out, out, proj_out, workspace, workspace_bytes,
+                                  (hipStream_t)stream);
 }
 
 extern "C" int pccnn_kpconv_backward(const float *pts, const float *feats, const float *samples,
                                      const int32_t *neigh, const int32_t *ends, const float *radii,
                                      const float *kernel_pts, float sigma, const float *weights,
-                                     const float *in_grads, int64_t n, int64_t m, int64_t t, int d, int c_in, int k,
-                                     int c_out, float *d_weights, float *d_feats, float *d_kernel_pts, float *d_pts,
-                                     float *d_samples, void *workspace, size_t workspace_bytes, void *stream)
+                                     const float *in_grads, const float *proj, int grad_mask, int64_t n, int64_t m,
+                                     int64_t t, int d, int c_in, int k, int c_out, float *d_weights, float *d_feats,
+                                     float *d_kernel_pts, float *d_pts, float *d_samples, void *workspace,
+                                     size_t workspace_bytes, void *stream)
 {
     int rc = conv_validate("pccnn_kpconv_backward", n, m, t, d, c_in, k, 1, c_out);
     if (rc != PCCNN_OK) return rc;
     PCCNN_REQUIRE(sigma > 0.0f, PCCNN_ERR_INVALID, "pccnn_kpconv_backward: sigma=%g", sigma);
-    PCCNN_REQUIRE(d_weights && d_kernel_pts && kernel_pts && weights && radii && (n == 0 || (d_feats && d_pts && pts && feats)) &&
-                      (m == 0 || (d_samples && samples && ends && in_grads)) && (t == 0 || neigh),
-                  PCCNN_ERR_INVALID, "pccnn_kpconv_backward: null pointer");
+    PCCNN_REQUIRE(kernel_pts && weights && radii && (n == 0 || (pts && feats)) &&
+                      (m == 0 || (samples && ends && in_grads)) && (t == 0 || neigh),
+                  PCCNN_ERR_INVALID, "pccnn_kpconv_backward: null input pointer");
+    PCCNN_REQUIRE((!(grad_mask & PCCNN_GRAD_WEIGHTS) || d_weights) && (!(grad_mask & PCCNN_GRAD_FEATS) || d_feats || n == 0) &&
+                      (!(grad_mask & PCCNN_GRAD_BASIS_PARAMS) || d_kernel_pts) &&
+                      (!(grad_mask & PCCNN_GRAD_PTS) || ((d_pts || n == 0) && (d_samples || m == 0))),
+                  PCCNN_ERR_INVALID, "pccnn_kpconv_backward: a requested gradient has a null output pointer");
     ConvGeom g = {pts, samples, (const int2 *)neigh, ends, radii, nullptr, kernel_pts, nullptr, sigma, n, m, t, c_in, k};
-    return conv_backward<BASIS_KP>(g, feats, weights, in_grads, 1, c_out, d_weights, d_feats, d_kernel_pts, nullptr,
-                                   nullptr, d_pts, d_samples, workspace, workspace_bytes, (hipStream_t)stream);
+    return conv_backward<BASIS_KP>(g, feats, weights, in_grads, 1, c_out, proj, grad_mask, d_weights, d_feats,
+                                   d_kernel_pts, nullptr, nullptr, d_pts, d_samples, workspace, workspace_bytes,
+                                   (hipStream_t)stream);
 }
 
 extern "C" int pccnn_mcconv_forward(const float *pts, const float *pdf, const float *feats, const float *samples,
                                     const int32_t *neigh, const int32_t *ends, const float *radii, const float *axis,
                                     const float *bias, const float *weights, int64_t n, int64_t m, int64_t t, int d,
-                                    int c_in, int k, int num_mlps, int c_out, float *out, void *workspace,
-                                    size_t workspace_bytes, void *stream)
+                                    int c_in, int k, int num_mlps, int c_out, float *out, float *proj_out,
+                                    void *workspace, size_t workspace_bytes, void *stream)
 {
     int rc = conv_validate("pccnn_mcconv_forward", n, m, t, d, c_in, k, num_mlps, c_out);
     if (rc != PCCNN_OK) return rc;
@@ -703,25 +768,30 @@ extern "C" int pccnn_mcconv_forward(const float *pts, const float *pdf, const fl
                              (t == 0 || neigh)),
                   PCCNN_ERR_INVALID, "pccnn_mcconv_forward: null pointer");
     ConvGeom g = {pts, samples, (const int2 *)neigh, ends, radii, pdf, axis, bias, 1.0f, n, m, t, c_in, k};
-    return conv_forward<BASIS_MLP>(g, feats, weights, num_mlps, c_out, out, workspace, workspace_bytes,
+    return conv_forward<BASIS_MLP>(g, feats, weights, num_mlps, c_out, out, proj_out, workspace, workspace_bytes,
                                    (hipStream_t)stream);
 }
 
 extern "C" int pccnn_mcconv_backward(const float *pts, const float *pdf, const float *feats, const float *samples,
                                      const int32_t *neigh, const int32_t *ends, const float *radii,
                                      const float *axis, const float *bias, const float *weights,
-                                     const float *in_grads, int64_t n, int64_t m, int64_t t, int d, int c_in, int k,
-                                     int num_mlps, int c_out, float *d_weights, float *d_feats, float *d_axis,
-                                     float *d_bias, float *d_pdf, float *d_pts, float *d_samples, void *workspace,
-                                     size_t workspace_bytes, void *stream)
+                                     const float *in_grads, const float *proj, int grad_mask, int64_t n, int64_t m,
+                                     int64_t t, int d, int c_in, int k, int num_mlps, int c_out, float *d_weights,
+                                     float *d_feats, float *d_axis, float *d_bias, float *d_pdf, float *d_pts,
+                                     float *d_samples, void *workspace, size_t workspace_bytes, void *stream)
 {
     int rc = conv_validate("pccnn_mcconv_backward", n, m, t, d, c_in, k, num_mlps, c_out);
     if (rc != PCCNN_OK) return rc;
-    PCCNN_REQUIRE(d_weights && d_axis && d_bias && axis && bias && weights && radii &&
-                      (n == 0 || (d_feats && d_pts && d_pdf && pts && pdf && feats)) &&
-                      (m == 0 || (d_samples && samples && ends && in_grads)) && (t == 0 || neigh),
-                  PCCNN_ERR_INVALID, "pccnn_mcconv_backward: null pointer");
+    PCCNN_REQUIRE(axis && bias && weights && radii && (n == 0 || (pts && pdf && feats)) &&
+                      (m == 0 || (samples && ends && in_grads)) && (t == 0 || neigh),
+                  PCCNN_ERR_INVALID, "pccnn_mcconv_backward: null input pointer");
+    PCCNN_REQUIRE((!(grad_mask & PCCNN_GRAD_WEIGHTS) || d_weights) && (!(grad_mask & PCCNN_GRAD_FEATS) || d_feats || n == 0) &&
+                      (!(grad_mask & PCCNN_GRAD_BASIS_PARAMS) || (d_axis && d_bias)) &&
+                      (!(grad_mask & PCCNN_GRAD_PDF) || d_pdf || n == 0) &&
+                      (!(grad_mask & PCCNN_GRAD_PTS) || ((d_pts || n == 0) && (d_samples || m == 0))),
+                  PCCNN_ERR_INVALID, "pccnn_mcconv_backward: a requested gradient has a null output pointer");
     ConvGeom g = {pts, samples, (const int2 *)neigh, ends, radii, pdf, axis, bias, 1.0f, n, m, t, c_in, k};
-    return conv_backward<BASIS_MLP>(g, feats, weights, in_grads, num_mlps, c_out, d_weights, d_feats, d_axis, d_bias,
-                                    d_pdf, d_pts, d_samples, workspace, workspace_bytes, (hipStream_t)stream);
+    return conv_backward<BASIS_MLP>(g, feats, weights, in_grads, num_mlps, c_out, proj, grad_mask, d_weights, d_feats,
+                                    d_axis, d_bias, d_pdf, d_pts, d_samples, workspace, workspace_bytes,
+                                    (hipStream_t)stream);
 }

@@ -29,9 +29,10 @@ struct GemmArgs {
 
 // Global -> registers for one 128 x 16 operand tile.  `KCONTIG`: the reduction index is the
 // contiguous one in memory (element (x, k) at p[x * ld + k]); otherwise element (x, k) at p[k * ld + x].
-template <bool KCONTIG>
+// `FAST`: the tile is fully inside the matrix and 16-byte aligned, so it is read with float4 loads.
+template <bool KCONTIG, bool FAST>
 __device__ __forceinline__ void tile_load(const float *__restrict__ p, int64_t ld, int64_t x0, int64_t x_end,
-                                          int64_t k0, int64_t k_end, bool fast, float4 (&r)[2])
+                                          int64_t k0, int64_t k_end, float4 (&r)[2])
 {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -39,7 +40,7 @@ __device__ __forceinline__ void tile_load(const float *__restrict__ p, int64_t l
         int64_t x, k;
         if (KCONTIG) { x = x0 + idx / 4; k = k0 + (idx % 4) * 4; }
         else { k = k0 + idx / 32; x = x0 + (idx % 32) * 4; }
-        if (fast) {
+        if (FAST) {
             r[i] = KCONTIG ? *(const float4 *)(p + x * ld + k) : *(const float4 *)(p + k * ld + x);
         } else {
             float v[4];
@@ -74,6 +75,66 @@ __device__ __forceinline__ void tile_store(float (*lds)[GT_LD], const float4 (&r
     }
 }
 
+// The k loop of one workgroup tile.  Global loads of tile kt+1 are issued before the MFMAs of tile kt and
+// parked in LDS after them; inside a tile the LDS fragments of sub-step ks+1 are read before the MFMAs of
+// sub-step ks are issued, so the matrix pipe never waits on an LDS round trip.
+template <bool AT, bool BT, bool FAST>
+__device__ __forceinline__ void gemm_tile_loop(const GemmArgs &g, const float *__restrict__ a,
+                                               const float *__restrict__ b, int64_t bm, int64_t bn, int64_t k_begin,
+                                               int64_t k_end, float (*As)[GT_K][GT_LD], float (*Bs)[GT_K][GT_LD],
+                                               floatx16 (&acc)[2][2])
+{
+    const int lane = pccnn_lane();
+    const int wave = threadIdx.x >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int frag_k = lane >> 5, frag_c = lane & 31;
+    float4 ra[2], rb[2];
+    const int64_t nk = (k_end - k_begin + GT_K - 1) / GT_K;
+    if (nk > 0) {
+        // A stored [rows, inner] (AT = false) has the reduction index contiguous; B stored
+        // [inner, cols] (BT = false) has the column index contiguous.
+        tile_load<!AT, FAST>(a, g.lda, bm, g.rows, k_begin, k_end, ra);
+        tile_load<BT, FAST>(b, g.ldb, bn, g.cols, k_begin, k_end, rb);
+        tile_store<!AT>(As[0], ra);
+        tile_store<BT>(Bs[0], rb);
+    }
+    __syncthreads();
+    for (int64_t kt = 0; kt < nk; ++kt) {
+        const int buf = (int)(kt & 1);
+        const bool more = kt + 1 < nk;
+        if (more) {
+            const int64_t k0 = k_begin + (kt + 1) * GT_K;
+            tile_load<!AT, FAST>(a, g.lda, bm, g.rows, k0, k_end, ra);
+            tile_load<BT, FAST>(b, g.ldb, bn, g.cols, k0, k_end, rb);
+        }
+        float fa[2][2], fb[2][2];
+        fa[0][0] = As[buf][frag_k][wm * 64 + frag_c];
+        fa[0][1] = As[buf][frag_k][wm * 64 + 32 + frag_c];
+        fb[0][0] = Bs[buf][frag_k][wn * 64 + frag_c];
+        fb[0][1] = Bs[buf][frag_k][wn * 64 + 32 + frag_c];
+#pragma unroll
+        for (int ks = 0; ks < GT_K / 2; ++ks) {
+            const int cur = ks & 1, nxt = cur ^ 1;
+            if (ks + 1 < GT_K / 2) {
+                const int kr = 2 * (ks + 1) + frag_k;
+                fa[nxt][0] = As[buf][kr][wm * 64 + frag_c];
+                fa[nxt][1] = As[buf][kr][wm * 64 + 32 + frag_c];
+                fb[nxt][0] = Bs[buf][kr][wn * 64 + frag_c];
+                fb[nxt][1] = Bs[buf][kr][wn * 64 + 32 + frag_c];
+            }
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][0], fb[cur][0], acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][0], fb[cur][1], acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][1], fb[cur][0], acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][1], fb[cur][1], acc[1][1], 0, 0, 0);
+        }
+        if (more) {
+            tile_store<!AT>(As[buf ^ 1], ra);
+            tile_store<BT>(Bs[buf ^ 1], rb);
+        }
+        __syncthreads();
+    }
+}
+
 template <bool AT, bool BT>
 __global__ void __launch_bounds__(256)
 gemm_f32_mfma_kernel(GemmArgs g, float *__restrict__ partial)
@@ -102,44 +163,8 @@ gemm_f32_mfma_kernel(GemmArgs g, float *__restrict__ partial)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    float4 ra[2], rb[2];
-    const int64_t nk = (k_end - k_begin + GT_K - 1) / GT_K;
-    if (nk > 0) {
-        // A stored [rows, inner] (AT = false) has the reduction index contiguous; B stored
-        // [inner, cols] (BT = false) has the column index contiguous.
-        tile_load<!AT>(a, g.lda, bm, g.rows, k_begin, k_end, fast, ra);
-        tile_load<BT>(b, g.ldb, bn, g.cols, k_begin, k_end, fast, rb);
-        tile_store<!AT>(As[0], ra);
-        tile_store<BT>(Bs[0], rb);
-    }
-    __syncthreads();
-    for (int64_t kt = 0; kt < nk; ++kt) {
-        const int buf = (int)(kt & 1);
-        const bool more = kt + 1 < nk;
-        if (more) {
-            const int64_t k0 = k_begin + (kt + 1) * GT_K;
-            tile_load<!AT>(a, g.lda, bm, g.rows, k0, k_end, fast, ra);
-            tile_load<BT>(b, g.ldb, bn, g.cols, k0, k_end, fast, rb);
-        }
-#pragma unroll
-        for (int ks = 0; ks < GT_K / 2; ++ks) {
-            const int kr = 2 * ks + (lane >> 5);
-            const int c = lane & 31;
-            const float a0 = As[buf][kr][wm * 64 + c];
-            const float a1 = As[buf][kr][wm * 64 + 32 + c];
-            const float b0 = Bs[buf][kr][wn * 64 + c];
-            const float b1 = Bs[buf][kr][wn * 64 + 32 + c];
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
-        }
-        if (more) {
-            tile_store<!AT>(As[buf ^ 1], ra);
-            tile_store<BT>(Bs[buf ^ 1], rb);
-        }
-        __syncthreads();
-    }
+    if (fast) gemm_tile_loop<AT, BT, true>(g, a, b, bm, bn, k_begin, k_end, As, Bs, acc);
+    else gemm_tile_loop<AT, BT, false>(g, a, b, bm, bn, k_begin, k_end, As, Bs, acc);
 
     // Accumulator layout of the 32x32 MFMA: register v of lane l holds
     // row 8*(v/4) + 4*(l/32) + v%4, column l%32 of the tile.

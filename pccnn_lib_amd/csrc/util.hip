@@ -35,14 +35,14 @@ PccnnTimed::PccnnTimed(int id_, hipStream_t s) : id(id_), stream(s), stop(nullpt
     if (!on) return;
     hipEvent_t start;
     if (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess) { on = false; return; }
-    hipEventRecord(start, stream);
+    (void)hipEventRecord(start, stream);
     std::lock_guard<std::mutex> lk(g_timing_mu);
     g_timing_pending[id].push_back({start, stop});
 }
 
 PccnnTimed::~PccnnTimed()
 {
-    if (on) hipEventRecord(stop, stream);
+    if (on) (void)hipEventRecord(stop, stream);
 }
 
 static void timing_drain()
@@ -54,8 +54,8 @@ static void timing_drain()
                 g_timing_ms[i] += ms;
                 g_timing_n[i] += 1;
             }
-            hipEventDestroy(pr.start);
-            hipEventDestroy(pr.stop);
+            (void)hipEventDestroy(pr.start);
+            (void)hipEventDestroy(pr.stop);
         }
         g_timing_pending[i].clear();
     }

@@ -6,23 +6,30 @@ from .. import pccnn_lib_ops
 class ComputeKPConv(torch.autograd.Function):
     """apply(pts, features, samples, neighbors, start_ids, radii, kernel_pts, sigma, conv_weights) -> [M, Cout].
     Gradients are routed to (pts, features, samples, -, -, -, kernel_pts, -, conv_weights)
-    (pccnn_lib/op_wrappers/compute_kpconv.py:14-73)."""
+    (pccnn_lib/op_wrappers/compute_kpconv.py:14-73).  The projection built by the forward pass is kept for the
+    backward pass, and only the gradients autograd asks for are computed."""
 
     @staticmethod
     def forward(ctx, p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_kernel_pts, p_sigma,
                 p_conv_weights):
+        out, proj = pccnn_lib_ops.kp_conv(p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii,
+                                          p_kernel_pts, p_sigma, p_conv_weights, return_proj=True)
         ctx.save_for_backward(p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_kernel_pts,
-                              p_conv_weights)
+                              p_conv_weights, proj)
         ctx.sigma_ = p_sigma
-        return pccnn_lib_ops.kp_conv(p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_kernel_pts,
-                                     p_sigma, p_conv_weights)
+        return out
 
     @staticmethod
     def backward(ctx, p_grads):
-        pts, features, samples, neighbors, start_ids, radii, kernel_pts, conv_weights = ctx.saved_tensors
+        pts, features, samples, neighbors, start_ids, radii, kernel_pts, conv_weights, proj = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        mask = (pccnn_lib_ops.GRAD_PTS if (need[0] or need[2]) else 0) | (pccnn_lib_ops.GRAD_FEATS if need[1] else 0) \
+            | (pccnn_lib_ops.GRAD_BASIS_PARAMS if need[6] else 0) | (pccnn_lib_ops.GRAD_WEIGHTS if need[8] else 0)
         weight_grads, feat_grads, kernel_pts_grads, pt_grads, sample_grads = pccnn_lib_ops.kp_conv_grads(
-            pts, features, samples, neighbors, start_ids, radii, kernel_pts, ctx.sigma_, conv_weights, p_grads)
-        return pt_grads, feat_grads, sample_grads, None, None, None, kernel_pts_grads, None, weight_grads
+            pts, features, samples, neighbors, start_ids, radii, kernel_pts, ctx.sigma_, conv_weights, p_grads,
+            proj=proj, grad_mask=mask)
+        return pt_grads if need[0] else None, feat_grads, sample_grads if need[2] else None, None, None, None, \
+            kernel_pts_grads, None, weight_grads
 
 
 class ComputeKPConvWeightVar(torch.autograd.Function):

@@ -6,23 +6,31 @@ from .. import pccnn_lib_ops
 class ComputeMCConv(torch.autograd.Function):
     """apply(pts, pdf, features, samples, neighbors, start_ids, radii, proj_axis, proj_bias, conv_weights)
     -> [M, Cout].  Gradients are routed to (pts, pdf, features, samples, -, -, -, proj_axis, proj_bias,
-    conv_weights) (pccnn_lib/op_wrappers/compute_mcconv.py:14-75)."""
+    conv_weights) (pccnn_lib/op_wrappers/compute_mcconv.py:14-75).  The projection built by the forward pass is
+    kept for the backward pass, and only the gradients autograd asks for are computed."""
 
     @staticmethod
     def forward(ctx, p_pts, p_pdf, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_proj_axis,
                 p_proj_bias, p_conv_weights):
+        out, proj = pccnn_lib_ops.mc_conv(p_pts, p_pdf, p_features, p_samples, p_neighbors, p_start_ids, p_radii,
+                                          p_proj_axis, p_proj_bias, p_conv_weights, return_proj=True)
         ctx.save_for_backward(p_pts, p_pdf, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_proj_axis,
-                              p_proj_bias, p_conv_weights)
-        return pccnn_lib_ops.mc_conv(p_pts, p_pdf, p_features, p_samples, p_neighbors, p_start_ids, p_radii,
-                                     p_proj_axis, p_proj_bias, p_conv_weights)
+                              p_proj_bias, p_conv_weights, proj)
+        return out
 
     @staticmethod
     def backward(ctx, p_grads):
-        pts, pdf, features, samples, neighbors, start_ids, radii, axis, bias, conv_weights = ctx.saved_tensors
+        pts, pdf, features, samples, neighbors, start_ids, radii, axis, bias, conv_weights, proj = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        ops = pccnn_lib_ops
+        mask = (ops.GRAD_PTS if (need[0] or need[3]) else 0) | (ops.GRAD_PDF if need[1] else 0) \
+            | (ops.GRAD_FEATS if need[2] else 0) | (ops.GRAD_BASIS_PARAMS if (need[7] or need[8]) else 0) \
+            | (ops.GRAD_WEIGHTS if need[9] else 0)
         weight_grads, feat_grads, axis_grads, bias_grads, pdf_grads, pt_grads, sample_grads = \
-            pccnn_lib_ops.mc_conv_grads(pts, pdf, features, samples, neighbors, start_ids, radii, axis, bias,
-                                        conv_weights, p_grads)
-        return pt_grads, pdf_grads, feat_grads, sample_grads, None, None, None, axis_grads, bias_grads, weight_grads
+            ops.mc_conv_grads(pts, pdf, features, samples, neighbors, start_ids, radii, axis, bias, conv_weights,
+                              p_grads, proj=proj, grad_mask=mask)
+        return pt_grads if need[0] else None, pdf_grads, feat_grads, sample_grads if need[3] else None, None, None, \
+            None, axis_grads if need[7] else None, bias_grads if need[8] else None, weight_grads
 
 
 class ComputeMCConvWeightVar(torch.autograd.Function):

@@ -286,6 +286,10 @@ def poisson_disk_sampling(sorted_keys, neigh, ends, grid_size):
 
 # ----------------------------------------------------------------------------- conv
 
+# Gradient groups of the backward entry points (PCCNN_GRAD_* in include/pccnn_hip.h).
+GRAD_WEIGHTS, GRAD_FEATS, GRAD_BASIS_PARAMS, GRAD_PDF, GRAD_PTS, GRAD_ALL = 1, 2, 4, 8, 16, 31
+
+
 
 def _conv_args(name, pts, feats, samples, neigh, ends, radii):
     _chk(pts, name + ": pts", torch.float32, 2)
@@ -302,9 +306,10 @@ def _conv_args(name, pts, feats, samples, neigh, ends, radii):
     return d, dev
 
 
-def kp_conv(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights):
+def kp_conv(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights, return_proj=False):
     """kp_conv(pts, feats, samples, neighbors, start_ids, radii, kernel_pts f32[K,D], sigma, weights f32[K*Cin,Cout])
-    -> f32[M,Cout] (pccnn_lib_ops/pcconvs/kpconv.cuh:32-41)."""
+    -> f32[M,Cout] (pccnn_lib_ops/pcconvs/kpconv.cuh:32-41).  ``return_proj=True`` also returns the projection
+    f32[M,Cin,K] the call built, for kp_conv_grads(..., proj=...)."""
     name = "kp_conv"
     d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
     _chk(kernel_pts, name + ": kernel_pts", torch.float32, 2, dev)
@@ -314,16 +319,18 @@ def kp_conv(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights)
     if kernel_pts.shape[1] != d or weights.shape[0] != k * c_in:
         raise RuntimeError(name + ": weights must be [K*Cin, Cout] and kernel_pts [K, D]")
     out = torch.empty((m, c_out), dtype=torch.float32, device=dev)
-    ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 0), dev)
+    proj = torch.empty((m, c_in, k), dtype=torch.float32, device=dev)
     _lib.call("pccnn_kpconv_forward", _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends), _ptr(radii),
-              _ptr(kernel_pts), float(sigma), _ptr(weights), n, m, t, d, c_in, k, c_out, _ptr(out), _ptr(ws),
-              ws.numel(), _stream())
-    return out
+              _ptr(kernel_pts), float(sigma), _ptr(weights), n, m, t, d, c_in, k, c_out, _ptr(out), _ptr(proj),
+              _P(0), 0, _stream())
+    return (out, proj) if return_proj else out
 
 
-def kp_conv_grads(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights, in_grads):
+def kp_conv_grads(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights, in_grads, proj=None,
+                  grad_mask=GRAD_ALL):
     """kp_conv_grads(..., in_grads f32[M,Cout]) -> [dW, dFeat, dKernelPts, dPts, dSamples]
-    (pccnn_lib_ops/pcconvs/kpconv.cuh:56-67)."""
+    (pccnn_lib_ops/pcconvs/kpconv.cuh:56-67).  ``proj``: projection kept from kp_conv(return_proj=True);
+    ``grad_mask``: GRAD_* groups to compute, the others come back as None."""
     name = "kp_conv_grads"
     d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
     _chk(kernel_pts, name + ": kernel_pts", torch.float32, 2, dev)
@@ -333,13 +340,29 @@ def kp_conv_grads(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, we
         weights.shape[1]
     if kernel_pts.shape[1] != d or weights.shape[0] != k * c_in or tuple(in_grads.shape) != (m, c_out):
         raise RuntimeError(name + ": inconsistent shapes")
-    d_w, d_f = torch.empty_like(weights), torch.empty_like(feats)
-    d_kp, d_p, d_s = torch.empty_like(kernel_pts), torch.empty_like(pts), torch.empty_like(samples)
+    grad_mask = int(grad_mask)
+    alloc = lambda like, bit: torch.empty_like(like) if grad_mask & bit else None
+    d_w, d_f, d_kp = alloc(weights, GRAD_WEIGHTS), alloc(feats, GRAD_FEATS), alloc(kernel_pts, GRAD_BASIS_PARAMS)
+    d_p, d_s = alloc(pts, GRAD_PTS), alloc(samples, GRAD_PTS)
+    proj_p = _conv_proj_arg(name, proj, m, c_in, k, dev)
     ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
     _lib.call("pccnn_kpconv_backward", _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends), _ptr(radii),
-              _ptr(kernel_pts), float(sigma), _ptr(weights), _ptr(in_grads), n, m, t, d, c_in, k, c_out, _ptr(d_w),
-              _ptr(d_f), _ptr(d_kp), _ptr(d_p), _ptr(d_s), _ptr(ws), ws.numel(), _stream())
+              _ptr(kernel_pts), float(sigma), _ptr(weights), _ptr(in_grads), proj_p, grad_mask, n, m, t, d, c_in, k,
+              c_out, _optr(d_w), _optr(d_f), _optr(d_kp), _optr(d_p), _optr(d_s), _ptr(ws), ws.numel(), _stream())
     return [d_w, d_f, d_kp, d_p, d_s]
+
+
+def _optr(t):
+    return _P(t.data_ptr()) if t is not None else _P(0)
+
+
+def _conv_proj_arg(name, proj, m, c_in, k, dev):
+    if proj is None:
+        return _P(0)
+    _chk(proj, name + ": proj", torch.float32, 3, dev)
+    if tuple(proj.shape) != (m, c_in, k):
+        raise RuntimeError(name + ": proj must be [M, Cin, K]")
+    return _ptr(proj)
 
 
 def _mc_args(name, pts, pdf, axis, bias, weights, c_in, d, dev):
@@ -355,24 +378,26 @@ def _mc_args(name, pts, pdf, axis, bias, weights, c_in, d, dev):
     return k, num_mlps, c_out
 
 
-def mc_conv(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights):
+def mc_conv(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights, return_proj=False):
     """mc_conv(pts, pdf f32[N], feats, samples, neighbors, start_ids, radii, axis f32[D,H*m], bias f32[1,H*m],
-    weights f32[m, H*Cin, Cout/m]) -> f32[M,Cout] (pccnn_lib_ops/pcconvs/mcconv.cuh:32-42)."""
+    weights f32[m, H*Cin, Cout/m]) -> f32[M,Cout] (pccnn_lib_ops/pcconvs/mcconv.cuh:32-42).
+    ``return_proj=True`` also returns the projection f32[M,Cin,H*m] for mc_conv_grads(..., proj=...)."""
     name = "mc_conv"
     d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
     n, m, t, c_in = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1]
     k, num_mlps, c_out = _mc_args(name, pts, pdf, axis, bias, weights, c_in, d, dev)
     out = torch.empty((m, c_out), dtype=torch.float32, device=dev)
-    ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 0), dev)
+    proj = torch.empty((m, c_in, k), dtype=torch.float32, device=dev)
     _lib.call("pccnn_mcconv_forward", _ptr(pts), _ptr(pdf), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends),
               _ptr(radii), _ptr(axis), _ptr(bias), _ptr(weights), n, m, t, d, c_in, k, num_mlps, c_out, _ptr(out),
-              _ptr(ws), ws.numel(), _stream())
-    return out
+              _ptr(proj), _P(0), 0, _stream())
+    return (out, proj) if return_proj else out
 
 
-def mc_conv_grads(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights, in_grads):
+def mc_conv_grads(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights, in_grads, proj=None,
+                  grad_mask=GRAD_ALL):
     """mc_conv_grads(..., in_grads f32[M,Cout]) -> [dW, dFeat, dAxis, dBias f32[1,H*m], dPdf f32[N], dPts, dSamples]
-    (pccnn_lib_ops/pcconvs/mcconv.cuh:57-69)."""
+    (pccnn_lib_ops/pcconvs/mcconv.cuh:57-69).  ``proj`` / ``grad_mask`` as in kp_conv_grads."""
     name = "mc_conv_grads"
     d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
     n, m, t, c_in = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1]
@@ -380,14 +405,17 @@ def mc_conv_grads(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weig
     in_grads = _chk(in_grads.contiguous(), name + ": in_grads", torch.float32, 2, dev)
     if tuple(in_grads.shape) != (m, c_out):
         raise RuntimeError(name + ": in_grads must be [M, Cout]")
-    d_w, d_f = torch.empty_like(weights), torch.empty_like(feats)
-    d_axis, d_bias, d_pdf = torch.empty_like(axis), torch.empty_like(bias), torch.empty_like(pdf)
-    d_p, d_s = torch.empty_like(pts), torch.empty_like(samples)
+    grad_mask = int(grad_mask)
+    alloc = lambda like, bit: torch.empty_like(like) if grad_mask & bit else None
+    d_w, d_f = alloc(weights, GRAD_WEIGHTS), alloc(feats, GRAD_FEATS)
+    d_axis, d_bias, d_pdf = alloc(axis, GRAD_BASIS_PARAMS), alloc(bias, GRAD_BASIS_PARAMS), alloc(pdf, GRAD_PDF)
+    d_p, d_s = alloc(pts, GRAD_PTS), alloc(samples, GRAD_PTS)
+    proj_p = _conv_proj_arg(name, proj, m, c_in, k, dev)
     ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
     _lib.call("pccnn_mcconv_backward", _ptr(pts), _ptr(pdf), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends),
-              _ptr(radii), _ptr(axis), _ptr(bias), _ptr(weights), _ptr(in_grads), n, m, t, d, c_in, k, num_mlps, c_out,
-              _ptr(d_w), _ptr(d_f), _ptr(d_axis), _ptr(d_bias), _ptr(d_pdf), _ptr(d_p), _ptr(d_s), _ptr(ws),
-              ws.numel(), _stream())
+              _ptr(radii), _ptr(axis), _ptr(bias), _ptr(weights), _ptr(in_grads), proj_p, grad_mask, n, m, t, d, c_in, k,
+              num_mlps, c_out, _optr(d_w), _optr(d_f), _optr(d_axis), _optr(d_bias), _optr(d_pdf), _optr(d_p),
+              _optr(d_s), _ptr(ws), ws.numel(), _stream())
     return [d_w, d_f, d_axis, d_bias, d_pdf, d_p, d_s]
 
 

@@ -56,7 +56,7 @@ def test_argument_validation_needs_no_gpu(lib_path):
                              None, 0, None)
     assert rc == -3 and b"workspace" in lib.pccnn_last_error()
     rc = lib.pccnn_kpconv_forward(None, None, None, None, None, None, None, 0.5, None, 10, 10, 10, 3, 8, 65, 8, None,
-                                  None, 0, None)
+                                  None, None, 0, None)
     assert rc == -2 and b"k=65" in lib.pccnn_last_error()
     assert lib.pccnn_conv_workspace_bytes(1000, 5000, 32, 16, 64, 0) >= 1000 * 32 * 16 * 4
     assert lib.pccnn_find_neighbors_workspace_bytes(1000) >= 4000

@@ -233,6 +233,44 @@ def test_hierarchy_level_with_pooling(oracle):
     assert relerr(p(out), exp) < 2e-5
 
 
+def test_cached_projection_and_gradient_masks(ops, oracle):
+    # the projection kept from the forward call gives the same gradients as rebuilding it, and a gradient
+    # mask returns exactly the requested groups (the others are None), each equal to the full call's
+    pts, ids, smp, nb, rng = _conv_case(oracle, ops, 91, 2, 1200, 0.12, True)
+    d = nb["dev"]
+    c_in, c_out, k = 32, 16, 16
+    feats = t(rng.normal(size=(pts.shape[0], c_in)).astype(np.float32))
+    pdf = t(rng.uniform(0.5, 2.0, pts.shape[0]).astype(np.float32))
+    axis = t(rng.normal(0, 0.6, (3, k)).astype(np.float32))
+    bias = t(rng.normal(0, 0.1, (1, k)).astype(np.float32))
+    w = t(rng.normal(0, 0.1, (1, k * c_in, c_out)).astype(np.float32))
+    g = t(rng.normal(size=(smp.shape[0], c_out)).astype(np.float32))
+    args = (d["pts"], pdf, feats, d["samples"], d["neigh"], d["ends"], d["radii"], axis, bias, w)
+    out, proj = ops.mc_conv(*args, return_proj=True)
+    assert tuple(proj.shape) == (smp.shape[0], c_in, k) and torch.equal(out, ops.mc_conv(*args))
+    full = ops.mc_conv_grads(*args, g)
+    cached = ops.mc_conv_grads(*args, g, proj=proj)
+    for a, b in zip(full, cached):
+        assert relerr(a.cpu().numpy(), b.cpu().numpy()) < 1e-6
+    fw = ops.mc_conv_grads(*args, g, proj=proj, grad_mask=ops.GRAD_WEIGHTS | ops.GRAD_FEATS)
+    assert [x is None for x in fw] == [False, False, True, True, True, True, True]
+    assert torch.equal(fw[0], cached[0]) and relerr(fw[1].cpu().numpy(), full[1].cpu().numpy()) < 1e-6
+    par = ops.mc_conv_grads(*args, g, grad_mask=ops.GRAD_BASIS_PARAMS | ops.GRAD_PDF)
+    assert [x is None for x in par] == [True, True, False, False, False, True, True]
+    assert relerr(par[2].cpu().numpy(), full[2].cpu().numpy()) < 1e-6
+    assert relerr(par[4].cpu().numpy(), full[4].cpu().numpy()) < 1e-5
+    ptsg = ops.mc_conv_grads(*args, g, grad_mask=ops.GRAD_PTS)
+    assert relerr(ptsg[5].cpu().numpy(), full[5].cpu().numpy()) < 1e-5
+    assert relerr(ptsg[6].cpu().numpy(), full[6].cpu().numpy()) < 1e-6
+    # autograd asks only for what requires grad
+    from pccnn_lib_amd.op_wrappers import ComputeMCConv
+    wr = w.clone().requires_grad_(True)
+    fr = feats.clone().requires_grad_(True)
+    res = ComputeMCConv.apply(d["pts"], pdf, fr, d["samples"], d["neigh"], d["ends"], d["radii"], axis, bias, wr)
+    gw, gf = torch.autograd.grad(res, [wr, fr], g)
+    assert torch.equal(gw, cached[0]) and relerr(gf.cpu().numpy(), full[1].cpu().numpy()) < 1e-6
+
+
 def test_weight_variance_ops_and_layer_warmup(ops, oracle):
     import pccnn_lib_amd as lib
     pts, ids, smp, nb, rng = _conv_case(oracle, ops, 77, 2, 1500, 0.12, True)
