@@ -1,12 +1,14 @@
 // fp32 GEMM on the CDNA matrix cores (v_mfma_f32_32x32x2_f32), used for the
 // [M, K*Cin] x [K*Cin, Cout] contraction of the convolutions and its two transposes.
 //
-// Workgroup tile 128 x 128, inner step 16, 256 threads = 4 wavefronts in a 2 x 2 arrangement,
-// each wavefront owning a 64 x 64 block as 2 x 2 MFMA tiles (64 accumulator registers).
+// Workgroup tile 128 x 128 (4 wavefronts as 2 x 2, each a 64 x 64 block of 2 x 2 MFMA tiles) or, when the
+// grid would otherwise be too small to fill the chip, 64 x 128 (1 x 4 wavefronts of 64 x 32); inner step 16.
 // Both operand tiles are staged in LDS k-major ([16][128] plus padding) whatever their layout
 // in memory, so every fragment read is 32 consecutive floats; tiles are double-buffered and the
 // next tile's global loads are issued before the current tile's MFMAs (one barrier per step).
 // Split-K writes partial products to a workspace that a second kernel sums in a fixed order.
+#include <stdlib.h>
+
 #include "common.h"
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -30,16 +32,16 @@ struct GemmArgs {
 // Global -> registers for one 128 x 16 operand tile.  `KCONTIG`: the reduction index is the
 // contiguous one in memory (element (x, k) at p[x * ld + k]); otherwise element (x, k) at p[k * ld + x].
 // `FAST`: the tile is fully inside the matrix and 16-byte aligned, so it is read with float4 loads.
-template <bool KCONTIG, bool FAST>
+template <bool KCONTIG, bool FAST, int TILE_X>
 __device__ __forceinline__ void tile_load(const float *__restrict__ p, int64_t ld, int64_t x0, int64_t x_end,
-                                          int64_t k0, int64_t k_end, float4 (&r)[2])
+                                          int64_t k0, int64_t k_end, float4 (&r)[TILE_X / 64])
 {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < TILE_X / 64; ++i) {
         const int idx = threadIdx.x + 256 * i;
         int64_t x, k;
         if (KCONTIG) { x = x0 + idx / 4; k = k0 + (idx % 4) * 4; }
-        else { k = k0 + idx / 32; x = x0 + (idx % 32) * 4; }
+        else { k = k0 + idx / (TILE_X / 4); x = x0 + (idx % (TILE_X / 4)) * 4; }
         if (FAST) {
             r[i] = KCONTIG ? *(const float4 *)(p + x * ld + k) : *(const float4 *)(p + k * ld + x);
         } else {
@@ -55,11 +57,11 @@ __device__ __forceinline__ void tile_load(const float *__restrict__ p, int64_t l
     }
 }
 
-template <bool KCONTIG>
-__device__ __forceinline__ void tile_store(float (*lds)[GT_LD], const float4 (&r)[2])
+template <bool KCONTIG, int TILE_X>
+__device__ __forceinline__ void tile_store(float (*lds)[GT_LD], const float4 (&r)[TILE_X / 64])
 {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < TILE_X / 64; ++i) {
         const int idx = threadIdx.x + 256 * i;
         if (KCONTIG) {
             const int x = idx / 4, k = (idx % 4) * 4;
@@ -68,7 +70,7 @@ __device__ __forceinline__ void tile_store(float (*lds)[GT_LD], const float4 (&r
             lds[k + 2][x] = r[i].z;
             lds[k + 3][x] = r[i].w;
         } else {
-            const int k = idx / 32, x = (idx % 32) * 4;
+            const int k = idx / (TILE_X / 4), x = (idx % (TILE_X / 4)) * 4;
             *(float2 *)&lds[k][x] = make_float2(r[i].x, r[i].y);
             *(float2 *)&lds[k][x + 2] = make_float2(r[i].z, r[i].w);
         }
@@ -78,25 +80,27 @@ __device__ __forceinline__ void tile_store(float (*lds)[GT_LD], const float4 (&r
 // The k loop of one workgroup tile.  Global loads of tile kt+1 are issued before the MFMAs of tile kt and
 // parked in LDS after them; inside a tile the LDS fragments of sub-step ks+1 are read before the MFMAs of
 // sub-step ks are issued, so the matrix pipe never waits on an LDS round trip.
-template <bool AT, bool BT, bool FAST>
+template <bool AT, bool BT, bool FAST, int BM>
 __device__ __forceinline__ void gemm_tile_loop(const GemmArgs &g, const float *__restrict__ a,
                                                const float *__restrict__ b, int64_t bm, int64_t bn, int64_t k_begin,
                                                int64_t k_end, float (*As)[GT_K][GT_LD], float (*Bs)[GT_K][GT_LD],
-                                               floatx16 (&acc)[2][2])
+                                               floatx16 (&acc)[2][BM / 64])
 {
+    constexpr int WN = 4 / (BM / 64);                               // wavefronts along the columns
+    constexpr int TN = BM / 64;                                     // 32-column MFMA tiles per wavefront
     const int lane = pccnn_lane();
     const int wave = threadIdx.x >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
     const int frag_k = lane >> 5, frag_c = lane & 31;
-    float4 ra[2], rb[2];
+    float4 ra[BM / 64], rb[2];
     const int64_t nk = (k_end - k_begin + GT_K - 1) / GT_K;
     if (nk > 0) {
         // A stored [rows, inner] (AT = false) has the reduction index contiguous; B stored
         // [inner, cols] (BT = false) has the column index contiguous.
-        tile_load<!AT, FAST>(a, g.lda, bm, g.rows, k_begin, k_end, ra);
-        tile_load<BT, FAST>(b, g.ldb, bn, g.cols, k_begin, k_end, rb);
-        tile_store<!AT>(As[0], ra);
-        tile_store<BT>(Bs[0], rb);
+        tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k_begin, k_end, ra);
+        tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k_begin, k_end, rb);
+        tile_store<!AT, BM>(As[0], ra);
+        tile_store<BT, GT_N>(Bs[0], rb);
     }
     __syncthreads();
     for (int64_t kt = 0; kt < nk; ++kt) {
@@ -104,67 +108,70 @@ __device__ __forceinline__ void gemm_tile_loop(const GemmArgs &g, const float *_
         const bool more = kt + 1 < nk;
         if (more) {
             const int64_t k0 = k_begin + (kt + 1) * GT_K;
-            tile_load<!AT, FAST>(a, g.lda, bm, g.rows, k0, k_end, ra);
-            tile_load<BT, FAST>(b, g.ldb, bn, g.cols, k0, k_end, rb);
+            tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k0, k_end, ra);
+            tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k0, k_end, rb);
         }
-        float fa[2][2], fb[2][2];
-        fa[0][0] = As[buf][frag_k][wm * 64 + frag_c];
-        fa[0][1] = As[buf][frag_k][wm * 64 + 32 + frag_c];
-        fb[0][0] = Bs[buf][frag_k][wn * 64 + frag_c];
-        fb[0][1] = Bs[buf][frag_k][wn * 64 + 32 + frag_c];
+        float fa[2][2], fb[2][TN];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) fa[0][i] = As[buf][frag_k][wm * 64 + i * 32 + frag_c];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[0][j] = Bs[buf][frag_k][wn * (32 * TN) + j * 32 + frag_c];
 #pragma unroll
         for (int ks = 0; ks < GT_K / 2; ++ks) {
             const int cur = ks & 1, nxt = cur ^ 1;
             if (ks + 1 < GT_K / 2) {
                 const int kr = 2 * (ks + 1) + frag_k;
-                fa[nxt][0] = As[buf][kr][wm * 64 + frag_c];
-                fa[nxt][1] = As[buf][kr][wm * 64 + 32 + frag_c];
-                fb[nxt][0] = Bs[buf][kr][wn * 64 + frag_c];
-                fb[nxt][1] = Bs[buf][kr][wn * 64 + 32 + frag_c];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) fa[nxt][i] = As[buf][kr][wm * 64 + i * 32 + frag_c];
+#pragma unroll
+                for (int j = 0; j < TN; ++j) fb[nxt][j] = Bs[buf][kr][wn * (32 * TN) + j * 32 + frag_c];
             }
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][0], fb[cur][0], acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][0], fb[cur][1], acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][1], fb[cur][0], acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][1], fb[cur][1], acc[1][1], 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
         }
         if (more) {
-            tile_store<!AT>(As[buf ^ 1], ra);
-            tile_store<BT>(Bs[buf ^ 1], rb);
+            tile_store<!AT, BM>(As[buf ^ 1], ra);
+            tile_store<BT, GT_N>(Bs[buf ^ 1], rb);
         }
         __syncthreads();
     }
 }
 
-template <bool AT, bool BT>
+template <bool AT, bool BT, int BM>
 __global__ void __launch_bounds__(256)
 gemm_f32_mfma_kernel(GemmArgs g, float *__restrict__ partial)
 {
     __shared__ __attribute__((aligned(16))) float As[2][GT_K][GT_LD];
     __shared__ __attribute__((aligned(16))) float Bs[2][GT_K][GT_LD];
+    constexpr int WN = 4 / (BM / 64);
+    constexpr int TN = BM / 64;
 
     const int lane = pccnn_lane();
     const int wave = threadIdx.x >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
     const int batch = blockIdx.z / g.split_k;
     const int split = blockIdx.z % g.split_k;
-    const int64_t bm = (int64_t)blockIdx.y * GT_M;
+    const int64_t bm = (int64_t)blockIdx.y * BM;
     const int64_t bn = (int64_t)blockIdx.x * GT_N;
     const float *a = g.a + (int64_t)batch * g.stride_a;
     const float *b = g.b + (int64_t)batch * g.stride_b;
     const int64_t k_begin = (int64_t)split * g.k_chunk;
     const int64_t k_end = (k_begin + g.k_chunk < g.inner) ? k_begin + g.k_chunk : g.inner;
-    const bool fast = g.aligned && (bm + GT_M <= g.rows) && (bn + GT_N <= g.cols) && ((k_end - k_begin) % GT_K == 0);
+    const bool fast = g.aligned && (bm + BM <= g.rows) && (bn + GT_N <= g.cols) && ((k_end - k_begin) % GT_K == 0);
 
-    floatx16 acc[2][2];
+    floatx16 acc[2][TN];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    if (fast) gemm_tile_loop<AT, BT, true>(g, a, b, bm, bn, k_begin, k_end, As, Bs, acc);
-    else gemm_tile_loop<AT, BT, false>(g, a, b, bm, bn, k_begin, k_end, As, Bs, acc);
+    if (fast) gemm_tile_loop<AT, BT, true, BM>(g, a, b, bm, bn, k_begin, k_end, As, Bs, acc);
+    else gemm_tile_loop<AT, BT, false, BM>(g, a, b, bm, bn, k_begin, k_end, As, Bs, acc);
 
     // Accumulator layout of the 32x32 MFMA: register v of lane l holds
     // row 8*(v/4) + 4*(l/32) + v%4, column l%32 of the tile.
@@ -180,8 +187,8 @@ gemm_f32_mfma_kernel(GemmArgs g, float *__restrict__ partial)
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int64_t col = bn + wn * 64 + j * 32 + (lane & 31);
+        for (int j = 0; j < TN; ++j) {
+            const int64_t col = bn + wn * (32 * TN) + j * 32 + (lane & 31);
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int64_t row = bm + wm * 64 + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
@@ -237,15 +244,25 @@ extern "C" int pccnn_gemm_f32(const float *a, const float *b, float *c, int64_t 
         partial = (float *)workspace;
     }
     hipStream_t s = (hipStream_t)stream;
-    dim3 grid((unsigned)pccnn_ceil_div(cols, GT_N), (unsigned)pccnn_ceil_div(rows, GT_M), (unsigned)(batch * split_k));
+    // 128-row tiles unless that leaves the chip short of workgroups (fewer than ~4 per CU): then 64-row tiles
+    const int64_t wg128 = pccnn_ceil_div(cols, GT_N) * pccnn_ceil_div(rows, 128) * batch * split_k;
+    const char *force = getenv("PCCNN_GEMM_BM");
+    const int bm_tile = force ? atoi(force) : (wg128 >= 1024 ? 128 : 64);
+    dim3 grid((unsigned)pccnn_ceil_div(cols, GT_N), (unsigned)pccnn_ceil_div(rows, bm_tile), (unsigned)(batch * split_k));
     PCCNN_REQUIRE(grid.y <= 65535u && grid.z <= 65535u, PCCNN_ERR_UNSUPPORTED,
                   "pccnn_gemm_f32: grid too large");
     {
         PccnnTimed timed(PCCNN_T_GEMM, s);
-        if (!a_trans && !b_trans) gemm_f32_mfma_kernel<false, false><<<grid, 256, 0, s>>>(g, partial);
-        else if (!a_trans && b_trans) gemm_f32_mfma_kernel<false, true><<<grid, 256, 0, s>>>(g, partial);
-        else if (a_trans && !b_trans) gemm_f32_mfma_kernel<true, false><<<grid, 256, 0, s>>>(g, partial);
-        else gemm_f32_mfma_kernel<true, true><<<grid, 256, 0, s>>>(g, partial);
+#define GEMM_GO(AT, BT)                                                                       \
+    do {                                                                                      \
+        if (bm_tile == 128) gemm_f32_mfma_kernel<AT, BT, 128><<<grid, 256, 0, s>>>(g, partial); \
+        else gemm_f32_mfma_kernel<AT, BT, 64><<<grid, 256, 0, s>>>(g, partial);                 \
+    } while (0)
+        if (!a_trans && !b_trans) GEMM_GO(false, false);
+        else if (!a_trans && b_trans) GEMM_GO(false, true);
+        else if (a_trans && !b_trans) GEMM_GO(true, false);
+        else GEMM_GO(true, true);
+#undef GEMM_GO
     }
     PCCNN_LAUNCH_CHECK();
     if (split_k > 1) {
