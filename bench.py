@@ -15,7 +15,8 @@ density pipeline are timed as well and reported as extra keys of the same JSON l
 
   roofline      the dominant kernel of the step (the fp32 MFMA contraction): algorithmic flops per launch
                 divided by its mean launch duration, taken live with HIP events on the launch stream;
-  roofline_neighbors   the same for the neighbor fill kernel against HBM bandwidth;
+  roofline_neighbors   the same for the neighbor fill kernel against HBM bandwidth, measured on the
+                million-point room of config 4 (`scene` carries that leg's pairs / second);
   cpu_baseline  the CPU oracle (scalar C + numpy, one thread) on a bounded sample of the same workload.
 
 Exactly one JSON line goes to stdout; progress goes to stderr.
@@ -101,6 +102,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-scene", action="store_true", help="skip the million-point neighbor-search leg")
+    ap.add_argument("--scene-points", type=int, default=1000000)
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on one GPU only; --gpus %d is not supported "
@@ -208,9 +211,44 @@ def main():
     fill_n, fill_total_ms = nb_kernels.get("nb_fill", (0, 0.0))
     fill_avg_ms = fill_total_ms / max(fill_n, 1)
     fill_gbps = nb_bytes / (fill_avg_ms * 1e-3) / 1e9 if fill_n else 0.0
-    roofline_nb = {"kernel": "neighbors_kernel<fill>", "bound": "hbm", "achieved": fill_gbps, "peak": HBM_PEAK_GBPS,
+    roofline_nb = {"kernel": "neighbors_kernel<fill>", "workload": "config 2", "bound": "hbm", "achieved": fill_gbps, "peak": HBM_PEAK_GBPS,
                    "unit": "GB/s", "frac": fill_gbps / HBM_PEAK_GBPS, "traffic": TRAFFIC_NB_FILL_BYTES,
                    "bytes_per_launch": nb_bytes, "avg_launch_ms": fill_avg_ms, "launches": fill_n}
+
+    # ---- scene-scale neighbor search (config 4: one room of 10^6 points, cell = radius = 0.05 m): the
+    # neighbor kernels only show their throughput at this size, so their roofline entry is taken here
+    scene = None
+    if not args.no_scene:
+        from pccnn_lib_amd import synthetic
+        spts = t(synthetic.room(4, args.scene_points))
+        sids = torch.zeros((spts.shape[0],), dtype=torch.int32, device=dev)
+        sradii = torch.full((3,), 0.05, dtype=torch.float32, device=dev)
+        spc = lib.pc.Pointcloud(spts, sids)
+
+        def scene_step():
+            p = lib.pc.Pointcloud.__new__(lib.pc.Pointcloud)
+            p.__dict__.update(spc.__dict__)
+            return lib.pc.layers.conv_base.build_neighborhood(p, p, sradii, 0)
+
+        snb = scene_step()
+        s_pairs = int(snb.neighbors_.shape[0])
+        s_ms, s_kernels = timed(scene_step, max(args.steps // 2, 3), 2)
+        n_s = spts.shape[0]
+        s_grid = 8 * int(np.prod(snb.grid_.num_cells_host()[0:2]))
+        s_bytes = 8.0 * s_pairs + 24.0 * n_s + 20.0 * n_s + s_grid
+        f_n, f_ms = s_kernels.get("nb_fill", (0, 0.0))
+        f_avg = f_ms / max(f_n, 1)
+        s_gbps = s_bytes / (f_avg * 1e-3) / 1e9 if f_n else 0.0
+        roofline_nb = {"kernel": "neighbors_kernel<fill>", "workload": "config 4: %d room points, radius 0.05" % n_s,
+                       "bound": "hbm", "achieved": s_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                       "frac": s_gbps / HBM_PEAK_GBPS, "traffic": TRAFFIC_NB_FILL_BYTES, "bytes_per_launch": s_bytes,
+                       "avg_launch_ms": f_avg, "launches": f_n}
+        scene = {"points": n_s, "pairs": s_pairs, "neighborhood_ms": s_ms,
+                 "neighbor_pairs_per_sec": s_pairs / (s_ms * 1e-3),
+                 "kernels_us": {k: round(1e3 * v[1] / v[0], 2) for k, v in s_kernels.items()}}
+        log("scene: %d points, %d pairs, neighborhood %.3f ms -> %.2f G pairs/s" % (n_s, s_pairs, s_ms,
+                                                                                  s_pairs / s_ms / 1e6))
+        log("scene", {k: "%d x %.1f us" % (v[0], 1e3 * v[1] / v[0]) for k, v in s_kernels.items()})
 
     cpu = None
     if not args.no_cpu_baseline:
@@ -230,7 +268,7 @@ def main():
         "density_ms": pdf_ms,
         "kernels_us": {leg: {k: round(1e3 * v[1] / v[0], 2) for k, v in ks.items()}
                        for leg, ks in (("conv", conv_kernels), ("neighborhood", nb_kernels), ("density", pdf_kernels))},
-        "roofline": roofline, "roofline_neighbors": roofline_nb, "cpu_baseline": cpu,
+        "scene": scene, "roofline": roofline, "roofline_neighbors": roofline_nb, "cpu_baseline": cpu,
     }
     print(json.dumps(result), flush=True)
     return 0

@@ -129,6 +129,13 @@ int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t *pt_keys_so
  * pt_grads_out f32[n,d]. */
 int pccnn_compute_pdf(int manifold_dims, const float *bandwidth, const float *pts, int64_t n, int d,
                       const int32_t *neigh, int64_t t, const int32_t *ends, float *pdf_out, void *stream);
+/* Same estimate for a pair list left in sorted-index space (pccnn_find_neighbors_fill without point_remap):
+ * column 0 of neigh_sorted indexes pts_sorted, sample i is samples[i] (the cloud in its original order).  The
+ * neighbors of a sample are then runs of consecutive rows of pts_sorted, which makes the gather coalesced;
+ * the reference has no such variant (it always remaps first, pccnn_lib/pc/Neighborhood.py:47-53). */
+int pccnn_compute_pdf_sorted(int manifold_dims, const float *bandwidth, const float *pts_sorted,
+                             const float *samples, int64_t n, int d, const int32_t *neigh_sorted, int64_t t,
+                             const int32_t *ends, float *pdf_out, void *stream);
 int pccnn_compute_pdf_grads(int manifold_dims, const float *bandwidth, const float *pts, int64_t n, int d,
                             const int32_t *neigh, int64_t t, const int32_t *ends, const float *in_grads,
                             float *pt_grads_out, void *stream);

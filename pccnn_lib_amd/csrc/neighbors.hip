@@ -36,7 +36,7 @@ struct NbArgs {
     int32_t *neigh;            // FILL: [t,2]
 };
 
-template <bool FILL>
+template <bool FILL, bool CAPPED>
 __global__ void __launch_bounds__(NB_THREADS)
 neighbors_kernel(NbArgs a)
 {
@@ -68,17 +68,17 @@ neighbors_kernel(NbArgs a)
     unsigned long long headmask = __ballot(head);
 
     int my_cnt = 0;                                            // hits seen so far for this lane's sample
-    int my_off = 0, my_raw = 0;
+    int my_off = 0, my_raw = 0;                                // FILL: first output slot / uncapped hit count
     if (FILL && valid) {
         my_off = s > 0 ? a.ends[s - 1] : 0;
-        my_raw = a.counts[s];
+        if (CAPPED) my_raw = a.counts[s];
     }
     const unsigned long long lt = pccnn_lanemask_lt();
 
     while (headmask) {
         const int h = __builtin_ctzll(headmask);
         headmask &= headmask - 1;
-        const int e = headmask ? __builtin_ctzll(headmask) : nvalid;
+        const int e = __builtin_amdgcn_readfirstlane(headmask ? __builtin_ctzll(headmask) : nvalid);
         const long long runkey = pccnn_bcast_ll(key, h);
 
         // key -> (batch, c0, c1, c2); 32-bit arithmetic whenever the key allows it
@@ -175,17 +175,20 @@ neighbors_kernel(NbArgs a)
                 const unsigned long long bal = __ballot(hit);
                 const int c = __popcll(bal);
                 if (FILL) {
-                    const int qoff = pccnn_bcast_i(my_off, q);
-                    const int qdone = pccnn_bcast_i(my_cnt, q);
-                    const int qraw = pccnn_bcast_i(my_raw, q);
+                    // my_off + my_cnt of lane q = next free slot of that sample (uncapped case)
+                    const int qoff = pccnn_bcast_i(CAPPED ? my_off : my_off + my_cnt, q);
                     const int qs = pccnn_bcast_i(s, q);
                     if (hit) {
-                        const int r = qdone + __popcll(bal & lt);
-                        int slot = r;
+                        int slot = __popcll(bal & lt);
                         bool take = true;
-                        if (a.max_neighbors > 0 && qraw > a.max_neighbors) {
-                            slot = (int)(((long long)r * a.max_neighbors) / qraw);
-                            take = (int)(((long long)(r + 1) * a.max_neighbors) / qraw) > slot;
+                        if (CAPPED) {
+                            const int qraw = pccnn_bcast_i(my_raw, q);
+                            const int r = pccnn_bcast_i(my_cnt, q) + slot;
+                            slot = r;
+                            if (qraw > a.max_neighbors) {
+                                slot = (int)(((long long)r * a.max_neighbors) / qraw);
+                                take = (int)(((long long)(r + 1) * a.max_neighbors) / qraw) > slot;
+                            }
                         }
                         const int64_t pos = (int64_t)qoff + slot;
                         if (take && pos < a.t) {
@@ -203,27 +206,34 @@ neighbors_kernel(NbArgs a)
     if (!FILL && valid) a.counts[s] = my_cnt;
 }
 
-// table[c] = index of the first sorted point whose key is >= c, for c in [0, total_cells]; the thread of
-// every point that starts a new key fills the entries between the previous key and its own.
+// table[c] = index of the first sorted point whose key is >= c, for c in [0, total_cells].  The lane of
+// every point that starts a new key owns the entries between the previous key and its own (lane n owns
+// the tail); the 64 lanes of a wavefront then fill each other's gaps together, so a long run of empty
+// cells is written as coalesced stores instead of by a single thread.
 __global__ void __launch_bounds__(256)
 cell_table_kernel(const int64_t *__restrict__ keys, int64_t n, int64_t total_cells, int32_t *__restrict__ table)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i > n) return;
-    long long from, to;                                             // table[from..to] = i
+    long long from = 0, to = -1;                                    // table[from..to] = i (empty when to < from)
     if (i == n) {
         from = (n > 0 ? keys[n - 1] + 1 : 0);
         to = total_cells;
-    } else {
+    } else if (i < n) {
         const long long key = keys[i];
         const long long prev = i > 0 ? keys[i - 1] : -1;
-        if (key == prev) return;
-        from = prev + 1;
-        to = key;
+        if (key != prev) { from = prev + 1; to = key; }
     }
     if (from < 0) from = 0;
     if (to > total_cells) to = total_cells;
-    for (long long c = from; c <= to; ++c) table[c] = (int32_t)i;
+    const int lane = pccnn_lane();
+    unsigned long long todo = __ballot(to >= from);
+    while (todo) {
+        const int src = __builtin_ctzll(todo);
+        todo &= todo - 1;
+        const long long f = pccnn_bcast_ll(from, src), t = pccnn_bcast_ll(to, src);
+        const int32_t v = (int32_t)pccnn_bcast_ll((long long)i, src);
+        for (long long c = f + lane; c <= t; c += 64) table[c] = v;
+    }
 }
 
 extern "C" int pccnn_build_cell_table(const int64_t *sorted_keys, int64_t n, int64_t total_cells,
@@ -294,7 +304,7 @@ extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t
     int64_t waves = pccnn_ceil_div(m, 64);
     {
         PccnnTimed timed(PCCNN_T_NB_COUNT, s);
-        neighbors_kernel<false><<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
+        neighbors_kernel<false, false><<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
     }
     PCCNN_LAUNCH_CHECK();
     PccnnTimed timed(PCCNN_T_SCAN, s);
@@ -330,7 +340,10 @@ extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t 
     int64_t waves = pccnn_ceil_div(m, 64);
     {
         PccnnTimed timed(PCCNN_T_NB_FILL, s);
-        neighbors_kernel<true><<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
+        if (max_neighbors > 0)
+            neighbors_kernel<true, true><<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
+        else
+            neighbors_kernel<true, false><<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
     }
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;

@@ -11,10 +11,12 @@
 
 template <int G, bool GRADS>
 __global__ void __launch_bounds__(256)
-pdf_kernel(double norm_const, const float *__restrict__ bandwidth, const float *__restrict__ pts, int64_t n,
-           const int2 *__restrict__ neigh, const int32_t *__restrict__ ends, const float *__restrict__ in_grads,
-           float *__restrict__ out)
+pdf_kernel(double norm_const, const float *__restrict__ bandwidth, const float *__restrict__ pts,
+           const float *__restrict__ samples, int64_t n, const int2 *__restrict__ neigh,
+           const int32_t *__restrict__ ends, const float *__restrict__ in_grads, float *__restrict__ out)
 {
+    // `samples` holds the coordinates of sample gid, `pts` the array the pair list's point column indexes;
+    // they are the same array unless the caller searched in sorted-index space.
     const int64_t gid = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / G;
     const int sub = threadIdx.x % G;
     const bool valid = gid < n;
@@ -28,9 +30,9 @@ pdf_kernel(double norm_const, const float *__restrict__ bandwidth, const float *
     if (valid) {
         lo = gid > 0 ? ends[gid - 1] : 0;
         hi = ends[gid];
-        cx = pts[gid * 3 + 0];
-        cy = pts[gid * 3 + 1];
-        cz = pts[gid * 3 + 2];
+        cx = samples[gid * 3 + 0];
+        cy = samples[gid * 3 + 1];
+        cz = samples[gid * 3 + 2];
         if (GRADS) g = in_grads[gid];
     }
     double acc = 0.0;
@@ -74,16 +76,17 @@ pdf_kernel(double norm_const, const float *__restrict__ bandwidth, const float *
 }
 
 template <bool GRADS>
-static int pdf_launch(int manifold_dims, const float *bandwidth, const float *pts, int64_t n, const int32_t *neigh,
-                      int64_t t, const int32_t *ends, const float *in_grads, float *out, hipStream_t s)
+static int pdf_launch(int manifold_dims, const float *bandwidth, const float *pts, const float *samples, int64_t n,
+                      const int32_t *neigh, int64_t t, const int32_t *ends, const float *in_grads, float *out,
+                      hipStream_t s)
 {
     const double norm_const = 1.0 / pow(2.0 * 3.1415, (double)(float)manifold_dims / 2.0);
     const int64_t avg = n > 0 ? t / n : 0;
     const int2 *nb = (const int2 *)neigh;
     PccnnTimed timed(PCCNN_T_PDF, s);
 #define PDF_GO(G)                                                                                         \
-    pdf_kernel<G, GRADS><<<(unsigned)pccnn_ceil_div(n * G, 256), 256, 0, s>>>(norm_const, bandwidth, pts, n, nb, \
-                                                                              ends, in_grads, out)
+    pdf_kernel<G, GRADS><<<(unsigned)pccnn_ceil_div(n * G, 256), 256, 0, s>>>(norm_const, bandwidth, pts, samples, n, \
+                                                                              nb, ends, in_grads, out)
     if (avg <= 6) PDF_GO(4);
     else if (avg <= 12) PDF_GO(8);
     else if (avg <= 24) PDF_GO(16);
@@ -110,7 +113,19 @@ extern "C" int pccnn_compute_pdf(int manifold_dims, const float *bandwidth, cons
 {
     int rc = pdf_validate("pccnn_compute_pdf", bandwidth, pts, n, d, neigh, t, ends, pdf_out);
     if (rc != PCCNN_OK || n == 0) return rc;
-    return pdf_launch<false>(manifold_dims, bandwidth, pts, n, neigh, t, ends, nullptr, pdf_out, (hipStream_t)stream);
+    return pdf_launch<false>(manifold_dims, bandwidth, pts, pts, n, neigh, t, ends, nullptr, pdf_out,
+                             (hipStream_t)stream);
+}
+
+extern "C" int pccnn_compute_pdf_sorted(int manifold_dims, const float *bandwidth, const float *pts_sorted,
+                                        const float *samples, int64_t n, int d, const int32_t *neigh_sorted, int64_t t,
+                                        const int32_t *ends, float *pdf_out, void *stream)
+{
+    int rc = pdf_validate("pccnn_compute_pdf_sorted", bandwidth, pts_sorted, n, d, neigh_sorted, t, ends, pdf_out);
+    if (rc != PCCNN_OK || n == 0) return rc;
+    PCCNN_REQUIRE(samples, PCCNN_ERR_INVALID, "pccnn_compute_pdf_sorted: null samples");
+    return pdf_launch<false>(manifold_dims, bandwidth, pts_sorted, samples, n, neigh_sorted, t, ends, nullptr, pdf_out,
+                             (hipStream_t)stream);
 }
 
 extern "C" int pccnn_compute_pdf_grads(int manifold_dims, const float *bandwidth, const float *pts, int64_t n,
@@ -122,6 +137,6 @@ extern "C" int pccnn_compute_pdf_grads(int manifold_dims, const float *bandwidth
     PCCNN_REQUIRE(in_grads, PCCNN_ERR_INVALID, "pccnn_compute_pdf_grads: null in_grads");
     rc = pccnn_fill_f32(pt_grads_out, 0.0f, n * 3, (hipStream_t)stream);
     if (rc != PCCNN_OK) return rc;
-    return pdf_launch<true>(manifold_dims, bandwidth, pts, n, neigh, t, ends, in_grads, pt_grads_out,
+    return pdf_launch<true>(manifold_dims, bandwidth, pts, pts, n, neigh, t, ends, in_grads, pt_grads_out,
                             (hipStream_t)stream);
 }

@@ -1,5 +1,6 @@
 import torch
 
+from .. import pccnn_lib_ops
 from ..op_wrappers import ComputePDF
 
 
@@ -48,9 +49,20 @@ class Pointcloud(object):
         grid = Grid(self, aabb, radii)
         grid.compute_cell_ids()
         grid.build_ds()
-        neigh = Neighborhood(grid, self, 300)
-        self.pts_unnorm_pdf_ = ComputePDF.apply(self.pts_, neigh.neighbors_, neigh.start_ids_, bandwidth,
-                                                self.dim_manifold_)
+        if self.pts_.requires_grad:
+            neigh = Neighborhood(grid, self, 300)
+            self.pts_unnorm_pdf_ = ComputePDF.apply(self.pts_, neigh.neighbors_, neigh.start_ids_, bandwidth,
+                                                    self.dim_manifold_)
+        else:
+            # no gradient wanted: keep the pair list in sorted-index space (no remap) and gather the
+            # neighbor coordinates from the sorted copy of the points, where they are contiguous
+            with torch.no_grad():
+                neigh_sorted, ends = pccnn_lib_ops.find_neighbors_ex(
+                    grid.sorted_pts_, grid.sorted_cell_ids_, self.pts_, grid.cell_ids_, grid.grid_ds_,
+                    grid.num_cells_, grid.cell_size_, 300, sample_order=grid.sorted_ids_i32_,
+                    cell_table=grid.cell_table_)
+                self.pts_unnorm_pdf_ = pccnn_lib_ops.compute_pdf_sorted(
+                    self.dim_manifold_, bandwidth, grid.sorted_pts_, self.pts_, neigh_sorted, ends)
         num_pts = torch.index_select(self.get_num_points_per_batch(), 0, self.batch_ids_.to(torch.int64))
         self.pts_pdf_ = self.pts_unnorm_pdf_ / num_pts.to(torch.float32)
 

@@ -244,6 +244,19 @@ def compute_pdf(manifold_dims, bandwidth, pts, neigh, ends):
     return out
 
 
+def compute_pdf_sorted(manifold_dims, bandwidth, pts_sorted, samples, neigh_sorted, ends):
+    """compute_pdf for a pair list in sorted-index space: column 0 of ``neigh_sorted`` indexes ``pts_sorted``,
+    sample i is ``samples[i]``.  Returns f32[N] in the samples' order."""
+    d = _pdf_args("compute_pdf_sorted", bandwidth, pts_sorted, neigh_sorted, ends)
+    _chk(samples, "compute_pdf_sorted: samples", torch.float32, 2, pts_sorted.device)
+    if tuple(samples.shape) != tuple(pts_sorted.shape):
+        raise RuntimeError("compute_pdf_sorted: samples and pts_sorted must have the same shape")
+    out = torch.empty((samples.shape[0],), dtype=torch.float32, device=samples.device)
+    _lib.call("pccnn_compute_pdf_sorted", int(manifold_dims), _ptr(bandwidth), _ptr(pts_sorted), _ptr(samples),
+              samples.shape[0], d, _ptr(neigh_sorted), neigh_sorted.shape[0], _ptr(ends), _ptr(out), _stream())
+    return out
+
+
 def compute_pdf_grads(manifold_dims, bandwidth, pts, neigh, ends, in_grads):
     """compute_pdf_grads(..., in_grads f32[N]) -> f32[N,D] (pccnn_lib_ops/compute_pdf/compute_pdf.cuh:45-51)."""
     d = _pdf_args("compute_pdf_grads", bandwidth, pts, neigh, ends)
