@@ -284,9 +284,11 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
 // read; the offset / density gradients are reduced across the KPAD lanes with shuffles; the point and
 // density gradients are scattered with one float atomic per pair and coordinate, the sample's own gradient
 // is accumulated in registers and stored once.  Every lane keeps the parameter gradients of its own k in
-// registers; a workgroup reduces them in LDS and stores one partial row that conv_param_reduce_kernel sums
+// registers; a workgroup reduces them in LDS and stores one partial row that the conv_param_reduce kernels sum
 // in a fixed order.  param layout: KP -> d_kernel_pts [K,3];  MLP -> d_axis [3,K] followed by d_bias [K].
 #define BB_UNROLL 4
+#define BB_SAMPLES_PER_WAVE 4
+#define BB_SAMPLES_PER_BLOCK (4 * BB_SAMPLES_PER_WAVE)
 
 template <int BASIS, int KPAD>
 __global__ void __launch_bounds__(256)
@@ -305,8 +307,6 @@ conv_basis_bwd_kernel(ConvGeom g, const float *__restrict__ basis_grads, float *
     const int k = lane % KPAD;
     const int sub = lane / KPAD;
     const bool kvalid = k < g.k;
-    const int64_t s = (int64_t)blockIdx.x * 4 + wave;
-    const bool svalid = s < g.m;
     const float ir0 = 1.0f / g.radii[0], ir1 = 1.0f / g.radii[1], ir2 = 1.0f / g.radii[2];
     float c0 = 0.f, c1 = 0.f, c2 = 0.f, c3 = 0.f;                   // this lane's basis parameters
     if (kvalid) {
@@ -317,6 +317,9 @@ conv_basis_bwd_kernel(ConvGeom g, const float *__restrict__ basis_grads, float *
         }
     }
     float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;                   // parameter gradient sums of this lane's k
+  for (int rep = 0; rep < BB_SAMPLES_PER_WAVE; ++rep) {
+    const int64_t s = ((int64_t)blockIdx.x * BB_SAMPLES_PER_WAVE + rep) * 4 + wave;
+    const bool svalid = s < g.m;
     float sgx = 0.f, sgy = 0.f, sgz = 0.f;                          // the sample's own gradient (before the sign)
     int lo = 0, hi = 0;
     float sx = 0.f, sy = 0.f, sz = 0.f;
@@ -394,15 +397,19 @@ conv_basis_bwd_kernel(ConvGeom g, const float *__restrict__ basis_grads, float *
         sgx += __shfl_xor(sgx, o);
         sgy += __shfl_xor(sgy, o);
         sgz += __shfl_xor(sgz, o);
-        p0 += __shfl_xor(p0, o);
-        p1 += __shfl_xor(p1, o);
-        p2 += __shfl_xor(p2, o);
-        p3 += __shfl_xor(p3, o);
     }
     if (svalid && lane == 0 && d_samples) {
         d_samples[s * 3 + 0] = -sgx;
         d_samples[s * 3 + 1] = -sgy;
         d_samples[s * 3 + 2] = -sgz;
+    }
+  }
+#pragma unroll
+    for (int o = KPAD; o < 64; o <<= 1) {
+        p0 += __shfl_xor(p0, o);
+        p1 += __shfl_xor(p1, o);
+        p2 += __shfl_xor(p2, o);
+        p3 += __shfl_xor(p3, o);
     }
     if (sub == 0) {
         lds_param[wave][k] = p0;
@@ -420,29 +427,33 @@ conv_basis_bwd_kernel(ConvGeom g, const float *__restrict__ basis_grads, float *
     param_partials[(int64_t)blockIdx.x * 256 + i] = v;
 }
 
-// Sums the per-workgroup partial rows ([rows][4][64]) in a fixed order; block b handles component b / 64,
-// basis index b % 64 and writes it to its place in the parameter gradient tensors.
+// Sums the per-workgroup partial rows ([rows][256], column = component * 64 + basis index) in a fixed order.
+// Stage 1: workgroup b adds the rows b, b + G, b + 2G, ... (thread = column, coalesced); stage 2: one
+// workgroup adds the G stage-1 rows and writes every value to its place in the parameter gradient tensors.
+#define PARAM_REDUCE_GROUPS 64
+
+__global__ void __launch_bounds__(256)
+conv_param_reduce1_kernel(const float *__restrict__ partials, int64_t rows, float *__restrict__ stage)
+{
+    float acc = 0.0f;
+    for (int64_t r = blockIdx.x; r < rows; r += PARAM_REDUCE_GROUPS) acc += partials[r * 256 + threadIdx.x];
+    stage[(int64_t)blockIdx.x * 256 + threadIdx.x] = acc;
+}
+
 template <int BASIS>
 __global__ void __launch_bounds__(256)
-conv_param_reduce_kernel(const float *__restrict__ partials, int64_t rows, int k_basis, float *__restrict__ dst_a,
-                         float *__restrict__ dst_b)
+conv_param_reduce2_kernel(const float *__restrict__ stage, int k_basis, float *__restrict__ dst_a,
+                          float *__restrict__ dst_b)
 {
-    __shared__ float red[256];
-    const int comp = blockIdx.x >> 6, kk = blockIdx.x & 63;
+    const int comp = threadIdx.x >> 6, kk = threadIdx.x & 63;
     float acc = 0.0f;
-    for (int64_t r = threadIdx.x; r < rows; r += 256) acc += partials[r * 256 + blockIdx.x];
-    red[threadIdx.x] = acc;
-    __syncthreads();
-    for (int o = 128; o > 0; o >>= 1) {
-        if (threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
-        __syncthreads();
-    }
-    if (threadIdx.x == 0 && kk < k_basis && dst_a) {
+    for (int r = 0; r < PARAM_REDUCE_GROUPS; ++r) acc += stage[r * 256 + threadIdx.x];
+    if (kk < k_basis && dst_a) {
         if (BASIS == BASIS_KP) {
-            if (comp < 3) dst_a[kk * 3 + comp] = red[0];            // d_kernel_pts [K,3]
+            if (comp < 3) dst_a[kk * 3 + comp] = acc;               // d_kernel_pts [K,3]
         } else {
-            if (comp < 3) dst_a[comp * k_basis + kk] = red[0];      // d_axis [3,K]
-            else dst_b[kk] = red[0];                                // d_bias [K]
+            if (comp < 3) dst_a[comp * k_basis + kk] = acc;         // d_axis [3,K]
+            else dst_b[kk] = acc;                                   // d_bias [K]
         }
     }
 }
@@ -549,7 +560,7 @@ extern "C" size_t pccnn_conv_workspace_bytes(int64_t m, int64_t t, int c_in, int
     if (!backward) return proj + 256;
     size_t basis_g = pccnn_align((size_t)t * k * sizeof(float));
     size_t splitk = pccnn_align((size_t)CONV_SPLIT_K * c_in * k * c_out * sizeof(float));
-    size_t partials = pccnn_align((size_t)pccnn_ceil_div(m, 4) * 256 * sizeof(float));
+    size_t partials = pccnn_align(((size_t)pccnn_ceil_div(m, BB_SAMPLES_PER_BLOCK) + PARAM_REDUCE_GROUPS) * 256 * sizeof(float));
     return 2 * proj + basis_g + splitk + partials + 256;
 }
 
@@ -596,8 +607,9 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     const bool want_basis = want_par || want_pts || want_pdf;
     int rc;
     PccnnArena arena(workspace, workspace_bytes);
-    const int64_t partial_rows = pccnn_ceil_div(g.m > 0 ? g.m : 1, 4);
-    float *partials = arena.take<float>((size_t)partial_rows * 256);
+    const int64_t partial_rows = pccnn_ceil_div(g.m > 0 ? g.m : 1, BB_SAMPLES_PER_BLOCK);
+    float *partials = arena.take<float>((size_t)(partial_rows + PARAM_REDUCE_GROUPS) * 256);
+    float *stage = partials + partial_rows * 256;
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv backward: workspace of %zu bytes, need %zu", workspace_bytes,
                   pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 1));
     if (want_f && (rc = pccnn_fill_f32(d_feats, 0.0f, g.n * g.c_in, s)) != PCCNN_OK) return rc;
@@ -656,7 +668,9 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     }
     PCCNN_LAUNCH_CHECK();
     if (want_par) {
-        conv_param_reduce_kernel<BASIS><<<256, 256, 0, s>>>(partials, partial_rows, g.k, d_param_a, d_param_b);
+        conv_param_reduce1_kernel<<<PARAM_REDUCE_GROUPS, 256, 0, s>>>(partials, partial_rows, stage);
+        PCCNN_LAUNCH_CHECK();
+        conv_param_reduce2_kernel<BASIS><<<1, 256, 0, s>>>(stage, g.k, d_param_a, d_param_b);
         PCCNN_LAUNCH_CHECK();
     }
     return PCCNN_OK;
