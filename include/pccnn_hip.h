@@ -208,6 +208,66 @@ int pccnn_mcconv_backward(const float *pts, const float *pdf, const float *feats
                           float *d_pts, float *d_samples,
                           void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- the other convolution families -----------------------------------------
+ * One descriptor-driven triple covers KPConvN, PCCNN, PointConv and SPHConv (and, redundantly, KPConv and
+ * MCConv).  It replaces kp_conv_n* (pccnn_lib_ops/pcconvs/kpconvn.cuh:32-93), pccnn* (pccnn.cuh:32-93),
+ * point_conv / point_conv_grads / point_conv_weight_var (pointconv.cuh:37-56) and sph_conv*
+ * (sphconv.cuh:19-55); they differ only in the basis evaluated per pair and in SPHConv's division of the
+ * output by the neighbor count (`divide_by_count`).
+ *
+ *   kind       a                      b               c             other fields
+ *   KP         kernel_pts f32[k,3]    -               -             sigma
+ *   MLP        axis f32[3,k]          bias f32[k]     -             pdf f32[n]
+ *   KPN        kernel_pts f32[k,3]    -               -             sigma, pdf      (KP value / pdf)
+ *   GAUSS      kernel_pts f32[k,3]    -               -             sigma, pdf      (exp(-|kp-d|^2/(2 sigma^2)) / pdf)
+ *   EXPLICIT   basis f32[t,k]         -               -             (values given per pair: PointConv)
+ *   SPH        radial edges f32[nb0]  azimuth [nb1]   polar [nb2]   k is nb0*nb1*nb2 + 1 (one-hot spherical bin)
+ *
+ * Backward outputs: d_param_a = d_kernel_pts [k,3] (KP, KPN, GAUSS), d_axis [3,k] (MLP) or the basis gradient
+ * f32[t,k] (EXPLICIT); d_param_b = d_bias [k] (MLP); d_pdf only for MLP and GAUSS; d_pts / d_samples for the
+ * kinds whose basis depends on the positions (not EXPLICIT, not SPH).  Groups a kind does not have are ignored. */
+#define PCCNN_BASIS_KP 0
+#define PCCNN_BASIS_MLP 1
+#define PCCNN_BASIS_KPN 2
+#define PCCNN_BASIS_GAUSS 3
+#define PCCNN_BASIS_EXPLICIT 4
+#define PCCNN_BASIS_SPH 5
+typedef struct pccnn_basis {
+    int kind;
+    int k;
+    const float *a, *b, *c;
+    int nb0, nb1, nb2;
+    float sigma;
+    const float *pdf;
+} pccnn_basis;
+int pccnn_conv_forward(const pccnn_basis *basis, const float *pts, const float *feats, const float *samples,
+                       const int32_t *neigh, const int32_t *ends, const float *radii, const float *weights,
+                       int64_t n, int64_t m, int64_t t, int d, int c_in, int num_mlps, int c_out, int divide_by_count,
+                       float *out, float *proj_out, void *workspace, size_t workspace_bytes, void *stream);
+int pccnn_conv_backward(const pccnn_basis *basis, const float *pts, const float *feats, const float *samples,
+                        const int32_t *neigh, const int32_t *ends, const float *radii, const float *weights,
+                        const float *in_grads, const float *proj, int grad_mask,
+                        int64_t n, int64_t m, int64_t t, int d, int c_in, int num_mlps, int c_out, int divide_by_count,
+                        float *d_weights, float *d_feats, float *d_param_a, float *d_param_b, float *d_pdf,
+                        float *d_pts, float *d_samples, void *workspace, size_t workspace_bytes, void *stream);
+int pccnn_conv_weight_var(const pccnn_basis *basis, const float *pts, const float *feats, const float *samples,
+                          const int32_t *neigh, const int32_t *ends, const float *radii,
+                          int64_t n, int64_t m, int64_t t, int d, int c_in, int divide_by_count, float *out,
+                          void *workspace, size_t workspace_bytes, void *stream);
+
+/* PointConv's per-pair basis op and its gradient: replaces point_conv_basis / point_conv_basis_grads
+ * (pccnn_lib_ops/pcconvs/pointconv.cuh:20-35): basis_out f32[t,k] = ((pts[n_t] - samples[s_t]) / radii) . axis + bias;
+ * backward: d_pts f32[n,3], d_samples f32[m,3], d_axis f32[3,k], d_bias f32[k] from basis_grads f32[t,k]. */
+int pccnn_linear_basis_forward(const float *pts, const float *samples, const int32_t *neigh, const float *radii,
+                               const float *axis, const float *bias, int64_t n, int64_t m, int64_t t, int d, int k,
+                               float *basis_out, void *stream);
+size_t pccnn_linear_basis_workspace_bytes(int64_t t);
+int pccnn_linear_basis_backward(const float *pts, const float *samples, const int32_t *neigh, const float *radii,
+                                const float *axis, const float *bias, const float *basis_grads,
+                                int64_t n, int64_t m, int64_t t, int d, int k,
+                                float *d_pts, float *d_samples, float *d_axis, float *d_bias,
+                                void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- variance statistic of the weight initialisation -----------------------
  * Replaces kp_conv_weight_var / mc_conv_weight_var (pccnn_lib_ops/pcconvs/kpconv.cuh:82-90, mcconv.cuh:83-92;
  * kernel pccnn_lib_ops/pcconvs/shared/compute_variance_weights.cu:24-170): out[0] (one float, device) =

@@ -402,3 +402,215 @@ def mcconv_weight_var(pts, pdf, feats, samples, neigh, ends, radii, axis, bias):
     """pccnn_lib_ops/pcconvs/mcconv.cu:145-172."""
     basis, _ = conv_basis(MLP, pts, samples, neigh, radii, axis, bias=bias, pdf=pdf)
     return variance_weights(basis, feats, neigh, ends)[0]
+
+
+# ------------------------------------------------ the other convolution families
+#
+# They reuse the pair offsets and the KPConv basis of orc_conv_basis and the projection / projection-gradient
+# routines above; what differs per family is restated here in numpy, fp32 where the reference computes in fp32
+# (the basis values), float64 for the sums the tolerance leaves open.
+
+
+def _dense(proj, weights):
+    m = proj.shape[0]
+    return (proj.reshape(m, -1).astype(np.float64) @ _f32(weights).astype(np.float64)).astype(np.float32)
+
+
+def _dense_grads(proj, weights, in_grads):
+    m = proj.shape[0]
+    g = _f32(in_grads).astype(np.float64)
+    dw = (proj.reshape(m, -1).astype(np.float64).T @ g).astype(np.float32)
+    dproj = (g @ _f32(weights).astype(np.float64).T).astype(np.float32)
+    return dw, dproj
+
+
+def _kp_basis_grads(diff, kernel_pts, sigma, dbasis):
+    """kernel_pts_basis.cu:41-70 -> (dDiff [T,D] float64, dKernelPts [K,D] float32)."""
+    sig = np.float32(sigma)
+    diff_kp = kernel_pts[None, :, :] - diff[:, None, :]
+    sq = diff_kp * diff_kp
+    dist = sq[..., 0]
+    for i in range(1, sq.shape[-1]):
+        dist = dist + sq[..., i]
+    dist = np.sqrt(np.maximum(dist, np.float32(0.0)))
+    result = np.float32(1.0) - dist / sig
+    inv_dist = (np.float32(1.0) / (dist + np.float32(1e-6))).astype(np.float64)
+    mask = (result >= 0.0).astype(np.float64)
+    cur = -(dbasis.astype(np.float64) * mask) / np.float64(sig)
+    cur = cur[..., None] * inv_dist[..., None] * diff_kp.astype(np.float64)
+    return -cur.sum(axis=1), cur.sum(axis=0).astype(np.float32)
+
+
+def kpconvn_basis(pts, pdf, samples, neigh, radii, kernel_pts, sigma):
+    """kpconvn.cu:37-46: the KPConv correlation divided (fp32) by the density of the neighbor."""
+    basis, diff = conv_basis(KP, pts, samples, neigh, radii, kernel_pts, sigma=sigma)
+    npdf = _f32(pdf)[_i32(neigh)[:, 0]].reshape(-1, 1)
+    return (basis / npdf).astype(np.float32), diff, npdf
+
+
+def kpconvn(pts, pdf, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights):
+    """pccnn_lib_ops/pcconvs/kpconvn.cu:25-58."""
+    basis, _, _ = kpconvn_basis(pts, pdf, samples, neigh, radii, kernel_pts, sigma)
+    return _dense(feat_basis_proj(basis, feats, neigh, ends), weights)
+
+
+def kpconvn_grads(pts, pdf, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights, in_grads):
+    """pccnn_lib_ops/pcconvs/kpconvn.cu:61-113.  Returns [dW, dFeat, dKernelPts, dPts, dSamples]."""
+    pts, samples, neigh, kernel_pts = _f32(pts), _f32(samples), _i32(neigh), _f32(kernel_pts)
+    basis, diff, npdf = kpconvn_basis(pts, pdf, samples, neigh, radii, kernel_pts, sigma)
+    dw, dproj = _dense_grads(feat_basis_proj(basis, feats, neigh, ends), weights, in_grads)
+    dfeat, dbasis = feat_basis_proj_grads(basis, feats, neigh, ends, dproj)
+    aux = (dbasis / npdf).astype(np.float32)                                  # :103
+    ddiff, dkp = _kp_basis_grads(diff, kernel_pts, sigma, aux)
+    dpts, dsamples = _pt_diff_grads(pts.shape[0], samples.shape[0], neigh, radii, ddiff)
+    return [dw, dfeat, dkp, dpts, dsamples]
+
+
+def kpconvn_weight_var(pts, pdf, feats, samples, neigh, ends, radii, kernel_pts, sigma):
+    """pccnn_lib_ops/pcconvs/kpconvn.cu:116-139."""
+    basis, _, _ = kpconvn_basis(pts, pdf, samples, neigh, radii, kernel_pts, sigma)
+    return variance_weights(basis, feats, neigh, ends)[0]
+
+
+def gauss_basis(pts, pdf, samples, neigh, radii, kernel_pts, sigma):
+    """kernel_pts_basis.cu:72-87 (fp32) then pccnn.cu:36-38: exp(-|kp - d|^2 / (2 sigma^2)) / pdf[n]."""
+    pts, samples, neigh, kernel_pts = _f32(pts), _f32(samples), _i32(neigh), _f32(kernel_pts)
+    _, diff = conv_basis(KP, pts, samples, neigh, radii, kernel_pts, sigma=1.0)
+    diff_kp = kernel_pts[None, :, :] - diff[:, None, :]
+    sq = diff_kp * diff_kp
+    d2 = sq[..., 0]
+    for i in range(1, sq.shape[-1]):
+        d2 = d2 + sq[..., i]
+    sig = np.float32(sigma)
+    gauss = np.exp(-(d2 / (np.float32(2.0) * sig * sig))).astype(np.float32)
+    npdf = _f32(pdf)[neigh[:, 0]].reshape(-1, 1)
+    return (gauss / npdf).astype(np.float32), gauss, diff, diff_kp, npdf
+
+
+def pccnn(pts, feats, pdf, samples, neigh, ends, radii, kernel_pts, sigma, weights):
+    """pccnn_lib_ops/pcconvs/pccnn.cu:18-47."""
+    basis = gauss_basis(pts, pdf, samples, neigh, radii, kernel_pts, sigma)[0]
+    return _dense(feat_basis_proj(basis, feats, neigh, ends), weights)
+
+
+def pccnn_grads(pts, feats, pdf, samples, neigh, ends, radii, kernel_pts, sigma, weights, in_grads):
+    """pccnn_lib_ops/pcconvs/pccnn.cu:50-105 with kernel_pts_basis.cu:89-111.
+    Returns [dW, dFeat, dKernelPts, dPdf, dPts, dSamples]."""
+    pts, samples, neigh = _f32(pts), _f32(samples), _i32(neigh)
+    basis, gauss, diff, diff_kp, npdf = gauss_basis(pts, pdf, samples, neigh, radii, kernel_pts, sigma)
+    dw, dproj = _dense_grads(feat_basis_proj(basis, feats, neigh, ends), weights, in_grads)
+    dfeat, dbasis = feat_basis_proj_grads(basis, feats, neigh, ends, dproj)
+    npdf64, db64 = npdf.astype(np.float64), dbasis.astype(np.float64)
+    dpdf_pair = ((-1.0 * basis.astype(np.float64) * db64) / npdf64).sum(axis=1)          # :91-92
+    dpdf = np.zeros(_f32(pdf).shape[0], np.float64)
+    np.add.at(dpdf, neigh[:, 0], dpdf_pair)
+    gin = db64 / npdf64                                                                  # :98
+    sig = np.float64(np.float32(sigma))
+    gkp = -gin[..., None] * gauss.astype(np.float64)[..., None] * diff_kp.astype(np.float64) * (1.0 / (sig * sig))
+    ddiff = (-gkp).sum(axis=1)
+    dkp = gkp.sum(axis=0).astype(np.float32)
+    dpts, dsamples = _pt_diff_grads(pts.shape[0], samples.shape[0], neigh, radii, ddiff)
+    return [dw, dfeat, dkp, dpdf.astype(np.float32), dpts, dsamples]
+
+
+def pccnn_weight_var(pts, feats, pdf, samples, neigh, ends, radii, kernel_pts, sigma):
+    """pccnn_lib_ops/pcconvs/pccnn.cu:108-131."""
+    basis = gauss_basis(pts, pdf, samples, neigh, radii, kernel_pts, sigma)[0]
+    return variance_weights(basis, feats, neigh, ends)[0]
+
+
+def pointconv_basis(pts, radii, samples, neigh, axis, bias):
+    """pccnn_lib_ops/pcconvs/pointconv.cu:17-32: matmul(pt_diff, axis) + bias -> [T,K] (float64 sums, rounded)."""
+    axis = _f32(axis)
+    _, diff = conv_basis(KP, pts, samples, neigh, radii, np.zeros((1, 3), np.float32), sigma=1.0)
+    out = diff.astype(np.float64) @ axis.astype(np.float64) + _f32(bias).reshape(1, -1).astype(np.float64)
+    return out.astype(np.float32), diff
+
+
+def pointconv_basis_grads(pts, radii, samples, neigh, axis, bias, in_grads):
+    """pccnn_lib_ops/pcconvs/pointconv.cu:34-59.  Returns [dPts, dSamples, dAxis, dBias [1,K]]."""
+    pts, samples, neigh, axis = _f32(pts), _f32(samples), _i32(neigh), _f32(axis)
+    g = _f32(in_grads).astype(np.float64)
+    _, diff = pointconv_basis(pts, radii, samples, neigh, axis, bias)
+    dbias = g.sum(axis=0, keepdims=True).astype(np.float32)
+    daxis = (diff.astype(np.float64).T @ g).astype(np.float32)
+    ddiff = g @ axis.astype(np.float64).T
+    dpts, dsamples = _pt_diff_grads(pts.shape[0], samples.shape[0], neigh, radii, ddiff)
+    return [dpts, dsamples, daxis, dbias]
+
+
+def pointconv(basis, feats, neigh, ends, weights):
+    """pccnn_lib_ops/pcconvs/pointconv.cu:61-74."""
+    return _dense(feat_basis_proj(basis, feats, neigh, ends), weights)
+
+
+def pointconv_grads(basis, feats, neigh, ends, weights, in_grads):
+    """pccnn_lib_ops/pcconvs/pointconv.cu:76-101.  Returns [dW, dFeat, dBasis]."""
+    dw, dproj = _dense_grads(feat_basis_proj(basis, feats, neigh, ends), weights, in_grads)
+    dfeat, dbasis = feat_basis_proj_grads(basis, feats, neigh, ends, dproj)
+    return [dw, dfeat, dbasis]
+
+
+def pointconv_weight_var(basis, feats, neigh, ends):
+    """pccnn_lib_ops/pcconvs/pointconv.cu:103-111."""
+    return variance_weights(basis, feats, neigh, ends)[0]
+
+
+def _first_bin(values, edges):
+    """spherical_basis.cu:42-46: first i with value <= edges[i], the last bin when there is none."""
+    ids = np.full(values.shape[0], -1, np.int64)
+    for i in range(edges.shape[0]):
+        ids = np.where((values <= edges[i]) & (ids < 0), i, ids)
+    return np.where(ids < 0, edges.shape[0] - 1, ids)
+
+
+def spherical_basis(pts, samples, neigh, radii, radial_bins, azimuth_bins, polar_bins, with_angles=False):
+    """spherical_basis.cu:24-66,136-156: one-hot [T, R*A*P+1]; fp32 distance, atan(y/(x+1e-6)),
+    acos(clamp(z/(dist+1e-6), +-0.99999)); bin 0 holds pairs closer than 1e-4."""
+    rb, ab, pb = _f32(radial_bins), _f32(azimuth_bins), _f32(polar_bins)
+    _, diff = conv_basis(KP, pts, samples, neigh, radii, np.zeros((1, 3), np.float32), sigma=1.0)
+    sq = diff * diff
+    dist = np.sqrt((sq[:, 0] + sq[:, 1]) + sq[:, 2])
+    azimuth = np.arctan(diff[:, 1] / (diff[:, 0] + np.float32(1e-6))).astype(np.float32)
+    cosine = np.clip(diff[:, 2] / (dist + np.float32(1e-6)), np.float32(-0.99999), np.float32(0.99999))
+    polar = np.arccos(cosine).astype(np.float32)
+    ids = _first_bin(dist, rb) * (ab.shape[0] * pb.shape[0]) + _first_bin(azimuth, ab) * pb.shape[0] \
+        + _first_bin(polar, pb) + 1
+    ids = np.where(dist < 1e-4, 0, ids)
+    k = rb.shape[0] * ab.shape[0] * pb.shape[0] + 1
+    basis = np.zeros((diff.shape[0], k), np.float32)
+    basis[np.arange(diff.shape[0]), ids] = 1.0
+    if with_angles:
+        return basis, (dist, azimuth, polar)
+    return basis
+
+
+def _counts(ends):
+    ends = _i32(ends)
+    return np.diff(np.concatenate([[0], ends])).astype(np.float32)
+
+
+def sphconv(pts, feats, samples, neigh, ends, radii, radial_bins, azimuth_bins, polar_bins, weights):
+    """pccnn_lib_ops/pcconvs/sphconv.cu:18-51: correlation / (neighbor count + 1e-6)."""
+    basis = spherical_basis(pts, samples, neigh, radii, radial_bins, azimuth_bins, polar_bins)
+    out = _dense(feat_basis_proj(basis, feats, neigh, ends), weights)
+    return (out / (_counts(ends).reshape(-1, 1) + np.float32(1e-6))).astype(np.float32)
+
+
+def sphconv_grads(pts, feats, samples, neigh, ends, radii, radial_bins, azimuth_bins, polar_bins, weights, in_grads):
+    """pccnn_lib_ops/pcconvs/sphconv.cu:53-95.  Returns [dW, dFeat]."""
+    basis = spherical_basis(pts, samples, neigh, radii, radial_bins, azimuth_bins, polar_bins)
+    g = (_f32(in_grads) / (_counts(ends).reshape(-1, 1) + np.float32(1e-6))).astype(np.float32)
+    dw, dproj = _dense_grads(feat_basis_proj(basis, feats, neigh, ends), weights, g)
+    dfeat, _ = feat_basis_proj_grads(basis, feats, neigh, ends, dproj)
+    return [dw, dfeat]
+
+
+def sphconv_weight_var(pts, feats, samples, neigh, ends, radii, radial_bins, azimuth_bins, polar_bins):
+    """pccnn_lib_ops/pcconvs/sphconv.cu:97-117 with compute_variance_weights.cu:31-36 (pDivideNumNeighs = true):
+    each sample's sum is scaled by 1 / count^2 before the mean."""
+    basis = spherical_basis(pts, samples, neigh, radii, radial_bins, azimuth_bins, polar_bins)
+    _, per = variance_weights(basis, feats, neigh, ends)
+    cnt = _counts(ends).astype(np.float64)
+    per = np.where(cnt > 0, per / np.maximum(cnt, 1.0) ** 2, 0.0)
+    return np.float32(1.0 / per.mean())

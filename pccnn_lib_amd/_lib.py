@@ -16,6 +16,17 @@ I32 = ctypes.c_int
 F32 = ctypes.c_float
 SZ = ctypes.c_size_t
 
+
+
+class Basis(ctypes.Structure):
+    """struct pccnn_basis of include/pccnn_hip.h."""
+    _fields_ = [("kind", ctypes.c_int), ("k", ctypes.c_int), ("a", P), ("b", P), ("c", P),
+                ("nb0", ctypes.c_int), ("nb1", ctypes.c_int), ("nb2", ctypes.c_int), ("sigma", ctypes.c_float),
+                ("pdf", P)]
+
+
+BP = ctypes.POINTER(Basis)
+
 # name -> (restype, argtypes); mirrors include/pccnn_hip.h declaration by declaration.
 SIGNATURES = {
     "pccnn_last_error": (ctypes.c_char_p, []),
@@ -47,6 +58,13 @@ SIGNATURES = {
     "pccnn_conv_weight_var_workspace_bytes": (SZ, [I64, I32, I32]),
     "pccnn_kpconv_weight_var": (I32, [P, P, P, P, P, P, P, F32, I64, I64, I64, I32, I32, I32, P, P, SZ, P]),
     "pccnn_mcconv_weight_var": (I32, [P, P, P, P, P, P, P, P, P, I64, I64, I64, I32, I32, I32, P, P, SZ, P]),
+    "pccnn_conv_forward": (I32, [BP, P, P, P, P, P, P, P, I64, I64, I64, I32, I32, I32, I32, I32, P, P, P, SZ, P]),
+    "pccnn_conv_backward": (I32, [BP, P, P, P, P, P, P, P, P, P, I32, I64, I64, I64, I32, I32, I32, I32, I32,
+                                  P, P, P, P, P, P, P, P, SZ, P]),
+    "pccnn_conv_weight_var": (I32, [BP, P, P, P, P, P, P, I64, I64, I64, I32, I32, I32, P, P, SZ, P]),
+    "pccnn_linear_basis_forward": (I32, [P, P, P, P, P, P, I64, I64, I64, I32, I32, P, P]),
+    "pccnn_linear_basis_workspace_bytes": (SZ, [I64]),
+    "pccnn_linear_basis_backward": (I32, [P, P, P, P, P, P, P, I64, I64, I64, I32, I32, P, P, P, P, P, SZ, P]),
     "pccnn_timing_enable": (I32, [I32]),
     "pccnn_timing_reset": (I32, []),
     "pccnn_timing_count": (I32, []),

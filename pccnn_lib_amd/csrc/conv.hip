@@ -15,7 +15,24 @@
 // derivative and accumulates point, sample, density and basis-parameter gradients.
 #include "common.h"
 
-enum { BASIS_KP = 0, BASIS_MLP = 1 };
+// Basis families (values = PCCNN_BASIS_* of the C header).
+//   KP     clamp(1 - |kp_k - d| / sigma, 0, 1)                      (KPConv)
+//   MLP    leaky_relu(d . A_k + b_k, 0.2) / pdf                     (MCConv)
+//   KPN    the KP value / pdf                                       (KPConvN)
+//   GAUSS  exp(-|kp_k - d|^2 / (2 sigma^2)) / pdf                   (PCCNN)
+//   EXPLICIT  values given per pair in a [T, K] tensor              (PointConv)
+//   SPH    one-hot spherical bin of d, bin 0 = the centre           (SPHConv)
+//   LINEAR d . A_k + b_k                                            (PointConv's own basis op)
+enum { BASIS_KP = 0, BASIS_MLP = 1, BASIS_KPN = 2, BASIS_GAUSS = 3, BASIS_EXPLICIT = 4, BASIS_SPH = 5,
+       BASIS_LINEAR = 6 };
+
+template <int BASIS> struct BasisTraits {
+    static constexpr bool kernel_pts = BASIS == BASIS_KP || BASIS == BASIS_KPN || BASIS == BASIS_GAUSS;
+    static constexpr bool axis = BASIS == BASIS_MLP || BASIS == BASIS_LINEAR;
+    static constexpr bool uses_pdf = BASIS == BASIS_MLP || BASIS == BASIS_KPN || BASIS == BASIS_GAUSS;
+    static constexpr bool pdf_grad = BASIS == BASIS_MLP || BASIS == BASIS_GAUSS;
+    static constexpr bool differentiable = kernel_pts || axis;       // has a basis_bwd stage
+};
 
 struct ConvGeom {
     const float *pts;       // [n,3]
@@ -23,46 +40,83 @@ struct ConvGeom {
     const int2 *neigh;      // [t] (point, sample)
     const int32_t *ends;    // [m]
     const float *radii;     // [3]
-    const float *pdf;       // [n] (MLP) or null
-    const float *basis_a;   // KP: kernel points [K,3]; MLP: axis [3,K]
-    const float *basis_b;   // MLP: bias [K]
-    float sigma;            // KP
+    const float *pdf;       // [n] or null
+    const float *basis_a;   // kernel points [K,3] | axis [3,K] | explicit basis [T,K] | radial bin edges
+    const float *basis_b;   // bias [K] | azimuth bin edges
+    float sigma;
     int64_t n, m, t;
     int c_in, k;
+    const float *basis_c;   // polar bin edges
+    int nb0, nb1, nb2;      // spherical bin counts
 };
+
+// First bin whose upper edge is >= v, the last bin when there is none.
+__device__ __forceinline__ int sph_bin(float v, const float *__restrict__ edges, int count)
+{
+    int id = -1;
+    for (int i = 0; i < count; ++i)
+        if (v <= edges[i] && id < 0) id = i;
+    return id < 0 ? count - 1 : id;
+}
 
 template <int BASIS> struct LaneBasis {
     float c0, c1, c2, c3;
+    int kk;
     bool active;
     __device__ __forceinline__ void load(const ConvGeom &g, int k)
     {
         active = k < g.k;
+        kk = k;
         c0 = c1 = c2 = c3 = 0.0f;
         if (active) {
-            if (BASIS == BASIS_KP) {
+            if (BasisTraits<BASIS>::kernel_pts) {
                 c0 = g.basis_a[k * 3 + 0]; c1 = g.basis_a[k * 3 + 1]; c2 = g.basis_a[k * 3 + 2];
-            } else {
+            } else if (BasisTraits<BASIS>::axis) {
                 c0 = g.basis_a[k]; c1 = g.basis_a[g.k + k]; c2 = g.basis_a[2 * g.k + k]; c3 = g.basis_b[k];
             }
         }
     }
     // Basis value of this lane's k for a pair with normalised offset (dx,dy,dz).
-    __device__ __forceinline__ float eval(float dx, float dy, float dz, float pdf, float sigma) const
+    __device__ __forceinline__ float eval(const ConvGeom &g, float dx, float dy, float dz, float pdf) const
     {
-        float w;
-        if (BASIS == BASIS_KP) {
+        float w = 0.0f;
+        if (BASIS == BASIS_KP || BASIS == BASIS_KPN) {
             const float vx = c0 - dx, vy = c1 - dy, vz = c2 - dz;
             const float d2 = fmaxf(vx * vx + vy * vy + vz * vz, 0.0f);
-            const float r = 1.0f - sqrtf(d2) / sigma;
+            const float r = 1.0f - sqrtf(d2) / g.sigma;
             w = fminf(fmaxf(r, 0.0f), 1.0f);
-        } else {
+            if (BASIS == BASIS_KPN) w = w / pdf;
+        } else if (BASIS == BASIS_GAUSS) {
+            const float vx = c0 - dx, vy = c1 - dy, vz = c2 - dz;
+            const float d2 = vx * vx + vy * vy + vz * vz;
+            w = expf(-(d2 / (2.0f * g.sigma * g.sigma))) / pdf;
+        } else if (BASIS == BASIS_MLP) {
             float a = dx * c0 + dy * c1 + dz * c2 + c3;
             a = a > 0.0f ? a : a * 0.2f;
             w = a / pdf;
+        } else if (BASIS == BASIS_LINEAR) {
+            w = dx * c0 + dy * c1 + dz * c2 + c3;
+        } else if (BASIS == BASIS_SPH) {
+            const float dist = sqrtf(dx * dx + dy * dy + dz * dz);
+            const float azimuth = atanf(dy / (dx + 1e-6f));
+            const float polar = acosf(fminf(fmaxf(dz / (dist + 1e-6f), -0.99999f), 0.99999f));
+            int id = sph_bin(dist, g.basis_a, g.nb0) * g.nb1 * g.nb2 + sph_bin(azimuth, g.basis_b, g.nb1) * g.nb2 +
+                     sph_bin(polar, g.basis_c, g.nb2) + 1;
+            if (dist < 1e-4f) id = 0;
+            w = (id == kk) ? 1.0f : 0.0f;
         }
         return active ? w : 0.0f;
     }
 };
+
+// Basis value for pair `pair` (global pair index) of the chunk: evaluated, or read when given explicitly.
+template <int BASIS>
+__device__ __forceinline__ float pair_basis(const ConvGeom &g, const LaneBasis<BASIS> &lb, int64_t pair, float dx,
+                                            float dy, float dz, float pdf)
+{
+    if (BASIS == BASIS_EXPLICIT) return lb.active ? g.basis_a[pair * g.k + lb.kk] : 0.0f;
+    return lb.eval(g, dx, dy, dz, pdf);
+}
 
 // ------------------------------------------------------------------------------- forward
 
@@ -83,8 +137,12 @@ conv_proj_fwd_kernel(ConvGeom g, const float *__restrict__ feats, float *__restr
     const int k = lane % KPAD, part = lane / KPAD;
     const int lo = s > 0 ? g.ends[s - 1] : 0;
     const int hi = g.ends[s];
-    const float sx = g.samples[s * 3 + 0], sy = g.samples[s * 3 + 1], sz = g.samples[s * 3 + 2];
-    const float ir0 = 1.0f / g.radii[0], ir1 = 1.0f / g.radii[1], ir2 = 1.0f / g.radii[2];
+    constexpr bool GEOM = BASIS != BASIS_EXPLICIT;      // explicit basis values need no positions
+    float sx = 0.f, sy = 0.f, sz = 0.f, ir0 = 1.f, ir1 = 1.f, ir2 = 1.f;
+    if (GEOM) {
+        sx = g.samples[s * 3 + 0]; sy = g.samples[s * 3 + 1]; sz = g.samples[s * 3 + 2];
+        ir0 = 1.0f / g.radii[0]; ir1 = 1.0f / g.radii[1]; ir2 = 1.0f / g.radii[2];
+    }
     LaneBasis<BASIS> lb;
     lb.load(g, k);
 
@@ -98,15 +156,20 @@ conv_proj_fwd_kernel(ConvGeom g, const float *__restrict__ feats, float *__restr
         float dx = 0.f, dy = 0.f, dz = 0.f, pd = 1.0f;
         if (lane < cnt) {
             nidx = g.neigh[cb + lane].x;
-            dx = (g.pts[(int64_t)nidx * 3 + 0] - sx) * ir0;
-            dy = (g.pts[(int64_t)nidx * 3 + 1] - sy) * ir1;
-            dz = (g.pts[(int64_t)nidx * 3 + 2] - sz) * ir2;
-            if (BASIS == BASIS_MLP) pd = g.pdf[nidx];
+            if (GEOM) {
+                dx = (g.pts[(int64_t)nidx * 3 + 0] - sx) * ir0;
+                dy = (g.pts[(int64_t)nidx * 3 + 1] - sy) * ir1;
+                dz = (g.pts[(int64_t)nidx * 3 + 2] - sz) * ir2;
+            }
+            if (BasisTraits<BASIS>::uses_pdf) pd = g.pdf[nidx];
         }
         for (int p = 0; p * PARTS < cnt; ++p) {
             const int j = p * PARTS + part;
-            const float w = lb.eval(__shfl(dx, j), __shfl(dy, j), __shfl(dz, j), __shfl(pd, j), g.sigma);
-            w_lds[j][k] = (j < cnt) ? w : 0.0f;
+            // the shuffles stay outside the condition: every lane must take part, a lane that sits out
+            // would hand zeros to the lanes reading from it
+            const float jx = __shfl(dx, j), jy = __shfl(dy, j), jz = __shfl(dz, j), jp = __shfl(pd, j);
+            const float w = (j < cnt) ? pair_basis<BASIS>(g, lb, (int64_t)cb + j, jx, jy, jz, jp) : 0.0f;
+            w_lds[j][k] = w;
         }
         __syncthreads();
         for (int j0 = 0; j0 < cnt; j0 += ROWS) {
@@ -173,8 +236,12 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
     const int k = lane % KPAD, part = lane / KPAD;
     const int lo = s > 0 ? g.ends[s - 1] : 0;
     const int hi = g.ends[s];
-    const float sx = g.samples[s * 3 + 0], sy = g.samples[s * 3 + 1], sz = g.samples[s * 3 + 2];
-    const float ir0 = 1.0f / g.radii[0], ir1 = 1.0f / g.radii[1], ir2 = 1.0f / g.radii[2];
+    constexpr bool GEOM = BASIS != BASIS_EXPLICIT;      // explicit basis values need no positions
+    float sx = 0.f, sy = 0.f, sz = 0.f, ir0 = 1.f, ir1 = 1.f, ir2 = 1.f;
+    if (GEOM) {
+        sx = g.samples[s * 3 + 0]; sy = g.samples[s * 3 + 1]; sz = g.samples[s * 3 + 2];
+        ir0 = 1.0f / g.radii[0]; ir1 = 1.0f / g.radii[1]; ir2 = 1.0f / g.radii[2];
+    }
     LaneBasis<BASIS> lb;
     lb.load(g, k);
     const int fblocks = (g.c_in + 63) / 64;
@@ -185,16 +252,21 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
         float dx = 0.f, dy = 0.f, dz = 0.f, pd = 1.0f;
         if (lane < cnt) {
             nidx = g.neigh[cb + lane].x;
-            dx = (g.pts[(int64_t)nidx * 3 + 0] - sx) * ir0;
-            dy = (g.pts[(int64_t)nidx * 3 + 1] - sy) * ir1;
-            dz = (g.pts[(int64_t)nidx * 3 + 2] - sz) * ir2;
-            if (BASIS == BASIS_MLP) pd = g.pdf[nidx];
+            if (GEOM) {
+                dx = (g.pts[(int64_t)nidx * 3 + 0] - sx) * ir0;
+                dy = (g.pts[(int64_t)nidx * 3 + 1] - sy) * ir1;
+                dz = (g.pts[(int64_t)nidx * 3 + 2] - sz) * ir2;
+            }
+            if (BasisTraits<BASIS>::uses_pdf) pd = g.pdf[nidx];
         }
         // basis values of the chunk: pass p evaluates pairs p*PARTS .. p*PARTS + PARTS - 1
         for (int p = 0; p * PARTS < cnt; ++p) {
             const int j = p * PARTS + part;
-            const float w = lb.eval(__shfl(dx, j), __shfl(dy, j), __shfl(dz, j), __shfl(pd, j), g.sigma);
-            w_lds[j][k] = (j < cnt) ? w : 0.0f;
+            // the shuffles stay outside the condition: every lane must take part, a lane that sits out
+            // would hand zeros to the lanes reading from it
+            const float jx = __shfl(dx, j), jy = __shfl(dy, j), jz = __shfl(dz, j), jp = __shfl(pd, j);
+            const float w = (j < cnt) ? pair_basis<BASIS>(g, lb, (int64_t)cb + j, jx, jy, jz, jp) : 0.0f;
+            w_lds[j][k] = w;
             db_lds[j][k] = 0.0f;
         }
         __syncthreads();
@@ -310,7 +382,7 @@ conv_basis_bwd_kernel(ConvGeom g, const float *__restrict__ basis_grads, float *
     const float ir0 = 1.0f / g.radii[0], ir1 = 1.0f / g.radii[1], ir2 = 1.0f / g.radii[2];
     float c0 = 0.f, c1 = 0.f, c2 = 0.f, c3 = 0.f;                   // this lane's basis parameters
     if (kvalid) {
-        if (BASIS == BASIS_KP) {
+        if (BasisTraits<BASIS>::kernel_pts) {
             c0 = g.basis_a[k * 3 + 0]; c1 = g.basis_a[k * 3 + 1]; c2 = g.basis_a[k * 3 + 2];
         } else {
             c0 = g.basis_a[k]; c1 = g.basis_a[g.k + k]; c2 = g.basis_a[2 * g.k + k]; c3 = g.basis_b[k];
@@ -344,23 +416,38 @@ conv_basis_bwd_kernel(ConvGeom g, const float *__restrict__ basis_grads, float *
             px[u] = g.pts[(int64_t)nidx[u] * 3 + 0];
             py[u] = g.pts[(int64_t)nidx[u] * 3 + 1];
             pz[u] = g.pts[(int64_t)nidx[u] * 3 + 2];
-            pdv[u] = (BASIS == BASIS_MLP) ? g.pdf[nidx[u]] : 1.0f;
+            pdv[u] = BasisTraits<BASIS>::uses_pdf ? g.pdf[nidx[u]] : 1.0f;
         }
 #pragma unroll
         for (int u = 0; u < BB_UNROLL; ++u) {
             float gx = 0.f, gy = 0.f, gz = 0.f, gpdf = 0.f;
             if (tv[u] && kvalid) {
                 const float dx = (px[u] - sx) * ir0, dy = (py[u] - sy) * ir1, dz = (pz[u] - sz) * ir2;
-                if (BASIS == BASIS_KP) {
+                if (BASIS == BASIS_KP || BASIS == BASIS_KPN) {
+                    // kernel_pts_basis_grads; KPConvN feeds it the gradient already divided by the density
+                    const float gin = (BASIS == BASIS_KPN) ? gk[u] / pdv[u] : gk[u];
                     const float vx = c0 - dx, vy = c1 - dy, vz = c2 - dz;
                     const float dist = sqrtf(fmaxf(vx * vx + vy * vy + vz * vz, 0.0f));
                     const float res = 1.0f - dist / g.sigma;
                     if (res >= 0.0f) {
-                        const float c = -(gk[u] / g.sigma) * (1.0f / (dist + 1e-6f));
+                        const float c = -(gin / g.sigma) * (1.0f / (dist + 1e-6f));
                         const float cx = c * vx, cy = c * vy, cz = c * vz;
                         gx = -cx; gy = -cy; gz = -cz;
                         p0 += cx; p1 += cy; p2 += cz;
                     }
+                } else if (BASIS == BASIS_GAUSS) {
+                    const float vx = c0 - dx, vy = c1 - dy, vz = c2 - dz;
+                    const float e = expf(-((vx * vx + vy * vy + vz * vz) / (2.0f * g.sigma * g.sigma)));
+                    const float gin = gk[u] / pdv[u];
+                    gpdf = -((e / pdv[u]) * gk[u]) / pdv[u];
+                    const float c = -gin * e * (1.0f / (g.sigma * g.sigma));
+                    const float cx = c * vx, cy = c * vy, cz = c * vz;
+                    gx = -cx; gy = -cy; gz = -cz;
+                    p0 += cx; p1 += cy; p2 += cz;
+                } else if (BASIS == BASIS_LINEAR) {
+                    const float c = gk[u];
+                    gx = c * c0; gy = c * c1; gz = c * c2;
+                    p0 += dx * c; p1 += dy * c; p2 += dz * c; p3 += c;
                 } else {
                     const float inv_pd = 1.0f / pdv[u];
                     float act = dx * c0 + dy * c1 + dz * c2 + c3;
@@ -377,7 +464,7 @@ conv_basis_bwd_kernel(ConvGeom g, const float *__restrict__ basis_grads, float *
                 gx += __shfl_xor(gx, o);
                 gy += __shfl_xor(gy, o);
                 gz += __shfl_xor(gz, o);
-                if (BASIS == BASIS_MLP) gpdf += __shfl_xor(gpdf, o);
+                if (BasisTraits<BASIS>::pdf_grad) gpdf += __shfl_xor(gpdf, o);
             }
             if (tv[u] && k == 0) {
                 gx *= ir0; gy *= ir1; gz *= ir2;
@@ -386,7 +473,7 @@ conv_basis_bwd_kernel(ConvGeom g, const float *__restrict__ basis_grads, float *
                     unsafeAtomicAdd(&d_pts[(int64_t)nidx[u] * 3 + 1], gy);
                     unsafeAtomicAdd(&d_pts[(int64_t)nidx[u] * 3 + 2], gz);
                 }
-                if (BASIS == BASIS_MLP && d_pdf) unsafeAtomicAdd(&d_pdf[nidx[u]], gpdf);
+                if (BasisTraits<BASIS>::pdf_grad && d_pdf) unsafeAtomicAdd(&d_pdf[nidx[u]], gpdf);
                 sgx += gx; sgy += gy; sgz += gz;
             }
         }
@@ -449,7 +536,7 @@ conv_param_reduce2_kernel(const float *__restrict__ stage, int k_basis, float *_
     float acc = 0.0f;
     for (int r = 0; r < PARAM_REDUCE_GROUPS; ++r) acc += stage[r * 256 + threadIdx.x];
     if (kk < k_basis && dst_a) {
-        if (BASIS == BASIS_KP) {
+        if (BasisTraits<BASIS>::kernel_pts) {
             if (comp < 3) dst_a[kk * 3 + comp] = acc;               // d_kernel_pts [K,3]
         } else {
             if (comp < 3) dst_a[comp * k_basis + kk] = acc;         // d_axis [3,K]
@@ -486,6 +573,115 @@ mean_reciprocal_kernel(const float *__restrict__ vals, int64_t count, float *__r
         __syncthreads();
     }
     if (threadIdx.x == 0) out[0] = (float)(1.0 / (red[0] / (double)count));
+}
+
+// out[s][c] = in[s][c] / (number of neighbors of s + 1e-6): the SPHConv normalisation.
+__global__ void __launch_bounds__(256)
+scale_by_count_kernel(const float *__restrict__ in, float *__restrict__ out, const int32_t *__restrict__ ends,
+                      int64_t m, int c_out)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= m * c_out) return;
+    const int64_t s = i / c_out;
+    const float cnt = (float)(ends[s] - (s > 0 ? ends[s - 1] : 0));
+    out[i] = in[i] / (cnt + 1e-6f);
+}
+
+// Squared row norms divided by the squared neighbor count (weight variance with division).
+__global__ void __launch_bounds__(256)
+divide_by_count_sq_kernel(float *__restrict__ rows, const int32_t *__restrict__ ends, int64_t m)
+{
+    const int64_t s = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (s >= m) return;
+    const int cnt = ends[s] - (s > 0 ? ends[s - 1] : 0);
+    const float inv = cnt > 0 ? 1.0f / (float)cnt : 0.0f;
+    rows[s] = rows[s] * inv * inv;
+}
+
+// PointConv's own basis op: basis[t][k] = d_t . A[:,k] + b[k], one thread per (pair, k).
+__global__ void __launch_bounds__(256)
+linear_basis_fwd_kernel(ConvGeom g, float *__restrict__ basis_out)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= g.t * g.k) return;
+    const int64_t t = i / g.k;
+    const int k = (int)(i % g.k);
+    const int2 pr = g.neigh[t];
+    const float dx = (g.pts[(int64_t)pr.x * 3 + 0] - g.samples[(int64_t)pr.y * 3 + 0]) * (1.0f / g.radii[0]);
+    const float dy = (g.pts[(int64_t)pr.x * 3 + 1] - g.samples[(int64_t)pr.y * 3 + 1]) * (1.0f / g.radii[1]);
+    const float dz = (g.pts[(int64_t)pr.x * 3 + 2] - g.samples[(int64_t)pr.y * 3 + 2]) * (1.0f / g.radii[2]);
+    basis_out[i] = dx * g.basis_a[k] + dy * g.basis_a[g.k + k] + dz * g.basis_a[2 * g.k + k] + g.basis_b[k];
+}
+
+// Its backward, pair-parallel (the op gets no segment offsets): KPAD lanes per pair as in
+// conv_basis_bwd_kernel, float atomics for the point and the sample gradients.
+template <int KPAD>
+__global__ void __launch_bounds__(256)
+linear_basis_bwd_kernel(ConvGeom g, const float *__restrict__ basis_grads, float *__restrict__ d_pts,
+                        float *__restrict__ d_samples, float *__restrict__ param_partials)
+{
+    __shared__ float lds_param[4][4 * 64];
+    constexpr int PAIRS = 64 / KPAD;
+    const int lane = pccnn_lane(), wave = threadIdx.x >> 6;
+    const int k = lane % KPAD, sub = lane / KPAD;
+    const bool kvalid = k < g.k;
+    const float ir0 = 1.0f / g.radii[0], ir1 = 1.0f / g.radii[1], ir2 = 1.0f / g.radii[2];
+    float c0 = 0.f, c1 = 0.f, c2 = 0.f;
+    if (kvalid) { c0 = g.basis_a[k]; c1 = g.basis_a[g.k + k]; c2 = g.basis_a[2 * g.k + k]; }
+    float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
+    const int64_t gw = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int64_t nw = ((int64_t)gridDim.x * blockDim.x) >> 6;
+    for (int64_t base = gw * PAIRS; base < g.t; base += nw * PAIRS) {
+        const int64_t t = base + sub;
+        const bool tv = t < g.t;
+        float gx = 0.f, gy = 0.f, gz = 0.f;
+        int2 pr = make_int2(0, 0);
+        if (tv) {
+            pr = g.neigh[t];
+            if (kvalid) {
+                const float dx = (g.pts[(int64_t)pr.x * 3 + 0] - g.samples[(int64_t)pr.y * 3 + 0]) * ir0;
+                const float dy = (g.pts[(int64_t)pr.x * 3 + 1] - g.samples[(int64_t)pr.y * 3 + 1]) * ir1;
+                const float dz = (g.pts[(int64_t)pr.x * 3 + 2] - g.samples[(int64_t)pr.y * 3 + 2]) * ir2;
+                const float c = basis_grads[t * g.k + k];
+                gx = c * c0; gy = c * c1; gz = c * c2;
+                p0 += dx * c; p1 += dy * c; p2 += dz * c; p3 += c;
+            }
+        }
+#pragma unroll
+        for (int o = KPAD / 2; o > 0; o >>= 1) {
+            gx += __shfl_xor(gx, o);
+            gy += __shfl_xor(gy, o);
+            gz += __shfl_xor(gz, o);
+        }
+        if (tv && k == 0) {
+            gx *= ir0; gy *= ir1; gz *= ir2;
+            unsafeAtomicAdd(&d_pts[(int64_t)pr.x * 3 + 0], gx);
+            unsafeAtomicAdd(&d_pts[(int64_t)pr.x * 3 + 1], gy);
+            unsafeAtomicAdd(&d_pts[(int64_t)pr.x * 3 + 2], gz);
+            unsafeAtomicAdd(&d_samples[(int64_t)pr.y * 3 + 0], -gx);
+            unsafeAtomicAdd(&d_samples[(int64_t)pr.y * 3 + 1], -gy);
+            unsafeAtomicAdd(&d_samples[(int64_t)pr.y * 3 + 2], -gz);
+        }
+    }
+#pragma unroll
+    for (int o = KPAD; o < 64; o <<= 1) {
+        p0 += __shfl_xor(p0, o);
+        p1 += __shfl_xor(p1, o);
+        p2 += __shfl_xor(p2, o);
+        p3 += __shfl_xor(p3, o);
+    }
+    if (sub == 0) {
+        lds_param[wave][k] = p0;
+        lds_param[wave][64 + k] = p1;
+        lds_param[wave][128 + k] = p2;
+        lds_param[wave][192 + k] = p3;
+    }
+    __syncthreads();
+    const int i = threadIdx.x, comp = i >> 6, kk = i & 63;
+    float v = 0.0f;
+    if (kk < KPAD) v = lds_param[0][comp * 64 + kk] + lds_param[1][comp * 64 + kk] + lds_param[2][comp * 64 + kk] +
+                       lds_param[3][comp * 64 + kk];
+    param_partials[(int64_t)blockIdx.x * 256 + i] = v;
 }
 
 // ------------------------------------------------------------------------------- host side
@@ -561,7 +757,8 @@ extern "C" size_t pccnn_conv_workspace_bytes(int64_t m, int64_t t, int c_in, int
     size_t basis_g = pccnn_align((size_t)t * k * sizeof(float));
     size_t splitk = pccnn_align((size_t)CONV_SPLIT_K * c_in * k * c_out * sizeof(float));
     size_t partials = pccnn_align(((size_t)pccnn_ceil_div(m, BB_SAMPLES_PER_BLOCK) + PARAM_REDUCE_GROUPS) * 256 * sizeof(float));
-    return 2 * proj + basis_g + splitk + partials + 256;
+    size_t scaled = pccnn_align((size_t)m * c_out * sizeof(float));
+    return 2 * proj + basis_g + splitk + partials + scaled + 256;
 }
 
 // out[m, c_out] = P[m, c_in*k] x W, with the feature axis split over num_mlps independent
@@ -577,7 +774,8 @@ static int contraction_fwd(const float *proj, const float *weights, float *out, 
 
 template <int BASIS>
 static int conv_forward(ConvGeom g, const float *feats, const float *weights, int num_mlps, int c_out, float *out,
-                        float *proj_out, void *workspace, size_t workspace_bytes, hipStream_t s)
+                        float *proj_out, void *workspace, size_t workspace_bytes, hipStream_t s,
+                        bool divide_by_count = false)
 {
     if (g.m == 0) return PCCNN_OK;
     float *proj = proj_out;
@@ -589,7 +787,11 @@ static int conv_forward(ConvGeom g, const float *feats, const float *weights, in
     }
     int rc = launch_proj_fwd<BASIS>(g, feats, proj, s);
     if (rc != PCCNN_OK) return rc;
-    return contraction_fwd(proj, weights, out, g.m, g.c_in, g.k, num_mlps, c_out, s);
+    rc = contraction_fwd(proj, weights, out, g.m, g.c_in, g.k, num_mlps, c_out, s);
+    if (rc != PCCNN_OK || !divide_by_count) return rc;
+    scale_by_count_kernel<<<(unsigned)pccnn_ceil_div(g.m * c_out, 256), 256, 0, s>>>(out, out, g.ends, g.m, c_out);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
 }
 
 // Gradients are produced only for the groups named in `mask`; pointers of groups not requested may be null.
@@ -597,13 +799,17 @@ template <int BASIS>
 static int conv_backward(ConvGeom g, const float *feats, const float *weights, const float *in_grads, int num_mlps,
                          int c_out, const float *proj_in, int mask, float *d_weights, float *d_feats,
                          float *d_param_a, float *d_param_b, float *d_pdf, float *d_pts, float *d_samples,
-                         void *workspace, size_t workspace_bytes, hipStream_t s)
+                         void *workspace, size_t workspace_bytes, hipStream_t s, bool divide_by_count = false)
 {
-    // d_param_a: d_kernel_pts [K,3] (KP) or d_axis [3,K] (MLP); d_param_b: d_bias [K] (MLP only)
-    const int count_a = 3 * g.k, count_b = (BASIS == BASIS_KP ? 0 : g.k);
+    // d_param_a: d_kernel_pts [K,3] (kernel-point families), d_axis [3,K] (MLP) or the per-pair basis
+    // gradient [T,K] (EXPLICIT); d_param_b: d_bias [K] (MLP only)
+    typedef BasisTraits<BASIS> Tr;
+    const int64_t count_a = (BASIS == BASIS_EXPLICIT) ? g.t * g.k : 3 * g.k;
+    const int count_b = (BASIS == BASIS_MLP ? g.k : 0);
     const bool want_w = mask & PCCNN_GRAD_WEIGHTS, want_f = mask & PCCNN_GRAD_FEATS;
-    const bool want_par = mask & PCCNN_GRAD_BASIS_PARAMS, want_pts = mask & PCCNN_GRAD_PTS;
-    const bool want_pdf = (mask & PCCNN_GRAD_PDF) && BASIS == BASIS_MLP;
+    const bool want_par = (mask & PCCNN_GRAD_BASIS_PARAMS) && (Tr::differentiable || BASIS == BASIS_EXPLICIT);
+    const bool want_pts = (mask & PCCNN_GRAD_PTS) && Tr::differentiable;
+    const bool want_pdf = (mask & PCCNN_GRAD_PDF) && Tr::pdf_grad;
     const bool want_basis = want_par || want_pts || want_pdf;
     int rc;
     PccnnArena arena(workspace, workspace_bytes);
@@ -629,10 +835,18 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     float *basis_g = arena.take<float>((size_t)g.t * g.k);
     size_t splitk_elems = (size_t)CONV_SPLIT_K * g.c_in * g.k * c_out;
     float *splitk = arena.take<float>(splitk_elems);
+    float *scaled_grads = arena.take<float>((size_t)g.m * c_out);
+    if (BASIS == BASIS_EXPLICIT && want_par) basis_g = d_param_a;    // the basis gradient is itself an output
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv backward: workspace of %zu bytes, need %zu", workspace_bytes,
                   pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 1));
     const int64_t inner = (int64_t)g.c_in * g.k / num_mlps;
     const int64_t co = c_out / num_mlps;
+    if (divide_by_count) {
+        scale_by_count_kernel<<<(unsigned)pccnn_ceil_div(g.m * c_out, 256), 256, 0, s>>>(in_grads, scaled_grads, g.ends,
+                                                                                        g.m, c_out);
+        PCCNN_LAUNCH_CHECK();
+        in_grads = scaled_grads;
+    }
     if (want_w) {
         // d_weights = P^T x dOut; P comes from the caller (kept from the forward call) or is rebuilt here
         const float *proj = proj_in;
@@ -653,32 +867,34 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     if ((rc = launch_proj_bwd<BASIS>(g, feats, d_proj, want_f ? d_feats : nullptr, want_basis ? basis_g : nullptr,
                                      s)) != PCCNN_OK)
         return rc;
-    if (!want_basis) return PCCNN_OK;
+    if (!want_basis || !Tr::differentiable) return PCCNN_OK;
     const unsigned blocks = (unsigned)partial_rows;
     float *o_pts = want_pts ? d_pts : nullptr, *o_smp = want_pts ? d_samples : nullptr;
     float *o_pdf = want_pdf ? d_pdf : nullptr;
-    {
-        PccnnTimed timed(PCCNN_T_BASIS_BWD, s);
-        switch (kpad_of(g.k)) {
-        case 8: conv_basis_bwd_kernel<BASIS, 8><<<blocks, 256, 0, s>>>(g, basis_g, o_pts, o_smp, o_pdf, partials); break;
-        case 16: conv_basis_bwd_kernel<BASIS, 16><<<blocks, 256, 0, s>>>(g, basis_g, o_pts, o_smp, o_pdf, partials); break;
-        case 32: conv_basis_bwd_kernel<BASIS, 32><<<blocks, 256, 0, s>>>(g, basis_g, o_pts, o_smp, o_pdf, partials); break;
-        default: conv_basis_bwd_kernel<BASIS, 64><<<blocks, 256, 0, s>>>(g, basis_g, o_pts, o_smp, o_pdf, partials); break;
+    if constexpr (Tr::differentiable) {
+        {
+            PccnnTimed timed(PCCNN_T_BASIS_BWD, s);
+            switch (kpad_of(g.k)) {
+            case 8: conv_basis_bwd_kernel<BASIS, 8><<<blocks, 256, 0, s>>>(g, basis_g, o_pts, o_smp, o_pdf, partials); break;
+            case 16: conv_basis_bwd_kernel<BASIS, 16><<<blocks, 256, 0, s>>>(g, basis_g, o_pts, o_smp, o_pdf, partials); break;
+            case 32: conv_basis_bwd_kernel<BASIS, 32><<<blocks, 256, 0, s>>>(g, basis_g, o_pts, o_smp, o_pdf, partials); break;
+            default: conv_basis_bwd_kernel<BASIS, 64><<<blocks, 256, 0, s>>>(g, basis_g, o_pts, o_smp, o_pdf, partials); break;
+            }
         }
-    }
-    PCCNN_LAUNCH_CHECK();
-    if (want_par) {
-        conv_param_reduce1_kernel<<<PARAM_REDUCE_GROUPS, 256, 0, s>>>(partials, partial_rows, stage);
         PCCNN_LAUNCH_CHECK();
-        conv_param_reduce2_kernel<BASIS><<<1, 256, 0, s>>>(stage, g.k, d_param_a, d_param_b);
-        PCCNN_LAUNCH_CHECK();
+        if (want_par) {
+            conv_param_reduce1_kernel<<<PARAM_REDUCE_GROUPS, 256, 0, s>>>(partials, partial_rows, stage);
+            PCCNN_LAUNCH_CHECK();
+            conv_param_reduce2_kernel<BASIS><<<1, 256, 0, s>>>(stage, g.k, d_param_a, d_param_b);
+            PCCNN_LAUNCH_CHECK();
+        }
     }
     return PCCNN_OK;
 }
 
 template <int BASIS>
 static int conv_weight_var(ConvGeom g, const float *feats, float *out, void *workspace, size_t workspace_bytes,
-                           hipStream_t s)
+                           hipStream_t s, bool divide_by_count = false)
 {
     PCCNN_REQUIRE(g.m > 0, PCCNN_ERR_INVALID, "conv weight variance: no samples");
     PccnnArena arena(workspace, workspace_bytes);
@@ -690,6 +906,10 @@ static int conv_weight_var(ConvGeom g, const float *feats, float *out, void *wor
     if (rc != PCCNN_OK) return rc;
     row_sumsq_kernel<<<(unsigned)pccnn_ceil_div(g.m, 4), 256, 0, s>>>(proj, g.m, (int64_t)g.c_in * g.k, rows);
     PCCNN_LAUNCH_CHECK();
+    if (divide_by_count) {
+        divide_by_count_sq_kernel<<<(unsigned)pccnn_ceil_div(g.m, 256), 256, 0, s>>>(rows, g.ends, g.m);
+        PCCNN_LAUNCH_CHECK();
+    }
     mean_reciprocal_kernel<<<1, 256, 0, s>>>(rows, g.m, out);
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
@@ -808,4 +1028,175 @@ extern "C" int pccnn_mcconv_backward(const float *pts, const float *pdf, const f
     return conv_backward<BASIS_MLP>(g, feats, weights, in_grads, num_mlps, c_out, proj, grad_mask, d_weights, d_feats,
                                     d_axis, d_bias, d_pdf, d_pts, d_samples, workspace, workspace_bytes,
                                     (hipStream_t)stream);
+}
+
+// ------------------------------------------------------------------- generic entry points
+
+static int basis_geom(const char *who, const pccnn_basis *b, const float *pts, const float *samples,
+                      const int32_t *neigh, const int32_t *ends, const float *radii, int64_t n, int64_t m, int64_t t,
+                      int c_in, ConvGeom &g)
+{
+    PCCNN_REQUIRE(b != nullptr, PCCNN_ERR_INVALID, "%s: null basis descriptor", who);
+    PCCNN_REQUIRE(b->kind >= PCCNN_BASIS_KP && b->kind <= PCCNN_BASIS_SPH, PCCNN_ERR_INVALID, "%s: basis kind %d", who,
+                  b->kind);
+    int k = b->k;
+    if (b->kind == PCCNN_BASIS_SPH) {
+        PCCNN_REQUIRE(b->nb0 > 0 && b->nb1 > 0 && b->nb2 > 0 && b->a && b->b && b->c, PCCNN_ERR_INVALID,
+                      "%s: spherical basis needs three non-empty bin edge arrays", who);
+        k = b->nb0 * b->nb1 * b->nb2 + 1;
+    } else {
+        PCCNN_REQUIRE(b->a != nullptr || (b->kind == PCCNN_BASIS_EXPLICIT && t == 0), PCCNN_ERR_INVALID,
+                      "%s: null basis parameter", who);
+    }
+    PCCNN_REQUIRE(k >= 1 && k <= 64, PCCNN_ERR_UNSUPPORTED, "%s: basis size k=%d outside [1,64]", who, k);
+    const bool kp = b->kind == PCCNN_BASIS_KP || b->kind == PCCNN_BASIS_KPN || b->kind == PCCNN_BASIS_GAUSS;
+    const bool with_pdf = b->kind == PCCNN_BASIS_MLP || b->kind == PCCNN_BASIS_KPN || b->kind == PCCNN_BASIS_GAUSS;
+    PCCNN_REQUIRE(!kp || b->sigma > 0.0f, PCCNN_ERR_INVALID, "%s: sigma=%g", who, b->sigma);
+    PCCNN_REQUIRE(!with_pdf || b->pdf || n == 0, PCCNN_ERR_INVALID, "%s: this basis needs the point densities", who);
+    PCCNN_REQUIRE(b->kind != PCCNN_BASIS_MLP || b->b, PCCNN_ERR_INVALID, "%s: null bias", who);
+    g = ConvGeom{pts, samples, (const int2 *)neigh, ends, radii, b->pdf, b->a, b->b, b->sigma, n, m, t, c_in, k,
+                 b->c, b->nb0, b->nb1, b->nb2};
+    return PCCNN_OK;
+}
+
+#define BASIS_DISPATCH(kind, CALL)                                                       \
+    switch (kind) {                                                                      \
+    case PCCNN_BASIS_KP: return CALL(BASIS_KP);                                          \
+    case PCCNN_BASIS_MLP: return CALL(BASIS_MLP);                                        \
+    case PCCNN_BASIS_KPN: return CALL(BASIS_KPN);                                        \
+    case PCCNN_BASIS_GAUSS: return CALL(BASIS_GAUSS);                                    \
+    case PCCNN_BASIS_EXPLICIT: return CALL(BASIS_EXPLICIT);                              \
+    default: return CALL(BASIS_SPH);                                                     \
+    }
+
+extern "C" int pccnn_conv_forward(const pccnn_basis *basis, const float *pts, const float *feats,
+                                  const float *samples, const int32_t *neigh, const int32_t *ends, const float *radii,
+                                  const float *weights, int64_t n, int64_t m, int64_t t, int d, int c_in, int num_mlps,
+                                  int c_out, int divide_by_count, float *out, float *proj_out, void *workspace,
+                                  size_t workspace_bytes, void *stream)
+{
+    ConvGeom g;
+    int rc = basis_geom("pccnn_conv_forward", basis, pts, samples, neigh, ends, radii, n, m, t, c_in, g);
+    if (rc != PCCNN_OK) return rc;
+    if ((rc = conv_validate("pccnn_conv_forward", n, m, t, d, c_in, g.k, num_mlps, c_out)) != PCCNN_OK) return rc;
+    const bool geom = basis->kind != PCCNN_BASIS_EXPLICIT;
+    PCCNN_REQUIRE(m == 0 || (feats && ends && weights && out && (t == 0 || neigh) && (!geom || (pts && samples && radii))),
+                  PCCNN_ERR_INVALID, "pccnn_conv_forward: null pointer");
+#define CALL(B) conv_forward<B>(g, feats, weights, num_mlps, c_out, out, proj_out, workspace, workspace_bytes, \
+                                (hipStream_t)stream, divide_by_count != 0)
+    BASIS_DISPATCH(basis->kind, CALL)
+#undef CALL
+}
+
+extern "C" int pccnn_conv_backward(const pccnn_basis *basis, const float *pts, const float *feats,
+                                   const float *samples, const int32_t *neigh, const int32_t *ends,
+                                   const float *radii, const float *weights, const float *in_grads, const float *proj,
+                                   int grad_mask, int64_t n, int64_t m, int64_t t, int d, int c_in, int num_mlps,
+                                   int c_out, int divide_by_count, float *d_weights, float *d_feats, float *d_param_a,
+                                   float *d_param_b, float *d_pdf, float *d_pts, float *d_samples, void *workspace,
+                                   size_t workspace_bytes, void *stream)
+{
+    ConvGeom g;
+    int rc = basis_geom("pccnn_conv_backward", basis, pts, samples, neigh, ends, radii, n, m, t, c_in, g);
+    if (rc != PCCNN_OK) return rc;
+    if ((rc = conv_validate("pccnn_conv_backward", n, m, t, d, c_in, g.k, num_mlps, c_out)) != PCCNN_OK) return rc;
+    const int kind = basis->kind;
+    const bool geom = kind != PCCNN_BASIS_EXPLICIT;
+    PCCNN_REQUIRE(weights && (n == 0 || feats) && (m == 0 || (ends && in_grads)) && (t == 0 || neigh) &&
+                      (!geom || (radii && (n == 0 || pts) && (m == 0 || samples))),
+                  PCCNN_ERR_INVALID, "pccnn_conv_backward: null input pointer");
+    const bool has_param = kind != PCCNN_BASIS_SPH;
+    const bool has_pts = kind != PCCNN_BASIS_SPH && kind != PCCNN_BASIS_EXPLICIT;
+    const bool has_pdf = kind == PCCNN_BASIS_MLP || kind == PCCNN_BASIS_GAUSS;
+    PCCNN_REQUIRE((!(grad_mask & PCCNN_GRAD_WEIGHTS) || d_weights) &&
+                      (!(grad_mask & PCCNN_GRAD_FEATS) || d_feats || n == 0) &&
+                      (!(grad_mask & PCCNN_GRAD_BASIS_PARAMS) || !has_param || d_param_a) &&
+                      (!(grad_mask & PCCNN_GRAD_BASIS_PARAMS) || kind != PCCNN_BASIS_MLP || d_param_b) &&
+                      (!(grad_mask & PCCNN_GRAD_PDF) || !has_pdf || d_pdf || n == 0) &&
+                      (!(grad_mask & PCCNN_GRAD_PTS) || !has_pts || ((d_pts || n == 0) && (d_samples || m == 0))),
+                  PCCNN_ERR_INVALID, "pccnn_conv_backward: a requested gradient has a null output pointer");
+#define CALL(B) conv_backward<B>(g, feats, weights, in_grads, num_mlps, c_out, proj, grad_mask, d_weights, d_feats, \
+                                 d_param_a, d_param_b, d_pdf, d_pts, d_samples, workspace, workspace_bytes,           \
+                                 (hipStream_t)stream, divide_by_count != 0)
+    BASIS_DISPATCH(kind, CALL)
+#undef CALL
+}
+
+extern "C" int pccnn_conv_weight_var(const pccnn_basis *basis, const float *pts, const float *feats,
+                                     const float *samples, const int32_t *neigh, const int32_t *ends,
+                                     const float *radii, int64_t n, int64_t m, int64_t t, int d, int c_in,
+                                     int divide_by_count, float *out, void *workspace, size_t workspace_bytes,
+                                     void *stream)
+{
+    ConvGeom g;
+    int rc = basis_geom("pccnn_conv_weight_var", basis, pts, samples, neigh, ends, radii, n, m, t, c_in, g);
+    if (rc != PCCNN_OK) return rc;
+    if ((rc = conv_validate("pccnn_conv_weight_var", n, m, t, d, c_in, g.k, 1, 1)) != PCCNN_OK) return rc;
+    const bool geom = basis->kind != PCCNN_BASIS_EXPLICIT;
+    PCCNN_REQUIRE(feats && ends && out && (t == 0 || neigh) && (!geom || (pts && samples && radii)), PCCNN_ERR_INVALID,
+                  "pccnn_conv_weight_var: null pointer");
+#define CALL(B) conv_weight_var<B>(g, feats, out, workspace, workspace_bytes, (hipStream_t)stream, divide_by_count != 0)
+    BASIS_DISPATCH(basis->kind, CALL)
+#undef CALL
+}
+
+extern "C" int pccnn_linear_basis_forward(const float *pts, const float *samples, const int32_t *neigh,
+                                          const float *radii, const float *axis, const float *bias, int64_t n,
+                                          int64_t m, int64_t t, int d, int k, float *basis_out, void *stream)
+{
+    int rc = conv_validate("pccnn_linear_basis_forward", n, m, t, d, 1, k, 1, 1);
+    if (rc != PCCNN_OK || t == 0) return rc;
+    PCCNN_REQUIRE(pts && samples && neigh && radii && axis && bias && basis_out, PCCNN_ERR_INVALID,
+                  "pccnn_linear_basis_forward: null pointer");
+    ConvGeom g = {pts, samples, (const int2 *)neigh, nullptr, radii, nullptr, axis, bias, 1.0f, n, m, t, 1, k};
+    linear_basis_fwd_kernel<<<(unsigned)pccnn_ceil_div(t * k, 256), 256, 0, (hipStream_t)stream>>>(g, basis_out);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
+extern "C" size_t pccnn_linear_basis_workspace_bytes(int64_t t)
+{
+    (void)t;
+    return pccnn_align((size_t)(1024 + PARAM_REDUCE_GROUPS) * 256 * sizeof(float)) + 256;
+}
+
+extern "C" int pccnn_linear_basis_backward(const float *pts, const float *samples, const int32_t *neigh,
+                                           const float *radii, const float *axis, const float *bias,
+                                           const float *basis_grads, int64_t n, int64_t m, int64_t t, int d, int k,
+                                           float *d_pts, float *d_samples, float *d_axis, float *d_bias,
+                                           void *workspace, size_t workspace_bytes, void *stream)
+{
+    int rc = conv_validate("pccnn_linear_basis_backward", n, m, t, d, 1, k, 1, 1);
+    if (rc != PCCNN_OK) return rc;
+    PCCNN_REQUIRE(radii && axis && bias && d_axis && d_bias && (n == 0 || (pts && d_pts)) && (m == 0 || (samples && d_samples)) &&
+                      (t == 0 || (neigh && basis_grads)),
+                  PCCNN_ERR_INVALID, "pccnn_linear_basis_backward: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    if ((rc = pccnn_fill_f32(d_pts, 0.0f, n * 3, s)) != PCCNN_OK) return rc;
+    if ((rc = pccnn_fill_f32(d_samples, 0.0f, m * 3, s)) != PCCNN_OK) return rc;
+    if (t == 0) {
+        if ((rc = pccnn_fill_f32(d_axis, 0.0f, 3 * k, s)) != PCCNN_OK) return rc;
+        return pccnn_fill_f32(d_bias, 0.0f, k, s);
+    }
+    const int kpad = kpad_of(k);
+    int64_t blocks = pccnn_ceil_div(t, (int64_t)4 * (64 / kpad) * 8);
+    if (blocks > 1024) blocks = 1024;
+    PccnnArena arena(workspace, workspace_bytes);
+    float *partials = arena.take<float>((size_t)(blocks + PARAM_REDUCE_GROUPS) * 256);
+    PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "pccnn_linear_basis_backward: workspace of %zu bytes, need %zu",
+                  workspace_bytes, pccnn_linear_basis_workspace_bytes(t));
+    float *stage = partials + blocks * 256;
+    ConvGeom g = {pts, samples, (const int2 *)neigh, nullptr, radii, nullptr, axis, bias, 1.0f, n, m, t, 1, k};
+    switch (kpad) {
+    case 8: linear_basis_bwd_kernel<8><<<(unsigned)blocks, 256, 0, s>>>(g, basis_grads, d_pts, d_samples, partials); break;
+    case 16: linear_basis_bwd_kernel<16><<<(unsigned)blocks, 256, 0, s>>>(g, basis_grads, d_pts, d_samples, partials); break;
+    case 32: linear_basis_bwd_kernel<32><<<(unsigned)blocks, 256, 0, s>>>(g, basis_grads, d_pts, d_samples, partials); break;
+    default: linear_basis_bwd_kernel<64><<<(unsigned)blocks, 256, 0, s>>>(g, basis_grads, d_pts, d_samples, partials); break;
+    }
+    PCCNN_LAUNCH_CHECK();
+    conv_param_reduce1_kernel<<<PARAM_REDUCE_GROUPS, 256, 0, s>>>(partials, blocks, stage);
+    PCCNN_LAUNCH_CHECK();
+    conv_param_reduce2_kernel<BASIS_MLP><<<1, 256, 0, s>>>(stage, k, d_axis, d_bias);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
 }

@@ -6,13 +6,14 @@ signatures and return conventions; each call validates its tensors, allocates th
 workspace with torch (device memory and the current stream are all torch is used for) and
 forwards raw pointers to ``libpccnn_hip.so``.  Tensors must be CUDA/HIP tensors, contiguous and of
 exactly the reference's dtypes; anything else raises ``RuntimeError`` (the reference reads such
-input as raw memory).  The op families outside the KPConv / MCConv path raise
-``NotImplementedError``.
+input as raw memory).
 
 Beyond the reference's names, ``bounding_box``, ``sort_keys`` and ``find_neighbors_ex`` expose the
 native replacements of the torch / torch_scatter glue the reference keeps in Python
 (pccnn_lib/pc/BoundingBox.py:17-18, pccnn_lib/pc/Grid.py:52,68-70, pccnn_lib/pc/Neighborhood.py:27-53).
 """
+import ctypes
+
 import torch
 
 from . import _lib
@@ -466,23 +467,261 @@ def mc_conv_weight_var(pts, pdf, feats, samples, neigh, ends, radii, axis, bias)
     return out.reshape(())
 
 
-# ------------------------------------------------------------- names outside this path
+# ------------------------------------------------- the other convolution families
+
+BASIS_KP, BASIS_MLP, BASIS_KPN, BASIS_GAUSS, BASIS_EXPLICIT, BASIS_SPH = range(6)
 
 
-def _not_on_path(name):
-    def fn(*_args, **_kwargs):
-        raise NotImplementedError(
-            "pccnn_lib_ops.%s belongs to an operator family that this build does not implement "
-            "(only the KPConv / MCConv path is built)" % name)
-    fn.__name__ = name
-    return fn
+def _basis(kind, k=0, a=None, b=None, c=None, sigma=1.0, pdf=None):
+    """struct pccnn_basis for one call; the tensors it points to must stay alive until the call returns."""
+    desc = _lib.Basis()
+    desc.kind, desc.k, desc.sigma = kind, k, float(sigma)
+    desc.a, desc.b, desc.c, desc.pdf = (None if x is None else x.data_ptr() for x in (a, b, c, pdf))
+    if kind == BASIS_SPH:
+        desc.nb0, desc.nb1, desc.nb2 = a.shape[0], b.shape[0], c.shape[0]
+    return desc
 
 
-for _n in ("point_conv_basis", "point_conv_basis_grads", "point_conv",
-           "point_conv_grads", "point_conv_weight_var", "kp_conv_n", "kp_conv_n_grads", "kp_conv_n_weight_var",
-           "sph_conv", "sph_conv_grads", "sph_conv_weight_var", "pccnn", "pccnn_grads", "pccnn_weight_variance"):
-    globals()[_n] = _not_on_path(_n)
-del _n
+def _generic_forward(name, desc, k, pts, feats, samples, neigh, ends, radii, weights, divide_by_count, return_proj):
+    dev = feats.device
+    _chk(weights, name + ": weights", torch.float32, 2, dev)
+    n, m, t, c_in, c_out = feats.shape[0], ends.shape[0], neigh.shape[0], feats.shape[1], weights.shape[1]
+    if weights.shape[0] != k * c_in:
+        raise RuntimeError(name + ": weights must be [K*Cin, Cout]")
+    out = torch.empty((m, c_out), dtype=torch.float32, device=dev)
+    proj = torch.empty((m, c_in, k), dtype=torch.float32, device=dev)
+    _lib.call("pccnn_conv_forward", ctypes.byref(desc), _optr(pts), _ptr(feats), _optr(samples), _ptr(neigh),
+              _ptr(ends), _optr(radii), _ptr(weights), n, m, t, 3, c_in, 1, c_out, int(divide_by_count), _ptr(out),
+              _ptr(proj), _P(0), 0, _stream())
+    return (out, proj) if return_proj else out
+
+
+def _generic_backward(name, desc, k, pts, feats, samples, neigh, ends, radii, weights, in_grads, proj, grad_mask,
+                      divide_by_count, d_param_a=None, d_pdf=None, with_pts=True):
+    dev = feats.device
+    _chk(weights, name + ": weights", torch.float32, 2, dev)
+    in_grads = _chk(in_grads.contiguous(), name + ": in_grads", torch.float32, 2, dev)
+    n, m, t, c_in, c_out = feats.shape[0], ends.shape[0], neigh.shape[0], feats.shape[1], weights.shape[1]
+    if weights.shape[0] != k * c_in or tuple(in_grads.shape) != (m, c_out):
+        raise RuntimeError(name + ": inconsistent shapes")
+    grad_mask = int(grad_mask)
+    d_w = torch.empty_like(weights) if grad_mask & GRAD_WEIGHTS else None
+    d_f = torch.empty_like(feats) if grad_mask & GRAD_FEATS else None
+    d_p = torch.empty_like(pts) if with_pts and grad_mask & GRAD_PTS else None
+    d_s = torch.empty_like(samples) if with_pts and grad_mask & GRAD_PTS else None
+    proj_p = _conv_proj_arg(name, proj, m, c_in, k, dev)
+    ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
+    _lib.call("pccnn_conv_backward", ctypes.byref(desc), _optr(pts), _ptr(feats), _optr(samples), _ptr(neigh),
+              _ptr(ends), _optr(radii), _ptr(weights), _ptr(in_grads), proj_p, grad_mask, n, m, t, 3, c_in, 1, c_out,
+              int(divide_by_count), _optr(d_w), _optr(d_f), _optr(d_param_a), _P(0), _optr(d_pdf), _optr(d_p),
+              _optr(d_s), _ptr(ws), ws.numel(), _stream())
+    return d_w, d_f, d_p, d_s
+
+
+def _generic_weight_var(name, desc, k, pts, feats, samples, neigh, ends, radii, divide_by_count):
+    dev = feats.device
+    n, m, t, c_in = feats.shape[0], ends.shape[0], neigh.shape[0], feats.shape[1]
+    out = torch.empty((1,), dtype=torch.float32, device=dev)
+    ws = _workspace(_lib.load().pccnn_conv_weight_var_workspace_bytes(m, c_in, k), dev)
+    _lib.call("pccnn_conv_weight_var", ctypes.byref(desc), _optr(pts), _ptr(feats), _optr(samples), _ptr(neigh),
+              _ptr(ends), _optr(radii), n, m, t, 3, c_in, int(divide_by_count), _ptr(out), _ptr(ws), ws.numel(),
+              _stream())
+    return out.reshape(())
+
+
+def _kernel_pts_args(name, pts, pdf, feats, samples, neigh, ends, radii, kernel_pts):
+    d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
+    _chk(pdf, name + ": pdf", torch.float32, 1, dev)
+    _chk(kernel_pts, name + ": kernel_pts", torch.float32, 2, dev)
+    if pdf.shape[0] != pts.shape[0] or kernel_pts.shape[1] != d:
+        raise RuntimeError(name + ": pdf must be [N] and kernel_pts [K, D]")
+    return kernel_pts.shape[0]
+
+
+def kp_conv_n(pts, pdf, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights, return_proj=False):
+    """kp_conv_n(pts, pdf f32[N], feats, samples, neighbors, start_ids, radii, kernel_pts f32[K,D], sigma,
+    weights f32[K*Cin,Cout]) -> f32[M,Cout]: KPConv whose correlation is divided by the density of the neighbor
+    (pccnn_lib_ops/pcconvs/kpconvn.cuh:32-42)."""
+    name = "kp_conv_n"
+    k = _kernel_pts_args(name, pts, pdf, feats, samples, neigh, ends, radii, kernel_pts)
+    desc = _basis(BASIS_KPN, k, kernel_pts, sigma=sigma, pdf=pdf)
+    return _generic_forward(name, desc, k, pts, feats, samples, neigh, ends, radii, weights, False, return_proj)
+
+
+def kp_conv_n_grads(pts, pdf, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights, in_grads, proj=None,
+                    grad_mask=GRAD_ALL):
+    """kp_conv_n_grads(..., in_grads) -> [dW, dFeat, dKernelPts, dPts, dSamples]; the density gets no gradient
+    (pccnn_lib_ops/pcconvs/kpconvn.cuh:57-68)."""
+    name = "kp_conv_n_grads"
+    k = _kernel_pts_args(name, pts, pdf, feats, samples, neigh, ends, radii, kernel_pts)
+    desc = _basis(BASIS_KPN, k, kernel_pts, sigma=sigma, pdf=pdf)
+    d_kp = torch.empty_like(kernel_pts) if int(grad_mask) & GRAD_BASIS_PARAMS else None
+    d_w, d_f, d_p, d_s = _generic_backward(name, desc, k, pts, feats, samples, neigh, ends, radii, weights, in_grads,
+                                           proj, grad_mask, False, d_param_a=d_kp)
+    return [d_w, d_f, d_kp, d_p, d_s]
+
+
+def kp_conv_n_weight_var(pts, pdf, feats, samples, neigh, ends, radii, kernel_pts, sigma):
+    """kp_conv_n_weight_var(...) -> 0-d float tensor (pccnn_lib_ops/pcconvs/kpconvn.cuh:83-92)."""
+    name = "kp_conv_n_weight_var"
+    k = _kernel_pts_args(name, pts, pdf, feats, samples, neigh, ends, radii, kernel_pts)
+    desc = _basis(BASIS_KPN, k, kernel_pts, sigma=sigma, pdf=pdf)
+    return _generic_weight_var(name, desc, k, pts, feats, samples, neigh, ends, radii, False)
+
+
+def pccnn(pts, feats, pdf, samples, neigh, ends, radii, kernel_pts, sigma, weights, return_proj=False):
+    """pccnn(pts, feats, pdf f32[N], samples, neighbors, start_ids, radii, kernel_pts f32[K,D], sigma,
+    weights f32[K*Cin,Cout]) -> f32[M,Cout]: gaussian kernel-point correlation divided by the density
+    (pccnn_lib_ops/pcconvs/pccnn.cuh:32-42; note the feats-before-pdf argument order)."""
+    name = "pccnn"
+    k = _kernel_pts_args(name, pts, pdf, feats, samples, neigh, ends, radii, kernel_pts)
+    desc = _basis(BASIS_GAUSS, k, kernel_pts, sigma=sigma, pdf=pdf)
+    return _generic_forward(name, desc, k, pts, feats, samples, neigh, ends, radii, weights, False, return_proj)
+
+
+def pccnn_grads(pts, feats, pdf, samples, neigh, ends, radii, kernel_pts, sigma, weights, in_grads, proj=None,
+                grad_mask=GRAD_ALL):
+    """pccnn_grads(..., in_grads) -> [dW, dFeat, dKernelPts, dPdf, dPts, dSamples]
+    (pccnn_lib_ops/pcconvs/pccnn.cuh:57-68)."""
+    name = "pccnn_grads"
+    k = _kernel_pts_args(name, pts, pdf, feats, samples, neigh, ends, radii, kernel_pts)
+    desc = _basis(BASIS_GAUSS, k, kernel_pts, sigma=sigma, pdf=pdf)
+    d_kp = torch.empty_like(kernel_pts) if int(grad_mask) & GRAD_BASIS_PARAMS else None
+    d_pdf = torch.empty_like(pdf) if int(grad_mask) & GRAD_PDF else None
+    d_w, d_f, d_p, d_s = _generic_backward(name, desc, k, pts, feats, samples, neigh, ends, radii, weights, in_grads,
+                                           proj, grad_mask, False, d_param_a=d_kp, d_pdf=d_pdf)
+    return [d_w, d_f, d_kp, d_pdf, d_p, d_s]
+
+
+def pccnn_weight_variance(pts, feats, pdf, samples, neigh, ends, radii, kernel_pts, sigma):
+    """pccnn_weight_variance(...) -> 0-d float tensor (pccnn_lib_ops/pcconvs/pccnn.cuh:83-92)."""
+    name = "pccnn_weight_variance"
+    k = _kernel_pts_args(name, pts, pdf, feats, samples, neigh, ends, radii, kernel_pts)
+    desc = _basis(BASIS_GAUSS, k, kernel_pts, sigma=sigma, pdf=pdf)
+    return _generic_weight_var(name, desc, k, pts, feats, samples, neigh, ends, radii, False)
+
+
+def _sph_args(name, pts, feats, samples, neigh, ends, radii, radial_bins, azimuth_bins, polar_bins):
+    d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
+    for b, what in ((radial_bins, "radial"), (azimuth_bins, "azimuth"), (polar_bins, "polar")):
+        _chk(b, "%s: %s bins" % (name, what), torch.float32, 1, dev)
+        if b.shape[0] < 1:
+            raise RuntimeError("%s: empty %s bins" % (name, what))
+    k = radial_bins.shape[0] * azimuth_bins.shape[0] * polar_bins.shape[0] + 1
+    return k, _basis(BASIS_SPH, k, radial_bins, azimuth_bins, polar_bins)
+
+
+def sph_conv(pts, feats, samples, neigh, ends, radii, radial_bins, azimuth_bins, polar_bins, weights,
+             return_proj=False):
+    """sph_conv(pts, feats, samples, neighbors, start_ids, radii, radial_bins f32[R], azimuth_bins f32[A],
+    polar_bins f32[P], weights f32[(R*A*P+1)*Cin, Cout]) -> f32[M,Cout]: one-hot spherical-bin correlation, divided
+    by the neighbor count (pccnn_lib_ops/pcconvs/sphconv.cuh:19-29)."""
+    name = "sph_conv"
+    k, desc = _sph_args(name, pts, feats, samples, neigh, ends, radii, radial_bins, azimuth_bins, polar_bins)
+    return _generic_forward(name, desc, k, pts, feats, samples, neigh, ends, radii, weights, True, return_proj)
+
+
+def sph_conv_grads(pts, feats, samples, neigh, ends, radii, radial_bins, azimuth_bins, polar_bins, weights, in_grads,
+                   proj=None, grad_mask=GRAD_WEIGHTS | GRAD_FEATS):
+    """sph_conv_grads(..., in_grads) -> [dW, dFeat] (pccnn_lib_ops/pcconvs/sphconv.cuh:31-42)."""
+    name = "sph_conv_grads"
+    k, desc = _sph_args(name, pts, feats, samples, neigh, ends, radii, radial_bins, azimuth_bins, polar_bins)
+    d_w, d_f, _, _ = _generic_backward(name, desc, k, pts, feats, samples, neigh, ends, radii, weights, in_grads,
+                                       proj, int(grad_mask) & (GRAD_WEIGHTS | GRAD_FEATS), True, with_pts=False)
+    return [d_w, d_f]
+
+
+def sph_conv_weight_var(pts, feats, samples, neigh, ends, radii, radial_bins, azimuth_bins, polar_bins):
+    """sph_conv_weight_var(...) -> 0-d float tensor; the per-sample sums are divided by the squared neighbor count
+    (pccnn_lib_ops/pcconvs/sphconv.cuh:44-55)."""
+    name = "sph_conv_weight_var"
+    k, desc = _sph_args(name, pts, feats, samples, neigh, ends, radii, radial_bins, azimuth_bins, polar_bins)
+    return _generic_weight_var(name, desc, k, pts, feats, samples, neigh, ends, radii, True)
+
+
+def _linear_basis_args(name, pts, radii, samples, neigh, axis, bias):
+    _chk(pts, name + ": pts", torch.float32, 2)
+    dev = pts.device
+    d = _dims(pts, name)
+    _chk(samples, name + ": samples", torch.float32, 2, dev)
+    _chk(neigh, name + ": neighbors", torch.int32, 2, dev)
+    _chk(radii, name + ": radii", torch.float32, 1, dev)
+    _chk(axis, name + ": axis", torch.float32, 2, dev)
+    bias = _chk(bias, name + ": bias", torch.float32, None, dev)
+    k = axis.shape[1]
+    if samples.shape[1] != d or neigh.shape[1] != 2 or radii.shape[0] != d or axis.shape[0] != d or bias.numel() != k:
+        raise RuntimeError(name + ": axis must be [D, K], bias [1, K] or [K], radii [D]")
+    return d, dev, k
+
+
+def point_conv_basis(pts, radii, samples, neigh, axis, bias):
+    """point_conv_basis(pts, radii, samples, neighbors, axis f32[D,K], bias f32[1,K]) -> f32[T,K]: the affine map
+    of the normalised offsets that PointConv feeds to its own layers (pccnn_lib_ops/pcconvs/pointconv.cuh:20-26)."""
+    name = "point_conv_basis"
+    d, dev, k = _linear_basis_args(name, pts, radii, samples, neigh, axis, bias)
+    t = neigh.shape[0]
+    out = torch.empty((t, k), dtype=torch.float32, device=dev)
+    _lib.call("pccnn_linear_basis_forward", _ptr(pts), _ptr(samples), _ptr(neigh), _ptr(radii), _ptr(axis),
+              _ptr(bias), pts.shape[0], samples.shape[0], t, d, k, _ptr(out), _stream())
+    return out
+
+
+def point_conv_basis_grads(pts, radii, samples, neigh, axis, bias, in_grads):
+    """point_conv_basis_grads(..., in_grads f32[T,K]) -> [dPts, dSamples, dAxis, dBias f32[1,K]]
+    (pccnn_lib_ops/pcconvs/pointconv.cuh:28-35)."""
+    name = "point_conv_basis_grads"
+    d, dev, k = _linear_basis_args(name, pts, radii, samples, neigh, axis, bias)
+    t = neigh.shape[0]
+    in_grads = _chk(in_grads.contiguous(), name + ": in_grads", torch.float32, 2, dev)
+    if tuple(in_grads.shape) != (t, k):
+        raise RuntimeError(name + ": in_grads must be [T, K]")
+    d_p, d_s, d_a = torch.empty_like(pts), torch.empty_like(samples), torch.empty_like(axis)
+    d_b = torch.empty((1, k), dtype=torch.float32, device=dev)
+    ws = _workspace(_lib.load().pccnn_linear_basis_workspace_bytes(t), dev)
+    _lib.call("pccnn_linear_basis_backward", _ptr(pts), _ptr(samples), _ptr(neigh), _ptr(radii), _ptr(axis),
+              _ptr(bias), _ptr(in_grads), pts.shape[0], samples.shape[0], t, d, k, _ptr(d_p), _ptr(d_s), _ptr(d_a),
+              _ptr(d_b), _ptr(ws), ws.numel(), _stream())
+    return [d_p, d_s, d_a, d_b]
+
+
+def _explicit_args(name, basis, feats, neigh, ends):
+    _chk(basis, name + ": basis", torch.float32, 2)
+    dev = basis.device
+    _chk(feats, name + ": features", torch.float32, 2, dev)
+    _chk(neigh, name + ": neighbors", torch.int32, 2, dev)
+    _chk(ends, name + ": start_ids", torch.int32, 1, dev)
+    if basis.shape[0] != neigh.shape[0] or neigh.shape[1] != 2:
+        raise RuntimeError(name + ": basis must be [T, K] and neighbors [T, 2]")
+    k = basis.shape[1]
+    return k, _basis(BASIS_EXPLICIT, k, basis)
+
+
+def point_conv(basis, feats, neigh, ends, weights, return_proj=False):
+    """point_conv(basis f32[T,K], feats, neighbors, start_ids, weights f32[K*Cin,Cout]) -> f32[M,Cout]: the
+    correlation with per-pair basis values given by the caller (pccnn_lib_ops/pcconvs/pointconv.cuh:37-42)."""
+    name = "point_conv"
+    k, desc = _explicit_args(name, basis, feats, neigh, ends)
+    return _generic_forward(name, desc, k, None, feats, None, neigh, ends, None, weights, False, return_proj)
+
+
+def point_conv_grads(basis, feats, neigh, ends, weights, in_grads, proj=None, grad_mask=GRAD_ALL):
+    """point_conv_grads(..., in_grads) -> [dW, dFeat, dBasis f32[T,K]] (pccnn_lib_ops/pcconvs/pointconv.cuh:44-50)."""
+    name = "point_conv_grads"
+    k, desc = _explicit_args(name, basis, feats, neigh, ends)
+    d_b = torch.empty_like(basis) if int(grad_mask) & GRAD_BASIS_PARAMS else None
+    d_w, d_f, _, _ = _generic_backward(name, desc, k, None, feats, None, neigh, ends, None, weights, in_grads, proj,
+                                       int(grad_mask) & (GRAD_WEIGHTS | GRAD_FEATS | GRAD_BASIS_PARAMS), False,
+                                       d_param_a=d_b, with_pts=False)
+    return [d_w, d_f, d_b]
+
+
+def point_conv_weight_var(basis, feats, neigh, ends):
+    """point_conv_weight_var(basis, feats, neighbors, start_ids) -> 0-d float tensor
+    (pccnn_lib_ops/pcconvs/pointconv.cuh:52-56)."""
+    name = "point_conv_weight_var"
+    k, desc = _explicit_args(name, basis, feats, neigh, ends)
+    return _generic_weight_var(name, desc, k, None, feats, None, neigh, ends, None, False)
+
 
 REFERENCE_NAMES = (
     "build_grid_ds", "compute_keys", "find_neighbors", "compute_pdf", "compute_pdf_grads", "poisson_disk_sampling",

@@ -156,6 +156,17 @@ def _torch_forward(kind, pts, samples, feats, neigh, ends, radii, basis_params, 
         kp, sigma = basis_params
         dist = torch.sqrt(((kp[None] - diff[:, None, :]) ** 2).sum(-1))
         basis = torch.clamp(1.0 - dist / sigma, 0.0, 1.0)
+    elif kind == "kpn":
+        # kpconvn.cu:37-46; the reference gives the density no gradient, so it enters as a constant
+        kp, sigma, pdf = basis_params
+        dist = torch.sqrt(((kp[None] - diff[:, None, :]) ** 2).sum(-1))
+        basis = torch.clamp(1.0 - dist / sigma, 0.0, 1.0) / pdf.detach()[n_idx][:, None]
+    elif kind == "gauss":
+        kp, sigma, pdf = basis_params
+        d2 = ((kp[None] - diff[:, None, :]) ** 2).sum(-1)
+        basis = torch.exp(-d2 / (2.0 * sigma * sigma)) / pdf[n_idx][:, None]
+    elif kind == "explicit":
+        basis = basis_params
     else:
         axis, bias, pdf = basis_params
         basis = torch.nn.functional.leaky_relu(diff @ axis + bias, 0.2) / pdf[n_idx][:, None]
@@ -240,3 +251,145 @@ def test_weight_variance_equals_projection_norm(oracle, models):
     one = oracle.variance_weights(basis[:1], feats, neigh[:1], np.array([1], np.int32))[0]
     f0 = feats[neigh[0, 0]].astype(np.float64)
     assert np.isclose(1.0 / one, (basis[0].astype(np.float64) ** 2).sum() * (f0 ** 2).sum(), rtol=1e-6)
+
+
+# ----------------------------------------------------- the other convolution families
+#
+# The reference ships no unit test for KPConvN, PCCNN, PointConv or SPHConv, so their restatements are pinned by
+# float64 torch formulations of the forward (kpconvn.cu, pccnn.cu, pointconv.cu, sphconv.cu read as formulas),
+# autograd for the gradients, and special cases.
+
+def _two_sets(oracle, models, c_in, seed, radius=0.25):
+    pts, ids, nb, feats, rng = _setup(oracle, models, radius, c_in, seed)
+    smp = (pts[::3] + rng.normal(0, 0.01, pts[::3].shape)).astype(np.float32)
+    nb = oracle.neighborhood(pts, ids, smp, ids[::3], radius)
+    return pts, smp, feats, nb["neighbors"], nb["ends"], nb["radii"], rng
+
+
+def test_kpconvn_matches_float64_and_autograd(oracle, models):
+    c_in, c_out, k = 8, 6, 16
+    pts, smp, feats, neigh, ends, radii, rng = _two_sets(oracle, models, c_in, 11)
+    kp, sigma = synthetic.kernel_points_sphere(3, k)
+    pdf = rng.uniform(0.5, 2.0, pts.shape[0]).astype(np.float32)
+    w = rng.normal(0, 0.2, (k * c_in, c_out)).astype(np.float32)
+    g = rng.normal(size=(smp.shape[0], c_out)).astype(np.float32)
+    tp, ts, tf, tkp, tw = [torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in (pts, smp, feats, kp, w)]
+    tpdf = torch.tensor(pdf, dtype=torch.float64)
+    out = _torch_forward("kpn", tp, ts, tf, neigh, ends, radii, (tkp, float(np.float32(sigma)), tpdf), tw)
+    got = oracle.kpconvn(pts, pdf, feats, smp, neigh, ends, radii, kp, sigma, w)
+    assert _relerr(got, out.detach().numpy()) < 1e-5
+    # dividing by a constant density c scales the KPConv result by 1/c
+    half = oracle.kpconvn(pts, np.full_like(pdf, 2.0), feats, smp, neigh, ends, radii, kp, sigma, w)
+    assert _relerr(half, 0.5 * oracle.kpconv(pts, feats, smp, neigh, ends, radii, kp, sigma, w)) < 1e-6
+    (out * torch.tensor(g, dtype=torch.float64)).sum().backward()
+    grads = oracle.kpconvn_grads(pts, pdf, feats, smp, neigh, ends, radii, kp, sigma, w, g)
+    for mine, ref, name in zip(grads, (tw, tf, tkp, tp, ts), ("dW", "dFeat", "dKp", "dPts", "dSamples")):
+        assert _relerr(mine, ref.grad.numpy()) < 1e-4, name
+
+
+def test_pccnn_matches_float64_and_autograd(oracle, models):
+    c_in, c_out, k = 8, 6, 16
+    pts, smp, feats, neigh, ends, radii, rng = _two_sets(oracle, models, c_in, 12)
+    kp, _ = synthetic.kernel_points_sphere(5, k)
+    sigma = 0.4
+    pdf = rng.uniform(0.5, 2.0, pts.shape[0]).astype(np.float32)
+    w = rng.normal(0, 0.2, (k * c_in, c_out)).astype(np.float32)
+    g = rng.normal(size=(smp.shape[0], c_out)).astype(np.float32)
+    tp, tpdf, ts, tf, tkp, tw = [torch.tensor(a, dtype=torch.float64, requires_grad=True)
+                                 for a in (pts, pdf, smp, feats, kp, w)]
+    out = _torch_forward("gauss", tp, ts, tf, neigh, ends, radii, (tkp, float(np.float32(sigma)), tpdf), tw)
+    got = oracle.pccnn(pts, feats, pdf, smp, neigh, ends, radii, kp, sigma, w)
+    assert _relerr(got, out.detach().numpy()) < 1e-5
+    (out * torch.tensor(g, dtype=torch.float64)).sum().backward()
+    grads = oracle.pccnn_grads(pts, feats, pdf, smp, neigh, ends, radii, kp, sigma, w, g)
+    names = ("dW", "dFeat", "dKp", "dPdf", "dPts", "dSamples")
+    for mine, ref, name in zip(grads, (tw, tf, tkp, tpdf, tp, ts), names):
+        assert mine.shape == tuple(ref.shape), name
+        assert _relerr(mine, ref.grad.numpy()) < 1e-4, name
+    # a pair sitting on a kernel point has basis exactly 1 / pdf
+    one = oracle.gauss_basis(np.zeros((1, 3), np.float32), np.array([4.0], np.float32), np.zeros((1, 3), np.float32),
+                             np.array([[0, 0]], np.int32), np.ones(3, np.float32), np.zeros((1, 3), np.float32), 0.3)[0]
+    assert one[0, 0] == 0.25
+
+
+def test_pointconv_matches_float64_and_autograd(oracle, models):
+    c_in, c_out, k = 8, 6, 16
+    pts, smp, feats, neigh, ends, radii, rng = _two_sets(oracle, models, c_in, 13)
+    axis = rng.normal(0, 0.6, (3, k)).astype(np.float32)
+    bias = rng.normal(0, 0.2, (1, k)).astype(np.float32)
+    w = rng.normal(0, 0.2, (k * c_in, c_out)).astype(np.float32)
+    t = neigh.shape[0]
+    n_idx, s_idx = neigh[:, 0].astype(np.int64), neigh[:, 1].astype(np.int64)
+    # basis op (pointconv.cu:17-32) and its gradients
+    tp, ts, ta, tb = [torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in (pts, smp, axis, bias)]
+    inv_r = torch.tensor((np.float32(1.0) / radii).astype(np.float64))
+    tbasis = ((tp[n_idx] - ts[s_idx]) * inv_r) @ ta + tb
+    basis, _ = oracle.pointconv_basis(pts, radii, smp, neigh, axis, bias)
+    assert basis.shape == (t, k) and _relerr(basis, tbasis.detach().numpy()) < 1e-6
+    gb = rng.normal(size=(t, k)).astype(np.float32)
+    (tbasis * torch.tensor(gb, dtype=torch.float64)).sum().backward()
+    grads = oracle.pointconv_basis_grads(pts, radii, smp, neigh, axis, bias, gb)
+    for mine, ref, name in zip(grads, (tp, ts, ta, tb), ("dPts", "dSamples", "dAxis", "dBias")):
+        assert mine.shape == tuple(ref.shape), name
+        assert _relerr(mine, ref.grad.numpy()) < 1e-4, name
+    # conv op with explicit basis values (pointconv.cu:61-101)
+    act = np.maximum(basis, 0).astype(np.float32)
+    g = rng.normal(size=(smp.shape[0], c_out)).astype(np.float32)
+    tact, tf, tw = [torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in (act, feats, w)]
+    out = _torch_forward("explicit", tp.detach(), ts.detach(), tf, neigh, ends, radii, tact, tw)
+    assert _relerr(oracle.pointconv(act, feats, neigh, ends, w), out.detach().numpy()) < 1e-5
+    (out * torch.tensor(g, dtype=torch.float64)).sum().backward()
+    for mine, ref, name in zip(oracle.pointconv_grads(act, feats, neigh, ends, w, g), (tw, tf, tact),
+                               ("dW", "dFeat", "dBasis")):
+        assert _relerr(mine, ref.grad.numpy()) < 1e-4, name
+    proj = oracle.feat_basis_proj(act, feats, neigh, ends).astype(np.float64)
+    assert np.isclose(oracle.pointconv_weight_var(act, feats, neigh, ends), 1.0 / (proj ** 2).sum(axis=(1, 2)).mean(),
+                      rtol=1e-5)
+
+
+def test_spherical_basis_bins(oracle):
+    # Hand-placed offsets (radius 1): the bin of each is fixed by spherical_basis.cu:36-63.
+    radial = np.array([0.5, 1.0], np.float32)
+    azimuth = np.array([0.0, np.pi / 2], np.float32)          # atan() lies in (-pi/2, pi/2)
+    polar = np.array([np.pi / 2, np.pi], np.float32)
+    offs = np.array([[0.0, 0.0, 0.0],        # centre -> bin 0
+                     [0.3, 0.1, 0.1],        # r<0.5, azimuth>0, polar<pi/2 -> (0,1,0)
+                     [0.3, -0.1, -0.1],      # r<0.5, azimuth<0, polar>pi/2 -> (0,0,1)
+                     [0.6, 0.5, 0.2],        # 0.5<r<1 -> (1,1,0)
+                     [2.0, -1.0, -1.0]],     # r>1 clamps to the last radial bin -> (1,0,1)
+                    np.float32)
+    pts = offs
+    smp = np.zeros((1, 3), np.float32)
+    neigh = np.stack([np.arange(5), np.zeros(5)], axis=1).astype(np.int32)
+    basis = oracle.spherical_basis(pts, smp, neigh, np.ones(3, np.float32), radial, azimuth, polar)
+    assert basis.shape == (5, 9) and np.all(basis.sum(axis=1) == 1)
+    expect = [0, 1 + (0 * 2 + 1) * 2 + 0, 1 + (0 * 2 + 0) * 2 + 1, 1 + (1 * 2 + 1) * 2 + 0, 1 + (1 * 2 + 0) * 2 + 1]
+    assert list(basis.argmax(axis=1)) == expect
+
+
+def test_sphconv_matches_float64_and_autograd(oracle, models):
+    c_in, c_out = 8, 6
+    pts, smp, feats, neigh, ends, radii, rng = _two_sets(oracle, models, c_in, 14)
+    radial = np.array([0.4, 0.7, 1.0], np.float32)
+    azimuth = np.linspace(-np.pi / 2, np.pi / 2, 5)[1:].astype(np.float32)
+    polar = np.linspace(0, np.pi, 4)[1:].astype(np.float32)
+    k = 3 * 4 * 3 + 1
+    w = rng.normal(0, 0.2, (k * c_in, c_out)).astype(np.float32)
+    g = rng.normal(size=(smp.shape[0], c_out)).astype(np.float32)
+    basis = oracle.spherical_basis(pts, smp, neigh, radii, radial, azimuth, polar)
+    assert basis.shape[1] == k and len(np.unique(basis.argmax(axis=1))) > 20
+    cnt = np.diff(ends, prepend=0).astype(np.float64)
+    tf, tw = [torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in (feats, w)]
+    out = _torch_forward("explicit", torch.tensor(pts, dtype=torch.float64), torch.tensor(smp, dtype=torch.float64), tf,
+                         neigh, ends, radii, torch.tensor(basis, dtype=torch.float64), tw)
+    out = out / (torch.tensor(cnt)[:, None] + 1e-6)
+    got = oracle.sphconv(pts, feats, smp, neigh, ends, radii, radial, azimuth, polar, w)
+    assert _relerr(got, out.detach().numpy()) < 1e-5
+    (out * torch.tensor(g, dtype=torch.float64)).sum().backward()
+    grads = oracle.sphconv_grads(pts, feats, smp, neigh, ends, radii, radial, azimuth, polar, w, g)
+    assert _relerr(grads[0], tw.grad.numpy()) < 1e-4 and _relerr(grads[1], tf.grad.numpy()) < 1e-4
+    # weight variance: mean over samples of |projection tile|^2 / count^2 (compute_variance_weights.cu:31-63)
+    proj = oracle.feat_basis_proj(basis, feats, neigh, ends).astype(np.float64)
+    per = np.where(cnt > 0, (proj ** 2).sum(axis=(1, 2)) / np.maximum(cnt, 1) ** 2, 0.0)
+    val = oracle.sphconv_weight_var(pts, feats, smp, neigh, ends, radii, radial, azimuth, polar)
+    assert np.isclose(val, 1.0 / per.mean(), rtol=1e-5)
