@@ -5,7 +5,7 @@ from .grid import Grid
 from .neighborhood import Neighborhood
 from .point_pooling import PointPooling
 from . import layers
-from .layers import IConvLayer, IConvLayerFactory, KPConv, KPConvFactory, MCConv, MCConvFactory
+from .layers import *  # noqa: F401,F403
+from .layers import __all__ as _layer_names
 
-__all__ = ["Pointcloud", "BoundingBox", "Grid", "Neighborhood", "PointPooling", "layers", "IConvLayer",
-           "IConvLayerFactory", "KPConv", "KPConvFactory", "MCConv", "MCConvFactory"]
+__all__ = ["Pointcloud", "BoundingBox", "Grid", "Neighborhood", "PointPooling", "layers"] + list(_layer_names)

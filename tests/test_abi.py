@@ -58,6 +58,17 @@ def test_argument_validation_needs_no_gpu(lib_path):
     rc = lib.pccnn_kpconv_forward(None, None, None, None, None, None, None, 0.5, None, 10, 10, 10, 3, 8, 65, 8, None,
                                   None, None, 0, None)
     assert rc == -2 and b"k=65" in lib.pccnn_last_error()
+    from pccnn_lib_amd import pccnn_lib_ops as ops
+    desc = _lib.Basis()
+    desc.kind = 9
+    rc = lib.pccnn_conv_forward(ctypes.byref(desc), None, None, None, None, None, None, None, 10, 10, 10, 3, 8, 1, 8,
+                                0, None, None, None, 0, None)
+    assert rc == -1 and b"basis kind 9" in lib.pccnn_last_error()
+    desc.kind, desc.nb0, desc.nb1, desc.nb2 = ops.BASIS_SPH, 4, 4, 4
+    desc.a = desc.b = desc.c = 16
+    rc = lib.pccnn_conv_weight_var(ctypes.byref(desc), None, None, None, None, None, None, 10, 10, 10, 3, 8, 0, None,
+                                   None, 0, None)
+    assert rc == -2 and b"k=65" in lib.pccnn_last_error()
     assert lib.pccnn_conv_workspace_bytes(1000, 5000, 32, 16, 64, 0) >= 1000 * 32 * 16 * 4
     assert lib.pccnn_find_neighbors_workspace_bytes(1000) >= 4000
 
@@ -67,8 +78,13 @@ def test_op_module_exports_reference_names():
     assert len(pccnn_lib_ops.REFERENCE_NAMES) == 26
     for name in pccnn_lib_ops.REFERENCE_NAMES:
         assert callable(getattr(pccnn_lib_ops, name))
-    with pytest.raises(NotImplementedError):
-        pccnn_lib_ops.sph_conv()
+    # every family validates its tensors before touching the library
+    import torch
+    z = torch.zeros(4, 3)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        pccnn_lib_ops.sph_conv(z, z, z, z, z, z, z, z, z, z)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        pccnn_lib_ops.point_conv(z, z, z, z, z)
 
 
 def test_ops_reject_cpu_tensors():
@@ -88,3 +104,13 @@ def test_layers_keep_reference_parameter_names():
     mc = MCConv(3, 8, 16, 16, 2)
     assert set(mc.state_dict()) == {"proj_axis_", "proj_bias_", "conv_weights_"}
     assert tuple(mc.conv_weights_.shape) == (2, 16 * 8, 8) and tuple(mc.proj_axis_.shape) == (3, 32)
+    from pccnn_lib_amd.pc.layers import KPConvN, PCCNN, PointConv, SPHConv
+    for cls, scale in ((KPConvN, 2.0), (PCCNN, 0.4)):
+        layer = cls(3, 8, 16, 16)
+        assert set(layer.state_dict()) == {"kernel_pts_", "sigma_", "conv_weights_"}
+        assert abs(float(layer.sigma_) / float(KPConv(3, 8, 16, 16).sigma_) - scale) < 1e-6
+    sph = SPHConv(3, 8, 16, 2, 5, 3)
+    assert set(sph.state_dict()) == {"radial_bins_", "azimuz_bins_", "polar_bins_", "conv_weights_"}
+    assert tuple(sph.conv_weights_.shape) == (31 * 8, 16)
+    pcv = PointConv(3, 8, 16, 16)
+    assert {"proj_axis_", "proj_bias_", "conv_weights_", "pdf_mlp_.0.weight", "pdf_mlp_.2.weight"} <= set(pcv.state_dict())

@@ -186,3 +186,126 @@ def test_families_empty_and_error_paths(ops):
     grads = ops.point_conv_basis_grads(d["pts"], d["radii"], d["samples"], none, torch.ones((3, 8), device=DEV),
                                        torch.zeros((1, 8), device=DEV), torch.zeros((0, 8), device=DEV))
     assert all(float(g.abs().max()) == 0.0 for g in grads)
+
+
+# --------------------------------------------------------------------------- layer modules
+
+def _layer_case(seed, c_in):
+    import pccnn_lib_amd as lib
+    pts, ids = synthetic.primitives(seed, 2, 1200)
+    rng = np.random.default_rng(seed)
+    feats = rng.normal(size=(pts.shape[0], c_in)).astype(np.float32)
+    pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+    pc.compute_pdf(np.full(3, 0.02, np.float32))
+    return lib, pts, feats, pc, rng
+
+
+def _host(x):
+    return x.detach().cpu().numpy()
+
+
+@pytest.mark.parametrize("kind", ["KPConvN", "PCCNN"])
+def test_density_kernel_point_layers(oracle, kind):
+    lib, pts, feats, pc, rng = _layer_case(31, 16)
+    torch.manual_seed(3)
+    layer = getattr(lib.pc.layers, kind)(3, 16, 24, 16).to(DEV)
+    tf = t(feats).requires_grad_(True)
+    out, nbh = layer(pc, pc, tf, 0.1)
+    g = rng.normal(size=tuple(out.shape)).astype(np.float32)
+    out.backward(t(g))
+    neigh, ends = _host(nbh.neighbors_), _host(nbh.start_ids_)
+    radii = np.full(3, 0.1, np.float32)
+    pdf = _host(pc.pts_unnorm_pdf_ * torch.prod(t(radii)))
+    kp, sigma, w = _host(layer.kernel_pts_), float(layer.sigma_.item()), _host(layer.conv_weights_)
+    if kind == "KPConvN":
+        exp = oracle.kpconvn(pts, pdf, feats, pts, neigh, ends, radii, kp, sigma, w)
+        exp_g = oracle.kpconvn_grads(pts, pdf, feats, pts, neigh, ends, radii, kp, sigma, w, g)
+    else:
+        exp = oracle.pccnn(pts, feats, pdf, pts, neigh, ends, radii, kp, sigma, w)
+        exp_g = oracle.pccnn_grads(pts, feats, pdf, pts, neigh, ends, radii, kp, sigma, w, g)
+    assert relerr(_host(out), exp) < FWD_TOL
+    assert relerr(_host(layer.conv_weights_.grad), exp_g[0]) < GRAD_TOL
+    assert relerr(_host(tf.grad), exp_g[1]) < GRAD_TOL
+    # variance-aware initialisation: the statistic of the warm-up pass is the op's
+    factory = getattr(lib.pc.layers, kind + "Factory")(16, True)
+    warm = factory.create_conv_layer(3, 16, 24).to(DEV)
+    factory.set_init_warmup_state_convs(True)
+    warm(pc, pc, t(feats), 0.1, nbh)
+    var = (oracle.kpconvn_weight_var(pts, pdf, feats, pts, neigh, ends, radii, _host(warm.kernel_pts_),
+                                     float(warm.sigma_.item())) if kind == "KPConvN" else
+           oracle.pccnn_weight_var(pts, feats, pdf, pts, neigh, ends, radii, _host(warm.kernel_pts_),
+                                   float(warm.sigma_.item())))
+    assert abs(warm.accum_weight_var_ - 1.0 / float(var)) < 1e-4 * abs(1.0 / float(var))
+
+
+def test_sphconv_layer(oracle):
+    lib, pts, feats, pc, rng = _layer_case(32, 8)
+    torch.manual_seed(4)
+    layer = lib.pc.layers.SPHConvFactory(2, 5, 3).create_conv_layer(3, 8, 12).to(DEV)
+    assert layer.num_basis_ == 31 and tuple(layer.conv_weights_.shape) == (31 * 8, 12)
+    tf = t(feats).requires_grad_(True)
+    out, nbh = layer(pc, pc, tf, 0.1)
+    g = rng.normal(size=tuple(out.shape)).astype(np.float32)
+    out.backward(t(g))
+    neigh, ends = _host(nbh.neighbors_), _host(nbh.start_ids_)
+    radii = np.full(3, 0.1, np.float32)
+    bins = [_host(b) for b in (layer.radial_bins_, layer.azimuz_bins_, layer.polar_bins_)]
+    w = _host(layer.conv_weights_)
+    assert relerr(_host(out), oracle.sphconv(pts, feats, pts, neigh, ends, radii, *bins, w)) < FWD_TOL
+    exp_g = oracle.sphconv_grads(pts, feats, pts, neigh, ends, radii, *bins, w, g)
+    assert relerr(_host(layer.conv_weights_.grad), exp_g[0]) < GRAD_TOL
+    assert relerr(_host(tf.grad), exp_g[1]) < GRAD_TOL
+
+
+@pytest.mark.parametrize("norm", ["none", "bn", "gn"])
+def test_pointconv_layer(oracle, norm):
+    lib, pts, feats, pc, rng = _layer_case(33, 8)
+    torch.manual_seed(5)
+    layer = lib.pc.layers.PointConvFactory(16, False, 1.0, norm == "bn", norm == "gn", 4) \
+        .create_conv_layer(3, 8, 12).to(DEV)
+    layer.proj_bias_.data.normal_(0, 0.1)
+    tf = t(feats).requires_grad_(True)
+    out, nbh = layer(pc, pc, tf, 0.1)
+    g = rng.normal(size=tuple(out.shape)).astype(np.float32)
+    out.backward(t(g))
+    # (as in the reference, the group norm of the basis never feeds the output, so its parameters get no gradient)
+    assert all(p.grad is not None and torch.isfinite(p.grad).all()
+               for n, p in layer.named_parameters() if not n.startswith("basis_gn_"))
+    if norm != "none":
+        return
+    # without normalisation layers the module is: basis op -> relu -> * density network -> conv op
+    neigh, ends = _host(nbh.neighbors_), _host(nbh.start_ids_)
+    scale = _host(layer.__density_scale__(pc, nbh))
+    assert scale.shape == (neigh.shape[0], 1) and 0.0 < scale.min() and scale.max() < 1.0
+    basis, _ = oracle.pointconv_basis(pts, np.ones(3, np.float32), pts, neigh, _host(layer.proj_axis_),
+                                      _host(layer.proj_bias_))
+    act = (np.maximum(basis, 0) * scale).astype(np.float32)
+    w = _host(layer.conv_weights_)
+    assert relerr(_host(out), oracle.pointconv(act, feats, neigh, ends, w)) < 2e-5
+    exp_g = oracle.pointconv_grads(act, feats, neigh, ends, w, g)
+    assert relerr(_host(layer.conv_weights_.grad), exp_g[0]) < GRAD_TOL
+    assert relerr(_host(tf.grad), exp_g[1]) < GRAD_TOL
+    # the basis gradient flows on through relu and the basis op into the projection parameters
+    dbasis = exp_g[2] * scale * (basis > 0)
+    exp_b = oracle.pointconv_basis_grads(pts, np.ones(3, np.float32), pts, neigh, _host(layer.proj_axis_),
+                                         _host(layer.proj_bias_), dbasis.astype(np.float32))
+    assert relerr(_host(layer.proj_axis_.grad), exp_b[2]) < GRAD_TOL
+    assert relerr(_host(layer.proj_bias_.grad), exp_b[3]) < GRAD_TOL
+
+
+def test_group_normalization_and_bias():
+    import pccnn_lib_amd as lib
+    pts, ids = synthetic.primitives(3, 3, 200)
+    pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+    feats = torch.randn((600, 8), device=DEV) * 3 + 1
+    gn = lib.pc.layers.GroupNormalization(8, 4).to(DEV)
+    out = gn(feats, pc).detach()
+    # per cloud and group column the normalised values have zero mean and unit variance
+    view = out.reshape(-1, 4)
+    vid = pc.batch_ids_.reshape(-1, 1).repeat(1, 2).reshape(-1).to(torch.int64)
+    for b in range(3):
+        sel = view[vid == b]
+        assert float(sel.mean(dim=0).abs().max()) < 1e-5 and float((sel.var(dim=0, unbiased=False) - 1).abs().max()) < 1e-4
+    bias = lib.pc.layers.Bias(8).to(DEV)
+    bias.bias_.data.fill_(0.5)
+    assert torch.equal(bias(feats), feats + 0.5)
