@@ -195,19 +195,70 @@ conv_proj_fwd_kernel(ConvGeom g, const float *__restrict__ feats, float *__restr
         }
         __syncthreads();
     }
-    if (fvalid) {
-        float *dst = proj + ((int64_t)s * g.c_in + f) * g.k;
-        if (g.k == KPAD && (KPAD % 4) == 0) {
+    // The tile of this workgroup, [features][k], is contiguous in memory: hand the accumulators over through
+    // LDS so that every store instruction writes one contiguous run instead of 64 rows' worth of pieces.
+    float *tile = &w_lds[0][0];
 #pragma unroll
-            for (int q = 0; q < KPAD; q += 4) {
-                float4 v = make_float4(acc[q], acc[q + 1], acc[q + 2], acc[q + 3]);
-                *(float4 *)(dst + q) = v;
-            }
-        } else {
-#pragma unroll
-            for (int q = 0; q < KPAD; ++q)
-                if (q < g.k) dst[q] = acc[q];
+    for (int q = 0; q < KPAD; q += 4)
+        *(float4 *)&tile[lane * KPAD + q] = make_float4(acc[q], acc[q + 1], acc[q + 2], acc[q + 3]);
+    __syncthreads();
+    const int f0 = blockIdx.y * 64;
+    const int nf = (g.c_in - f0) < 64 ? (g.c_in - f0) : 64;
+    float *dst = proj + ((int64_t)s * g.c_in + f0) * g.k;
+    if (g.k == KPAD) {
+        for (int i = lane; i < nf * (KPAD / 4); i += 64) ((float4 *)dst)[i] = ((const float4 *)tile)[i];
+    } else {
+        for (int idx = lane; idx < nf * g.k; idx += 64) {
+            const int ff = idx / g.k, q = idx - ff * g.k;
+            dst[idx] = tile[ff * KPAD + q];
         }
+    }
+}
+
+// Derivative of one basis value w.r.t. the pair's normalised offset, the neighbor's density and the basis
+// parameters of this lane's k.  gk = upstream gradient of the basis value; (gx, gy, gz, gpdf) receive the
+// offset / density gradients, (p0..p3) accumulate the parameter gradients.
+template <int BASIS>
+__device__ __forceinline__ void basis_derivative(const ConvGeom &g, const LaneBasis<BASIS> &lb, float dx, float dy,
+                                                 float dz, float pdf, float gk, float &gx, float &gy, float &gz,
+                                                 float &gpdf, float &p0, float &p1, float &p2, float &p3)
+{
+    // The KPConv correlation has a kink where a pair sits exactly one sigma away from a kernel
+    // point, and every self pair (offset 0) does so for the kernel points closest to the centre.
+    // Which side of the kink such a pair falls on is decided by the last bit of the fp32
+    // distance, so the distance is evaluated exactly as written: no fused multiply-add.
+#pragma clang fp contract(off)
+    const float c0 = lb.c0, c1 = lb.c1, c2 = lb.c2, c3 = lb.c3;
+    if (BASIS == BASIS_KP || BASIS == BASIS_KPN) {
+        // kernel_pts_basis_grads; KPConvN feeds it the gradient already divided by the density
+        const float gin = (BASIS == BASIS_KPN) ? gk / pdf : gk;
+        const float vx = c0 - dx, vy = c1 - dy, vz = c2 - dz;
+        const float dist = sqrtf(fmaxf(vx * vx + vy * vy + vz * vz, 0.0f));
+        const float res = 1.0f - dist / g.sigma;
+        if (res >= 0.0f) {
+            const float c = -(gin / g.sigma) * (1.0f / (dist + 1e-6f));
+            const float cx = c * vx, cy = c * vy, cz = c * vz;
+            gx = -cx; gy = -cy; gz = -cz;
+            p0 += cx; p1 += cy; p2 += cz;
+        }
+    } else if (BASIS == BASIS_GAUSS) {
+        const float vx = c0 - dx, vy = c1 - dy, vz = c2 - dz;
+        const float e = expf(-((vx * vx + vy * vy + vz * vz) / (2.0f * g.sigma * g.sigma)));
+        const float gin = gk / pdf;
+        gpdf = -((e / pdf) * gk) / pdf;
+        const float c = -gin * e * (1.0f / (g.sigma * g.sigma));
+        const float cx = c * vx, cy = c * vy, cz = c * vz;
+        gx = -cx; gy = -cy; gz = -cz;
+        p0 += cx; p1 += cy; p2 += cz;
+    } else if (BASIS == BASIS_MLP) {
+        const float inv_pd = 1.0f / pdf;
+        float act = dx * c0 + dy * c1 + dz * c2 + c3;
+        const bool pos = act > 0.0f;
+        act = pos ? act : act * 0.2f;
+        gpdf = -(act * gk * inv_pd * inv_pd);
+        const float c = gk * inv_pd * (pos ? 1.0f : 0.2f);
+        gx = c * c0; gy = c * c1; gz = c * c2;
+        p0 += dx * c; p1 += dy * c; p2 += dz * c; p3 += c;
     }
 }
 
@@ -219,12 +270,24 @@ conv_proj_fwd_kernel(ConvGeom g, const float *__restrict__ feats, float *__restr
 // The basis values of up to 64 pairs are evaluated once (KPAD lanes per pair) and parked in LDS, from where
 // the dF stage reads them as broadcasts; the neighbor's feature row is read coalesced from memory, used by
 // the dF stage from registers and handed to the dw stage through LDS, so that each stage runs KPAD
-// multiply-adds per pair and lane.  dw is accumulated in LDS over the feature blocks and stored coalesced.
+// multiply-adds per pair and lane.  dw is accumulated in LDS over the feature blocks.
+//
+// For a basis given by the caller (EXPLICIT) dw is the result and is stored coalesced.  For the parametric
+// bases the kernel goes on while the chunk is still in LDS: KPAD lanes per pair apply the basis derivative
+// (lane = basis index k), shuffles reduce the offset / density gradients over k, and the chunk's values are
+// scattered with float atomics, sixteen pairs x (x, y, z, density) per instruction.  The sample's own gradient
+// and the basis-parameter gradients stay in registers until the end; the latter are added to one of
+// PARAM_ROWS partial rows ([component][k], 256 floats) that the conv_param_reduce kernels sum afterwards.
+#define PARAM_ROWS 256
+
 template <int BASIS, int KPAD, bool want_df, bool want_db>
 __global__ void __launch_bounds__(64)
 conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *__restrict__ proj_grads,
-                     float *__restrict__ feat_grads, float *__restrict__ basis_grads)
+                     float *__restrict__ feat_grads, float *__restrict__ basis_grads, float *__restrict__ d_pts,
+                     float *__restrict__ d_samples, float *__restrict__ d_pdf, float *__restrict__ param_partials)
 {
+    constexpr bool FUSED = want_db && BasisTraits<BASIS>::differentiable;   // basis derivative applied here
+    __shared__ __attribute__((aligned(16))) float g_lds[FUSED ? 64 : 1][4];
     // want_df / want_db: which of the two stages this instantiation runs
     constexpr int PARTS = 64 / KPAD;                                // feature groups of the dw stage
     constexpr int ROWS = 4;                                         // feature rows in flight
@@ -245,6 +308,8 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
     LaneBasis<BASIS> lb;
     lb.load(g, k);
     const int fblocks = (g.c_in + 63) / 64;
+    float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;       // parameter gradients of this lane's k (FUSED)
+    float sg = 0.f;                                     // component (lane & 3) of the sample's gradient, unsigned
 
     for (int cb = lo; cb < hi; cb += 64) {
         const int cnt = (hi - cb) < 64 ? (hi - cb) : 64;
@@ -340,7 +405,37 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
             }
         }
         __syncthreads();
-        if (want_db) {
+        if (FUSED) {
+            for (int p = 0; p * PARTS < cnt; ++p) {
+                const int j = p * PARTS + part;
+                const float jx = __shfl(dx, j), jy = __shfl(dy, j), jz = __shfl(dz, j), jp = __shfl(pd, j);
+                float gx = 0.f, gy = 0.f, gz = 0.f, gpdf = 0.f;
+                if (j < cnt && lb.active)
+                    basis_derivative<BASIS>(g, lb, jx, jy, jz, jp, db_lds[j][k], gx, gy, gz, gpdf, p0, p1, p2, p3);
+#pragma unroll
+                for (int o = KPAD / 2; o > 0; o >>= 1) {
+                    gx += __shfl_xor(gx, o);
+                    gy += __shfl_xor(gy, o);
+                    gz += __shfl_xor(gz, o);
+                    if (BasisTraits<BASIS>::pdf_grad) gpdf += __shfl_xor(gpdf, o);
+                }
+                if (k < 4) g_lds[j][k] = (k == 0) ? gx * ir0 : (k == 1) ? gy * ir1 : (k == 2) ? gz * ir2 : gpdf;
+            }
+            __syncthreads();
+            for (int i = 0; i * 16 < cnt; ++i) {
+                const int j = i * 16 + (lane >> 2), comp = lane & 3;
+                const int jn = __shfl(nidx, j);
+                if (j < cnt) {
+                    const float v = g_lds[j][comp];
+                    if (comp < 3) {
+                        if (d_pts) unsafeAtomicAdd(&d_pts[(int64_t)jn * 3 + comp], v);
+                        sg += v;
+                    } else if (BasisTraits<BASIS>::pdf_grad && d_pdf) {
+                        unsafeAtomicAdd(&d_pdf[jn], v);
+                    }
+                }
+            }
+        } else if (want_db) {
             for (int idx = lane; idx < cnt * KPAD; idx += 64) {
                 const int j = idx / KPAD, kk = idx % KPAD;
                 if (kk < g.k) basis_grads[(int64_t)(cb + j) * g.k + kk] = db_lds[j][kk];
@@ -348,173 +443,29 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
         }
         __syncthreads();
     }
+    if (FUSED) {
+#pragma unroll
+        for (int o = 4; o < 64; o <<= 1) sg += __shfl_xor(sg, o);
+        if (lane < 3 && d_samples) d_samples[s * 3 + lane] = -sg;
+        if (param_partials) {
+#pragma unroll
+            for (int o = KPAD; o < 64; o <<= 1) {
+                p0 += __shfl_xor(p0, o);
+                p1 += __shfl_xor(p1, o);
+                p2 += __shfl_xor(p2, o);
+                if (BasisTraits<BASIS>::axis) p3 += __shfl_xor(p3, o);
+            }
+            float *row = param_partials + (int64_t)(blockIdx.x % PARAM_ROWS) * 256;
+            constexpr int COMPS = BasisTraits<BASIS>::axis ? 4 : 3;
+            for (int c = part; c < COMPS; c += PARTS) {
+                const float v = (c == 0) ? p0 : (c == 1) ? p1 : (c == 2) ? p2 : p3;
+                unsafeAtomicAdd(&row[c * 64 + k], v);
+            }
+        }
+    }
 }
 
-// Derivative of the basis w.r.t. its inputs and parameters, one wavefront per sample.
-// KPAD lanes own one pair (lane = basis index k), so 64 / KPAD pairs are handled per step and BB_UNROLL
-// steps are in flight at once (their loads are independent).  Per-pair basis gradients are one coalesced
-// read; the offset / density gradients are reduced across the KPAD lanes with shuffles; the point and
-// density gradients are scattered with one float atomic per pair and coordinate, the sample's own gradient
-// is accumulated in registers and stored once.  Every lane keeps the parameter gradients of its own k in
-// registers; a workgroup reduces them in LDS and stores one partial row that the conv_param_reduce kernels sum
-// in a fixed order.  param layout: KP -> d_kernel_pts [K,3];  MLP -> d_axis [3,K] followed by d_bias [K].
-#define BB_UNROLL 4
-#define BB_SAMPLES_PER_WAVE 4
-#define BB_SAMPLES_PER_BLOCK (4 * BB_SAMPLES_PER_WAVE)
-
-template <int BASIS, int KPAD>
-__global__ void __launch_bounds__(256)
-conv_basis_bwd_kernel(ConvGeom g, const float *__restrict__ basis_grads, float *__restrict__ d_pts,
-                      float *__restrict__ d_samples, float *__restrict__ d_pdf, float *__restrict__ param_partials)
-{
-    // The KPConv correlation has a kink where a pair sits exactly one sigma away from a kernel
-    // point, and every self pair (offset 0) does so for the kernel points closest to the centre.
-    // Which side of the kink such a pair falls on is decided by the last bit of the fp32
-    // distance, so the distance is evaluated exactly as written: no fused multiply-add.
-#pragma clang fp contract(off)
-    __shared__ float lds_param[4][4 * 64];
-    constexpr int PAIRS = 64 / KPAD;                                // pairs per step
-    const int lane = pccnn_lane();
-    const int wave = threadIdx.x >> 6;
-    const int k = lane % KPAD;
-    const int sub = lane / KPAD;
-    const bool kvalid = k < g.k;
-    const float ir0 = 1.0f / g.radii[0], ir1 = 1.0f / g.radii[1], ir2 = 1.0f / g.radii[2];
-    float c0 = 0.f, c1 = 0.f, c2 = 0.f, c3 = 0.f;                   // this lane's basis parameters
-    if (kvalid) {
-        if (BasisTraits<BASIS>::kernel_pts) {
-            c0 = g.basis_a[k * 3 + 0]; c1 = g.basis_a[k * 3 + 1]; c2 = g.basis_a[k * 3 + 2];
-        } else {
-            c0 = g.basis_a[k]; c1 = g.basis_a[g.k + k]; c2 = g.basis_a[2 * g.k + k]; c3 = g.basis_b[k];
-        }
-    }
-    float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;                   // parameter gradient sums of this lane's k
-  for (int rep = 0; rep < BB_SAMPLES_PER_WAVE; ++rep) {
-    const int64_t s = ((int64_t)blockIdx.x * BB_SAMPLES_PER_WAVE + rep) * 4 + wave;
-    const bool svalid = s < g.m;
-    float sgx = 0.f, sgy = 0.f, sgz = 0.f;                          // the sample's own gradient (before the sign)
-    int lo = 0, hi = 0;
-    float sx = 0.f, sy = 0.f, sz = 0.f;
-    if (svalid) {
-        lo = s > 0 ? g.ends[s - 1] : 0;
-        hi = g.ends[s];
-        sx = g.samples[s * 3 + 0]; sy = g.samples[s * 3 + 1]; sz = g.samples[s * 3 + 2];
-    }
-    for (int base = lo; base < hi; base += PAIRS * BB_UNROLL) {
-        int nidx[BB_UNROLL];
-        float px[BB_UNROLL], py[BB_UNROLL], pz[BB_UNROLL], pdv[BB_UNROLL], gk[BB_UNROLL];
-        bool tv[BB_UNROLL];
-#pragma unroll
-        for (int u = 0; u < BB_UNROLL; ++u) {
-            const int t = base + u * PAIRS + sub;
-            tv[u] = t < hi;
-            nidx[u] = tv[u] ? g.neigh[t].x : 0;
-            gk[u] = (tv[u] && kvalid) ? basis_grads[(int64_t)t * g.k + k] : 0.0f;
-        }
-#pragma unroll
-        for (int u = 0; u < BB_UNROLL; ++u) {
-            px[u] = g.pts[(int64_t)nidx[u] * 3 + 0];
-            py[u] = g.pts[(int64_t)nidx[u] * 3 + 1];
-            pz[u] = g.pts[(int64_t)nidx[u] * 3 + 2];
-            pdv[u] = BasisTraits<BASIS>::uses_pdf ? g.pdf[nidx[u]] : 1.0f;
-        }
-#pragma unroll
-        for (int u = 0; u < BB_UNROLL; ++u) {
-            float gx = 0.f, gy = 0.f, gz = 0.f, gpdf = 0.f;
-            if (tv[u] && kvalid) {
-                const float dx = (px[u] - sx) * ir0, dy = (py[u] - sy) * ir1, dz = (pz[u] - sz) * ir2;
-                if (BASIS == BASIS_KP || BASIS == BASIS_KPN) {
-                    // kernel_pts_basis_grads; KPConvN feeds it the gradient already divided by the density
-                    const float gin = (BASIS == BASIS_KPN) ? gk[u] / pdv[u] : gk[u];
-                    const float vx = c0 - dx, vy = c1 - dy, vz = c2 - dz;
-                    const float dist = sqrtf(fmaxf(vx * vx + vy * vy + vz * vz, 0.0f));
-                    const float res = 1.0f - dist / g.sigma;
-                    if (res >= 0.0f) {
-                        const float c = -(gin / g.sigma) * (1.0f / (dist + 1e-6f));
-                        const float cx = c * vx, cy = c * vy, cz = c * vz;
-                        gx = -cx; gy = -cy; gz = -cz;
-                        p0 += cx; p1 += cy; p2 += cz;
-                    }
-                } else if (BASIS == BASIS_GAUSS) {
-                    const float vx = c0 - dx, vy = c1 - dy, vz = c2 - dz;
-                    const float e = expf(-((vx * vx + vy * vy + vz * vz) / (2.0f * g.sigma * g.sigma)));
-                    const float gin = gk[u] / pdv[u];
-                    gpdf = -((e / pdv[u]) * gk[u]) / pdv[u];
-                    const float c = -gin * e * (1.0f / (g.sigma * g.sigma));
-                    const float cx = c * vx, cy = c * vy, cz = c * vz;
-                    gx = -cx; gy = -cy; gz = -cz;
-                    p0 += cx; p1 += cy; p2 += cz;
-                } else if (BASIS == BASIS_LINEAR) {
-                    const float c = gk[u];
-                    gx = c * c0; gy = c * c1; gz = c * c2;
-                    p0 += dx * c; p1 += dy * c; p2 += dz * c; p3 += c;
-                } else {
-                    const float inv_pd = 1.0f / pdv[u];
-                    float act = dx * c0 + dy * c1 + dz * c2 + c3;
-                    const bool pos = act > 0.0f;
-                    act = pos ? act : act * 0.2f;
-                    gpdf = -(act * gk[u] * inv_pd * inv_pd);
-                    const float c = gk[u] * inv_pd * (pos ? 1.0f : 0.2f);
-                    gx = c * c0; gy = c * c1; gz = c * c2;
-                    p0 += dx * c; p1 += dy * c; p2 += dz * c; p3 += c;
-                }
-            }
-#pragma unroll
-            for (int o = KPAD / 2; o > 0; o >>= 1) {
-                gx += __shfl_xor(gx, o);
-                gy += __shfl_xor(gy, o);
-                gz += __shfl_xor(gz, o);
-                if (BasisTraits<BASIS>::pdf_grad) gpdf += __shfl_xor(gpdf, o);
-            }
-            if (tv[u] && k == 0) {
-                gx *= ir0; gy *= ir1; gz *= ir2;
-                if (d_pts) {
-                    unsafeAtomicAdd(&d_pts[(int64_t)nidx[u] * 3 + 0], gx);
-                    unsafeAtomicAdd(&d_pts[(int64_t)nidx[u] * 3 + 1], gy);
-                    unsafeAtomicAdd(&d_pts[(int64_t)nidx[u] * 3 + 2], gz);
-                }
-                if (BasisTraits<BASIS>::pdf_grad && d_pdf) unsafeAtomicAdd(&d_pdf[nidx[u]], gpdf);
-                sgx += gx; sgy += gy; sgz += gz;
-            }
-        }
-    }
-    // the sample's gradient: sum over the lanes that own a pair (k == 0 of every sub-group)
-#pragma unroll
-    for (int o = KPAD; o < 64; o <<= 1) {
-        sgx += __shfl_xor(sgx, o);
-        sgy += __shfl_xor(sgy, o);
-        sgz += __shfl_xor(sgz, o);
-    }
-    if (svalid && lane == 0 && d_samples) {
-        d_samples[s * 3 + 0] = -sgx;
-        d_samples[s * 3 + 1] = -sgy;
-        d_samples[s * 3 + 2] = -sgz;
-    }
-  }
-#pragma unroll
-    for (int o = KPAD; o < 64; o <<= 1) {
-        p0 += __shfl_xor(p0, o);
-        p1 += __shfl_xor(p1, o);
-        p2 += __shfl_xor(p2, o);
-        p3 += __shfl_xor(p3, o);
-    }
-    if (sub == 0) {
-        lds_param[wave][k] = p0;
-        lds_param[wave][64 + k] = p1;
-        lds_param[wave][128 + k] = p2;
-        lds_param[wave][192 + k] = p3;
-    }
-    __syncthreads();
-    // one partial row of 4 * 64 floats per workgroup: [component][k]
-    const int i = threadIdx.x;
-    const int comp = i >> 6, kk = i & 63;
-    float v = 0.0f;
-    if (kk < KPAD) v = lds_param[0][comp * 64 + kk] + lds_param[1][comp * 64 + kk] + lds_param[2][comp * 64 + kk] +
-                       lds_param[3][comp * 64 + kk];
-    param_partials[(int64_t)blockIdx.x * 256 + i] = v;
-}
-
-// Sums the per-workgroup partial rows ([rows][256], column = component * 64 + basis index) in a fixed order.
+// Sums partial rows ([rows][256], column = component * 64 + basis index) in a fixed order.
 // Stage 1: workgroup b adds the rows b, b + G, b + 2G, ... (thread = column, coalesced); stage 2: one
 // workgroup adds the G stage-1 rows and writes every value to its place in the parameter gradient tensors.
 #define PARAM_REDUCE_GROUPS 64
@@ -703,30 +654,40 @@ static int launch_proj_fwd(const ConvGeom &g, const float *feats, float *proj, h
     return PCCNN_OK;
 }
 
+// Where the basis stage of the backward kernel puts its results; members a call does not want are null.
+struct BasisGradOut {
+    float *basis_grads;     // [t,k], EXPLICIT only
+    float *d_pts, *d_samples, *d_pdf;
+    float *partials;        // [PARAM_ROWS][256], zeroed by the caller
+};
+
 template <int BASIS, int KPAD>
 static void launch_proj_bwd_k(const ConvGeom &g, const float *feats, const float *proj_grads, float *feat_grads,
-                              float *basis_grads, hipStream_t s)
+                              bool want_basis, const BasisGradOut &o, hipStream_t s)
 {
     dim3 grid((unsigned)g.m);
-    if (feat_grads && basis_grads)
-        conv_proj_bwd_kernel<BASIS, KPAD, true, true><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads);
+    if (feat_grads && want_basis)
+        conv_proj_bwd_kernel<BASIS, KPAD, true, true><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, o.basis_grads,
+                                                                          o.d_pts, o.d_samples, o.d_pdf, o.partials);
     else if (feat_grads)
-        conv_proj_bwd_kernel<BASIS, KPAD, true, false><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads);
+        conv_proj_bwd_kernel<BASIS, KPAD, true, false><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, nullptr,
+                                                                           nullptr, nullptr, nullptr, nullptr);
     else
-        conv_proj_bwd_kernel<BASIS, KPAD, false, true><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, basis_grads);
+        conv_proj_bwd_kernel<BASIS, KPAD, false, true><<<grid, 64, 0, s>>>(g, feats, proj_grads, nullptr, o.basis_grads,
+                                                                           o.d_pts, o.d_samples, o.d_pdf, o.partials);
 }
 
 template <int BASIS>
 static int launch_proj_bwd(const ConvGeom &g, const float *feats, const float *proj_grads, float *feat_grads,
-                           float *basis_grads, hipStream_t s)
+                           bool want_basis, const BasisGradOut &o, hipStream_t s)
 {
-    if (!feat_grads && !basis_grads) return PCCNN_OK;
+    if (!feat_grads && !want_basis) return PCCNN_OK;
     PccnnTimed timed(PCCNN_T_PROJ_BWD, s);
     switch (kpad_of(g.k)) {
-    case 8: launch_proj_bwd_k<BASIS, 8>(g, feats, proj_grads, feat_grads, basis_grads, s); break;
-    case 16: launch_proj_bwd_k<BASIS, 16>(g, feats, proj_grads, feat_grads, basis_grads, s); break;
-    case 32: launch_proj_bwd_k<BASIS, 32>(g, feats, proj_grads, feat_grads, basis_grads, s); break;
-    default: launch_proj_bwd_k<BASIS, 64>(g, feats, proj_grads, feat_grads, basis_grads, s); break;
+    case 8: launch_proj_bwd_k<BASIS, 8>(g, feats, proj_grads, feat_grads, want_basis, o, s); break;
+    case 16: launch_proj_bwd_k<BASIS, 16>(g, feats, proj_grads, feat_grads, want_basis, o, s); break;
+    case 32: launch_proj_bwd_k<BASIS, 32>(g, feats, proj_grads, feat_grads, want_basis, o, s); break;
+    default: launch_proj_bwd_k<BASIS, 64>(g, feats, proj_grads, feat_grads, want_basis, o, s); break;
     }
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
@@ -756,7 +717,7 @@ extern "C" size_t pccnn_conv_workspace_bytes(int64_t m, int64_t t, int c_in, int
     if (!backward) return proj + 256;
     size_t basis_g = pccnn_align((size_t)t * k * sizeof(float));
     size_t splitk = pccnn_align((size_t)CONV_SPLIT_K * c_in * k * c_out * sizeof(float));
-    size_t partials = pccnn_align(((size_t)pccnn_ceil_div(m, BB_SAMPLES_PER_BLOCK) + PARAM_REDUCE_GROUPS) * 256 * sizeof(float));
+    size_t partials = pccnn_align(((size_t)PARAM_ROWS + PARAM_REDUCE_GROUPS) * 256 * sizeof(float));
     size_t scaled = pccnn_align((size_t)m * c_out * sizeof(float));
     return 2 * proj + basis_g + splitk + partials + scaled + 256;
 }
@@ -813,7 +774,7 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     const bool want_basis = want_par || want_pts || want_pdf;
     int rc;
     PccnnArena arena(workspace, workspace_bytes);
-    const int64_t partial_rows = pccnn_ceil_div(g.m > 0 ? g.m : 1, BB_SAMPLES_PER_BLOCK);
+    const int64_t partial_rows = PARAM_ROWS;
     float *partials = arena.take<float>((size_t)(partial_rows + PARAM_REDUCE_GROUPS) * 256);
     float *stage = partials + partial_rows * 256;
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv backward: workspace of %zu bytes, need %zu", workspace_bytes,
@@ -864,30 +825,16 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     rc = pccnn_gemm_f32(in_grads, weights, d_proj, g.m, inner, co, 0, 1, c_out, co, (int64_t)g.c_in * g.k, num_mlps, co,
                         inner * co, inner, 1, nullptr, 0, s);
     if (rc != PCCNN_OK) return rc;
-    if ((rc = launch_proj_bwd<BASIS>(g, feats, d_proj, want_f ? d_feats : nullptr, want_basis ? basis_g : nullptr,
-                                     s)) != PCCNN_OK)
+    BasisGradOut o = {basis_g, want_pts ? d_pts : nullptr, want_pts ? d_samples : nullptr, want_pdf ? d_pdf : nullptr,
+                      (want_par && Tr::differentiable) ? partials : nullptr};
+    if (o.partials && (rc = pccnn_fill_f32(partials, 0.0f, partial_rows * 256, s)) != PCCNN_OK) return rc;
+    if ((rc = launch_proj_bwd<BASIS>(g, feats, d_proj, want_f ? d_feats : nullptr, want_basis, o, s)) != PCCNN_OK)
         return rc;
-    if (!want_basis || !Tr::differentiable) return PCCNN_OK;
-    const unsigned blocks = (unsigned)partial_rows;
-    float *o_pts = want_pts ? d_pts : nullptr, *o_smp = want_pts ? d_samples : nullptr;
-    float *o_pdf = want_pdf ? d_pdf : nullptr;
-    if constexpr (Tr::differentiable) {
-        {
-            PccnnTimed timed(PCCNN_T_BASIS_BWD, s);
-            switch (kpad_of(g.k)) {
-            case 8: conv_basis_bwd_kernel<BASIS, 8><<<blocks, 256, 0, s>>>(g, basis_g, o_pts, o_smp, o_pdf, partials); break;
-            case 16: conv_basis_bwd_kernel<BASIS, 16><<<blocks, 256, 0, s>>>(g, basis_g, o_pts, o_smp, o_pdf, partials); break;
-            case 32: conv_basis_bwd_kernel<BASIS, 32><<<blocks, 256, 0, s>>>(g, basis_g, o_pts, o_smp, o_pdf, partials); break;
-            default: conv_basis_bwd_kernel<BASIS, 64><<<blocks, 256, 0, s>>>(g, basis_g, o_pts, o_smp, o_pdf, partials); break;
-            }
-        }
+    if (o.partials) {
+        conv_param_reduce1_kernel<<<PARAM_REDUCE_GROUPS, 256, 0, s>>>(partials, partial_rows, stage);
         PCCNN_LAUNCH_CHECK();
-        if (want_par) {
-            conv_param_reduce1_kernel<<<PARAM_REDUCE_GROUPS, 256, 0, s>>>(partials, partial_rows, stage);
-            PCCNN_LAUNCH_CHECK();
-            conv_param_reduce2_kernel<BASIS><<<1, 256, 0, s>>>(stage, g.k, d_param_a, d_param_b);
-            PCCNN_LAUNCH_CHECK();
-        }
+        conv_param_reduce2_kernel<BASIS><<<1, 256, 0, s>>>(stage, g.k, d_param_a, d_param_b);
+        PCCNN_LAUNCH_CHECK();
     }
     return PCCNN_OK;
 }
