@@ -147,9 +147,11 @@ def main():
     from pccnn_lib_amd.op_wrappers import ComputeMCConv
     leaves = [x.clone().requires_grad_(True) for x in (pts, pdf, feats, axis, bias, weights)]
 
+    mirror = nbh.mirror()        # the samples are the points: symmetric pair list (built once per neighborhood)
+
     def conv_step():
         p, q, f, a, b, w = leaves
-        out = ComputeMCConv.apply(p, q, f, p, neigh, ends, radii, a, b, w)
+        out = ComputeMCConv.apply(p, q, f, p, neigh, ends, radii, a, b, w, mirror)
         return torch.autograd.grad(out, leaves, out_grads)
 
     def conv_step_fw_only():

@@ -171,12 +171,15 @@ int pccnn_compact_selected(const int32_t *selected, const int32_t *selected_scan
  *
  * 1 <= k <= 64.
  *
- * Two arguments go beyond the reference's interface.  `proj_out` / `proj` (nullable): the projection
+ * Three arguments go beyond the reference's interface.  `proj_out` / `proj` (nullable): the projection
  * P f32[m, c_in, k] (k fastest) that the forward call builds on its way to `out`; a caller that keeps it
  * (proj_out != NULL) can hand it to the backward call, which otherwise rebuilds it like the reference does
  * (kpconv.cu:78-87).  `grad_mask`: which gradients to produce (PCCNN_GRAD_* bits; PCCNN_GRAD_ALL is the
  * reference's behaviour).  Requested outputs are fully overwritten; outputs not requested may be NULL and are
- * not touched. */
+ * not touched.  `mirror` (nullable, i32[t]): for a symmetric neighborhood (the samples are the points, so
+ * n == m, and the search was not capped) the index of pair (b, a) for every pair (a, b), from
+ * pccnn_mirror_pairs; with it d_pts and d_pdf are summed per point in a fixed order instead of with float
+ * atomics (the reference scatters with index_add_ atomics, pt_diff.cu:51-80). */
 #define PCCNN_GRAD_WEIGHTS 1
 #define PCCNN_GRAD_FEATS 2
 #define PCCNN_GRAD_BASIS_PARAMS 4 /* d_kernel_pts, or d_axis and d_bias */
@@ -184,14 +187,18 @@ int pccnn_compact_selected(const int32_t *selected, const int32_t *selected_scan
 #define PCCNN_GRAD_PTS 16         /* d_pts and d_samples */
 #define PCCNN_GRAD_ALL 31
 size_t pccnn_conv_workspace_bytes(int64_t m, int64_t t, int c_in, int k, int c_out, int backward);
+/* mirror_out i32[t]: index of the pair (point b, sample a) for pair t = (point a, sample b), -1 when absent;
+ * *missing_out i32 = number of pairs without a mirror (0 for a symmetric neighborhood). */
+int pccnn_mirror_pairs(const int32_t *neigh, const int32_t *ends, int64_t t, int64_t m, int32_t *mirror_out,
+                       int32_t *missing_out, void *stream);
 int pccnn_kpconv_forward(const float *pts, const float *feats, const float *samples, const int32_t *neigh,
                          const int32_t *ends, const float *radii, const float *kernel_pts, float sigma,
                          const float *weights, int64_t n, int64_t m, int64_t t, int d, int c_in, int k, int c_out,
                          float *out, float *proj_out, void *workspace, size_t workspace_bytes, void *stream);
 int pccnn_kpconv_backward(const float *pts, const float *feats, const float *samples, const int32_t *neigh,
                           const int32_t *ends, const float *radii, const float *kernel_pts, float sigma,
-                          const float *weights, const float *in_grads, const float *proj, int grad_mask,
-                          int64_t n, int64_t m, int64_t t, int d, int c_in, int k, int c_out,
+                          const float *weights, const float *in_grads, const float *proj, const int32_t *mirror,
+                          int grad_mask, int64_t n, int64_t m, int64_t t, int d, int c_in, int k, int c_out,
                           float *d_weights, float *d_feats, float *d_kernel_pts, float *d_pts, float *d_samples,
                           void *workspace, size_t workspace_bytes, void *stream);
 int pccnn_mcconv_forward(const float *pts, const float *pdf, const float *feats, const float *samples,
@@ -202,7 +209,7 @@ int pccnn_mcconv_forward(const float *pts, const float *pdf, const float *feats,
 int pccnn_mcconv_backward(const float *pts, const float *pdf, const float *feats, const float *samples,
                           const int32_t *neigh, const int32_t *ends, const float *radii, const float *axis,
                           const float *bias, const float *weights, const float *in_grads, const float *proj,
-                          int grad_mask,
+                          const int32_t *mirror, int grad_mask,
                           int64_t n, int64_t m, int64_t t, int d, int c_in, int k, int num_mlps, int c_out,
                           float *d_weights, float *d_feats, float *d_axis, float *d_bias, float *d_pdf,
                           float *d_pts, float *d_samples,
@@ -246,7 +253,7 @@ int pccnn_conv_forward(const pccnn_basis *basis, const float *pts, const float *
                        float *out, float *proj_out, void *workspace, size_t workspace_bytes, void *stream);
 int pccnn_conv_backward(const pccnn_basis *basis, const float *pts, const float *feats, const float *samples,
                         const int32_t *neigh, const int32_t *ends, const float *radii, const float *weights,
-                        const float *in_grads, const float *proj, int grad_mask,
+                        const float *in_grads, const float *proj, const int32_t *mirror, int grad_mask,
                         int64_t n, int64_t m, int64_t t, int d, int c_in, int num_mlps, int c_out, int divide_by_count,
                         float *d_weights, float *d_feats, float *d_param_a, float *d_param_b, float *d_pdf,
                         float *d_pts, float *d_samples, void *workspace, size_t workspace_bytes, void *stream);

@@ -49,17 +49,18 @@ SIGNATURES = {
     "pccnn_compact_selected": (I32, [P, P, I64, P, P]),
     "pccnn_conv_workspace_bytes": (SZ, [I64, I64, I32, I32, I32, I32]),
     "pccnn_kpconv_forward": (I32, [P, P, P, P, P, P, P, F32, P, I64, I64, I64, I32, I32, I32, I32, P, P, P, SZ, P]),
-    "pccnn_kpconv_backward": (I32, [P, P, P, P, P, P, P, F32, P, P, P, I32, I64, I64, I64, I32, I32, I32, I32,
+    "pccnn_mirror_pairs": (I32, [P, P, I64, I64, P, P, P]),
+    "pccnn_kpconv_backward": (I32, [P, P, P, P, P, P, P, F32, P, P, P, P, I32, I64, I64, I64, I32, I32, I32, I32,
                                     P, P, P, P, P, P, SZ, P]),
     "pccnn_mcconv_forward": (I32, [P, P, P, P, P, P, P, P, P, P, I64, I64, I64, I32, I32, I32, I32, I32,
                                    P, P, P, SZ, P]),
-    "pccnn_mcconv_backward": (I32, [P, P, P, P, P, P, P, P, P, P, P, P, I32, I64, I64, I64, I32, I32, I32, I32, I32,
+    "pccnn_mcconv_backward": (I32, [P, P, P, P, P, P, P, P, P, P, P, P, P, I32, I64, I64, I64, I32, I32, I32, I32, I32,
                                     P, P, P, P, P, P, P, P, SZ, P]),
     "pccnn_conv_weight_var_workspace_bytes": (SZ, [I64, I32, I32]),
     "pccnn_kpconv_weight_var": (I32, [P, P, P, P, P, P, P, F32, I64, I64, I64, I32, I32, I32, P, P, SZ, P]),
     "pccnn_mcconv_weight_var": (I32, [P, P, P, P, P, P, P, P, P, I64, I64, I64, I32, I32, I32, P, P, SZ, P]),
     "pccnn_conv_forward": (I32, [BP, P, P, P, P, P, P, P, I64, I64, I64, I32, I32, I32, I32, I32, P, P, P, SZ, P]),
-    "pccnn_conv_backward": (I32, [BP, P, P, P, P, P, P, P, P, P, I32, I64, I64, I64, I32, I32, I32, I32, I32,
+    "pccnn_conv_backward": (I32, [BP, P, P, P, P, P, P, P, P, P, P, I32, I64, I64, I64, I32, I32, I32, I32, I32,
                                   P, P, P, P, P, P, P, P, SZ, P]),
     "pccnn_conv_weight_var": (I32, [BP, P, P, P, P, P, P, I64, I64, I64, I32, I32, I32, P, P, SZ, P]),
     "pccnn_linear_basis_forward": (I32, [P, P, P, P, P, P, I64, I64, I64, I32, I32, P, P]),

@@ -275,7 +275,8 @@ __device__ __forceinline__ void basis_derivative(const ConvGeom &g, const LaneBa
 // For a basis given by the caller (EXPLICIT) dw is the result and is stored coalesced.  For the parametric
 // bases the kernel goes on while the chunk is still in LDS: KPAD lanes per pair apply the basis derivative
 // (lane = basis index k), shuffles reduce the offset / density gradients over k, and the chunk's values are
-// scattered with float atomics, sixteen pairs x (x, y, z, density) per instruction.  The sample's own gradient
+// scattered with float atomics, sixteen pairs x (x, y, z, density) per instruction - or, when the caller has
+// the mirror index of a symmetric neighborhood, stored per pair for a gather without atomics.  The sample's own gradient
 // and the basis-parameter gradients stay in registers until the end; the latter are added to one of
 // PARAM_ROWS partial rows ([component][k], 256 floats) that the conv_param_reduce kernels sum afterwards.
 #define PARAM_ROWS 256
@@ -284,7 +285,8 @@ template <int BASIS, int KPAD, bool want_df, bool want_db>
 __global__ void __launch_bounds__(64)
 conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *__restrict__ proj_grads,
                      float *__restrict__ feat_grads, float *__restrict__ basis_grads, float *__restrict__ d_pts,
-                     float *__restrict__ d_samples, float *__restrict__ d_pdf, float *__restrict__ param_partials)
+                     float *__restrict__ d_samples, float *__restrict__ d_pdf, float *__restrict__ param_partials,
+                     float *__restrict__ pair_grads)
 {
     constexpr bool FUSED = want_db && BasisTraits<BASIS>::differentiable;   // basis derivative applied here
     __shared__ __attribute__((aligned(16))) float g_lds[FUSED ? 64 : 1][4];
@@ -427,9 +429,12 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
                 const int jn = __shfl(nidx, j);
                 if (j < cnt) {
                     const float v = g_lds[j][comp];
-                    if (comp < 3) {
+                    if (comp < 3) sg += v;
+                    if (pair_grads) {
+                        // per-pair values, summed per point afterwards by conv_point_gather_kernel
+                        pair_grads[(int64_t)(cb + j) * 4 + comp] = v;
+                    } else if (comp < 3) {
                         if (d_pts) unsafeAtomicAdd(&d_pts[(int64_t)jn * 3 + comp], v);
-                        sg += v;
                     } else if (BasisTraits<BASIS>::pdf_grad && d_pdf) {
                         unsafeAtomicAdd(&d_pdf[jn], v);
                     }
@@ -462,6 +467,47 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
                 unsafeAtomicAdd(&row[c * 64 + k], v);
             }
         }
+    }
+}
+
+// Symmetric neighborhoods (samples are the points, uncapped search): pair (a, b) exists iff (b, a) does.
+// mirror[t] of pair t = (point a, sample b) is the index of pair (point b, sample a), found by scanning
+// sample a's segment; -1 and a count in *missing when there is none (the neighborhood is not symmetric).
+__global__ void __launch_bounds__(256)
+mirror_pairs_kernel(const int2 *__restrict__ neigh, const int32_t *__restrict__ ends, int64_t t, int64_t m,
+                    int32_t *__restrict__ mirror, int32_t *__restrict__ missing)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= t) return;
+    const int2 pr = neigh[i];
+    int found = -1;
+    if (pr.x >= 0 && pr.x < m) {
+        const int lo = pr.x > 0 ? ends[pr.x - 1] : 0, hi = ends[pr.x];
+        for (int j = lo; j < hi; ++j)
+            if (neigh[j].x == pr.y) { found = j; break; }
+    }
+    mirror[i] = found;
+    if (found < 0) atomicAdd(missing, 1);
+}
+
+// d_pts[n] and d_pdf[n] of a symmetric neighborhood: the pairs in which n is the point are the mirrors of
+// the pairs of sample n.  Four lanes per point, one per component of the per-pair values.
+__global__ void __launch_bounds__(256)
+conv_point_gather_kernel(const float *__restrict__ pair_grads, const int32_t *__restrict__ mirror,
+                         const int32_t *__restrict__ ends, int64_t m, float *__restrict__ d_pts,
+                         float *__restrict__ d_pdf)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t n = i >> 2;
+    const int comp = (int)(i & 3);
+    if (n >= m) return;
+    const int lo = n > 0 ? ends[n - 1] : 0, hi = ends[n];
+    float acc = 0.0f;
+    for (int j = lo; j < hi; ++j) acc += pair_grads[(int64_t)mirror[j] * 4 + comp];
+    if (comp < 3) {
+        if (d_pts) d_pts[n * 3 + comp] = acc;
+    } else if (d_pdf) {
+        d_pdf[n] = acc;
     }
 }
 
@@ -659,6 +705,7 @@ struct BasisGradOut {
     float *basis_grads;     // [t,k], EXPLICIT only
     float *d_pts, *d_samples, *d_pdf;
     float *partials;        // [PARAM_ROWS][256], zeroed by the caller
+    float *pair_grads;      // [t][4] per-pair (x, y, z, density) values instead of atomics on d_pts / d_pdf
 };
 
 template <int BASIS, int KPAD>
@@ -668,13 +715,15 @@ static void launch_proj_bwd_k(const ConvGeom &g, const float *feats, const float
     dim3 grid((unsigned)g.m);
     if (feat_grads && want_basis)
         conv_proj_bwd_kernel<BASIS, KPAD, true, true><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, o.basis_grads,
-                                                                          o.d_pts, o.d_samples, o.d_pdf, o.partials);
+                                                                          o.d_pts, o.d_samples, o.d_pdf, o.partials,
+                                                                          o.pair_grads);
     else if (feat_grads)
         conv_proj_bwd_kernel<BASIS, KPAD, true, false><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, nullptr,
-                                                                           nullptr, nullptr, nullptr, nullptr);
+                                                                           nullptr, nullptr, nullptr, nullptr, nullptr);
     else
         conv_proj_bwd_kernel<BASIS, KPAD, false, true><<<grid, 64, 0, s>>>(g, feats, proj_grads, nullptr, o.basis_grads,
-                                                                           o.d_pts, o.d_samples, o.d_pdf, o.partials);
+                                                                           o.d_pts, o.d_samples, o.d_pdf, o.partials,
+                                                                           o.pair_grads);
 }
 
 template <int BASIS>
@@ -719,7 +768,8 @@ extern "C" size_t pccnn_conv_workspace_bytes(int64_t m, int64_t t, int c_in, int
     size_t splitk = pccnn_align((size_t)CONV_SPLIT_K * c_in * k * c_out * sizeof(float));
     size_t partials = pccnn_align(((size_t)PARAM_ROWS + PARAM_REDUCE_GROUPS) * 256 * sizeof(float));
     size_t scaled = pccnn_align((size_t)m * c_out * sizeof(float));
-    return 2 * proj + basis_g + splitk + partials + scaled + 256;
+    size_t pair_g = pccnn_align((size_t)t * 4 * sizeof(float));
+    return 2 * proj + basis_g + splitk + partials + scaled + pair_g + 256;
 }
 
 // out[m, c_out] = P[m, c_in*k] x W, with the feature axis split over num_mlps independent
@@ -760,7 +810,8 @@ template <int BASIS>
 static int conv_backward(ConvGeom g, const float *feats, const float *weights, const float *in_grads, int num_mlps,
                          int c_out, const float *proj_in, int mask, float *d_weights, float *d_feats,
                          float *d_param_a, float *d_param_b, float *d_pdf, float *d_pts, float *d_samples,
-                         void *workspace, size_t workspace_bytes, hipStream_t s, bool divide_by_count = false)
+                         void *workspace, size_t workspace_bytes, hipStream_t s, bool divide_by_count = false,
+                         const int32_t *mirror = nullptr)
 {
     // d_param_a: d_kernel_pts [K,3] (kernel-point families), d_axis [3,K] (MLP) or the per-pair basis
     // gradient [T,K] (EXPLICIT); d_param_b: d_bias [K] (MLP only)
@@ -797,6 +848,7 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     size_t splitk_elems = (size_t)CONV_SPLIT_K * g.c_in * g.k * c_out;
     float *splitk = arena.take<float>(splitk_elems);
     float *scaled_grads = arena.take<float>((size_t)g.m * c_out);
+    float *pair_grads = arena.take<float>((size_t)g.t * 4);
     if (BASIS == BASIS_EXPLICIT && want_par) basis_g = d_param_a;    // the basis gradient is itself an output
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv backward: workspace of %zu bytes, need %zu", workspace_bytes,
                   pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 1));
@@ -825,11 +877,17 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     rc = pccnn_gemm_f32(in_grads, weights, d_proj, g.m, inner, co, 0, 1, c_out, co, (int64_t)g.c_in * g.k, num_mlps, co,
                         inner * co, inner, 1, nullptr, 0, s);
     if (rc != PCCNN_OK) return rc;
+    const bool gather = mirror != nullptr && Tr::differentiable && (want_pts || want_pdf);
     BasisGradOut o = {basis_g, want_pts ? d_pts : nullptr, want_pts ? d_samples : nullptr, want_pdf ? d_pdf : nullptr,
-                      (want_par && Tr::differentiable) ? partials : nullptr};
+                      (want_par && Tr::differentiable) ? partials : nullptr, gather ? pair_grads : nullptr};
     if (o.partials && (rc = pccnn_fill_f32(partials, 0.0f, partial_rows * 256, s)) != PCCNN_OK) return rc;
     if ((rc = launch_proj_bwd<BASIS>(g, feats, d_proj, want_f ? d_feats : nullptr, want_basis, o, s)) != PCCNN_OK)
         return rc;
+    if (gather) {
+        conv_point_gather_kernel<<<(unsigned)pccnn_ceil_div(g.m * 4, 256), 256, 0, s>>>(pair_grads, mirror, g.ends, g.m,
+                                                                                        o.d_pts, o.d_pdf);
+        PCCNN_LAUNCH_CHECK();
+    }
     if (o.partials) {
         conv_param_reduce1_kernel<<<PARAM_REDUCE_GROUPS, 256, 0, s>>>(partials, partial_rows, stage);
         PCCNN_LAUNCH_CHECK();
@@ -916,13 +974,16 @@ extern "C" int pccnn_kpconv_forward(const float *pts, const float *feats, const 
 extern "C" int pccnn_kpconv_backward(const float *pts, const float *feats, const float *samples,
                                      const int32_t *neigh, const int32_t *ends, const float *radii,
                                      const float *kernel_pts, float sigma, const float *weights,
-                                     const float *in_grads, const float *proj, int grad_mask, int64_t n, int64_t m,
-                                     int64_t t, int d, int c_in, int k, int c_out, float *d_weights, float *d_feats,
-                                     float *d_kernel_pts, float *d_pts, float *d_samples, void *workspace,
-                                     size_t workspace_bytes, void *stream)
+                                     const float *in_grads, const float *proj, const int32_t *mirror, int grad_mask,
+                                     int64_t n, int64_t m, int64_t t, int d, int c_in, int k, int c_out,
+                                     float *d_weights, float *d_feats, float *d_kernel_pts, float *d_pts,
+                                     float *d_samples, void *workspace, size_t workspace_bytes, void *stream)
 {
     int rc = conv_validate("pccnn_kpconv_backward", n, m, t, d, c_in, k, 1, c_out);
     if (rc != PCCNN_OK) return rc;
+    PCCNN_REQUIRE(mirror == nullptr || n == m, PCCNN_ERR_INVALID,
+                  "pccnn_kpconv_backward: a mirror index needs samples == points (n=%lld, m=%lld)", (long long)n,
+                  (long long)m);
     PCCNN_REQUIRE(sigma > 0.0f, PCCNN_ERR_INVALID, "pccnn_kpconv_backward: sigma=%g", sigma);
     PCCNN_REQUIRE(kernel_pts && weights && radii && (n == 0 || (pts && feats)) &&
                       (m == 0 || (samples && ends && in_grads)) && (t == 0 || neigh),
@@ -934,7 +995,7 @@ extern "C" int pccnn_kpconv_backward(const float *pts, const float *feats, const
     ConvGeom g = {pts, samples, (const int2 *)neigh, ends, radii, nullptr, kernel_pts, nullptr, sigma, n, m, t, c_in, k};
     return conv_backward<BASIS_KP>(g, feats, weights, in_grads, 1, c_out, proj, grad_mask, d_weights, d_feats,
                                    d_kernel_pts, nullptr, nullptr, d_pts, d_samples, workspace, workspace_bytes,
-                                   (hipStream_t)stream);
+                                   (hipStream_t)stream, false, mirror);
 }
 
 extern "C" int pccnn_mcconv_forward(const float *pts, const float *pdf, const float *feats, const float *samples,
@@ -956,13 +1017,17 @@ extern "C" int pccnn_mcconv_forward(const float *pts, const float *pdf, const fl
 extern "C" int pccnn_mcconv_backward(const float *pts, const float *pdf, const float *feats, const float *samples,
                                      const int32_t *neigh, const int32_t *ends, const float *radii,
                                      const float *axis, const float *bias, const float *weights,
-                                     const float *in_grads, const float *proj, int grad_mask, int64_t n, int64_t m,
-                                     int64_t t, int d, int c_in, int k, int num_mlps, int c_out, float *d_weights,
-                                     float *d_feats, float *d_axis, float *d_bias, float *d_pdf, float *d_pts,
-                                     float *d_samples, void *workspace, size_t workspace_bytes, void *stream)
+                                     const float *in_grads, const float *proj, const int32_t *mirror, int grad_mask,
+                                     int64_t n, int64_t m, int64_t t, int d, int c_in, int k, int num_mlps, int c_out,
+                                     float *d_weights, float *d_feats, float *d_axis, float *d_bias, float *d_pdf,
+                                     float *d_pts, float *d_samples, void *workspace, size_t workspace_bytes,
+                                     void *stream)
 {
     int rc = conv_validate("pccnn_mcconv_backward", n, m, t, d, c_in, k, num_mlps, c_out);
     if (rc != PCCNN_OK) return rc;
+    PCCNN_REQUIRE(mirror == nullptr || n == m, PCCNN_ERR_INVALID,
+                  "pccnn_mcconv_backward: a mirror index needs samples == points (n=%lld, m=%lld)", (long long)n,
+                  (long long)m);
     PCCNN_REQUIRE(axis && bias && weights && radii && (n == 0 || (pts && pdf && feats)) &&
                       (m == 0 || (samples && ends && in_grads)) && (t == 0 || neigh),
                   PCCNN_ERR_INVALID, "pccnn_mcconv_backward: null input pointer");
@@ -974,7 +1039,7 @@ extern "C" int pccnn_mcconv_backward(const float *pts, const float *pdf, const f
     ConvGeom g = {pts, samples, (const int2 *)neigh, ends, radii, pdf, axis, bias, 1.0f, n, m, t, c_in, k};
     return conv_backward<BASIS_MLP>(g, feats, weights, in_grads, num_mlps, c_out, proj, grad_mask, d_weights, d_feats,
                                     d_axis, d_bias, d_pdf, d_pts, d_samples, workspace, workspace_bytes,
-                                    (hipStream_t)stream);
+                                    (hipStream_t)stream, false, mirror);
 }
 
 // ------------------------------------------------------------------- generic entry points
@@ -1038,7 +1103,7 @@ extern "C" int pccnn_conv_forward(const pccnn_basis *basis, const float *pts, co
 extern "C" int pccnn_conv_backward(const pccnn_basis *basis, const float *pts, const float *feats,
                                    const float *samples, const int32_t *neigh, const int32_t *ends,
                                    const float *radii, const float *weights, const float *in_grads, const float *proj,
-                                   int grad_mask, int64_t n, int64_t m, int64_t t, int d, int c_in, int num_mlps,
+                                   const int32_t *mirror, int grad_mask, int64_t n, int64_t m, int64_t t, int d, int c_in, int num_mlps,
                                    int c_out, int divide_by_count, float *d_weights, float *d_feats, float *d_param_a,
                                    float *d_param_b, float *d_pdf, float *d_pts, float *d_samples, void *workspace,
                                    size_t workspace_bytes, void *stream)
@@ -1047,6 +1112,9 @@ extern "C" int pccnn_conv_backward(const pccnn_basis *basis, const float *pts, c
     int rc = basis_geom("pccnn_conv_backward", basis, pts, samples, neigh, ends, radii, n, m, t, c_in, g);
     if (rc != PCCNN_OK) return rc;
     if ((rc = conv_validate("pccnn_conv_backward", n, m, t, d, c_in, g.k, num_mlps, c_out)) != PCCNN_OK) return rc;
+    PCCNN_REQUIRE(mirror == nullptr || n == m, PCCNN_ERR_INVALID,
+                  "pccnn_conv_backward: a mirror index needs samples == points (n=%lld, m=%lld)", (long long)n,
+                  (long long)m);
     const int kind = basis->kind;
     const bool geom = kind != PCCNN_BASIS_EXPLICIT;
     PCCNN_REQUIRE(weights && (n == 0 || feats) && (m == 0 || (ends && in_grads)) && (t == 0 || neigh) &&
@@ -1064,7 +1132,7 @@ extern "C" int pccnn_conv_backward(const pccnn_basis *basis, const float *pts, c
                   PCCNN_ERR_INVALID, "pccnn_conv_backward: a requested gradient has a null output pointer");
 #define CALL(B) conv_backward<B>(g, feats, weights, in_grads, num_mlps, c_out, proj, grad_mask, d_weights, d_feats, \
                                  d_param_a, d_param_b, d_pdf, d_pts, d_samples, workspace, workspace_bytes,           \
-                                 (hipStream_t)stream, divide_by_count != 0)
+                                 (hipStream_t)stream, divide_by_count != 0, mirror)
     BASIS_DISPATCH(kind, CALL)
 #undef CALL
 }
@@ -1144,6 +1212,22 @@ extern "C" int pccnn_linear_basis_backward(const float *pts, const float *sample
     conv_param_reduce1_kernel<<<PARAM_REDUCE_GROUPS, 256, 0, s>>>(partials, blocks, stage);
     PCCNN_LAUNCH_CHECK();
     conv_param_reduce2_kernel<BASIS_MLP><<<1, 256, 0, s>>>(stage, k, d_axis, d_bias);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
+extern "C" int pccnn_mirror_pairs(const int32_t *neigh, const int32_t *ends, int64_t t, int64_t m, int32_t *mirror_out,
+                                  int32_t *missing_out, void *stream)
+{
+    PCCNN_REQUIRE(t >= 0 && m >= 0 && t < (1ll << 31) && m < (1ll << 31), PCCNN_ERR_INVALID,
+                  "pccnn_mirror_pairs: t=%lld m=%lld", (long long)t, (long long)m);
+    PCCNN_REQUIRE(missing_out && (t == 0 || (neigh && ends && mirror_out)), PCCNN_ERR_INVALID,
+                  "pccnn_mirror_pairs: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    int rc = pccnn_fill_i32(missing_out, 0, 1, s);
+    if (rc != PCCNN_OK || t == 0) return rc;
+    mirror_pairs_kernel<<<(unsigned)pccnn_ceil_div(t, 256), 256, 0, s>>>((const int2 *)neigh, ends, t, m, mirror_out,
+                                                                         missing_out);
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
 }

@@ -8,16 +8,18 @@ class ComputeKPConvN(torch.autograd.Function):
     KPConv whose correlation is divided by the density of each neighbor.  Gradients go to
     (pts, -, features, samples, -, -, -, kernel_pts, -, conv_weights); the density gets none
     (pccnn_lib/op_wrappers/compute_kpconvn.py:9-74).  The projection of the forward pass is kept for the
-    backward pass and only the gradients autograd asks for are computed."""
+    backward pass and only the gradients autograd asks for are computed.  An optional last argument takes the
+    mirror index of a symmetric neighborhood (pccnn_lib_ops.mirror_pairs), used to sum point gradients without atomics."""
 
     @staticmethod
     def forward(ctx, p_pts, p_pdfs, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_kernel_pts, p_sigma,
-                p_conv_weights):
+                p_conv_weights, p_mirror=None):
         out, proj = pccnn_lib_ops.kp_conv_n(p_pts, p_pdfs, p_features, p_samples, p_neighbors, p_start_ids, p_radii,
                                             p_kernel_pts, p_sigma, p_conv_weights, return_proj=True)
         ctx.save_for_backward(p_pts, p_pdfs, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_kernel_pts,
                               p_conv_weights, proj)
         ctx.sigma_ = p_sigma
+        ctx.mirror_ = p_mirror
         return out
 
     @staticmethod
@@ -29,9 +31,9 @@ class ComputeKPConvN(torch.autograd.Function):
             | (ops.GRAD_BASIS_PARAMS if need[7] else 0) | (ops.GRAD_WEIGHTS if need[9] else 0)
         weight_grads, feat_grads, kernel_pts_grads, pt_grads, sample_grads = ops.kp_conv_n_grads(
             pts, pdfs, features, samples, neighbors, start_ids, radii, kernel_pts, ctx.sigma_, conv_weights, p_grads,
-            proj=proj, grad_mask=mask)
+            proj=proj, grad_mask=mask, mirror=ctx.mirror_)
         return pt_grads if need[0] else None, None, feat_grads, sample_grads if need[3] else None, None, None, \
-            None, kernel_pts_grads, None, weight_grads
+            None, kernel_pts_grads, None, weight_grads, None
 
 
 class ComputeKPConvNWeightVar(torch.autograd.Function):

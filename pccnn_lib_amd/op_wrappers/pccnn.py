@@ -11,12 +11,13 @@ class ComputePCCNN(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, p_pts, p_pt_pdf, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_kernel_pts, p_sigma,
-                p_conv_weights):
+                p_conv_weights, p_mirror=None):
         out, proj = pccnn_lib_ops.pccnn(p_pts, p_features, p_pt_pdf, p_samples, p_neighbors, p_start_ids, p_radii,
                                         p_kernel_pts, p_sigma, p_conv_weights, return_proj=True)
         ctx.save_for_backward(p_pts, p_pt_pdf, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_kernel_pts,
                               p_conv_weights, proj)
         ctx.sigma_ = p_sigma
+        ctx.mirror_ = p_mirror
         return out
 
     @staticmethod
@@ -29,9 +30,9 @@ class ComputePCCNN(torch.autograd.Function):
             | (ops.GRAD_WEIGHTS if need[9] else 0)
         weight_grads, feat_grads, kernel_pts_grads, pt_pdf_grads, pt_grads, sample_grads = ops.pccnn_grads(
             pts, features, pt_pdf, samples, neighbors, start_ids, radii, kernel_pts, ctx.sigma_, conv_weights, p_grads,
-            proj=proj, grad_mask=mask)
+            proj=proj, grad_mask=mask, mirror=ctx.mirror_)
         return pt_grads if need[0] else None, pt_pdf_grads, feat_grads, sample_grads if need[3] else None, None, \
-            None, None, kernel_pts_grads, None, weight_grads
+            None, None, kernel_pts_grads, None, weight_grads, None
 
 
 class ComputePCCNNWeightVar(torch.autograd.Function):

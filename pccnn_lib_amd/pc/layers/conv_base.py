@@ -14,6 +14,15 @@ def build_neighborhood(p_pc_in, p_pc_out, p_radius, p_max_neighs):
     return Neighborhood(grid, p_pc_out, p_max_neighs)
 
 
+def mirror_if_needed(p_neighborhood, *p_geometry):
+    """The neighborhood's mirror index when one of the tensors that receive point-side gradients (positions,
+    densities) requires a gradient; None otherwise, or for a neighborhood object that has none."""
+    if torch.is_grad_enabled() and any(x is not None and x.requires_grad for x in p_geometry) \
+            and hasattr(p_neighborhood, "mirror"):
+        return p_neighborhood.mirror()
+    return None
+
+
 class IConvLayer(torch.nn.Module):
     """Base of the point convolutions (pccnn_lib/pc/layers/IConvLayer.py:8-157):
     ``forward(pc_in, pc_out, in_features, radius, neighborhood=None, max_neighs=0)`` returns the output

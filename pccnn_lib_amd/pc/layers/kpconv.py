@@ -7,7 +7,7 @@ import time
 
 from ...op_wrappers import ComputeKPConv, ComputeKPConvWeightVar, ComputeKPConvN, ComputeKPConvNWeightVar, \
     ComputePCCNN, ComputePCCNNWeightVar
-from .conv_base import IConvLayer, IConvLayerFactory
+from .conv_base import IConvLayer, IConvLayerFactory, mirror_if_needed
 from .kernel_points import kernel_pts_dict
 
 
@@ -70,7 +70,8 @@ class KPConv(IConvLayer):
             self.conv_weights_.data.normal_(0.0, stdv)
         return ComputeKPConv.apply(
             p_pc_in.pts_, p_in_features, p_pc_out.pts_, p_neighborhood.neighbors_, p_neighborhood.start_ids_,
-            p_radius, self.kernel_pts_, self.sigma_cpu_, self.conv_weights_)
+            p_radius, self.kernel_pts_, self.sigma_cpu_, self.conv_weights_,
+            mirror_if_needed(p_neighborhood, p_pc_in.pts_))
 
 
 class KPConvFactory(IConvLayerFactory):
@@ -123,7 +124,8 @@ class _DensityKernelPointConv(IConvLayer):
             self.conv_weights_.data.normal_(0.0, stdv)
         return self.conv_op_.apply(
             p_pc_in.pts_, cur_pdf, p_in_features, p_pc_out.pts_, p_neighborhood.neighbors_, p_neighborhood.start_ids_,
-            p_radius, self.kernel_pts_, self.sigma_cpu_, self.conv_weights_)
+            p_radius, self.kernel_pts_, self.sigma_cpu_, self.conv_weights_,
+            mirror_if_needed(p_neighborhood, p_pc_in.pts_, cur_pdf))
 
 
 class KPConvN(_DensityKernelPointConv):

@@ -3,7 +3,7 @@ import math
 import torch
 
 from ...op_wrappers import ComputeMCConv, ComputeMCConvWeightVar
-from .conv_base import IConvLayer, IConvLayerFactory
+from .conv_base import IConvLayer, IConvLayerFactory, mirror_if_needed
 
 
 class MCConv(IConvLayer):
@@ -43,7 +43,8 @@ class MCConv(IConvLayer):
             self.conv_weights_.data.normal_(0.0, stdv)
         return ComputeMCConv.apply(
             p_pc_in.pts_, cur_pdf, p_in_features, p_pc_out.pts_, p_neighborhood.neighbors_,
-            p_neighborhood.start_ids_, p_radius, self.proj_axis_, self.proj_bias_, self.conv_weights_)
+            p_neighborhood.start_ids_, p_radius, self.proj_axis_, self.proj_bias_, self.conv_weights_,
+            mirror_if_needed(p_neighborhood, p_pc_in.pts_, cur_pdf))
 
 
 class MCConvFactory(IConvLayerFactory):

@@ -15,6 +15,8 @@ class Neighborhood(object):
     def __init__(self, p_grid, p_samples, p_max_neighbors=0):
         self.grid_ = p_grid
         self.samples_ = p_samples
+        self.max_neighbors_ = p_max_neighbors
+        self.mirror_ = False            # not computed yet; None = the neighborhood is not symmetric
         grid = p_grid
         with torch.no_grad():
             sample_pts = p_samples.pts_.detach()
@@ -29,6 +31,16 @@ class Neighborhood(object):
                 grid.sorted_pts_, grid.sorted_cell_ids_, sample_pts, sample_keys, grid.grid_ds_, grid.num_cells_,
                 grid.cell_size_, p_max_neighbors, sample_order=order, point_remap=grid.sorted_ids_i32_,
                 cell_table=grid.cell_table_)
+
+    def mirror(self):
+        """int32 [T]: for every pair (a, b) the index of pair (b, a), when the samples are the gridded cloud
+        itself and the search was not capped (then the pair list is symmetric); else None.  Computed on first
+        use; the convolutions' backward passes use it to sum point gradients without atomics."""
+        if self.mirror_ is False:
+            self.mirror_ = None
+            if self.samples_ is self.grid_.pointcloud_ and self.max_neighbors_ == 0:
+                self.mirror_ = pccnn_lib_ops.mirror_pairs(self.neighbors_, self.start_ids_)
+        return self.mirror_
 
     def __repr__(self):
         return "### Neighbors:\n{}\n### Start indices:\n{}".format(self.neighbors_, self.start_ids_)

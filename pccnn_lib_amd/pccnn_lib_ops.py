@@ -340,11 +340,33 @@ def kp_conv(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights,
     return (out, proj) if return_proj else out
 
 
+def _mirror_arg(name, mirror, neigh, pts, samples):
+    if mirror is None:
+        return _P(0)
+    _chk(mirror, name + ": mirror", torch.int32, 1, neigh.device)
+    if mirror.shape[0] != neigh.shape[0] or pts.shape[0] != samples.shape[0]:
+        raise RuntimeError(name + ": mirror must be [T] and needs samples == points")
+    return _ptr(mirror)
+
+
+def mirror_pairs(neigh, ends):
+    """Mirror index of a symmetric neighborhood (samples are the points, uncapped search): int32 [T] with the
+    index of pair (b, a) for every pair (a, b), or None when some pair has no mirror.  Reads one int back."""
+    _chk(neigh, "mirror_pairs: neighbors", torch.int32, 2)
+    _chk(ends, "mirror_pairs: start_ids", torch.int32, 1, neigh.device)
+    mirror = torch.empty((neigh.shape[0],), dtype=torch.int32, device=neigh.device)
+    missing = torch.empty((1,), dtype=torch.int32, device=neigh.device)
+    _lib.call("pccnn_mirror_pairs", _ptr(neigh), _ptr(ends), neigh.shape[0], ends.shape[0], _ptr(mirror),
+              _ptr(missing), _stream())
+    return mirror if int(missing.item()) == 0 else None
+
+
 def kp_conv_grads(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights, in_grads, proj=None,
-                  grad_mask=GRAD_ALL):
+                  grad_mask=GRAD_ALL, mirror=None):
     """kp_conv_grads(..., in_grads f32[M,Cout]) -> [dW, dFeat, dKernelPts, dPts, dSamples]
     (pccnn_lib_ops/pcconvs/kpconv.cuh:56-67).  ``proj``: projection kept from kp_conv(return_proj=True);
-    ``grad_mask``: GRAD_* groups to compute, the others come back as None."""
+    ``grad_mask``: GRAD_* groups to compute, the others come back as None; ``mirror``: result of mirror_pairs()
+    for a symmetric neighborhood, which lets dPts (and dPdf) be summed per point without atomics."""
     name = "kp_conv_grads"
     d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
     _chk(kernel_pts, name + ": kernel_pts", torch.float32, 2, dev)
@@ -361,7 +383,8 @@ def kp_conv_grads(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, we
     proj_p = _conv_proj_arg(name, proj, m, c_in, k, dev)
     ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
     _lib.call("pccnn_kpconv_backward", _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends), _ptr(radii),
-              _ptr(kernel_pts), float(sigma), _ptr(weights), _ptr(in_grads), proj_p, grad_mask, n, m, t, d, c_in, k,
+              _ptr(kernel_pts), float(sigma), _ptr(weights), _ptr(in_grads), proj_p,
+              _mirror_arg(name, mirror, neigh, pts, samples), grad_mask, n, m, t, d, c_in, k,
               c_out, _optr(d_w), _optr(d_f), _optr(d_kp), _optr(d_p), _optr(d_s), _ptr(ws), ws.numel(), _stream())
     return [d_w, d_f, d_kp, d_p, d_s]
 
@@ -409,9 +432,9 @@ def mc_conv(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights, r
 
 
 def mc_conv_grads(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights, in_grads, proj=None,
-                  grad_mask=GRAD_ALL):
+                  grad_mask=GRAD_ALL, mirror=None):
     """mc_conv_grads(..., in_grads f32[M,Cout]) -> [dW, dFeat, dAxis, dBias f32[1,H*m], dPdf f32[N], dPts, dSamples]
-    (pccnn_lib_ops/pcconvs/mcconv.cuh:57-69).  ``proj`` / ``grad_mask`` as in kp_conv_grads."""
+    (pccnn_lib_ops/pcconvs/mcconv.cuh:57-69).  ``proj`` / ``grad_mask`` / ``mirror`` as in kp_conv_grads."""
     name = "mc_conv_grads"
     d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
     n, m, t, c_in = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1]
@@ -427,8 +450,8 @@ def mc_conv_grads(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weig
     proj_p = _conv_proj_arg(name, proj, m, c_in, k, dev)
     ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
     _lib.call("pccnn_mcconv_backward", _ptr(pts), _ptr(pdf), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends),
-              _ptr(radii), _ptr(axis), _ptr(bias), _ptr(weights), _ptr(in_grads), proj_p, grad_mask, n, m, t, d, c_in, k,
-              num_mlps, c_out, _optr(d_w), _optr(d_f), _optr(d_axis), _optr(d_bias), _optr(d_pdf), _optr(d_p),
+              _ptr(radii), _ptr(axis), _ptr(bias), _ptr(weights), _ptr(in_grads), proj_p,
+              _mirror_arg(name, mirror, neigh, pts, samples), grad_mask, n, m, t, d, c_in, k, num_mlps, c_out, _optr(d_w), _optr(d_f), _optr(d_axis), _optr(d_bias), _optr(d_pdf), _optr(d_p),
               _optr(d_s), _ptr(ws), ws.numel(), _stream())
     return [d_w, d_f, d_axis, d_bias, d_pdf, d_p, d_s]
 
@@ -497,7 +520,7 @@ def _generic_forward(name, desc, k, pts, feats, samples, neigh, ends, radii, wei
 
 
 def _generic_backward(name, desc, k, pts, feats, samples, neigh, ends, radii, weights, in_grads, proj, grad_mask,
-                      divide_by_count, d_param_a=None, d_pdf=None, with_pts=True):
+                      divide_by_count, d_param_a=None, d_pdf=None, with_pts=True, mirror=None):
     dev = feats.device
     _chk(weights, name + ": weights", torch.float32, 2, dev)
     in_grads = _chk(in_grads.contiguous(), name + ": in_grads", torch.float32, 2, dev)
@@ -512,7 +535,8 @@ def _generic_backward(name, desc, k, pts, feats, samples, neigh, ends, radii, we
     proj_p = _conv_proj_arg(name, proj, m, c_in, k, dev)
     ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
     _lib.call("pccnn_conv_backward", ctypes.byref(desc), _optr(pts), _ptr(feats), _optr(samples), _ptr(neigh),
-              _ptr(ends), _optr(radii), _ptr(weights), _ptr(in_grads), proj_p, grad_mask, n, m, t, 3, c_in, 1, c_out,
+              _ptr(ends), _optr(radii), _ptr(weights), _ptr(in_grads), proj_p,
+              _mirror_arg(name, mirror, neigh, pts, samples) if with_pts else _P(0), grad_mask, n, m, t, 3, c_in, 1, c_out,
               int(divide_by_count), _optr(d_w), _optr(d_f), _optr(d_param_a), _P(0), _optr(d_pdf), _optr(d_p),
               _optr(d_s), _ptr(ws), ws.numel(), _stream())
     return d_w, d_f, d_p, d_s
@@ -549,7 +573,7 @@ def kp_conv_n(pts, pdf, feats, samples, neigh, ends, radii, kernel_pts, sigma, w
 
 
 def kp_conv_n_grads(pts, pdf, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights, in_grads, proj=None,
-                    grad_mask=GRAD_ALL):
+                    grad_mask=GRAD_ALL, mirror=None):
     """kp_conv_n_grads(..., in_grads) -> [dW, dFeat, dKernelPts, dPts, dSamples]; the density gets no gradient
     (pccnn_lib_ops/pcconvs/kpconvn.cuh:57-68)."""
     name = "kp_conv_n_grads"
@@ -557,7 +581,7 @@ def kp_conv_n_grads(pts, pdf, feats, samples, neigh, ends, radii, kernel_pts, si
     desc = _basis(BASIS_KPN, k, kernel_pts, sigma=sigma, pdf=pdf)
     d_kp = torch.empty_like(kernel_pts) if int(grad_mask) & GRAD_BASIS_PARAMS else None
     d_w, d_f, d_p, d_s = _generic_backward(name, desc, k, pts, feats, samples, neigh, ends, radii, weights, in_grads,
-                                           proj, grad_mask, False, d_param_a=d_kp)
+                                           proj, grad_mask, False, d_param_a=d_kp, mirror=mirror)
     return [d_w, d_f, d_kp, d_p, d_s]
 
 
@@ -580,7 +604,7 @@ def pccnn(pts, feats, pdf, samples, neigh, ends, radii, kernel_pts, sigma, weigh
 
 
 def pccnn_grads(pts, feats, pdf, samples, neigh, ends, radii, kernel_pts, sigma, weights, in_grads, proj=None,
-                grad_mask=GRAD_ALL):
+                grad_mask=GRAD_ALL, mirror=None):
     """pccnn_grads(..., in_grads) -> [dW, dFeat, dKernelPts, dPdf, dPts, dSamples]
     (pccnn_lib_ops/pcconvs/pccnn.cuh:57-68)."""
     name = "pccnn_grads"
@@ -589,7 +613,7 @@ def pccnn_grads(pts, feats, pdf, samples, neigh, ends, radii, kernel_pts, sigma,
     d_kp = torch.empty_like(kernel_pts) if int(grad_mask) & GRAD_BASIS_PARAMS else None
     d_pdf = torch.empty_like(pdf) if int(grad_mask) & GRAD_PDF else None
     d_w, d_f, d_p, d_s = _generic_backward(name, desc, k, pts, feats, samples, neigh, ends, radii, weights, in_grads,
-                                           proj, grad_mask, False, d_param_a=d_kp, d_pdf=d_pdf)
+                                           proj, grad_mask, False, d_param_a=d_kp, d_pdf=d_pdf, mirror=mirror)
     return [d_w, d_f, d_kp, d_pdf, d_p, d_s]
 
 

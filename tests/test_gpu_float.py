@@ -316,3 +316,68 @@ def test_error_paths(ops):
     with pytest.raises(RuntimeError, match="k=65"):
         ops.kp_conv(tp, feats, tp, nb["neigh"], nb["ends"], nb["radii"], torch.zeros((65, 3), device=DEV), 0.3,
                     torch.zeros((65 * 4, 2), device=DEV))
+
+
+def test_mirror_index_and_atomic_free_point_gradients(ops, oracle):
+    # samples == points, uncapped search: the pair list is symmetric, its mirror index exists, and the backward
+    # pass that gathers per point with it gives the gradients of the atomic path and of the oracle
+    pts, ids, smp, nb, rng = _conv_case(oracle, ops, 77, 2, 1500, 0.12, False)
+    d = nb["dev"]
+    neigh, ends, radii = nb["neighbors"], nb["ends"], nb["radii"]
+    mirror = ops.mirror_pairs(d["neigh"], d["ends"])
+    assert mirror is not None
+    mi = mirror.cpu().numpy()
+    assert np.array_equal(mi[mi], np.arange(mi.shape[0]))
+    assert np.array_equal(neigh[mi], neigh[:, ::-1])
+    k, c_in, c_out = 16, 32, 24
+    pdf = rng.uniform(0.5, 2.0, pts.shape[0]).astype(np.float32)
+    feats = rng.normal(size=(pts.shape[0], c_in)).astype(np.float32)
+    g = rng.normal(size=(pts.shape[0], c_out)).astype(np.float32)
+    axis = rng.normal(0, np.sqrt(1 / 3), (3, k)).astype(np.float32)
+    bias = rng.normal(0, 0.1, (1, k)).astype(np.float32)
+    w = rng.normal(0, np.sqrt(1.0 / (c_in * k)), (1, k * c_in, c_out)).astype(np.float32)
+    args = (d["pts"], t(pdf), t(feats), d["samples"], d["neigh"], d["ends"], d["radii"], t(axis), t(bias), t(w), t(g))
+    atomic = ops.mc_conv_grads(*args)
+    gathered = ops.mc_conv_grads(*args, mirror=mirror)
+    exp = oracle.mcconv_grads(pts, pdf, feats, pts, neigh, ends, radii, axis, bias, w, g)
+    for a, b, e, name in zip(atomic, gathered, exp, ("dW", "dFeat", "dAxis", "dBias", "dPdf", "dPts", "dSamples")):
+        assert relerr(b.cpu().numpy(), e) < GRAD_TOL, name
+        assert relerr(b.cpu().numpy(), a.cpu().numpy()) < GRAD_TOL, name
+    # the gather sums in a fixed order: two runs agree bit for bit
+    again = ops.mc_conv_grads(*args, mirror=mirror)
+    assert torch.equal(again[5], gathered[5]) and torch.equal(again[4], gathered[4])
+    kp, sigma = synthetic.kernel_points_sphere(1, 15)
+    wk = rng.normal(0, 0.1, (15 * c_in, c_out)).astype(np.float32)
+    kargs = (d["pts"], t(feats), d["samples"], d["neigh"], d["ends"], d["radii"], t(kp), sigma, t(wk), t(g))
+    got = ops.kp_conv_grads(*kargs, mirror=mirror)
+    exp = oracle.kpconv_grads(pts, feats, pts, neigh, ends, radii, kp, sigma, wk, g)
+    for b, e, name in zip(got, exp, ("dW", "dFeat", "dKernelPts", "dPts", "dSamples")):
+        assert relerr(b.cpu().numpy(), e) < GRAD_TOL, name
+    # a subset of the points as samples is not symmetric: no mirror index, and passing one is refused
+    _, _, smp2, nb2, _ = _conv_case(oracle, ops, 78, 2, 900, 0.12, True)
+    d2 = nb2["dev"]
+    assert ops.mirror_pairs(d2["neigh"], d2["ends"]) is None
+    with pytest.raises(RuntimeError, match="mirror"):
+        ops.kp_conv_grads(d2["pts"], torch.zeros((d2["pts"].shape[0], c_in), device=DEV), d2["samples"], d2["neigh"],
+                          d2["ends"], d2["radii"], t(kp), sigma, t(wk),
+                          torch.zeros((d2["samples"].shape[0], c_out), device=DEV),
+                          mirror=torch.zeros(d2["neigh"].shape[0], dtype=torch.int32, device=DEV))
+
+
+def test_layer_uses_mirror_for_point_gradients(oracle):
+    import pccnn_lib_amd as lib
+    pts, ids = synthetic.primitives(21, 2, 1000)
+    rng = np.random.default_rng(21)
+    feats = rng.normal(size=(pts.shape[0], 8)).astype(np.float32)
+    torch.manual_seed(7)
+    layer = lib.pc.layers.KPConv(3, 8, 12, 15).to(DEV)
+    tp = t(pts).requires_grad_(True)
+    pc = lib.pc.Pointcloud(tp, ids, device=DEV)
+    out, nbh = layer(pc, pc, t(feats), 0.1)
+    assert nbh.mirror_ is not False and nbh.mirror_ is not None          # computed because the points need gradients
+    g = rng.normal(size=tuple(out.shape)).astype(np.float32)
+    out.backward(t(g))
+    exp = oracle.kpconv_grads(pts, feats, pts, nbh.neighbors_.cpu().numpy(), nbh.start_ids_.cpu().numpy(),
+                              np.full(3, 0.1, np.float32), layer.kernel_pts_.cpu().numpy(), float(layer.sigma_.item()),
+                              layer.conv_weights_.detach().cpu().numpy(), g)
+    assert relerr(tp.grad.cpu().numpy(), exp[3] + exp[4]) < GRAD_TOL
