@@ -175,15 +175,21 @@ def main():
         return p
 
     def timed(fn, steps, warmup):
+        """(ms per step, per-kernel timings).  The step time comes from a pass without the library's event
+        hooks (they serialise the stream around every hooked launch); a second pass of the same steps with
+        the hooks on gives the per-kernel durations."""
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
-        _lib.timing(enable=True, reset=True)
         t0 = time.perf_counter()
         for _ in range(steps):
             fn()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
+        _lib.timing(enable=True, reset=True)
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
         kernels = _lib.timing(enable=False)
         return dt / steps * 1e3, kernels
 

@@ -289,13 +289,14 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
                      float *__restrict__ pair_grads)
 {
     constexpr bool FUSED = want_db && BasisTraits<BASIS>::differentiable;   // basis derivative applied here
-    __shared__ __attribute__((aligned(16))) float g_lds[FUSED ? 64 : 1][4];
+    constexpr int CH = 32;                                          // pairs staged in LDS at a time
+    __shared__ __attribute__((aligned(16))) float g_lds[FUSED ? CH : 1][4];
     // want_df / want_db: which of the two stages this instantiation runs
     constexpr int PARTS = 64 / KPAD;                                // feature groups of the dw stage
     constexpr int ROWS = 4;                                         // feature rows in flight
-    __shared__ __attribute__((aligned(16))) float w_lds[64][KPAD];
-    __shared__ __attribute__((aligned(16))) float db_lds[64][KPAD];
-    __shared__ __attribute__((aligned(16))) float row_lds[ROWS][64];
+    __shared__ __attribute__((aligned(16))) float w_lds[CH][KPAD];
+    __shared__ __attribute__((aligned(16))) float db_lds[want_db ? CH : 1][KPAD];
+    __shared__ __attribute__((aligned(16))) float row_lds[want_db ? ROWS : 1][64];
     const int lane = threadIdx.x;
     const int64_t s = blockIdx.x;
     const int k = lane % KPAD, part = lane / KPAD;
@@ -313,8 +314,8 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
     float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;       // parameter gradients of this lane's k (FUSED)
     float sg = 0.f;                                     // component (lane & 3) of the sample's gradient, unsigned
 
-    for (int cb = lo; cb < hi; cb += 64) {
-        const int cnt = (hi - cb) < 64 ? (hi - cb) : 64;
+    for (int cb = lo; cb < hi; cb += CH) {
+        const int cnt = (hi - cb) < CH ? (hi - cb) : CH;
         int nidx = 0;
         float dx = 0.f, dy = 0.f, dz = 0.f, pd = 1.0f;
         if (lane < cnt) {
@@ -333,8 +334,10 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
             // would hand zeros to the lanes reading from it
             const float jx = __shfl(dx, j), jy = __shfl(dy, j), jz = __shfl(dz, j), jp = __shfl(pd, j);
             const float w = (j < cnt) ? pair_basis<BASIS>(g, lb, (int64_t)cb + j, jx, jy, jz, jp) : 0.0f;
-            w_lds[j][k] = w;
-            db_lds[j][k] = 0.0f;
+            if (j < CH) {
+                w_lds[j][k] = w;
+                if (want_db) db_lds[j][k] = 0.0f;
+            }
         }
         __syncthreads();
         for (int fb = 0; fb < fblocks; ++fb) {
@@ -375,8 +378,8 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
                 if (want_db) {
 #pragma unroll
                     for (int u = 0; u < ROWS; ++u) row_lds[u][lane] = row[u];
+                    __syncthreads();
                 }
-                __syncthreads();
 #pragma unroll
                 for (int u = 0; u < ROWS; ++u) {
                     const int j = j0 + u;
@@ -403,7 +406,7 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
                         }
                     }
                 }
-                __syncthreads();
+                if (want_db) __syncthreads();
             }
         }
         __syncthreads();
@@ -421,7 +424,7 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
                     gz += __shfl_xor(gz, o);
                     if (BasisTraits<BASIS>::pdf_grad) gpdf += __shfl_xor(gpdf, o);
                 }
-                if (k < 4) g_lds[j][k] = (k == 0) ? gx * ir0 : (k == 1) ? gy * ir1 : (k == 2) ? gz * ir2 : gpdf;
+                if (k < 4 && j < CH) g_lds[j][k] = (k == 0) ? gx * ir0 : (k == 1) ? gy * ir1 : (k == 2) ? gz * ir2 : gpdf;
             }
             __syncthreads();
             for (int i = 0; i * 16 < cnt; ++i) {
@@ -831,8 +834,10 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv backward: workspace of %zu bytes, need %zu", workspace_bytes,
                   pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 1));
     if (want_f && (rc = pccnn_fill_f32(d_feats, 0.0f, g.n * g.c_in, s)) != PCCNN_OK) return rc;
-    if (want_pts && (rc = pccnn_fill_f32(d_pts, 0.0f, g.n * 3, s)) != PCCNN_OK) return rc;
-    if (want_pdf && (rc = pccnn_fill_f32(d_pdf, 0.0f, g.n, s)) != PCCNN_OK) return rc;
+    // with a mirror index the point-side gradients are written once per point, not accumulated
+    const bool gather = mirror != nullptr && Tr::differentiable && (want_pts || want_pdf) && g.m > 0 && g.t > 0;
+    if (want_pts && !gather && (rc = pccnn_fill_f32(d_pts, 0.0f, g.n * 3, s)) != PCCNN_OK) return rc;
+    if (want_pdf && !gather && (rc = pccnn_fill_f32(d_pdf, 0.0f, g.n, s)) != PCCNN_OK) return rc;
     if (g.m == 0 || g.t == 0) {
         if (want_pts && (rc = pccnn_fill_f32(d_samples, 0.0f, g.m * 3, s)) != PCCNN_OK) return rc;
         if (want_par && (rc = pccnn_fill_f32(d_param_a, 0.0f, count_a, s)) != PCCNN_OK) return rc;
@@ -877,7 +882,6 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     rc = pccnn_gemm_f32(in_grads, weights, d_proj, g.m, inner, co, 0, 1, c_out, co, (int64_t)g.c_in * g.k, num_mlps, co,
                         inner * co, inner, 1, nullptr, 0, s);
     if (rc != PCCNN_OK) return rc;
-    const bool gather = mirror != nullptr && Tr::differentiable && (want_pts || want_pdf);
     BasisGradOut o = {basis_g, want_pts ? d_pts : nullptr, want_pts ? d_samples : nullptr, want_pdf ? d_pdf : nullptr,
                       (want_par && Tr::differentiable) ? partials : nullptr, gather ? pair_grads : nullptr};
     if (o.partials && (rc = pccnn_fill_f32(partials, 0.0f, partial_rows * 256, s)) != PCCNN_OK) return rc;

@@ -34,13 +34,13 @@ struct GemmArgs {
 // `FAST`: the tile is fully inside the matrix and 16-byte aligned, so it is read with float4 loads.
 template <bool KCONTIG, bool FAST, int TILE_X>
 __device__ __forceinline__ void tile_load(const float *__restrict__ p, int64_t ld, int64_t x0, int64_t x_end,
-                                          int64_t k0, int64_t k_end, float4 (&r)[TILE_X / 64])
+                                          int64_t k0, int64_t k_end, float4 (&r)[TILE_X / 64 * (GT_K / 16)])
 {
 #pragma unroll
-    for (int i = 0; i < TILE_X / 64; ++i) {
+    for (int i = 0; i < TILE_X / 64 * (GT_K / 16); ++i) {
         const int idx = threadIdx.x + 256 * i;
         int64_t x, k;
-        if (KCONTIG) { x = x0 + idx / 4; k = k0 + (idx % 4) * 4; }
+        if (KCONTIG) { x = x0 + idx / (GT_K / 4); k = k0 + (idx % (GT_K / 4)) * 4; }
         else { k = k0 + idx / (TILE_X / 4); x = x0 + (idx % (TILE_X / 4)) * 4; }
         if (FAST) {
             r[i] = KCONTIG ? *(const float4 *)(p + x * ld + k) : *(const float4 *)(p + k * ld + x);
@@ -58,13 +58,13 @@ __device__ __forceinline__ void tile_load(const float *__restrict__ p, int64_t l
 }
 
 template <bool KCONTIG, int TILE_X>
-__device__ __forceinline__ void tile_store(float (*lds)[GT_LD], const float4 (&r)[TILE_X / 64])
+__device__ __forceinline__ void tile_store(float (*lds)[GT_LD], const float4 (&r)[TILE_X / 64 * (GT_K / 16)])
 {
 #pragma unroll
-    for (int i = 0; i < TILE_X / 64; ++i) {
+    for (int i = 0; i < TILE_X / 64 * (GT_K / 16); ++i) {
         const int idx = threadIdx.x + 256 * i;
         if (KCONTIG) {
-            const int x = idx / 4, k = (idx % 4) * 4;
+            const int x = idx / (GT_K / 4), k = (idx % (GT_K / 4)) * 4;
             lds[k + 0][x] = r[i].x;
             lds[k + 1][x] = r[i].y;
             lds[k + 2][x] = r[i].z;
@@ -77,9 +77,9 @@ __device__ __forceinline__ void tile_store(float (*lds)[GT_LD], const float4 (&r
     }
 }
 
-// The k loop of one workgroup tile.  Global loads of tile kt+1 are issued before the MFMAs of tile kt and
-// parked in LDS after them; inside a tile the LDS fragments of sub-step ks+1 are read before the MFMAs of
-// sub-step ks are issued, so the matrix pipe never waits on an LDS round trip.
+// The k loop of one workgroup tile.  Global loads run two tiles ahead of the MFMAs (registers, then the free
+// LDS buffer); inside a tile the LDS fragments of sub-step ks+1 are read before the MFMAs of sub-step ks are
+// issued, so the matrix pipe never waits on an LDS round trip.
 template <bool AT, bool BT, bool FAST, int BM>
 __device__ __forceinline__ void gemm_tile_loop(const GemmArgs &g, const float *__restrict__ a,
                                                const float *__restrict__ b, int64_t bm, int64_t bn, int64_t k_begin,
@@ -92,25 +92,26 @@ __device__ __forceinline__ void gemm_tile_loop(const GemmArgs &g, const float *_
     const int wave = threadIdx.x >> 6;
     const int wm = wave / WN, wn = wave % WN;
     const int frag_k = lane >> 5, frag_c = lane & 31;
-    float4 ra[BM / 64], rb[2];
+    float4 ra[BM / 64 * (GT_K / 16)], rb[2 * (GT_K / 16)];
     const int64_t nk = (k_end - k_begin + GT_K - 1) / GT_K;
+    // A stored [rows, inner] (AT = false) has the reduction index contiguous; B stored
+    // [inner, cols] (BT = false) has the column index contiguous.
     if (nk > 0) {
-        // A stored [rows, inner] (AT = false) has the reduction index contiguous; B stored
-        // [inner, cols] (BT = false) has the column index contiguous.
         tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k_begin, k_end, ra);
         tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k_begin, k_end, rb);
         tile_store<!AT, BM>(As[0], ra);
         tile_store<BT, GT_N>(Bs[0], rb);
     }
+    if (nk > 1) {
+        tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k_begin + GT_K, k_end, ra);
+        tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k_begin + GT_K, k_end, rb);
+    }
     __syncthreads();
     for (int64_t kt = 0; kt < nk; ++kt) {
         const int buf = (int)(kt & 1);
-        const bool more = kt + 1 < nk;
-        if (more) {
-            const int64_t k0 = k_begin + (kt + 1) * GT_K;
-            tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k0, k_end, ra);
-            tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k0, k_end, rb);
-        }
+        // Tile kt+1 sits in registers since the previous step: it is parked in the other LDS buffer (free
+        // since the barrier that ended step kt-1) and the registers are reused for the loads of tile kt+2,
+        // which get a whole step of MFMAs to arrive.
         float fa[2][2], fb[2][TN];
 #pragma unroll
         for (int i = 0; i < 2; ++i) fa[0][i] = As[buf][frag_k][wm * 64 + i * 32 + frag_c];
@@ -131,10 +132,18 @@ __device__ __forceinline__ void gemm_tile_loop(const GemmArgs &g, const float *_
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
-        }
-        if (more) {
-            tile_store<!AT, BM>(As[buf ^ 1], ra);
-            tile_store<BT, GT_N>(Bs[buf ^ 1], rb);
+            if (ks == 0) {
+                // behind the first MFMAs of the step, so the matrix pipe is busy while this wave moves data
+                if (kt + 1 < nk) {
+                    tile_store<!AT, BM>(As[buf ^ 1], ra);
+                    tile_store<BT, GT_N>(Bs[buf ^ 1], rb);
+                }
+                if (kt + 2 < nk) {
+                    const int64_t k0 = k_begin + (kt + 2) * GT_K;
+                    tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k0, k_end, ra);
+                    tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k0, k_end, rb);
+                }
+            }
         }
         __syncthreads();
     }
