@@ -315,6 +315,11 @@ int pccnn_timing_count(void);
 const char *pccnn_timing_name(int id);
 int pccnn_timing_read(int id, int64_t *h_launches, double *h_total_ms);
 
+/* Measurement helper with no counterpart in the reference: copies `count` floats (a multiple of 4, 16-byte
+ * aligned pointers) with plain loads and stores.  A profiler's memory-traffic counters read for this kernel,
+ * whose traffic is known (4*count bytes each way), give the scale for the same counters on the other kernels. */
+int pccnn_calibration_copy(const float *src, float *dst, int64_t count, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -27,7 +27,16 @@ struct GemmArgs {
     int split_k;
     int64_t k_chunk;       // inner elements per split (multiple of GT_K)
     int aligned;           // pointers, leading dimensions and batch strides allow float4 loads
+    int tiles_x, tiles_y;  // workgroup tiles along the columns / rows
+    int64_t total_wg;      // tiles_x * tiles_y * batch * split_k
 };
+
+// Workgroups are handed to the 8 XCDs round-robin by their linear id, and each XCD has its own L2.  The
+// launch is one-dimensional and padded to a multiple of 8; workgroup i works on logical tile
+// (i % 8) * (padded / 8) + i / 8, so every XCD owns one contiguous run of logical tiles.  Logical tiles are
+// ordered column tile fastest, then row tile, then batch / split: neighbours in that order share their A
+// row tile (or, with one column tile, their B chunk), which is then fetched from HBM by one XCD, once.
+#define GEMM_XCDS 8
 
 // Global -> registers for one 128 x 16 operand tile.  `KCONTIG`: the reduction index is the
 // contiguous one in memory (element (x, k) at p[x * ld + k]); otherwise element (x, k) at p[k * ld + x].
@@ -161,10 +170,16 @@ gemm_f32_mfma_kernel(GemmArgs g, float *__restrict__ partial)
     const int lane = pccnn_lane();
     const int wave = threadIdx.x >> 6;
     const int wm = wave / WN, wn = wave % WN;
-    const int batch = blockIdx.z / g.split_k;
-    const int split = blockIdx.z % g.split_k;
-    const int64_t bm = (int64_t)blockIdx.y * BM;
-    const int64_t bn = (int64_t)blockIdx.x * GT_N;
+    const int64_t per_xcd = (int64_t)gridDim.x / GEMM_XCDS;
+    const int64_t tile = (int64_t)(blockIdx.x % GEMM_XCDS) * per_xcd + blockIdx.x / GEMM_XCDS;
+    if (tile >= g.total_wg) return;                                 // padding of the launch
+    const int tx = (int)(tile % g.tiles_x);
+    const int ty = (int)((tile / g.tiles_x) % g.tiles_y);
+    const int tz = (int)(tile / ((int64_t)g.tiles_x * g.tiles_y));
+    const int batch = tz / g.split_k;
+    const int split = tz % g.split_k;
+    const int64_t bm = (int64_t)ty * BM;
+    const int64_t bn = (int64_t)tx * GT_N;
     const float *a = g.a + (int64_t)batch * g.stride_a;
     const float *b = g.b + (int64_t)batch * g.stride_b;
     const int64_t k_begin = (int64_t)split * g.k_chunk;
@@ -257,9 +272,11 @@ extern "C" int pccnn_gemm_f32(const float *a, const float *b, float *c, int64_t 
     const int64_t wg128 = pccnn_ceil_div(cols, GT_N) * pccnn_ceil_div(rows, 128) * batch * split_k;
     const char *force = getenv("PCCNN_GEMM_BM");
     const int bm_tile = force ? atoi(force) : (wg128 >= 1024 ? 128 : 64);
-    dim3 grid((unsigned)pccnn_ceil_div(cols, GT_N), (unsigned)pccnn_ceil_div(rows, bm_tile), (unsigned)(batch * split_k));
-    PCCNN_REQUIRE(grid.y <= 65535u && grid.z <= 65535u, PCCNN_ERR_UNSUPPORTED,
-                  "pccnn_gemm_f32: grid too large");
+    g.tiles_x = (int)pccnn_ceil_div(cols, GT_N);
+    g.tiles_y = (int)pccnn_ceil_div(rows, bm_tile);
+    g.total_wg = (int64_t)g.tiles_x * g.tiles_y * batch * split_k;
+    PCCNN_REQUIRE(g.total_wg < (1ll << 31) - GEMM_XCDS, PCCNN_ERR_UNSUPPORTED, "pccnn_gemm_f32: grid too large");
+    dim3 grid((unsigned)(pccnn_ceil_div(g.total_wg, GEMM_XCDS) * GEMM_XCDS));
     {
         PccnnTimed timed(PCCNN_T_GEMM, s);
 #define GEMM_GO(AT, BT)                                                                       \

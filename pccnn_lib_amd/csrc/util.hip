@@ -114,6 +114,29 @@ template <typename T> static int fill_impl(T *p, T v, int64_t n, hipStream_t s)
 int pccnn_fill_i32(int32_t *p, int32_t v, int64_t n, hipStream_t s) { return fill_impl<int32_t>(p, v, n, s); }
 int pccnn_fill_f32(float *p, float v, int64_t n, hipStream_t s) { return fill_impl<float>(p, v, n, s); }
 
+// A plain float4 copy: the known-size yardstick that hardware traffic counters are scaled against.
+__global__ void __launch_bounds__(256) calibration_copy_kernel(const float4 *__restrict__ src,
+                                                               float4 *__restrict__ dst, int64_t n4)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n4; i += stride) dst[i] = src[i];
+}
+
+extern "C" int pccnn_calibration_copy(const float *src, float *dst, int64_t count, void *stream)
+{
+    PCCNN_REQUIRE(count >= 0 && count % 4 == 0, PCCNN_ERR_INVALID, "pccnn_calibration_copy: count=%lld must be a multiple of 4",
+                  (long long)count);
+    if (count == 0) return PCCNN_OK;
+    PCCNN_REQUIRE(src && dst && (uintptr_t)src % 16 == 0 && (uintptr_t)dst % 16 == 0, PCCNN_ERR_INVALID,
+                  "pccnn_calibration_copy: null or unaligned pointer");
+    int64_t blocks = pccnn_ceil_div(count / 4, 256);
+    if (blocks > 16384) blocks = 16384;
+    calibration_copy_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const float4 *)src, (float4 *)dst, count / 4);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
 // ------------------------------------------------------------------- scan
 // Three launches: per-tile inclusive scan + tile totals, scan of the totals by one
 // workgroup, add of the tile prefix.  Tiles are SCAN_TILE consecutive elements.
