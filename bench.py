@@ -35,10 +35,12 @@ sys.path.insert(0, ROOT)
 MFMA_FP32_PEAK_TFLOPS = 157.3     # MI355X dense fp32 matrix peak
 HBM_PEAK_GBPS = 8000.0            # MI355X HBM3E peak
 
-# HBM bytes per launch of the dominant kernels, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# command (see profiles/); None until measured for the current kernels.
-TRAFFIC_GEMM_BYTES = None
-TRAFFIC_NB_FILL_BYTES = None
+# Bytes per launch that the dominant kernels move past the L2, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# of this command scaled by a copy kernel of known size (profiles/bench_mcconv_16x4096_hbm_traffic.md).  They
+# hold for the default workloads only (config 2; the scene leg at 1 000 000 points) and are reported as null otherwise.
+TRAFFIC_GEMM_BYTES = 319.3e6            # mean of the three contraction launches of a step (algorithmic: 313.5e6)
+TRAFFIC_NB_FILL_BYTES_CONFIG2 = None    # not separated from the scene-scale launches in the counter runs
+TRAFFIC_NB_FILL_BYTES_SCENE = 777.2e6   # algorithmic: 194.6e6
 
 
 def log(*a):
@@ -231,7 +233,7 @@ def main():
     fill_avg_ms = fill_total_ms / max(fill_n, 1)
     fill_gbps = nb_bytes / (fill_avg_ms * 1e-3) / 1e9 if fill_n else 0.0
     roofline_nb = {"kernel": "neighbors_kernel<fill>", "workload": "config 2", "bound": "hbm", "achieved": fill_gbps, "peak": HBM_PEAK_GBPS,
-                   "unit": "GB/s", "frac": fill_gbps / HBM_PEAK_GBPS, "traffic": TRAFFIC_NB_FILL_BYTES,
+                   "unit": "GB/s", "frac": fill_gbps / HBM_PEAK_GBPS, "traffic": TRAFFIC_NB_FILL_BYTES_CONFIG2,
                    "bytes_per_launch": nb_bytes, "avg_launch_ms": fill_avg_ms, "launches": fill_n}
 
     # ---- scene-scale neighbor search (config 4: one room of 10^6 points, cell = radius = 0.05 m): the
@@ -260,7 +262,8 @@ def main():
         s_gbps = s_bytes / (f_avg * 1e-3) / 1e9 if f_n else 0.0
         roofline_nb = {"kernel": "neighbors_kernel<fill>", "workload": "config 4: %d room points, radius 0.05" % n_s,
                        "bound": "hbm", "achieved": s_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                       "frac": s_gbps / HBM_PEAK_GBPS, "traffic": TRAFFIC_NB_FILL_BYTES, "bytes_per_launch": s_bytes,
+                       "frac": s_gbps / HBM_PEAK_GBPS,
+                       "traffic": TRAFFIC_NB_FILL_BYTES_SCENE if n_s == 1000000 else None, "bytes_per_launch": s_bytes,
                        "avg_launch_ms": f_avg, "launches": f_n}
         scene = {"points": n_s, "pairs": s_pairs, "neighborhood_ms": s_ms,
                  "neighbor_pairs_per_sec": s_pairs / (s_ms * 1e-3),
