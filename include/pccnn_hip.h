@@ -97,8 +97,9 @@ int pccnn_build_grid_ds(const int64_t *sorted_keys, int64_t n, const int32_t *nu
  * point_remap[sorted index] (fuses pccnn_lib/pc/Neighborhood.py:47-53), else the
  * sorted index as in the reference op.  Pairs are grouped by ascending sample
  * index; inside a sample they are in ascending sorted-point order.
- * Both calls take the same workspace (count leaves per-sample raw counts in it). */
-size_t pccnn_find_neighbors_workspace_bytes(int64_t m);
+ * Both calls take the same workspace of pccnn_find_neighbors_workspace_bytes(n, m) bytes (count leaves the
+ * per-sample raw counts in it; fill packs the sorted points into 16-byte records there). */
+size_t pccnn_find_neighbors_workspace_bytes(int64_t n, int64_t m);
 /* Optional accelerator for the search (no counterpart in the reference, which binary-searches the sorted
  * keys inside each pillar, find_ranges_grid_ds.cu:111-163): cell_table_out i32[total_cells + 1], entry c =
  * index of the first sorted point with key >= c, total_cells = batch_size * prod(num_cells).  When passed to

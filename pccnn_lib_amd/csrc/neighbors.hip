@@ -1,18 +1,24 @@
 // Radius neighbor search on the pillar grid: count pass, device scan, fill pass.
 //
 // One wavefront owns a tile of 64 consecutive samples of `sample_order` (key order when the
-// caller provides it).  Inside a tile, samples with the same cell key form a run; the run's
-// 3 x 3 pillar walk (9 binary searches on the sorted keys) is done once by lanes 0..8, the
-// candidate points of the 9 ranges are then spread over the 64 lanes (coalesced reads of the
-// sorted xyz array) and every sample of the run is tested against them in turn: one ballot
-// per (sample, 64 candidates).  The fill pass repeats the walk and writes each sample's hits
-// as one contiguous, rank-ordered store, so no atomics are used and the output is deterministic.
+// caller provides it), one sample per lane.  Every lane decodes its own cell, looks up the
+// 3 x 3 pillar walk of that cell (two reads of the cell start table per pillar, or two binary
+// searches in the pillar's slice of the sorted keys) and parks the non-empty index ranges in LDS.
+// The lanes then walk their own candidate lists side by side, a few candidates per lane and
+// iteration: neighbouring lanes sit in the same or adjacent cells, so their loads of the sorted
+// points fall into the same few cache lines.  The fill pass repeats the walk over 16-byte
+// (x, y, z, output id) records packed beforehand and stores the hits straight into the sample's
+// segment, two pairs per store, in ascending sorted-point order, so no atomics are used and the
+// output is deterministic.
 #include "common.h"
 
 // fp32 expressions in this file must round exactly as written (no fused multiply-add).
 #pragma clang fp contract(off)
 
 #define NB_THREADS 256
+#define NB_WAVES (NB_THREADS / 64)
+#define NB_UNROLL_COUNT 4                              // candidates per lane and iteration of the walk
+#define NB_UNROLL_FILL 8
 
 struct NbArgs {
     const float *pts;          // sorted points [n,3]
@@ -34,18 +40,85 @@ struct NbArgs {
     const int32_t *remap;      // FILL: nullable
     int64_t t;                 // FILL: number of output pairs
     int32_t *neigh;            // FILL: [t,2]
+    const float4 *rec;         // FILL: packed (x, y, z, id) of the sorted points
 };
 
-template <bool FILL, bool CAPPED>
+// Four consecutive ints at an 8-byte aligned address as one store instruction.
+struct __attribute__((packed, aligned(8))) NbQuad { int v[4]; };
+__device__ __forceinline__ void nb_store4(int *dst, int a0, int a1, int a2, int a3)
+{
+    NbQuad q;
+    q.v[0] = a0; q.v[1] = a1; q.v[2] = a2; q.v[3] = a3;
+    *reinterpret_cast<NbQuad *>(dst) = q;
+}
+
+// Index range [first, first + len) of the sorted points that lie in cells cmin..cmax of `pillar`.
+__device__ __forceinline__ void nb_pillar_range(const NbArgs &a, long long pillar, int nc2, int cmin, int cmax,
+                                                int &first, int &len)
+{
+    first = 0;
+    len = 0;
+    const long long kbase = pillar * nc2;
+    if (a.cell_table) {
+        // cells cmin..cmax of the pillar are consecutive keys: two table reads give their range
+        if (pillar >= 0 && kbase + cmax + 1 <= a.total_cells) {
+            first = a.cell_table[kbase + cmin];
+            len = a.cell_table[kbase + cmax + 1] - first;
+            if (first < 0 || len < 0 || (int64_t)first + len > a.n) len = 0;
+        }
+    } else if (pillar >= 0 && pillar < a.num_pillars) {
+        int lo = a.grid_ds[2 * pillar], hi = a.grid_ds[2 * pillar + 1];
+        lo = lo < 0 ? 0 : lo;
+        hi = hi > a.n ? (int)a.n : hi;
+        if (hi > lo) {
+            const long long kmin = kbase + cmin;
+            const long long kmax = kbase + cmax;
+            int lb = lo, ub = hi;
+            while (lb < ub) {
+                int mid = (lb + ub) >> 1;
+                if (a.pt_keys[mid] < kmin) lb = mid + 1; else ub = mid;
+            }
+            first = lb;
+            ub = hi;
+            while (lb < ub) {
+                int mid = (lb + ub) >> 1;
+                if (a.pt_keys[mid] <= kmax) lb = mid + 1; else ub = mid;
+            }
+            len = lb - first;
+        }
+    }
+}
+
+// rec[i] = (x, y, z, bits of the id to report for sorted point i): one aligned 16-byte load per candidate
+// gives the fill pass the coordinates and the output id together.
+__global__ void __launch_bounds__(256)
+pack_points_kernel(const float *__restrict__ pts, const int32_t *__restrict__ remap, int64_t n,
+                   float4 *__restrict__ rec)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float4 v;
+    v.x = pts[i * 3 + 0];
+    v.y = pts[i * 3 + 1];
+    v.z = pts[i * 3 + 2];
+    v.w = __int_as_float(remap ? remap[i] : (int)i);
+    rec[i] = v;
+}
+
+template <bool FILL, bool CAPPED, int UNROLL>
 __global__ void __launch_bounds__(NB_THREADS)
 neighbors_kernel(NbArgs a)
 {
+    // ranges[w][r][lane] = r-th non-empty (first, len) range of the lane's sample; written and read by the
+    // same lane only, so no barrier is involved
+    __shared__ int2 ranges[NB_WAVES][9][64];
+
     const int lane = pccnn_lane();
+    const int wib = threadIdx.x >> 6;
     const int64_t wave = ((int64_t)blockIdx.x * NB_THREADS + threadIdx.x) >> 6;
     const int64_t base = wave * 64;
     if (base >= a.m) return;                                   // wave-uniform
-    const int nvalid = (int)((a.m - base) < 64 ? (a.m - base) : 64);
-    const bool valid = lane < nvalid;
+    const bool valid = base + lane < a.m;
 
     int s = 0;
     long long key = -1;
@@ -62,148 +135,137 @@ neighbors_kernel(NbArgs a)
     const float ir1 = __fdiv_rn(1.0f, a.radii[1]);
     const float ir2 = __fdiv_rn(1.0f, a.radii[2]);
 
-    int key_lo = (int)(key & 0xffffffffll), key_hi = (int)(key >> 32);
-    int prev_lo = __shfl_up(key_lo, 1), prev_hi = __shfl_up(key_hi, 1);
-    const bool head = valid && (lane == 0 || prev_lo != key_lo || prev_hi != key_hi);
-    unsigned long long headmask = __ballot(head);
-
-    int my_cnt = 0;                                            // hits seen so far for this lane's sample
-    int my_off = 0, my_raw = 0;                                // FILL: first output slot / uncapped hit count
-    if (FILL && valid) {
-        my_off = s > 0 ? a.ends[s - 1] : 0;
-        if (CAPPED) my_raw = a.counts[s];
+    // key -> (pillar = (batch * nc0 + c0) * nc1 + c1, c0, c1, c2); 32-bit arithmetic when the whole tile allows it
+    long long pil = 0;
+    int c0 = 0, c1 = 0, c2 = 0;
+    const bool usable = valid && key >= 0;
+    if (__all(!usable || key < 0x7fffffffll)) {
+        unsigned int k = usable ? (unsigned int)key : 0u;
+        c2 = (int)(k % (unsigned int)nc2); k /= (unsigned int)nc2;
+        c1 = (int)(k % (unsigned int)nc1); pil = k; k /= (unsigned int)nc1;
+        c0 = (int)(k % (unsigned int)nc0);
+    } else {
+        long long k = usable ? key : 0;
+        c2 = (int)(k % nc2); k /= nc2;
+        c1 = (int)(k % nc1); pil = k; k /= nc1;
+        c0 = (int)(k % nc0);
     }
-    const unsigned long long lt = pccnn_lanemask_lt();
 
-    while (headmask) {
-        const int h = __builtin_ctzll(headmask);
-        headmask &= headmask - 1;
-        const int e = __builtin_amdgcn_readfirstlane(headmask ? __builtin_ctzll(headmask) : nvalid);
-        const long long runkey = pccnn_bcast_ll(key, h);
-
-        // key -> (batch, c0, c1, c2); 32-bit arithmetic whenever the key allows it
-        long long pil;                                         // (batch * nc0 + c0) * nc1 + c1
-        int c0, c1, c2;
-        if (runkey >= 0 && runkey < 0x7fffffffll) {
-            unsigned int k = (unsigned int)runkey;
-            c2 = (int)(k % (unsigned int)nc2); k /= (unsigned int)nc2;
-            c1 = (int)(k % (unsigned int)nc1); pil = k; k /= (unsigned int)nc1;
-            c0 = (int)(k % (unsigned int)nc0);
-        } else {
-            long long k = runkey;
-            c2 = (int)(k % nc2); k /= nc2;
-            c1 = (int)(k % nc1); pil = k; k /= nc1;
-            c0 = (int)(k % nc0);
-        }
-
-        int first = 0, len = 0;
-        if (lane < 9 && runkey >= 0) {
-            const int dx = lane / 3 - 1, dy = lane % 3 - 1;
+    int nr = 0;
+    if (usable) {
+        const int cmin = c2 > 0 ? c2 - 1 : 0, cmax = c2 + 1 < nc2 ? c2 + 1 : nc2 - 1;
+#pragma unroll
+        for (int o = 0; o < 9; ++o) {
+            const int dx = o / 3 - 1, dy = o % 3 - 1;
             const int x = c0 + dx, y = c1 + dy;
             if (x >= 0 && x < nc0 && y >= 0 && y < nc1) {
-                const long long pillar = pil + (long long)dx * nc1 + dy;
-                const int cmin = c2 > 0 ? c2 - 1 : 0, cmax = c2 + 1 < nc2 ? c2 + 1 : nc2 - 1;
-                if (a.cell_table) {
-                    // cells cmin..cmax of the pillar are consecutive keys: two table reads give their range
-                    const long long kbase = pillar * nc2;
-                    if (pillar >= 0 && kbase + cmax + 1 <= a.total_cells) {
-                        first = a.cell_table[kbase + cmin];
-                        len = a.cell_table[kbase + cmax + 1] - first;
-                        if (first < 0 || len < 0 || (int64_t)first + len > a.n) len = 0;
-                    }
-                } else if (pillar >= 0 && pillar < a.num_pillars) {
-                    int lo = a.grid_ds[2 * pillar], hi = a.grid_ds[2 * pillar + 1];
-                    lo = lo < 0 ? 0 : lo;
-                    hi = hi > a.n ? (int)a.n : hi;
-                    if (hi > lo) {
-                        // keys of the cells c2-1 .. c2+1 of this pillar
-                        const long long kbase = pillar * nc2;
-                        const long long kmin = kbase + cmin;
-                        const long long kmax = kbase + cmax;
-                        int lb = lo, ub = hi;
-                        while (lb < ub) {
-                            int mid = (lb + ub) >> 1;
-                            if (a.pt_keys[mid] < kmin) lb = mid + 1; else ub = mid;
-                        }
-                        first = lb;
-                        ub = hi;
-                        while (lb < ub) {
-                            int mid = (lb + ub) >> 1;
-                            if (a.pt_keys[mid] <= kmax) lb = mid + 1; else ub = mid;
-                        }
-                        len = lb - first;
-                    }
+                int first, len;
+                nb_pillar_range(a, pil + (long long)dx * nc1 + dy, nc2, cmin, cmax, first, len);
+                if (len > 0) {
+                    ranges[wib][nr][lane] = make_int2(first, len);
+                    ++nr;
                 }
             }
         }
-        int st[9], ln[9], total = 0;
-#pragma unroll
-        for (int o = 0; o < 9; ++o) {
-            st[o] = __builtin_amdgcn_readlane(first, o);
-            ln[o] = __builtin_amdgcn_readlane(len, o);
-            total += ln[o];
+    }
+
+    unsigned int my_off = 0;                                    // FILL: next output slot of this lane's sample
+    int raw = 0, take_step = 0;                                 // capped: see below
+    if (FILL && valid) {
+        my_off = s > 0 ? (unsigned int)a.ends[s - 1] : 0u;
+        if (CAPPED) {
+            raw = a.counts[s];
+            take_step = raw < a.max_neighbors ? raw : a.max_neighbors;
         }
+    }
+    const unsigned int out_limit = FILL ? (unsigned int)a.t : 0u;
+    int held = -1;                                              // FILL: a kept hit waiting for a partner
 
-        for (int cb = 0; cb < total; cb += 64) {
-            const int j = cb + lane;
-            const bool cvalid = j < total;
-            int idx = 0, rem = j;
+    // Capped samples keep hit number r (0-based, in walk order) iff floor((r+1)*cap/raw) > floor(r*cap/raw),
+    // at slot floor(r*cap/raw): with err = (r*cap) mod raw this is "err + cap >= raw", and the slot advances by one
+    // with every kept hit.  Samples at or below the cap use step = raw, which keeps every hit.
+    int cnt = 0, err = 0;
+    int r = 0, j = 0, first = 0, len = 0;
+    bool active = nr > 0;
+    if (active) {
+        const int2 g = ranges[wib][0][lane];
+        first = g.x;
+        len = g.y;
+    }
+    while (__any(active)) {
+        if (active) {
+            // UNROLL consecutive candidates of the current range per iteration: their loads are issued
+            // together; slots past the end of the range re-read its first candidate and are masked out
+            const int idx = first + j;
+            const int left = len - j;
+            float px[UNROLL], py[UNROLL], pz[UNROLL];
+            int id[UNROLL];
 #pragma unroll
-            for (int o = 0; o < 9; ++o) {
-                if (rem >= 0 && rem < ln[o]) idx = st[o] + rem;
-                rem -= ln[o];
+            for (int u = 0; u < UNROLL; ++u) {
+                const int iu = idx + (u < left ? u : 0);
+                if (FILL) {
+                    const float4 v = a.rec[iu];
+                    px[u] = v.x; py[u] = v.y; pz[u] = v.z;
+                    id[u] = __float_as_int(v.w);
+                } else {
+                    px[u] = a.pts[(int64_t)iu * 3 + 0];
+                    py[u] = a.pts[(int64_t)iu * 3 + 1];
+                    pz[u] = a.pts[(int64_t)iu * 3 + 2];
+                    id[u] = 0;
+                }
             }
-            float px = 0.f, py = 0.f, pz = 0.f;
-            if (cvalid) {
-                px = a.pts[(int64_t)idx * 3 + 0];
-                py = a.pts[(int64_t)idx * 3 + 1];
-                pz = a.pts[(int64_t)idx * 3 + 2];
-            }
-            int out_id = idx;
-            if (FILL && cvalid && a.remap) out_id = a.remap[idx];
-
-            for (int q = h; q < e; ++q) {
-                const float qx = pccnn_bcast_f(sx, q), qy = pccnn_bcast_f(sy, q), qz = pccnn_bcast_f(sz, q);
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
                 // fp32, no contraction: ((s - p) * (1/r)) squared, summed x, y, z; the reference tests
                 // sqrt(acc) < 1, which for a correctly rounded fp32 sqrt holds exactly when acc < 1
                 // (the largest float below 1 has a root below the midpoint to 1, so it rounds down).
-                const float vx = (qx - px) * ir0;
-                const float vy = (qy - py) * ir1;
-                const float vz = (qz - pz) * ir2;
+                const float vx = (sx - px[u]) * ir0;
+                const float vy = (sy - py[u]) * ir1;
+                const float vz = (sz - pz[u]) * ir2;
                 const float acc = ((0.0f + vx * vx) + vy * vy) + vz * vz;
-                const bool hit = cvalid && (acc < 1.0f);
-                const unsigned long long bal = __ballot(hit);
-                const int c = __popcll(bal);
-                if (FILL) {
-                    // my_off + my_cnt of lane q = next free slot of that sample (uncapped case)
-                    const int qoff = pccnn_bcast_i(CAPPED ? my_off : my_off + my_cnt, q);
-                    const int qs = pccnn_bcast_i(s, q);
-                    if (hit) {
-                        int slot = __popcll(bal & lt);
+                if (u < left && acc < 1.0f) {
+                    if (FILL) {
                         bool take = true;
                         if (CAPPED) {
-                            const int qraw = pccnn_bcast_i(my_raw, q);
-                            const int r = pccnn_bcast_i(my_cnt, q) + slot;
-                            slot = r;
-                            if (qraw > a.max_neighbors) {
-                                slot = (int)(((long long)r * a.max_neighbors) / qraw);
-                                take = (int)(((long long)(r + 1) * a.max_neighbors) / qraw) > slot;
+                            err += take_step;
+                            take = err >= raw;
+                            if (take) err -= raw;
+                        }
+                        if (take) {
+                            // kept hits leave in pairs: one 16-byte store per two pairs of the sample's segment
+                            if (held < 0) {
+                                held = id[u];
+                            } else {
+                                if (my_off + 1u < out_limit) {
+                                    int *dst = a.neigh + 2 * (size_t)my_off;
+                                    nb_store4(dst, held, s, id[u], s);
+                                }
+                                my_off += 2u;
+                                held = -1;
                             }
                         }
-                        const int64_t pos = (int64_t)qoff + slot;
-                        if (take && pos < a.t) {
-                            int2 pr;
-                            pr.x = out_id;
-                            pr.y = qs;
-                            ((int2 *)a.neigh)[pos] = pr;
-                        }
                     }
+                    ++cnt;
                 }
-                if (lane == q) my_cnt += c;
+            }
+            j += UNROLL;
+            if (j >= len) {
+                j = 0;
+                if (++r < nr) {
+                    const int2 g = ranges[wib][r][lane];
+                    first = g.x;
+                    len = g.y;
+                } else {
+                    active = false;
+                }
             }
         }
     }
-    if (!FILL && valid) a.counts[s] = my_cnt;
+    if (FILL) {
+        if (held >= 0 && my_off < out_limit) ((int2 *)a.neigh)[my_off] = make_int2(held, s);
+    } else if (valid) {
+        a.counts[s] = cnt;
+    }
 }
 
 // table[c] = index of the first sorted point whose key is >= c, for c in [0, total_cells].  The lane of
@@ -249,10 +311,15 @@ extern "C" int pccnn_build_cell_table(const int64_t *sorted_keys, int64_t n, int
     return PCCNN_OK;
 }
 
-extern "C" size_t pccnn_find_neighbors_workspace_bytes(int64_t m)
+// Workspace layout, shared by the two calls: raw counts i32[m] | scan scratch (count) overlaid by the packed
+// point records float4[n] (fill).
+extern "C" size_t pccnn_find_neighbors_workspace_bytes(int64_t n, int64_t m)
 {
     if (m < 1) m = 1;
-    return pccnn_align((size_t)m * sizeof(int32_t)) + pccnn_align(pccnn_scan_tmp_elems(m) * sizeof(int32_t)) + 256;
+    if (n < 1) n = 1;
+    size_t scan = pccnn_align(pccnn_scan_tmp_elems(m) * sizeof(int32_t));
+    size_t rec = pccnn_align((size_t)n * sizeof(float4));
+    return pccnn_align((size_t)m * sizeof(int32_t)) + (scan > rec ? scan : rec) + 256;
 }
 
 static int nb_validate(const char *who, const float *pts_sorted, const int64_t *pt_keys_sorted, int64_t n,
@@ -270,9 +337,9 @@ static int nb_validate(const char *who, const float *pts_sorted, const int64_t *
     PCCNN_REQUIRE(grid_ds && num_cells && radii, PCCNN_ERR_INVALID, "%s: null grid pointer", who);
     PCCNN_REQUIRE(n == 0 || (pts_sorted && pt_keys_sorted), PCCNN_ERR_INVALID, "%s: null point pointer", who);
     PCCNN_REQUIRE(m == 0 || (samples && sample_keys), PCCNN_ERR_INVALID, "%s: null sample pointer", who);
-    PCCNN_REQUIRE(workspace && workspace_bytes >= pccnn_find_neighbors_workspace_bytes(m), PCCNN_ERR_WORKSPACE,
+    PCCNN_REQUIRE(workspace && workspace_bytes >= pccnn_find_neighbors_workspace_bytes(n, m), PCCNN_ERR_WORKSPACE,
                   "%s: workspace of %zu bytes, need %zu", who, workspace_bytes,
-                  pccnn_find_neighbors_workspace_bytes(m));
+                  pccnn_find_neighbors_workspace_bytes(n, m));
     return PCCNN_OK;
 }
 
@@ -300,11 +367,11 @@ extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t
     a.order = sample_order; a.grid_ds = grid_ds; a.num_pillars = num_pillars;
     a.cell_table = cell_table; a.total_cells = total_cells;
     a.num_cells = num_cells; a.radii = radii; a.max_neighbors = max_neighbors;
-    a.counts = counts; a.ends = nullptr; a.remap = nullptr; a.t = 0; a.neigh = nullptr;
+    a.counts = counts; a.ends = nullptr; a.remap = nullptr; a.t = 0; a.neigh = nullptr; a.rec = nullptr;
     int64_t waves = pccnn_ceil_div(m, 64);
     {
         PccnnTimed timed(PCCNN_T_NB_COUNT, s);
-        neighbors_kernel<false, false><<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
+        neighbors_kernel<false, false, NB_UNROLL_COUNT><<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
     }
     PCCNN_LAUNCH_CHECK();
     PccnnTimed timed(PCCNN_T_SCAN, s);
@@ -329,6 +396,7 @@ extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t 
     hipStream_t s = (hipStream_t)stream;
     PccnnArena arena(workspace, workspace_bytes);
     int32_t *counts = arena.take<int32_t>((size_t)m);
+    float4 *rec = arena.take<float4>((size_t)(n > 0 ? n : 1));
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "pccnn_find_neighbors_fill: workspace too small");
     NbArgs a;
     a.pts = pts_sorted; a.pt_keys = pt_keys_sorted; a.n = n;
@@ -336,14 +404,17 @@ extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t 
     a.order = sample_order; a.grid_ds = grid_ds; a.num_pillars = num_pillars;
     a.cell_table = cell_table; a.total_cells = total_cells;
     a.num_cells = num_cells; a.radii = radii; a.max_neighbors = max_neighbors;
-    a.counts = counts; a.ends = ends; a.remap = point_remap; a.t = t; a.neigh = neigh_out;
+    a.counts = counts; a.ends = ends; a.remap = point_remap; a.t = t; a.neigh = neigh_out; a.rec = rec;
     int64_t waves = pccnn_ceil_div(m, 64);
     {
         PccnnTimed timed(PCCNN_T_NB_FILL, s);
+        if (n > 0) pack_points_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(pts_sorted, point_remap, n, rec);
         if (max_neighbors > 0)
-            neighbors_kernel<true, true><<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
+            neighbors_kernel<true, true, NB_UNROLL_FILL>
+                <<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
         else
-            neighbors_kernel<true, false><<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
+            neighbors_kernel<true, false, NB_UNROLL_FILL>
+                <<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
     }
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;

@@ -187,7 +187,7 @@ def find_neighbors_ex(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, ra
     ends = torch.empty((m,), dtype=torch.int32, device=dev)
     if m == 0:
         return [torch.empty((0, 2), dtype=torch.int32, device=dev), ends]
-    ws = _workspace(_lib.load().pccnn_find_neighbors_workspace_bytes(m), dev)
+    ws = _workspace(_lib.load().pccnn_find_neighbors_workspace_bytes(n, m), dev)
     order_p = _ptr(sample_order) if sample_order is not None else _P(0)
     _lib.call("pccnn_find_neighbors_count", _ptr(pts), _ptr(pt_keys), n, _ptr(samples), _ptr(sample_keys), m, order_p,
               _ptr(grid_ds), pillars, table_p, total_cells, _ptr(grid_size), _ptr(radii), d, max_neighbors, _ptr(ends),

@@ -70,7 +70,7 @@ def test_argument_validation_needs_no_gpu(lib_path):
                                    None, 0, None)
     assert rc == -2 and b"k=65" in lib.pccnn_last_error()
     assert lib.pccnn_conv_workspace_bytes(1000, 5000, 32, 16, 64, 0) >= 1000 * 32 * 16 * 4
-    assert lib.pccnn_find_neighbors_workspace_bytes(1000) >= 4000
+    assert lib.pccnn_find_neighbors_workspace_bytes(500, 1000) >= 4000 + 500 * 16
 
 
 def test_op_module_exports_reference_names():
