@@ -304,6 +304,34 @@ int pccnn_gemm_f32(const float *a, const float *b, float *c, int64_t rows, int64
                    int batch, int64_t stride_a, int64_t stride_b, int64_t stride_c,
                    int split_k, void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- bf16 contraction ----------------------------------------------------
+ * A mode the reference does not have (its contraction is an fp32 torch::matmul, mcconv.cu:64-68,111-120,
+ * kpconv.cu:56-57,90-96): the operands of the three contractions of a convolution -- the projection P, the
+ * weights and the output gradients -- are rounded to bf16 (nearest even) and multiplied on the bf16 matrix
+ * pipe with fp32 accumulation; bases, aggregation, every result and every other gradient stay fp32.
+ * pccnn_conv_forward_bf16 / pccnn_conv_backward_bf16 take the arguments of pccnn_conv_forward /
+ * pccnn_conv_backward, except that the projection handed from forward to backward is uint16_t[m, c_in*k] of
+ * bf16 bit patterns; workspace size as for the fp32 calls.
+ * pccnn_gemm_bf16 is that contraction on its own (arguments as pccnn_gemm_f32, A and B bf16 bit patterns, C fp32);
+ * pccnn_f32_to_bf16 is the rounding the library applies (dst[i] = bf16(src[i])). */
+int pccnn_f32_to_bf16(const float *src, uint16_t *dst, int64_t count, void *stream);
+int pccnn_gemm_bf16(const uint16_t *a, const uint16_t *b, float *c, int64_t rows, int64_t cols, int64_t inner,
+                    int a_trans, int b_trans, int64_t lda, int64_t ldb, int64_t ldc,
+                    int batch, int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                    int split_k, void *workspace, size_t workspace_bytes, void *stream);
+int pccnn_conv_forward_bf16(const pccnn_basis *basis, const float *pts, const float *feats, const float *samples,
+                            const int32_t *neigh, const int32_t *ends, const float *radii, const float *weights,
+                            int64_t n, int64_t m, int64_t t, int d, int c_in, int num_mlps, int c_out,
+                            int divide_by_count, float *out, uint16_t *proj_out,
+                            void *workspace, size_t workspace_bytes, void *stream);
+int pccnn_conv_backward_bf16(const pccnn_basis *basis, const float *pts, const float *feats, const float *samples,
+                             const int32_t *neigh, const int32_t *ends, const float *radii, const float *weights,
+                             const float *in_grads, const uint16_t *proj, const int32_t *mirror, int grad_mask,
+                             int64_t n, int64_t m, int64_t t, int d, int c_in, int num_mlps, int c_out,
+                             int divide_by_count, float *d_weights, float *d_feats, float *d_param_a,
+                             float *d_param_b, float *d_pdf, float *d_pts, float *d_samples,
+                             void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- per-kernel timing ---------------------------------------------------
  * Measurement hooks with no counterpart in the reference (it has no profiler hooks).  While
  * enabled, the entry points above bracket their main kernels with HIP events on the launch

@@ -295,25 +295,45 @@ def _pt_diff_grads(n, m, neigh, radii, diff_grads):
     return dp.astype(np.float32), (-dsm).astype(np.float32)
 
 
-def kpconv(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights):
-    """pccnn_lib_ops/pcconvs/kpconv.cu:32-60."""
+def bf16_round(a):
+    """fp32 -> nearest bf16 (ties to even) -> fp32.  The reference has no bf16 mode; this is the operand rounding
+    of the bf16 contraction of config 5 ("features bf16 for the MFMA contraction with fp32 accumulation")."""
+    a = _f32(a)
+    u = a.view(np.uint32).astype(np.uint64)
+    r = (((u + 0x7fff + ((u >> 16) & 1)) >> 16) << 16).astype(np.uint32).view(np.float32)
+    return np.where(np.isnan(a), a, r).astype(np.float32)
+
+
+def _operands(contraction):
+    if contraction == "f32":
+        return lambda x: x
+    if contraction == "bf16":
+        return bf16_round
+    raise ValueError("contraction must be 'f32' or 'bf16'")
+
+
+def kpconv(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights, contraction="f32"):
+    """pccnn_lib_ops/pcconvs/kpconv.cu:32-60.  contraction="bf16": both operands of the matmul rounded to bf16."""
+    rnd = _operands(contraction)
     basis, _ = conv_basis(KP, pts, samples, neigh, radii, kernel_pts, sigma=sigma)
     proj = feat_basis_proj(basis, feats, neigh, ends)
     m = ends.shape[0]
-    out = proj.reshape(m, -1).astype(np.float64) @ _f32(weights).astype(np.float64)
+    out = rnd(proj.reshape(m, -1)).astype(np.float64) @ rnd(_f32(weights)).astype(np.float64)
     return out.astype(np.float32)
 
 
-def kpconv_grads(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights, in_grads):
+def kpconv_grads(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights, in_grads, contraction="f32"):
     """pccnn_lib_ops/pcconvs/kpconv.cu:63-112 with kernel_pts_basis.cu:41-70.
-    Returns [dW, dFeat, dKernelPts, dPts, dSamples]."""
+    Returns [dW, dFeat, dKernelPts, dPts, dSamples].  contraction="bf16": the operands of both matmuls (projection,
+    weights, incoming gradients) rounded to bf16."""
+    rnd = _operands(contraction)
     pts, samples, neigh, kernel_pts = _f32(pts), _f32(samples), _i32(neigh), _f32(kernel_pts)
     weights, in_grads = _f32(weights), _f32(in_grads)
     m = ends.shape[0]
     basis, diff = conv_basis(KP, pts, samples, neigh, radii, kernel_pts, sigma=sigma)
     proj = feat_basis_proj(basis, feats, neigh, ends).reshape(m, -1)
-    dw = (proj.astype(np.float64).T @ in_grads.astype(np.float64)).astype(np.float32)
-    dproj = (in_grads.astype(np.float64) @ weights.astype(np.float64).T).astype(np.float32)
+    dw = (rnd(proj).astype(np.float64).T @ rnd(in_grads).astype(np.float64)).astype(np.float32)
+    dproj = (rnd(in_grads).astype(np.float64) @ rnd(weights).astype(np.float64).T).astype(np.float32)
     dfeat, dbasis = feat_basis_proj_grads(basis, feats, neigh, ends, dproj)
     # kernel_pts_basis_grads: fp32 distances and mask as the reference forms them.
     sig = np.float32(sigma)
@@ -334,32 +354,34 @@ def kpconv_grads(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, wei
     return [dw, dfeat, dkp, dpts, dsamples]
 
 
-def mcconv(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights):
-    """pccnn_lib_ops/pcconvs/mcconv.cu:32-71 (weights [numMLPs, H*Cin/.., Cout/numMLPs])."""
+def mcconv(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights, contraction="f32"):
+    """pccnn_lib_ops/pcconvs/mcconv.cu:32-71 (weights [numMLPs, H*Cin/.., Cout/numMLPs]).  contraction as in kpconv."""
+    rnd = _operands(contraction)
     weights = _f32(weights)
     num_mlps = weights.shape[0]
     basis, _ = conv_basis(MLP, pts, samples, neigh, radii, axis, bias=bias, pdf=pdf)
     proj = feat_basis_proj(basis, feats, neigh, ends)
     m = ends.shape[0]
-    proj = proj.reshape(m, num_mlps, -1).transpose(1, 0, 2).astype(np.float64)
-    out = np.matmul(proj, weights.astype(np.float64))                        # [mlps, M, Cout/mlps]
+    proj = rnd(proj).reshape(m, num_mlps, -1).transpose(1, 0, 2).astype(np.float64)
+    out = np.matmul(proj, rnd(weights).astype(np.float64))                   # [mlps, M, Cout/mlps]
     return out.transpose(1, 0, 2).reshape(m, -1).astype(np.float32)
 
 
-def mcconv_grads(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights, in_grads):
+def mcconv_grads(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights, in_grads, contraction="f32"):
     """pccnn_lib_ops/pcconvs/mcconv.cu:73-143 with mlp_basis.cu:50-96.
-    Returns [dW, dFeat, dAxis, dBias, dPdf, dPts, dSamples]."""
+    Returns [dW, dFeat, dAxis, dBias, dPdf, dPts, dSamples].  contraction as in kpconv_grads."""
+    rnd = _operands(contraction)
     pts, samples, neigh, axis = _f32(pts), _f32(samples), _i32(neigh), _f32(axis)
     weights, in_grads, pdf = _f32(weights), _f32(in_grads), _f32(pdf)
     bias = _f32(bias).reshape(1, -1)
     num_mlps = weights.shape[0]
     m = ends.shape[0]
-    g = in_grads.reshape(m, num_mlps, -1).transpose(1, 0, 2).astype(np.float64)
+    g = rnd(in_grads).reshape(m, num_mlps, -1).transpose(1, 0, 2).astype(np.float64)
     basis, diff = conv_basis(MLP, pts, samples, neigh, radii, axis, bias=bias, pdf=pdf)
     proj = feat_basis_proj(basis, feats, neigh, ends)
-    projr = proj.reshape(m, num_mlps, -1).transpose(1, 0, 2).astype(np.float64)
+    projr = rnd(proj).reshape(m, num_mlps, -1).transpose(1, 0, 2).astype(np.float64)
     dw = np.matmul(projr.transpose(0, 2, 1), g).astype(np.float32)
-    dproj = np.matmul(g, weights.astype(np.float64).transpose(0, 2, 1))
+    dproj = np.matmul(g, rnd(weights).astype(np.float64).transpose(0, 2, 1))
     dproj = dproj.transpose(1, 0, 2).reshape(m, -1).astype(np.float32)
     dfeat, dbasis = feat_basis_proj_grads(basis, feats, neigh, ends, dproj)
     # mlp_basis_grads (pDiv = true): activations in fp32 as the forward forms them.

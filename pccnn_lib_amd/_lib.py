@@ -62,6 +62,12 @@ SIGNATURES = {
     "pccnn_conv_forward": (I32, [BP, P, P, P, P, P, P, P, I64, I64, I64, I32, I32, I32, I32, I32, P, P, P, SZ, P]),
     "pccnn_conv_backward": (I32, [BP, P, P, P, P, P, P, P, P, P, P, I32, I64, I64, I64, I32, I32, I32, I32, I32,
                                   P, P, P, P, P, P, P, P, SZ, P]),
+    "pccnn_conv_forward_bf16": (I32, [BP, P, P, P, P, P, P, P, I64, I64, I64, I32, I32, I32, I32, I32, P, P, P, SZ,
+                                      P]),
+    "pccnn_conv_backward_bf16": (I32, [BP, P, P, P, P, P, P, P, P, P, P, I32, I64, I64, I64, I32, I32, I32, I32, I32,
+                                       P, P, P, P, P, P, P, P, SZ, P]),
+    "pccnn_f32_to_bf16": (I32, [P, P, I64, P]),
+    "pccnn_gemm_bf16": (I32, [P, P, P, I64, I64, I64, I32, I32, I64, I64, I64, I32, I64, I64, I64, I32, P, SZ, P]),
     "pccnn_conv_weight_var": (I32, [BP, P, P, P, P, P, P, I64, I64, I64, I32, I32, I32, P, P, SZ, P]),
     "pccnn_linear_basis_forward": (I32, [P, P, P, P, P, P, I64, I64, I64, I32, I32, P, P]),
     "pccnn_linear_basis_workspace_bytes": (SZ, [I64]),

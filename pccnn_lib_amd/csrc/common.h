@@ -72,6 +72,15 @@ __device__ __forceinline__ long long pccnn_bcast_ll(long long v, int src)
     return ((long long)hi << 32) | (unsigned int)lo;
 }
 
+// fp32 -> bf16 bit pattern, round to nearest even; a NaN stays a (quiet) NaN.
+__device__ __forceinline__ uint16_t pccnn_bf16_bits(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
 __device__ __forceinline__ float pccnn_wave_sum(float v)
 {
 #pragma unroll
@@ -100,6 +109,13 @@ struct PccnnTimed {
 size_t pccnn_scan_tmp_elems(int64_t n);
 int pccnn_scan_inclusive_i32(const int32_t *in, int32_t *out, int64_t n, int clamp_max, int32_t *tmp,
                              hipStream_t stream);
+
+// bf16 contraction (gemm_bf16.hip), used by conv.hip.
+extern "C" int pccnn_f32_to_bf16(const float *src, uint16_t *dst, int64_t count, void *stream);
+extern "C" int pccnn_gemm_bf16(const uint16_t *a, const uint16_t *b, float *c, int64_t rows, int64_t cols,
+                               int64_t inner, int a_trans, int b_trans, int64_t lda, int64_t ldb, int64_t ldc,
+                               int batch, int64_t stride_a, int64_t stride_b, int64_t stride_c, int split_k,
+                               void *workspace, size_t workspace_bytes, void *stream);
 
 // Internal sort entry used by other translation units.
 int pccnn_fill_i32(int32_t *p, int32_t value, int64_t count, hipStream_t stream);

@@ -120,9 +120,9 @@ __device__ __forceinline__ float pair_basis(const ConvGeom &g, const LaneBasis<B
 
 // ------------------------------------------------------------------------------- forward
 
-template <int BASIS, int KPAD>
+template <int BASIS, int KPAD, bool BF16>
 __global__ void __launch_bounds__(64)
-conv_proj_fwd_kernel(ConvGeom g, const float *__restrict__ feats, float *__restrict__ proj)
+conv_proj_fwd_kernel(ConvGeom g, const float *__restrict__ feats, void *__restrict__ proj_out)
 {
     // One single-wavefront workgroup per (sample, block of 64 features).  The basis values of up to 64 pairs
     // are evaluated once, KPAD lanes per pair, and parked in LDS; every lane then reads them back as
@@ -204,13 +204,33 @@ conv_proj_fwd_kernel(ConvGeom g, const float *__restrict__ feats, float *__restr
     __syncthreads();
     const int f0 = blockIdx.y * 64;
     const int nf = (g.c_in - f0) < 64 ? (g.c_in - f0) : 64;
-    float *dst = proj + ((int64_t)s * g.c_in + f0) * g.k;
-    if (g.k == KPAD) {
-        for (int i = lane; i < nf * (KPAD / 4); i += 64) ((float4 *)dst)[i] = ((const float4 *)tile)[i];
+    const int64_t dst_at = ((int64_t)s * g.c_in + f0) * g.k;
+    if (BF16) {
+        // the projection leaves as bf16 (round to nearest even): the operand format of the bf16 contraction
+        uint16_t *dst = (uint16_t *)proj_out + dst_at;
+        if (g.k == KPAD) {
+            for (int i = lane; i < nf * (KPAD / 4); i += 64) {
+                const float4 v = ((const float4 *)tile)[i];
+                uint2 o;
+                o.x = pccnn_bf16_bits(v.x) | ((uint32_t)pccnn_bf16_bits(v.y) << 16);
+                o.y = pccnn_bf16_bits(v.z) | ((uint32_t)pccnn_bf16_bits(v.w) << 16);
+                ((uint2 *)dst)[i] = o;
+            }
+        } else {
+            for (int idx = lane; idx < nf * g.k; idx += 64) {
+                const int ff = idx / g.k, q = idx - ff * g.k;
+                dst[idx] = pccnn_bf16_bits(tile[ff * KPAD + q]);
+            }
+        }
     } else {
-        for (int idx = lane; idx < nf * g.k; idx += 64) {
-            const int ff = idx / g.k, q = idx - ff * g.k;
-            dst[idx] = tile[ff * KPAD + q];
+        float *dst = (float *)proj_out + dst_at;
+        if (g.k == KPAD) {
+            for (int i = lane; i < nf * (KPAD / 4); i += 64) ((float4 *)dst)[i] = ((const float4 *)tile)[i];
+        } else {
+            for (int idx = lane; idx < nf * g.k; idx += 64) {
+                const int ff = idx / g.k, q = idx - ff * g.k;
+                dst[idx] = tile[ff * KPAD + q];
+            }
         }
     }
 }
@@ -688,17 +708,24 @@ linear_basis_bwd_kernel(ConvGeom g, const float *__restrict__ basis_grads, float
 
 static int kpad_of(int k) { return k <= 8 ? 8 : (k <= 16 ? 16 : (k <= 32 ? 32 : 64)); }
 
+// `bf16`: proj is uint16_t[m, c_in * k] of bf16 bit patterns instead of float[m, c_in * k].
 template <int BASIS>
-static int launch_proj_fwd(const ConvGeom &g, const float *feats, float *proj, hipStream_t s)
+static int launch_proj_fwd(const ConvGeom &g, const float *feats, void *proj, hipStream_t s, bool bf16 = false)
 {
     dim3 grid((unsigned)g.m, (unsigned)((g.c_in + 63) / 64));
     PccnnTimed timed(PCCNN_T_PROJ_FWD, s);
+#define PROJ_GO(KP)                                                                         \
+    do {                                                                                    \
+        if (bf16) conv_proj_fwd_kernel<BASIS, KP, true><<<grid, 64, 0, s>>>(g, feats, proj);  \
+        else conv_proj_fwd_kernel<BASIS, KP, false><<<grid, 64, 0, s>>>(g, feats, proj);      \
+    } while (0)
     switch (kpad_of(g.k)) {
-    case 8: conv_proj_fwd_kernel<BASIS, 8><<<grid, 64, 0, s>>>(g, feats, proj); break;
-    case 16: conv_proj_fwd_kernel<BASIS, 16><<<grid, 64, 0, s>>>(g, feats, proj); break;
-    case 32: conv_proj_fwd_kernel<BASIS, 32><<<grid, 64, 0, s>>>(g, feats, proj); break;
-    default: conv_proj_fwd_kernel<BASIS, 64><<<grid, 64, 0, s>>>(g, feats, proj); break;
+    case 8: PROJ_GO(8); break;
+    case 16: PROJ_GO(16); break;
+    case 32: PROJ_GO(32); break;
+    default: PROJ_GO(64); break;
     }
+#undef PROJ_GO
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
 }
@@ -766,13 +793,15 @@ extern "C" size_t pccnn_conv_workspace_bytes(int64_t m, int64_t t, int c_in, int
     if (m < 1) m = 1;
     if (t < 1) t = 1;
     size_t proj = pccnn_align((size_t)m * c_in * k * sizeof(float));
-    if (!backward) return proj + 256;
+    size_t w16 = pccnn_align((size_t)c_in * k * c_out * sizeof(uint16_t));       // bf16 copy of the weights
+    if (!backward) return proj + w16 + 256;
     size_t basis_g = pccnn_align((size_t)t * k * sizeof(float));
     size_t splitk = pccnn_align((size_t)CONV_SPLIT_K * c_in * k * c_out * sizeof(float));
     size_t partials = pccnn_align(((size_t)PARAM_ROWS + PARAM_REDUCE_GROUPS) * 256 * sizeof(float));
     size_t scaled = pccnn_align((size_t)m * c_out * sizeof(float));
     size_t pair_g = pccnn_align((size_t)t * 4 * sizeof(float));
-    return 2 * proj + basis_g + splitk + partials + scaled + pair_g + 256;
+    size_t g16 = pccnn_align((size_t)m * c_out * sizeof(uint16_t));               // bf16 copy of the output gradients
+    return 2 * proj + basis_g + splitk + partials + scaled + pair_g + w16 + g16 + 256;
 }
 
 // out[m, c_out] = P[m, c_in*k] x W, with the feature axis split over num_mlps independent
@@ -786,22 +815,32 @@ static int contraction_fwd(const float *proj, const float *weights, float *out, 
                           inner * co, co, 1, nullptr, 0, s);
 }
 
+// `bf16`: the projection (proj_out, when given, is uint16_t[m, c_in * k]) and a copy of the weights are kept as
+// bf16 and contracted on the bf16 matrix pipe with fp32 accumulation; everything else stays fp32.
 template <int BASIS>
 static int conv_forward(ConvGeom g, const float *feats, const float *weights, int num_mlps, int c_out, float *out,
-                        float *proj_out, void *workspace, size_t workspace_bytes, hipStream_t s,
-                        bool divide_by_count = false)
+                        void *proj_out, void *workspace, size_t workspace_bytes, hipStream_t s,
+                        bool divide_by_count = false, bool bf16 = false)
 {
     if (g.m == 0) return PCCNN_OK;
-    float *proj = proj_out;
-    if (proj == nullptr) {
-        PccnnArena arena(workspace, workspace_bytes);
-        proj = arena.take<float>((size_t)g.m * g.c_in * g.k);
-        PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv forward: workspace of %zu bytes, need %zu",
-                      workspace_bytes, pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 0));
-    }
-    int rc = launch_proj_fwd<BASIS>(g, feats, proj, s);
+    PccnnArena arena(workspace, workspace_bytes);
+    void *proj = proj_out;
+    if (proj == nullptr) proj = arena.take<float>((size_t)g.m * g.c_in * g.k);
+    const int64_t w_count = (int64_t)g.c_in * g.k * c_out / num_mlps;
+    uint16_t *w16 = bf16 ? arena.take<uint16_t>((size_t)w_count) : nullptr;
+    PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv forward: workspace of %zu bytes, need %zu", workspace_bytes,
+                  pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 0));
+    int rc = launch_proj_fwd<BASIS>(g, feats, proj, s, bf16);
     if (rc != PCCNN_OK) return rc;
-    rc = contraction_fwd(proj, weights, out, g.m, g.c_in, g.k, num_mlps, c_out, s);
+    if (bf16) {
+        const int64_t inner = (int64_t)g.c_in * g.k / num_mlps;
+        const int64_t co = c_out / num_mlps;
+        if ((rc = pccnn_f32_to_bf16(weights, w16, w_count, s)) != PCCNN_OK) return rc;
+        rc = pccnn_gemm_bf16((const uint16_t *)proj, w16, out, g.m, co, inner, 0, 0, (int64_t)g.c_in * g.k, co, c_out,
+                             num_mlps, inner, inner * co, co, 1, nullptr, 0, s);
+    } else {
+        rc = contraction_fwd((const float *)proj, weights, out, g.m, g.c_in, g.k, num_mlps, c_out, s);
+    }
     if (rc != PCCNN_OK || !divide_by_count) return rc;
     scale_by_count_kernel<<<(unsigned)pccnn_ceil_div(g.m * c_out, 256), 256, 0, s>>>(out, out, g.ends, g.m, c_out);
     PCCNN_LAUNCH_CHECK();
@@ -811,11 +850,13 @@ static int conv_forward(ConvGeom g, const float *feats, const float *weights, in
 // Gradients are produced only for the groups named in `mask`; pointers of groups not requested may be null.
 template <int BASIS>
 static int conv_backward(ConvGeom g, const float *feats, const float *weights, const float *in_grads, int num_mlps,
-                         int c_out, const float *proj_in, int mask, float *d_weights, float *d_feats,
+                         int c_out, const void *proj_in, int mask, float *d_weights, float *d_feats,
                          float *d_param_a, float *d_param_b, float *d_pdf, float *d_pts, float *d_samples,
                          void *workspace, size_t workspace_bytes, hipStream_t s, bool divide_by_count = false,
-                         const int32_t *mirror = nullptr)
+                         const int32_t *mirror = nullptr, bool bf16 = false)
 {
+    // bf16: proj_in (when given) is uint16_t[m, c_in * k]; the two contractions take bf16 copies of the weights
+    // and of the output gradients, accumulate in fp32 and return fp32 (d_weights, d_proj)
     // d_param_a: d_kernel_pts [K,3] (kernel-point families), d_axis [3,K] (MLP) or the per-pair basis
     // gradient [T,K] (EXPLICIT); d_param_b: d_bias [K] (MLP only)
     typedef BasisTraits<BASIS> Tr;
@@ -854,6 +895,9 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     float *splitk = arena.take<float>(splitk_elems);
     float *scaled_grads = arena.take<float>((size_t)g.m * c_out);
     float *pair_grads = arena.take<float>((size_t)g.t * 4);
+    const int64_t w_count = (int64_t)g.c_in * g.k * c_out / num_mlps;
+    uint16_t *w16 = bf16 ? arena.take<uint16_t>((size_t)w_count) : nullptr;
+    uint16_t *g16 = bf16 ? arena.take<uint16_t>((size_t)g.m * c_out) : nullptr;
     if (BASIS == BASIS_EXPLICIT && want_par) basis_g = d_param_a;    // the basis gradient is itself an output
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv backward: workspace of %zu bytes, need %zu", workspace_bytes,
                   pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 1));
@@ -865,22 +909,35 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
         PCCNN_LAUNCH_CHECK();
         in_grads = scaled_grads;
     }
+    if (bf16 && (rc = pccnn_f32_to_bf16(in_grads, g16, g.m * c_out, s)) != PCCNN_OK) return rc;
     if (want_w) {
         // d_weights = P^T x dOut; P comes from the caller (kept from the forward call) or is rebuilt here
-        const float *proj = proj_in;
+        const void *proj = proj_in;
         if (proj == nullptr) {
-            if ((rc = launch_proj_fwd<BASIS>(g, feats, proj_ws, s)) != PCCNN_OK) return rc;
+            if ((rc = launch_proj_fwd<BASIS>(g, feats, proj_ws, s, bf16)) != PCCNN_OK) return rc;
             proj = proj_ws;
         }
         const int split = (int)(g.m >= 4096 ? CONV_SPLIT_K : 1);
-        rc = pccnn_gemm_f32(proj, in_grads, d_weights, inner, co, g.m, 1, 0, (int64_t)g.c_in * g.k, c_out, co, num_mlps,
-                            inner, co, inner * co, split, splitk, splitk_elems * sizeof(float), s);
+        if (bf16)
+            rc = pccnn_gemm_bf16((const uint16_t *)proj, g16, d_weights, inner, co, g.m, 1, 0, (int64_t)g.c_in * g.k,
+                                 c_out, co, num_mlps, inner, co, inner * co, split, splitk,
+                                 splitk_elems * sizeof(float), s);
+        else
+            rc = pccnn_gemm_f32((const float *)proj, in_grads, d_weights, inner, co, g.m, 1, 0, (int64_t)g.c_in * g.k,
+                                c_out, co, num_mlps, inner, co, inner * co, split, splitk,
+                                splitk_elems * sizeof(float), s);
         if (rc != PCCNN_OK) return rc;
     }
     if (!want_f && !want_basis) return PCCNN_OK;
     // d_proj = dOut x W^T
-    rc = pccnn_gemm_f32(in_grads, weights, d_proj, g.m, inner, co, 0, 1, c_out, co, (int64_t)g.c_in * g.k, num_mlps, co,
-                        inner * co, inner, 1, nullptr, 0, s);
+    if (bf16) {
+        if ((rc = pccnn_f32_to_bf16(weights, w16, w_count, s)) != PCCNN_OK) return rc;
+        rc = pccnn_gemm_bf16(g16, w16, d_proj, g.m, inner, co, 0, 1, c_out, co, (int64_t)g.c_in * g.k, num_mlps, co,
+                             inner * co, inner, 1, nullptr, 0, s);
+    } else {
+        rc = pccnn_gemm_f32(in_grads, weights, d_proj, g.m, inner, co, 0, 1, c_out, co, (int64_t)g.c_in * g.k, num_mlps,
+                            co, inner * co, inner, 1, nullptr, 0, s);
+    }
     if (rc != PCCNN_OK) return rc;
     BasisGradOut o = {basis_g, want_pts ? d_pts : nullptr, want_pts ? d_samples : nullptr, want_pdf ? d_pdf : nullptr,
                       (want_par && Tr::differentiable) ? partials : nullptr, gather ? pair_grads : nullptr};
@@ -1085,45 +1142,67 @@ static int basis_geom(const char *who, const pccnn_basis *b, const float *pts, c
     default: return CALL(BASIS_SPH);                                                     \
     }
 
+static int conv_forward_entry(const char *who, bool bf16, const pccnn_basis *basis, const float *pts, const float *feats,
+                                  const float *samples, const int32_t *neigh, const int32_t *ends, const float *radii,
+                                  const float *weights, int64_t n, int64_t m, int64_t t, int d, int c_in, int num_mlps,
+                                  int c_out, int divide_by_count, float *out, void *proj_out, void *workspace,
+                                  size_t workspace_bytes, void *stream)
+{
+    ConvGeom g;
+    int rc = basis_geom(who, basis, pts, samples, neigh, ends, radii, n, m, t, c_in, g);
+    if (rc != PCCNN_OK) return rc;
+    if ((rc = conv_validate(who, n, m, t, d, c_in, g.k, num_mlps, c_out)) != PCCNN_OK) return rc;
+    const bool geom = basis->kind != PCCNN_BASIS_EXPLICIT;
+    PCCNN_REQUIRE(m == 0 || (feats && ends && weights && out && (t == 0 || neigh) && (!geom || (pts && samples && radii))),
+                  PCCNN_ERR_INVALID, "%s: null pointer", who);
+#define CALL(B) conv_forward<B>(g, feats, weights, num_mlps, c_out, out, proj_out, workspace, workspace_bytes, \
+                                (hipStream_t)stream, divide_by_count != 0, bf16)
+    BASIS_DISPATCH(basis->kind, CALL)
+#undef CALL
+}
+
 extern "C" int pccnn_conv_forward(const pccnn_basis *basis, const float *pts, const float *feats,
                                   const float *samples, const int32_t *neigh, const int32_t *ends, const float *radii,
                                   const float *weights, int64_t n, int64_t m, int64_t t, int d, int c_in, int num_mlps,
                                   int c_out, int divide_by_count, float *out, float *proj_out, void *workspace,
                                   size_t workspace_bytes, void *stream)
 {
-    ConvGeom g;
-    int rc = basis_geom("pccnn_conv_forward", basis, pts, samples, neigh, ends, radii, n, m, t, c_in, g);
-    if (rc != PCCNN_OK) return rc;
-    if ((rc = conv_validate("pccnn_conv_forward", n, m, t, d, c_in, g.k, num_mlps, c_out)) != PCCNN_OK) return rc;
-    const bool geom = basis->kind != PCCNN_BASIS_EXPLICIT;
-    PCCNN_REQUIRE(m == 0 || (feats && ends && weights && out && (t == 0 || neigh) && (!geom || (pts && samples && radii))),
-                  PCCNN_ERR_INVALID, "pccnn_conv_forward: null pointer");
-#define CALL(B) conv_forward<B>(g, feats, weights, num_mlps, c_out, out, proj_out, workspace, workspace_bytes, \
-                                (hipStream_t)stream, divide_by_count != 0)
-    BASIS_DISPATCH(basis->kind, CALL)
-#undef CALL
+    return conv_forward_entry("pccnn_conv_forward", false, basis, pts, feats, samples, neigh, ends, radii, weights, n, m,
+                              t, d, c_in, num_mlps, c_out, divide_by_count, out, proj_out, workspace, workspace_bytes,
+                              stream);
 }
 
-extern "C" int pccnn_conv_backward(const pccnn_basis *basis, const float *pts, const float *feats,
+extern "C" int pccnn_conv_forward_bf16(const pccnn_basis *basis, const float *pts, const float *feats,
+                                       const float *samples, const int32_t *neigh, const int32_t *ends,
+                                       const float *radii, const float *weights, int64_t n, int64_t m, int64_t t, int d,
+                                       int c_in, int num_mlps, int c_out, int divide_by_count, float *out,
+                                       uint16_t *proj_out, void *workspace, size_t workspace_bytes, void *stream)
+{
+    return conv_forward_entry("pccnn_conv_forward_bf16", true, basis, pts, feats, samples, neigh, ends, radii, weights,
+                              n, m, t, d, c_in, num_mlps, c_out, divide_by_count, out, proj_out, workspace,
+                              workspace_bytes, stream);
+}
+
+static int conv_backward_entry(const char *who, bool bf16, const pccnn_basis *basis, const float *pts, const float *feats,
                                    const float *samples, const int32_t *neigh, const int32_t *ends,
-                                   const float *radii, const float *weights, const float *in_grads, const float *proj,
+                                   const float *radii, const float *weights, const float *in_grads, const void *proj,
                                    const int32_t *mirror, int grad_mask, int64_t n, int64_t m, int64_t t, int d, int c_in, int num_mlps,
                                    int c_out, int divide_by_count, float *d_weights, float *d_feats, float *d_param_a,
                                    float *d_param_b, float *d_pdf, float *d_pts, float *d_samples, void *workspace,
                                    size_t workspace_bytes, void *stream)
 {
     ConvGeom g;
-    int rc = basis_geom("pccnn_conv_backward", basis, pts, samples, neigh, ends, radii, n, m, t, c_in, g);
+    int rc = basis_geom(who, basis, pts, samples, neigh, ends, radii, n, m, t, c_in, g);
     if (rc != PCCNN_OK) return rc;
-    if ((rc = conv_validate("pccnn_conv_backward", n, m, t, d, c_in, g.k, num_mlps, c_out)) != PCCNN_OK) return rc;
+    if ((rc = conv_validate(who, n, m, t, d, c_in, g.k, num_mlps, c_out)) != PCCNN_OK) return rc;
     PCCNN_REQUIRE(mirror == nullptr || n == m, PCCNN_ERR_INVALID,
-                  "pccnn_conv_backward: a mirror index needs samples == points (n=%lld, m=%lld)", (long long)n,
+                  "%s: a mirror index needs samples == points (n=%lld, m=%lld)", who, (long long)n,
                   (long long)m);
     const int kind = basis->kind;
     const bool geom = kind != PCCNN_BASIS_EXPLICIT;
     PCCNN_REQUIRE(weights && (n == 0 || feats) && (m == 0 || (ends && in_grads)) && (t == 0 || neigh) &&
                       (!geom || (radii && (n == 0 || pts) && (m == 0 || samples))),
-                  PCCNN_ERR_INVALID, "pccnn_conv_backward: null input pointer");
+                  PCCNN_ERR_INVALID, "%s: null input pointer", who);
     const bool has_param = kind != PCCNN_BASIS_SPH;
     const bool has_pts = kind != PCCNN_BASIS_SPH && kind != PCCNN_BASIS_EXPLICIT;
     const bool has_pdf = kind == PCCNN_BASIS_MLP || kind == PCCNN_BASIS_GAUSS;
@@ -1133,12 +1212,41 @@ extern "C" int pccnn_conv_backward(const pccnn_basis *basis, const float *pts, c
                       (!(grad_mask & PCCNN_GRAD_BASIS_PARAMS) || kind != PCCNN_BASIS_MLP || d_param_b) &&
                       (!(grad_mask & PCCNN_GRAD_PDF) || !has_pdf || d_pdf || n == 0) &&
                       (!(grad_mask & PCCNN_GRAD_PTS) || !has_pts || ((d_pts || n == 0) && (d_samples || m == 0))),
-                  PCCNN_ERR_INVALID, "pccnn_conv_backward: a requested gradient has a null output pointer");
+                  PCCNN_ERR_INVALID, "%s: a requested gradient has a null output pointer", who);
 #define CALL(B) conv_backward<B>(g, feats, weights, in_grads, num_mlps, c_out, proj, grad_mask, d_weights, d_feats, \
                                  d_param_a, d_param_b, d_pdf, d_pts, d_samples, workspace, workspace_bytes,           \
-                                 (hipStream_t)stream, divide_by_count != 0, mirror)
+                                 (hipStream_t)stream, divide_by_count != 0, mirror, bf16)
     BASIS_DISPATCH(kind, CALL)
 #undef CALL
+}
+
+extern "C" int pccnn_conv_backward(const pccnn_basis *basis, const float *pts, const float *feats,
+                                   const float *samples, const int32_t *neigh, const int32_t *ends,
+                                   const float *radii, const float *weights, const float *in_grads, const float *proj,
+                                   const int32_t *mirror, int grad_mask, int64_t n, int64_t m, int64_t t, int d, int c_in,
+                                   int num_mlps, int c_out, int divide_by_count, float *d_weights, float *d_feats,
+                                   float *d_param_a, float *d_param_b, float *d_pdf, float *d_pts, float *d_samples,
+                                   void *workspace, size_t workspace_bytes, void *stream)
+{
+    return conv_backward_entry("pccnn_conv_backward", false, basis, pts, feats, samples, neigh, ends, radii, weights,
+                               in_grads, proj, mirror, grad_mask, n, m, t, d, c_in, num_mlps, c_out, divide_by_count,
+                               d_weights, d_feats, d_param_a, d_param_b, d_pdf, d_pts, d_samples, workspace,
+                               workspace_bytes, stream);
+}
+
+extern "C" int pccnn_conv_backward_bf16(const pccnn_basis *basis, const float *pts, const float *feats,
+                                        const float *samples, const int32_t *neigh, const int32_t *ends,
+                                        const float *radii, const float *weights, const float *in_grads,
+                                        const uint16_t *proj, const int32_t *mirror, int grad_mask, int64_t n,
+                                        int64_t m, int64_t t, int d, int c_in, int num_mlps, int c_out,
+                                        int divide_by_count, float *d_weights, float *d_feats, float *d_param_a,
+                                        float *d_param_b, float *d_pdf, float *d_pts, float *d_samples,
+                                        void *workspace, size_t workspace_bytes, void *stream)
+{
+    return conv_backward_entry("pccnn_conv_backward_bf16", true, basis, pts, feats, samples, neigh, ends, radii,
+                               weights, in_grads, proj, mirror, grad_mask, n, m, t, d, c_in, num_mlps, c_out,
+                               divide_by_count, d_weights, d_feats, d_param_a, d_param_b, d_pdf, d_pts, d_samples,
+                               workspace, workspace_bytes, stream);
 }
 
 extern "C" int pccnn_conv_weight_var(const pccnn_basis *basis, const float *pts, const float *feats,

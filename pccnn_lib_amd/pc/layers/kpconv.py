@@ -46,6 +46,7 @@ class KPConv(IConvLayer):
         super(KPConv, self).__init__(p_dims, p_in_features, p_out_features, p_constant_weight_var,
                                      p_const_var_value)
         self.num_kernel_pts_ = p_num_kernel_pts
+        self.contraction_ = "f32"       # "bf16": bf16 operands, fp32 accumulation in the [M,K*Cin] x [K*Cin,Cout] products
         kernel_pts, sigma = _kernel_point_buffers(p_dims, p_num_kernel_pts, 1.0, 15)
         self.register_buffer('kernel_pts_', kernel_pts)
         self.register_buffer('sigma_', sigma)
@@ -71,7 +72,7 @@ class KPConv(IConvLayer):
         return ComputeKPConv.apply(
             p_pc_in.pts_, p_in_features, p_pc_out.pts_, p_neighborhood.neighbors_, p_neighborhood.start_ids_,
             p_radius, self.kernel_pts_, self.sigma_cpu_, self.conv_weights_,
-            mirror_if_needed(p_neighborhood, p_pc_in.pts_))
+            mirror_if_needed(p_neighborhood, p_pc_in.pts_), self.contraction_)
 
 
 class KPConvFactory(IConvLayerFactory):

@@ -10,7 +10,9 @@ class MCConv(IConvLayer):
     """Monte-Carlo convolution with a one-hidden-layer kernel (pccnn_lib/pc/layers/MCConv.py:11-140).
     Parameters keep the reference's names and shapes: ``proj_axis_`` [D, H*m], ``proj_bias_`` [1, H*m],
     ``conv_weights_`` [m, H*Cin, Cout/m].  The input cloud must carry a density (``compute_pdf``); the op
-    receives it multiplied by the product of the radii (MCConv.py:93-94)."""
+    receives it multiplied by the product of the radii (MCConv.py:93-94).  ``contraction_`` ("f32" by default;
+    "bf16" = bf16 operands with fp32 accumulation, a mode the reference does not have) selects the precision of the
+    [M, H*Cin] x [H*Cin, Cout] products of the forward and backward pass."""
 
     def __init__(self, p_dims, p_in_features, p_out_features, p_hidden_size, p_num_mlps=1,
                  p_constant_weight_var=True, p_const_var_value=1.0):
@@ -18,6 +20,7 @@ class MCConv(IConvLayer):
                                      p_const_var_value)
         self.hidden_size_ = p_hidden_size
         self.num_mlps_ = p_num_mlps
+        self.contraction_ = "f32"
         self.proj_axis_ = torch.nn.Parameter(torch.empty(self.num_dims_, self.hidden_size_ * self.num_mlps_))
         self.proj_bias_ = torch.nn.Parameter(torch.empty(1, self.hidden_size_ * self.num_mlps_))
         self.conv_weights_ = torch.nn.Parameter(
@@ -44,7 +47,7 @@ class MCConv(IConvLayer):
         return ComputeMCConv.apply(
             p_pc_in.pts_, cur_pdf, p_in_features, p_pc_out.pts_, p_neighborhood.neighbors_,
             p_neighborhood.start_ids_, p_radius, self.proj_axis_, self.proj_bias_, self.conv_weights_,
-            mirror_if_needed(p_neighborhood, p_pc_in.pts_, cur_pdf))
+            mirror_if_needed(p_neighborhood, p_pc_in.pts_, cur_pdf), self.contraction_)
 
 
 class MCConvFactory(IConvLayerFactory):

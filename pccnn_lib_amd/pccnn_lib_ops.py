@@ -320,11 +320,15 @@ def _conv_args(name, pts, feats, samples, neigh, ends, radii):
     return d, dev
 
 
-def kp_conv(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights, return_proj=False):
+def kp_conv(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights, return_proj=False,
+            contraction="f32"):
     """kp_conv(pts, feats, samples, neighbors, start_ids, radii, kernel_pts f32[K,D], sigma, weights f32[K*Cin,Cout])
     -> f32[M,Cout] (pccnn_lib_ops/pcconvs/kpconv.cuh:32-41).  ``return_proj=True`` also returns the projection
-    f32[M,Cin,K] the call built, for kp_conv_grads(..., proj=...)."""
+    f32[M,Cin,K] the call built, for kp_conv_grads(..., proj=...).  ``contraction="bf16"`` (no counterpart in the
+    reference) rounds the operands of the [M,K*Cin] x [K*Cin,Cout] product to bf16 and accumulates in fp32; the
+    projection returned is then bf16."""
     name = "kp_conv"
+    bf16 = _contraction(name, contraction)
     d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
     _chk(kernel_pts, name + ": kernel_pts", torch.float32, 2, dev)
     _chk(weights, name + ": weights", torch.float32, 2, dev)
@@ -332,12 +336,42 @@ def kp_conv(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights,
         weights.shape[1]
     if kernel_pts.shape[1] != d or weights.shape[0] != k * c_in:
         raise RuntimeError(name + ": weights must be [K*Cin, Cout] and kernel_pts [K, D]")
+    if bf16:
+        desc = _basis(BASIS_KP, k, a=kernel_pts, sigma=sigma)
+        out, proj = _bf16_forward(name, desc, pts, feats, samples, neigh, ends, radii, weights, k, 1, c_out)
+        return (out, proj) if return_proj else out
     out = torch.empty((m, c_out), dtype=torch.float32, device=dev)
     proj = torch.empty((m, c_in, k), dtype=torch.float32, device=dev)
     _lib.call("pccnn_kpconv_forward", _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends), _ptr(radii),
               _ptr(kernel_pts), float(sigma), _ptr(weights), n, m, t, d, c_in, k, c_out, _ptr(out), _ptr(proj),
               _P(0), 0, _stream())
     return (out, proj) if return_proj else out
+
+
+def _bf16_forward(name, desc, pts, feats, samples, neigh, ends, radii, weights, k, num_mlps, c_out):
+    """Forward call with the contraction operands in bf16; returns (out f32[M,Cout], proj bf16[M,Cin,K])."""
+    dev = feats.device
+    n, m, t, c_in = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1]
+    out = torch.empty((m, c_out), dtype=torch.float32, device=dev)
+    proj = torch.empty((m, c_in, k), dtype=torch.bfloat16, device=dev)
+    ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 0), dev)
+    _lib.call("pccnn_conv_forward_bf16", ctypes.byref(desc), _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh),
+              _ptr(ends), _ptr(radii), _ptr(weights), n, m, t, 3, c_in, num_mlps, c_out, 0, _ptr(out), _ptr(proj),
+              _ptr(ws), ws.numel(), _stream())
+    return out, proj
+
+
+def _bf16_backward(name, desc, pts, feats, samples, neigh, ends, radii, weights, in_grads, proj, mirror, grad_mask,
+                   k, num_mlps, c_out, d_w, d_f, d_a, d_b, d_pdf, d_p, d_s):
+    dev = feats.device
+    n, m, t, c_in = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1]
+    proj_p = _conv_proj_arg(name, proj, m, c_in, k, dev, bf16=True)
+    ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
+    _lib.call("pccnn_conv_backward_bf16", ctypes.byref(desc), _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh),
+              _ptr(ends), _ptr(radii), _ptr(weights), _ptr(in_grads), proj_p,
+              _mirror_arg(name, mirror, neigh, pts, samples), grad_mask, n, m, t, 3, c_in, num_mlps, c_out, 0,
+              _optr(d_w), _optr(d_f), _optr(d_a), _optr(d_b), _optr(d_pdf), _optr(d_p), _optr(d_s), _ptr(ws),
+              ws.numel(), _stream())
 
 
 def _mirror_arg(name, mirror, neigh, pts, samples):
@@ -362,12 +396,13 @@ def mirror_pairs(neigh, ends):
 
 
 def kp_conv_grads(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights, in_grads, proj=None,
-                  grad_mask=GRAD_ALL, mirror=None):
+                  grad_mask=GRAD_ALL, mirror=None, contraction="f32"):
     """kp_conv_grads(..., in_grads f32[M,Cout]) -> [dW, dFeat, dKernelPts, dPts, dSamples]
     (pccnn_lib_ops/pcconvs/kpconv.cuh:56-67).  ``proj``: projection kept from kp_conv(return_proj=True);
     ``grad_mask``: GRAD_* groups to compute, the others come back as None; ``mirror``: result of mirror_pairs()
     for a symmetric neighborhood, which lets dPts (and dPdf) be summed per point without atomics."""
     name = "kp_conv_grads"
+    bf16 = _contraction(name, contraction)
     d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
     _chk(kernel_pts, name + ": kernel_pts", torch.float32, 2, dev)
     _chk(weights, name + ": weights", torch.float32, 2, dev)
@@ -380,6 +415,11 @@ def kp_conv_grads(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, we
     alloc = lambda like, bit: torch.empty_like(like) if grad_mask & bit else None
     d_w, d_f, d_kp = alloc(weights, GRAD_WEIGHTS), alloc(feats, GRAD_FEATS), alloc(kernel_pts, GRAD_BASIS_PARAMS)
     d_p, d_s = alloc(pts, GRAD_PTS), alloc(samples, GRAD_PTS)
+    if bf16:
+        desc = _basis(BASIS_KP, k, a=kernel_pts, sigma=sigma)
+        _bf16_backward(name, desc, pts, feats, samples, neigh, ends, radii, weights, in_grads, proj, mirror, grad_mask,
+                       k, 1, c_out, d_w, d_f, d_kp, None, None, d_p, d_s)
+        return [d_w, d_f, d_kp, d_p, d_s]
     proj_p = _conv_proj_arg(name, proj, m, c_in, k, dev)
     ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
     _lib.call("pccnn_kpconv_backward", _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends), _ptr(radii),
@@ -393,10 +433,19 @@ def _optr(t):
     return _P(t.data_ptr()) if t is not None else _P(0)
 
 
-def _conv_proj_arg(name, proj, m, c_in, k, dev):
+CONTRACTIONS = ("f32", "bf16")
+
+
+def _contraction(name, contraction):
+    if contraction not in CONTRACTIONS:
+        raise RuntimeError("%s: contraction must be one of %s, got %r" % (name, CONTRACTIONS, contraction))
+    return contraction == "bf16"
+
+
+def _conv_proj_arg(name, proj, m, c_in, k, dev, bf16=False):
     if proj is None:
         return _P(0)
-    _chk(proj, name + ": proj", torch.float32, 3, dev)
+    _chk(proj, name + ": proj", torch.bfloat16 if bf16 else torch.float32, 3, dev)
     if tuple(proj.shape) != (m, c_in, k):
         raise RuntimeError(name + ": proj must be [M, Cin, K]")
     return _ptr(proj)
@@ -415,14 +464,21 @@ def _mc_args(name, pts, pdf, axis, bias, weights, c_in, d, dev):
     return k, num_mlps, c_out
 
 
-def mc_conv(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights, return_proj=False):
+def mc_conv(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights, return_proj=False,
+            contraction="f32"):
     """mc_conv(pts, pdf f32[N], feats, samples, neighbors, start_ids, radii, axis f32[D,H*m], bias f32[1,H*m],
     weights f32[m, H*Cin, Cout/m]) -> f32[M,Cout] (pccnn_lib_ops/pcconvs/mcconv.cuh:32-42).
-    ``return_proj=True`` also returns the projection f32[M,Cin,H*m] for mc_conv_grads(..., proj=...)."""
+    ``return_proj=True`` also returns the projection f32[M,Cin,H*m] for mc_conv_grads(..., proj=...);
+    ``contraction`` as in kp_conv."""
     name = "mc_conv"
+    bf16 = _contraction(name, contraction)
     d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
     n, m, t, c_in = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1]
     k, num_mlps, c_out = _mc_args(name, pts, pdf, axis, bias, weights, c_in, d, dev)
+    if bf16:
+        desc = _basis(BASIS_MLP, k, a=axis, b=bias, pdf=pdf)
+        out, proj = _bf16_forward(name, desc, pts, feats, samples, neigh, ends, radii, weights, k, num_mlps, c_out)
+        return (out, proj) if return_proj else out
     out = torch.empty((m, c_out), dtype=torch.float32, device=dev)
     proj = torch.empty((m, c_in, k), dtype=torch.float32, device=dev)
     _lib.call("pccnn_mcconv_forward", _ptr(pts), _ptr(pdf), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends),
@@ -432,10 +488,11 @@ def mc_conv(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights, r
 
 
 def mc_conv_grads(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights, in_grads, proj=None,
-                  grad_mask=GRAD_ALL, mirror=None):
+                  grad_mask=GRAD_ALL, mirror=None, contraction="f32"):
     """mc_conv_grads(..., in_grads f32[M,Cout]) -> [dW, dFeat, dAxis, dBias f32[1,H*m], dPdf f32[N], dPts, dSamples]
     (pccnn_lib_ops/pcconvs/mcconv.cuh:57-69).  ``proj`` / ``grad_mask`` / ``mirror`` as in kp_conv_grads."""
     name = "mc_conv_grads"
+    bf16 = _contraction(name, contraction)
     d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
     n, m, t, c_in = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1]
     k, num_mlps, c_out = _mc_args(name, pts, pdf, axis, bias, weights, c_in, d, dev)
@@ -447,6 +504,11 @@ def mc_conv_grads(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weig
     d_w, d_f = alloc(weights, GRAD_WEIGHTS), alloc(feats, GRAD_FEATS)
     d_axis, d_bias, d_pdf = alloc(axis, GRAD_BASIS_PARAMS), alloc(bias, GRAD_BASIS_PARAMS), alloc(pdf, GRAD_PDF)
     d_p, d_s = alloc(pts, GRAD_PTS), alloc(samples, GRAD_PTS)
+    if bf16:
+        desc = _basis(BASIS_MLP, k, a=axis, b=bias, pdf=pdf)
+        _bf16_backward(name, desc, pts, feats, samples, neigh, ends, radii, weights, in_grads, proj, mirror, grad_mask,
+                       k, num_mlps, c_out, d_w, d_f, d_axis, d_bias, d_pdf, d_p, d_s)
+        return [d_w, d_f, d_axis, d_bias, d_pdf, d_p, d_s]
     proj_p = _conv_proj_arg(name, proj, m, c_in, k, dev)
     ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
     _lib.call("pccnn_mcconv_backward", _ptr(pts), _ptr(pdf), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends),
