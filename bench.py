@@ -33,6 +33,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 MFMA_FP32_PEAK_TFLOPS = 157.3     # MI355X dense fp32 matrix peak
+MFMA_BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 matrix peak
 HBM_PEAK_GBPS = 8000.0            # MI355X HBM3E peak
 
 # Bytes per launch that the dominant kernels move past the L2, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
@@ -173,6 +174,12 @@ def main():
         out = ComputeMCConv.apply(pts, pdf, f, pts, neigh, ends, radii, axis, bias, w)
         return torch.autograd.grad(out, [f, w], out_grads)
 
+    def conv_step_bf16():
+        # the same step with the three contractions on the bf16 matrix pipe (bf16 operands, fp32 accumulation)
+        p, q, f, a, b, w = leaves
+        out = ComputeMCConv.apply(p, q, f, p, neigh, ends, radii, a, b, w, mirror, "bf16")
+        return torch.autograd.grad(out, leaves, out_grads)
+
     def pc_fresh():
         p = lib.pc.Pointcloud.__new__(lib.pc.Pointcloud)         # same tensors, no cached grid
         p.__dict__.update(pc.__dict__)
@@ -208,11 +215,14 @@ def main():
 
     conv_ms, conv_kernels = timed(conv_step, args.steps, args.warmup)
     fw_ms, _ = timed(conv_step_fw_only, args.steps, args.warmup)
+    bf_ms, bf_kernels = timed(conv_step_bf16, args.steps, args.warmup)
     nb_ms, nb_kernels = timed(neighbor_step, args.steps, args.warmup)
     pdf_ms, pdf_kernels = timed(pdf_step, args.steps, args.warmup)
     log("conv fwd+bwd %.3f ms (features+weights grads only: %.3f ms) | neighborhood %.3f ms | density %.3f ms"
         % (conv_ms, fw_ms, nb_ms, pdf_ms))
-    for name, ks in (("conv", conv_kernels), ("neighbors", nb_kernels), ("pdf", pdf_kernels)):
+    log("conv fwd+bwd with bf16 contraction operands: %.3f ms" % bf_ms)
+    for name, ks in (("conv", conv_kernels), ("conv bf16", bf_kernels), ("neighbors", nb_kernels),
+                     ("pdf", pdf_kernels)):
         log(name, {k: "%d x %.1f us" % (v[0], 1e3 * v[1] / v[0]) for k, v in ks.items()})
 
     # ---- roofline of the dominant kernel: the contraction (three launches per step, equal flops)
@@ -225,6 +235,17 @@ def main():
                 "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": gemm_tflops / MFMA_FP32_PEAK_TFLOPS,
                 "traffic": TRAFFIC_GEMM_BYTES, "flops_per_launch": gemm_flops, "avg_launch_ms": gemm_avg_ms,
                 "launches": gemm_n}
+
+    # the same three launches on the bf16 pipe (reported beside the fp32 figures; `value` is the fp32 step)
+    bf_n, bf_total_ms = bf_kernels.get("gemm", (0, 0.0))
+    bf_avg_ms = bf_total_ms / max(bf_n, 1)
+    bf_tflops = gemm_flops / (bf_avg_ms * 1e-3) / 1e12 if bf_n else 0.0
+    bf16_leg = {"ms_per_step": bf_ms, "points_per_sec": m / (bf_ms * 1e-3), "dtype": "bf16 operands, f32 accumulate",
+                "kernels_us": {k: round(1e3 * v[1] / v[0], 2) for k, v in bf_kernels.items()},
+                "roofline": {"kernel": "gemm_bf16_mfma_kernel", "bound": "mfma", "achieved": bf_tflops,
+                             "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                             "frac": bf_tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                             "flops_per_launch": gemm_flops, "avg_launch_ms": bf_avg_ms, "launches": bf_n}}
 
     # ---- neighbor fill kernel against HBM: 8T out + 24M (sample xyz, key, order, offsets) + 20N (point xyz, key)
     grid_bytes = 8 * wl["batch"] * int(np.prod(nbh.grid_.num_cells_host()[0:2]))
@@ -290,7 +311,7 @@ def main():
         "density_ms": pdf_ms,
         "kernels_us": {leg: {k: round(1e3 * v[1] / v[0], 2) for k, v in ks.items()}
                        for leg, ks in (("conv", conv_kernels), ("neighborhood", nb_kernels), ("density", pdf_kernels))},
-        "scene": scene, "roofline": roofline, "roofline_neighbors": roofline_nb, "cpu_baseline": cpu,
+        "bf16_contraction": bf16_leg, "scene": scene, "roofline": roofline, "roofline_neighbors": roofline_nb, "cpu_baseline": cpu,
     }
     print(json.dumps(result), flush=True)
     return 0
