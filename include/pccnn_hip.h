@@ -90,7 +90,10 @@ int pccnn_build_grid_ds(const int64_t *sorted_keys, int64_t n, const int32_t *nu
  * points' grid; grid_ds i32[num_pillars,2] from pccnn_build_grid_ds; radii f32[d] (device).
  * sample_order i32[m] (nullable): a permutation that lists the samples in
  * ascending key order -- tiles of consecutive entries then share their cell
- * walk; NULL means natural order.  max_neighbors 0 = unlimited; otherwise a
+ * walk; NULL means natural order.  samples_presorted != 0 (only with a sample_order): the arrays `samples`
+ * and `sample_keys` are already listed in that order (entry i belongs to sample sample_order[i]), as
+ * pccnn_sort_keys leaves them, so the kernels read them as contiguous runs instead of gathering.
+ * max_neighbors 0 = unlimited; otherwise a
  * sample with more hits keeps max_neighbors of them, evenly spaced in its hit
  * order (the reference keeps a time-seeded random subset there).
  * point_remap i32[n] (nullable): when given, column 0 of neigh_out is
@@ -109,14 +112,16 @@ int pccnn_build_cell_table(const int64_t *sorted_keys, int64_t n, int64_t total_
                            void *stream);
 int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t *pt_keys_sorted, int64_t n,
                                const float *samples, const int64_t *sample_keys, int64_t m,
-                               const int32_t *sample_order, const int32_t *grid_ds, int64_t num_pillars,
+                               const int32_t *sample_order, int samples_presorted,
+                               const int32_t *grid_ds, int64_t num_pillars,
                                const int32_t *cell_table, int64_t total_cells,
                                const int32_t *num_cells, const float *radii, int d, int max_neighbors,
                                int32_t *ends_out,
                                void *workspace, size_t workspace_bytes, void *stream);
 int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t *pt_keys_sorted, int64_t n,
                               const float *samples, const int64_t *sample_keys, int64_t m,
-                              const int32_t *sample_order, const int32_t *grid_ds, int64_t num_pillars,
+                              const int32_t *sample_order, int samples_presorted,
+                              const int32_t *grid_ds, int64_t num_pillars,
                               const int32_t *cell_table, int64_t total_cells,
                               const int32_t *num_cells, const float *radii, int d, int max_neighbors,
                               const int32_t *ends,

@@ -153,6 +153,10 @@ __device__ __forceinline__ void gemm_tile_loop(const GemmArgs &g, const float *_
                     tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k0, k_end, rb);
                 }
             }
+            // keep the order written above in the instruction stream: the fragment reads of the next sub-step go
+            // out before this sub-step's MFMAs, so their LDS latency is covered by the matrix pipe
+            if (ks + 1 < GT_K / 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 2 * TN, 0);
         }
         __syncthreads();
     }

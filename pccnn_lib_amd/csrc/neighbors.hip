@@ -28,6 +28,7 @@ struct NbArgs {
     const int64_t *sample_keys;
     int64_t m;
     const int32_t *order;      // nullable
+    int presorted;             // samples / sample_keys are listed in `order` order already
     const int32_t *grid_ds;    // [num_pillars,2]
     int64_t num_pillars;
     const int32_t *cell_table; // nullable: [total_cells + 1] first sorted index of every cell
@@ -125,10 +126,13 @@ neighbors_kernel(NbArgs a)
     float sx = 0.f, sy = 0.f, sz = 0.f;
     if (valid) {
         s = a.order ? a.order[base + lane] : (int)(base + lane);
-        key = a.sample_keys[s];
-        sx = a.samples[(int64_t)s * 3 + 0];
-        sy = a.samples[(int64_t)s * 3 + 1];
-        sz = a.samples[(int64_t)s * 3 + 2];
+        // entry of this sample in the sample arrays: its place in the walk order when the caller lists them
+        // that way (coalesced reads), else its index (a gather)
+        const int64_t at = a.presorted ? base + lane : (int64_t)s;
+        key = a.sample_keys[at];
+        sx = a.samples[at * 3 + 0];
+        sy = a.samples[at * 3 + 1];
+        sz = a.samples[at * 3 + 2];
     }
     const int nc0 = a.num_cells[0], nc1 = a.num_cells[1], nc2 = a.num_cells[2];
     const float ir0 = __fdiv_rn(1.0f, a.radii[0]);
@@ -345,10 +349,11 @@ static int nb_validate(const char *who, const float *pts_sorted, const int64_t *
 
 extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t *pt_keys_sorted, int64_t n,
                                           const float *samples, const int64_t *sample_keys, int64_t m,
-                                          const int32_t *sample_order, const int32_t *grid_ds,
-                                          int64_t num_pillars, const int32_t *cell_table, int64_t total_cells,
-                                          const int32_t *num_cells, const float *radii, int d, int max_neighbors,
-                                          int32_t *ends_out, void *workspace, size_t workspace_bytes, void *stream)
+                                          const int32_t *sample_order, int samples_presorted,
+                                          const int32_t *grid_ds, int64_t num_pillars, const int32_t *cell_table,
+                                          int64_t total_cells, const int32_t *num_cells, const float *radii, int d,
+                                          int max_neighbors, int32_t *ends_out, void *workspace,
+                                          size_t workspace_bytes, void *stream)
 {
     int rc = nb_validate("pccnn_find_neighbors_count", pts_sorted, pt_keys_sorted, n, samples, sample_keys, m, grid_ds,
                          num_pillars, cell_table, total_cells, num_cells, radii, d, max_neighbors, workspace,
@@ -364,7 +369,8 @@ extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t
     NbArgs a;
     a.pts = pts_sorted; a.pt_keys = pt_keys_sorted; a.n = n;
     a.samples = samples; a.sample_keys = sample_keys; a.m = m;
-    a.order = sample_order; a.grid_ds = grid_ds; a.num_pillars = num_pillars;
+    a.order = sample_order; a.presorted = (sample_order != nullptr && samples_presorted != 0);
+    a.grid_ds = grid_ds; a.num_pillars = num_pillars;
     a.cell_table = cell_table; a.total_cells = total_cells;
     a.num_cells = num_cells; a.radii = radii; a.max_neighbors = max_neighbors;
     a.counts = counts; a.ends = nullptr; a.remap = nullptr; a.t = 0; a.neigh = nullptr; a.rec = nullptr;
@@ -380,10 +386,10 @@ extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t
 
 extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t *pt_keys_sorted, int64_t n,
                                          const float *samples, const int64_t *sample_keys, int64_t m,
-                                         const int32_t *sample_order, const int32_t *grid_ds,
-                                         int64_t num_pillars, const int32_t *cell_table, int64_t total_cells,
-                                          const int32_t *num_cells, const float *radii, int d, int max_neighbors,
-                                         const int32_t *ends, const int32_t *point_remap, int64_t t,
+                                         const int32_t *sample_order, int samples_presorted,
+                                         const int32_t *grid_ds, int64_t num_pillars, const int32_t *cell_table,
+                                         int64_t total_cells, const int32_t *num_cells, const float *radii, int d,
+                                         int max_neighbors, const int32_t *ends, const int32_t *point_remap, int64_t t,
                                          int32_t *neigh_out, void *workspace, size_t workspace_bytes, void *stream)
 {
     int rc = nb_validate("pccnn_find_neighbors_fill", pts_sorted, pt_keys_sorted, n, samples, sample_keys, m, grid_ds,
@@ -401,7 +407,8 @@ extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t 
     NbArgs a;
     a.pts = pts_sorted; a.pt_keys = pt_keys_sorted; a.n = n;
     a.samples = samples; a.sample_keys = sample_keys; a.m = m;
-    a.order = sample_order; a.grid_ds = grid_ds; a.num_pillars = num_pillars;
+    a.order = sample_order; a.presorted = (sample_order != nullptr && samples_presorted != 0);
+    a.grid_ds = grid_ds; a.num_pillars = num_pillars;
     a.cell_table = cell_table; a.total_cells = total_cells;
     a.num_cells = num_cells; a.radii = radii; a.max_neighbors = max_neighbors;
     a.counts = counts; a.ends = ends; a.remap = point_remap; a.t = t; a.neigh = neigh_out; a.rec = rec;

@@ -20,17 +20,18 @@ class Neighborhood(object):
         grid = p_grid
         with torch.no_grad():
             sample_pts = p_samples.pts_.detach()
+            # the samples go to the search in key order (a wavefront's 64 samples then share their cell walk and
+            # read their coordinates as one run): the gridded cloud itself is sorted already
             if p_samples is grid.pointcloud_:
-                sample_keys = grid.cell_ids_
-                order = grid.sorted_ids_i32_
+                sorted_keys, order, sorted_pts = grid.sorted_cell_ids_, grid.sorted_ids_i32_, grid.sorted_pts_
             else:
                 sample_keys = ComputeKeys.apply(sample_pts, p_samples.batch_ids_, grid.bounding_box_.min_,
                                                 grid.num_cells_, grid.cell_size_)
-                _, order, _ = pccnn_lib_ops.sort_keys(sample_keys, grid.key_bits())
+                sorted_keys, order, sorted_pts = pccnn_lib_ops.sort_keys(sample_keys, grid.key_bits(), sample_pts)
             self.neighbors_, self.start_ids_ = pccnn_lib_ops.find_neighbors_ex(
-                grid.sorted_pts_, grid.sorted_cell_ids_, sample_pts, sample_keys, grid.grid_ds_, grid.num_cells_,
+                grid.sorted_pts_, grid.sorted_cell_ids_, sorted_pts, sorted_keys, grid.grid_ds_, grid.num_cells_,
                 grid.cell_size_, p_max_neighbors, sample_order=order, point_remap=grid.sorted_ids_i32_,
-                cell_table=grid.cell_table_)
+                cell_table=grid.cell_table_, samples_presorted=True)
 
     def mirror(self):
         """int32 [T]: for every pair (a, b) the index of pair (b, a), when the samples are the gridded cloud

@@ -58,9 +58,9 @@ class Pointcloud(object):
             # neighbor coordinates from the sorted copy of the points, where they are contiguous
             with torch.no_grad():
                 neigh_sorted, ends = pccnn_lib_ops.find_neighbors_ex(
-                    grid.sorted_pts_, grid.sorted_cell_ids_, self.pts_, grid.cell_ids_, grid.grid_ds_,
+                    grid.sorted_pts_, grid.sorted_cell_ids_, grid.sorted_pts_, grid.sorted_cell_ids_, grid.grid_ds_,
                     grid.num_cells_, grid.cell_size_, 300, sample_order=grid.sorted_ids_i32_,
-                    cell_table=grid.cell_table_)
+                    cell_table=grid.cell_table_, samples_presorted=True)
                 self.pts_unnorm_pdf_ = pccnn_lib_ops.compute_pdf_sorted(
                     self.dim_manifold_, bandwidth, grid.sorted_pts_, self.pts_, neigh_sorted, ends)
         num_pts = torch.index_select(self.get_num_points_per_batch(), 0, self.batch_ids_.to(torch.int64))

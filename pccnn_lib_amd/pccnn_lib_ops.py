@@ -150,10 +150,12 @@ def build_cell_table(sorted_keys, total_cells):
 
 
 def find_neighbors_ex(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, radii, max_neighbors,
-                      sample_order=None, point_remap=None, cell_table=None):
+                      sample_order=None, point_remap=None, cell_table=None, samples_presorted=False):
     """find_neighbors with the native extras: ``sample_order`` (i32[M], samples listed in key order),
-    ``point_remap`` (i32[N], written through to column 0 of the result) and ``cell_table`` (from
-    build_cell_table: replaces the per-pillar binary searches by two table reads)."""
+    ``point_remap`` (i32[N], written through to column 0 of the result), ``cell_table`` (from
+    build_cell_table: replaces the per-pillar binary searches by two table reads) and ``samples_presorted``
+    (``samples`` / ``sample_keys`` are given in ``sample_order`` order, as sort_keys returns them; the result
+    still refers to the samples by their own indices ``sample_order[i]``)."""
     name = "find_neighbors"
     _chk(pts, name + ": pts", torch.float32, 2)
     dev = pts.device
@@ -189,13 +191,14 @@ def find_neighbors_ex(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, ra
         return [torch.empty((0, 2), dtype=torch.int32, device=dev), ends]
     ws = _workspace(_lib.load().pccnn_find_neighbors_workspace_bytes(n, m), dev)
     order_p = _ptr(sample_order) if sample_order is not None else _P(0)
+    presorted = 1 if (samples_presorted and sample_order is not None) else 0
     _lib.call("pccnn_find_neighbors_count", _ptr(pts), _ptr(pt_keys), n, _ptr(samples), _ptr(sample_keys), m, order_p,
-              _ptr(grid_ds), pillars, table_p, total_cells, _ptr(grid_size), _ptr(radii), d, max_neighbors, _ptr(ends),
+              presorted, _ptr(grid_ds), pillars, table_p, total_cells, _ptr(grid_size), _ptr(radii), d, max_neighbors, _ptr(ends),
               _ptr(ws), ws.numel(), _stream())
     total = int(ends[-1].item())                      # the one host read-back, as in the reference
     neigh = torch.empty((total, 2), dtype=torch.int32, device=dev)
     _lib.call("pccnn_find_neighbors_fill", _ptr(pts), _ptr(pt_keys), n, _ptr(samples), _ptr(sample_keys), m, order_p,
-              _ptr(grid_ds), pillars, table_p, total_cells, _ptr(grid_size), _ptr(radii), d, max_neighbors, _ptr(ends),
+              presorted, _ptr(grid_ds), pillars, table_p, total_cells, _ptr(grid_size), _ptr(radii), d, max_neighbors, _ptr(ends),
               _ptr(point_remap) if point_remap is not None else _P(0), total, _ptr(neigh), _ptr(ws), ws.numel(),
               _stream())
     return [neigh, ends]
@@ -212,10 +215,12 @@ def find_neighbors(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, radii
         # queries are walked in cell order so that a wavefront's 64 queries share their cell walk
         cells = grid_size.tolist()
         bits = key_bits_for(cells, grid_ds.shape[0])
-        _, order, _ = sort_keys(sample_keys, bits)
+        skeys, order, spts = sort_keys(sample_keys, bits, samples)
         total = grid_ds.shape[0] * cells[0] * cells[1] * cells[2]
         if total <= CELL_TABLE_MAX_CELLS:
             table = build_cell_table(pt_keys, total)
+        return find_neighbors_ex(pts, pt_keys, spts, skeys, grid_ds, grid_size, radii, max_neighbors, order,
+                                 cell_table=table, samples_presorted=True)
     return find_neighbors_ex(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, radii, max_neighbors, order,
                              cell_table=table)
 

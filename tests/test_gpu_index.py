@@ -83,6 +83,25 @@ def test_capped_neighbors(ops, oracle, models, cap):
     assert np.array_equal(got["neigh_sorted"], exp["neigh_sorted"])
 
 
+def test_presorted_samples_give_the_same_lists(ops):
+    # samples handed over in key order (as sort_keys leaves them) against the same samples gathered through
+    # sample_order: identical pair lists, for samples that are the points and for a distinct sample set, capped or not
+    pts, ids = synthetic.primitives(31, 3, 2000)
+    rng = np.random.default_rng(31)
+    pick = np.sort(rng.choice(pts.shape[0], 1500, replace=False))
+    for smp, sids in ((pts, ids), (pts[pick] + np.float32(0.003), ids[pick])):
+        for cap in (0, 7):
+            g = gpu_neighborhood(ops, pts, ids, smp, sids, 0.08, 3, max_neighbors=cap)
+            d = g["dev"]
+            ts, tsi = t(smp), t(sids)
+            skey = ops.compute_keys(ts, tsi, t(g["aabb_min"]), d["nc"], d["radii"])
+            bits = ops.key_bits_for(d["nc"].tolist(), 3)
+            sk, order, sp = ops.sort_keys(skey, bits, ts)
+            neigh, ends = ops.find_neighbors_ex(d["spts"], d["skeys"], sp, sk, d["ds"], d["nc"], d["radii"], cap, order,
+                                                d["perm"], samples_presorted=True)
+            assert np.array_equal(neigh.cpu().numpy(), g["neighbors"]) and np.array_equal(ends.cpu().numpy(), g["ends"])
+
+
 def test_degenerate_inputs(ops, oracle):
     # all points in one cell; a single point; duplicate points
     pts = np.tile(np.array([[0.5, 0.5, 0.5]], np.float32), (130, 1))
