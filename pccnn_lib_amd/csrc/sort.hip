@@ -9,20 +9,27 @@
 #include "common.h"
 
 #define RS_THREADS 256
-#define RS_ITEMS 8
-#define RS_TILE (RS_THREADS * RS_ITEMS)
+#define RS_MAX_ITEMS 8                                  // keys per thread and tile, at most
 #define RS_WAVES (RS_THREADS / PCCNN_WAVE)
 
+// Keys per thread of a tile: small inputs get small tiles, so that the launch still has a few hundred
+// workgroups (a tile is walked in `items` rounds with barriers in between: few large tiles leave the chip
+// idle), large inputs get the largest tiles (every tile pays a fixed set-up and a row of the histogram table).
+static int rs_items_for(int64_t n)
+{
+    int64_t items = pccnn_ceil_div(n, (int64_t)RS_THREADS * 512);
+    return (int)(items < 1 ? 1 : (items > RS_MAX_ITEMS ? RS_MAX_ITEMS : items));
+}
+
 __global__ void __launch_bounds__(RS_THREADS)
-radix_hist_kernel(const int64_t *__restrict__ keys, int64_t n, int shift, int32_t *__restrict__ tile_hist,
+radix_hist_kernel(const int64_t *__restrict__ keys, int64_t n, int shift, int items, int32_t *__restrict__ tile_hist,
                   int64_t num_tiles)
 {
     __shared__ int hist[256];
     hist[threadIdx.x] = 0;
     __syncthreads();
-    int64_t base = (int64_t)blockIdx.x * RS_TILE;
-#pragma unroll
-    for (int r = 0; r < RS_ITEMS; ++r) {
+    int64_t base = (int64_t)blockIdx.x * RS_THREADS * items;
+    for (int r = 0; r < items; ++r) {
         int64_t i = base + r * RS_THREADS + threadIdx.x;
         if (i < n) atomicAdd(&hist[(int)((keys[i] >> shift) & 0xff)], 1);
     }
@@ -67,7 +74,7 @@ radix_scan_kernel(int32_t *__restrict__ tile_hist, int64_t num_tiles, int32_t *_
 template <bool FIRST, bool GATHER>
 __global__ void __launch_bounds__(RS_THREADS)
 radix_scatter_kernel(const int64_t *__restrict__ keys_in, const int32_t *__restrict__ vals_in, int64_t n, int shift,
-                     const int32_t *__restrict__ tile_offsets, int64_t num_tiles,
+                     int items, const int32_t *__restrict__ tile_offsets, int64_t num_tiles,
                      const int32_t *__restrict__ digit_totals, int64_t *__restrict__ keys_out, int32_t *__restrict__ vals_out,
                      const float *__restrict__ pts, float *__restrict__ pts_out)
 {
@@ -96,9 +103,9 @@ radix_scatter_kernel(const int64_t *__restrict__ keys_in, const int32_t *__restr
 #pragma unroll
     for (int w = 0; w < RS_WAVES; ++w) wave_cnt[w][threadIdx.x] = 0;
     __syncthreads();
-    int64_t base = (int64_t)blockIdx.x * RS_TILE;
+    int64_t base = (int64_t)blockIdx.x * RS_THREADS * items;
     unsigned long long lt = pccnn_lanemask_lt();
-    for (int r = 0; r < RS_ITEMS; ++r) {
+    for (int r = 0; r < items; ++r) {
         int64_t i = base + r * RS_THREADS + threadIdx.x;
         bool valid = i < n;
         long long key = valid ? keys_in[i] : 0;
@@ -141,7 +148,7 @@ radix_scatter_kernel(const int64_t *__restrict__ keys_in, const int32_t *__restr
 extern "C" size_t pccnn_sort_keys_workspace_bytes(int64_t n)
 {
     if (n < 0) n = 0;
-    int64_t tiles = pccnn_ceil_div(n > 0 ? n : 1, RS_TILE);
+    int64_t tiles = pccnn_ceil_div(n > 0 ? n : 1, (int64_t)RS_THREADS * rs_items_for(n));
     return pccnn_align((size_t)n * sizeof(int64_t)) + pccnn_align((size_t)n * sizeof(int32_t)) +
            pccnn_align((size_t)tiles * 256 * sizeof(int32_t)) + pccnn_align(256 * sizeof(int32_t)) + 256;
 }
@@ -163,7 +170,8 @@ extern "C" int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int
     hipStream_t s = (hipStream_t)stream;
     if (key_bits <= 0 || key_bits > 63) key_bits = 63;     // keys are non-negative
     int passes = (key_bits + 7) / 8;
-    int64_t tiles = pccnn_ceil_div(n, RS_TILE);
+    const int items = rs_items_for(n);
+    int64_t tiles = pccnn_ceil_div(n, (int64_t)RS_THREADS * items);
     PccnnArena arena(workspace, workspace_bytes);
     int64_t *tmp_keys = arena.take<int64_t>((size_t)n);
     int32_t *tmp_vals = arena.take<int32_t>((size_t)n);
@@ -180,7 +188,7 @@ extern "C" int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int
         int32_t *dst_v = to_out ? perm_out : tmp_vals;
         int shift = 8 * p;
         bool last = (p == passes - 1);
-        radix_hist_kernel<<<(unsigned)tiles, RS_THREADS, 0, s>>>(src_k, n, shift, hist, tiles);
+        radix_hist_kernel<<<(unsigned)tiles, RS_THREADS, 0, s>>>(src_k, n, shift, items, hist, tiles);
         PCCNN_LAUNCH_CHECK();
         radix_scan_kernel<<<256, 256, 0, s>>>(hist, tiles, totals);
         PCCNN_LAUNCH_CHECK();
@@ -188,17 +196,17 @@ extern "C" int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int
         if (p == 0) {
             if (gather)
                 radix_scatter_kernel<true, true><<<(unsigned)tiles, RS_THREADS, 0, s>>>(
-                    src_k, src_v, n, shift, hist, tiles, totals, dst_k, dst_v, pts, sorted_pts_out);
+                    src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, pts, sorted_pts_out);
             else
                 radix_scatter_kernel<true, false><<<(unsigned)tiles, RS_THREADS, 0, s>>>(
-                    src_k, src_v, n, shift, hist, tiles, totals, dst_k, dst_v, nullptr, nullptr);
+                    src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, nullptr, nullptr);
         } else {
             if (gather)
                 radix_scatter_kernel<false, true><<<(unsigned)tiles, RS_THREADS, 0, s>>>(
-                    src_k, src_v, n, shift, hist, tiles, totals, dst_k, dst_v, pts, sorted_pts_out);
+                    src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, pts, sorted_pts_out);
             else
                 radix_scatter_kernel<false, false><<<(unsigned)tiles, RS_THREADS, 0, s>>>(
-                    src_k, src_v, n, shift, hist, tiles, totals, dst_k, dst_v, nullptr, nullptr);
+                    src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, nullptr, nullptr);
         }
         PCCNN_LAUNCH_CHECK();
         src_k = dst_k;

@@ -7,7 +7,7 @@ class BoundingBox(object):
 
     def __init__(self, p_point_cloud):
         self.min_, self.max_ = pccnn_lib_ops.bounding_box(
-            p_point_cloud.pts_.detach(), p_point_cloud.batch_ids_, int(p_point_cloud.batch_size_))
+            p_point_cloud.pts_.detach(), p_point_cloud.batch_ids_, p_point_cloud.batch_size_host())
 
     def __repr__(self):
         return "### Min:\n{}\n### Max:\n{}".format(self.min_, self.max_)

@@ -25,12 +25,19 @@ class Grid(object):
             self.num_cells_ = torch.max(num_cells.to(torch.int32) + 1, dim=0)[0].contiguous()
         self.num_cells_host_ = None
         self.cell_ids_ = None
-        self.sorted_ids_ = None
+        self.sorted_ids_i64_ = None
         self.sorted_ids_i32_ = None
         self.sorted_cell_ids_ = None
         self.sorted_pts_ = None
         self.grid_ds_ = None
         self.cell_table_ = None
+
+    @property
+    def sorted_ids_(self):
+        """int64 [N] permutation, as the reference keeps it; converted from the native int32 one on first use."""
+        if self.sorted_ids_i64_ is None and self.sorted_ids_i32_ is not None:
+            self.sorted_ids_i64_ = self.sorted_ids_i32_.to(torch.int64)
+        return self.sorted_ids_i64_
 
     def num_cells_host(self):
         if self.num_cells_host_ is None:
@@ -38,7 +45,7 @@ class Grid(object):
         return self.num_cells_host_
 
     def key_bits(self):
-        return pccnn_lib_ops.key_bits_for(self.num_cells_host(), int(self.pointcloud_.batch_size_))
+        return pccnn_lib_ops.key_bits_for(self.num_cells_host(), self.pointcloud_.batch_size_host())
 
     def compute_cell_ids(self):
         if self.cell_ids_ is None:
@@ -48,18 +55,17 @@ class Grid(object):
                                                    self.num_cells_, self.cell_size_)
                 self.sorted_cell_ids_, self.sorted_ids_i32_, self.sorted_pts_ = pccnn_lib_ops.sort_keys(
                     self.cell_ids_, self.key_bits(), pts)
-                self.sorted_ids_ = self.sorted_ids_i32_.to(torch.int64)
 
     def build_ds(self):
-        if self.cell_ids_ is None or self.sorted_ids_ is None:
+        if self.cell_ids_ is None or self.sorted_ids_i32_ is None:
             raise RuntimeError('In order to build the data structure first the keys for each point has to be '
                                'computed.')
         if self.grid_ds_ is None:
             with torch.no_grad():
-                shape = [int(self.pointcloud_.batch_size_)] + self.num_cells_host()[0:2] + [2]
+                shape = [self.pointcloud_.batch_size_host()] + self.num_cells_host()[0:2] + [2]
                 self.grid_ds_ = pccnn_lib_ops.build_grid_ds(self.sorted_cell_ids_, self.num_cells_, shape)
                 cells = self.num_cells_host()
-                total = int(self.pointcloud_.batch_size_) * cells[0] * cells[1] * cells[2]
+                total = self.pointcloud_.batch_size_host() * cells[0] * cells[1] * cells[2]
                 if total <= pccnn_lib_ops.CELL_TABLE_MAX_CELLS:
                     # per-cell start offsets: the search then needs no binary search inside a pillar
                     self.cell_table_ = pccnn_lib_ops.build_cell_table(self.sorted_cell_ids_, total)

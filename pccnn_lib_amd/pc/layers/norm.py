@@ -36,7 +36,7 @@ class GroupNormalization(torch.nn.Module):
         group_size = self.num_features_ // self.num_groups_
         cur_feats = p_feats.reshape((-1, self.num_groups_))
         ids = p_pc.batch_ids_.reshape((-1, 1)).repeat(1, group_size).to(torch.int64).reshape((-1,))
-        num_batches = int(p_pc.batch_size_)
+        num_batches = p_pc.batch_size_host()
         means = _mean_per_batch(cur_feats, ids, num_batches)[ids]
         variances = _mean_per_batch((cur_feats - means) ** 2, ids, num_batches)[ids]
         cur_feats = (cur_feats - means) / torch.sqrt(variances + eps_val)

@@ -18,6 +18,8 @@ class Pointcloud(object):
         self.pts_ = torch.as_tensor(p_pts, **kwargs)
         self.batch_ids_ = torch.as_tensor(p_batch_ids, **kwargs)
         self.batch_size_ = torch.max(self.batch_ids_) + 1
+        self.batch_size_host_ = None            # int(batch_size_), read back once
+        self.num_pts_per_batch_ = None          # cached result of get_num_points_per_batch()
         if self.pts_with_grads_:
             self.pts_.requires_grad = True
         self.pts_pdf_ = None
@@ -31,9 +33,18 @@ class Pointcloud(object):
             self.pts_unnorm_pdf_ = self.pts_unnorm_pdf_.to(p_device)
             self.pts_pdf_ = self.pts_pdf_.to(p_device)
 
+    def batch_size_host(self):
+        """``batch_size_`` as a Python int (one read-back per cloud; the batch ids of a cloud do not change)."""
+        if self.batch_size_host_ is None:
+            self.batch_size_host_ = int(self.batch_size_)
+        return self.batch_size_host_
+
     def get_num_points_per_batch(self):
-        with torch.no_grad():
-            return torch.bincount(self.batch_ids_.to(torch.int64), minlength=int(self.batch_size_)).to(torch.int32)
+        if self.num_pts_per_batch_ is None or self.num_pts_per_batch_.device != self.batch_ids_.device:
+            with torch.no_grad():
+                self.num_pts_per_batch_ = torch.bincount(self.batch_ids_.to(torch.int64),
+                                                         minlength=self.batch_size_host()).to(torch.int32)
+        return self.num_pts_per_batch_
 
     def compute_pdf(self, p_badnwidth):
         """Kernel density estimate per point (Pointcloud.py:81-109): neighbors within 4 bandwidths, at most 300
@@ -69,7 +80,7 @@ class Pointcloud(object):
     def global_pooling(self, p_in_tensor, p_pooling_method="avg"):
         """Per-cloud reduction of a per-point tensor (Pointcloud.py:113-131)."""
         index = self.batch_ids_.to(torch.int64).reshape(-1, 1).expand(-1, p_in_tensor.shape[1])
-        out = torch.zeros((int(self.batch_size_), p_in_tensor.shape[1]), dtype=p_in_tensor.dtype,
+        out = torch.zeros((self.batch_size_host(), p_in_tensor.shape[1]), dtype=p_in_tensor.dtype,
                           device=p_in_tensor.device)
         reduce = {"max": "amax", "min": "amin", "avg": "mean", "sum": "sum"}[p_pooling_method]
         return out.scatter_reduce(0, index, p_in_tensor, reduce=reduce, include_self=False)
