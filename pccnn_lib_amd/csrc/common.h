@@ -7,6 +7,20 @@
 #include "../../include/pccnn_hip.h"
 
 #define PCCNN_WAVE 64
+#define PCCNN_MAX_DIMS 6                                // point dimensions handled: 2 .. 6, as the reference's tests use
+
+// KERNEL<D> LAUNCH for the run-time dimension d (2 .. 6), e.g.
+//   PCCNN_DIM_DISPATCH(d, my_kernel, <<<grid, block, 0, stream>>>(args));
+#define PCCNN_DIM_DISPATCH(d, KERNEL, ...)                                               \
+    do {                                                                                 \
+        switch (d) {                                                                     \
+        case 2: KERNEL<2> __VA_ARGS__; break;                                              \
+        case 3: KERNEL<3> __VA_ARGS__; break;                                              \
+        case 4: KERNEL<4> __VA_ARGS__; break;                                              \
+        case 5: KERNEL<5> __VA_ARGS__; break;                                              \
+        default: KERNEL<6> __VA_ARGS__; break;                                             \
+        }                                                                                \
+    } while (0)
 
 void pccnn_set_error(const char *fmt, ...);
 

@@ -121,7 +121,8 @@ __global__ void bbox_pad_kernel(float *mn, float *mx, int count)
 extern "C" int pccnn_bounding_box(const float *pts, const int32_t *batch_ids, int64_t n, int d, int batch_size,
                                   float *aabb_min_out, float *aabb_max_out, void *stream)
 {
-    PCCNN_REQUIRE(d == 3, PCCNN_ERR_UNSUPPORTED, "pccnn_bounding_box: d=%d is not supported (d must be 3)", d);
+    PCCNN_REQUIRE(d >= 2 && d <= PCCNN_MAX_DIMS, PCCNN_ERR_UNSUPPORTED,
+                  "pccnn_bounding_box: d=%d is not supported (2 <= d <= 6)", d);
     PCCNN_REQUIRE(n >= 0 && batch_size > 0, PCCNN_ERR_INVALID, "pccnn_bounding_box: n=%lld batch_size=%d",
                   (long long)n, batch_size);
     PCCNN_REQUIRE(aabb_min_out && aabb_max_out && (n == 0 || (pts && batch_ids)), PCCNN_ERR_INVALID,
@@ -133,8 +134,8 @@ extern "C" int pccnn_bounding_box(const float *pts, const int32_t *batch_ids, in
     if (n > 0) {
         int64_t blocks = pccnn_ceil_div(n, 256 * 8);
         if (blocks > 256) blocks = 256;
-        bbox_reduce_kernel<3><<<(unsigned)blocks, 256, 0, s>>>(pts, batch_ids, n, batch_size, aabb_min_out,
-                                                               aabb_max_out);
+        PCCNN_DIM_DISPATCH(d, bbox_reduce_kernel, <<<(unsigned)blocks, 256, 0, s>>>(pts, batch_ids, n, batch_size,
+                                                                                    aabb_min_out, aabb_max_out));
         PCCNN_LAUNCH_CHECK();
     }
     bbox_pad_kernel<<<(unsigned)pccnn_ceil_div(count, 256), 256, 0, s>>>(aabb_min_out, aabb_max_out, count);
@@ -173,14 +174,15 @@ extern "C" int pccnn_compute_keys(const float *pts, const int32_t *batch_ids, co
                                   const int32_t *num_cells, const float *cell_size, int64_t n, int d,
                                   int64_t *keys_out, void *stream)
 {
-    PCCNN_REQUIRE(d == 3, PCCNN_ERR_UNSUPPORTED, "pccnn_compute_keys: d=%d is not supported (d must be 3)", d);
+    PCCNN_REQUIRE(d >= 2 && d <= PCCNN_MAX_DIMS, PCCNN_ERR_UNSUPPORTED,
+                  "pccnn_compute_keys: d=%d is not supported (2 <= d <= 6)", d);
     PCCNN_REQUIRE(n >= 0, PCCNN_ERR_INVALID, "pccnn_compute_keys: n=%lld", (long long)n);
     if (n == 0) return PCCNN_OK;
     PCCNN_REQUIRE(pts && batch_ids && aabb_min && num_cells && cell_size && keys_out, PCCNN_ERR_INVALID,
                   "pccnn_compute_keys: null pointer");
     PccnnTimed timed(PCCNN_T_KEYS, (hipStream_t)stream);
-    compute_keys_kernel<3><<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, (hipStream_t)stream>>>(
-        pts, batch_ids, aabb_min, num_cells, cell_size, n, (int64_t *)keys_out);
+    PCCNN_DIM_DISPATCH(d, compute_keys_kernel, <<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, (hipStream_t)stream>>>(
+        pts, batch_ids, aabb_min, num_cells, cell_size, n, (int64_t *)keys_out));
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
 }
@@ -208,7 +210,8 @@ build_grid_kernel(const int64_t *__restrict__ keys, int64_t n, const int32_t *__
 extern "C" int pccnn_build_grid_ds(const int64_t *sorted_keys, int64_t n, const int32_t *num_cells, int d,
                                    int64_t num_pillars, int32_t *grid_ds_out, void *stream)
 {
-    PCCNN_REQUIRE(d == 3, PCCNN_ERR_UNSUPPORTED, "pccnn_build_grid_ds: d=%d is not supported (d must be 3)", d);
+    PCCNN_REQUIRE(d >= 2 && d <= PCCNN_MAX_DIMS, PCCNN_ERR_UNSUPPORTED,
+                  "pccnn_build_grid_ds: d=%d is not supported (2 <= d <= 6)", d);
     PCCNN_REQUIRE(n >= 0 && num_pillars > 0 && num_pillars < (1ll << 30), PCCNN_ERR_INVALID,
                   "pccnn_build_grid_ds: n=%lld num_pillars=%lld", (long long)n, (long long)num_pillars);
     PCCNN_REQUIRE(grid_ds_out && num_cells && (n == 0 || sorted_keys), PCCNN_ERR_INVALID,
@@ -218,8 +221,8 @@ extern "C" int pccnn_build_grid_ds(const int64_t *sorted_keys, int64_t n, const 
     int rc = pccnn_fill_i32(grid_ds_out, 0, num_pillars * 2, s);
     if (rc != PCCNN_OK) return rc;
     if (n == 0) return PCCNN_OK;
-    build_grid_kernel<3><<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(sorted_keys, n, num_cells, num_pillars,
-                                                                        grid_ds_out);
+    PCCNN_DIM_DISPATCH(d, build_grid_kernel, <<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(sorted_keys, n, num_cells,
+                                                                                          num_pillars, grid_ds_out));
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
 }

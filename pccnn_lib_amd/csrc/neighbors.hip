@@ -272,6 +272,126 @@ neighbors_kernel(NbArgs a)
     }
 }
 
+// Any other dimension (2, 4, 5, 6): the walk of the reference, restated per lane without the shortcuts that
+// three dimensions allow.  Offsets run over {-1, 0, 1} in every dimension but the last (in both when D == 2), in
+// the reference's order (find_ranges_grid_ds.cu:306-338); an offset cell selects its pillar (batch, c0, c1) in the
+// pillar table, and inside it the run of keys in [key - 1, key + 1] clamped to the batch
+// (find_ranges_grid_ds.cu:65-165; for D == 2 the whole pillar, :203-236).  One sample per lane, ranges walked one
+// after the other, hits stored one pair at a time.
+template <bool FILL, bool CAPPED, int D>
+__global__ void __launch_bounds__(NB_THREADS)
+neighbors_generic_kernel(NbArgs a)
+{
+    const int lane = pccnn_lane();
+    const int64_t wave = ((int64_t)blockIdx.x * NB_THREADS + threadIdx.x) >> 6;
+    const int64_t base = wave * 64;
+    if (base >= a.m) return;                                   // wave-uniform
+    if (base + lane >= a.m) return;
+    const int s = a.order ? a.order[base + lane] : (int)(base + lane);
+    const int64_t at = a.presorted ? base + lane : (int64_t)s;
+    const long long key0 = a.sample_keys[at];
+    float sp[D], ir[D];
+    int nc[D];
+    long long total_cells = 1;
+#pragma unroll
+    for (int i = 0; i < D; ++i) {
+        sp[i] = a.samples[at * D + i];
+        ir[i] = __fdiv_rn(1.0f, a.radii[i]);
+        nc[i] = a.num_cells[i];
+        total_cells *= nc[i];
+    }
+    int cell0[D];
+    long long aux = key0 < 0 ? 0 : key0;
+#pragma unroll
+    for (int i = D - 1; i >= 0; --i) { cell0[i] = (int)(aux % nc[i]); aux /= nc[i]; }
+    const long long batch = aux;
+    constexpr int TOP = (D - 2 > 1) ? D - 2 : 1;                 // offsets vary in dimensions 0 .. TOP
+    int n_off = 3;
+#pragma unroll
+    for (int i = 0; i < TOP; ++i) n_off *= 3;
+    constexpr int CHK = (D == 2) ? D : D - 1;                    // dimensions whose bounds are checked
+
+    unsigned int my_off = 0;
+    int raw = 0, take_step = 0, cnt = 0, err = 0;
+    if (FILL) {
+        my_off = s > 0 ? (unsigned int)a.ends[s - 1] : 0u;
+        if (CAPPED) {
+            raw = a.counts[s];
+            take_step = raw < a.max_neighbors ? raw : a.max_neighbors;
+        }
+    }
+    const unsigned int out_limit = FILL ? (unsigned int)a.t : 0u;
+
+    for (int o = 0; o < n_off && key0 >= 0; ++o) {
+        int cell[D];
+        int rem = o;
+        bool inside = true;
+#pragma unroll
+        for (int i = D - 1; i >= 0; --i) {
+            int off = 0;
+            if (i <= TOP) { off = rem % 3 - 1; rem /= 3; }
+            if (D != 2 && i == D - 1) off = 0;
+            cell[i] = cell0[i] + off;
+            if (i < CHK) inside = inside && cell[i] >= 0 && cell[i] < nc[i];
+        }
+        if (!inside) continue;
+        const long long pillar = (batch * nc[0] + cell[0]) * nc[1] + cell[1];
+        if (pillar < 0 || pillar >= a.num_pillars) continue;
+        int lo = a.grid_ds[2 * pillar], hi = a.grid_ds[2 * pillar + 1];
+        lo = lo < 0 ? 0 : lo;
+        hi = hi > a.n ? (int)a.n : hi;
+        if (hi <= lo) continue;
+        int first = lo, last = hi;
+        if (D != 2) {
+            long long key = 0, accum = 1;
+#pragma unroll
+            for (int i = D - 1; i >= 0; --i) { key += (long long)cell[i] * accum; accum *= nc[i]; }
+            key += accum * batch;
+            long long max_key = key + 1, min_key = key - 1;
+            if (key / total_cells != max_key / total_cells) max_key = (key / total_cells) * total_cells + total_cells - 1;
+            if (key / total_cells != min_key / total_cells) min_key = (key / total_cells) * total_cells;
+            int lb = lo, ub = hi;
+            while (lb < ub) {
+                const int mid = lb + ((ub - lb) >> 1);
+                if (a.pt_keys[mid] < min_key) lb = mid + 1; else ub = mid;
+            }
+            first = lb;
+            lb = lo; ub = hi;
+            while (lb < ub) {
+                const int mid = lb + ((ub - lb) >> 1);
+                if (a.pt_keys[mid] <= max_key) lb = mid + 1; else ub = mid;
+            }
+            last = lb;
+        }
+        for (int j = first; j < last; ++j) {
+            // fp32, no contraction: ((s - p) * (1/r)) squared, summed over the dimensions in order from 0
+            float acc = 0.0f;
+#pragma unroll
+            for (int i = 0; i < D; ++i) {
+                const float v = (sp[i] - a.pts[(int64_t)j * D + i]) * ir[i];
+                acc = acc + v * v;
+            }
+            if (acc < 1.0f) {
+                if (FILL) {
+                    bool take = true;
+                    if (CAPPED) {
+                        err += take_step;
+                        take = err >= raw;
+                        if (take) err -= raw;
+                    }
+                    if (take) {
+                        if (my_off < out_limit)
+                            ((int2 *)a.neigh)[my_off] = make_int2(a.remap ? a.remap[j] : j, s);
+                        ++my_off;
+                    }
+                }
+                ++cnt;
+            }
+        }
+    }
+    if (!FILL) a.counts[s] = cnt;
+}
+
 // table[c] = index of the first sorted point whose key is >= c, for c in [0, total_cells].  The lane of
 // every point that starts a new key owns the entries between the previous key and its own (lane n owns
 // the tail); the 64 lanes of a wavefront then fill each other's gaps together, so a long run of empty
@@ -331,7 +451,7 @@ static int nb_validate(const char *who, const float *pts_sorted, const int64_t *
                        int64_t num_pillars, const int32_t *cell_table, int64_t total_cells, const int32_t *num_cells, const float *radii, int d, int max_neighbors, void *workspace,
                        size_t workspace_bytes)
 {
-    PCCNN_REQUIRE(d == 3, PCCNN_ERR_UNSUPPORTED, "%s: d=%d is not supported (d must be 3)", who, d);
+    PCCNN_REQUIRE(d >= 2 && d <= PCCNN_MAX_DIMS, PCCNN_ERR_UNSUPPORTED, "%s: d=%d is not supported (2 <= d <= 6)", who, d);
     PCCNN_REQUIRE(n >= 0 && m >= 0 && n < (1ll << 31) && m < (1ll << 31), PCCNN_ERR_INVALID, "%s: n=%lld m=%lld",
                   who, (long long)n, (long long)m);
     PCCNN_REQUIRE(max_neighbors >= 0, PCCNN_ERR_INVALID, "%s: max_neighbors=%d", who, max_neighbors);
@@ -377,7 +497,14 @@ extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t
     int64_t waves = pccnn_ceil_div(m, 64);
     {
         PccnnTimed timed(PCCNN_T_NB_COUNT, s);
-        neighbors_kernel<false, false, NB_UNROLL_COUNT><<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
+        const unsigned blocks = (unsigned)pccnn_ceil_div(waves, NB_THREADS / 64);
+        switch (d) {
+        case 3: neighbors_kernel<false, false, NB_UNROLL_COUNT><<<blocks, NB_THREADS, 0, s>>>(a); break;
+        case 2: neighbors_generic_kernel<false, false, 2><<<blocks, NB_THREADS, 0, s>>>(a); break;
+        case 4: neighbors_generic_kernel<false, false, 4><<<blocks, NB_THREADS, 0, s>>>(a); break;
+        case 5: neighbors_generic_kernel<false, false, 5><<<blocks, NB_THREADS, 0, s>>>(a); break;
+        default: neighbors_generic_kernel<false, false, 6><<<blocks, NB_THREADS, 0, s>>>(a); break;
+        }
     }
     PCCNN_LAUNCH_CHECK();
     PccnnTimed timed(PCCNN_T_SCAN, s);
@@ -415,13 +542,25 @@ extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t 
     int64_t waves = pccnn_ceil_div(m, 64);
     {
         PccnnTimed timed(PCCNN_T_NB_FILL, s);
-        if (n > 0) pack_points_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(pts_sorted, point_remap, n, rec);
-        if (max_neighbors > 0)
-            neighbors_kernel<true, true, NB_UNROLL_FILL>
-                <<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
-        else
-            neighbors_kernel<true, false, NB_UNROLL_FILL>
-                <<<(unsigned)pccnn_ceil_div(waves, NB_THREADS / 64), NB_THREADS, 0, s>>>(a);
+        const unsigned blocks = (unsigned)pccnn_ceil_div(waves, NB_THREADS / 64);
+        if (d == 3) {
+            if (n > 0) pack_points_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(pts_sorted, point_remap, n, rec);
+            if (max_neighbors > 0) neighbors_kernel<true, true, NB_UNROLL_FILL><<<blocks, NB_THREADS, 0, s>>>(a);
+            else neighbors_kernel<true, false, NB_UNROLL_FILL><<<blocks, NB_THREADS, 0, s>>>(a);
+        } else {
+#define NB_GENERIC(D)                                                                            \
+    do {                                                                                         \
+        if (max_neighbors > 0) neighbors_generic_kernel<true, true, D><<<blocks, NB_THREADS, 0, s>>>(a); \
+        else neighbors_generic_kernel<true, false, D><<<blocks, NB_THREADS, 0, s>>>(a);           \
+    } while (0)
+            switch (d) {
+            case 2: NB_GENERIC(2); break;
+            case 4: NB_GENERIC(4); break;
+            case 5: NB_GENERIC(5); break;
+            default: NB_GENERIC(6); break;
+            }
+#undef NB_GENERIC
+        }
     }
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;

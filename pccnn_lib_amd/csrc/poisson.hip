@@ -52,7 +52,8 @@ extern "C" int pccnn_poisson_disk_select(const int64_t *sorted_keys, int64_t n, 
                                          int32_t *selected_out, int32_t *selected_scan_out, void *workspace,
                                          size_t workspace_bytes, void *stream)
 {
-    PCCNN_REQUIRE(d == 3, PCCNN_ERR_UNSUPPORTED, "pccnn_poisson_disk_select: d=%d is not supported (d must be 3)", d);
+    PCCNN_REQUIRE(d >= 2 && d <= PCCNN_MAX_DIMS, PCCNN_ERR_UNSUPPORTED,
+                  "pccnn_poisson_disk_select: d=%d is not supported (2 <= d <= 6)", d);
     PCCNN_REQUIRE(n >= 0 && t >= 0 && n < (1ll << 31), PCCNN_ERR_INVALID, "pccnn_poisson_disk_select: n=%lld t=%lld",
                   (long long)n, (long long)t);
     if (n == 0) return PCCNN_OK;
@@ -64,9 +65,9 @@ extern "C" int pccnn_poisson_disk_select(const int64_t *sorted_keys, int64_t n, 
     hipStream_t s = (hipStream_t)stream;
     int rc = pccnn_fill_i32(selected_out, 0, n, s);
     if (rc != PCCNN_OK) return rc;
-    for (int colour = 0; colour < 8; ++colour) {
-        poisson_pass_kernel<3><<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(
-            sorted_keys, n, (const int2 *)neigh, ends, num_cells, colour, selected_out);
+    for (int colour = 0; colour < (1 << d); ++colour) {
+        PCCNN_DIM_DISPATCH(d, poisson_pass_kernel, <<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(
+            sorted_keys, n, (const int2 *)neigh, ends, num_cells, colour, selected_out));
         PCCNN_LAUNCH_CHECK();
     }
     return pccnn_scan_inclusive_i32(selected_out, selected_scan_out, n, 0, (int32_t *)workspace, s);

@@ -76,7 +76,7 @@ __global__ void __launch_bounds__(RS_THREADS)
 radix_scatter_kernel(const int64_t *__restrict__ keys_in, const int32_t *__restrict__ vals_in, int64_t n, int shift,
                      int items, const int32_t *__restrict__ tile_offsets, int64_t num_tiles,
                      const int32_t *__restrict__ digit_totals, int64_t *__restrict__ keys_out, int32_t *__restrict__ vals_out,
-                     const float *__restrict__ pts, float *__restrict__ pts_out)
+                     const float *__restrict__ pts, float *__restrict__ pts_out, int dims)
 {
     __shared__ int running[256];                       // next free output slot per digit
     __shared__ int wave_cnt[RS_WAVES][256];
@@ -130,7 +130,8 @@ radix_scatter_kernel(const int64_t *__restrict__ keys_in, const int32_t *__restr
             vals_out[dst] = val;
             if (GATHER) {
 #pragma unroll
-                for (int k = 0; k < 3; ++k) pts_out[(int64_t)dst * 3 + k] = pts[(int64_t)val * 3 + k];
+                for (int k = 0; k < PCCNN_MAX_DIMS; ++k)
+                    if (k < dims) pts_out[(int64_t)dst * dims + k] = pts[(int64_t)val * dims + k];
             }
         }
         __syncthreads();
@@ -160,8 +161,8 @@ extern "C" int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int
     PCCNN_REQUIRE(n >= 0 && n < (1ll << 31), PCCNN_ERR_INVALID, "pccnn_sort_keys: n=%lld", (long long)n);
     PCCNN_REQUIRE((pts == nullptr) == (sorted_pts_out == nullptr), PCCNN_ERR_INVALID,
                   "pccnn_sort_keys: pts and sorted_pts_out must be given together");
-    PCCNN_REQUIRE(pts == nullptr || d == 3, PCCNN_ERR_UNSUPPORTED,
-                  "pccnn_sort_keys: d=%d is not supported (d must be 3)", d);
+    PCCNN_REQUIRE(pts == nullptr || (d >= 2 && d <= PCCNN_MAX_DIMS), PCCNN_ERR_UNSUPPORTED,
+                  "pccnn_sort_keys: d=%d is not supported (2 <= d <= 6)", d);
     if (n == 0) return PCCNN_OK;
     PCCNN_REQUIRE(keys && sorted_keys_out && perm_out, PCCNN_ERR_INVALID, "pccnn_sort_keys: null pointer");
     PCCNN_REQUIRE(workspace_bytes >= pccnn_sort_keys_workspace_bytes(n), PCCNN_ERR_WORKSPACE,
@@ -196,17 +197,17 @@ extern "C" int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int
         if (p == 0) {
             if (gather)
                 radix_scatter_kernel<true, true><<<(unsigned)tiles, RS_THREADS, 0, s>>>(
-                    src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, pts, sorted_pts_out);
+                    src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, pts, sorted_pts_out, d);
             else
                 radix_scatter_kernel<true, false><<<(unsigned)tiles, RS_THREADS, 0, s>>>(
-                    src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, nullptr, nullptr);
+                    src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, nullptr, nullptr, d);
         } else {
             if (gather)
                 radix_scatter_kernel<false, true><<<(unsigned)tiles, RS_THREADS, 0, s>>>(
-                    src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, pts, sorted_pts_out);
+                    src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, pts, sorted_pts_out, d);
             else
                 radix_scatter_kernel<false, false><<<(unsigned)tiles, RS_THREADS, 0, s>>>(
-                    src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, nullptr, nullptr);
+                    src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, nullptr, nullptr, d);
         }
         PCCNN_LAUNCH_CHECK();
         src_k = dst_k;

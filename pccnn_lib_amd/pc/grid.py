@@ -65,8 +65,10 @@ class Grid(object):
                 shape = [self.pointcloud_.batch_size_host()] + self.num_cells_host()[0:2] + [2]
                 self.grid_ds_ = pccnn_lib_ops.build_grid_ds(self.sorted_cell_ids_, self.num_cells_, shape)
                 cells = self.num_cells_host()
-                total = self.pointcloud_.batch_size_host() * cells[0] * cells[1] * cells[2]
-                if total <= pccnn_lib_ops.CELL_TABLE_MAX_CELLS:
+                total = self.pointcloud_.batch_size_host()
+                for c in cells:
+                    total *= c
+                if len(cells) == 3 and total <= pccnn_lib_ops.CELL_TABLE_MAX_CELLS:
                     # per-cell start offsets: the search then needs no binary search inside a pillar
                     self.cell_table_ = pccnn_lib_ops.build_cell_table(self.sorted_cell_ids_, total)
 

@@ -49,10 +49,14 @@ def _workspace(nbytes, device):
     return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
 
 
+MIN_DIMS, MAX_DIMS = 2, 6
+
+
 def _dims(pts, name):
     d = pts.shape[1]
-    if d != 3:
-        raise RuntimeError("%s: %d-dimensional points are not supported (only 3)" % (name, d))
+    if d < MIN_DIMS or d > MAX_DIMS:
+        raise RuntimeError("%s: %d-dimensional points are not supported (%d to %d dimensions)"
+                           % (name, d, MIN_DIMS, MAX_DIMS))
     return d
 
 
@@ -118,12 +122,14 @@ def build_grid_ds(keys, grid_size, out_shape):
     _chk(keys, "build_grid_ds: keys", torch.int64, 1)
     _chk(grid_size, "build_grid_ds: grid_size", torch.int32, 1, keys.device)
     out_shape = [int(v) for v in out_shape]
-    if grid_size.shape[0] != 3:
-        raise RuntimeError("build_grid_ds: only 3-dimensional grids are supported")
+    d = grid_size.shape[0]
+    if d < MIN_DIMS or d > MAX_DIMS:
+        raise RuntimeError("build_grid_ds: %d-dimensional grids are not supported (%d to %d dimensions)"
+                           % (d, MIN_DIMS, MAX_DIMS))
     if len(out_shape) != 4 or out_shape[3] != 2 or min(out_shape) < 1:
         raise RuntimeError("build_grid_ds: out_shape must be [batch, cells0, cells1, 2], got %s" % (out_shape,))
     ds = torch.empty(out_shape, dtype=torch.int32, device=keys.device)
-    _lib.call("pccnn_build_grid_ds", _ptr(keys), keys.shape[0], _ptr(grid_size), 3,
+    _lib.call("pccnn_build_grid_ds", _ptr(keys), keys.shape[0], _ptr(grid_size), d,
               out_shape[0] * out_shape[1] * out_shape[2], _ptr(ds), _stream())
     return ds
 
@@ -288,7 +294,8 @@ def poisson_disk_sampling(sorted_keys, neigh, ends, grid_size):
     _chk(ends, name + ": start_ids", torch.int32, 1, dev)
     _chk(grid_size, name + ": grid_size", torch.int32, 1, dev)
     n = sorted_keys.shape[0]
-    if ends.shape[0] != n or grid_size.shape[0] != 3 or neigh.shape[1] != 2:
+    d = grid_size.shape[0]
+    if ends.shape[0] != n or d < MIN_DIMS or d > MAX_DIMS or neigh.shape[1] != 2:
         raise RuntimeError(name + ": inconsistent shapes")
     if n == 0:
         return torch.empty((0, 1), dtype=torch.int64, device=dev)
@@ -296,7 +303,7 @@ def poisson_disk_sampling(sorted_keys, neigh, ends, grid_size):
     scan = torch.empty_like(sel)
     ws = _workspace(_lib.load().pccnn_poisson_disk_workspace_bytes(n), dev)
     _lib.call("pccnn_poisson_disk_select", _ptr(sorted_keys), n, _ptr(neigh), neigh.shape[0], _ptr(ends),
-              _ptr(grid_size), 3, _ptr(sel), _ptr(scan), _ptr(ws), ws.numel(), _stream())
+              _ptr(grid_size), d, _ptr(sel), _ptr(scan), _ptr(ws), ws.numel(), _stream())
     count = int(scan[-1].item())
     ids = torch.empty((count, 1), dtype=torch.int64, device=dev)
     _lib.call("pccnn_compact_selected", _ptr(sel), _ptr(scan), n, _ptr(ids), _stream())
@@ -310,6 +317,13 @@ GRAD_WEIGHTS, GRAD_FEATS, GRAD_BASIS_PARAMS, GRAD_PDF, GRAD_PTS, GRAD_ALL = 1, 2
 
 
 
+def _conv_dims(pts, name):
+    d = pts.shape[1]
+    if d != 3:
+        raise RuntimeError("%s: %d-dimensional points are not supported by the convolutions (only 3)" % (name, d))
+    return d
+
+
 def _conv_args(name, pts, feats, samples, neigh, ends, radii):
     _chk(pts, name + ": pts", torch.float32, 2)
     dev = pts.device
@@ -318,7 +332,7 @@ def _conv_args(name, pts, feats, samples, neigh, ends, radii):
     _chk(neigh, name + ": neighbors", torch.int32, 2, dev)
     _chk(ends, name + ": start_ids", torch.int32, 1, dev)
     _chk(radii, name + ": radii", torch.float32, 1, dev)
-    d = _dims(pts, name)
+    d = _conv_dims(pts, name)
     if feats.shape[0] != pts.shape[0] or samples.shape[1] != d or ends.shape[0] != samples.shape[0] \
             or neigh.shape[1] != 2 or radii.shape[0] != d:
         raise RuntimeError(name + ": inconsistent shapes")
@@ -733,7 +747,7 @@ def sph_conv_weight_var(pts, feats, samples, neigh, ends, radii, radial_bins, az
 def _linear_basis_args(name, pts, radii, samples, neigh, axis, bias):
     _chk(pts, name + ": pts", torch.float32, 2)
     dev = pts.device
-    d = _dims(pts, name)
+    d = _conv_dims(pts, name)
     _chk(samples, name + ": samples", torch.float32, 2, dev)
     _chk(neigh, name + ": neighbors", torch.int32, 2, dev)
     _chk(radii, name + ": radii", torch.float32, 1, dev)

@@ -17,7 +17,8 @@ def gpu_neighborhood(ops, pts, ids, samples, sample_ids, radius, batch_size, max
     oracle.neighborhood()."""
     tp, ti = t(pts), t(ids)
     ts, tsi = t(samples), t(sample_ids)
-    radii = torch.full((3,), float(radius), dtype=torch.float32, device=DEV) if np.isscalar(radius) else t(radius)
+    radii = torch.full((pts.shape[1],), float(radius), dtype=torch.float32, device=DEV) if np.isscalar(radius) \
+        else t(radius)
     mn, mx = ops.bounding_box(tp, ti, batch_size)
     nc = torch.max(((mx - mn) / radii).to(torch.int32) + 1, dim=0)[0].contiguous()
     keys = ops.compute_keys(tp, ti, mn, nc, radii)

@@ -47,8 +47,11 @@ def test_argument_validation_needs_no_gpu(lib_path):
     from pccnn_lib_amd import _lib
     lib = _lib.load()
     assert lib.pccnn_version() == 1
+    for bad in (1, 7):
+        rc = lib.pccnn_compute_keys(None, None, None, None, None, 10, bad, None, None)
+        assert rc == -2 and b"d=%d" % bad in lib.pccnn_last_error()
     rc = lib.pccnn_compute_keys(None, None, None, None, None, 10, 2, None, None)
-    assert rc == -2 and b"d=2" in lib.pccnn_last_error()
+    assert rc == -1 and b"null" in lib.pccnn_last_error()
     rc = lib.pccnn_compute_keys(None, None, None, None, None, 10, 3, None, None)
     assert rc == -1 and b"null" in lib.pccnn_last_error()
     assert lib.pccnn_compute_keys(None, None, None, None, None, 0, 3, None, None) == 0

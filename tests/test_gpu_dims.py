@@ -1,0 +1,134 @@
+"""The path in 2, 4, 5 and 6 dimensions (the reference's own tests run in 2, 3, 4 and 6: unit_test/utest_*.ini).
+Index results bit-exact against the oracle, which follows the reference's D-dimensional walk (offsets over all
+dimensions but the last, key interval [k - 1, k + 1] inside the pillar of the first two); densities 1e-5, their
+gradients 1e-4."""
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_helpers import DEV, gpu_neighborhood, relerr, t
+
+pytestmark = pytest.mark.gpu
+
+# (dimensions, clouds, points per cloud, radius): sparse in high dimensions, so the radius grows with D
+CASES = [(2, 4, 1500, 0.05), (2, 2, 300, 0.3), (4, 3, 1200, 0.25), (5, 2, 1000, 0.4), (6, 2, 900, 0.5),
+         (6, 1, 200, 1.0)]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from pccnn_lib_amd import pccnn_lib_ops
+    return pccnn_lib_ops
+
+
+def _cloud(dims, batch, num_pts, seed):
+    rng = np.random.default_rng(seed)
+    pts = rng.uniform(0.0, 1.0, (batch * num_pts, dims)).astype(np.float32)
+    # squeeze every second cloud along the last axis so that boxes and grids differ between clouds
+    ids = np.repeat(np.arange(batch, dtype=np.int32), num_pts)
+    pts[ids % 2 == 1, -1] *= np.float32(0.5)
+    return pts, ids
+
+
+def _check_index(oracle, got, exp):
+    for name in ("aabb_min", "aabb_max", "num_cells", "keys", "perm", "sorted_keys", "sorted_pts", "grid_ds",
+                 "sample_keys", "ends"):
+        assert np.array_equal(np.asarray(got[name]), np.asarray(exp[name])), name
+    assert np.array_equal(oracle.canonical_pairs(got["neighbors"]), oracle.canonical_pairs(exp["neighbors"]))
+    assert np.array_equal(oracle.canonical_pairs(got["neigh_sorted"]), oracle.canonical_pairs(exp["neigh_sorted"]))
+
+
+@pytest.mark.parametrize("dims,batch,num_pts,radius", CASES)
+def test_neighborhood_bit_exact(ops, oracle, dims, batch, num_pts, radius):
+    pts, ids = _cloud(dims, batch, num_pts, 100 + dims)
+    exp = oracle.neighborhood(pts, ids, pts, ids, radius)
+    for use_order in (True, False):
+        got = gpu_neighborhood(ops, pts, ids, pts, ids, radius, batch, use_order=use_order)
+        _check_index(oracle, got, exp)
+    # Brute force: the walk loses no pair.  Beyond three dimensions the reference takes the last dimension as the key
+    # interval [k - 1, k + 1] inside a pillar that also spans dimensions 2 .. D-2, so at the first / last cell of the
+    # last dimension the interval reaches into the neighbouring row of the pillar (find_ranges_grid_ds.cu:100-105).
+    # With three or more cells along the last dimension that row is too far away to hold a neighbor; with two it is a
+    # true neighbor cell that another offset visits as well, and the reference lists such pairs twice.  Oracle and
+    # HIP path reproduce that; the set of distinct pairs is the brute-force set in every case.
+    bf, bf_ends = oracle.brute_force_neighbors(pts, ids, pts, ids, np.full(dims, radius, np.float32))
+    canon = oracle.canonical_pairs(exp["neighbors"])
+    keep = np.ones(canon.shape[0], bool)
+    keep[1:] = np.any(canon[1:] != canon[:-1], axis=1)
+    assert np.array_equal(canon[keep], oracle.canonical_pairs(bf))
+    if dims <= 3 or int(exp["num_cells"][-1]) >= 3:
+        assert np.array_equal(exp["ends"], bf_ends)
+
+
+@pytest.mark.parametrize("dims,batch,num_pts,radius", [(2, 3, 800, 0.1), (4, 2, 900, 0.3), (6, 2, 700, 0.6)])
+def test_distinct_samples_and_cap(ops, oracle, dims, batch, num_pts, radius):
+    pts, ids = _cloud(dims, batch, num_pts, 200 + dims)
+    rng = np.random.default_rng(dims)
+    pick = np.sort(rng.choice(pts.shape[0], pts.shape[0] // 3, replace=False))
+    smp, sids = (pts[pick] + np.float32(0.004)).astype(np.float32), ids[pick]
+    for cap in (0, 5):
+        exp = oracle.neighborhood(pts, ids, smp, sids, radius, max_neighbors=cap)
+        got = gpu_neighborhood(ops, pts, ids, smp, sids, radius, batch, max_neighbors=cap)
+        assert np.array_equal(got["ends"], exp["ends"])
+        # the capped subset depends on the walk order, so the lists must agree pair for pair
+        assert np.array_equal(got["neigh_sorted"], exp["neigh_sorted"])
+        assert np.array_equal(got["neighbors"], exp["neighbors"])
+
+
+@pytest.mark.parametrize("dims,batch,num_pts,radius", [(2, 2, 1000, 0.08), (4, 2, 800, 0.3), (6, 2, 600, 0.6)])
+def test_pdf_and_gradients(ops, oracle, dims, batch, num_pts, radius):
+    pts, ids = _cloud(dims, batch, num_pts, 300 + dims)
+    got = gpu_neighborhood(ops, pts, ids, pts, ids, radius, batch)
+    d = got["dev"]
+    bw = np.full(dims, 0.25 * radius, np.float32)
+    for manifold in (dims, 2):
+        pdf = ops.compute_pdf(manifold, t(bw), d["pts"], d["neigh"], d["ends"])
+        exp = oracle.compute_pdf(manifold, bw, pts, got["neighbors"], got["ends"])
+        assert relerr(pdf.cpu().numpy(), exp) < 1e-5
+        spdf = ops.compute_pdf_sorted(manifold, t(bw), d["spts"], d["pts"], t(got["neigh_sorted"]), d["ends"])
+        assert relerr(spdf.cpu().numpy(), exp) < 1e-5
+    g = np.random.default_rng(dims).normal(size=pts.shape[0]).astype(np.float32)
+    grads = ops.compute_pdf_grads(dims, t(bw), d["pts"], d["neigh"], d["ends"], t(g))
+    exp_g = oracle.compute_pdf_grads(dims, bw, pts, got["neighbors"], got["ends"], g)
+    assert tuple(grads.shape) == pts.shape and relerr(grads.cpu().numpy(), exp_g) < 1e-4
+
+
+@pytest.mark.parametrize("dims,batch,num_pts,radius", [(2, 3, 1500, 0.05), (4, 2, 1000, 0.3), (6, 2, 800, 0.6)])
+def test_poisson_disk(ops, oracle, dims, batch, num_pts, radius):
+    pts, ids = _cloud(dims, batch, num_pts, 400 + dims)
+    exp = oracle.neighborhood(pts, ids, pts, ids, radius)
+    e_neigh, e_ends = oracle.find_neighbors(exp["sorted_pts"], exp["sorted_keys"], exp["sorted_pts"],
+                                            exp["sorted_keys"], exp["grid_ds"], exp["num_cells"], exp["radii"])
+    e_sel = oracle.poisson_disk_sampling(exp["sorted_keys"], e_neigh, e_ends, exp["num_cells"])
+    g = gpu_neighborhood(ops, pts, ids, pts, ids, radius, batch)["dev"]
+    neigh, ends = ops.find_neighbors_ex(g["spts"], g["skeys"], g["spts"], g["skeys"], g["ds"], g["nc"], g["radii"], 0)
+    sel = ops.poisson_disk_sampling(g["skeys"], neigh, ends, g["nc"])
+    assert np.array_equal(sel.cpu().numpy(), e_sel)
+    # the defining property, per cloud: selected points are at least one radius apart
+    chosen = exp["sorted_pts"][e_sel[:, 0]].astype(np.float64)
+    cid = ids[exp["perm"]][e_sel[:, 0]]
+    for b in range(batch):
+        q = chosen[cid == b]
+        dist = np.linalg.norm(q[:, None] - q[None], axis=-1) + np.eye(q.shape[0]) * 1e9
+        assert dist.min() >= radius * (1 - 1e-6)
+
+
+def test_object_api_in_two_dimensions(oracle):
+    # Pointcloud / Grid / Neighborhood / PointPooling / compute_pdf on planar clouds
+    import pccnn_lib_amd as lib
+    pts, ids = _cloud(2, 3, 2000, 7)
+    pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+    radii = torch.full((2,), 0.05, device=DEV)
+    nbh = lib.pc.layers.conv_base.build_neighborhood(pc, pc, radii, 0)
+    exp = oracle.neighborhood(pts, ids, pts, ids, 0.05)
+    assert np.array_equal(oracle.canonical_pairs(nbh.neighbors_.cpu().numpy()), oracle.canonical_pairs(exp["neighbors"]))
+    assert np.array_equal(nbh.start_ids_.cpu().numpy(), exp["ends"])
+    pc.compute_pdf(np.full(2, 0.02, np.float32))
+    unnorm, norm, _ = oracle.pointcloud_pdf(pts, ids, 0.02)
+    assert relerr(pc.pts_unnorm_pdf_.cpu().numpy(), unnorm) < 1e-5
+    assert relerr(pc.pts_pdf_.cpu().numpy(), norm) < 1e-5
+    pool = lib.pc.PointPooling(pc, radii)
+    sel = pool.pooling_ids_.cpu().numpy().reshape(-1)
+    q = pts[sel][ids[sel] == 1].astype(np.float64)
+    dist = np.linalg.norm(q[:, None] - q[None], axis=-1) + np.eye(q.shape[0]) * 1e9
+    assert dist.min() >= 0.05 * (1 - 1e-6)
