@@ -15,18 +15,26 @@ def _fibonacci_sphere(count):
     return np.stack([np.cos(theta) * np.sin(phi), np.sin(theta) * np.sin(phi), np.cos(phi)], axis=1)
 
 
+def _circle(count, phase=0.0):
+    a = 2.0 * np.pi * (np.arange(count) + phase) / max(count, 1)
+    return np.stack([np.cos(a), np.sin(a)], axis=1)
+
+
 def kernel_points(num_dims, num_kernel_pts):
-    if num_dims != 3:
-        raise RuntimeError("kernel point layouts exist for 3 dimensions only")
+    """A centre point plus one shell (up to 16 points) or two shells (inner one at half the radius) of evenly
+    spread directions: on the unit sphere in 3 dimensions, on the unit circle in 2."""
+    if num_dims not in (2, 3):
+        raise RuntimeError("kernel point layouts exist for 2 and 3 dimensions only")
     if not 2 <= num_kernel_pts <= 64:
         raise RuntimeError("the number of kernel points must lie in [2, 64]")
+    spread = _fibonacci_sphere if num_dims == 3 else _circle
     rest = num_kernel_pts - 1
     if num_kernel_pts <= 16:
-        shell = _fibonacci_sphere(rest)
+        shell = spread(rest)
     else:
         inner = rest // 4
-        shell = np.concatenate([0.5 * _fibonacci_sphere(inner), _fibonacci_sphere(rest - inner)], axis=0)
-    return np.concatenate([np.zeros((1, 3)), shell], axis=0)
+        shell = np.concatenate([0.5 * spread(inner), spread(rest - inner)], axis=0)
+    return np.concatenate([np.zeros((1, num_dims)), shell], axis=0)
 
 
 class _Layouts(dict):

@@ -320,8 +320,29 @@ GRAD_WEIGHTS, GRAD_FEATS, GRAD_BASIS_PARAMS, GRAD_PDF, GRAD_PTS, GRAD_ALL = 1, 2
 def _conv_dims(pts, name):
     d = pts.shape[1]
     if d != 3:
-        raise RuntimeError("%s: %d-dimensional points are not supported by the convolutions (only 3)" % (name, d))
+        raise RuntimeError("%s: %d-dimensional points are not supported by the convolutions (2 or 3)" % (name, d))
     return d
+
+
+# Planar clouds run through the 3-D kernels with a zero third coordinate: positions, samples and kernel points get
+# a zero column, axis matrices a zero row, the radii a 1; every term the extra coordinate adds is an exact zero, so
+# the results are those of the 2-D formulas, and the extra gradient components are dropped.
+def _is_planar(pts):
+    return isinstance(pts, torch.Tensor) and pts.dim() == 2 and pts.shape[1] == 2
+
+
+def _pad_cols(x, value=0.0):
+    """[n, 2] -> [n, 3] (or [2] -> [3])."""
+    return torch.nn.functional.pad(x, (0, 1), value=value).contiguous()
+
+
+def _pad_rows(x):
+    """[2, k] -> [3, k]."""
+    return torch.nn.functional.pad(x, (0, 0, 0, 1)).contiguous()
+
+
+def _cut(x):
+    return None if x is None else x[:, :2].contiguous()
 
 
 def _conv_args(name, pts, feats, samples, neigh, ends, radii):
@@ -347,6 +368,9 @@ def kp_conv(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights,
     reference) rounds the operands of the [M,K*Cin] x [K*Cin,Cout] product to bf16 and accumulates in fp32; the
     projection returned is then bf16."""
     name = "kp_conv"
+    if _is_planar(pts):
+        return kp_conv(_pad_cols(pts), feats, _pad_cols(samples), neigh, ends, _pad_cols(radii, 1.0),
+                       _pad_cols(kernel_pts), sigma, weights, return_proj, contraction)
     bf16 = _contraction(name, contraction)
     d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
     _chk(kernel_pts, name + ": kernel_pts", torch.float32, 2, dev)
@@ -421,6 +445,11 @@ def kp_conv_grads(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, we
     ``grad_mask``: GRAD_* groups to compute, the others come back as None; ``mirror``: result of mirror_pairs()
     for a symmetric neighborhood, which lets dPts (and dPdf) be summed per point without atomics."""
     name = "kp_conv_grads"
+    if _is_planar(pts):
+        d_w, d_f, d_kp, d_p, d_s = kp_conv_grads(_pad_cols(pts), feats, _pad_cols(samples), neigh, ends,
+                                                 _pad_cols(radii, 1.0), _pad_cols(kernel_pts), sigma, weights, in_grads,
+                                                 proj, grad_mask, mirror, contraction)
+        return [d_w, d_f, _cut(d_kp), _cut(d_p), _cut(d_s)]
     bf16 = _contraction(name, contraction)
     d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
     _chk(kernel_pts, name + ": kernel_pts", torch.float32, 2, dev)
@@ -490,6 +519,9 @@ def mc_conv(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights, r
     ``return_proj=True`` also returns the projection f32[M,Cin,H*m] for mc_conv_grads(..., proj=...);
     ``contraction`` as in kp_conv."""
     name = "mc_conv"
+    if _is_planar(pts):
+        return mc_conv(_pad_cols(pts), pdf, feats, _pad_cols(samples), neigh, ends, _pad_cols(radii, 1.0),
+                       _pad_rows(axis), bias, weights, return_proj, contraction)
     bf16 = _contraction(name, contraction)
     d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
     n, m, t, c_in = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1]
@@ -511,6 +543,10 @@ def mc_conv_grads(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weig
     """mc_conv_grads(..., in_grads f32[M,Cout]) -> [dW, dFeat, dAxis, dBias f32[1,H*m], dPdf f32[N], dPts, dSamples]
     (pccnn_lib_ops/pcconvs/mcconv.cuh:57-69).  ``proj`` / ``grad_mask`` / ``mirror`` as in kp_conv_grads."""
     name = "mc_conv_grads"
+    if _is_planar(pts):
+        g = mc_conv_grads(_pad_cols(pts), pdf, feats, _pad_cols(samples), neigh, ends, _pad_cols(radii, 1.0),
+                          _pad_rows(axis), bias, weights, in_grads, proj, grad_mask, mirror, contraction)
+        return [g[0], g[1], None if g[2] is None else g[2][:2].contiguous(), g[3], g[4], _cut(g[5]), _cut(g[6])]
     bf16 = _contraction(name, contraction)
     d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
     n, m, t, c_in = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1]
@@ -541,6 +577,9 @@ def kp_conv_weight_var(pts, feats, samples, neigh, ends, radii, kernel_pts, sigm
     """kp_conv_weight_var(pts, feats, samples, neighbors, start_ids, radii, kernel_pts, sigma) -> 0-d float tensor
     (pccnn_lib_ops/pcconvs/kpconv.cuh:82-90)."""
     name = "kp_conv_weight_var"
+    if _is_planar(pts):
+        return kp_conv_weight_var(_pad_cols(pts), feats, _pad_cols(samples), neigh, ends, _pad_cols(radii, 1.0),
+                                  _pad_cols(kernel_pts), sigma)
     d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
     _chk(kernel_pts, name + ": kernel_pts", torch.float32, 2, dev)
     n, m, t, c_in, k = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1], kernel_pts.shape[0]
@@ -557,6 +596,9 @@ def mc_conv_weight_var(pts, pdf, feats, samples, neigh, ends, radii, axis, bias)
     """mc_conv_weight_var(pts, pdf, feats, samples, neighbors, start_ids, radii, axis, bias) -> 0-d float tensor
     (pccnn_lib_ops/pcconvs/mcconv.cuh:83-92)."""
     name = "mc_conv_weight_var"
+    if _is_planar(pts):
+        return mc_conv_weight_var(_pad_cols(pts), pdf, feats, _pad_cols(samples), neigh, ends, _pad_cols(radii, 1.0),
+                                  _pad_rows(axis), bias)
     d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
     _chk(pdf, name + ": pdf", torch.float32, 1, dev)
     _chk(axis, name + ": axis", torch.float32, 2, dev)
@@ -648,6 +690,9 @@ def kp_conv_n(pts, pdf, feats, samples, neigh, ends, radii, kernel_pts, sigma, w
     weights f32[K*Cin,Cout]) -> f32[M,Cout]: KPConv whose correlation is divided by the density of the neighbor
     (pccnn_lib_ops/pcconvs/kpconvn.cuh:32-42)."""
     name = "kp_conv_n"
+    if _is_planar(pts):
+        return kp_conv_n(_pad_cols(pts), pdf, feats, _pad_cols(samples), neigh, ends, _pad_cols(radii, 1.0),
+                         _pad_cols(kernel_pts), sigma, weights, return_proj)
     k = _kernel_pts_args(name, pts, pdf, feats, samples, neigh, ends, radii, kernel_pts)
     desc = _basis(BASIS_KPN, k, kernel_pts, sigma=sigma, pdf=pdf)
     return _generic_forward(name, desc, k, pts, feats, samples, neigh, ends, radii, weights, False, return_proj)
@@ -658,6 +703,10 @@ def kp_conv_n_grads(pts, pdf, feats, samples, neigh, ends, radii, kernel_pts, si
     """kp_conv_n_grads(..., in_grads) -> [dW, dFeat, dKernelPts, dPts, dSamples]; the density gets no gradient
     (pccnn_lib_ops/pcconvs/kpconvn.cuh:57-68)."""
     name = "kp_conv_n_grads"
+    if _is_planar(pts):
+        g = kp_conv_n_grads(_pad_cols(pts), pdf, feats, _pad_cols(samples), neigh, ends, _pad_cols(radii, 1.0),
+                            _pad_cols(kernel_pts), sigma, weights, in_grads, proj, grad_mask, mirror)
+        return [g[0], g[1], _cut(g[2]), _cut(g[3]), _cut(g[4])]
     k = _kernel_pts_args(name, pts, pdf, feats, samples, neigh, ends, radii, kernel_pts)
     desc = _basis(BASIS_KPN, k, kernel_pts, sigma=sigma, pdf=pdf)
     d_kp = torch.empty_like(kernel_pts) if int(grad_mask) & GRAD_BASIS_PARAMS else None
@@ -669,6 +718,9 @@ def kp_conv_n_grads(pts, pdf, feats, samples, neigh, ends, radii, kernel_pts, si
 def kp_conv_n_weight_var(pts, pdf, feats, samples, neigh, ends, radii, kernel_pts, sigma):
     """kp_conv_n_weight_var(...) -> 0-d float tensor (pccnn_lib_ops/pcconvs/kpconvn.cuh:83-92)."""
     name = "kp_conv_n_weight_var"
+    if _is_planar(pts):
+        return kp_conv_n_weight_var(_pad_cols(pts), pdf, feats, _pad_cols(samples), neigh, ends, _pad_cols(radii, 1.0),
+                                    _pad_cols(kernel_pts), sigma)
     k = _kernel_pts_args(name, pts, pdf, feats, samples, neigh, ends, radii, kernel_pts)
     desc = _basis(BASIS_KPN, k, kernel_pts, sigma=sigma, pdf=pdf)
     return _generic_weight_var(name, desc, k, pts, feats, samples, neigh, ends, radii, False)
@@ -679,6 +731,9 @@ def pccnn(pts, feats, pdf, samples, neigh, ends, radii, kernel_pts, sigma, weigh
     weights f32[K*Cin,Cout]) -> f32[M,Cout]: gaussian kernel-point correlation divided by the density
     (pccnn_lib_ops/pcconvs/pccnn.cuh:32-42; note the feats-before-pdf argument order)."""
     name = "pccnn"
+    if _is_planar(pts):
+        return pccnn(_pad_cols(pts), feats, pdf, _pad_cols(samples), neigh, ends, _pad_cols(radii, 1.0),
+                     _pad_cols(kernel_pts), sigma, weights, return_proj)
     k = _kernel_pts_args(name, pts, pdf, feats, samples, neigh, ends, radii, kernel_pts)
     desc = _basis(BASIS_GAUSS, k, kernel_pts, sigma=sigma, pdf=pdf)
     return _generic_forward(name, desc, k, pts, feats, samples, neigh, ends, radii, weights, False, return_proj)
@@ -689,6 +744,10 @@ def pccnn_grads(pts, feats, pdf, samples, neigh, ends, radii, kernel_pts, sigma,
     """pccnn_grads(..., in_grads) -> [dW, dFeat, dKernelPts, dPdf, dPts, dSamples]
     (pccnn_lib_ops/pcconvs/pccnn.cuh:57-68)."""
     name = "pccnn_grads"
+    if _is_planar(pts):
+        g = pccnn_grads(_pad_cols(pts), feats, pdf, _pad_cols(samples), neigh, ends, _pad_cols(radii, 1.0),
+                        _pad_cols(kernel_pts), sigma, weights, in_grads, proj, grad_mask, mirror)
+        return [g[0], g[1], _cut(g[2]), g[3], _cut(g[4]), _cut(g[5])]
     k = _kernel_pts_args(name, pts, pdf, feats, samples, neigh, ends, radii, kernel_pts)
     desc = _basis(BASIS_GAUSS, k, kernel_pts, sigma=sigma, pdf=pdf)
     d_kp = torch.empty_like(kernel_pts) if int(grad_mask) & GRAD_BASIS_PARAMS else None
@@ -701,6 +760,9 @@ def pccnn_grads(pts, feats, pdf, samples, neigh, ends, radii, kernel_pts, sigma,
 def pccnn_weight_variance(pts, feats, pdf, samples, neigh, ends, radii, kernel_pts, sigma):
     """pccnn_weight_variance(...) -> 0-d float tensor (pccnn_lib_ops/pcconvs/pccnn.cuh:83-92)."""
     name = "pccnn_weight_variance"
+    if _is_planar(pts):
+        return pccnn_weight_variance(_pad_cols(pts), feats, pdf, _pad_cols(samples), neigh, ends,
+                                     _pad_cols(radii, 1.0), _pad_cols(kernel_pts), sigma)
     k = _kernel_pts_args(name, pts, pdf, feats, samples, neigh, ends, radii, kernel_pts)
     desc = _basis(BASIS_GAUSS, k, kernel_pts, sigma=sigma, pdf=pdf)
     return _generic_weight_var(name, desc, k, pts, feats, samples, neigh, ends, radii, False)
@@ -763,6 +825,8 @@ def point_conv_basis(pts, radii, samples, neigh, axis, bias):
     """point_conv_basis(pts, radii, samples, neighbors, axis f32[D,K], bias f32[1,K]) -> f32[T,K]: the affine map
     of the normalised offsets that PointConv feeds to its own layers (pccnn_lib_ops/pcconvs/pointconv.cuh:20-26)."""
     name = "point_conv_basis"
+    if _is_planar(pts):
+        return point_conv_basis(_pad_cols(pts), _pad_cols(radii, 1.0), _pad_cols(samples), neigh, _pad_rows(axis), bias)
     d, dev, k = _linear_basis_args(name, pts, radii, samples, neigh, axis, bias)
     t = neigh.shape[0]
     out = torch.empty((t, k), dtype=torch.float32, device=dev)
@@ -775,6 +839,10 @@ def point_conv_basis_grads(pts, radii, samples, neigh, axis, bias, in_grads):
     """point_conv_basis_grads(..., in_grads f32[T,K]) -> [dPts, dSamples, dAxis, dBias f32[1,K]]
     (pccnn_lib_ops/pcconvs/pointconv.cuh:28-35)."""
     name = "point_conv_basis_grads"
+    if _is_planar(pts):
+        g = point_conv_basis_grads(_pad_cols(pts), _pad_cols(radii, 1.0), _pad_cols(samples), neigh, _pad_rows(axis),
+                                   bias, in_grads)
+        return [_cut(g[0]), _cut(g[1]), g[2][:2].contiguous(), g[3]]
     d, dev, k = _linear_basis_args(name, pts, radii, samples, neigh, axis, bias)
     t = neigh.shape[0]
     in_grads = _chk(in_grads.contiguous(), name + ": in_grads", torch.float32, 2, dev)

@@ -132,3 +132,74 @@ def test_object_api_in_two_dimensions(oracle):
     q = pts[sel][ids[sel] == 1].astype(np.float64)
     dist = np.linalg.norm(q[:, None] - q[None], axis=-1) + np.eye(q.shape[0]) * 1e9
     assert dist.min() >= 0.05 * (1 - 1e-6)
+
+
+@pytest.mark.parametrize("distinct", [False, True])
+def test_planar_kpconv_and_mcconv(ops, oracle, distinct):
+    # The reference's convolution tests also run in 2 dimensions (unit_test/utest_kpconv.ini, utest_mcconv.ini).
+    # Planar clouds go through the 3-D kernels with a zero third coordinate; results against the oracle's 2-D formulas.
+    pts, ids = _cloud(2, 2, 1200, 9)
+    rng = np.random.default_rng(9)
+    if distinct:
+        pick = np.sort(rng.choice(pts.shape[0], pts.shape[0] // 3, replace=False))
+        smp, sids = pts[pick].copy(), ids[pick]
+    else:
+        smp, sids = pts, ids
+    nb = gpu_neighborhood(ops, pts, ids, smp, sids, 0.08, 2)
+    neigh, ends, radii, d = nb["neighbors"], nb["ends"], nb["radii"], nb["dev"]
+    c_in, c_out, k = 16, 24, 16
+    feats = rng.normal(size=(pts.shape[0], c_in)).astype(np.float32)
+    g = rng.normal(size=(smp.shape[0], c_out)).astype(np.float32)
+    # KPConv: centre + 15 directions on the circle, normalised like the layer does
+    ang = 2 * np.pi * np.arange(k - 1) / (k - 1)
+    kp = np.concatenate([np.zeros((1, 2)), np.stack([np.cos(ang), np.sin(ang)], 1)]).astype(np.float32) / np.float32(2.0)
+    sigma = 0.5
+    w = rng.normal(0, np.sqrt(1.0 / (k * c_in)), (k * c_in, c_out)).astype(np.float32)
+    args = (d["pts"], t(feats), d["samples"], d["neigh"], d["ends"], d["radii"], t(kp), sigma, t(w))
+    host = (pts, feats, smp, neigh, ends, radii, kp, sigma, w)
+    assert relerr(ops.kp_conv(*args).cpu().numpy(), oracle.kpconv(*host)) < 1e-5
+    grads = ops.kp_conv_grads(*args, t(g))
+    for got, e, name in zip(grads, oracle.kpconv_grads(*host, g), ("dW", "dFeat", "dKernelPts", "dPts", "dSamples")):
+        assert tuple(got.shape) == e.shape, name
+        assert relerr(got.cpu().numpy(), e) < 1e-4, name
+    assert relerr(ops.kp_conv_weight_var(*args[:-1]).cpu().numpy(), oracle.kpconv_weight_var(*host[:-1])) < 1e-4
+    # MCConv
+    pdf = rng.uniform(0.5, 2.0, pts.shape[0]).astype(np.float32)
+    axis = rng.normal(0, np.sqrt(0.5), (2, k)).astype(np.float32)
+    bias = rng.normal(0, 0.1, (1, k)).astype(np.float32)
+    wm = rng.normal(0, np.sqrt(1.0 / (k * c_in)), (1, k * c_in, c_out)).astype(np.float32)
+    margs = (d["pts"], t(pdf), t(feats), d["samples"], d["neigh"], d["ends"], d["radii"], t(axis), t(bias), t(wm))
+    mhost = (pts, pdf, feats, smp, neigh, ends, radii, axis, bias, wm)
+    assert relerr(ops.mc_conv(*margs).cpu().numpy(), oracle.mcconv(*mhost)) < 1e-5
+    names = ("dW", "dFeat", "dAxis", "dBias", "dPdf", "dPts", "dSamples")
+    for got, e, name in zip(ops.mc_conv_grads(*margs, t(g)), oracle.mcconv_grads(*mhost, g), names):
+        assert tuple(got.shape) == e.shape, name
+        assert relerr(got.cpu().numpy(), e) < 1e-4, name
+
+
+def test_planar_layers(oracle):
+    import pccnn_lib_amd as lib
+    pts, ids = _cloud(2, 2, 1500, 21)
+    rng = np.random.default_rng(21)
+    feats = rng.normal(size=(pts.shape[0], 8)).astype(np.float32)
+    pc = lib.pc.Pointcloud(pts, ids, device=DEV, requires_grad=True)
+    pc.compute_pdf(np.full(2, 0.02, np.float32))
+    torch.manual_seed(3)
+    kp_layer = lib.pc.layers.KPConv(2, 8, 12, 16).to(DEV)
+    mc_layer = lib.pc.layers.MCConv(2, 8, 12, 8).to(DEV)
+    tf = t(feats).requires_grad_(True)
+    out_kp, nbh = kp_layer(pc, pc, tf, 0.06)
+    out_mc = mc_layer(pc, pc, tf, 0.06, nbh)
+    (out_kp.sum() + out_mc.sum()).backward()
+    p = lambda x: x.detach().cpu().numpy()
+    radii = np.full(2, 0.06, np.float32)
+    nb = (p(nbh.neighbors_), p(nbh.start_ids_))
+    exp = oracle.kpconv(pts, feats, pts, nb[0], nb[1], radii, p(kp_layer.kernel_pts_), float(kp_layer.sigma_.item()),
+                        p(kp_layer.conv_weights_))
+    assert relerr(p(out_kp), exp) < 1e-5
+    pdf = p(pc.pts_unnorm_pdf_ * torch.prod(t(radii)))
+    exp = oracle.mcconv(pts, pdf, feats, pts, nb[0], nb[1], radii, p(mc_layer.proj_axis_), p(mc_layer.proj_bias_),
+                        p(mc_layer.conv_weights_))
+    assert relerr(p(out_mc), exp) < 1e-5
+    assert tuple(pc.pts_.grad.shape) == pts.shape and bool(torch.isfinite(pc.pts_.grad).all())
+    assert tuple(tf.grad.shape) == feats.shape
