@@ -175,7 +175,11 @@ int pccnn_compact_selected(const int32_t *selected, const int32_t *selected_scan
  * d_weights (same shape), d_feats, d_axis f32[d,k], d_bias f32[k], d_pdf f32[n],
  * d_pts, d_samples.
  *
- * 1 <= k <= 64.
+ * 1 <= k <= 64.  2 <= d <= 6 (the reference's tests run the convolutions in 2, 3 and 4 dimensions,
+ * unit_test/utest_kpconv.ini, utest_mcconv.ini).  d == 3 runs kernels that fuse the basis into the gather; any other
+ * d evaluates the basis per pair into f32[t,k] in the workspace, runs the convolution on it as a caller-given basis
+ * and maps the basis gradient back per pair.  For d != 3 the forward calls need a workspace too
+ * (pccnn_conv_workspace_bytes(..., backward = 0)) and `mirror` is ignored.
  *
  * Three arguments go beyond the reference's interface.  `proj_out` / `proj` (nullable): the projection
  * P f32[m, c_in, k] (k fastest) that the forward call builds on its way to `out`; a caller that keeps it
@@ -229,14 +233,14 @@ int pccnn_mcconv_backward(const float *pts, const float *pdf, const float *feats
  * output by the neighbor count (`divide_by_count`).
  *
  *   kind       a                      b               c             other fields
- *   KP         kernel_pts f32[k,3]    -               -             sigma
- *   MLP        axis f32[3,k]          bias f32[k]     -             pdf f32[n]
- *   KPN        kernel_pts f32[k,3]    -               -             sigma, pdf      (KP value / pdf)
- *   GAUSS      kernel_pts f32[k,3]    -               -             sigma, pdf      (exp(-|kp-d|^2/(2 sigma^2)) / pdf)
+ *   KP         kernel_pts f32[k,d]    -               -             sigma
+ *   MLP        axis f32[d,k]          bias f32[k]     -             pdf f32[n]
+ *   KPN        kernel_pts f32[k,d]    -               -             sigma, pdf      (KP value / pdf)
+ *   GAUSS      kernel_pts f32[k,d]    -               -             sigma, pdf      (exp(-|kp-d|^2/(2 sigma^2)) / pdf)
  *   EXPLICIT   basis f32[t,k]         -               -             (values given per pair: PointConv)
- *   SPH        radial edges f32[nb0]  azimuth [nb1]   polar [nb2]   k is nb0*nb1*nb2 + 1 (one-hot spherical bin)
+ *   SPH        radial edges f32[nb0]  azimuth [nb1]   polar [nb2]   k is nb0*nb1*nb2 + 1 (one-hot spherical bin; d == 3 only)
  *
- * Backward outputs: d_param_a = d_kernel_pts [k,3] (KP, KPN, GAUSS), d_axis [3,k] (MLP) or the basis gradient
+ * Backward outputs: d_param_a = d_kernel_pts [k,d] (KP, KPN, GAUSS), d_axis [d,k] (MLP) or the basis gradient
  * f32[t,k] (EXPLICIT); d_param_b = d_bias [k] (MLP); d_pdf only for MLP and GAUSS; d_pts / d_samples for the
  * kinds whose basis depends on the positions (not EXPLICIT, not SPH).  Groups a kind does not have are ignored. */
 #define PCCNN_BASIS_KP 0
@@ -270,7 +274,7 @@ int pccnn_conv_weight_var(const pccnn_basis *basis, const float *pts, const floa
 
 /* PointConv's per-pair basis op and its gradient: replaces point_conv_basis / point_conv_basis_grads
  * (pccnn_lib_ops/pcconvs/pointconv.cuh:20-35): basis_out f32[t,k] = ((pts[n_t] - samples[s_t]) / radii) . axis + bias;
- * backward: d_pts f32[n,3], d_samples f32[m,3], d_axis f32[3,k], d_bias f32[k] from basis_grads f32[t,k]. */
+ * backward: d_pts f32[n,d], d_samples f32[m,d], d_axis f32[d,k], d_bias f32[k] from basis_grads f32[t,k]. */
 int pccnn_linear_basis_forward(const float *pts, const float *samples, const int32_t *neigh, const float *radii,
                                const float *axis, const float *bias, int64_t n, int64_t m, int64_t t, int d, int k,
                                float *basis_out, void *stream);
@@ -286,7 +290,7 @@ int pccnn_linear_basis_backward(const float *pts, const float *samples, const in
  * kernel pccnn_lib_ops/pcconvs/shared/compute_variance_weights.cu:24-170): out[0] (one float, device) =
  * 1 / mean over the samples of sum_{i,j in N(s)} (w_i . w_j)(F_i . F_j), evaluated as the squared norm of the
  * sample's projection tile.  Same tensor arguments as the forward calls, without the weights. */
-size_t pccnn_conv_weight_var_workspace_bytes(int64_t m, int c_in, int k);
+size_t pccnn_conv_weight_var_workspace_bytes(int64_t m, int64_t t, int c_in, int k);
 int pccnn_kpconv_weight_var(const float *pts, const float *feats, const float *samples, const int32_t *neigh,
                             const int32_t *ends, const float *radii, const float *kernel_pts, float sigma,
                             int64_t n, int64_t m, int64_t t, int d, int c_in, int k, float *out,

@@ -56,7 +56,7 @@ SIGNATURES = {
                                    P, P, P, SZ, P]),
     "pccnn_mcconv_backward": (I32, [P, P, P, P, P, P, P, P, P, P, P, P, P, I32, I64, I64, I64, I32, I32, I32, I32, I32,
                                     P, P, P, P, P, P, P, P, SZ, P]),
-    "pccnn_conv_weight_var_workspace_bytes": (SZ, [I64, I32, I32]),
+    "pccnn_conv_weight_var_workspace_bytes": (SZ, [I64, I64, I32, I32]),
     "pccnn_kpconv_weight_var": (I32, [P, P, P, P, P, P, P, F32, I64, I64, I64, I32, I32, I32, P, P, SZ, P]),
     "pccnn_mcconv_weight_var": (I32, [P, P, P, P, P, P, P, P, P, I64, I64, I64, I32, I32, I32, P, P, SZ, P]),
     "pccnn_conv_forward": (I32, [BP, P, P, P, P, P, P, P, I64, I64, I64, I32, I32, I32, I32, I32, P, P, P, SZ, P]),

@@ -775,7 +775,7 @@ static int launch_proj_bwd(const ConvGeom &g, const float *feats, const float *p
 static int conv_validate(const char *who, int64_t n, int64_t m, int64_t t, int d, int c_in, int k, int num_mlps,
                          int c_out)
 {
-    PCCNN_REQUIRE(d == 3, PCCNN_ERR_UNSUPPORTED, "%s: d=%d is not supported (d must be 3)", who, d);
+    PCCNN_REQUIRE(d >= 2 && d <= PCCNN_MAX_DIMS, PCCNN_ERR_UNSUPPORTED, "%s: d=%d is not supported (2 <= d <= 6)", who, d);
     PCCNN_REQUIRE(n >= 0 && m >= 0 && t >= 0 && n < (1ll << 31) && m < (1ll << 31) && t < (1ll << 31),
                   PCCNN_ERR_INVALID, "%s: n=%lld m=%lld t=%lld", who, (long long)n, (long long)m, (long long)t);
     PCCNN_REQUIRE(c_in >= 1 && c_out >= 1, PCCNN_ERR_INVALID, "%s: c_in=%d c_out=%d", who, c_in, c_out);
@@ -794,14 +794,15 @@ extern "C" size_t pccnn_conv_workspace_bytes(int64_t m, int64_t t, int c_in, int
     if (t < 1) t = 1;
     size_t proj = pccnn_align((size_t)m * c_in * k * sizeof(float));
     size_t w16 = pccnn_align((size_t)c_in * k * c_out * sizeof(uint16_t));       // bf16 copy of the weights
-    if (!backward) return proj + w16 + 256;
+    size_t pair_b = 2 * pccnn_align((size_t)t * k * sizeof(float));              // basis (+ its gradient) when d != 3
+    if (!backward) return proj + w16 + pair_b + 256;
     size_t basis_g = pccnn_align((size_t)t * k * sizeof(float));
     size_t splitk = pccnn_align((size_t)CONV_SPLIT_K * c_in * k * c_out * sizeof(float));
     size_t partials = pccnn_align(((size_t)PARAM_ROWS + PARAM_REDUCE_GROUPS) * 256 * sizeof(float));
     size_t scaled = pccnn_align((size_t)m * c_out * sizeof(float));
     size_t pair_g = pccnn_align((size_t)t * 4 * sizeof(float));
     size_t g16 = pccnn_align((size_t)m * c_out * sizeof(uint16_t));               // bf16 copy of the output gradients
-    return 2 * proj + basis_g + splitk + partials + scaled + pair_g + w16 + g16 + 256;
+    return 2 * proj + basis_g + splitk + partials + scaled + pair_g + w16 + g16 + pair_b + 256;
 }
 
 // out[m, c_out] = P[m, c_in*k] x W, with the feature axis split over num_mlps independent
@@ -967,7 +968,7 @@ static int conv_weight_var(ConvGeom g, const float *feats, float *out, void *wor
     float *proj = arena.take<float>((size_t)g.m * g.c_in * g.k);
     float *rows = arena.take<float>((size_t)g.m);
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv weight variance: workspace of %zu bytes, need %zu",
-                  workspace_bytes, pccnn_conv_weight_var_workspace_bytes(g.m, g.c_in, g.k));
+                  workspace_bytes, pccnn_conv_weight_var_workspace_bytes(g.m, 0, g.c_in, g.k));
     int rc = launch_proj_fwd<BASIS>(g, feats, proj, s);
     if (rc != PCCNN_OK) return rc;
     row_sumsq_kernel<<<(unsigned)pccnn_ceil_div(g.m, 4), 256, 0, s>>>(proj, g.m, (int64_t)g.c_in * g.k, rows);
@@ -981,10 +982,27 @@ static int conv_weight_var(ConvGeom g, const float *feats, float *out, void *wor
     return PCCNN_OK;
 }
 
-extern "C" size_t pccnn_conv_weight_var_workspace_bytes(int64_t m, int c_in, int k)
+// Defined with the generic entry points below; the dedicated entry points hand clouds that are not 3-D to them.
+static int conv_forward_entry(const char *who, bool bf16, const pccnn_basis *basis, const float *pts, const float *feats,
+                              const float *samples, const int32_t *neigh, const int32_t *ends, const float *radii,
+                              const float *weights, int64_t n, int64_t m, int64_t t, int d, int c_in, int num_mlps,
+                              int c_out, int divide_by_count, float *out, void *proj_out, void *workspace,
+                              size_t workspace_bytes, void *stream);
+static int conv_backward_entry(const char *who, bool bf16, const pccnn_basis *basis, const float *pts, const float *feats,
+                                   const float *samples, const int32_t *neigh, const int32_t *ends,
+                                   const float *radii, const float *weights, const float *in_grads, const void *proj,
+                                   const int32_t *mirror, int grad_mask, int64_t n, int64_t m, int64_t t, int d, int c_in, int num_mlps,
+                                   int c_out, int divide_by_count, float *d_weights, float *d_feats, float *d_param_a,
+                                   float *d_param_b, float *d_pdf, float *d_pts, float *d_samples, void *workspace,
+                                   size_t workspace_bytes, void *stream);
+
+extern "C" size_t pccnn_conv_weight_var_workspace_bytes(int64_t m, int64_t t, int c_in, int k)
 {
     if (m < 1) m = 1;
-    return pccnn_align((size_t)m * c_in * k * sizeof(float)) + pccnn_align((size_t)m * sizeof(float)) + 256;
+    if (t < 1) t = 1;
+    // projection, per-sample sums and (for clouds that are not 3-D) the per-pair basis
+    return pccnn_align((size_t)m * c_in * k * sizeof(float)) + pccnn_align((size_t)m * sizeof(float)) +
+           pccnn_align((size_t)t * k * sizeof(float)) + 256;
 }
 
 extern "C" int pccnn_kpconv_weight_var(const float *pts, const float *feats, const float *samples,
@@ -993,6 +1011,11 @@ extern "C" int pccnn_kpconv_weight_var(const float *pts, const float *feats, con
                                        int c_in, int k, float *out, void *workspace, size_t workspace_bytes,
                                        void *stream)
 {
+    if (d != 3) {
+        const pccnn_basis b = {PCCNN_BASIS_KP, k, kernel_pts, nullptr, nullptr, 0, 0, 0, sigma, nullptr};
+        return pccnn_conv_weight_var(&b, pts, feats, samples, neigh, ends, radii, n, m, t, d, c_in, 0, out, workspace,
+                                     workspace_bytes, stream);
+    }
     int rc = conv_validate("pccnn_kpconv_weight_var", n, m, t, d, c_in, k, 1, 1);
     if (rc != PCCNN_OK) return rc;
     PCCNN_REQUIRE(sigma > 0.0f, PCCNN_ERR_INVALID, "pccnn_kpconv_weight_var: sigma=%g", sigma);
@@ -1008,6 +1031,11 @@ extern "C" int pccnn_mcconv_weight_var(const float *pts, const float *pdf, const
                                        int c_in, int k, float *out, void *workspace, size_t workspace_bytes,
                                        void *stream)
 {
+    if (d != 3) {
+        const pccnn_basis b = {PCCNN_BASIS_MLP, k, axis, bias, nullptr, 0, 0, 0, 1.0f, pdf};
+        return pccnn_conv_weight_var(&b, pts, feats, samples, neigh, ends, radii, n, m, t, d, c_in, 0, out, workspace,
+                                     workspace_bytes, stream);
+    }
     int rc = conv_validate("pccnn_mcconv_weight_var", n, m, t, d, c_in, k, 1, 1);
     if (rc != PCCNN_OK) return rc;
     PCCNN_REQUIRE(pts && pdf && feats && samples && ends && radii && axis && bias && out && (t == 0 || neigh),
@@ -1022,6 +1050,11 @@ extern "C" int pccnn_kpconv_forward(const float *pts, const float *feats, const 
                                     int c_out, float *out, float *proj_out, void *workspace, size_t workspace_bytes,
                                     void *stream)
 {
+    if (d != 3) {
+        const pccnn_basis b = {PCCNN_BASIS_KP, k, kernel_pts, nullptr, nullptr, 0, 0, 0, sigma, nullptr};
+        return conv_forward_entry("pccnn_kpconv_forward", false, &b, pts, feats, samples, neigh, ends, radii, weights, n,
+                                  m, t, d, c_in, 1, c_out, 0, out, proj_out, workspace, workspace_bytes, stream);
+    }
     int rc = conv_validate("pccnn_kpconv_forward", n, m, t, d, c_in, k, 1, c_out);
     if (rc != PCCNN_OK) return rc;
     PCCNN_REQUIRE(sigma > 0.0f, PCCNN_ERR_INVALID, "pccnn_kpconv_forward: sigma=%g", sigma);
@@ -1040,6 +1073,12 @@ extern "C" int pccnn_kpconv_backward(const float *pts, const float *feats, const
                                      float *d_weights, float *d_feats, float *d_kernel_pts, float *d_pts,
                                      float *d_samples, void *workspace, size_t workspace_bytes, void *stream)
 {
+    if (d != 3) {
+        const pccnn_basis b = {PCCNN_BASIS_KP, k, kernel_pts, nullptr, nullptr, 0, 0, 0, sigma, nullptr};
+        return conv_backward_entry("pccnn_kpconv_backward", false, &b, pts, feats, samples, neigh, ends, radii, weights,
+                                   in_grads, proj, mirror, grad_mask, n, m, t, d, c_in, 1, c_out, 0, d_weights, d_feats,
+                                   d_kernel_pts, nullptr, nullptr, d_pts, d_samples, workspace, workspace_bytes, stream);
+    }
     int rc = conv_validate("pccnn_kpconv_backward", n, m, t, d, c_in, k, 1, c_out);
     if (rc != PCCNN_OK) return rc;
     PCCNN_REQUIRE(mirror == nullptr || n == m, PCCNN_ERR_INVALID,
@@ -1065,6 +1104,11 @@ extern "C" int pccnn_mcconv_forward(const float *pts, const float *pdf, const fl
                                     int c_in, int k, int num_mlps, int c_out, float *out, float *proj_out,
                                     void *workspace, size_t workspace_bytes, void *stream)
 {
+    if (d != 3) {
+        const pccnn_basis b = {PCCNN_BASIS_MLP, k, axis, bias, nullptr, 0, 0, 0, 1.0f, pdf};
+        return conv_forward_entry("pccnn_mcconv_forward", false, &b, pts, feats, samples, neigh, ends, radii, weights, n,
+                                  m, t, d, c_in, num_mlps, c_out, 0, out, proj_out, workspace, workspace_bytes, stream);
+    }
     int rc = conv_validate("pccnn_mcconv_forward", n, m, t, d, c_in, k, num_mlps, c_out);
     if (rc != PCCNN_OK) return rc;
     PCCNN_REQUIRE(m == 0 || (pts && pdf && feats && samples && ends && radii && axis && bias && weights && out &&
@@ -1084,6 +1128,12 @@ extern "C" int pccnn_mcconv_backward(const float *pts, const float *pdf, const f
                                      float *d_pts, float *d_samples, void *workspace, size_t workspace_bytes,
                                      void *stream)
 {
+    if (d != 3) {
+        const pccnn_basis b = {PCCNN_BASIS_MLP, k, axis, bias, nullptr, 0, 0, 0, 1.0f, pdf};
+        return conv_backward_entry("pccnn_mcconv_backward", false, &b, pts, feats, samples, neigh, ends, radii, weights,
+                                   in_grads, proj, mirror, grad_mask, n, m, t, d, c_in, num_mlps, c_out, 0, d_weights,
+                                   d_feats, d_axis, d_bias, d_pdf, d_pts, d_samples, workspace, workspace_bytes, stream);
+    }
     int rc = conv_validate("pccnn_mcconv_backward", n, m, t, d, c_in, k, num_mlps, c_out);
     if (rc != PCCNN_OK) return rc;
     PCCNN_REQUIRE(mirror == nullptr || n == m, PCCNN_ERR_INVALID,
@@ -1101,6 +1151,203 @@ extern "C" int pccnn_mcconv_backward(const float *pts, const float *pdf, const f
     return conv_backward<BASIS_MLP>(g, feats, weights, in_grads, num_mlps, c_out, proj, grad_mask, d_weights, d_feats,
                                     d_axis, d_bias, d_pdf, d_pts, d_samples, workspace, workspace_bytes,
                                     (hipStream_t)stream, false, mirror);
+}
+
+// ---------------------------------------------------------------- other dimensions (2, 4, 5, 6)
+// The fused kernels above are written for three dimensions.  In any other dimension the basis is evaluated per
+// pair into a [T, K] tensor by the kernel below, the convolution then runs with that tensor as a caller-given basis
+// (the EXPLICIT family: projection, contraction, projection backward unchanged), and a second per-pair kernel turns
+// the basis gradient it returns into the point, sample, density and basis-parameter gradients.  Same formulas as
+// LaneBasis::eval and basis_derivative, with the sums over the dimensions in order from 0.
+
+struct PairGeom {
+    const float *pts, *samples;     // [n,d], [m,d]
+    const int2 *neigh;              // [t] (point, sample)
+    const float *radii;             // [d]
+    const float *pdf;               // [n] or null
+    const float *a, *b;             // kernel points [k,d] | axis [d,k]; bias [k]
+    float sigma;
+    int64_t t;
+    int d, k;
+};
+
+template <int BASIS>
+__global__ void __launch_bounds__(256)
+pair_basis_fwd_kernel(PairGeom g, float *__restrict__ basis)
+{
+#pragma clang fp contract(off)
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= g.t * g.k) return;
+    const int64_t t = idx / g.k;
+    const int k = (int)(idx - t * g.k);
+    const int2 pr = g.neigh[t];
+    float acc = 0.0f;
+    for (int i = 0; i < g.d; ++i) {
+        const float diff = (g.pts[(int64_t)pr.x * g.d + i] - g.samples[(int64_t)pr.y * g.d + i]) * (1.0f / g.radii[i]);
+        if (BasisTraits<BASIS>::kernel_pts) {
+            const float v = g.a[k * g.d + i] - diff;
+            acc = acc + v * v;
+        } else {
+            acc = acc + diff * g.a[i * g.k + k];
+        }
+    }
+    float w;
+    if (BASIS == BASIS_KP || BASIS == BASIS_KPN) {
+        const float r = 1.0f - sqrtf(fmaxf(acc, 0.0f)) / g.sigma;
+        w = fminf(fmaxf(r, 0.0f), 1.0f);
+        if (BASIS == BASIS_KPN) w = w / g.pdf[pr.x];
+    } else if (BASIS == BASIS_GAUSS) {
+        w = expf(-(acc / (2.0f * g.sigma * g.sigma))) / g.pdf[pr.x];
+    } else if (BASIS == BASIS_LINEAR) {
+        w = acc + g.b[k];
+    } else {
+        acc = acc + g.b[k];
+        acc = acc > 0.0f ? acc : acc * 0.2f;
+        w = acc / g.pdf[pr.x];
+    }
+    basis[idx] = w;
+}
+
+// One thread per pair, a loop over the basis index.  Parameter gradients are summed per workgroup in LDS
+// ([k][d + 1]) and flushed with one float atomic per entry; the point-side gradients are float atomics per pair.
+template <int BASIS>
+__global__ void __launch_bounds__(256)
+pair_basis_bwd_kernel(PairGeom g, const float *__restrict__ basis_grads, float *d_pts, float *d_samples,
+                      float *d_pdf, float *d_a, float *d_b)
+{
+#pragma clang fp contract(off)
+    __shared__ float part[64 * (PCCNN_MAX_DIMS + 1)];
+    const int comps = g.d + 1;
+    for (int i = threadIdx.x; i < g.k * comps; i += blockDim.x) part[i] = 0.0f;
+    __syncthreads();
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t < g.t) {
+        const int2 pr = g.neigh[t];
+        float diff[PCCNN_MAX_DIMS], ir[PCCNN_MAX_DIMS], gd[PCCNN_MAX_DIMS];
+        for (int i = 0; i < PCCNN_MAX_DIMS; ++i) {
+            diff[i] = 0.0f; ir[i] = 0.0f; gd[i] = 0.0f;
+            if (i < g.d) {
+                ir[i] = 1.0f / g.radii[i];
+                diff[i] = (g.pts[(int64_t)pr.x * g.d + i] - g.samples[(int64_t)pr.y * g.d + i]) * ir[i];
+            }
+        }
+        const float pdf = BasisTraits<BASIS>::uses_pdf ? g.pdf[pr.x] : 1.0f;
+        float gpdf = 0.0f;
+        for (int k = 0; k < g.k; ++k) {
+            const float gk = basis_grads[t * g.k + k];
+            if (BasisTraits<BASIS>::kernel_pts) {
+                float v[PCCNN_MAX_DIMS];
+                float acc = 0.0f;
+                for (int i = 0; i < PCCNN_MAX_DIMS; ++i) {
+                    v[i] = 0.0f;
+                    if (i < g.d) { v[i] = g.a[k * g.d + i] - diff[i]; acc = acc + v[i] * v[i]; }
+                }
+                float c = 0.0f;
+                if (BASIS == BASIS_GAUSS) {
+                    const float e = expf(-(acc / (2.0f * g.sigma * g.sigma)));
+                    gpdf += -((e / pdf) * gk) / pdf;
+                    c = -(gk / pdf) * e * (1.0f / (g.sigma * g.sigma));
+                } else {
+                    const float gin = (BASIS == BASIS_KPN) ? gk / pdf : gk;
+                    const float dist = sqrtf(fmaxf(acc, 0.0f));
+                    if (1.0f - dist / g.sigma >= 0.0f) c = -(gin / g.sigma) * (1.0f / (dist + 1e-6f));
+                }
+                for (int i = 0; i < PCCNN_MAX_DIMS; ++i)
+                    if (i < g.d) {
+                        const float ci = c * v[i];
+                        gd[i] -= ci;
+                        if (d_a && ci != 0.0f) atomicAdd(&part[k * comps + i], ci);
+                    }
+            } else {
+                float act = 0.0f;
+                for (int i = 0; i < PCCNN_MAX_DIMS; ++i)
+                    if (i < g.d) act = act + diff[i] * g.a[i * g.k + k];
+                act = act + g.b[k];
+                const bool pos = act > 0.0f || BASIS == BASIS_LINEAR;
+                act = pos ? act : act * 0.2f;
+                const float inv_pd = 1.0f / pdf;
+                gpdf += -(act * gk * inv_pd * inv_pd);
+                const float c = gk * inv_pd * (pos ? 1.0f : 0.2f);
+                for (int i = 0; i < PCCNN_MAX_DIMS; ++i)
+                    if (i < g.d) {
+                        gd[i] += c * g.a[i * g.k + k];
+                        if (d_a) atomicAdd(&part[k * comps + i], diff[i] * c);
+                    }
+                if (d_b) atomicAdd(&part[k * comps + g.d], c);
+            }
+        }
+        for (int i = 0; i < PCCNN_MAX_DIMS; ++i)
+            if (i < g.d) {
+                const float v = gd[i] * ir[i];
+                if (d_pts) unsafeAtomicAdd(&d_pts[(int64_t)pr.x * g.d + i], v);
+                if (d_samples) unsafeAtomicAdd(&d_samples[(int64_t)pr.y * g.d + i], -v);
+            }
+        if (BasisTraits<BASIS>::pdf_grad && d_pdf) unsafeAtomicAdd(&d_pdf[pr.x], gpdf);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < g.k * comps; i += blockDim.x) {
+        const int k = i / comps, c = i - k * comps;
+        const float v = part[i];
+        if (v == 0.0f) continue;
+        if (c < g.d) {
+            // kernel points are stored [k][d], axis matrices [d][k]
+            if (d_a) unsafeAtomicAdd(&d_a[BasisTraits<BASIS>::kernel_pts ? k * g.d + c : c * g.k + k], v);
+        } else if (d_b) {
+            unsafeAtomicAdd(&d_b[k], v);
+        }
+    }
+}
+
+#define PAIR_BASIS_LINEAR (-1)   // PointConv's affine basis; not one of the public PCCNN_BASIS_* kinds
+
+static bool pair_basis_kind(int kind)
+{
+    return kind == PCCNN_BASIS_KP || kind == PCCNN_BASIS_MLP || kind == PCCNN_BASIS_KPN || kind == PCCNN_BASIS_GAUSS;
+}
+
+static int pair_basis_forward(int kind, const PairGeom &g, float *basis, hipStream_t s)
+{
+    if (g.t == 0) return PCCNN_OK;
+    const unsigned blocks = (unsigned)pccnn_ceil_div(g.t * g.k, 256);
+    switch (kind) {
+    case PCCNN_BASIS_KP: pair_basis_fwd_kernel<BASIS_KP><<<blocks, 256, 0, s>>>(g, basis); break;
+    case PCCNN_BASIS_MLP: pair_basis_fwd_kernel<BASIS_MLP><<<blocks, 256, 0, s>>>(g, basis); break;
+    case PCCNN_BASIS_KPN: pair_basis_fwd_kernel<BASIS_KPN><<<blocks, 256, 0, s>>>(g, basis); break;
+    case PAIR_BASIS_LINEAR: pair_basis_fwd_kernel<BASIS_LINEAR><<<blocks, 256, 0, s>>>(g, basis); break;
+    default: pair_basis_fwd_kernel<BASIS_GAUSS><<<blocks, 256, 0, s>>>(g, basis); break;
+    }
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
+static int pair_basis_backward(int kind, const PairGeom &g, const float *basis_grads, float *d_pts, float *d_samples,
+                               float *d_pdf, float *d_a, float *d_b, hipStream_t s)
+{
+    if (g.t == 0) return PCCNN_OK;
+    const unsigned blocks = (unsigned)pccnn_ceil_div(g.t, 256);
+    switch (kind) {
+    case PCCNN_BASIS_KP:
+        pair_basis_bwd_kernel<BASIS_KP><<<blocks, 256, 0, s>>>(g, basis_grads, d_pts, d_samples, d_pdf, d_a, d_b); break;
+    case PCCNN_BASIS_MLP:
+        pair_basis_bwd_kernel<BASIS_MLP><<<blocks, 256, 0, s>>>(g, basis_grads, d_pts, d_samples, d_pdf, d_a, d_b); break;
+    case PCCNN_BASIS_KPN:
+        pair_basis_bwd_kernel<BASIS_KPN><<<blocks, 256, 0, s>>>(g, basis_grads, d_pts, d_samples, d_pdf, d_a, d_b); break;
+    case PAIR_BASIS_LINEAR:
+        pair_basis_bwd_kernel<BASIS_LINEAR><<<blocks, 256, 0, s>>>(g, basis_grads, d_pts, d_samples, d_pdf, d_a, d_b); break;
+    default:
+        pair_basis_bwd_kernel<BASIS_GAUSS><<<blocks, 256, 0, s>>>(g, basis_grads, d_pts, d_samples, d_pdf, d_a, d_b); break;
+    }
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
+// The part of a workspace that is left after `bytes` have been set aside at its start.
+static void *ws_after(void *workspace, size_t workspace_bytes, size_t bytes, size_t &rest)
+{
+    bytes = pccnn_align(bytes);
+    if (workspace == nullptr || workspace_bytes < bytes) { rest = 0; return nullptr; }
+    rest = workspace_bytes - bytes;
+    return (char *)workspace + bytes;
 }
 
 // ------------------------------------------------------------------- generic entry points
@@ -1155,6 +1402,24 @@ static int conv_forward_entry(const char *who, bool bf16, const pccnn_basis *bas
     const bool geom = basis->kind != PCCNN_BASIS_EXPLICIT;
     PCCNN_REQUIRE(m == 0 || (feats && ends && weights && out && (t == 0 || neigh) && (!geom || (pts && samples && radii))),
                   PCCNN_ERR_INVALID, "%s: null pointer", who);
+    if (d != 3 && geom) {
+        // basis per pair, then the convolution on it as a caller-given basis
+        PCCNN_REQUIRE(pair_basis_kind(basis->kind), PCCNN_ERR_UNSUPPORTED, "%s: basis kind %d needs 3 dimensions (d=%d)",
+                      who, basis->kind, d);
+        if (m == 0) return PCCNN_OK;
+        size_t rest = 0;
+        void *ws = ws_after(workspace, workspace_bytes, (size_t)(t > 0 ? t : 1) * g.k * sizeof(float), rest);
+        PCCNN_REQUIRE(ws != nullptr, PCCNN_ERR_WORKSPACE, "%s: workspace of %zu bytes, need %zu", who, workspace_bytes,
+                      pccnn_conv_workspace_bytes(m, t, c_in, g.k, c_out, 0));
+        float *pair_w = (float *)workspace;
+        const PairGeom pg = {pts, samples, (const int2 *)neigh, radii, basis->pdf, basis->a, basis->b, basis->sigma, t, d,
+                             g.k};
+        if ((rc = pair_basis_forward(basis->kind, pg, pair_w, (hipStream_t)stream)) != PCCNN_OK) return rc;
+        ConvGeom ge = {nullptr, nullptr, (const int2 *)neigh, ends, nullptr, nullptr, pair_w, nullptr, 1.0f, n, m, t,
+                       c_in, g.k};
+        return conv_forward<BASIS_EXPLICIT>(ge, feats, weights, num_mlps, c_out, out, proj_out, ws, rest,
+                                            (hipStream_t)stream, divide_by_count != 0, bf16);
+    }
 #define CALL(B) conv_forward<B>(g, feats, weights, num_mlps, c_out, out, proj_out, workspace, workspace_bytes, \
                                 (hipStream_t)stream, divide_by_count != 0, bf16)
     BASIS_DISPATCH(basis->kind, CALL)
@@ -1213,6 +1478,40 @@ static int conv_backward_entry(const char *who, bool bf16, const pccnn_basis *ba
                       (!(grad_mask & PCCNN_GRAD_PDF) || !has_pdf || d_pdf || n == 0) &&
                       (!(grad_mask & PCCNN_GRAD_PTS) || !has_pts || ((d_pts || n == 0) && (d_samples || m == 0))),
                   PCCNN_ERR_INVALID, "%s: a requested gradient has a null output pointer", who);
+    if (d != 3 && geom) {
+        PCCNN_REQUIRE(pair_basis_kind(kind), PCCNN_ERR_UNSUPPORTED, "%s: basis kind %d needs 3 dimensions (d=%d)", who,
+                      kind, d);
+        hipStream_t s = (hipStream_t)stream;
+        const bool want_par = grad_mask & PCCNN_GRAD_BASIS_PARAMS, want_pts = grad_mask & PCCNN_GRAD_PTS;
+        const bool want_pdf = (grad_mask & PCCNN_GRAD_PDF) && has_pdf;
+        const bool want_basis = want_par || want_pts || want_pdf;
+        // outputs of the per-pair stage are accumulated with atomics: they start at zero
+        if (want_pts && (rc = pccnn_fill_f32(d_pts, 0.0f, n * d, s)) != PCCNN_OK) return rc;
+        if (want_pts && (rc = pccnn_fill_f32(d_samples, 0.0f, m * d, s)) != PCCNN_OK) return rc;
+        if (want_pdf && (rc = pccnn_fill_f32(d_pdf, 0.0f, n, s)) != PCCNN_OK) return rc;
+        if (want_par && (rc = pccnn_fill_f32(d_param_a, 0.0f, (int64_t)g.k * d, s)) != PCCNN_OK) return rc;
+        if (want_par && kind == PCCNN_BASIS_MLP && (rc = pccnn_fill_f32(d_param_b, 0.0f, g.k, s)) != PCCNN_OK) return rc;
+        const size_t tk = (size_t)(t > 0 ? t : 1) * g.k * sizeof(float);
+        size_t rest = 0;
+        void *ws = ws_after(workspace, workspace_bytes, 2 * pccnn_align(tk), rest);
+        PCCNN_REQUIRE(ws != nullptr, PCCNN_ERR_WORKSPACE, "%s: workspace of %zu bytes, need %zu", who, workspace_bytes,
+                      pccnn_conv_workspace_bytes(m, t, c_in, g.k, c_out, 1));
+        float *pair_w = (float *)workspace;
+        float *pair_g = (float *)((char *)workspace + pccnn_align(tk));
+        const PairGeom pg = {pts, samples, (const int2 *)neigh, radii, basis->pdf, basis->a, basis->b, basis->sigma, t, d,
+                             g.k};
+        if (m > 0 && (rc = pair_basis_forward(kind, pg, pair_w, s)) != PCCNN_OK) return rc;
+        ConvGeom ge = {nullptr, nullptr, (const int2 *)neigh, ends, nullptr, nullptr, pair_w, nullptr, 1.0f, n, m, t,
+                       c_in, g.k};
+        const int mask = (grad_mask & (PCCNN_GRAD_WEIGHTS | PCCNN_GRAD_FEATS)) | (want_basis ? PCCNN_GRAD_BASIS_PARAMS : 0);
+        rc = conv_backward<BASIS_EXPLICIT>(ge, feats, weights, in_grads, num_mlps, c_out, proj, mask, d_weights, d_feats,
+                                           pair_g, nullptr, nullptr, nullptr, nullptr, ws, rest, s, divide_by_count != 0,
+                                           nullptr, bf16);
+        if (rc != PCCNN_OK || !want_basis || m == 0 || t == 0) return rc;
+        return pair_basis_backward(kind, pg, pair_g, want_pts ? d_pts : nullptr, want_pts ? d_samples : nullptr,
+                                   want_pdf ? d_pdf : nullptr, want_par ? d_param_a : nullptr,
+                                   want_par ? d_param_b : nullptr, s);
+    }
 #define CALL(B) conv_backward<B>(g, feats, weights, in_grads, num_mlps, c_out, proj, grad_mask, d_weights, d_feats, \
                                  d_param_a, d_param_b, d_pdf, d_pts, d_samples, workspace, workspace_bytes,           \
                                  (hipStream_t)stream, divide_by_count != 0, mirror, bf16)
@@ -1262,6 +1561,21 @@ extern "C" int pccnn_conv_weight_var(const pccnn_basis *basis, const float *pts,
     const bool geom = basis->kind != PCCNN_BASIS_EXPLICIT;
     PCCNN_REQUIRE(feats && ends && out && (t == 0 || neigh) && (!geom || (pts && samples && radii)), PCCNN_ERR_INVALID,
                   "pccnn_conv_weight_var: null pointer");
+    if (d != 3 && geom) {
+        PCCNN_REQUIRE(pair_basis_kind(basis->kind), PCCNN_ERR_UNSUPPORTED,
+                      "pccnn_conv_weight_var: basis kind %d needs 3 dimensions (d=%d)", basis->kind, d);
+        size_t rest = 0;
+        void *ws = ws_after(workspace, workspace_bytes, (size_t)(t > 0 ? t : 1) * g.k * sizeof(float), rest);
+        PCCNN_REQUIRE(ws != nullptr, PCCNN_ERR_WORKSPACE, "pccnn_conv_weight_var: workspace of %zu bytes, need %zu",
+                      workspace_bytes, pccnn_conv_weight_var_workspace_bytes(m, t, c_in, g.k));
+        float *pair_w = (float *)workspace;
+        const PairGeom pg = {pts, samples, (const int2 *)neigh, radii, basis->pdf, basis->a, basis->b, basis->sigma, t, d,
+                             g.k};
+        if ((rc = pair_basis_forward(basis->kind, pg, pair_w, (hipStream_t)stream)) != PCCNN_OK) return rc;
+        ConvGeom ge = {nullptr, nullptr, (const int2 *)neigh, ends, nullptr, nullptr, pair_w, nullptr, 1.0f, n, m, t,
+                       c_in, g.k};
+        return conv_weight_var<BASIS_EXPLICIT>(ge, feats, out, ws, rest, (hipStream_t)stream, divide_by_count != 0);
+    }
 #define CALL(B) conv_weight_var<B>(g, feats, out, workspace, workspace_bytes, (hipStream_t)stream, divide_by_count != 0)
     BASIS_DISPATCH(basis->kind, CALL)
 #undef CALL
@@ -1275,6 +1589,10 @@ extern "C" int pccnn_linear_basis_forward(const float *pts, const float *samples
     if (rc != PCCNN_OK || t == 0) return rc;
     PCCNN_REQUIRE(pts && samples && neigh && radii && axis && bias && basis_out, PCCNN_ERR_INVALID,
                   "pccnn_linear_basis_forward: null pointer");
+    if (d != 3) {
+        const PairGeom pg = {pts, samples, (const int2 *)neigh, radii, nullptr, axis, bias, 1.0f, t, d, k};
+        return pair_basis_forward(PAIR_BASIS_LINEAR, pg, basis_out, (hipStream_t)stream);
+    }
     ConvGeom g = {pts, samples, (const int2 *)neigh, nullptr, radii, nullptr, axis, bias, 1.0f, n, m, t, 1, k};
     linear_basis_fwd_kernel<<<(unsigned)pccnn_ceil_div(t * k, 256), 256, 0, (hipStream_t)stream>>>(g, basis_out);
     PCCNN_LAUNCH_CHECK();
@@ -1299,11 +1617,13 @@ extern "C" int pccnn_linear_basis_backward(const float *pts, const float *sample
                       (t == 0 || (neigh && basis_grads)),
                   PCCNN_ERR_INVALID, "pccnn_linear_basis_backward: null pointer");
     hipStream_t s = (hipStream_t)stream;
-    if ((rc = pccnn_fill_f32(d_pts, 0.0f, n * 3, s)) != PCCNN_OK) return rc;
-    if ((rc = pccnn_fill_f32(d_samples, 0.0f, m * 3, s)) != PCCNN_OK) return rc;
-    if (t == 0) {
-        if ((rc = pccnn_fill_f32(d_axis, 0.0f, 3 * k, s)) != PCCNN_OK) return rc;
-        return pccnn_fill_f32(d_bias, 0.0f, k, s);
+    if ((rc = pccnn_fill_f32(d_pts, 0.0f, n * d, s)) != PCCNN_OK) return rc;
+    if ((rc = pccnn_fill_f32(d_samples, 0.0f, m * d, s)) != PCCNN_OK) return rc;
+    if (t == 0 || d != 3) {
+        if ((rc = pccnn_fill_f32(d_axis, 0.0f, (int64_t)d * k, s)) != PCCNN_OK) return rc;
+        if ((rc = pccnn_fill_f32(d_bias, 0.0f, k, s)) != PCCNN_OK || t == 0) return rc;
+        const PairGeom pg = {pts, samples, (const int2 *)neigh, radii, nullptr, axis, bias, 1.0f, t, d, k};
+        return pair_basis_backward(PAIR_BASIS_LINEAR, pg, basis_grads, d_pts, d_samples, nullptr, d_axis, d_bias, s);
     }
     const int kpad = kpad_of(k);
     int64_t blocks = pccnn_ceil_div(t, (int64_t)4 * (64 / kpad) * 8);

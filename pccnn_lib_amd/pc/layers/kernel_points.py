@@ -2,8 +2,8 @@
 
 The reference ships hard-coded layouts for K in {8, 16, 32, 64}
 (pccnn_lib/pc/layers/kernel_points/kernel_points.py); this build generates its own, deterministically:
-one centre point plus K - 1 points on one Fibonacci-lattice shell (K <= 16) or on two shells of radius
-0.5 and 1 (K > 16).  Any K in [2, 64] is available.  A layout only has to start with the centre point:
+one centre point plus K - 1 points on one shell (K <= 16) or on two shells of radius 0.5 and 1 (K > 16), in 2 to 6
+dimensions (the reference's table covers 2, 3 and 4).  Any K in [2, 64] is available.  A layout only has to start with the centre point:
 the layer normalises it by its largest norm (pccnn_lib/pc/layers/KPConv.py:46-57)."""
 import numpy as np
 
@@ -20,14 +20,46 @@ def _circle(count, phase=0.0):
     return np.stack([np.cos(a), np.sin(a)], axis=1)
 
 
+def _hypersphere(num_dims, count):
+    """`count` directions spread over the unit sphere of `num_dims` >= 4 dimensions: a low-discrepancy sequence
+    (additive recurrence on the roots of x^(n+1) = x + 1) pushed through Box-Muller and normalised, then evened out by
+    a fixed number of repulsion steps along the sphere.  Deterministic: no random numbers."""
+    if count == 0:
+        return np.zeros((0, num_dims))
+    cols = 2 * ((num_dims + 1) // 2)
+    g = 2.0
+    for _ in range(64):
+        g = (1.0 + g) ** (1.0 / (cols + 1))
+    alpha = (1.0 / g) ** np.arange(1, cols + 1)
+    u = np.mod(0.5 + np.outer(np.arange(1, count + 1), alpha), 1.0)
+    r = np.sqrt(-2.0 * np.log(np.maximum(u[:, 0::2], 1e-12)))
+    a = 2.0 * np.pi * u[:, 1::2]
+    x = np.concatenate([r * np.cos(a), r * np.sin(a)], axis=1)[:, :num_dims]
+    x /= np.linalg.norm(x, axis=1, keepdims=True)
+    for step in range(200):
+        diff = x[:, None, :] - x[None, :, :]
+        dist2 = np.sum(diff * diff, axis=-1) + np.eye(count)
+        force = np.sum(diff / dist2[..., None] ** 1.5, axis=1)
+        force -= np.sum(force * x, axis=1, keepdims=True) * x          # keep the step on the sphere
+        norm = np.linalg.norm(force, axis=1, keepdims=True)
+        x = x + 0.1 * (0.98 ** step) * force / np.maximum(norm.max(), 1e-12)
+        x /= np.linalg.norm(x, axis=1, keepdims=True)
+    return x
+
+
 def kernel_points(num_dims, num_kernel_pts):
     """A centre point plus one shell (up to 16 points) or two shells (inner one at half the radius) of evenly
-    spread directions: on the unit sphere in 3 dimensions, on the unit circle in 2."""
-    if num_dims not in (2, 3):
-        raise RuntimeError("kernel point layouts exist for 2 and 3 dimensions only")
+    spread directions: on the unit circle in 2 dimensions, the unit sphere in 3, the unit hypersphere beyond."""
+    if not 2 <= num_dims <= 6:
+        raise RuntimeError("kernel point layouts exist for 2 to 6 dimensions")
     if not 2 <= num_kernel_pts <= 64:
         raise RuntimeError("the number of kernel points must lie in [2, 64]")
-    spread = _fibonacci_sphere if num_dims == 3 else _circle
+    if num_dims == 2:
+        spread = _circle
+    elif num_dims == 3:
+        spread = _fibonacci_sphere
+    else:
+        spread = lambda count: _hypersphere(num_dims, count)
     rest = num_kernel_pts - 1
     if num_kernel_pts <= 16:
         shell = spread(rest)

@@ -317,11 +317,26 @@ GRAD_WEIGHTS, GRAD_FEATS, GRAD_BASIS_PARAMS, GRAD_PDF, GRAD_PTS, GRAD_ALL = 1, 2
 
 
 
-def _conv_dims(pts, name):
+def _conv_dims(pts, name, only_3d=False):
     d = pts.shape[1]
-    if d != 3:
-        raise RuntimeError("%s: %d-dimensional points are not supported by the convolutions (2 or 3)" % (name, d))
+    if d < MIN_DIMS or d > MAX_DIMS or (only_3d and d != 3):
+        raise RuntimeError("%s: %d-dimensional points are not supported (%s)"
+                           % (name, d, "3 only" if only_3d else "%d to %d" % (MIN_DIMS, MAX_DIMS)))
     return d
+
+
+def _forward_workspace(pts, m, t, c_in, k, c_out, dev):
+    """(pointer, bytes) of the forward call's workspace: only clouds that are not 3-D need one, for the per-pair
+    basis (the projection is an output tensor here).  Returns the tensor too, to keep it alive over the call."""
+    if pts is None or pts.shape[1] == 3:
+        return _P(0), 0, None
+    ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 0), dev)
+    return _ptr(ws), ws.numel(), ws
+
+
+def _dims_of(pts):
+    """Dimension argument of the generic entry points; a caller-given basis has no geometry."""
+    return 3 if pts is None else pts.shape[1]
 
 
 # Planar clouds run through the 3-D kernels with a zero third coordinate: positions, samples and kernel points get
@@ -385,9 +400,10 @@ def kp_conv(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights,
         return (out, proj) if return_proj else out
     out = torch.empty((m, c_out), dtype=torch.float32, device=dev)
     proj = torch.empty((m, c_in, k), dtype=torch.float32, device=dev)
+    ws_p, ws_n, _ws = _forward_workspace(pts, m, t, c_in, k, c_out, dev)
     _lib.call("pccnn_kpconv_forward", _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends), _ptr(radii),
               _ptr(kernel_pts), float(sigma), _ptr(weights), n, m, t, d, c_in, k, c_out, _ptr(out), _ptr(proj),
-              _P(0), 0, _stream())
+              ws_p, ws_n, _stream())
     return (out, proj) if return_proj else out
 
 
@@ -399,8 +415,8 @@ def _bf16_forward(name, desc, pts, feats, samples, neigh, ends, radii, weights, 
     proj = torch.empty((m, c_in, k), dtype=torch.bfloat16, device=dev)
     ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 0), dev)
     _lib.call("pccnn_conv_forward_bf16", ctypes.byref(desc), _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh),
-              _ptr(ends), _ptr(radii), _ptr(weights), n, m, t, 3, c_in, num_mlps, c_out, 0, _ptr(out), _ptr(proj),
-              _ptr(ws), ws.numel(), _stream())
+              _ptr(ends), _ptr(radii), _ptr(weights), n, m, t, _dims_of(pts), c_in, num_mlps, c_out, 0, _ptr(out),
+              _ptr(proj), _ptr(ws), ws.numel(), _stream())
     return out, proj
 
 
@@ -412,7 +428,7 @@ def _bf16_backward(name, desc, pts, feats, samples, neigh, ends, radii, weights,
     ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
     _lib.call("pccnn_conv_backward_bf16", ctypes.byref(desc), _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh),
               _ptr(ends), _ptr(radii), _ptr(weights), _ptr(in_grads), proj_p,
-              _mirror_arg(name, mirror, neigh, pts, samples), grad_mask, n, m, t, 3, c_in, num_mlps, c_out, 0,
+              _mirror_arg(name, mirror, neigh, pts, samples), grad_mask, n, m, t, _dims_of(pts), c_in, num_mlps, c_out, 0,
               _optr(d_w), _optr(d_f), _optr(d_a), _optr(d_b), _optr(d_pdf), _optr(d_p), _optr(d_s), _ptr(ws),
               ws.numel(), _stream())
 
@@ -532,9 +548,10 @@ def mc_conv(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights, r
         return (out, proj) if return_proj else out
     out = torch.empty((m, c_out), dtype=torch.float32, device=dev)
     proj = torch.empty((m, c_in, k), dtype=torch.float32, device=dev)
+    ws_p, ws_n, _ws = _forward_workspace(pts, m, t, c_in, k, c_out, dev)
     _lib.call("pccnn_mcconv_forward", _ptr(pts), _ptr(pdf), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends),
               _ptr(radii), _ptr(axis), _ptr(bias), _ptr(weights), n, m, t, d, c_in, k, num_mlps, c_out, _ptr(out),
-              _ptr(proj), _P(0), 0, _stream())
+              _ptr(proj), ws_p, ws_n, _stream())
     return (out, proj) if return_proj else out
 
 
@@ -586,7 +603,7 @@ def kp_conv_weight_var(pts, feats, samples, neigh, ends, radii, kernel_pts, sigm
     if kernel_pts.shape[1] != d:
         raise RuntimeError(name + ": kernel_pts must be [K, D]")
     out = torch.empty((1,), dtype=torch.float32, device=dev)
-    ws = _workspace(_lib.load().pccnn_conv_weight_var_workspace_bytes(m, c_in, k), dev)
+    ws = _workspace(_lib.load().pccnn_conv_weight_var_workspace_bytes(m, t, c_in, k), dev)
     _lib.call("pccnn_kpconv_weight_var", _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends), _ptr(radii),
               _ptr(kernel_pts), float(sigma), n, m, t, d, c_in, k, _ptr(out), _ptr(ws), ws.numel(), _stream())
     return out.reshape(())
@@ -607,7 +624,7 @@ def mc_conv_weight_var(pts, pdf, feats, samples, neigh, ends, radii, axis, bias)
     if pdf.shape[0] != n or axis.shape[0] != d or tuple(bias.shape) != (1, k):
         raise RuntimeError(name + ": axis must be [D, H*mlps], bias [1, H*mlps], pdf [N]")
     out = torch.empty((1,), dtype=torch.float32, device=dev)
-    ws = _workspace(_lib.load().pccnn_conv_weight_var_workspace_bytes(m, c_in, k), dev)
+    ws = _workspace(_lib.load().pccnn_conv_weight_var_workspace_bytes(m, t, c_in, k), dev)
     _lib.call("pccnn_mcconv_weight_var", _ptr(pts), _ptr(pdf), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends),
               _ptr(radii), _ptr(axis), _ptr(bias), n, m, t, d, c_in, k, _ptr(out), _ptr(ws), ws.numel(), _stream())
     return out.reshape(())
@@ -636,9 +653,10 @@ def _generic_forward(name, desc, k, pts, feats, samples, neigh, ends, radii, wei
         raise RuntimeError(name + ": weights must be [K*Cin, Cout]")
     out = torch.empty((m, c_out), dtype=torch.float32, device=dev)
     proj = torch.empty((m, c_in, k), dtype=torch.float32, device=dev)
+    ws_p, ws_n, _ws = _forward_workspace(pts, m, t, c_in, k, c_out, dev)
     _lib.call("pccnn_conv_forward", ctypes.byref(desc), _optr(pts), _ptr(feats), _optr(samples), _ptr(neigh),
-              _ptr(ends), _optr(radii), _ptr(weights), n, m, t, 3, c_in, 1, c_out, int(divide_by_count), _ptr(out),
-              _ptr(proj), _P(0), 0, _stream())
+              _ptr(ends), _optr(radii), _ptr(weights), n, m, t, _dims_of(pts), c_in, 1, c_out, int(divide_by_count),
+              _ptr(out), _ptr(proj), ws_p, ws_n, _stream())
     return (out, proj) if return_proj else out
 
 
@@ -659,7 +677,8 @@ def _generic_backward(name, desc, k, pts, feats, samples, neigh, ends, radii, we
     ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
     _lib.call("pccnn_conv_backward", ctypes.byref(desc), _optr(pts), _ptr(feats), _optr(samples), _ptr(neigh),
               _ptr(ends), _optr(radii), _ptr(weights), _ptr(in_grads), proj_p,
-              _mirror_arg(name, mirror, neigh, pts, samples) if with_pts else _P(0), grad_mask, n, m, t, 3, c_in, 1, c_out,
+              _mirror_arg(name, mirror, neigh, pts, samples) if with_pts else _P(0), grad_mask, n, m, t, _dims_of(pts), c_in, 1,
+              c_out,
               int(divide_by_count), _optr(d_w), _optr(d_f), _optr(d_param_a), _P(0), _optr(d_pdf), _optr(d_p),
               _optr(d_s), _ptr(ws), ws.numel(), _stream())
     return d_w, d_f, d_p, d_s
@@ -669,9 +688,9 @@ def _generic_weight_var(name, desc, k, pts, feats, samples, neigh, ends, radii, 
     dev = feats.device
     n, m, t, c_in = feats.shape[0], ends.shape[0], neigh.shape[0], feats.shape[1]
     out = torch.empty((1,), dtype=torch.float32, device=dev)
-    ws = _workspace(_lib.load().pccnn_conv_weight_var_workspace_bytes(m, c_in, k), dev)
+    ws = _workspace(_lib.load().pccnn_conv_weight_var_workspace_bytes(m, t, c_in, k), dev)
     _lib.call("pccnn_conv_weight_var", ctypes.byref(desc), _optr(pts), _ptr(feats), _optr(samples), _ptr(neigh),
-              _ptr(ends), _optr(radii), n, m, t, 3, c_in, int(divide_by_count), _ptr(out), _ptr(ws), ws.numel(),
+              _ptr(ends), _optr(radii), n, m, t, _dims_of(pts), c_in, int(divide_by_count), _ptr(out), _ptr(ws), ws.numel(),
               _stream())
     return out.reshape(())
 
@@ -770,6 +789,7 @@ def pccnn_weight_variance(pts, feats, pdf, samples, neigh, ends, radii, kernel_p
 
 def _sph_args(name, pts, feats, samples, neigh, ends, radii, radial_bins, azimuth_bins, polar_bins):
     d, dev = _conv_args(name, pts, feats, samples, neigh, ends, radii)
+    _conv_dims(pts, name, only_3d=True)      # spherical coordinates
     for b, what in ((radial_bins, "radial"), (azimuth_bins, "azimuth"), (polar_bins, "polar")):
         _chk(b, "%s: %s bins" % (name, what), torch.float32, 1, dev)
         if b.shape[0] < 1:

@@ -203,3 +203,141 @@ def test_planar_layers(oracle):
     assert relerr(p(out_mc), exp) < 1e-5
     assert tuple(pc.pts_.grad.shape) == pts.shape and bool(torch.isfinite(pc.pts_.grad).all())
     assert tuple(tf.grad.shape) == feats.shape
+
+
+def _kernel_points(dims, k):
+    from pccnn_lib_amd.pc.layers.kernel_points import kernel_points
+    kp = kernel_points(dims, k)
+    return (kp / (2.0 * np.linalg.norm(kp, axis=1).max())).astype(np.float32)
+
+
+@pytest.mark.parametrize("dims,radius,distinct", [(4, 0.3, False), (4, 0.3, True), (5, 0.45, True), (6, 0.6, False)])
+def test_convolutions_beyond_three_dimensions(ops, oracle, dims, radius, distinct):
+    # The reference's convolution tests run in 4 dimensions too (unit_test/utest_kpconv.ini Test_4, utest_mcconv.ini
+    # Test_4).  There the basis is evaluated per pair and the convolution runs on it as a caller-given basis.
+    pts, ids = _cloud(dims, 2, 700, 500 + dims)
+    rng = np.random.default_rng(dims)
+    if distinct:
+        pick = np.sort(rng.choice(pts.shape[0], pts.shape[0] // 3, replace=False))
+        smp, sids = pts[pick].copy(), ids[pick]
+    else:
+        smp, sids = pts, ids
+    nb = gpu_neighborhood(ops, pts, ids, smp, sids, radius, 2)
+    neigh, ends, radii, d = nb["neighbors"], nb["ends"], nb["radii"], nb["dev"]
+    assert neigh.shape[0] > 4 * smp.shape[0]
+    c_in, c_out, k = 12, 10, 16
+    feats = rng.normal(size=(pts.shape[0], c_in)).astype(np.float32)
+    g = rng.normal(size=(smp.shape[0], c_out)).astype(np.float32)
+    kp, sigma = _kernel_points(dims, k), 0.5
+    w = rng.normal(0, np.sqrt(1.0 / (k * c_in)), (k * c_in, c_out)).astype(np.float32)
+    pdf = rng.uniform(0.5, 2.0, pts.shape[0]).astype(np.float32)
+
+    def check(grads, expect, names):
+        for got, e, name in zip(grads, expect, names):
+            assert tuple(got.shape) == e.shape, name
+            assert relerr(got.cpu().numpy(), e) < 1e-4, name
+
+    # KPConv, against the oracle and against the closed form the reference's own test uses (unit_test/test_kpconv.py:63-80)
+    args = (d["pts"], t(feats), d["samples"], d["neigh"], d["ends"], d["radii"], t(kp), sigma, t(w))
+    host = (pts, feats, smp, neigh, ends, radii, kp, sigma, w)
+    out = ops.kp_conv(*args).cpu().numpy()
+    assert relerr(out, oracle.kpconv(*host)) < 1e-5
+    diff = (pts[neigh[:, 0]].astype(np.float64) - smp[neigh[:, 1]]) / radii
+    corr = np.clip(1.0 - np.linalg.norm(diff[:, None, :] - kp[None], axis=-1) / sigma, 0.0, 1.0)
+    proj = np.zeros((smp.shape[0], c_in, k))
+    np.add.at(proj, neigh[:, 1], feats[neigh[:, 0]][:, :, None] * corr[:, None, :])
+    closed = proj.reshape(smp.shape[0], -1) @ w.astype(np.float64)
+    assert relerr(out, closed) < 1e-5
+    check(ops.kp_conv_grads(*args, t(g)), oracle.kpconv_grads(*host, g), ("dW", "dFeat", "dKernelPts", "dPts", "dSamples"))
+    assert relerr(ops.kp_conv_weight_var(*args[:-1]).cpu().numpy(), oracle.kpconv_weight_var(*host[:-1])) < 1e-4
+    part = ops.kp_conv_grads(*args, t(g), grad_mask=ops.GRAD_WEIGHTS | ops.GRAD_PTS)
+    assert part[1] is None and part[2] is None
+    full = oracle.kpconv_grads(*host, g)
+    assert relerr(part[0].cpu().numpy(), full[0]) < 1e-4 and relerr(part[3].cpu().numpy(), full[3]) < 1e-4
+
+    # MCConv with two MLPs
+    axis = rng.normal(0, np.sqrt(1.0 / dims), (dims, k)).astype(np.float32)
+    bias = rng.normal(0, 0.1, (1, k)).astype(np.float32)
+    wm = rng.normal(0, np.sqrt(2.0 / (k * c_in)), (2, k * c_in // 2, c_out // 2)).astype(np.float32)
+    margs = (d["pts"], t(pdf), t(feats), d["samples"], d["neigh"], d["ends"], d["radii"], t(axis), t(bias), t(wm))
+    mhost = (pts, pdf, feats, smp, neigh, ends, radii, axis, bias, wm)
+    assert relerr(ops.mc_conv(*margs).cpu().numpy(), oracle.mcconv(*mhost)) < 1e-5
+    check(ops.mc_conv_grads(*margs, t(g)), oracle.mcconv_grads(*mhost, g),
+          ("dW", "dFeat", "dAxis", "dBias", "dPdf", "dPts", "dSamples"))
+    assert relerr(ops.mc_conv_weight_var(*margs[:-1]).cpu().numpy(), oracle.mcconv_weight_var(*mhost[:-1])) < 1e-4
+    out16 = ops.mc_conv(*margs, contraction="bf16").cpu().numpy()
+    assert relerr(out16, oracle.mcconv(*mhost, contraction="bf16")) < 3e-3
+
+    # KPConvN and PCCNN through the generic entry points
+    nargs = (d["pts"], t(pdf), t(feats), d["samples"], d["neigh"], d["ends"], d["radii"], t(kp), sigma, t(w))
+    assert relerr(ops.kp_conv_n(*nargs).cpu().numpy(),
+                  oracle.kpconvn(pts, pdf, feats, smp, neigh, ends, radii, kp, sigma, w)) < 1e-5
+    check(ops.kp_conv_n_grads(*nargs, t(g)), oracle.kpconvn_grads(pts, pdf, feats, smp, neigh, ends, radii, kp, sigma, w, g),
+          ("dW", "dFeat", "dKernelPts", "dPts", "dSamples"))
+    var = ops.kp_conv_n_weight_var(*nargs[:-1])
+    exp = oracle.kpconvn_weight_var(pts, pdf, feats, smp, neigh, ends, radii, kp, sigma)
+    assert abs(float(var) - float(exp)) < 1e-4 * abs(float(exp))
+    gargs = (d["pts"], t(feats), t(pdf), d["samples"], d["neigh"], d["ends"], d["radii"], t(kp), 0.35, t(w))
+    assert relerr(ops.pccnn(*gargs).cpu().numpy(),
+                  oracle.pccnn(pts, feats, pdf, smp, neigh, ends, radii, kp, 0.35, w)) < 1e-5
+    check(ops.pccnn_grads(*gargs, t(g)), oracle.pccnn_grads(pts, feats, pdf, smp, neigh, ends, radii, kp, 0.35, w, g),
+          ("dW", "dFeat", "dKernelPts", "dPdf", "dPts", "dSamples"))
+
+    # PointConv's basis op
+    bargs = (d["pts"], d["radii"], d["samples"], d["neigh"], t(axis), t(bias))
+    exp_basis, _ = oracle.pointconv_basis(pts, radii, smp, neigh, axis, bias)
+    assert relerr(ops.point_conv_basis(*bargs).cpu().numpy(), exp_basis) < 1e-5
+    gb = rng.normal(size=exp_basis.shape).astype(np.float32)
+    check(ops.point_conv_basis_grads(*bargs, t(gb)), oracle.pointconv_basis_grads(pts, radii, smp, neigh, axis, bias, gb),
+          ("dPts", "dSamples", "dAxis", "dBias"))
+
+    # spherical bins need three coordinates
+    edges = t(np.array([0.5, 1.0], np.float32))
+    with pytest.raises(RuntimeError):
+        ops.sph_conv(d["pts"], t(feats), d["samples"], d["neigh"], d["ends"], d["radii"], edges, edges, edges,
+                     t(rng.normal(size=(9 * c_in, c_out)).astype(np.float32)))
+
+
+def test_empty_neighborhood_in_four_dimensions(ops):
+    pts = t(np.random.default_rng(0).uniform(size=(50, 4)).astype(np.float32))
+    feats = torch.ones((50, 4), device=DEV)
+    none = torch.zeros((0, 2), dtype=torch.int32, device=DEV)
+    ends = torch.zeros((50,), dtype=torch.int32, device=DEV)
+    radii = torch.full((4,), 0.1, device=DEV)
+    kp = t(_kernel_points(4, 8))
+    w = torch.ones((8 * 4, 3), device=DEV)
+    assert float(ops.kp_conv(pts, feats, pts, none, ends, radii, kp, 0.5, w).abs().max()) == 0.0
+    grads = ops.kp_conv_grads(pts, feats, pts, none, ends, radii, kp, 0.5, w, torch.ones((50, 3), device=DEV))
+    assert all(float(x.abs().max()) == 0.0 for x in grads)
+    assert tuple(grads[3].shape) == (50, 4) and tuple(grads[2].shape) == (8, 4)
+
+
+def test_layers_in_four_dimensions(oracle):
+    # the shape of the reference's 4-D cases: unit_test/utest_kpconv.ini Test_4, utest_mcconv.ini Test_4
+    import pccnn_lib_amd as lib
+    pts, ids = _cloud(4, 4, 250, 33)
+    rng = np.random.default_rng(33)
+    feats = rng.normal(size=(pts.shape[0], 32)).astype(np.float32)
+    pc = lib.pc.Pointcloud(pts, ids, device=DEV, requires_grad=True)
+    pc.compute_pdf(np.full(4, 0.1, np.float32))
+    torch.manual_seed(5)
+    kp_layer = lib.pc.layers.KPConv(4, 32, 4, 16).to(DEV)
+    mc_layer = lib.pc.layers.MCConv(4, 32, 4, 8).to(DEV)
+    tf = t(feats).requires_grad_(True)
+    out_kp, nbh = kp_layer(pc, pc, tf, 0.25)
+    out_mc = mc_layer(pc, pc, tf, 0.25, nbh)
+    (out_kp.sum() + out_mc.sum()).backward()
+    p = lambda x: x.detach().cpu().numpy()
+    radii = np.full(4, 0.25, np.float32)
+    neigh, ends = p(nbh.neighbors_), p(nbh.start_ids_)
+    kp, sigma, w = p(kp_layer.kernel_pts_), float(kp_layer.sigma_.item()), p(kp_layer.conv_weights_)
+    assert relerr(p(out_kp), oracle.kpconv(pts, feats, pts, neigh, ends, radii, kp, sigma, w)) < 1e-5
+    pdf = p(pc.pts_unnorm_pdf_ * torch.prod(t(radii)))
+    exp = oracle.mcconv(pts, pdf, feats, pts, neigh, ends, radii, p(mc_layer.proj_axis_), p(mc_layer.proj_bias_),
+                        p(mc_layer.conv_weights_))
+    assert relerr(p(out_mc), exp) < 1e-5
+    ones = np.ones((pts.shape[0], 4), np.float32)
+    e_kp = oracle.kpconv_grads(pts, feats, pts, neigh, ends, radii, kp, sigma, w, ones)
+    assert relerr(p(kp_layer.conv_weights_.grad), e_kp[0]) < 1e-4
+    assert tuple(pc.pts_.grad.shape) == pts.shape and bool(torch.isfinite(pc.pts_.grad).all())
+    assert tuple(tf.grad.shape) == feats.shape

@@ -308,7 +308,7 @@ def test_error_paths(ops):
     with pytest.raises(RuntimeError, match="dtype"):
         ops.compute_keys(tp, ti.to(torch.int64), tp[:1], torch.ones(3, dtype=torch.int32, device=DEV), tp[0])
     with pytest.raises(RuntimeError, match="not supported"):
-        ops.bounding_box(tp[:, :2].contiguous(), ti, 1)
+        ops.bounding_box(tp[:, :1].contiguous(), ti, 1)
     with pytest.raises(RuntimeError, match="contiguous"):
         ops.bounding_box(tp.t().contiguous().t(), ti, 1)
     nb = gpu_neighborhood(ops, pts, ids, pts, ids, 0.2, 1)["dev"]
