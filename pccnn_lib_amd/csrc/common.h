@@ -86,6 +86,77 @@ __device__ __forceinline__ long long pccnn_bcast_ll(long long v, int src)
     return ((long long)hi << 32) | (unsigned int)lo;
 }
 
+// ---- sums over groups of lanes without going through the LDS crossbar ----------------------------------------
+// A wavefront is four rows of sixteen lanes.  Inside a row, data-parallel-primitive operands (quad permutes, row
+// rotations, mirrors) come for free with the add; between rows, gfx950's row swaps (v_permlane16_swap: odd rows of
+// the first operand <-> even rows of the second; v_permlane32_swap: upper half of the first <-> lower half of the
+// second) exchange whole rows in one instruction.  All lanes must be active.
+template <int CTRL>
+__device__ __forceinline__ float pccnn_dpp(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+#define PCCNN_DPP_QUAD_XOR1 0xb1      // quad_perm [1,0,3,2]
+#define PCCNN_DPP_QUAD_XOR2 0x4e      // quad_perm [2,3,0,1]
+#define PCCNN_DPP_ROW_ROR(n) (0x120 + (n))
+#define PCCNN_DPP_ROW_MIRROR 0x140
+#define PCCNN_DPP_ROW_HALF_MIRROR 0x141
+
+// v + (v of the row 16 lanes away), in every lane: rows {0,1} and {2,3} are paired.
+__device__ __forceinline__ float pccnn_add_row_xor16(float v)
+{
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+// v + (v of the lane 32 away), in every lane.
+__device__ __forceinline__ float pccnn_add_row_xor32(float v)
+{
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// Sum over each aligned group of WIDTH consecutive lanes (WIDTH a power of two, 1..64), left in every lane of the
+// group.  The mirrors act as exchanges with the other half because the halves are uniform by then.
+template <int WIDTH>
+__device__ __forceinline__ float pccnn_group_sum(float v)
+{
+    if (WIDTH >= 2) v += pccnn_dpp<PCCNN_DPP_QUAD_XOR1>(v);
+    if (WIDTH >= 4) v += pccnn_dpp<PCCNN_DPP_QUAD_XOR2>(v);
+    if (WIDTH >= 8) v += pccnn_dpp<PCCNN_DPP_ROW_HALF_MIRROR>(v);
+    if (WIDTH >= 16) v += pccnn_dpp<PCCNN_DPP_ROW_MIRROR>(v);
+    if (WIDTH >= 32) v = pccnn_add_row_xor16(v);
+    if (WIDTH >= 64) v = pccnn_add_row_xor32(v);
+    return v;
+}
+
+// Sum over the lanes that share (lane % STRIDE) (STRIDE a power of two, 1..64), left in every one of them.
+// Inside a row the cosets are closed under rotation, so rotations by STRIDE, 2 STRIDE, ... add them up.
+template <int STRIDE>
+__device__ __forceinline__ float pccnn_strided_sum(float v)
+{
+    if (STRIDE <= 1) v += pccnn_dpp<PCCNN_DPP_ROW_ROR(1)>(v);
+    if (STRIDE <= 2) v += pccnn_dpp<PCCNN_DPP_ROW_ROR(2)>(v);
+    if (STRIDE <= 4) v += pccnn_dpp<PCCNN_DPP_ROW_ROR(4)>(v);
+    if (STRIDE <= 8) v += pccnn_dpp<PCCNN_DPP_ROW_ROR(8)>(v);
+    if (STRIDE <= 16) v = pccnn_add_row_xor16(v);
+    if (STRIDE <= 32) v = pccnn_add_row_xor32(v);
+    return v;
+}
+
+// Four values, each to be summed over the four rows (lanes l, l + 16, l + 32, l + 48): three row swaps and three
+// adds do all four at once.  On return the lanes of row r hold the sum of value pccnn_rows4_slot(r).
+__device__ __forceinline__ float pccnn_rows4_sum(float a0, float a1, float a2, float a3)
+{
+    const auto p = __builtin_amdgcn_permlane32_swap(__float_as_uint(a0), __float_as_uint(a1), false, false);
+    const auto q = __builtin_amdgcn_permlane32_swap(__float_as_uint(a2), __float_as_uint(a3), false, false);
+    // rows of u: a0(r0+r2), a0(r1+r3), a1(r0+r2), a1(r1+r3); v likewise for a2, a3
+    const float u = __uint_as_float(p[0]) + __uint_as_float(p[1]);
+    const float v = __uint_as_float(q[0]) + __uint_as_float(q[1]);
+    const auto w = __builtin_amdgcn_permlane16_swap(__float_as_uint(u), __float_as_uint(v), false, false);
+    return __uint_as_float(w[0]) + __uint_as_float(w[1]);          // rows: a0, a2, a1, a3
+}
+__device__ __forceinline__ int pccnn_rows4_slot(int row) { return ((row & 1) << 1) | (row >> 1); }
+
 // fp32 -> bf16 bit pattern, round to nearest even; a NaN stays a (quiet) NaN.
 __device__ __forceinline__ uint16_t pccnn_bf16_bits(float f)
 {

@@ -130,6 +130,7 @@ conv_proj_fwd_kernel(ConvGeom g, const float *__restrict__ feats, void *__restri
     constexpr int PARTS = 64 / KPAD;
     constexpr int ROWS = 4;
     __shared__ __attribute__((aligned(16))) float w_lds[64][KPAD];
+    __shared__ float4 geo_lds[64];                      // (offset, density) of the chunk's pairs
     const int lane = threadIdx.x;
     const int64_t s = blockIdx.x;
     const int f = blockIdx.y * 64 + lane;
@@ -163,12 +164,13 @@ conv_proj_fwd_kernel(ConvGeom g, const float *__restrict__ feats, void *__restri
             }
             if (BasisTraits<BASIS>::uses_pdf) pd = g.pdf[nidx];
         }
+        if (GEOM) geo_lds[lane] = make_float4(dx, dy, dz, pd);
+        __syncthreads();
         for (int p = 0; p * PARTS < cnt; ++p) {
-            const int j = p * PARTS + part;
-            // the shuffles stay outside the condition: every lane must take part, a lane that sits out
-            // would hand zeros to the lanes reading from it
-            const float jx = __shfl(dx, j), jy = __shfl(dy, j), jz = __shfl(dz, j), jp = __shfl(pd, j);
-            const float w = (j < cnt) ? pair_basis<BASIS>(g, lb, (int64_t)cb + j, jx, jy, jz, jp) : 0.0f;
+            const int j = p * PARTS + part;             // < 64: PARTS divides 64 and p * PARTS < cnt <= 64
+            float4 ge = make_float4(0.f, 0.f, 0.f, 1.f);
+            if (GEOM) ge = geo_lds[j];
+            const float w = (j < cnt) ? pair_basis<BASIS>(g, lb, (int64_t)cb + j, ge.x, ge.y, ge.z, ge.w) : 0.0f;
             w_lds[j][k] = w;
         }
         __syncthreads();
@@ -311,6 +313,8 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
     constexpr bool FUSED = want_db && BasisTraits<BASIS>::differentiable;   // basis derivative applied here
     constexpr int CH = 32;                                          // pairs staged in LDS at a time
     __shared__ __attribute__((aligned(16))) float g_lds[FUSED ? CH : 1][4];
+    __shared__ float4 geo_lds[CH];                                  // (offset, density) of the chunk's pairs
+    __shared__ int nidx_lds[CH];                                    // and their points
     // want_df / want_db: which of the two stages this instantiation runs
     constexpr int PARTS = 64 / KPAD;                                // feature groups of the dw stage
     constexpr int ROWS = 4;                                         // feature rows in flight
@@ -347,17 +351,19 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
             }
             if (BasisTraits<BASIS>::uses_pdf) pd = g.pdf[nidx];
         }
-        // basis values of the chunk: pass p evaluates pairs p*PARTS .. p*PARTS + PARTS - 1
+        if (lane < CH) {
+            if (GEOM) geo_lds[lane] = make_float4(dx, dy, dz, pd);
+            nidx_lds[lane] = nidx;
+        }
+        __syncthreads();
+        // basis values of the chunk: pass p evaluates pairs p*PARTS .. p*PARTS + PARTS - 1 (all below CH: PARTS
+        // divides CH and p * PARTS < cnt <= CH)
         for (int p = 0; p * PARTS < cnt; ++p) {
             const int j = p * PARTS + part;
-            // the shuffles stay outside the condition: every lane must take part, a lane that sits out
-            // would hand zeros to the lanes reading from it
-            const float jx = __shfl(dx, j), jy = __shfl(dy, j), jz = __shfl(dz, j), jp = __shfl(pd, j);
-            const float w = (j < cnt) ? pair_basis<BASIS>(g, lb, (int64_t)cb + j, jx, jy, jz, jp) : 0.0f;
-            if (j < CH) {
-                w_lds[j][k] = w;
-                if (want_db) db_lds[j][k] = 0.0f;
-            }
+            float4 ge = make_float4(0.f, 0.f, 0.f, 1.f);
+            if (GEOM) ge = geo_lds[j];
+            const float w = (j < cnt) ? pair_basis<BASIS>(g, lb, (int64_t)cb + j, ge.x, ge.y, ge.z, ge.w) : 0.0f;
+            w_lds[j][k] = w;
         }
         __syncthreads();
         for (int fb = 0; fb < fblocks; ++fb) {
@@ -380,11 +386,18 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
                         if (q < g.k) gp[q] = src[q];
                 }
             }
-            if (want_db && k < g.k) {
+            if (want_db) {
+                if (g.k == KPAD && (g.c_in & 63) == 0) {
+                    // full tile: one base address, the KPAD loads differ by constants
+                    const float *col = proj_grads + ((int64_t)s * g.c_in + fb * 64 + part * KPAD) * KPAD + k;
 #pragma unroll
-                for (int q = 0; q < KPAD; ++q) {
-                    const int ft = fb * 64 + part * KPAD + q;
-                    if (ft < g.c_in) gt[q] = proj_grads[((int64_t)s * g.c_in + ft) * g.k + k];
+                    for (int q = 0; q < KPAD; ++q) gt[q] = col[q * KPAD];
+                } else if (k < g.k) {
+#pragma unroll
+                    for (int q = 0; q < KPAD; ++q) {
+                        const int ft = fb * 64 + part * KPAD + q;
+                        if (ft < g.c_in) gt[q] = proj_grads[((int64_t)s * g.c_in + ft) * g.k + k];
+                    }
                 }
             }
             for (int j0 = 0; j0 < cnt; j0 += ROWS) {
@@ -400,11 +413,11 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
                     for (int u = 0; u < ROWS; ++u) row_lds[u][lane] = row[u];
                     __syncthreads();
                 }
+                if (want_df) {
 #pragma unroll
-                for (int u = 0; u < ROWS; ++u) {
-                    const int j = j0 + u;
-                    if (j < cnt) {                                  // uniform
-                        if (want_df) {
+                    for (int u = 0; u < ROWS; ++u) {
+                        const int j = j0 + u;
+                        if (j < cnt) {                              // uniform
                             float gf = 0.0f;
 #pragma unroll
                             for (int q = 0; q < KPAD; q += 4) {
@@ -413,16 +426,33 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
                             }
                             if (fvalid) unsafeAtomicAdd(&feat_grads[(int64_t)bn[u] * g.c_in + f], gf);
                         }
-                        if (want_db) {
-                            float acc = 0.0f;
+                    }
+                }
+                if (want_db) {
+                    // this lane's share (its KPAD features) of db[j0 + u][k]; rows past the chunk hold zeros
+                    float part_sum[ROWS];
+#pragma unroll
+                    for (int u = 0; u < ROWS; ++u) {
+                        float acc = 0.0f;
+                        if (j0 + u < cnt) {                         // uniform
 #pragma unroll
                             for (int q = 0; q < KPAD; q += 4) {
                                 const float4 rv = *(const float4 *)&row_lds[u][part * KPAD + q];
                                 acc += gt[q] * rv.x + gt[q + 1] * rv.y + gt[q + 2] * rv.z + gt[q + 3] * rv.w;
                             }
+                        }
+                        part_sum[u] = acc;
+                    }
+                    // summed over the feature groups (lanes k, k + KPAD, ...); the first feature block writes
+                    if (PARTS == 4 && ROWS == 4) {
+                        const float tot = pccnn_rows4_sum(part_sum[0], part_sum[1], part_sum[2], part_sum[3]);
+                        const int j = j0 + pccnn_rows4_slot(part);
+                        if (j < cnt) db_lds[j][k] = (fb == 0) ? tot : db_lds[j][k] + tot;
+                    } else {
 #pragma unroll
-                            for (int o = KPAD; o < 64; o <<= 1) acc += __shfl_xor(acc, o);
-                            if (part == 0) db_lds[j][k] += acc;
+                        for (int u = 0; u < ROWS; ++u) {
+                            const float tot = pccnn_strided_sum<KPAD>(part_sum[u]);
+                            if (part == 0 && j0 + u < cnt) db_lds[j0 + u][k] = (fb == 0) ? tot : db_lds[j0 + u][k] + tot;
                         }
                     }
                 }
@@ -433,24 +463,22 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
         if (FUSED) {
             for (int p = 0; p * PARTS < cnt; ++p) {
                 const int j = p * PARTS + part;
-                const float jx = __shfl(dx, j), jy = __shfl(dy, j), jz = __shfl(dz, j), jp = __shfl(pd, j);
+                const float4 ge = geo_lds[j];
                 float gx = 0.f, gy = 0.f, gz = 0.f, gpdf = 0.f;
                 if (j < cnt && lb.active)
-                    basis_derivative<BASIS>(g, lb, jx, jy, jz, jp, db_lds[j][k], gx, gy, gz, gpdf, p0, p1, p2, p3);
-#pragma unroll
-                for (int o = KPAD / 2; o > 0; o >>= 1) {
-                    gx += __shfl_xor(gx, o);
-                    gy += __shfl_xor(gy, o);
-                    gz += __shfl_xor(gz, o);
-                    if (BasisTraits<BASIS>::pdf_grad) gpdf += __shfl_xor(gpdf, o);
-                }
-                if (k < 4 && j < CH) g_lds[j][k] = (k == 0) ? gx * ir0 : (k == 1) ? gy * ir1 : (k == 2) ? gz * ir2 : gpdf;
+                    basis_derivative<BASIS>(g, lb, ge.x, ge.y, ge.z, ge.w, db_lds[j][k], gx, gy, gz, gpdf, p0, p1, p2, p3);
+                // summed over the basis index: the KPAD lanes of this pair
+                gx = pccnn_group_sum<KPAD>(gx);
+                gy = pccnn_group_sum<KPAD>(gy);
+                gz = pccnn_group_sum<KPAD>(gz);
+                if (BasisTraits<BASIS>::pdf_grad) gpdf = pccnn_group_sum<KPAD>(gpdf);
+                if (k < 4) g_lds[j][k] = (k == 0) ? gx * ir0 : (k == 1) ? gy * ir1 : (k == 2) ? gz * ir2 : gpdf;
             }
             __syncthreads();
             for (int i = 0; i * 16 < cnt; ++i) {
                 const int j = i * 16 + (lane >> 2), comp = lane & 3;
-                const int jn = __shfl(nidx, j);
                 if (j < cnt) {
+                    const int jn = nidx_lds[j];
                     const float v = g_lds[j][comp];
                     if (comp < 3) sg += v;
                     if (pair_grads) {
@@ -472,17 +500,13 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
         __syncthreads();
     }
     if (FUSED) {
-#pragma unroll
-        for (int o = 4; o < 64; o <<= 1) sg += __shfl_xor(sg, o);
+        sg = pccnn_strided_sum<4>(sg);
         if (lane < 3 && d_samples) d_samples[s * 3 + lane] = -sg;
         if (param_partials) {
-#pragma unroll
-            for (int o = KPAD; o < 64; o <<= 1) {
-                p0 += __shfl_xor(p0, o);
-                p1 += __shfl_xor(p1, o);
-                p2 += __shfl_xor(p2, o);
-                if (BasisTraits<BASIS>::axis) p3 += __shfl_xor(p3, o);
-            }
+            p0 = pccnn_strided_sum<KPAD>(p0);
+            p1 = pccnn_strided_sum<KPAD>(p1);
+            p2 = pccnn_strided_sum<KPAD>(p2);
+            if (BasisTraits<BASIS>::axis) p3 = pccnn_strided_sum<KPAD>(p3);
             float *row = param_partials + (int64_t)(blockIdx.x % PARAM_ROWS) * 256;
             constexpr int COMPS = BasisTraits<BASIS>::axis ? 4 : 3;
             for (int c = part; c < COMPS; c += PARTS) {
@@ -514,7 +538,9 @@ mirror_pairs_kernel(const int2 *__restrict__ neigh, const int32_t *__restrict__ 
 }
 
 // d_pts[n] and d_pdf[n] of a symmetric neighborhood: the pairs in which n is the point are the mirrors of
-// the pairs of sample n.  Four lanes per point, one per component of the per-pair values.
+// the pairs of sample n.  Four lanes per point: lane q adds the (x, y, z, density) records of the pairs
+// q, q + 4, ... of the segment (16-byte loads, independent between the lanes), two exchanges add the four
+// partial sums in a fixed order, and lane q stores component q.
 __global__ void __launch_bounds__(256)
 conv_point_gather_kernel(const float *__restrict__ pair_grads, const int32_t *__restrict__ mirror,
                          const int32_t *__restrict__ ends, int64_t m, float *__restrict__ d_pts,
@@ -522,15 +548,29 @@ conv_point_gather_kernel(const float *__restrict__ pair_grads, const int32_t *__
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t n = i >> 2;
-    const int comp = (int)(i & 3);
+    const int q = (int)(i & 3);
+    float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (n < m) {
+        const int lo = n > 0 ? ends[n - 1] : 0, hi = ends[n];
+        const float4 *rec = (const float4 *)pair_grads;
+        for (int j = lo + q; j < hi; j += 4) {
+            const float4 v = rec[mirror[j]];
+            acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+        }
+    }
+#pragma unroll
+    for (int o = 1; o < 4; o <<= 1) {
+        acc.x += __shfl_xor(acc.x, o);
+        acc.y += __shfl_xor(acc.y, o);
+        acc.z += __shfl_xor(acc.z, o);
+        acc.w += __shfl_xor(acc.w, o);
+    }
     if (n >= m) return;
-    const int lo = n > 0 ? ends[n - 1] : 0, hi = ends[n];
-    float acc = 0.0f;
-    for (int j = lo; j < hi; ++j) acc += pair_grads[(int64_t)mirror[j] * 4 + comp];
-    if (comp < 3) {
-        if (d_pts) d_pts[n * 3 + comp] = acc;
+    const float v = (q == 0) ? acc.x : (q == 1) ? acc.y : (q == 2) ? acc.z : acc.w;
+    if (q < 3) {
+        if (d_pts) d_pts[n * 3 + q] = v;
     } else if (d_pdf) {
-        d_pdf[n] = acc;
+        d_pdf[n] = v;
     }
 }
 
@@ -807,6 +847,19 @@ extern "C" size_t pccnn_conv_workspace_bytes(int64_t m, int64_t t, int c_in, int
 
 // out[m, c_out] = P[m, c_in*k] x W, with the feature axis split over num_mlps independent
 // weight blocks (num_mlps == 1 is the plain product).
+// Split of the sample dimension for d_weights = P^T x dOut, whose output ([K*Cin, Cout]) has few tiles: enough
+// workgroups for about four per CU, but at least 2048 samples each, so that the partial sums written and summed
+// again stay small beside the product itself.
+static int conv_split_k(int64_t inner, int64_t co, int num_mlps, int64_t m)
+{
+    if (m < 4096) return 1;
+    const int64_t tiles = pccnn_ceil_div(inner, 64) * pccnn_ceil_div(co, 128) * num_mlps;
+    int64_t split = 1024 / tiles;
+    if (split > m / 2048) split = m / 2048;
+    if (split > CONV_SPLIT_K) split = CONV_SPLIT_K;
+    return (int)(split < 1 ? 1 : split);
+}
+
 static int contraction_fwd(const float *proj, const float *weights, float *out, int64_t m, int c_in, int k,
                            int num_mlps, int c_out, hipStream_t s)
 {
@@ -918,7 +971,7 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
             if ((rc = launch_proj_fwd<BASIS>(g, feats, proj_ws, s, bf16)) != PCCNN_OK) return rc;
             proj = proj_ws;
         }
-        const int split = (int)(g.m >= 4096 ? CONV_SPLIT_K : 1);
+        const int split = conv_split_k(inner, co, num_mlps, g.m);
         if (bf16)
             rc = pccnn_gemm_bf16((const uint16_t *)proj, g16, d_weights, inner, co, g.m, 1, 0, (int64_t)g.c_in * g.k,
                                  c_out, co, num_mlps, inner, co, inner * co, split, splitk,
