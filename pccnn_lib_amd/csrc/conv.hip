@@ -151,12 +151,24 @@ conv_proj_fwd_kernel(ConvGeom g, const float *__restrict__ feats, void *__restri
 #pragma unroll
     for (int q = 0; q < KPAD; ++q) acc[q] = 0.0f;
 
+    // Feature rows of the pairs j0 .. j0 + ROWS - 1 of the chunk (zeros past its end).
+    auto load_rows = [&](int j0, int cnt, int nidx, float (&row)[ROWS]) {
+#pragma unroll
+        for (int u = 0; u < ROWS; ++u) {
+            const int bn = pccnn_bcast_i(nidx, (j0 + u) < cnt ? (j0 + u) : 0);
+            row[u] = (fvalid && (j0 + u) < cnt) ? feats[(int64_t)bn * g.c_in + f] : 0.0f;
+        }
+    };
+
     for (int cb = lo; cb < hi; cb += 64) {
         const int cnt = (hi - cb) < 64 ? (hi - cb) : 64;
         int nidx = 0;
         float dx = 0.f, dy = 0.f, dz = 0.f, pd = 1.0f;
+        if (lane < cnt) nidx = g.neigh[cb + lane].x;
+        // the first rows leave before the basis is evaluated; from then on one group is always in flight
+        float row[ROWS];
+        load_rows(0, cnt, nidx, row);
         if (lane < cnt) {
-            nidx = g.neigh[cb + lane].x;
             if (GEOM) {
                 dx = (g.pts[(int64_t)nidx * 3 + 0] - sx) * ir0;
                 dy = (g.pts[(int64_t)nidx * 3 + 1] - sy) * ir1;
@@ -175,12 +187,9 @@ conv_proj_fwd_kernel(ConvGeom g, const float *__restrict__ feats, void *__restri
         }
         __syncthreads();
         for (int j0 = 0; j0 < cnt; j0 += ROWS) {
-            float row[ROWS];
-#pragma unroll
-            for (int u = 0; u < ROWS; ++u) {
-                const int bn = pccnn_bcast_i(nidx, (j0 + u) < cnt ? (j0 + u) : 0);
-                row[u] = (fvalid && (j0 + u) < cnt) ? feats[(int64_t)bn * g.c_in + f] : 0.0f;
-            }
+            float row_next[ROWS];
+            const bool more = j0 + ROWS < cnt;                      // uniform
+            if (more) load_rows(j0 + ROWS, cnt, nidx, row_next);
 #pragma unroll
             for (int u = 0; u < ROWS; ++u) {
                 if (j0 + u < cnt) {                                 // uniform
@@ -193,6 +202,10 @@ conv_proj_fwd_kernel(ConvGeom g, const float *__restrict__ feats, void *__restri
                         acc[q + 3] += row[u] * wv.w;
                     }
                 }
+            }
+            if (more) {
+#pragma unroll
+                for (int u = 0; u < ROWS; ++u) row[u] = row_next[u];
             }
         }
         __syncthreads();
@@ -338,12 +351,64 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
     float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;       // parameter gradients of this lane's k (FUSED)
     float sg = 0.f;                                     // component (lane & 3) of the sample's gradient, unsigned
 
+    // The sample's tile of the projection gradient: row f = this lane's feature (gp, for the dF stage) and column
+    // k of the features of this lane's group (gt, for the dw stage).  With one feature block it is loaded once,
+    // first thing, so that it travels while the pair list is read.
+    auto load_tile = [&](int fb, float (&gp)[KPAD], float (&gt)[KPAD]) {
+        const int f = fb * 64 + lane;
+#pragma unroll
+        for (int q = 0; q < KPAD; ++q) { gp[q] = 0.0f; gt[q] = 0.0f; }
+        if (f < g.c_in) {
+            const float *src = proj_grads + ((int64_t)s * g.c_in + f) * g.k;
+            if (g.k == KPAD && (KPAD % 4) == 0) {
+#pragma unroll
+                for (int q = 0; q < KPAD; q += 4) {
+                    const float4 v = *(const float4 *)(src + q);
+                    gp[q] = v.x; gp[q + 1] = v.y; gp[q + 2] = v.z; gp[q + 3] = v.w;
+                }
+            } else {
+#pragma unroll
+                for (int q = 0; q < KPAD; ++q)
+                    if (q < g.k) gp[q] = src[q];
+            }
+        }
+        if (want_db) {
+            if (g.k == KPAD && (g.c_in & 63) == 0) {
+                // full tile: one base address, the KPAD loads differ by constants
+                const float *col = proj_grads + ((int64_t)s * g.c_in + fb * 64 + part * KPAD) * KPAD + k;
+#pragma unroll
+                for (int q = 0; q < KPAD; ++q) gt[q] = col[q * KPAD];
+            } else if (k < g.k) {
+#pragma unroll
+                for (int q = 0; q < KPAD; ++q) {
+                    const int ft = fb * 64 + part * KPAD + q;
+                    if (ft < g.c_in) gt[q] = proj_grads[((int64_t)s * g.c_in + ft) * g.k + k];
+                }
+            }
+        }
+    };
+    // Feature rows of the pairs j0 .. j0 + ROWS - 1 of the chunk (zeros past its end).
+    auto load_rows = [&](int fb, int j0, int cnt, int nidx, float (&row)[ROWS], int (&bn)[ROWS]) {
+        const int f = fb * 64 + lane;
+#pragma unroll
+        for (int u = 0; u < ROWS; ++u) {
+            bn[u] = pccnn_bcast_i(nidx, (j0 + u) < cnt ? (j0 + u) : 0);
+            row[u] = (f < g.c_in && (j0 + u) < cnt) ? feats[(int64_t)bn[u] * g.c_in + f] : 0.0f;
+        }
+    };
+    float gp[KPAD], gt[KPAD];
+    if (hi > lo) load_tile(0, gp, gt);
+
     for (int cb = lo; cb < hi; cb += CH) {
         const int cnt = (hi - cb) < CH ? (hi - cb) : CH;
         int nidx = 0;
         float dx = 0.f, dy = 0.f, dz = 0.f, pd = 1.0f;
+        if (lane < cnt) nidx = g.neigh[cb + lane].x;
+        // the first rows leave before the basis is evaluated; from then on one group is always in flight
+        float row[ROWS];
+        int bn[ROWS];
+        load_rows(0, 0, cnt, nidx, row, bn);
         if (lane < cnt) {
-            nidx = g.neigh[cb + lane].x;
             if (GEOM) {
                 dx = (g.pts[(int64_t)nidx * 3 + 0] - sx) * ir0;
                 dy = (g.pts[(int64_t)nidx * 3 + 1] - sy) * ir1;
@@ -369,45 +434,15 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
         for (int fb = 0; fb < fblocks; ++fb) {
             const int f = fb * 64 + lane;
             const bool fvalid = f < g.c_in;
-            float gp[KPAD], gt[KPAD];
-#pragma unroll
-            for (int q = 0; q < KPAD; ++q) { gp[q] = 0.0f; gt[q] = 0.0f; }
-            if (fvalid) {
-                const float *src = proj_grads + ((int64_t)s * g.c_in + f) * g.k;
-                if (g.k == KPAD && (KPAD % 4) == 0) {
-#pragma unroll
-                    for (int q = 0; q < KPAD; q += 4) {
-                        const float4 v = *(const float4 *)(src + q);
-                        gp[q] = v.x; gp[q + 1] = v.y; gp[q + 2] = v.z; gp[q + 3] = v.w;
-                    }
-                } else {
-#pragma unroll
-                    for (int q = 0; q < KPAD; ++q)
-                        if (q < g.k) gp[q] = src[q];
-                }
-            }
-            if (want_db) {
-                if (g.k == KPAD && (g.c_in & 63) == 0) {
-                    // full tile: one base address, the KPAD loads differ by constants
-                    const float *col = proj_grads + ((int64_t)s * g.c_in + fb * 64 + part * KPAD) * KPAD + k;
-#pragma unroll
-                    for (int q = 0; q < KPAD; ++q) gt[q] = col[q * KPAD];
-                } else if (k < g.k) {
-#pragma unroll
-                    for (int q = 0; q < KPAD; ++q) {
-                        const int ft = fb * 64 + part * KPAD + q;
-                        if (ft < g.c_in) gt[q] = proj_grads[((int64_t)s * g.c_in + ft) * g.k + k];
-                    }
-                }
+            if (fblocks > 1) {
+                load_tile(fb, gp, gt);
+                if (fb > 0) load_rows(fb, 0, cnt, nidx, row, bn);
             }
             for (int j0 = 0; j0 < cnt; j0 += ROWS) {
-                float row[ROWS];
-                int bn[ROWS];
-#pragma unroll
-                for (int u = 0; u < ROWS; ++u) {
-                    bn[u] = pccnn_bcast_i(nidx, (j0 + u) < cnt ? (j0 + u) : 0);
-                    row[u] = (fvalid && (j0 + u) < cnt) ? feats[(int64_t)bn[u] * g.c_in + f] : 0.0f;
-                }
+                float row_next[ROWS];
+                int bn_next[ROWS];
+                const bool more = j0 + ROWS < cnt;                  // uniform
+                if (more) load_rows(fb, j0 + ROWS, cnt, nidx, row_next, bn_next);
                 if (want_db) {
 #pragma unroll
                     for (int u = 0; u < ROWS; ++u) row_lds[u][lane] = row[u];
@@ -457,6 +492,10 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
                     }
                 }
                 if (want_db) __syncthreads();
+                if (more) {
+#pragma unroll
+                    for (int u = 0; u < ROWS; ++u) { row[u] = row_next[u]; bn[u] = bn_next[u]; }
+                }
             }
         }
         __syncthreads();
