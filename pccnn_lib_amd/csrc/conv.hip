@@ -887,11 +887,12 @@ extern "C" size_t pccnn_conv_workspace_bytes(int64_t m, int64_t t, int c_in, int
 // out[m, c_out] = P[m, c_in*k] x W, with the feature axis split over num_mlps independent
 // weight blocks (num_mlps == 1 is the plain product).
 // Split of the sample dimension for d_weights = P^T x dOut, whose output ([K*Cin, Cout]) has few tiles: enough
-// workgroups for about four per CU, but at least 2048 samples each, so that the partial sums written and summed
-// again stay small beside the product itself.
-static int conv_split_k(int64_t inner, int64_t co, int num_mlps, int64_t m)
+// workgroups for about four per CU, but (fp32 operands) at least 2048 samples each, so that the partial sums
+// written and summed again stay small beside the product itself.
+static int conv_split_k(int64_t inner, int64_t co, int num_mlps, int64_t m, bool bf16)
 {
     if (m < 4096) return 1;
+    if (bf16) return CONV_SPLIT_K;      // bound by its operand traffic: the more workgroups in flight the better
     const int64_t tiles = pccnn_ceil_div(inner, 64) * pccnn_ceil_div(co, 128) * num_mlps;
     int64_t split = 1024 / tiles;
     if (split > m / 2048) split = m / 2048;
@@ -1010,7 +1011,7 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
             if ((rc = launch_proj_fwd<BASIS>(g, feats, proj_ws, s, bf16)) != PCCNN_OK) return rc;
             proj = proj_ws;
         }
-        const int split = conv_split_k(inner, co, num_mlps, g.m);
+        const int split = conv_split_k(inner, co, num_mlps, g.m, bf16);
         if (bf16)
             rc = pccnn_gemm_bf16((const uint16_t *)proj, g16, d_weights, inner, co, g.m, 1, 0, (int64_t)g.c_in * g.k,
                                  c_out, co, num_mlps, inner, co, inner * co, split, splitk,

@@ -274,8 +274,7 @@ extern "C" int pccnn_gemm_f32(const float *a, const float *b, float *c, int64_t 
     hipStream_t s = (hipStream_t)stream;
     // 128-row tiles unless that leaves the chip short of workgroups (fewer than ~4 per CU): then 64-row tiles
     const int64_t wg128 = pccnn_ceil_div(cols, GT_N) * pccnn_ceil_div(rows, 128) * batch * split_k;
-    const char *force = getenv("PCCNN_GEMM_BM");
-    const int bm_tile = force ? atoi(force) : (wg128 >= 1024 ? 128 : 64);
+    const int bm_tile = wg128 >= 1024 ? 128 : 64;
     g.tiles_x = (int)pccnn_ceil_div(cols, GT_N);
     g.tiles_y = (int)pccnn_ceil_div(rows, bm_tile);
     g.total_wg = (int64_t)g.tiles_x * g.tiles_y * batch * split_k;
