@@ -302,18 +302,19 @@ __device__ __forceinline__ void basis_derivative(const ConvGeom &g, const LaneBa
 // Backward of the gather-aggregate for one sample per single-wavefront workgroup.
 //   dF[n_t][f]  += sum_k dP[s][f][k] * w[t][k]        (lane = feature f, dP row in registers)
 //   dw[t][k]     = sum_f dP[s][f][k] * F[n_t][f]      (lane = (k, group of KPAD features), dP column in registers)
-// The basis values of up to 64 pairs are evaluated once (KPAD lanes per pair) and parked in LDS, from where
-// the dF stage reads them as broadcasts; the neighbor's feature row is read coalesced from memory, used by
-// the dF stage from registers and handed to the dw stage through LDS, so that each stage runs KPAD
-// multiply-adds per pair and lane.  dw is accumulated in LDS over the feature blocks.
+// The basis values of up to 32 pairs are evaluated once (KPAD lanes per pair) and parked in LDS, from where
+// the dF stage reads them as broadcasts; the neighbor's feature row is read coalesced from memory (the rows of
+// the next four pairs travel while four are processed) and handed to the dw stage through LDS, so that each
+// stage runs KPAD multiply-adds per pair and lane.  The feature groups' partial sums of dw are added across the
+// lanes (row swaps for KPAD = 16) and accumulated in LDS over the feature blocks.
 //
 // For a basis given by the caller (EXPLICIT) dw is the result and is stored coalesced.  For the parametric
 // bases the kernel goes on while the chunk is still in LDS: KPAD lanes per pair apply the basis derivative
-// (lane = basis index k), shuffles reduce the offset / density gradients over k, and the chunk's values are
-// scattered with float atomics, sixteen pairs x (x, y, z, density) per instruction - or, when the caller has
-// the mirror index of a symmetric neighborhood, stored per pair for a gather without atomics.  The sample's own gradient
-// and the basis-parameter gradients stay in registers until the end; the latter are added to one of
-// PARAM_ROWS partial rows ([component][k], 256 floats) that the conv_param_reduce kernels sum afterwards.
+// (lane = basis index k), DPP sums over k give the pair's offset / density gradients, and the chunk's values
+// are scattered with float atomics, sixteen pairs x (x, y, z, density) per instruction - or, when the caller
+// has the mirror index of a symmetric neighborhood, stored per pair for a gather without atomics.  The sample's
+// own gradient and the basis-parameter gradients stay in registers until the end; the latter are added to one
+// of PARAM_ROWS partial rows ([component][k], 256 floats) that the conv_param_reduce kernels sum afterwards.
 #define PARAM_ROWS 256
 
 template <int BASIS, int KPAD, bool want_df, bool want_db>
