@@ -45,25 +45,41 @@ bbox_reduce_kernel(const float *__restrict__ pts, const int32_t *__restrict__ ba
     // a workgroup owns one contiguous chunk of the point list, so it rarely sees more than one cloud
     const int64_t chunk = (n + gridDim.x - 1) / gridDim.x;
     const int64_t chunk_end = ((int64_t)blockIdx.x + 1) * chunk < n ? ((int64_t)blockIdx.x + 1) * chunk : n;
-    for (int64_t i = (int64_t)blockIdx.x * chunk + threadIdx.x; i < chunk_end; i += blockDim.x) {
-        const int b = batch_ids[i];
-        if (b < 0 || b >= batch_size) continue;                       // ids outside the table are ignored
-        if (b != cur) {
-            if (cur >= 0) {
+    // four points per thread in flight: their loads do not depend on each other, the box update does
+    constexpr int UNROLL = 4;
+    for (int64_t i0 = (int64_t)blockIdx.x * chunk + threadIdx.x; i0 < chunk_end; i0 += (int64_t)UNROLL * blockDim.x) {
+        int bs[UNROLL];
+        float vs[UNROLL][D];
 #pragma unroll
-                for (int k = 0; k < D; ++k) {
-                    atomic_min_f32(&mn[cur * D + k], lo[k]);
-                    atomic_max_f32(&mx[cur * D + k], hi[k]);
-                    lo[k] = inf; hi[k] = -inf;
-                }
+        for (int u = 0; u < UNROLL; ++u) {
+            const int64_t i = i0 + (int64_t)u * blockDim.x;
+            bs[u] = -1;
+            if (i < chunk_end) {
+                bs[u] = batch_ids[i];
+#pragma unroll
+                for (int k = 0; k < D; ++k) vs[u][k] = pts[i * D + k];
             }
-            cur = b;
         }
 #pragma unroll
-        for (int k = 0; k < D; ++k) {
-            const float v = pts[i * D + k];
-            lo[k] = fminf(lo[k], v);
-            hi[k] = fmaxf(hi[k], v);
+        for (int u = 0; u < UNROLL; ++u) {
+            const int b = bs[u];
+            if (b < 0 || b >= batch_size) continue;                   // past the chunk, or an id outside the table
+            if (b != cur) {
+                if (cur >= 0) {
+#pragma unroll
+                    for (int k = 0; k < D; ++k) {
+                        atomic_min_f32(&mn[cur * D + k], lo[k]);
+                        atomic_max_f32(&mx[cur * D + k], hi[k]);
+                        lo[k] = inf; hi[k] = -inf;
+                    }
+                }
+                cur = b;
+            }
+#pragma unroll
+            for (int k = 0; k < D; ++k) {
+                lo[k] = fminf(lo[k], vs[u][k]);
+                hi[k] = fmaxf(hi[k], vs[u][k]);
+            }
         }
     }
     const int lane = pccnn_lane(), wave = threadIdx.x >> 6;
@@ -132,8 +148,10 @@ extern "C" int pccnn_bounding_box(const float *pts, const int32_t *batch_ids, in
     bbox_init_kernel<<<(unsigned)pccnn_ceil_div(count, 256), 256, 0, s>>>(aabb_min_out, aabb_max_out, count);
     PCCNN_LAUNCH_CHECK();
     if (n > 0) {
-        int64_t blocks = pccnn_ceil_div(n, 256 * 8);
-        if (blocks > 256) blocks = 256;
+        // enough workgroups to cover the load latency with a few rounds each; every workgroup ends with a handful of
+        // integer atomics per box corner
+        int64_t blocks = pccnn_ceil_div(n, 256 * 4);
+        if (blocks > 1024) blocks = 1024;
         PCCNN_DIM_DISPATCH(d, bbox_reduce_kernel, <<<(unsigned)blocks, 256, 0, s>>>(pts, batch_ids, n, batch_size,
                                                                                     aabb_min_out, aabb_max_out));
         PCCNN_LAUNCH_CHECK();

@@ -1,36 +1,100 @@
 // Poisson-disk selection over points in sorted (cell-key) order.
-// 2^D launches, one per cell-parity colour.  Cells of one colour are at least two cells apart
-// in every direction, so they never share a neighbor and can be processed concurrently; inside
-// a cell the points are visited serially in sorted order by the thread that owns the cell's
-// first point, and a point is selected iff none of its listed neighbors is selected yet.
+// 2^D launches, one per cell-parity colour.  Cells of one colour are at least two cells apart in every direction,
+// so they never share a neighbor and can be processed concurrently; inside a cell the points are taken in sorted
+// order, and a point is selected iff none of its listed neighbors is selected yet.
+//
+// One wavefront per cell, one point per lane (64 at a time).  Every lane scans its own neighbor list: a neighbor
+// outside the current 64 points is settled already (an earlier colour, an earlier round of this cell) or still
+// unselected, so its flag in memory decides; a neighbor among the current 64 with a smaller index is noted in a
+// 64-bit mask.  The serial part of the greedy rule is then a scalar loop over the candidates in order: candidate i
+// is selected iff none of its noted neighbors was selected before it.  The result is that of the one-thread-per-
+// cell walk of the reference (poisson_disk_sampling.cu:56-105), with the latency of a cell's ~10^3 dependent
+// loads paid across 64 lanes.
 #include "common.h"
+
+__global__ void __launch_bounds__(256)
+cell_flag_kernel(const int64_t *__restrict__ keys, int64_t n, int32_t *__restrict__ flags)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) flags[i] = (i == 0 || keys[i - 1] != keys[i]) ? 1 : 0;
+}
+
+// cell_first[c] = index of the first point of the c-th non-empty cell; *count = number of such cells.
+__global__ void __launch_bounds__(256)
+cell_list_kernel(const int32_t *__restrict__ flags, const int32_t *__restrict__ scan, int64_t n,
+                 int32_t *__restrict__ cell_first, int32_t *__restrict__ count)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    if (flags[i] != 0) cell_first[scan[i] - 1] = (int32_t)i;
+    if (i == n - 1) *count = scan[i];
+}
+
+#define POISSON_LOADS 4     // neighbor flags requested together by a lane
 
 template <int D>
 __global__ void __launch_bounds__(256)
 poisson_pass_kernel(const int64_t *__restrict__ keys, int64_t n, const int2 *__restrict__ neigh,
                     const int32_t *__restrict__ ends, const int32_t *__restrict__ num_cells, int colour,
-                    volatile int32_t *used)
+                    volatile int32_t *used, const int32_t *__restrict__ cell_first,
+                    const int32_t *__restrict__ cell_count)
 {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    const long long key = keys[i];
-    if (i > 0 && keys[i - 1] == key) return;          // not the first point of its cell
-    long long aux = key;
-    bool mine = true;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int64_t waves = ((int64_t)gridDim.x * blockDim.x) >> 6;
+    const int cells = *cell_count;
+    int nc[D];
 #pragma unroll
-    for (int k = D - 1; k >= 0; --k) {
-        const int nc = num_cells[k];
-        const int c = (int)(aux % nc);
-        aux /= nc;
-        mine = mine && ((c % 2) == ((colour >> k) & 1));
-    }
-    if (!mine) return;
-    for (int64_t p = i; p < n && keys[p] == key; ++p) {
-        const int lo = p > 0 ? ends[p - 1] : 0;
-        const int hi = ends[p];
-        bool free_spot = true;
-        for (int t = lo; t < hi && free_spot; ++t) free_spot = used[neigh[t].x] == 0;
-        if (free_spot) used[p] = 1;
+    for (int k = 0; k < D; ++k) nc[k] = num_cells[k];
+    for (int64_t c = wave; c < cells; c += waves) {
+        const int first = cell_first[c];
+        const int last = (c + 1 < cells) ? cell_first[c + 1] : (int)n;      // one past the cell's last point
+        long long aux = keys[first];
+        bool mine = true;
+#pragma unroll
+        for (int k = D - 1; k >= 0; --k) {
+            const int cc = (int)(aux % nc[k]);
+            aux /= nc[k];
+            mine = mine && ((cc % 2) == ((colour >> k) & 1));
+        }
+        if (!mine) continue;                                                // uniform: one key per wavefront
+        for (int base = first; base < last; base += 64) {
+            const int p = base + lane;
+            const bool valid = p < last;
+            bool cand = valid;
+            unsigned long long earlier = 0ull;      // neighbors among the current 64 points that come before p
+            if (valid) {
+                const int lo = p > 0 ? ends[p - 1] : 0;
+                const int hi = ends[p];
+                for (int t = lo; t < hi && cand; t += POISSON_LOADS) {
+                    int q[POISSON_LOADS], u[POISSON_LOADS];
+#pragma unroll
+                    for (int v = 0; v < POISSON_LOADS; ++v) q[v] = (t + v < hi) ? neigh[t + v].x : p;
+#pragma unroll
+                    for (int v = 0; v < POISSON_LOADS; ++v) {
+                        const bool in_round = q[v] >= base && q[v] < p;
+                        u[v] = (in_round || q[v] == p) ? 0 : used[q[v]];
+                        if (in_round) earlier |= 1ull << (q[v] - base);
+                    }
+#pragma unroll
+                    for (int v = 0; v < POISSON_LOADS; ++v) cand = cand && (u[v] == 0);
+                }
+            }
+            // the greedy rule among the current points, in order
+            unsigned long long todo = __ballot(cand);
+            unsigned long long selected = 0ull;
+            while (todo != 0ull) {
+                const int i = __ffsll((long long)todo) - 1;
+                todo &= todo - 1ull;
+                const unsigned lo32 = (unsigned)__builtin_amdgcn_readlane((int)(earlier & 0xffffffffull), i);
+                const unsigned hi32 = (unsigned)__builtin_amdgcn_readlane((int)(earlier >> 32), i);
+                const unsigned long long before = ((unsigned long long)hi32 << 32) | lo32;
+                if ((before & selected) == 0ull) selected |= 1ull << i;
+            }
+            if (valid && ((selected >> lane) & 1ull)) used[p] = 1;
+            // a later round of this cell reads these flags back
+            if (base + 64 < last) __threadfence();
+        }
     }
 }
 
@@ -44,7 +108,9 @@ compact_kernel(const int32_t *__restrict__ flags, const int32_t *__restrict__ sc
 
 extern "C" size_t pccnn_poisson_disk_workspace_bytes(int64_t n)
 {
-    return pccnn_align(pccnn_scan_tmp_elems(n) * sizeof(int32_t)) + 256;
+    if (n < 1) n = 1;
+    // scan scratch | cell flags | first point of every cell | cell count
+    return pccnn_align(pccnn_scan_tmp_elems(n) * sizeof(int32_t)) + 2 * pccnn_align((size_t)n * sizeof(int32_t)) + 512;
 }
 
 extern "C" int pccnn_poisson_disk_select(const int64_t *sorted_keys, int64_t n, const int32_t *neigh, int64_t t,
@@ -63,14 +129,31 @@ extern "C" int pccnn_poisson_disk_select(const int64_t *sorted_keys, int64_t n, 
                   "pccnn_poisson_disk_select: workspace of %zu bytes, need %zu", workspace_bytes,
                   pccnn_poisson_disk_workspace_bytes(n));
     hipStream_t s = (hipStream_t)stream;
-    int rc = pccnn_fill_i32(selected_out, 0, n, s);
+    PccnnArena arena(workspace, workspace_bytes);
+    int32_t *scan_tmp = arena.take<int32_t>(pccnn_scan_tmp_elems(n));
+    int32_t *flags = arena.take<int32_t>((size_t)n);
+    int32_t *cell_first = arena.take<int32_t>((size_t)n);
+    int32_t *cell_count = arena.take<int32_t>(1);
+    PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "pccnn_poisson_disk_select: workspace of %zu bytes, need %zu",
+                  workspace_bytes, pccnn_poisson_disk_workspace_bytes(n));
+    // the list of non-empty cells (selected_scan_out is free until the end and holds the scan of the flags)
+    const unsigned blocks = (unsigned)pccnn_ceil_div(n, 256);
+    cell_flag_kernel<<<blocks, 256, 0, s>>>(sorted_keys, n, flags);
+    PCCNN_LAUNCH_CHECK();
+    int rc = pccnn_scan_inclusive_i32(flags, selected_scan_out, n, 0, scan_tmp, s);
     if (rc != PCCNN_OK) return rc;
+    cell_list_kernel<<<blocks, 256, 0, s>>>(flags, selected_scan_out, n, cell_first, cell_count);
+    PCCNN_LAUNCH_CHECK();
+    if ((rc = pccnn_fill_i32(selected_out, 0, n, s)) != PCCNN_OK) return rc;
+    // a fixed number of wavefronts takes the cells in turn: the cell count stays on the device
+    int64_t pass_blocks = pccnn_ceil_div(n, 64);
+    if (pass_blocks > 2048) pass_blocks = 2048;
     for (int colour = 0; colour < (1 << d); ++colour) {
-        PCCNN_DIM_DISPATCH(d, poisson_pass_kernel, <<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(
-            sorted_keys, n, (const int2 *)neigh, ends, num_cells, colour, selected_out));
+        PCCNN_DIM_DISPATCH(d, poisson_pass_kernel, <<<(unsigned)pass_blocks, 256, 0, s>>>(
+            sorted_keys, n, (const int2 *)neigh, ends, num_cells, colour, selected_out, cell_first, cell_count));
         PCCNN_LAUNCH_CHECK();
     }
-    return pccnn_scan_inclusive_i32(selected_out, selected_scan_out, n, 0, (int32_t *)workspace, s);
+    return pccnn_scan_inclusive_i32(selected_out, selected_scan_out, n, 0, scan_tmp, s);
 }
 
 extern "C" int pccnn_compact_selected(const int32_t *selected, const int32_t *selected_scan, int64_t n,
