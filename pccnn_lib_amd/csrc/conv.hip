@@ -250,6 +250,114 @@ conv_proj_fwd_kernel(ConvGeom g, const float *__restrict__ feats, void *__restri
     }
 }
 
+// Forward projection for at most 32 input features.  With lane = feature, most of a wavefront would idle; here
+// G = 64 / FPAD pairs are processed side by side, lane = (pair slot, feature): every lane keeps K partial sums for
+// its feature over the pairs that fall into its slot, and the slots are added at the end (DPP rotations and row
+// swaps).  Basis values and pair records go through LDS as in the wide kernel.
+template <int BASIS, int KPAD, int FPAD, bool BF16>
+__global__ void __launch_bounds__(64)
+conv_proj_fwd_narrow_kernel(ConvGeom g, const float *__restrict__ feats, void *__restrict__ proj_out)
+{
+    constexpr int PARTS = 64 / KPAD;
+    constexpr int G = 64 / FPAD;                        // pairs per step
+    constexpr int STEPS = 4;                            // steps whose feature loads are in flight together
+    __shared__ __attribute__((aligned(16))) float w_lds[64][KPAD];
+    __shared__ float4 geo_lds[64];                      // (offset, density) of the chunk's pairs
+    __shared__ int nidx_lds[64];                        // and their points
+    const int lane = threadIdx.x;
+    const int64_t s = blockIdx.x;
+    const int f = lane % FPAD, slot = lane / FPAD;
+    const bool fvalid = f < g.c_in;
+    const int k = lane % KPAD, part = lane / KPAD;
+    const int lo = s > 0 ? g.ends[s - 1] : 0;
+    const int hi = g.ends[s];
+    constexpr bool GEOM = BASIS != BASIS_EXPLICIT;
+    float sx = 0.f, sy = 0.f, sz = 0.f, ir0 = 1.f, ir1 = 1.f, ir2 = 1.f;
+    if (GEOM) {
+        sx = g.samples[s * 3 + 0]; sy = g.samples[s * 3 + 1]; sz = g.samples[s * 3 + 2];
+        ir0 = 1.0f / g.radii[0]; ir1 = 1.0f / g.radii[1]; ir2 = 1.0f / g.radii[2];
+    }
+    LaneBasis<BASIS> lb;
+    lb.load(g, k);
+    float acc[KPAD];
+#pragma unroll
+    for (int q = 0; q < KPAD; ++q) acc[q] = 0.0f;
+
+    for (int cb = lo; cb < hi; cb += 64) {
+        const int cnt = (hi - cb) < 64 ? (hi - cb) : 64;
+        int nidx = 0;
+        float dx = 0.f, dy = 0.f, dz = 0.f, pd = 1.0f;
+        if (lane < cnt) {
+            nidx = g.neigh[cb + lane].x;
+            if (GEOM) {
+                dx = (g.pts[(int64_t)nidx * 3 + 0] - sx) * ir0;
+                dy = (g.pts[(int64_t)nidx * 3 + 1] - sy) * ir1;
+                dz = (g.pts[(int64_t)nidx * 3 + 2] - sz) * ir2;
+            }
+            if (BasisTraits<BASIS>::uses_pdf) pd = g.pdf[nidx];
+        }
+        nidx_lds[lane] = nidx;
+        if (GEOM) geo_lds[lane] = make_float4(dx, dy, dz, pd);
+        __syncthreads();
+        for (int p = 0; p * PARTS < cnt; ++p) {
+            const int j = p * PARTS + part;             // < 64: PARTS divides 64 and p * PARTS < cnt <= 64
+            float4 ge = make_float4(0.f, 0.f, 0.f, 1.f);
+            if (GEOM) ge = geo_lds[j];
+            const float w = (j < cnt) ? pair_basis<BASIS>(g, lb, (int64_t)cb + j, ge.x, ge.y, ge.z, ge.w) : 0.0f;
+            w_lds[j][k] = w;
+        }
+        __syncthreads();
+        for (int j0 = 0; j0 < cnt; j0 += G * STEPS) {
+            float row[STEPS];
+#pragma unroll
+            for (int u = 0; u < STEPS; ++u) {
+                const int j = j0 + u * G + slot;        // < 64 whenever it is below cnt
+                row[u] = (fvalid && j < cnt) ? feats[(int64_t)nidx_lds[j & 63] * g.c_in + f] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < STEPS; ++u) {
+                const int j = j0 + u * G + slot;
+                if (j < cnt) {
+#pragma unroll
+                    for (int q = 0; q < KPAD; q += 4) {
+                        const float4 wv = *(const float4 *)&w_lds[j][q];
+                        acc[q] += row[u] * wv.x;
+                        acc[q + 1] += row[u] * wv.y;
+                        acc[q + 2] += row[u] * wv.z;
+                        acc[q + 3] += row[u] * wv.w;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    // the slots' partial sums, then the tile [features][k] through LDS so that the stores are contiguous runs
+#pragma unroll
+    for (int q = 0; q < KPAD; ++q) acc[q] = pccnn_strided_sum<FPAD>(acc[q]);
+    float *tile = &w_lds[0][0];
+    if (slot == 0) {
+#pragma unroll
+        for (int q = 0; q < KPAD; q += 4)
+            *(float4 *)&tile[f * KPAD + q] = make_float4(acc[q], acc[q + 1], acc[q + 2], acc[q + 3]);
+    }
+    __syncthreads();
+    const int nf = g.c_in;
+    const int64_t dst_at = (int64_t)s * g.c_in * g.k;
+    if (BF16) {
+        uint16_t *dst = (uint16_t *)proj_out + dst_at;
+        for (int idx = lane; idx < nf * g.k; idx += 64) {
+            const int ff = idx / g.k, q = idx - ff * g.k;
+            dst[idx] = pccnn_bf16_bits(tile[ff * KPAD + q]);
+        }
+    } else {
+        float *dst = (float *)proj_out + dst_at;
+        for (int idx = lane; idx < nf * g.k; idx += 64) {
+            const int ff = idx / g.k, q = idx - ff * g.k;
+            dst[idx] = tile[ff * KPAD + q];
+        }
+    }
+}
+
 // Derivative of one basis value w.r.t. the pair's normalised offset, the neighbor's density and the basis
 // parameters of this lane's k.  gk = upstream gradient of the basis value; (gx, gy, gz, gpdf) receive the
 // offset / density gradients, (p0..p3) accumulate the parameter gradients.
@@ -557,6 +665,185 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
     }
 }
 
+// Backward projection for at most 32 input features (arguments and results as conv_proj_bwd_kernel).  Two lane
+// layouts, each using the whole wavefront: for dF, lane = (pair slot, feature f) with the f-th row of the sample's
+// gradient tile in registers, 64 / FPAD pairs per step; for dw, lane = (pair slot, basis index k) with column k of
+// the tile in registers and the pairs' feature rows in LDS, 64 / KPAD pairs per step - the sum over the features
+// runs inside the lane, so nothing is added across lanes.
+template <int BASIS, int KPAD, int FPAD, bool want_df, bool want_db>
+__global__ void __launch_bounds__(64)
+conv_proj_bwd_narrow_kernel(ConvGeom g, const float *__restrict__ feats, const float *__restrict__ proj_grads,
+                            float *__restrict__ feat_grads, float *__restrict__ basis_grads,
+                            float *__restrict__ d_pts, float *__restrict__ d_samples, float *__restrict__ d_pdf,
+                            float *__restrict__ param_partials, float *__restrict__ pair_grads)
+{
+    constexpr bool FUSED = want_db && BasisTraits<BASIS>::differentiable;   // basis derivative applied here
+    constexpr int CH = 32;                                          // pairs staged in LDS at a time
+    constexpr int PARTS = 64 / KPAD;                                // pairs per step of the dw / derivative stages
+    constexpr int GF = 64 / FPAD;                                   // pairs per step of the dF stage
+    constexpr bool GEOM = BASIS != BASIS_EXPLICIT;
+    __shared__ __attribute__((aligned(16))) float g_lds[FUSED ? CH : 1][4];
+    __shared__ float4 geo_lds[CH];                                  // (offset, density) of the chunk's pairs
+    __shared__ int nidx_lds[CH];                                    // and their points
+    __shared__ __attribute__((aligned(16))) float w_lds[CH][KPAD];
+    __shared__ __attribute__((aligned(16))) float db_lds[want_db ? CH : 1][KPAD];
+    __shared__ __attribute__((aligned(16))) float row_lds[want_db ? CH : 1][FPAD];
+    const int lane = threadIdx.x;
+    const int64_t s = blockIdx.x;
+    const int k = lane % KPAD, part = lane / KPAD;
+    const int f = lane % FPAD, slot = lane / FPAD;
+    const bool fvalid = f < g.c_in;
+    const int lo = s > 0 ? g.ends[s - 1] : 0;
+    const int hi = g.ends[s];
+    float sx = 0.f, sy = 0.f, sz = 0.f, ir0 = 1.f, ir1 = 1.f, ir2 = 1.f;
+    if (GEOM) {
+        sx = g.samples[s * 3 + 0]; sy = g.samples[s * 3 + 1]; sz = g.samples[s * 3 + 2];
+        ir0 = 1.0f / g.radii[0]; ir1 = 1.0f / g.radii[1]; ir2 = 1.0f / g.radii[2];
+    }
+    LaneBasis<BASIS> lb;
+    lb.load(g, k);
+    float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;       // parameter gradients of this lane's k (FUSED)
+    float sg = 0.f;                                     // component (lane & 3) of the sample's gradient, unsigned
+    // the sample's gradient tile: row f (dF stage) and column k (dw stage)
+    float gp[KPAD], gt[FPAD];
+#pragma unroll
+    for (int q = 0; q < KPAD; ++q) gp[q] = 0.0f;
+#pragma unroll
+    for (int q = 0; q < FPAD; ++q) gt[q] = 0.0f;
+    if (hi > lo) {
+        const float *tile = proj_grads + (int64_t)s * g.c_in * g.k;
+        if (want_df && fvalid) {
+#pragma unroll
+            for (int q = 0; q < KPAD; ++q)
+                if (q < g.k) gp[q] = tile[f * g.k + q];
+        }
+        if (want_db && k < g.k) {
+#pragma unroll
+            for (int q = 0; q < FPAD; ++q)
+                if (q < g.c_in) gt[q] = tile[q * g.k + k];
+        }
+    }
+
+    for (int cb = lo; cb < hi; cb += CH) {
+        const int cnt = (hi - cb) < CH ? (hi - cb) : CH;
+        int nidx = 0;
+        float dx = 0.f, dy = 0.f, dz = 0.f, pd = 1.0f;
+        if (lane < cnt) {
+            nidx = g.neigh[cb + lane].x;
+            if (GEOM) {
+                dx = (g.pts[(int64_t)nidx * 3 + 0] - sx) * ir0;
+                dy = (g.pts[(int64_t)nidx * 3 + 1] - sy) * ir1;
+                dz = (g.pts[(int64_t)nidx * 3 + 2] - sz) * ir2;
+            }
+            if (BasisTraits<BASIS>::uses_pdf) pd = g.pdf[nidx];
+        }
+        if (lane < CH) {
+            if (GEOM) geo_lds[lane] = make_float4(dx, dy, dz, pd);
+            nidx_lds[lane] = nidx;
+        }
+        __syncthreads();
+        if (want_db) {
+            // the pairs' feature rows, GF pairs per load instruction (zeros past the last feature)
+            for (int j0 = 0; j0 < cnt; j0 += GF) {
+                const int j = j0 + slot;
+                if (j < cnt) row_lds[j][f] = fvalid ? feats[(int64_t)nidx_lds[j] * g.c_in + f] : 0.0f;
+            }
+        }
+        // basis values of the chunk: pass p evaluates pairs p*PARTS .. p*PARTS + PARTS - 1
+        for (int p = 0; p * PARTS < cnt; ++p) {
+            const int j = p * PARTS + part;             // < CH: PARTS divides CH and p * PARTS < cnt <= CH
+            float4 ge = make_float4(0.f, 0.f, 0.f, 1.f);
+            if (GEOM) ge = geo_lds[j];
+            const float w = (j < cnt) ? pair_basis<BASIS>(g, lb, (int64_t)cb + j, ge.x, ge.y, ge.z, ge.w) : 0.0f;
+            w_lds[j][k] = w;
+        }
+        __syncthreads();
+        if (want_df) {
+            for (int j0 = 0; j0 < cnt; j0 += GF) {
+                const int j = j0 + slot;
+                if (j < cnt && fvalid) {
+                    float gf = 0.0f;
+#pragma unroll
+                    for (int q = 0; q < KPAD; q += 4) {
+                        const float4 wv = *(const float4 *)&w_lds[j][q];
+                        gf += gp[q] * wv.x + gp[q + 1] * wv.y + gp[q + 2] * wv.z + gp[q + 3] * wv.w;
+                    }
+                    unsafeAtomicAdd(&feat_grads[(int64_t)nidx_lds[j] * g.c_in + f], gf);
+                }
+            }
+        }
+        if (want_db) {
+            for (int j0 = 0; j0 < cnt; j0 += PARTS) {
+                const int j = j0 + part;
+                if (j < cnt) {
+                    float acc = 0.0f;
+#pragma unroll
+                    for (int q = 0; q < FPAD; q += 4) {
+                        const float4 rv = *(const float4 *)&row_lds[j][q];
+                        acc += gt[q] * rv.x + gt[q + 1] * rv.y + gt[q + 2] * rv.z + gt[q + 3] * rv.w;
+                    }
+                    db_lds[j][k] = acc;
+                }
+            }
+        }
+        __syncthreads();
+        if (FUSED) {
+            for (int p = 0; p * PARTS < cnt; ++p) {
+                const int j = p * PARTS + part;
+                const float4 ge = geo_lds[j];
+                float gx = 0.f, gy = 0.f, gz = 0.f, gpdf = 0.f;
+                if (j < cnt && lb.active)
+                    basis_derivative<BASIS>(g, lb, ge.x, ge.y, ge.z, ge.w, db_lds[j][k], gx, gy, gz, gpdf, p0, p1, p2, p3);
+                // summed over the basis index: the KPAD lanes of this pair
+                gx = pccnn_group_sum<KPAD>(gx);
+                gy = pccnn_group_sum<KPAD>(gy);
+                gz = pccnn_group_sum<KPAD>(gz);
+                if (BasisTraits<BASIS>::pdf_grad) gpdf = pccnn_group_sum<KPAD>(gpdf);
+                if (k < 4) g_lds[j][k] = (k == 0) ? gx * ir0 : (k == 1) ? gy * ir1 : (k == 2) ? gz * ir2 : gpdf;
+            }
+            __syncthreads();
+            for (int i = 0; i * 16 < cnt; ++i) {
+                const int j = i * 16 + (lane >> 2), comp = lane & 3;
+                if (j < cnt) {
+                    const int jn = nidx_lds[j];
+                    const float v = g_lds[j][comp];
+                    if (comp < 3) sg += v;
+                    if (pair_grads) {
+                        // per-pair values, summed per point afterwards by conv_point_gather_kernel
+                        pair_grads[(int64_t)(cb + j) * 4 + comp] = v;
+                    } else if (comp < 3) {
+                        if (d_pts) unsafeAtomicAdd(&d_pts[(int64_t)jn * 3 + comp], v);
+                    } else if (BasisTraits<BASIS>::pdf_grad && d_pdf) {
+                        unsafeAtomicAdd(&d_pdf[jn], v);
+                    }
+                }
+            }
+        } else if (want_db) {
+            for (int idx = lane; idx < cnt * KPAD; idx += 64) {
+                const int j = idx / KPAD, kk = idx % KPAD;
+                if (kk < g.k) basis_grads[(int64_t)(cb + j) * g.k + kk] = db_lds[j][kk];
+            }
+        }
+        __syncthreads();
+    }
+    if (FUSED) {
+        sg = pccnn_strided_sum<4>(sg);
+        if (lane < 3 && d_samples) d_samples[s * 3 + lane] = -sg;
+        if (param_partials) {
+            p0 = pccnn_strided_sum<KPAD>(p0);
+            p1 = pccnn_strided_sum<KPAD>(p1);
+            p2 = pccnn_strided_sum<KPAD>(p2);
+            if (BasisTraits<BASIS>::axis) p3 = pccnn_strided_sum<KPAD>(p3);
+            float *prow = param_partials + (int64_t)(blockIdx.x % PARAM_ROWS) * 256;
+            constexpr int COMPS = BasisTraits<BASIS>::axis ? 4 : 3;
+            for (int c = part; c < COMPS; c += PARTS) {
+                const float v = (c == 0) ? p0 : (c == 1) ? p1 : (c == 2) ? p2 : p3;
+                unsafeAtomicAdd(&prow[c * 64 + k], v);
+            }
+        }
+    }
+}
+
 // Symmetric neighborhoods (samples are the points, uncapped search): pair (a, b) exists iff (b, a) does.
 // mirror[t] of pair t = (point a, sample b) is the index of pair (point b, sample a), found by scanning
 // sample a's segment; -1 and a count in *missing when there is none (the neighborhood is not symmetric).
@@ -789,11 +1076,37 @@ linear_basis_bwd_kernel(ConvGeom g, const float *__restrict__ basis_grads, float
 static int kpad_of(int k) { return k <= 8 ? 8 : (k <= 16 ? 16 : (k <= 32 ? 32 : 64)); }
 
 // `bf16`: proj is uint16_t[m, c_in * k] of bf16 bit patterns instead of float[m, c_in * k].
+template <int BASIS, int KPAD>
+static void launch_proj_fwd_narrow(const ConvGeom &g, const float *feats, void *proj, hipStream_t s, bool bf16)
+{
+    dim3 grid((unsigned)g.m);
+#define NARROW_GO(FP)                                                                                   \
+    do {                                                                                                \
+        if (bf16) conv_proj_fwd_narrow_kernel<BASIS, KPAD, FP, true><<<grid, 64, 0, s>>>(g, feats, proj);  \
+        else conv_proj_fwd_narrow_kernel<BASIS, KPAD, FP, false><<<grid, 64, 0, s>>>(g, feats, proj);      \
+    } while (0)
+    if (g.c_in <= 8) NARROW_GO(8);
+    else if (g.c_in <= 16) NARROW_GO(16);
+    else NARROW_GO(32);
+#undef NARROW_GO
+}
+
 template <int BASIS>
 static int launch_proj_fwd(const ConvGeom &g, const float *feats, void *proj, hipStream_t s, bool bf16 = false)
 {
     dim3 grid((unsigned)g.m, (unsigned)((g.c_in + 63) / 64));
     PccnnTimed timed(PCCNN_T_PROJ_FWD, s);
+    if (g.c_in <= 32) {
+        // few input features: several pairs side by side instead of idle lanes
+        switch (kpad_of(g.k)) {
+        case 8: launch_proj_fwd_narrow<BASIS, 8>(g, feats, proj, s, bf16); break;
+        case 16: launch_proj_fwd_narrow<BASIS, 16>(g, feats, proj, s, bf16); break;
+        case 32: launch_proj_fwd_narrow<BASIS, 32>(g, feats, proj, s, bf16); break;
+        default: launch_proj_fwd_narrow<BASIS, 64>(g, feats, proj, s, bf16); break;
+        }
+        PCCNN_LAUNCH_CHECK();
+        return PCCNN_OK;
+    }
 #define PROJ_GO(KP)                                                                         \
     do {                                                                                    \
         if (bf16) conv_proj_fwd_kernel<BASIS, KP, true><<<grid, 64, 0, s>>>(g, feats, proj);  \
@@ -823,6 +1136,26 @@ static void launch_proj_bwd_k(const ConvGeom &g, const float *feats, const float
                               bool want_basis, const BasisGradOut &o, hipStream_t s)
 {
     dim3 grid((unsigned)g.m);
+    if (g.c_in <= 32) {
+        // few input features: several pairs side by side instead of idle lanes
+#define NARROW_GO(FP)                                                                                                  \
+    do {                                                                                                               \
+        if (feat_grads && want_basis)                                                                                  \
+            conv_proj_bwd_narrow_kernel<BASIS, KPAD, FP, true, true><<<grid, 64, 0, s>>>(                              \
+                g, feats, proj_grads, feat_grads, o.basis_grads, o.d_pts, o.d_samples, o.d_pdf, o.partials, o.pair_grads); \
+        else if (feat_grads)                                                                                           \
+            conv_proj_bwd_narrow_kernel<BASIS, KPAD, FP, true, false><<<grid, 64, 0, s>>>(                             \
+                g, feats, proj_grads, feat_grads, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr);               \
+        else                                                                                                           \
+            conv_proj_bwd_narrow_kernel<BASIS, KPAD, FP, false, true><<<grid, 64, 0, s>>>(                             \
+                g, feats, proj_grads, nullptr, o.basis_grads, o.d_pts, o.d_samples, o.d_pdf, o.partials, o.pair_grads); \
+    } while (0)
+        if (g.c_in <= 8) NARROW_GO(8);
+        else if (g.c_in <= 16) NARROW_GO(16);
+        else NARROW_GO(32);
+#undef NARROW_GO
+        return;
+    }
     if (feat_grads && want_basis)
         conv_proj_bwd_kernel<BASIS, KPAD, true, true><<<grid, 64, 0, s>>>(g, feats, proj_grads, feat_grads, o.basis_grads,
                                                                           o.d_pts, o.d_samples, o.d_pdf, o.partials,
