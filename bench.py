@@ -39,7 +39,7 @@ HBM_PEAK_GBPS = 8000.0            # MI355X HBM3E peak
 # Bytes per launch that the dominant kernels move past the L2, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # of this command scaled by a copy kernel of known size (profiles/bench_mcconv_16x4096_hbm_traffic.md).  They
 # hold for the default workloads only (config 2; the scene leg at 1 000 000 points) and are reported as null otherwise.
-TRAFFIC_GEMM_BYTES = 312.8e6            # mean of the three contraction launches of a step (algorithmic: 313.5e6)
+TRAFFIC_GEMM_BYTES = 312.7e6            # mean of the three contraction launches of a step (algorithmic: 313.5e6)
 TRAFFIC_NB_FILL_BYTES_CONFIG2 = 17.1e6  # launches of 65 536 samples (algorithmic: 10.3e6)
 TRAFFIC_NB_FILL_BYTES_SCENE = 610.2e6   # launches of 1 000 000 samples (algorithmic: 194.6e6)
 

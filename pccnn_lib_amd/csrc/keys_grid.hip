@@ -148,10 +148,10 @@ extern "C" int pccnn_bounding_box(const float *pts, const int32_t *batch_ids, in
     bbox_init_kernel<<<(unsigned)pccnn_ceil_div(count, 256), 256, 0, s>>>(aabb_min_out, aabb_max_out, count);
     PCCNN_LAUNCH_CHECK();
     if (n > 0) {
-        // enough workgroups to cover the load latency with a few rounds each; every workgroup ends with a handful of
-        // integer atomics per box corner
+        // every workgroup ends with a handful of integer atomics per box corner, and with one cloud they all meet on
+        // the same six addresses: few workgroups, each with four points per thread in flight
         int64_t blocks = pccnn_ceil_div(n, 256 * 4);
-        if (blocks > 1024) blocks = 1024;
+        if (blocks > 256) blocks = 256;
         PCCNN_DIM_DISPATCH(d, bbox_reduce_kernel, <<<(unsigned)blocks, 256, 0, s>>>(pts, batch_ids, n, batch_size,
                                                                                     aabb_min_out, aabb_max_out));
         PCCNN_LAUNCH_CHECK();
