@@ -30,7 +30,7 @@ cell_list_kernel(const int32_t *__restrict__ flags, const int32_t *__restrict__ 
     if (i == n - 1) *count = scan[i];
 }
 
-#define POISSON_LOADS 4     // neighbor flags requested together by a lane
+#define POISSON_LOADS 8     // neighbor flags requested together by a lane
 
 template <int D>
 __global__ void __launch_bounds__(256)
@@ -43,6 +43,7 @@ poisson_pass_kernel(const int64_t *__restrict__ keys, int64_t n, const int2 *__r
     const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     const int64_t waves = ((int64_t)gridDim.x * blockDim.x) >> 6;
     const int cells = *cell_count;
+    const int32_t *settled = (const int32_t *)used;
     int nc[D];
 #pragma unroll
     for (int k = 0; k < D; ++k) nc[k] = num_cells[k];
@@ -73,7 +74,12 @@ poisson_pass_kernel(const int64_t *__restrict__ keys, int64_t n, const int2 *__r
 #pragma unroll
                     for (int v = 0; v < POISSON_LOADS; ++v) {
                         const bool in_round = q[v] >= base && q[v] < p;
-                        u[v] = (in_round || q[v] == p) ? 0 : used[q[v]];
+                        // Flags of other cells were written by earlier launches (cells of one colour are never
+                        // neighbors), so an ordinary cached load sees them; only an earlier round of this very
+                        // cell, written by this wavefront a moment ago, has to be read past the caches.
+                        if (in_round || q[v] == p) u[v] = 0;
+                        else if (q[v] >= first && q[v] < base) u[v] = used[q[v]];
+                        else u[v] = settled[q[v]];
                         if (in_round) earlier |= 1ull << (q[v] - base);
                     }
 #pragma unroll
