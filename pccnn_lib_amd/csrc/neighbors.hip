@@ -272,6 +272,137 @@ neighbors_kernel(NbArgs a)
     }
 }
 
+// Few samples against many points (every pooling level of a hierarchy): with one sample per lane the launch has
+// too few wavefronts and every lane a long walk.  Here G lanes share a sample: lane 0..8 of the group look up the
+// nine pillar ranges, then the group strides over every range together, one candidate per lane and step; a ballot
+// over the group's lanes counts the hits of the step and ranks them, so the pairs of a sample still come out in
+// ascending sorted-point order, without atomics.  The capped subset is the same as in the one-lane walk: hit
+// number r is kept iff floor((r + 1) cap / raw) > floor(r cap / raw), at slot floor(r cap / raw).
+template <bool FILL, bool CAPPED, int G>
+__global__ void __launch_bounds__(NB_THREADS)
+neighbors_group_kernel(NbArgs a)
+{
+    constexpr int GROUPS = 64 / G;                              // samples per wavefront
+    __shared__ int2 ranges[NB_WAVES][GROUPS][9];
+    const int lane = pccnn_lane();
+    const int wib = threadIdx.x >> 6;
+    const int grp = lane / G, sub = lane % G;
+    const int64_t wave = ((int64_t)blockIdx.x * NB_THREADS + threadIdx.x) >> 6;
+    const int64_t at0 = wave * GROUPS + grp;                    // place of the group's sample in the walk order
+    if (wave * GROUPS >= a.m) return;                           // wave-uniform
+    const bool valid = at0 < a.m;
+
+    int s = 0;
+    long long key = -1;
+    float sx = 0.f, sy = 0.f, sz = 0.f;
+    if (valid) {
+        s = a.order ? a.order[at0] : (int)at0;
+        const int64_t at = a.presorted ? at0 : (int64_t)s;
+        key = a.sample_keys[at];
+        sx = a.samples[at * 3 + 0];
+        sy = a.samples[at * 3 + 1];
+        sz = a.samples[at * 3 + 2];
+    }
+    const int nc0 = a.num_cells[0], nc1 = a.num_cells[1], nc2 = a.num_cells[2];
+    const float ir0 = __fdiv_rn(1.0f, a.radii[0]);
+    const float ir1 = __fdiv_rn(1.0f, a.radii[1]);
+    const float ir2 = __fdiv_rn(1.0f, a.radii[2]);
+    const bool usable = valid && key >= 0;
+    long long k = usable ? key : 0;
+    const int c2 = (int)(k % nc2); k /= nc2;
+    const int c1 = (int)(k % nc1);
+    const long long pil = k; k /= nc1;
+    const int c0 = (int)(k % nc0);
+    // the nine ranges, in pillar order (ascending sorted index); lane o of the group looks up range o
+    for (int o = sub; o < 9; o += G) {
+        int first = 0, len = 0;
+        if (usable) {
+            const int cmin = c2 > 0 ? c2 - 1 : 0, cmax = c2 + 1 < nc2 ? c2 + 1 : nc2 - 1;
+            const int dx = o / 3 - 1, dy = o % 3 - 1;
+            const int x = c0 + dx, y = c1 + dy;
+            if (x >= 0 && x < nc0 && y >= 0 && y < nc1)
+                nb_pillar_range(a, pil + (long long)dx * nc1 + dy, nc2, cmin, cmax, first, len);
+        }
+        ranges[wib][grp][o] = make_int2(first, len);
+    }
+    // (a wavefront's own LDS writes are in order with its reads: no barrier between the lanes of a group)
+
+    unsigned int seg = 0;                                       // FILL: first output slot of the sample
+    long long raw = 0, cap = 0;
+    if (FILL && valid) {
+        seg = s > 0 ? (unsigned int)a.ends[s - 1] : 0u;
+        if (CAPPED) {
+            raw = a.counts[s];
+            cap = raw < a.max_neighbors ? raw : a.max_neighbors;
+        }
+    }
+    const unsigned int out_limit = FILL ? (unsigned int)a.t : 0u;
+    const unsigned long long group_bits = (G == 64) ? ~0ull : (((1ull << (G & 63)) - 1ull) << (grp * G));
+    const unsigned long long below = group_bits & pccnn_lanemask_lt();
+
+    int cnt = 0;                                                // hits of the sample so far (same in all its lanes)
+    int r = 0, j0 = 0;
+    int2 cur = ranges[wib][grp][0];
+    bool active = usable;
+    while (__any(active)) {
+        bool hit = false;
+        int id = 0;
+        if (active) {
+            const int j = j0 + sub;
+            if (j < cur.y) {
+                const int idx = cur.x + j;
+                float px, py, pz;
+                if (FILL) {
+                    const float4 v = a.rec[idx];
+                    px = v.x; py = v.y; pz = v.z;
+                    id = __float_as_int(v.w);
+                } else {
+                    px = a.pts[(int64_t)idx * 3 + 0];
+                    py = a.pts[(int64_t)idx * 3 + 1];
+                    pz = a.pts[(int64_t)idx * 3 + 2];
+                }
+                // fp32, no contraction: the predicate of the one-lane walk
+                const float vx = (sx - px) * ir0;
+                const float vy = (sy - py) * ir1;
+                const float vz = (sz - pz) * ir2;
+                const float acc = ((0.0f + vx * vx) + vy * vy) + vz * vz;
+                hit = acc < 1.0f;
+            }
+        }
+        const unsigned long long hits = __ballot(hit);
+        if (active) {
+            if (FILL && hit) {
+                const long long rank = cnt + __popcll(hits & below);        // number of this hit in walk order
+                bool take = true;
+                long long slot = rank;
+                if (CAPPED) {
+                    slot = rank * cap / raw;
+                    take = (rank + 1) * cap / raw > slot;
+                }
+                const unsigned long long at = (unsigned long long)seg + (unsigned long long)slot;
+                if (take && at < out_limit) ((int2 *)a.neigh)[at] = make_int2(id, s);
+            }
+            cnt += __popcll(hits & group_bits);
+            j0 += G;
+            if (j0 >= cur.y) {
+                j0 = 0;
+                if (++r < 9) cur = ranges[wib][grp][r];
+                else active = false;
+            }
+        }
+    }
+    if (!FILL && valid && sub == 0) a.counts[s] = cnt;
+}
+
+// Lanes per sample: one when there are about as many samples as points, more when the samples are few.
+static int nb_group_size(int64_t n, int64_t m, int d)
+{
+    if (d != 3 || m <= 0) return 1;
+    if (n >= 16 * m) return 64;
+    if (n >= 4 * m) return 16;
+    return 1;
+}
+
 // Any other dimension (2, 4, 5, 6): the walk of the reference, restated per lane without the shortcuts that
 // three dimensions allow.  Offsets run over {-1, 0, 1} in every dimension but the last (in both when D == 2), in
 // the reference's order (find_ranges_grid_ds.cu:306-338); an offset cell selects its pillar (batch, c0, c1) in the
@@ -494,11 +625,14 @@ extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t
     a.cell_table = cell_table; a.total_cells = total_cells;
     a.num_cells = num_cells; a.radii = radii; a.max_neighbors = max_neighbors;
     a.counts = counts; a.ends = nullptr; a.remap = nullptr; a.t = 0; a.neigh = nullptr; a.rec = nullptr;
-    int64_t waves = pccnn_ceil_div(m, 64);
+    const int group = nb_group_size(n, m, d);
+    int64_t waves = pccnn_ceil_div(m * group, 64);
     {
         PccnnTimed timed(PCCNN_T_NB_COUNT, s);
         const unsigned blocks = (unsigned)pccnn_ceil_div(waves, NB_THREADS / 64);
-        switch (d) {
+        if (group == 64) neighbors_group_kernel<false, false, 64><<<blocks, NB_THREADS, 0, s>>>(a);
+        else if (group == 16) neighbors_group_kernel<false, false, 16><<<blocks, NB_THREADS, 0, s>>>(a);
+        else switch (d) {
         case 3: neighbors_kernel<false, false, NB_UNROLL_COUNT><<<blocks, NB_THREADS, 0, s>>>(a); break;
         case 2: neighbors_generic_kernel<false, false, 2><<<blocks, NB_THREADS, 0, s>>>(a); break;
         case 4: neighbors_generic_kernel<false, false, 4><<<blocks, NB_THREADS, 0, s>>>(a); break;
@@ -539,13 +673,20 @@ extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t 
     a.cell_table = cell_table; a.total_cells = total_cells;
     a.num_cells = num_cells; a.radii = radii; a.max_neighbors = max_neighbors;
     a.counts = counts; a.ends = ends; a.remap = point_remap; a.t = t; a.neigh = neigh_out; a.rec = rec;
-    int64_t waves = pccnn_ceil_div(m, 64);
+    const int group = nb_group_size(n, m, d);
+    int64_t waves = pccnn_ceil_div(m * group, 64);
     {
         PccnnTimed timed(PCCNN_T_NB_FILL, s);
         const unsigned blocks = (unsigned)pccnn_ceil_div(waves, NB_THREADS / 64);
         if (d == 3) {
             if (n > 0) pack_points_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(pts_sorted, point_remap, n, rec);
-            if (max_neighbors > 0) neighbors_kernel<true, true, NB_UNROLL_FILL><<<blocks, NB_THREADS, 0, s>>>(a);
+            if (group == 64) {
+                if (max_neighbors > 0) neighbors_group_kernel<true, true, 64><<<blocks, NB_THREADS, 0, s>>>(a);
+                else neighbors_group_kernel<true, false, 64><<<blocks, NB_THREADS, 0, s>>>(a);
+            } else if (group == 16) {
+                if (max_neighbors > 0) neighbors_group_kernel<true, true, 16><<<blocks, NB_THREADS, 0, s>>>(a);
+                else neighbors_group_kernel<true, false, 16><<<blocks, NB_THREADS, 0, s>>>(a);
+            } else if (max_neighbors > 0) neighbors_kernel<true, true, NB_UNROLL_FILL><<<blocks, NB_THREADS, 0, s>>>(a);
             else neighbors_kernel<true, false, NB_UNROLL_FILL><<<blocks, NB_THREADS, 0, s>>>(a);
         } else {
 #define NB_GENERIC(D)                                                                            \

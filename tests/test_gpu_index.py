@@ -72,6 +72,27 @@ def test_samples_differ_from_points(ops, oracle):
         _compare_neighborhoods(oracle, got, exp)
 
 
+@pytest.mark.parametrize("num_samples", [1400, 330, 40])
+def test_few_samples_against_many_points(ops, oracle, num_samples):
+    # A pooling level: far fewer samples than points.  Below a quarter, and again below a sixteenth, of the point
+    # count several lanes share one sample; the lists (and the capped subsets, which depend on the walk order) must be
+    # those of the one-lane walk and of the oracle, pair for pair.
+    pts, ids = synthetic.primitives(9, 3, 2400)
+    rng = np.random.default_rng(num_samples)
+    pick = np.sort(rng.choice(pts.shape[0], num_samples, replace=False))
+    smp = (pts[pick] + rng.normal(0, 0.004, (num_samples, 3))).astype(np.float32)
+    sids = ids[pick]
+    for cap in (0, 9):
+        exp = oracle.neighborhood(pts, ids, smp, sids, 0.12, max_neighbors=cap)
+        for use_order, use_table in ((True, True), (False, False)):
+            got = gpu_neighborhood(ops, pts, ids, smp, sids, 0.12, 3, max_neighbors=cap, use_order=use_order,
+                                   use_table=use_table)
+            assert np.array_equal(got["ends"], exp["ends"])
+            assert np.array_equal(got["neigh_sorted"], exp["neigh_sorted"])
+            assert np.array_equal(got["neighbors"], exp["neighbors"])
+    assert np.diff(exp["ends"], prepend=0).max() == 9      # the cap binds
+
+
 @pytest.mark.parametrize("cap", [4, 16])
 def test_capped_neighbors(ops, oracle, models, cap):
     pts, ids = _cloud(models, 4, 1000)
