@@ -26,10 +26,40 @@ __global__ void bbox_init_kernel(float *mn, float *mx, int count)
     if (i < count) { mn[i] = __int_as_float(0x7f800000); mx[i] = __int_as_float(0xff800000); }
 }
 
-// Grid-stride reduction.  Every thread keeps a running box for the cloud it is currently in and flushes it
-// with atomics only when the cloud id changes (clouds are normally stored one after the other); at the end a
-// wavefront whose lanes all hold the same cloud reduces with shuffles, and a workgroup whose four wavefronts
-// agree combines them in LDS, so a launch issues a few hundred atomics per box corner at most.
+// The boxes the lanes of a wavefront hold (cloud `cur`, or none when cur < 0) go to memory: for every distinct
+// cloud among them, the lanes holding it are reduced with lane exchanges and one lane issues the
+// atomics.  All lanes of the wavefront must call this together.
+template <int D>
+__device__ __forceinline__ void bbox_flush_wave(int cur, const float (&lo)[D], const float (&hi)[D], float *mn,
+                                                float *mx)
+{
+    const float inf = __int_as_float(0x7f800000);
+    unsigned long long todo = __ballot(cur >= 0);
+    while (todo != 0ull) {
+        const int b = pccnn_bcast_i(cur, __builtin_ctzll(todo));
+        const bool mine = cur == b;
+#pragma unroll
+        for (int k = 0; k < D; ++k) {
+            float l = mine ? lo[k] : inf, h = mine ? hi[k] : -inf;
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                l = fminf(l, __shfl_xor(l, o));
+                h = fmaxf(h, __shfl_xor(h, o));
+            }
+            if (pccnn_lane() == 0) {
+                atomic_min_f32(&mn[b * D + k], l);
+                atomic_max_f32(&mx[b * D + k], h);
+            }
+        }
+        todo &= ~__ballot(mine);
+    }
+}
+
+// Chunked reduction.  A workgroup owns one contiguous chunk of the point list and every thread keeps a running box
+// for the cloud it is currently in (clouds are normally stored one after the other).  When some lane of a
+// wavefront meets another cloud, the wavefront flushes what it holds, one set of atomics per distinct cloud; at the
+// end a wavefront whose lanes all hold the same cloud reduces with exchanges, and a workgroup whose four
+// wavefronts agree combines them in LDS, so a launch issues a few hundred atomics per box corner at most.
 template <int D>
 __global__ void __launch_bounds__(256)
 bbox_reduce_kernel(const float *__restrict__ pts, const int32_t *__restrict__ batch_ids, int64_t n, int batch_size,
@@ -42,20 +72,21 @@ bbox_reduce_kernel(const float *__restrict__ pts, const int32_t *__restrict__ ba
     float lo[D], hi[D];
 #pragma unroll
     for (int k = 0; k < D; ++k) { lo[k] = inf; hi[k] = -inf; }
-    // a workgroup owns one contiguous chunk of the point list, so it rarely sees more than one cloud
     const int64_t chunk = (n + gridDim.x - 1) / gridDim.x;
     const int64_t chunk_end = ((int64_t)blockIdx.x + 1) * chunk < n ? ((int64_t)blockIdx.x + 1) * chunk : n;
-    // four points per thread in flight: their loads do not depend on each other, the box update does
+    // four points per thread in flight: their loads do not depend on each other, the box update does; the trip
+    // count is the same for all threads of the workgroup, so the wavefront-wide flush sits in uniform control flow
     constexpr int UNROLL = 4;
-    for (int64_t i0 = (int64_t)blockIdx.x * chunk + threadIdx.x; i0 < chunk_end; i0 += (int64_t)UNROLL * blockDim.x) {
+    for (int64_t w0 = (int64_t)blockIdx.x * chunk; w0 < chunk_end; w0 += (int64_t)UNROLL * blockDim.x) {
         int bs[UNROLL];
         float vs[UNROLL][D];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            const int64_t i = i0 + (int64_t)u * blockDim.x;
+            const int64_t i = w0 + (int64_t)u * blockDim.x + threadIdx.x;
             bs[u] = -1;
             if (i < chunk_end) {
-                bs[u] = batch_ids[i];
+                const int b = batch_ids[i];
+                bs[u] = (b >= 0 && b < batch_size) ? b : -1;          // ids outside the table are ignored
 #pragma unroll
                 for (int k = 0; k < D; ++k) vs[u][k] = pts[i * D + k];
             }
@@ -63,22 +94,19 @@ bbox_reduce_kernel(const float *__restrict__ pts, const int32_t *__restrict__ ba
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int b = bs[u];
-            if (b < 0 || b >= batch_size) continue;                   // past the chunk, or an id outside the table
-            if (b != cur) {
-                if (cur >= 0) {
+            if (__any(b >= 0 && cur >= 0 && b != cur)) {
+                bbox_flush_wave<D>(cur, lo, hi, mn, mx);
+                cur = -1;
 #pragma unroll
-                    for (int k = 0; k < D; ++k) {
-                        atomic_min_f32(&mn[cur * D + k], lo[k]);
-                        atomic_max_f32(&mx[cur * D + k], hi[k]);
-                        lo[k] = inf; hi[k] = -inf;
-                    }
-                }
-                cur = b;
+                for (int k = 0; k < D; ++k) { lo[k] = inf; hi[k] = -inf; }
             }
+            if (b >= 0) {
+                cur = b;
 #pragma unroll
-            for (int k = 0; k < D; ++k) {
-                lo[k] = fminf(lo[k], vs[u][k]);
-                hi[k] = fmaxf(hi[k], vs[u][k]);
+                for (int k = 0; k < D; ++k) {
+                    lo[k] = fminf(lo[k], vs[u][k]);
+                    hi[k] = fmaxf(hi[k], vs[u][k]);
+                }
             }
         }
     }
@@ -101,14 +129,8 @@ bbox_reduce_kernel(const float *__restrict__ pts, const int32_t *__restrict__ ba
             for (int k = 0; k < D; ++k) { lds_lo[wave][k] = lo[k]; lds_hi[wave][k] = hi[k]; }
         }
     } else {
-        if (lane == 0) lds_b[wave] = -2;                              // handled below, per lane
-        if (cur >= 0) {
-#pragma unroll
-            for (int k = 0; k < D; ++k) {
-                atomic_min_f32(&mn[cur * D + k], lo[k]);
-                atomic_max_f32(&mx[cur * D + k], hi[k]);
-            }
-        }
+        if (lane == 0) lds_b[wave] = -2;                              // flushed here, cloud by cloud
+        bbox_flush_wave<D>(cur, lo, hi, mn, mx);
     }
     __syncthreads();
     if (threadIdx.x == 0) {
