@@ -159,6 +159,16 @@ int pccnn_poisson_disk_select(const int64_t *sorted_keys, int64_t n, const int32
                               void *workspace, size_t workspace_bytes, void *stream);
 int pccnn_compact_selected(const int32_t *selected, const int32_t *selected_scan, int64_t n,
                            int64_t *ids_out, void *stream);
+/* The same selection straight from the grid, without a neighbor list (d == 3): what PointPooling needs from
+ * find_neighbors + poisson_disk_sampling (pccnn_lib/pc/PointPooling.py:58-65) in one call.  pts_sorted f32[n,3] and
+ * sorted_keys in key order, grid_ds / cell_table (nullable) as for pccnn_find_neighbors_count, radii f32[3] = the
+ * cell size.  Outputs and workspace as pccnn_poisson_disk_select; the result is identical to running that on the
+ * uncapped self-neighborhood of the sorted points. */
+int pccnn_poisson_disk_grid(const float *pts_sorted, const int64_t *sorted_keys, int64_t n,
+                            const int32_t *grid_ds, int64_t num_pillars, const int32_t *cell_table,
+                            int64_t total_cells, const int32_t *num_cells, const float *radii, int d,
+                            int32_t *selected_out, int32_t *selected_scan_out,
+                            void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- convolutions -------------------------------------------------------
  * Shapes: pts f32[n,d], feats f32[n,c_in], samples f32[m,d], neigh i32[t,2]

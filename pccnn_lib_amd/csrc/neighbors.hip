@@ -11,6 +11,7 @@
 // segment, two pairs per store, in ascending sorted-point order, so no atomics are used and the
 // output is deterministic.
 #include "common.h"
+#include "grid_walk.h"
 
 // fp32 expressions in this file must round exactly as written (no fused multiply-add).
 #pragma clang fp contract(off)
@@ -57,37 +58,8 @@ __device__ __forceinline__ void nb_store4(int *dst, int a0, int a1, int a2, int 
 __device__ __forceinline__ void nb_pillar_range(const NbArgs &a, long long pillar, int nc2, int cmin, int cmax,
                                                 int &first, int &len)
 {
-    first = 0;
-    len = 0;
-    const long long kbase = pillar * nc2;
-    if (a.cell_table) {
-        // cells cmin..cmax of the pillar are consecutive keys: two table reads give their range
-        if (pillar >= 0 && kbase + cmax + 1 <= a.total_cells) {
-            first = a.cell_table[kbase + cmin];
-            len = a.cell_table[kbase + cmax + 1] - first;
-            if (first < 0 || len < 0 || (int64_t)first + len > a.n) len = 0;
-        }
-    } else if (pillar >= 0 && pillar < a.num_pillars) {
-        int lo = a.grid_ds[2 * pillar], hi = a.grid_ds[2 * pillar + 1];
-        lo = lo < 0 ? 0 : lo;
-        hi = hi > a.n ? (int)a.n : hi;
-        if (hi > lo) {
-            const long long kmin = kbase + cmin;
-            const long long kmax = kbase + cmax;
-            int lb = lo, ub = hi;
-            while (lb < ub) {
-                int mid = (lb + ub) >> 1;
-                if (a.pt_keys[mid] < kmin) lb = mid + 1; else ub = mid;
-            }
-            first = lb;
-            ub = hi;
-            while (lb < ub) {
-                int mid = (lb + ub) >> 1;
-                if (a.pt_keys[mid] <= kmax) lb = mid + 1; else ub = mid;
-            }
-            len = lb - first;
-        }
-    }
+    const GridRef g = {a.cell_table, a.total_cells, a.grid_ds, a.num_pillars, a.pt_keys, a.n};
+    grid_pillar_range(g, pillar, nc2, cmin, cmax, first, len);
 }
 
 // rec[i] = (x, y, z, bits of the id to report for sorted point i): one aligned 16-byte load per candidate

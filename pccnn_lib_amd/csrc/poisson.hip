@@ -11,6 +11,7 @@
 // cell walk of the reference (poisson_disk_sampling.cu:56-105), with the latency of a cell's ~10^3 dependent
 // loads paid across 64 lanes.
 #include "common.h"
+#include "grid_walk.h"
 
 __global__ void __launch_bounds__(256)
 cell_flag_kernel(const int64_t *__restrict__ keys, int64_t n, int32_t *__restrict__ flags)
@@ -104,6 +105,110 @@ poisson_pass_kernel(const int64_t *__restrict__ keys, int64_t n, const int2 *__r
     }
 }
 
+// The same selection without a neighbor list (three dimensions).  A point can only be blocked by a point that is
+// already selected, and those are few: so instead of testing every candidate of the 27-cell walk against every point,
+// the wavefront of a cell reads the selection flags of the walk's index ranges (contiguous, 64 per load), and only
+// for the flagged candidates fetches the position and tests it against the cell's points, one per lane.  Neighbors
+// inside the cell are found by testing the cell's points against each other, and the greedy rule is resolved on the
+// masks as above.  The predicate is the neighbor search's, un-contracted fp32, with the deciding point in the role of
+// the sample (it is symmetric: the differences only change sign).
+struct PoissonGridArgs {
+    const float *pts;            // sorted points [n,3]
+    GridRef grid;
+    const int32_t *num_cells;    // [3]
+    const float *radii;          // [3]
+    volatile int32_t *used;      // [n] selection flags
+    const int32_t *cell_first;   // compact list of the non-empty cells
+    const int32_t *cell_count;
+};
+
+__global__ void __launch_bounds__(256)
+poisson_grid_pass_kernel(PoissonGridArgs a, int colour)
+{
+#pragma clang fp contract(off)
+    __shared__ int2 rng[4][9];
+    const int lane = threadIdx.x & 63;
+    const int wib = threadIdx.x >> 6;
+    const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int64_t waves = ((int64_t)gridDim.x * blockDim.x) >> 6;
+    const int cells = *a.cell_count;
+    const int32_t *settled = (const int32_t *)a.used;
+    const int nc0 = a.num_cells[0], nc1 = a.num_cells[1], nc2 = a.num_cells[2];
+    const float ir0 = __fdiv_rn(1.0f, a.radii[0]);
+    const float ir1 = __fdiv_rn(1.0f, a.radii[1]);
+    const float ir2 = __fdiv_rn(1.0f, a.radii[2]);
+    for (int64_t c = wave; c < cells; c += waves) {
+        const int first = a.cell_first[c];
+        const int last = (c + 1 < cells) ? a.cell_first[c + 1] : (int)a.grid.n;
+        long long k = a.grid.pt_keys[first];
+        const int c2 = (int)(k % nc2); k /= nc2;
+        const int c1 = (int)(k % nc1);
+        const long long pil = k; k /= nc1;
+        const int c0 = (int)(k % nc0);
+        if ((c0 & 1) != (colour & 1) || (c1 & 1) != ((colour >> 1) & 1) || (c2 & 1) != ((colour >> 2) & 1)) continue;
+        // the nine index ranges of the 27-cell walk (lane o looks up range o)
+        if (lane < 9) {
+            const int cmin = c2 > 0 ? c2 - 1 : 0, cmax = c2 + 1 < nc2 ? c2 + 1 : nc2 - 1;
+            const int dx = lane / 3 - 1, dy = lane % 3 - 1;
+            const int x = c0 + dx, y = c1 + dy;
+            int f = 0, l = 0;
+            if (x >= 0 && x < nc0 && y >= 0 && y < nc1)
+                grid_pillar_range(a.grid, pil + (long long)dx * nc1 + dy, nc2, cmin, cmax, f, l);
+            rng[wib][lane] = make_int2(f, l);
+        }
+        for (int base = first; base < last; base += 64) {
+            const int p = base + lane;
+            const bool valid = p < last;
+            float sx = 0.f, sy = 0.f, sz = 0.f;
+            if (valid) { sx = a.pts[(int64_t)p * 3 + 0]; sy = a.pts[(int64_t)p * 3 + 1]; sz = a.pts[(int64_t)p * 3 + 2]; }
+            bool cand = valid;
+            // selected points around the cell: flags first, positions only where a flag is set
+            for (int r = 0; r < 9; ++r) {
+                const int2 g = rng[wib][r];
+                for (int j0 = 0; j0 < g.y; j0 += 64) {
+                    const int q = g.x + j0 + lane;
+                    int flag = 0;
+                    if (j0 + lane < g.y) flag = (q >= first && q < base) ? a.used[q] : settled[q];
+                    unsigned long long set = __ballot(flag != 0);
+                    while (set != 0ull) {
+                        const int qi = g.x + j0 + __builtin_ctzll(set);
+                        set &= set - 1ull;
+                        const float vx = (sx - a.pts[(int64_t)qi * 3 + 0]) * ir0;
+                        const float vy = (sy - a.pts[(int64_t)qi * 3 + 1]) * ir1;
+                        const float vz = (sz - a.pts[(int64_t)qi * 3 + 2]) * ir2;
+                        const float acc = ((0.0f + vx * vx) + vy * vy) + vz * vz;
+                        if (acc < 1.0f) cand = false;
+                    }
+                }
+            }
+            // neighbors among the current points that come before p
+            unsigned long long earlier = 0ull;
+            const int cnt = (last - base) < 64 ? (last - base) : 64;
+            for (int i = 0; i + 1 < cnt; ++i) {
+                const float qx = pccnn_bcast_f(sx, i), qy = pccnn_bcast_f(sy, i), qz = pccnn_bcast_f(sz, i);
+                const float vx = (sx - qx) * ir0;
+                const float vy = (sy - qy) * ir1;
+                const float vz = (sz - qz) * ir2;
+                const float acc = ((0.0f + vx * vx) + vy * vy) + vz * vz;
+                if (i < lane && acc < 1.0f) earlier |= 1ull << i;
+            }
+            // the greedy rule among the current points, in order
+            unsigned long long todo = __ballot(cand);
+            unsigned long long selected = 0ull;
+            while (todo != 0ull) {
+                const int i = __ffsll((long long)todo) - 1;
+                todo &= todo - 1ull;
+                const unsigned lo32 = (unsigned)__builtin_amdgcn_readlane((int)(earlier & 0xffffffffull), i);
+                const unsigned hi32 = (unsigned)__builtin_amdgcn_readlane((int)(earlier >> 32), i);
+                const unsigned long long before = ((unsigned long long)hi32 << 32) | lo32;
+                if ((before & selected) == 0ull) selected |= 1ull << i;
+            }
+            if (valid && ((selected >> lane) & 1ull)) a.used[p] = 1;
+            if (base + 64 < last) __threadfence();
+        }
+    }
+}
+
 __global__ void __launch_bounds__(256)
 compact_kernel(const int32_t *__restrict__ flags, const int32_t *__restrict__ scan, int64_t n,
                int64_t *__restrict__ ids)
@@ -157,6 +262,50 @@ extern "C" int pccnn_poisson_disk_select(const int64_t *sorted_keys, int64_t n, 
     for (int colour = 0; colour < (1 << d); ++colour) {
         PCCNN_DIM_DISPATCH(d, poisson_pass_kernel, <<<(unsigned)pass_blocks, 256, 0, s>>>(
             sorted_keys, n, (const int2 *)neigh, ends, num_cells, colour, selected_out, cell_first, cell_count));
+        PCCNN_LAUNCH_CHECK();
+    }
+    return pccnn_scan_inclusive_i32(selected_out, selected_scan_out, n, 0, scan_tmp, s);
+}
+
+extern "C" int pccnn_poisson_disk_grid(const float *pts_sorted, const int64_t *sorted_keys, int64_t n,
+                                       const int32_t *grid_ds, int64_t num_pillars, const int32_t *cell_table,
+                                       int64_t total_cells, const int32_t *num_cells, const float *radii, int d,
+                                       int32_t *selected_out, int32_t *selected_scan_out, void *workspace,
+                                       size_t workspace_bytes, void *stream)
+{
+    PCCNN_REQUIRE(d == 3, PCCNN_ERR_UNSUPPORTED, "pccnn_poisson_disk_grid: d=%d is not supported (3 only)", d);
+    PCCNN_REQUIRE(n >= 0 && n < (1ll << 31) && num_pillars >= 0, PCCNN_ERR_INVALID,
+                  "pccnn_poisson_disk_grid: n=%lld num_pillars=%lld", (long long)n, (long long)num_pillars);
+    if (n == 0) return PCCNN_OK;
+    PCCNN_REQUIRE(pts_sorted && sorted_keys && grid_ds && num_cells && radii && selected_out && selected_scan_out,
+                  PCCNN_ERR_INVALID, "pccnn_poisson_disk_grid: null pointer");
+    PCCNN_REQUIRE(cell_table == nullptr || total_cells > 0, PCCNN_ERR_INVALID,
+                  "pccnn_poisson_disk_grid: a cell table needs its size");
+    hipStream_t s = (hipStream_t)stream;
+    PccnnArena arena(workspace, workspace_bytes);
+    int32_t *scan_tmp = arena.take<int32_t>(pccnn_scan_tmp_elems(n));
+    int32_t *flags = arena.take<int32_t>((size_t)n);
+    int32_t *cell_first = arena.take<int32_t>((size_t)n);
+    int32_t *cell_count = arena.take<int32_t>(1);
+    PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "pccnn_poisson_disk_grid: workspace of %zu bytes, need %zu",
+                  workspace_bytes, pccnn_poisson_disk_workspace_bytes(n));
+    const unsigned blocks = (unsigned)pccnn_ceil_div(n, 256);
+    cell_flag_kernel<<<blocks, 256, 0, s>>>(sorted_keys, n, flags);
+    PCCNN_LAUNCH_CHECK();
+    int rc = pccnn_scan_inclusive_i32(flags, selected_scan_out, n, 0, scan_tmp, s);
+    if (rc != PCCNN_OK) return rc;
+    cell_list_kernel<<<blocks, 256, 0, s>>>(flags, selected_scan_out, n, cell_first, cell_count);
+    PCCNN_LAUNCH_CHECK();
+    if ((rc = pccnn_fill_i32(selected_out, 0, n, s)) != PCCNN_OK) return rc;
+    PoissonGridArgs a;
+    a.pts = pts_sorted;
+    a.grid = GridRef{cell_table, total_cells, grid_ds, num_pillars, sorted_keys, n};
+    a.num_cells = num_cells; a.radii = radii; a.used = selected_out;
+    a.cell_first = cell_first; a.cell_count = cell_count;
+    int64_t pass_blocks = pccnn_ceil_div(n, 64);
+    if (pass_blocks > 2048) pass_blocks = 2048;
+    for (int colour = 0; colour < 8; ++colour) {
+        poisson_grid_pass_kernel<<<(unsigned)pass_blocks, 256, 0, s>>>(a, colour);
         PCCNN_LAUNCH_CHECK();
     }
     return pccnn_scan_inclusive_i32(selected_out, selected_scan_out, n, 0, scan_tmp, s);

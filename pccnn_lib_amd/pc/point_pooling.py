@@ -22,13 +22,19 @@ class PointPooling(object):
             grid.compute_cell_ids()
             if p_method == "poisson_disk":
                 grid.build_ds()
-                # self-neighborhood in sorted index space (PointPooling.py:58-62); the sorted points are
-                # already in key order, so the natural sample order is the cell order.
-                neighbors, start_ids = pccnn_lib_ops.find_neighbors_ex(
-                    grid.sorted_pts_, grid.sorted_cell_ids_, grid.sorted_pts_, grid.sorted_cell_ids_, grid.grid_ds_,
-                    grid.num_cells_, grid.cell_size_, 0, cell_table=grid.cell_table_)
-                sampled = pccnn_lib_ops.poisson_disk_sampling(grid.sorted_cell_ids_, neighbors, start_ids,
-                                                              grid.num_cells_).reshape(-1)
+                if grid.sorted_pts_.shape[1] == 3:
+                    # three dimensions: the selection straight from the grid, same result as the two calls below
+                    sampled = pccnn_lib_ops.poisson_disk_sampling_grid(
+                        grid.sorted_pts_, grid.sorted_cell_ids_, grid.grid_ds_, grid.num_cells_, grid.cell_size_,
+                        cell_table=grid.cell_table_).reshape(-1)
+                else:
+                    # self-neighborhood in sorted index space (PointPooling.py:58-62); the sorted points are
+                    # already in key order, so the natural sample order is the cell order.
+                    neighbors, start_ids = pccnn_lib_ops.find_neighbors_ex(
+                        grid.sorted_pts_, grid.sorted_cell_ids_, grid.sorted_pts_, grid.sorted_cell_ids_,
+                        grid.grid_ds_, grid.num_cells_, grid.cell_size_, 0, cell_table=grid.cell_table_)
+                    sampled = pccnn_lib_ops.poisson_disk_sampling(grid.sorted_cell_ids_, neighbors, start_ids,
+                                                                  grid.num_cells_).reshape(-1)
                 self.pooling_ids_ = torch.index_select(grid.sorted_ids_, 0, sampled)
             elif p_method == "cell_average":
                 unique_ids, inverse_ids = torch.unique(grid.cell_ids_, return_inverse=True)

@@ -310,6 +310,41 @@ def poisson_disk_sampling(sorted_keys, neigh, ends, grid_size):
     return ids
 
 
+def poisson_disk_sampling_grid(sorted_pts, sorted_keys, grid_ds, grid_size, radii, cell_table=None):
+    """Poisson-disk selection straight from the grid (no counterpart in the reference's module; it is what
+    pccnn_lib/pc/PointPooling.py:58-65 computes with find_neighbors + poisson_disk_sampling): sorted points
+    f32[N,3], sorted keys i64[N], pillar table, grid_size i32[3], radii f32[3] (= the cell size) -> i64[S,1] in
+    sorted-index space, identical to poisson_disk_sampling on the uncapped self-neighborhood."""
+    name = "poisson_disk_sampling_grid"
+    _chk(sorted_pts, name + ": pts", torch.float32, 2)
+    dev = sorted_pts.device
+    _chk(sorted_keys, name + ": keys", torch.int64, 1, dev)
+    _chk(grid_ds, name + ": grid_ds", torch.int32, 4, dev)
+    _chk(grid_size, name + ": grid_size", torch.int32, 1, dev)
+    _chk(radii, name + ": radii", torch.float32, 1, dev)
+    n = sorted_pts.shape[0]
+    if sorted_pts.shape[1] != 3 or sorted_keys.shape[0] != n or grid_size.shape[0] != 3 or radii.shape[0] != 3 \
+            or grid_ds.shape[3] != 2:
+        raise RuntimeError(name + ": 3-D points [N,3], keys [N], grid_ds [B,nc0,nc1,2], grid_size [3], radii [3]")
+    if n == 0:
+        return torch.empty((0, 1), dtype=torch.int64, device=dev)
+    total_cells = 0
+    if cell_table is not None:
+        _chk(cell_table, name + ": cell_table", torch.int32, 1, dev)
+        total_cells = cell_table.shape[0] - 1
+    sel = torch.empty((n,), dtype=torch.int32, device=dev)
+    scan = torch.empty_like(sel)
+    ws = _workspace(_lib.load().pccnn_poisson_disk_workspace_bytes(n), dev)
+    num_pillars = grid_ds.shape[0] * grid_ds.shape[1] * grid_ds.shape[2]
+    _lib.call("pccnn_poisson_disk_grid", _ptr(sorted_pts), _ptr(sorted_keys), n, _ptr(grid_ds), num_pillars,
+              _optr(cell_table), total_cells, _ptr(grid_size), _ptr(radii), 3, _ptr(sel), _ptr(scan), _ptr(ws),
+              ws.numel(), _stream())
+    count = int(scan[-1].item())
+    ids = torch.empty((count, 1), dtype=torch.int64, device=dev)
+    _lib.call("pccnn_compact_selected", _ptr(sel), _ptr(scan), n, _ptr(ids), _stream())
+    return ids
+
+
 # ----------------------------------------------------------------------------- conv
 
 # Gradient groups of the backward entry points (PCCNN_GRAD_* in include/pccnn_hip.h).

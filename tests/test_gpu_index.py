@@ -173,6 +173,27 @@ def test_poisson_disk_matches_oracle(ops, oracle, models):
         assert np.array_equal(sel.cpu().numpy(), e_sel)
 
 
+@pytest.mark.parametrize("batch,num_pts,radius,use_table", [(4, 1000, 0.1, True), (3, 4000, 0.05, False),
+                                                            (1, 3000, 0.45, True), (2, 2500, 0.3, False),
+                                                            (1, 40, 5.0, True)])
+def test_poisson_disk_from_the_grid_equals_the_list_version(ops, oracle, batch, num_pts, radius, use_table):
+    # The list-free selection (flags of the walk's index ranges, positions only of flagged candidates) must pick
+    # exactly the points the neighbor-list version and the oracle pick; the large radii put hundreds of points in a
+    # cell, so a cell takes several rounds of 64.
+    pts, ids = synthetic.primitives(70 + batch, batch, num_pts)
+    exp = oracle.neighborhood(pts, ids, pts, ids, radius)
+    e_neigh, e_ends = oracle.find_neighbors(exp["sorted_pts"], exp["sorted_keys"], exp["sorted_pts"],
+                                            exp["sorted_keys"], exp["grid_ds"], exp["num_cells"], exp["radii"])
+    e_sel = oracle.poisson_disk_sampling(exp["sorted_keys"], e_neigh, e_ends, exp["num_cells"])
+    g = gpu_neighborhood(ops, pts, ids, pts, ids, radius, batch)["dev"]
+    table = ops.build_cell_table(g["skeys"], batch * int(np.prod(g["nc"].tolist()))) if use_table else None
+    sel = ops.poisson_disk_sampling_grid(g["spts"], g["skeys"], g["ds"], g["nc"], g["radii"], cell_table=table)
+    assert sel.dtype == torch.int64 and sel.shape[1] == 1
+    assert np.array_equal(sel.cpu().numpy(), e_sel)
+    neigh, ends = ops.find_neighbors_ex(g["spts"], g["skeys"], g["spts"], g["skeys"], g["ds"], g["nc"], g["radii"], 0)
+    assert torch.equal(sel, ops.poisson_disk_sampling(g["skeys"], neigh, ends, g["nc"]))
+
+
 def test_run_twice_is_bitwise_identical(ops):
     pts, ids = synthetic.primitives(11, 2, 3000)
     a = gpu_neighborhood(ops, pts, ids, pts, ids, 0.06, 2)
