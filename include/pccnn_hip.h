@@ -46,6 +46,11 @@ int pccnn_version(void);
  * pts f32[n,d], batch_ids i32[n] in [0,batch_size) -> aabb_min/max f32[batch_size,d]. */
 int pccnn_bounding_box(const float *pts, const int32_t *batch_ids, int64_t n, int d, int batch_size,
                        float *aabb_min_out, float *aabb_max_out, void *stream);
+/* Grid size for a cell size: replaces the torch arithmetic of pccnn_lib/pc/Grid.py:26-28,
+ * num_cells[k] = max over the clouds of int32((aabb_max - aabb_min) / cell_size) + 1 (fp32 division, truncation).
+ * aabb_min/max f32[batch_size,d], cell_size f32[d] -> num_cells_out i32[d]. */
+int pccnn_num_cells(const float *aabb_min, const float *aabb_max, const float *cell_size, int batch_size, int d,
+                    int32_t *num_cells_out, void *stream);
 
 /* ---- cell keys ----------------------------------------------------------
  * Replaces compute_keys (pccnn_lib_ops/compute_keys/compute_keys.cuh:26-31,

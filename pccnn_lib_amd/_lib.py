@@ -32,6 +32,7 @@ SIGNATURES = {
     "pccnn_last_error": (ctypes.c_char_p, []),
     "pccnn_version": (I32, []),
     "pccnn_bounding_box": (I32, [P, P, I64, I32, I32, P, P, P]),
+    "pccnn_num_cells": (I32, [P, P, P, I32, I32, P, P]),
     "pccnn_compute_keys": (I32, [P, P, P, P, P, I64, I32, P, P]),
     "pccnn_sort_keys_workspace_bytes": (SZ, [I64]),
     "pccnn_sort_keys": (I32, [P, I64, I32, P, P, P, I32, P, P, SZ, P]),

@@ -183,6 +183,32 @@ extern "C" int pccnn_bounding_box(const float *pts, const int32_t *batch_ids, in
     return PCCNN_OK;
 }
 
+// num_cells[k] = max_b int((max[b][k] - min[b][k]) / cell[k]) + 1: one thread per dimension, clouds in order.
+__global__ void num_cells_kernel(const float *__restrict__ mn, const float *__restrict__ mx,
+                                 const float *__restrict__ cell, int batch_size, int d, int32_t *__restrict__ out)
+{
+    const int k = threadIdx.x;
+    if (k >= d) return;
+    int best = 0;
+    for (int b = 0; b < batch_size; ++b) {
+        const int c = (int)__fdiv_rn(mx[b * d + k] - mn[b * d + k], cell[k]) + 1;
+        best = (b == 0 || c > best) ? c : best;
+    }
+    out[k] = best;
+}
+
+extern "C" int pccnn_num_cells(const float *aabb_min, const float *aabb_max, const float *cell_size, int batch_size,
+                               int d, int32_t *num_cells_out, void *stream)
+{
+    PCCNN_REQUIRE(d >= 2 && d <= PCCNN_MAX_DIMS, PCCNN_ERR_UNSUPPORTED, "pccnn_num_cells: d=%d is not supported (2 <= d <= 6)",
+                  d);
+    PCCNN_REQUIRE(batch_size > 0, PCCNN_ERR_INVALID, "pccnn_num_cells: batch_size=%d", batch_size);
+    PCCNN_REQUIRE(aabb_min && aabb_max && cell_size && num_cells_out, PCCNN_ERR_INVALID, "pccnn_num_cells: null pointer");
+    num_cells_kernel<<<1, 64, 0, (hipStream_t)stream>>>(aabb_min, aabb_max, cell_size, batch_size, d, num_cells_out);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
 // ------------------------------------------------------------------- keys
 
 template <int D>

@@ -21,8 +21,8 @@ class Grid(object):
             self.cell_size_ = self.cell_size_.repeat(p_point_cloud.pts_.shape[1])
         with torch.no_grad():
             # Grid.py:26-28: fp32 division, truncation, + 1, maximum over the clouds.
-            num_cells = (self.bounding_box_.max_ - self.bounding_box_.min_) / self.cell_size_
-            self.num_cells_ = torch.max(num_cells.to(torch.int32) + 1, dim=0)[0].contiguous()
+            self.num_cells_ = pccnn_lib_ops.num_cells(self.bounding_box_.min_, self.bounding_box_.max_,
+                                                      self.cell_size_.contiguous())
         self.num_cells_host_ = None
         self.cell_ids_ = None
         self.sorted_ids_i64_ = None

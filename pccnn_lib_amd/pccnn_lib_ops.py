@@ -76,6 +76,21 @@ def bounding_box(pts, batch_ids, batch_size):
     return mn, mx
 
 
+def num_cells(aabb_min, aabb_max, cell_size):
+    """Grid size i32[D] = max over the clouds of int32((max - min) / cell_size) + 1 (pccnn_lib/pc/Grid.py:26-28)."""
+    name = "num_cells"
+    _chk(aabb_min, name + ": aabb_min", torch.float32, 2)
+    dev = aabb_min.device
+    _chk(aabb_max, name + ": aabb_max", torch.float32, 2, dev)
+    _chk(cell_size, name + ": cell_size", torch.float32, 1, dev)
+    b, d = aabb_min.shape
+    if tuple(aabb_max.shape) != (b, d) or cell_size.shape[0] != d or d < MIN_DIMS or d > MAX_DIMS or b < 1:
+        raise RuntimeError(name + ": aabb_min / aabb_max must be [B, D], cell_size [D], 2 <= D <= 6")
+    out = torch.empty((d,), dtype=torch.int32, device=dev)
+    _lib.call("pccnn_num_cells", _ptr(aabb_min), _ptr(aabb_max), _ptr(cell_size), b, d, _ptr(out), _stream())
+    return out
+
+
 def compute_keys(pts, batch_ids, aabb_min, grid_size, cell_size):
     """compute_keys(pts f32[N,D], batch_ids i32[N], aabb_min f32[B,D], grid_size i32[D], cell_size f32[D]) -> i64[N]
     (pccnn_lib_ops/compute_keys/compute_keys.cuh:26-31)."""

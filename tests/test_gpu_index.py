@@ -194,6 +194,19 @@ def test_poisson_disk_from_the_grid_equals_the_list_version(ops, oracle, batch, 
     assert torch.equal(sel, ops.poisson_disk_sampling(g["skeys"], neigh, ends, g["nc"]))
 
 
+def test_num_cells_matches_the_reference_arithmetic(ops, oracle):
+    # Grid.py:26-28: fp32 division, truncation towards zero, + 1, maximum over the clouds
+    rng = np.random.default_rng(12)
+    for dims in (2, 3, 6):
+        mn = rng.uniform(-2, 0, (5, dims)).astype(np.float32)
+        mx = (mn + rng.uniform(0.01, 3, (5, dims))).astype(np.float32)
+        for cell in (0.05, 0.1, 0.37):
+            cs = np.full(dims, cell, np.float32)
+            got = ops.num_cells(t(mn), t(mx), t(cs)).cpu().numpy()
+            assert np.array_equal(got, oracle.num_cells(mn, mx, cs))
+            assert np.array_equal(got, (((mx - mn) / cs).astype(np.int32) + 1).max(axis=0))
+
+
 def test_run_twice_is_bitwise_identical(ops):
     pts, ids = synthetic.primitives(11, 2, 3000)
     a = gpu_neighborhood(ops, pts, ids, pts, ids, 0.06, 2)
