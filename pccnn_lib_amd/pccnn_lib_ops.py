@@ -217,6 +217,9 @@ def find_neighbors_ex(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, ra
               presorted, _ptr(grid_ds), pillars, table_p, total_cells, _ptr(grid_size), _ptr(radii), d, max_neighbors, _ptr(ends),
               _ptr(ws), ws.numel(), _stream())
     total = int(ends[-1].item())                      # the one host read-back, as in the reference
+    if total < 0:
+        raise RuntimeError(name + ": more than 2^31 - 1 pairs; the pair offsets are 32-bit as in the reference, "
+                                  "use a smaller radius, a neighbor cap or fewer samples per call")
     neigh = torch.empty((total, 2), dtype=torch.int32, device=dev)
     _lib.call("pccnn_find_neighbors_fill", _ptr(pts), _ptr(pt_keys), n, _ptr(samples), _ptr(sample_keys), m, order_p,
               presorted, _ptr(grid_ds), pillars, table_p, total_cells, _ptr(grid_size), _ptr(radii), d, max_neighbors, _ptr(ends),
