@@ -17,7 +17,8 @@ density pipeline are timed as well and reported as extra keys of the same JSON l
                 divided by its mean launch duration, taken live with HIP events on the launch stream;
   roofline_neighbors   the same for the neighbor fill kernel against HBM bandwidth, measured on the
                 million-point room of config 4 (`scene` carries that leg's pairs / second);
-  cpu_baseline  the CPU oracle (scalar C + numpy, one thread) on a bounded sample of the same workload.
+  cpu_baseline  the same step on the host cores: the vectorised torch form of the oracle on all threads over the whole
+                workload, and the scalar oracle (C + numpy, one thread) on two clouds beside it.
 
 Exactly one JSON line goes to stdout; progress goes to stderr.
 """
@@ -63,40 +64,57 @@ def make_workload(seed=2, batch=16, num_pts=4096, c_in=64, c_out=128, hidden=16)
         c_in=c_in, c_out=c_out, hidden=hidden)
 
 
-def cpu_baseline(wl, clouds=2):
-    """The oracle's MCConv forward + backward on the first `clouds` clouds, one thread."""
-    from oracle import oracle
+def cpu_baseline(wl, scalar_clouds=2):
+    """The same MCConv forward + backward on the host cores: the vectorised torch form on all threads over the whole
+    workload (the reported baseline), and the scalar oracle on one thread over the first clouds beside it."""
+    import torch
+    from oracle import oracle, torch_cpu
     try:
         from threadpoolctl import threadpool_limits
     except ImportError:                                           # pragma: no cover
         threadpool_limits = None
-    n = clouds * wl["num_pts"]
-    pts, ids, feats = wl["pts"][:n], wl["ids"][:n], wl["feats"][:n]
+    n = wl["batch"] * wl["num_pts"]
+    pts, ids, feats = wl["pts"], wl["ids"], wl["feats"]
     unnorm, _, _ = oracle.pointcloud_pdf(pts, ids, wl["bandwidth"])
     nb = oracle.neighborhood(pts, ids, pts, ids, wl["radius"])
     pdf = (unnorm * np.prod(nb["radii"])).astype(np.float32)
-    args = (pts, pdf, feats, pts, nb["neighbors"], nb["ends"], nb["radii"], wl["axis"], wl["bias"], wl["weights"])
 
-    def run():
-        oracle.mcconv(*args)
-        oracle.mcconv_grads(*args, wl["out_grads"][:n])
-
-    ctx = threadpool_limits(limits=1) if threadpool_limits else None
-    try:
+    def timed(run, budget_s, max_reps):
         run()                                                     # warm-up
         t0 = time.perf_counter()
         reps = 0
-        while reps < 3 and (reps == 0 or time.perf_counter() - t0 < 20.0):
+        while reps < max_reps and (reps == 0 or time.perf_counter() - t0 < budget_s):
             run()
             reps += 1
-        dt = (time.perf_counter() - t0) / reps
+        return (time.perf_counter() - t0) / reps, reps
+
+    threads = torch.get_num_threads()
+    dt, reps = timed(lambda: torch_cpu.mcconv_step(pts, pdf, feats, nb["neighbors"], nb["ends"], nb["radii"], wl["axis"],
+                                                   wl["bias"], wl["weights"], wl["out_grads"]), 15.0, 20)
+    result = {"value": n / dt, "unit": "points/s", "cores": threads, "kind": "port",
+              "sample": "vectorised torch-CPU MCConv forward + all gradients (oracle/torch_cpu.py) on all %d clouds "
+                        "(%d points, %d pairs), %d repetition(s), neighbor search and density excluded like in `value`"
+                        % (wl["batch"], n, nb["neighbors"].shape[0], reps)}
+
+    ns = scalar_clouds * wl["num_pts"]
+    pairs = int(nb["ends"][ns - 1])
+    args = (pts[:ns], pdf[:ns], feats[:ns], pts[:ns], nb["neighbors"][:pairs], nb["ends"][:ns], nb["radii"], wl["axis"],
+            wl["bias"], wl["weights"])
+
+    def scalar():
+        oracle.mcconv(*args)
+        oracle.mcconv_grads(*args, wl["out_grads"][:ns])
+
+    ctx = threadpool_limits(limits=1) if threadpool_limits else None
+    try:
+        dts, _ = timed(scalar, 8.0, 3)
     finally:
         if ctx is not None:
             ctx.unregister() if hasattr(ctx, "unregister") else ctx.restore_original_limits()
-    return {"value": n / dt, "unit": "points/s", "cores": 1, "kind": "port",
-            "sample": "oracle mcconv + mcconv_grads on %d of %d clouds (%d points, %d pairs), %d repetition(s), "
-                      "neighbor search and density excluded like in `value`" % (clouds, wl["batch"], n,
-                                                                               nb["neighbors"].shape[0], reps)}
+    result["scalar_oracle"] = {"value": ns / dts, "unit": "points/s", "cores": 1,
+                               "sample": "oracle mcconv + mcconv_grads (scalar C + numpy) on %d of %d clouds"
+                                         % (scalar_clouds, wl["batch"])}
+    return result
 
 
 def main():

@@ -234,6 +234,29 @@ def test_mcconv_grads_match_autograd(oracle, models, num_mlps):
         assert _relerr(mine, ref.grad.numpy()) < 1e-4, name
 
 
+def test_torch_cpu_step_matches_the_scalar_oracle(oracle, models):
+    """The multi-threaded CPU baseline (padded, batched form) computes what the scalar oracle computes, including the
+    samples whose list is shorter than the padding, an empty list and a ragged last chunk."""
+    from oracle import torch_cpu
+    c_in, c_out, hidden = 8, 6, 8
+    pts, ids, nb, feats, rng = _setup(oracle, models, 0.2, c_in, 21)
+    pts[-1] += 50.0                                   # a point far from everything: its only neighbor is itself
+    nb = oracle.neighborhood(pts, ids, pts, ids, 0.2)
+    neigh, ends, radii = nb["neighbors"], nb["ends"], nb["radii"]
+    pdf = rng.uniform(0.5, 2.0, pts.shape[0]).astype(np.float32)
+    axis = rng.normal(0, 0.6, (3, hidden)).astype(np.float32)
+    bias = rng.normal(0, 0.2, (1, hidden)).astype(np.float32)
+    w = rng.normal(0, 0.2, (1, hidden * c_in, c_out)).astype(np.float32)
+    g = rng.normal(size=(pts.shape[0], c_out)).astype(np.float32)
+    out, grads = torch_cpu.mcconv_step(pts, pdf, feats, neigh, ends, radii, axis, bias, w, g, samples_per_chunk=300)
+    ref = oracle.mcconv(pts, pdf, feats, pts, neigh, ends, radii, axis, bias, w)
+    dw, dfeat, daxis, dbias, dpdf, dpts, dsmp = oracle.mcconv_grads(pts, pdf, feats, pts, neigh, ends, radii, axis, bias, w, g)
+    assert _relerr(out, ref) < 1e-5
+    for name, want in (("weights", dw), ("feats", dfeat), ("axis", daxis), ("bias", dbias), ("pdf", dpdf),
+                       ("pts", dpts + dsmp)):
+        assert _relerr(grads[name].reshape(want.shape), want) < 1e-4, name
+
+
 def test_weight_variance_equals_projection_norm(oracle, models):
     # The double sum over neighbor pairs of (w_i . w_j)(F_i . F_j) (compute_variance_weights.cu:38-108) is the
     # squared Frobenius norm of the sample's projection tile; the literal O(n^2) restatement must agree with it.
