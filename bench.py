@@ -155,6 +155,25 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    # what a plain float4 copy reaches on this part, as the practical ceiling beside the published 8 TB/s: 1 GiB read
+    # and 1 GiB written per launch (beyond every cache), timed with events on the launch stream
+    src = torch.ones(256 << 20, dtype=torch.float32, device=dev)
+    dst = torch.empty_like(src)
+    cs = torch.cuda.current_stream()
+    copy_call = lambda: _lib.call("pccnn_calibration_copy", _lib.P(src.data_ptr()), _lib.P(dst.data_ptr()), src.numel(),
+                                  _lib.P(cs.cuda_stream))
+    for _ in range(2):
+        copy_call()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(cs)
+    for _ in range(5):
+        copy_call()
+    e1.record(cs)
+    torch.cuda.synchronize()
+    copy_gbps = 5 * 2.0 * src.numel() * 4 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+    log("copy ceiling: %.0f GB/s" % copy_gbps)
+    del src, dst
+
     wl = make_workload()
     t = lambda a: torch.as_tensor(a, device=dev)
     pts, ids, feats = t(wl["pts"]), t(wl["ids"]), t(wl["feats"])
@@ -331,7 +350,8 @@ def main():
         "density_ms": pdf_ms,
         "kernels_us": {leg: {k: round(1e3 * v[1] / v[0], 2) for k, v in ks.items()}
                        for leg, ks in (("conv", conv_kernels), ("neighborhood", nb_kernels), ("density", pdf_kernels))},
-        "bf16_contraction": bf16_leg, "scene": scene, "roofline": roofline, "roofline_neighbors": roofline_nb, "cpu_baseline": cpu,
+        "bf16_contraction": bf16_leg, "scene": scene, "roofline": roofline, "roofline_neighbors": roofline_nb, "hbm_copy_ceiling_gbps": copy_gbps,
+        "cpu_baseline": cpu,
     }
     print(json.dumps(result), flush=True)
     return 0
