@@ -125,8 +125,6 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-scene", action="store_true", help="skip the million-point neighbor-search leg")
     ap.add_argument("--scene-points", type=int, default=1000000)
-    ap.add_argument("--calibration-copies", type=int, default=0,
-                    help="also launch this many 256 MiB calibration copies (for scaling rocprofv3 --pmc counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on one GPU only; --gpus %d is not supported "
@@ -146,17 +144,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    if args.calibration_copies > 0:
-        src = torch.ones(64 << 20, dtype=torch.float32, device=dev)
-        dst = torch.empty_like(src)
-        for _ in range(args.calibration_copies):
-            _lib.call("pccnn_calibration_copy", _lib.P(src.data_ptr()), _lib.P(dst.data_ptr()), src.numel(),
-                      _lib.P(torch.cuda.current_stream().cuda_stream))
-        torch.cuda.synchronize()
-        del src, dst
-
     # what a plain float4 copy reaches on this part, as the practical ceiling beside the published 8 TB/s: 1 GiB read
-    # and 1 GiB written per launch (beyond every cache), timed with events on the launch stream
+    # and 1 GiB written per launch (beyond every cache), timed with events on the launch stream.  The same launches
+    # are the known-size yardstick that rocprofv3's traffic counters are scaled against.
     src = torch.ones(256 << 20, dtype=torch.float32, device=dev)
     dst = torch.empty_like(src)
     cs = torch.cuda.current_stream()

@@ -5,6 +5,7 @@
 #include <math.h>
 
 #include "common.h"
+#include "grid_walk.h"
 
 // fp32 expressions in this file must round exactly as written (no fused multiply-add).
 #pragma clang fp contract(off)
@@ -146,6 +147,190 @@ extern "C" int pccnn_compute_pdf_sorted(int manifold_dims, const float *bandwidt
     PCCNN_REQUIRE(samples, PCCNN_ERR_INVALID, "pccnn_compute_pdf_sorted: null samples");
     return pdf_launch<false>(d, manifold_dims, bandwidth, pts_sorted, samples, n, neigh_sorted, t, ends, nullptr, pdf_out,
                              (hipStream_t)stream);
+}
+
+// ------------------------------------------------------------------- density straight from the grid
+// Pointcloud.compute_pdf of the reference (pccnn_lib/pc/Pointcloud.py:81-109) builds a neighbor list with radius
+// 4 x bandwidth and at most 300 neighbors only to sum a Gaussian over it and drop it.  Here one lane per point walks
+// the 3 x 3 pillar ranges around its cell (the walk of the neighbor search, same order, same fp32 predicate) and adds
+// the kernel values as it goes: no pair list, no count / scan / fill, no host read-back of the pair count.  A point
+// with more hits than the cap walks a second time and keeps the subset the capped neighbor search keeps (hit number
+// r iff floor((r + 1) cap / raw) > floor(r cap / raw)), so both routes sum the same terms in the same order.
+struct PdfGridArgs {
+    const float *pts;          // [n,3] in key order
+    const int64_t *keys;       // [n] sorted
+    const int32_t *order;      // nullable [n]: original index of sorted point i
+    GridRef grid;
+    const int32_t *num_cells;  // [3]
+    const float *radii;        // [3] search radii (= cell size)
+    const float *bandwidth;    // [3]
+    double norm_const;
+    int max_neighbors;
+    float *out;                // [n] in original order
+    int64_t n;
+};
+
+#define PDF_GRID_UNROLL 4
+
+template <bool CAPPED>
+__device__ __forceinline__ void pdf_grid_walk(const PdfGridArgs &a, const int2 (*ranges)[64], int lane, int nr, bool go,
+                                              float sx, float sy, float sz, const float (&ir)[3], const float (&ib)[3],
+                                              double scale, int raw, int step, double &sum, int &cnt)
+{
+    int r = 0, j = 0, first = 0, len = 0, err = 0;
+    bool active = go && nr > 0;
+    if (active) {
+        const int2 g = ranges[0][lane];
+        first = g.x;
+        len = g.y;
+    }
+    while (__any(active)) {
+        if (active) {
+            const int idx = first + j;
+            const int left = len - j;
+            float px[PDF_GRID_UNROLL], py[PDF_GRID_UNROLL], pz[PDF_GRID_UNROLL];
+#pragma unroll
+            for (int u = 0; u < PDF_GRID_UNROLL; ++u) {
+                const int64_t iu = idx + (u < left ? u : 0);
+                px[u] = a.pts[iu * 3 + 0];
+                py[u] = a.pts[iu * 3 + 1];
+                pz[u] = a.pts[iu * 3 + 2];
+            }
+#pragma unroll
+            for (int u = 0; u < PDF_GRID_UNROLL; ++u) {
+                // the predicate of the neighbor search: ((s - p) / r)^2 summed x, y, z in fp32, below 1
+                const float vx = (sx - px[u]) * ir[0];
+                const float vy = (sy - py[u]) * ir[1];
+                const float vz = (sz - pz[u]) * ir[2];
+                const float acc = ((0.0f + vx * vx) + vy * vy) + vz * vz;
+                if (u < left && acc < 1.0f) {
+                    bool take = true;
+                    if (CAPPED) {
+                        err += step;
+                        take = err >= raw;
+                        if (take) err -= raw;
+                    }
+                    if (take) {
+                        // the term of pdf_kernel: ((p - s) / bandwidth)^2 summed in fp32, exp in fp32, scaled in double
+                        const float d0 = (px[u] - sx) * ib[0];
+                        const float d1 = (py[u] - sy) * ib[1];
+                        const float d2 = (pz[u] - sz) * ib[2];
+                        const float dot = ((0.0f + d0 * d0) + d1 * d1) + d2 * d2;
+                        sum += scale * (double)expf(dot * (-0.5f));
+                    }
+                    ++cnt;
+                }
+            }
+            j += PDF_GRID_UNROLL;
+            if (j >= len) {
+                j = 0;
+                if (++r < nr) {
+                    const int2 g = ranges[r][lane];
+                    first = g.x;
+                    len = g.y;
+                } else {
+                    active = false;
+                }
+            }
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256)
+pdf_grid_kernel(PdfGridArgs a)
+{
+    __shared__ int2 ranges[4][9][64];          // written and read by the same lane only
+    const int lane = pccnn_lane();
+    const int wib = threadIdx.x >> 6;
+    const int64_t base = (((int64_t)blockIdx.x * 256 + threadIdx.x) >> 6) * 64;
+    if (base >= a.n) return;                   // wave-uniform
+    const int64_t i = base + lane;
+    const bool valid = i < a.n;
+    long long key = -1;
+    float sx = 0.f, sy = 0.f, sz = 0.f;
+    if (valid) {
+        key = a.keys[i];
+        sx = a.pts[i * 3 + 0];
+        sy = a.pts[i * 3 + 1];
+        sz = a.pts[i * 3 + 2];
+    }
+    const int nc0 = a.num_cells[0], nc1 = a.num_cells[1], nc2 = a.num_cells[2];
+    float ir[3], ib[3];
+    float prod = 1.0f;
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+        ir[c] = __fdiv_rn(1.0f, a.radii[c]);
+        ib[c] = __fdiv_rn(1.0f, a.bandwidth[c]);
+        prod = prod * ib[c];
+    }
+    const double scale = (double)prod * a.norm_const;
+    const bool usable = valid && key >= 0;
+    long long k = usable ? key : 0;
+    const int c2 = (int)(k % nc2); k /= nc2;
+    const int c1 = (int)(k % nc1);
+    const long long pil = k; k /= nc1;
+    const int c0 = (int)(k % nc0);
+    int nr = 0;
+    if (usable) {
+        const int cmin = c2 > 0 ? c2 - 1 : 0, cmax = c2 + 1 < nc2 ? c2 + 1 : nc2 - 1;
+#pragma unroll
+        for (int o = 0; o < 9; ++o) {
+            const int dx = o / 3 - 1, dy = o % 3 - 1;
+            const int x = c0 + dx, y = c1 + dy;
+            if (x >= 0 && x < nc0 && y >= 0 && y < nc1) {
+                int first, len;
+                grid_pillar_range(a.grid, pil + (long long)dx * nc1 + dy, nc2, cmin, cmax, first, len);
+                if (len > 0) {
+                    ranges[wib][nr][lane] = make_int2(first, len);
+                    ++nr;
+                }
+            }
+        }
+    }
+    double sum = 0.0;
+    int cnt = 0;
+    pdf_grid_walk<false>(a, ranges[wib], lane, nr, usable, sx, sy, sz, ir, ib, scale, 0, 0, sum, cnt);
+    const bool redo = a.max_neighbors > 0 && cnt > a.max_neighbors;
+    if (__any(redo)) {
+        double capped_sum = 0.0;
+        int again = 0;
+        pdf_grid_walk<true>(a, ranges[wib], lane, nr, redo, sx, sy, sz, ir, ib, scale, cnt, a.max_neighbors, capped_sum,
+                            again);
+        if (redo) sum = capped_sum;
+    }
+    if (valid) a.out[a.order ? (int64_t)a.order[i] : i] = (float)sum;
+}
+
+extern "C" int pccnn_compute_pdf_grid(int manifold_dims, const float *bandwidth, const float *pts_sorted,
+                                      const int64_t *sorted_keys, int64_t n, const int32_t *sample_order,
+                                      const int32_t *grid_ds, int64_t num_pillars, const int32_t *cell_table,
+                                      int64_t total_cells, const int32_t *num_cells, const float *radii, int d,
+                                      int max_neighbors, float *pdf_out, void *stream)
+{
+    PCCNN_REQUIRE(d == 3, PCCNN_ERR_UNSUPPORTED, "pccnn_compute_pdf_grid: d=%d is not supported (3 only; use "
+                  "pccnn_find_neighbors_* and pccnn_compute_pdf)", d);
+    PCCNN_REQUIRE(n >= 0 && n < (1ll << 31) && num_pillars >= 0 && max_neighbors >= 0, PCCNN_ERR_INVALID,
+                  "pccnn_compute_pdf_grid: n=%lld num_pillars=%lld max_neighbors=%d", (long long)n,
+                  (long long)num_pillars, max_neighbors);
+    if (n == 0) return PCCNN_OK;
+    PCCNN_REQUIRE(bandwidth && pts_sorted && sorted_keys && grid_ds && num_cells && radii && pdf_out, PCCNN_ERR_INVALID,
+                  "pccnn_compute_pdf_grid: null pointer");
+    PCCNN_REQUIRE(!cell_table || (total_cells > 0 && total_cells < (1ll << 40)), PCCNN_ERR_INVALID,
+                  "pccnn_compute_pdf_grid: total_cells=%lld", (long long)total_cells);
+    PdfGridArgs a;
+    a.pts = pts_sorted; a.keys = sorted_keys; a.order = sample_order;
+    a.grid.cell_table = cell_table; a.grid.total_cells = total_cells; a.grid.grid_ds = grid_ds;
+    a.grid.num_pillars = num_pillars; a.grid.pt_keys = sorted_keys; a.grid.n = n;
+    a.num_cells = num_cells; a.radii = radii; a.bandwidth = bandwidth;
+    a.norm_const = 1.0 / pow(2.0 * 3.1415, (double)(float)manifold_dims / 2.0);
+    a.max_neighbors = max_neighbors; a.out = pdf_out; a.n = n;
+    hipStream_t s = (hipStream_t)stream;
+    {
+        PccnnTimed timed(PCCNN_T_PDF, s);
+        pdf_grid_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(a);
+    }
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
 }
 
 extern "C" int pccnn_compute_pdf_grads(int manifold_dims, const float *bandwidth, const float *pts, int64_t n,

@@ -287,6 +287,45 @@ def compute_pdf_sorted(manifold_dims, bandwidth, pts_sorted, samples, neigh_sort
     return out
 
 
+def compute_pdf_grid(manifold_dims, bandwidth, sorted_pts, sorted_keys, sample_order, grid_ds, grid_size, radii,
+                     max_neighbors=0, cell_table=None):
+    """The density of every point straight from the grid (no counterpart in the reference's module; it is what
+    pccnn_lib/pc/Pointcloud.py:81-109 computes with find_neighbors + compute_pdf): sorted points f32[N,3], sorted
+    keys i64[N], sample_order i32[N] (original index of sorted point i; None = the points already are in key
+    order), pillar table, grid_size i32[3], radii f32[3] (the search radii = cell size) -> f32[N] in the original
+    order, the same terms in the same order as compute_pdf on the (capped) neighbor list."""
+    name = "compute_pdf_grid"
+    _chk(sorted_pts, name + ": pts", torch.float32, 2)
+    dev = sorted_pts.device
+    _chk(bandwidth, name + ": bandwidth", torch.float32, 1, dev)
+    _chk(sorted_keys, name + ": keys", torch.int64, 1, dev)
+    _chk(grid_ds, name + ": grid_ds", torch.int32, 4, dev)
+    _chk(grid_size, name + ": grid_size", torch.int32, 1, dev)
+    _chk(radii, name + ": radii", torch.float32, 1, dev)
+    n = sorted_pts.shape[0]
+    if sorted_pts.shape[1] != 3 or sorted_keys.shape[0] != n or grid_size.shape[0] != 3 or radii.shape[0] != 3 \
+            or bandwidth.shape[0] != 3 or grid_ds.shape[3] != 2:
+        raise RuntimeError(name + ": 3-D points [N,3], keys [N], grid_ds [B,nc0,nc1,2], grid_size / radii / "
+                                  "bandwidth [3]")
+    max_neighbors = int(max_neighbors)
+    if max_neighbors < 0:
+        raise RuntimeError(name + ": max_neighbors must be >= 0")
+    if sample_order is not None:
+        _chk(sample_order, name + ": sample_order", torch.int32, 1, dev)
+        if sample_order.shape[0] != n:
+            raise RuntimeError(name + ": sample_order has the wrong length")
+    total_cells = 0
+    if cell_table is not None:
+        _chk(cell_table, name + ": cell_table", torch.int32, 1, dev)
+        total_cells = cell_table.shape[0] - 1
+    out = torch.empty((n,), dtype=torch.float32, device=dev)
+    num_pillars = grid_ds.shape[0] * grid_ds.shape[1] * grid_ds.shape[2]
+    _lib.call("pccnn_compute_pdf_grid", int(manifold_dims), _ptr(bandwidth), _ptr(sorted_pts), _ptr(sorted_keys), n,
+              _optr(sample_order), _ptr(grid_ds), num_pillars, _optr(cell_table), total_cells, _ptr(grid_size),
+              _ptr(radii), 3, max_neighbors, _ptr(out), _stream())
+    return out
+
+
 def compute_pdf_grads(manifold_dims, bandwidth, pts, neigh, ends, in_grads):
     """compute_pdf_grads(..., in_grads f32[N]) -> f32[N,D] (pccnn_lib_ops/compute_pdf/compute_pdf.cuh:45-51)."""
     d = _pdf_args("compute_pdf_grads", bandwidth, pts, neigh, ends)

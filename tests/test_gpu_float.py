@@ -77,6 +77,38 @@ def test_pdf_matches_oracle(ops, oracle, models, bw):
     assert np.allclose(pc.pts_unnorm_pdf_.cpu().numpy(), exp_unnorm, rtol=1e-5, atol=0)
 
 
+@pytest.mark.parametrize("cap", [0, 300, 7])
+def test_pdf_from_the_grid_equals_the_list_route(ops, models, cap):
+    """compute_pdf_grid sums what compute_pdf sums over the (capped) neighbor list of the same grid, in the same
+    order: with double accumulation the two agree to the last bit or two of the fp32 result."""
+    import pccnn_lib_amd as lib
+    pts, ids = _cloud(models, 3, 1000)
+    rooms = (synthetic.room(11, 20000) / 10.0).astype(np.float32)
+    for cloud, cloud_ids, bw in ((pts, ids, 0.05), (rooms, np.zeros(rooms.shape[0], np.int32), 0.004)):
+        pc = lib.pc.Pointcloud(cloud, cloud_ids, device=DEV)
+        bandwidth = torch.full((3,), bw, device=DEV)
+        grid = lib.pc.Grid(pc, lib.pc.BoundingBox(pc), bandwidth * 4.0)
+        grid.compute_cell_ids()
+        grid.build_ds()
+        neigh, ends = ops.find_neighbors_ex(grid.sorted_pts_, grid.sorted_cell_ids_, grid.sorted_pts_,
+                                            grid.sorted_cell_ids_, grid.grid_ds_, grid.num_cells_, grid.cell_size_, cap,
+                                            sample_order=grid.sorted_ids_i32_, cell_table=grid.cell_table_,
+                                            samples_presorted=True)
+        want = ops.compute_pdf_sorted(3, bandwidth, grid.sorted_pts_, pc.pts_, neigh, ends)
+        for table in (grid.cell_table_, None):
+            got = ops.compute_pdf_grid(3, bandwidth, grid.sorted_pts_, grid.sorted_cell_ids_, grid.sorted_ids_i32_,
+                                       grid.grid_ds_, grid.num_cells_, grid.cell_size_, cap, cell_table=table)
+            torch.cuda.synchronize()
+            assert np.allclose(got.cpu().numpy(), want.cpu().numpy(), rtol=3e-7, atol=0)
+        if cap == 7:
+            counts = np.diff(np.concatenate([[0], ends.cpu().numpy()]))
+            assert counts.max() == 7                          # the cap is reached, the subset rule is exercised
+        # points already in key order, no sample_order: the result comes out in that order
+        direct = ops.compute_pdf_grid(3, bandwidth, grid.sorted_pts_, grid.sorted_cell_ids_, None, grid.grid_ds_,
+                                      grid.num_cells_, grid.cell_size_, cap, cell_table=grid.cell_table_)
+        assert torch.equal(direct, got[grid.sorted_ids_.to(torch.int64)])
+
+
 def test_pdf_grads_match_oracle(ops, oracle, models):
     pts, ids = _cloud(models, 2, 500)
     bw = np.full(3, 0.08, np.float32)
