@@ -1,5 +1,5 @@
-// Stable LSD radix sort of (64-bit cell key, 32-bit index) pairs, 8 bits per pass, only over
-// the significant key bits.  Per pass:
+// Stable LSD radix sort of (64-bit cell key, 32-bit index) pairs over the significant key bits only, 8 to 11
+// bits per pass (see rs_plan).  Per pass:
 //   1. radix_hist_kernel    : per-tile digit histogram staged in LDS, stored digit-major
 //   2. radix_scan_kernel    : one workgroup per digit scans that digit's per-tile counts
 //   3. radix_scatter_kernel : every tile re-reads its keys, ranks them with wave ballots
@@ -21,20 +21,28 @@ static int rs_items_for(int64_t n)
     return (int)(items < 1 ? 1 : (items > RS_MAX_ITEMS ? RS_MAX_ITEMS : items));
 }
 
+// BITS bits per pass, D = 2^BITS digits; thread t of a workgroup looks after digits t, t + 256, ...
+template <int BITS>
 __global__ void __launch_bounds__(RS_THREADS)
 radix_hist_kernel(const int64_t *__restrict__ keys, int64_t n, int shift, int items, int32_t *__restrict__ tile_hist,
                   int64_t num_tiles)
 {
-    __shared__ int hist[256];
-    hist[threadIdx.x] = 0;
+    constexpr int D = 1 << BITS;
+    __shared__ int hist[D];
+#pragma unroll
+    for (int q = 0; q < D / RS_THREADS; ++q) hist[threadIdx.x + q * RS_THREADS] = 0;
     __syncthreads();
     int64_t base = (int64_t)blockIdx.x * RS_THREADS * items;
     for (int r = 0; r < items; ++r) {
         int64_t i = base + r * RS_THREADS + threadIdx.x;
-        if (i < n) atomicAdd(&hist[(int)((keys[i] >> shift) & 0xff)], 1);
+        if (i < n) atomicAdd(&hist[(int)((keys[i] >> shift) & (D - 1))], 1);
     }
     __syncthreads();
-    tile_hist[(int64_t)threadIdx.x * num_tiles + blockIdx.x] = hist[threadIdx.x];
+#pragma unroll
+    for (int q = 0; q < D / RS_THREADS; ++q) {
+        const int d = threadIdx.x + q * RS_THREADS;
+        tile_hist[(int64_t)d * num_tiles + blockIdx.x] = hist[d];
+    }
 }
 
 // One workgroup per digit: exclusive scan of that digit's per-tile counts (contiguous in the digit-major
@@ -71,21 +79,30 @@ radix_scan_kernel(int32_t *__restrict__ tile_hist, int64_t num_tiles, int32_t *_
     if (threadIdx.x == 0) digit_totals[blockIdx.x] = carry;
 }
 
-template <bool FIRST, bool GATHER>
+template <int BITS, bool FIRST, bool GATHER>
 __global__ void __launch_bounds__(RS_THREADS)
 radix_scatter_kernel(const int64_t *__restrict__ keys_in, const int32_t *__restrict__ vals_in, int64_t n, int shift,
                      int items, const int32_t *__restrict__ tile_offsets, int64_t num_tiles,
                      const int32_t *__restrict__ digit_totals, int64_t *__restrict__ keys_out, int32_t *__restrict__ vals_out,
                      const float *__restrict__ pts, float *__restrict__ pts_out, int dims)
 {
-    __shared__ int running[256];                       // next free output slot per digit
-    __shared__ int wave_cnt[RS_WAVES][256];
+    constexpr int D = 1 << BITS;
+    constexpr int PER = D / RS_THREADS;
+    __shared__ int running[D];                         // next free output slot per digit
+    __shared__ int wave_cnt[RS_WAVES][D];
     int lane = pccnn_lane();
     int wave = threadIdx.x >> 6;
-    // first output slot of digit d for this tile = (keys with a smaller digit) + (same digit in earlier tiles)
+    // first output slot of digit d for this tile = (keys with a smaller digit) + (same digit in earlier tiles);
+    // for this prefix thread t takes the PER consecutive digits t * PER ...
     {
-        const int tot = digit_totals[threadIdx.x];
-        int incl = tot;
+        int tot[PER];
+        int sum = 0;
+#pragma unroll
+        for (int q = 0; q < PER; ++q) {
+            tot[q] = digit_totals[threadIdx.x * PER + q];
+            sum += tot[q];
+        }
+        int incl = sum;
 #pragma unroll
         for (int o = 1; o < 64; o <<= 1) {
             const int t = __shfl_up(incl, o);
@@ -93,15 +110,22 @@ radix_scatter_kernel(const int64_t *__restrict__ keys_in, const int32_t *__restr
         }
         if (lane == 63) wave_cnt[0][wave] = incl;
         __syncthreads();
-        int add = 0;
+        int excl = incl - sum;
 #pragma unroll
         for (int w = 0; w < RS_WAVES; ++w)
-            if (w < wave) add += wave_cnt[0][w];
-        running[threadIdx.x] = add + incl - tot + tile_offsets[(int64_t)threadIdx.x * num_tiles + blockIdx.x];
+            if (w < wave) excl += wave_cnt[0][w];
         __syncthreads();
+#pragma unroll
+        for (int q = 0; q < PER; ++q) {
+            const int d = threadIdx.x * PER + q;
+            running[d] = excl + tile_offsets[(int64_t)d * num_tiles + blockIdx.x];
+            excl += tot[q];
+        }
     }
 #pragma unroll
-    for (int w = 0; w < RS_WAVES; ++w) wave_cnt[w][threadIdx.x] = 0;
+    for (int w = 0; w < RS_WAVES; ++w)
+#pragma unroll
+        for (int q = 0; q < PER; ++q) wave_cnt[w][threadIdx.x + q * RS_THREADS] = 0;
     __syncthreads();
     int64_t base = (int64_t)blockIdx.x * RS_THREADS * items;
     unsigned long long lt = pccnn_lanemask_lt();
@@ -110,11 +134,11 @@ radix_scatter_kernel(const int64_t *__restrict__ keys_in, const int32_t *__restr
         bool valid = i < n;
         long long key = valid ? keys_in[i] : 0;
         int val = FIRST ? (int)i : (valid ? vals_in[i] : 0);
-        int digit = (int)((key >> shift) & 0xff);
+        int digit = (int)((key >> shift) & (D - 1));
         // lanes of this wave holding the same digit
         unsigned long long peers = __ballot(valid);
 #pragma unroll
-        for (int b = 0; b < 8; ++b) {
+        for (int b = 0; b < BITS; ++b) {
             unsigned long long bal = __ballot((digit >> b) & 1);
             peers &= ((digit >> b) & 1) ? bal : ~bal;
         }
@@ -135,15 +159,35 @@ radix_scatter_kernel(const int64_t *__restrict__ keys_in, const int32_t *__restr
             }
         }
         __syncthreads();
-        int tot = 0;
 #pragma unroll
-        for (int w = 0; w < RS_WAVES; ++w) {
-            tot += wave_cnt[w][threadIdx.x];
-            wave_cnt[w][threadIdx.x] = 0;
+        for (int q = 0; q < PER; ++q) {
+            const int d = threadIdx.x + q * RS_THREADS;
+            int tot = 0;
+#pragma unroll
+            for (int w = 0; w < RS_WAVES; ++w) {
+                tot += wave_cnt[w][d];
+                wave_cnt[w][d] = 0;
+            }
+            running[d] += tot;
         }
-        running[threadIdx.x] += tot;
         __syncthreads();
     }
+}
+
+// Passes and bits per pass for keys of `key_bits` significant bits: as few passes as the widest digit allows,
+// the bits spread evenly over them (18 bits: 2 x 9; 24: 3 x 8).  Wide digits pay where a pass is bound by its three
+// launches: up to 11 bits for at most 2^18 keys (65 536 keys of 18 bits: 26 us in 2 passes against 35 us in 3).
+// On a million keys a pass with 2^11 digits leaves two keys per digit and tile, its scattered stores and the
+// larger table cost more than the saved pass (22 bits: 116 us in 2 passes against 99 us in 3), and 9 bits are the
+// widest digit that still wins (800 000 keys of 18 bits: 72 us against 80 us).
+#define RS_MAX_BITS 11
+#define RS_MAX_DIGITS (1 << RS_MAX_BITS)
+static void rs_plan(int key_bits, int64_t n, int &passes, int &bits)
+{
+    const int widest = n <= (1 << 18) ? RS_MAX_BITS : 9;
+    passes = (key_bits + widest - 1) / widest;
+    bits = (key_bits + passes - 1) / passes;
+    if (bits < 8) bits = 8;
 }
 
 extern "C" size_t pccnn_sort_keys_workspace_bytes(int64_t n)
@@ -151,7 +195,7 @@ extern "C" size_t pccnn_sort_keys_workspace_bytes(int64_t n)
     if (n < 0) n = 0;
     int64_t tiles = pccnn_ceil_div(n > 0 ? n : 1, (int64_t)RS_THREADS * rs_items_for(n));
     return pccnn_align((size_t)n * sizeof(int64_t)) + pccnn_align((size_t)n * sizeof(int32_t)) +
-           pccnn_align((size_t)tiles * 256 * sizeof(int32_t)) + pccnn_align(256 * sizeof(int32_t)) + 256;
+           pccnn_align((size_t)tiles * RS_MAX_DIGITS * sizeof(int32_t)) + pccnn_align(RS_MAX_DIGITS * sizeof(int32_t)) + 256;
 }
 
 extern "C" int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int64_t *sorted_keys_out,
@@ -170,14 +214,15 @@ extern "C" int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int
                   pccnn_sort_keys_workspace_bytes(n));
     hipStream_t s = (hipStream_t)stream;
     if (key_bits <= 0 || key_bits > 63) key_bits = 63;     // keys are non-negative
-    int passes = (key_bits + 7) / 8;
+    int passes, bits;
+    rs_plan(key_bits, n, passes, bits);
     const int items = rs_items_for(n);
     int64_t tiles = pccnn_ceil_div(n, (int64_t)RS_THREADS * items);
     PccnnArena arena(workspace, workspace_bytes);
     int64_t *tmp_keys = arena.take<int64_t>((size_t)n);
     int32_t *tmp_vals = arena.take<int32_t>((size_t)n);
-    int32_t *hist = arena.take<int32_t>((size_t)tiles * 256);
-    int32_t *totals = arena.take<int32_t>(256);
+    int32_t *hist = arena.take<int32_t>((size_t)tiles * RS_MAX_DIGITS);
+    int32_t *totals = arena.take<int32_t>(RS_MAX_DIGITS);
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "pccnn_sort_keys: workspace too small");
 
     PccnnTimed timed(PCCNN_T_SORT, s);
@@ -187,29 +232,35 @@ extern "C" int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int
         bool to_out = ((passes - 1 - p) % 2) == 0;
         int64_t *dst_k = to_out ? sorted_keys_out : tmp_keys;
         int32_t *dst_v = to_out ? perm_out : tmp_vals;
-        int shift = 8 * p;
+        int shift = bits * p;
         bool last = (p == passes - 1);
-        radix_hist_kernel<<<(unsigned)tiles, RS_THREADS, 0, s>>>(src_k, n, shift, items, hist, tiles);
-        PCCNN_LAUNCH_CHECK();
-        radix_scan_kernel<<<256, 256, 0, s>>>(hist, tiles, totals);
-        PCCNN_LAUNCH_CHECK();
         bool gather = last && pts != nullptr;
-        if (p == 0) {
-            if (gather)
-                radix_scatter_kernel<true, true><<<(unsigned)tiles, RS_THREADS, 0, s>>>(
-                    src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, pts, sorted_pts_out, d);
-            else
-                radix_scatter_kernel<true, false><<<(unsigned)tiles, RS_THREADS, 0, s>>>(
-                    src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, nullptr, nullptr, d);
-        } else {
-            if (gather)
-                radix_scatter_kernel<false, true><<<(unsigned)tiles, RS_THREADS, 0, s>>>(
-                    src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, pts, sorted_pts_out, d);
-            else
-                radix_scatter_kernel<false, false><<<(unsigned)tiles, RS_THREADS, 0, s>>>(
-                    src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, nullptr, nullptr, d);
+        const unsigned grid = (unsigned)tiles;
+#define RS_SCATTER(B, FIRST, GATHER)                                                                            \
+    radix_scatter_kernel<B, FIRST, GATHER><<<grid, RS_THREADS, 0, s>>>(src_k, src_v, n, shift, items, hist, tiles, \
+                                                                       totals, dst_k, dst_v, GATHER ? pts : nullptr, \
+                                                                       GATHER ? sorted_pts_out : nullptr, d)
+#define RS_PASS(B)                                                                                   \
+    do {                                                                                             \
+        radix_hist_kernel<B><<<grid, RS_THREADS, 0, s>>>(src_k, n, shift, items, hist, tiles);       \
+        PCCNN_LAUNCH_CHECK();                                                                        \
+        radix_scan_kernel<<<1 << B, 256, 0, s>>>(hist, tiles, totals);                               \
+        PCCNN_LAUNCH_CHECK();                                                                        \
+        if (p == 0) {                                                                                \
+            if (gather) RS_SCATTER(B, true, true); else RS_SCATTER(B, true, false);                  \
+        } else {                                                                                     \
+            if (gather) RS_SCATTER(B, false, true); else RS_SCATTER(B, false, false);                \
+        }                                                                                            \
+        PCCNN_LAUNCH_CHECK();                                                                        \
+    } while (0)
+        switch (bits) {
+        case 8: RS_PASS(8); break;
+        case 9: RS_PASS(9); break;
+        case 10: RS_PASS(10); break;
+        default: RS_PASS(11); break;
         }
-        PCCNN_LAUNCH_CHECK();
+#undef RS_PASS
+#undef RS_SCATTER
         src_k = dst_k;
         src_v = dst_v;
     }

@@ -21,7 +21,14 @@ from . import _lib
 _P = _lib.P
 
 
+# torch's current stream as a raw hipStream_t: the C-level getter when this torch has it (a fraction of a
+# microsecond), else through the Stream object (several microseconds, once per native call)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream():
+    if _raw_stream is not None:
+        return _P(_raw_stream(torch.cuda.current_device()))
     return _P(torch.cuda.current_stream().cuda_stream)
 
 

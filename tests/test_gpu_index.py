@@ -148,7 +148,9 @@ def test_empty_sample_set(ops):
 
 def test_sort_is_stable_and_handles_many_passes(ops):
     rng = np.random.default_rng(7)
-    for n, bits in ((1, 8), (2049, 3), (100000, 20), (70001, 40), (5000, 63)):
+    # digit widths 8 to 11 and 1 to 6 passes: up to 2^18 keys take digits of up to 11 bits, more keys of up to 9
+    for n, bits in ((1, 8), (2049, 3), (100000, 20), (70001, 40), (5000, 63), (1000, 9), (4000, 11), (60000, 18),
+                    (60000, 22), (300000, 18), (300000, 26), (300000, 5)):
         keys = rng.integers(0, 2 ** min(bits, 62), n, dtype=np.int64)
         pts = rng.normal(size=(n, 3)).astype(np.float32)
         skeys, perm, spts = ops.sort_keys(t(keys), bits, t(pts))
