@@ -1,7 +1,6 @@
 import torch
 
 from .. import pccnn_lib_ops
-from ..op_wrappers import BuildGridDS, ComputeKeys
 
 
 class Grid(object):
@@ -51,8 +50,8 @@ class Grid(object):
         if self.cell_ids_ is None:
             with torch.no_grad():
                 pts = self.pointcloud_.pts_.detach()
-                self.cell_ids_ = ComputeKeys.apply(pts, self.pointcloud_.batch_ids_, self.bounding_box_.min_,
-                                                   self.num_cells_, self.cell_size_)
+                self.cell_ids_ = pccnn_lib_ops.compute_keys(pts, self.pointcloud_.batch_ids_, self.bounding_box_.min_,
+                                                            self.num_cells_, self.cell_size_)
                 self.sorted_cell_ids_, self.sorted_ids_i32_, self.sorted_pts_ = pccnn_lib_ops.sort_keys(
                     self.cell_ids_, self.key_bits(), pts)
 

@@ -1,7 +1,6 @@
 import torch
 
 from .. import pccnn_lib_ops
-from ..op_wrappers import ComputeKeys
 
 
 class Neighborhood(object):
@@ -25,8 +24,8 @@ class Neighborhood(object):
             if p_samples is grid.pointcloud_:
                 sorted_keys, order, sorted_pts = grid.sorted_cell_ids_, grid.sorted_ids_i32_, grid.sorted_pts_
             else:
-                sample_keys = ComputeKeys.apply(sample_pts, p_samples.batch_ids_, grid.bounding_box_.min_,
-                                                grid.num_cells_, grid.cell_size_)
+                sample_keys = pccnn_lib_ops.compute_keys(sample_pts, p_samples.batch_ids_, grid.bounding_box_.min_,
+                                                         grid.num_cells_, grid.cell_size_)
                 sorted_keys, order, sorted_pts = pccnn_lib_ops.sort_keys(sample_keys, grid.key_bits(), sample_pts)
             self.neighbors_, self.start_ids_ = pccnn_lib_ops.find_neighbors_ex(
                 grid.sorted_pts_, grid.sorted_cell_ids_, sorted_pts, sorted_keys, grid.grid_ds_, grid.num_cells_,

@@ -251,3 +251,52 @@ def test_config5_hierarchy_8x100k_properties(oracle):
                         (ends[sin] - p_lo).astype(np.int32), radii, p(layer.proj_axis_), p(layer.proj_bias_),
                         p(layer.conv_weights_), contraction="bf16")
     assert relerr(p(lv["out"])[sin], exp) < 3e-3
+
+
+def test_projection_with_more_than_two_to_the_31_elements(ops):
+    # Maximum sizes: 2.2 million samples x 64 features x 16 hidden units put 2.25e9 floats (9 GB) into the projection
+    # and as many into its gradient, past what 32-bit element offsets reach.  No oracle runs at this size; the check
+    # is that samples are independent: the convolution of the first and of the second part of the samples, run as two
+    # smaller calls on re-based pair lists, must give the rows of the full call (forward) and gradients that add up
+    # to the full call's (backward; summation order differs, hence the tolerance).
+    import pccnn_lib_amd as lib
+    n, c_in, hidden, c_out = 2_200_000, 64, 16, 32
+    rng = np.random.default_rng(31)
+    pts = t(rng.random((n, 3), dtype=np.float32))
+    ids = torch.zeros(n, dtype=torch.int32, device=DEV)
+    radii = torch.full((3,), 0.006, device=DEV)
+    pc = lib.pc.Pointcloud(pts, ids)
+    nbh = lib.pc.layers.conv_base.build_neighborhood(pc, pc, radii, 0)
+    neigh, ends = nbh.neighbors_, nbh.start_ids_
+    assert neigh.shape[0] > 2 * n                       # on average more than the point itself
+    gen = torch.Generator(device=DEV).manual_seed(31)
+    feats = torch.randn((n, c_in), device=DEV, generator=gen)
+    pdf = torch.rand((n,), device=DEV, generator=gen) + 0.5
+    axis = torch.randn((3, hidden), device=DEV, generator=gen) * 0.6
+    bias = torch.randn((1, hidden), device=DEV, generator=gen) * 0.2
+    w = torch.randn((1, hidden * c_in, c_out), device=DEV, generator=gen) * 0.03
+    g = torch.randn((n, c_out), device=DEV, generator=gen)
+
+    out, proj = ops.mc_conv(pts, pdf, feats, pts, neigh, ends, radii, axis, bias, w, return_proj=True)
+    assert proj.numel() > 2 ** 31
+    full = ops.mc_conv_grads(pts, pdf, feats, pts, neigh, ends, radii, axis, bias, w, g, proj=proj)
+    del proj
+    h = n // 2 + 12345
+    cut = int(ends[h - 1])
+    parts = []
+    for lo, hi, p_lo, p_hi in ((0, h, 0, cut), (h, n, cut, neigh.shape[0])):
+        nb = neigh[p_lo:p_hi].clone()
+        nb[:, 1] -= lo
+        en = (ends[lo:hi] - p_lo).contiguous()
+        smp = pts[lo:hi].contiguous()
+        o = ops.mc_conv(pts, pdf, feats, smp, nb, en, radii, axis, bias, w)
+        assert torch.allclose(o, out[lo:hi], rtol=1e-6, atol=1e-6), (lo, hi)
+        parts.append(ops.mc_conv_grads(pts, pdf, feats, smp, nb, en, radii, axis, bias, w, g[lo:hi].contiguous()))
+        del o, nb, en, smp
+    torch.cuda.synchronize()
+    names = ("dW", "dFeat", "dAxis", "dBias", "dPdf", "dPts")
+    for i, name in enumerate(names):
+        summed = parts[0][i] + parts[1][i]
+        assert relerr(summed.cpu().numpy(), full[i].cpu().numpy()) < GRAD_TOL, name
+    d_samples = torch.cat([parts[0][6], parts[1][6]])
+    assert relerr(d_samples.cpu().numpy(), full[6].cpu().numpy()) < GRAD_TOL

@@ -256,3 +256,14 @@ def test_scene_scale_properties(ops):
     bwd = neigh[:, 1].astype(np.int64) * pts.shape[0] + neigh[:, 0]
     assert np.array_equal(np.sort(fwd), np.sort(bwd))
     assert np.count_nonzero(neigh[:, 0] == neigh[:, 1]) == pts.shape[0]
+
+
+def test_pair_count_beyond_32_bits_is_an_error(ops):
+    # 50 000 points inside one search radius are 2.5e9 pairs: the offsets are 32-bit as in the reference, so the
+    # search refuses instead of returning wrapped offsets
+    import pccnn_lib_amd as lib
+    n = 50000
+    pts = t(np.random.default_rng(3).random((n, 3), dtype=np.float32) * 0.1)
+    pc = lib.pc.Pointcloud(pts, torch.zeros(n, dtype=torch.int32, device=DEV))
+    with pytest.raises(RuntimeError, match="pairs"):
+        lib.pc.layers.conv_base.build_neighborhood(pc, pc, torch.full((3,), 1.0, device=DEV), 0)
