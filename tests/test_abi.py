@@ -117,3 +117,20 @@ def test_layers_keep_reference_parameter_names():
     assert tuple(sph.conv_weights_.shape) == (31 * 8, 16)
     pcv = PointConv(3, 8, 16, 16)
     assert {"proj_axis_", "proj_bias_", "conv_weights_", "pdf_mlp_.0.weight", "pdf_mlp_.2.weight"} <= set(pcv.state_dict())
+
+
+def test_install_as_reference_resolves_the_reference_imports():
+    # in a process of its own: the call registers modules under the reference's names
+    import subprocess
+    import sys
+    code = ("import pccnn_lib_amd; pccnn_lib_amd.install_as_reference()\n"
+            "import pccnn_lib, pccnn_lib_ops\n"
+            "from pccnn_lib.pc import Pointcloud, BoundingBox, Grid, Neighborhood, PointPooling\n"
+            "from pccnn_lib.pc.layers import KPConv, MCConv, KPConvN, PCCNN, PointConv, SPHConv\n"
+            "from pccnn_lib.op_wrappers import ComputeKeys, BuildGridDS, FindNeighbors, ComputePDF\n"
+            "assert pccnn_lib.pc.Pointcloud is pccnn_lib_amd.pc.Pointcloud\n"
+            "assert callable(pccnn_lib_ops.compute_keys) and callable(pccnn_lib_ops.mc_conv_grads)\n")
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr
