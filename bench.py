@@ -313,12 +313,27 @@ def main():
                        "frac": s_gbps / HBM_PEAK_GBPS,
                        "traffic": TRAFFIC_NB_FILL_BYTES_SCENE if n_s == 1000000 else None, "bytes_per_launch": s_bytes,
                        "avg_launch_ms": f_avg, "launches": f_n}
+        # the density of the same scene (Pointcloud.compute_pdf, bandwidth 0.2 x radius: its own grid of cell size
+        # 4 x bandwidth, then the KDE walk on it)
+        sbw = np.full(3, 0.2 * 0.05, np.float32)
+
+        def scene_pdf_step():
+            p = lib.pc.Pointcloud.__new__(lib.pc.Pointcloud)
+            p.__dict__.update(spc.__dict__)
+            p.compute_pdf(sbw)
+            return p
+
+        scene_pdf_step()
+        sp_ms, sp_kernels = timed(scene_pdf_step, max(args.steps // 2, 3), 2)
         scene = {"points": n_s, "pairs": s_pairs, "neighborhood_ms": s_ms,
                  "neighbor_pairs_per_sec": s_pairs / (s_ms * 1e-3),
-                 "kernels_us": {k: round(1e3 * v[1] / v[0], 2) for k, v in s_kernels.items()}}
+                 "kernels_us": {k: round(1e3 * v[1] / v[0], 2) for k, v in s_kernels.items()},
+                 "density_ms": sp_ms, "density_bandwidth": 0.01,
+                 "density_kernels_us": {k: round(1e3 * v[1] / v[0], 2) for k, v in sp_kernels.items()}}
         log("scene: %d points, %d pairs, neighborhood %.3f ms -> %.2f G pairs/s" % (n_s, s_pairs, s_ms,
                                                                                   s_pairs / s_ms / 1e6))
         log("scene", {k: "%d x %.1f us" % (v[0], 1e3 * v[1] / v[0]) for k, v in s_kernels.items()})
+        log("scene density %.3f ms" % sp_ms, {k: "%d x %.1f us" % (v[0], 1e3 * v[1] / v[0]) for k, v in sp_kernels.items()})
 
     cpu = None
     if not args.no_cpu_baseline:

@@ -153,12 +153,14 @@ int pccnn_compute_pdf_sorted(int manifold_dims, const float *bandwidth, const fl
  * sorted_keys i64[n] in key order; sample_order i32[n] (nullable) = original index of sorted point i, the row of
  * pdf_out it is written to; grid_ds / cell_table (nullable) / num_cells / radii (the search radii = cell size) as
  * for pccnn_find_neighbors_count.  With max_neighbors > 0 a point with more hits sums the subset that the capped
- * search keeps.  The terms and their order are those of pccnn_compute_pdf on that list. */
+ * search keeps.  The terms and their order are those of pccnn_compute_pdf on that list.  pdf_norm_out (nullable)
+ * f32[n] receives the estimate divided by the number of points of the point's cloud (pts_pdf_ of
+ * Pointcloud.py:105-109). */
 int pccnn_compute_pdf_grid(int manifold_dims, const float *bandwidth, const float *pts_sorted,
                            const int64_t *sorted_keys, int64_t n, const int32_t *sample_order,
                            const int32_t *grid_ds, int64_t num_pillars, const int32_t *cell_table,
                            int64_t total_cells, const int32_t *num_cells, const float *radii, int d,
-                           int max_neighbors, float *pdf_out, void *stream);
+                           int max_neighbors, float *pdf_out, float *pdf_norm_out, void *stream);
 int pccnn_compute_pdf_grads(int manifold_dims, const float *bandwidth, const float *pts, int64_t n, int d,
                             const int32_t *neigh, int64_t t, const int32_t *ends, const float *in_grads,
                             float *pt_grads_out, void *stream);

@@ -45,7 +45,7 @@ SIGNATURES = {
     "pccnn_compute_pdf": (I32, [I32, P, P, I64, I32, P, I64, P, P, P]),
     "pccnn_compute_pdf_sorted": (I32, [I32, P, P, P, I64, I32, P, I64, P, P, P]),
     "pccnn_compute_pdf_grads": (I32, [I32, P, P, I64, I32, P, I64, P, P, P, P]),
-    "pccnn_compute_pdf_grid": (I32, [I32, P, P, P, I64, P, P, I64, P, I64, P, P, I32, I32, P, P]),
+    "pccnn_compute_pdf_grid": (I32, [I32, P, P, P, I64, P, P, I64, P, I64, P, P, I32, I32, P, P, P]),
     "pccnn_poisson_disk_workspace_bytes": (SZ, [I64]),
     "pccnn_poisson_disk_select": (I32, [P, I64, P, I64, P, P, I32, P, P, P, SZ, P]),
     "pccnn_compact_selected": (I32, [P, P, I64, P, P]),

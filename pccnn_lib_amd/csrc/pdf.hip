@@ -167,8 +167,28 @@ struct PdfGridArgs {
     double norm_const;
     int max_neighbors;
     float *out;                // [n] in original order
+    float *out_norm;           // nullable [n]: out divided by the number of points of the point's cloud
     int64_t n;
 };
+
+// Number of points of cloud b: its keys are the range [b * cells, (b + 1) * cells) of the sorted keys.
+__device__ __forceinline__ int pdf_grid_cloud_count(const PdfGridArgs &a, long long b, long long cells)
+{
+    const long long k_lo = b * cells, k_hi = k_lo + cells;
+    if (a.grid.cell_table && k_hi <= a.grid.total_cells) return a.grid.cell_table[k_hi] - a.grid.cell_table[k_lo];
+    int64_t bound[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+        const long long want = e == 0 ? k_lo : k_hi;        // first index whose key is >= want
+        int64_t lb = 0, ub = a.n;
+        while (lb < ub) {
+            const int64_t mid = (lb + ub) >> 1;
+            if (a.keys[mid] < want) lb = mid + 1; else ub = mid;
+        }
+        bound[e] = lb;
+    }
+    return (int)(bound[1] - bound[0]);
+}
 
 #define PDF_GRID_UNROLL 4
 
@@ -298,14 +318,24 @@ pdf_grid_kernel(PdfGridArgs a)
                             again);
         if (redo) sum = capped_sum;
     }
-    if (valid) a.out[a.order ? (int64_t)a.order[i] : i] = (float)sum;
+    if (valid) {
+        const int64_t at = a.order ? (int64_t)a.order[i] : i;
+        const float v = (float)sum;
+        a.out[at] = v;
+        if (a.out_norm) {
+            // Pointcloud.py:105-109: the estimate divided by the cloud's point count, both as fp32
+            const long long cells = (long long)nc0 * nc1 * nc2;
+            const int count = usable ? pdf_grid_cloud_count(a, key / cells, cells) : 1;
+            a.out_norm[at] = __fdiv_rn(v, (float)count);
+        }
+    }
 }
 
 extern "C" int pccnn_compute_pdf_grid(int manifold_dims, const float *bandwidth, const float *pts_sorted,
                                       const int64_t *sorted_keys, int64_t n, const int32_t *sample_order,
                                       const int32_t *grid_ds, int64_t num_pillars, const int32_t *cell_table,
                                       int64_t total_cells, const int32_t *num_cells, const float *radii, int d,
-                                      int max_neighbors, float *pdf_out, void *stream)
+                                      int max_neighbors, float *pdf_out, float *pdf_norm_out, void *stream)
 {
     PCCNN_REQUIRE(d == 3, PCCNN_ERR_UNSUPPORTED, "pccnn_compute_pdf_grid: d=%d is not supported (3 only; use "
                   "pccnn_find_neighbors_* and pccnn_compute_pdf)", d);
@@ -323,7 +353,7 @@ extern "C" int pccnn_compute_pdf_grid(int manifold_dims, const float *bandwidth,
     a.grid.num_pillars = num_pillars; a.grid.pt_keys = sorted_keys; a.grid.n = n;
     a.num_cells = num_cells; a.radii = radii; a.bandwidth = bandwidth;
     a.norm_const = 1.0 / pow(2.0 * 3.1415, (double)(float)manifold_dims / 2.0);
-    a.max_neighbors = max_neighbors; a.out = pdf_out; a.n = n;
+    a.max_neighbors = max_neighbors; a.out = pdf_out; a.out_norm = pdf_norm_out; a.n = n;
     hipStream_t s = (hipStream_t)stream;
     {
         PccnnTimed timed(PCCNN_T_PDF, s);

@@ -67,9 +67,11 @@ class Pointcloud(object):
         elif self.pts_.shape[1] == 3:
             # no gradient wanted, three dimensions: the sum straight from the grid, without a pair list
             with torch.no_grad():
-                self.pts_unnorm_pdf_ = pccnn_lib_ops.compute_pdf_grid(
+                self.pts_unnorm_pdf_, self.pts_pdf_ = pccnn_lib_ops.compute_pdf_grid(
                     self.dim_manifold_, bandwidth, grid.sorted_pts_, grid.sorted_cell_ids_, grid.sorted_ids_i32_,
-                    grid.grid_ds_, grid.num_cells_, grid.cell_size_, 300, cell_table=grid.cell_table_)
+                    grid.grid_ds_, grid.num_cells_, grid.cell_size_, 300, cell_table=grid.cell_table_,
+                    with_normalized=True)
+            return
         else:
             # no gradient wanted: keep the pair list in sorted-index space (no remap) and gather the
             # neighbor coordinates from the sorted copy of the points, where they are contiguous

@@ -295,12 +295,13 @@ def compute_pdf_sorted(manifold_dims, bandwidth, pts_sorted, samples, neigh_sort
 
 
 def compute_pdf_grid(manifold_dims, bandwidth, sorted_pts, sorted_keys, sample_order, grid_ds, grid_size, radii,
-                     max_neighbors=0, cell_table=None):
+                     max_neighbors=0, cell_table=None, with_normalized=False):
     """The density of every point straight from the grid (no counterpart in the reference's module; it is what
     pccnn_lib/pc/Pointcloud.py:81-109 computes with find_neighbors + compute_pdf): sorted points f32[N,3], sorted
     keys i64[N], sample_order i32[N] (original index of sorted point i; None = the points already are in key
     order), pillar table, grid_size i32[3], radii f32[3] (the search radii = cell size) -> f32[N] in the original
-    order, the same terms in the same order as compute_pdf on the (capped) neighbor list."""
+    order, the same terms in the same order as compute_pdf on the (capped) neighbor list.  With
+    ``with_normalized`` the result is the pair (estimate, estimate / number of points of the point's cloud)."""
     name = "compute_pdf_grid"
     _chk(sorted_pts, name + ": pts", torch.float32, 2)
     dev = sorted_pts.device
@@ -326,11 +327,12 @@ def compute_pdf_grid(manifold_dims, bandwidth, sorted_pts, sorted_keys, sample_o
         _chk(cell_table, name + ": cell_table", torch.int32, 1, dev)
         total_cells = cell_table.shape[0] - 1
     out = torch.empty((n,), dtype=torch.float32, device=dev)
+    norm = torch.empty_like(out) if with_normalized else None
     num_pillars = grid_ds.shape[0] * grid_ds.shape[1] * grid_ds.shape[2]
     _lib.call("pccnn_compute_pdf_grid", int(manifold_dims), _ptr(bandwidth), _ptr(sorted_pts), _ptr(sorted_keys), n,
               _optr(sample_order), _ptr(grid_ds), num_pillars, _optr(cell_table), total_cells, _ptr(grid_size),
-              _ptr(radii), 3, max_neighbors, _ptr(out), _stream())
-    return out
+              _ptr(radii), 3, max_neighbors, _ptr(out), _optr(norm), _stream())
+    return (out, norm) if with_normalized else out
 
 
 def compute_pdf_grads(manifold_dims, bandwidth, pts, neigh, ends, in_grads):

@@ -95,11 +95,14 @@ def test_pdf_from_the_grid_equals_the_list_route(ops, models, cap):
                                             sample_order=grid.sorted_ids_i32_, cell_table=grid.cell_table_,
                                             samples_presorted=True)
         want = ops.compute_pdf_sorted(3, bandwidth, grid.sorted_pts_, pc.pts_, neigh, ends)
+        per_cloud = pc.get_num_points_per_batch().to(torch.float32)[pc.batch_ids_.to(torch.int64)]
         for table in (grid.cell_table_, None):
-            got = ops.compute_pdf_grid(3, bandwidth, grid.sorted_pts_, grid.sorted_cell_ids_, grid.sorted_ids_i32_,
-                                       grid.grid_ds_, grid.num_cells_, grid.cell_size_, cap, cell_table=table)
+            got, normed = ops.compute_pdf_grid(3, bandwidth, grid.sorted_pts_, grid.sorted_cell_ids_,
+                                               grid.sorted_ids_i32_, grid.grid_ds_, grid.num_cells_, grid.cell_size_,
+                                               cap, cell_table=table, with_normalized=True)
             torch.cuda.synchronize()
             assert np.allclose(got.cpu().numpy(), want.cpu().numpy(), rtol=3e-7, atol=0)
+            assert torch.equal(normed, got / per_cloud)        # the cloud's point count, found from the sorted keys
         if cap == 7:
             counts = np.diff(np.concatenate([[0], ends.cpu().numpy()]))
             assert counts.max() == 7                          # the cap is reached, the subset rule is exercised
