@@ -416,3 +416,31 @@ def test_layer_uses_mirror_for_point_gradients(oracle):
                               np.full(3, 0.1, np.float32), layer.kernel_pts_.cpu().numpy(), float(layer.sigma_.item()),
                               layer.conv_weights_.detach().cpu().numpy(), g)
     assert relerr(tp.grad.cpu().numpy(), exp[3] + exp[4]) < GRAD_TOL
+
+
+def test_ops_run_on_torch_current_stream(ops, models):
+    # the native calls take torch's current stream: inside a stream context that is the side stream, and inputs
+    # produced there by a slow producer are consumed in order without any device-wide synchronisation
+    import pccnn_lib_amd as lib
+    pts, ids = _cloud(models, 2, 1000)
+    pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+    radii = torch.full((3,), 0.1, device=DEV)
+    rng = np.random.default_rng(12)
+    feats = t(rng.normal(size=(pts.shape[0], 16)).astype(np.float32))
+    kpts = t(rng.normal(0, 0.5, (15, 3)).astype(np.float32))
+    w = t(rng.normal(0, 0.2, (15 * 16, 8)).astype(np.float32))
+    nbh = lib.pc.layers.conv_base.build_neighborhood(pc, pc, radii, 0)
+    want = ops.kp_conv(pc.pts_, feats, pc.pts_, nbh.neighbors_, nbh.start_ids_, radii, kpts, 0.3, w)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    assert (ops._stream().value or 0) == torch.cuda.current_stream().cuda_stream
+    with torch.cuda.stream(side):
+        assert (ops._stream().value or 0) == side.cuda_stream
+        big = torch.randn((6144, 6144), device=DEV)
+        feats_side = feats + (big @ big).sum() * 0.0          # ready only after a few milliseconds of side-stream work
+        nbh_side = lib.pc.layers.conv_base.build_neighborhood(pc, pc, radii, 0)
+        got = ops.kp_conv(pc.pts_, feats_side, pc.pts_, nbh_side.neighbors_, nbh_side.start_ids_, radii, kpts, 0.3, w)
+    side.synchronize()
+    assert torch.equal(nbh_side.neighbors_, nbh.neighbors_)
+    assert torch.equal(got, want)
+    torch.cuda.synchronize()
