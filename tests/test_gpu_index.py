@@ -267,3 +267,18 @@ def test_pair_count_beyond_32_bits_is_an_error(ops):
     pc = lib.pc.Pointcloud(pts, torch.zeros(n, dtype=torch.int32, device=DEV))
     with pytest.raises(RuntimeError, match="pairs"):
         lib.pc.layers.conv_base.build_neighborhood(pc, pc, torch.full((3,), 1.0, device=DEV), 0)
+
+
+def test_grid_ops_on_an_empty_cloud(ops):
+    # no points: the grid-based selection and density return empty results without launching anything
+    pts, ids = synthetic.primitives(1, 1, 256)
+    g = gpu_neighborhood(ops, pts, ids, pts, ids, 0.1, 1)["dev"]
+    none_pts = torch.empty((0, 3), device=DEV)
+    none_keys = torch.empty((0,), dtype=torch.int64, device=DEV)
+    sel = ops.poisson_disk_sampling_grid(none_pts, none_keys, g["ds"], g["nc"], g["radii"])
+    assert tuple(sel.shape) == (0, 1) and sel.dtype == torch.int64
+    pdf, normed = ops.compute_pdf_grid(3, g["radii"] * 0.25, none_pts, none_keys, None, g["ds"], g["nc"], g["radii"], 300,
+                                       with_normalized=True)
+    assert tuple(pdf.shape) == (0,) and tuple(normed.shape) == (0,)
+    with pytest.raises(RuntimeError):
+        ops.compute_pdf_grid(3, g["radii"][:2].contiguous(), g["spts"], g["skeys"], None, g["ds"], g["nc"], g["radii"])
