@@ -86,9 +86,9 @@ __device__ __forceinline__ void tile_store(float (*lds)[GT_LD], const float4 (&r
     }
 }
 
-// The k loop of one workgroup tile.  Global loads run two tiles ahead of the MFMAs (registers, then the free
-// LDS buffer); inside a tile the LDS fragments of sub-step ks+1 are read before the MFMAs of sub-step ks are
-// issued, so the matrix pipe never waits on an LDS round trip.
+// The k loop of one workgroup tile.  Global loads run two or three tiles ahead of the MFMAs (one or two register
+// sets, then the free LDS buffer); inside a tile the LDS fragments of sub-step ks+1 are read before the MFMAs of
+// sub-step ks are issued, so the matrix pipe never waits on an LDS round trip.
 template <bool AT, bool BT, bool FAST, int BM>
 __device__ __forceinline__ void gemm_tile_loop(const GemmArgs &g, const float *__restrict__ a,
                                                const float *__restrict__ b, int64_t bm, int64_t bn, int64_t k_begin,
@@ -101,26 +101,42 @@ __device__ __forceinline__ void gemm_tile_loop(const GemmArgs &g, const float *_
     const int wave = threadIdx.x >> 6;
     const int wm = wave / WN, wn = wave % WN;
     const int frag_k = lane >> 5, frag_c = lane & 31;
-    float4 ra[BM / 64 * (GT_K / 16)], rb[2 * (GT_K / 16)];
+    constexpr int NA = BM / 64 * (GT_K / 16), NB = 2 * (GT_K / 16);
+    // 64-row tiles on the fast path travel in two register sets (tile j in set j & 1), so every global load has
+    // two whole steps of MFMAs to arrive (3 - 4 % on the products of 65 536 x 1024 x 128).  The 128-row tiles keep
+    // one set (AHEAD = 2): with two they pass 128 registers, which halves the waves per SIMD and costs 9 %; so does
+    // the bounds-checked path of edge tiles.
+    constexpr bool DEEP = FAST && BM == 64;
+    constexpr int AHEAD = DEEP ? 3 : 2;
+    float4 ra0[NA], rb0[NB], ra1[DEEP ? NA : 1], rb1[DEEP ? NB : 1];
     const int64_t nk = (k_end - k_begin + GT_K - 1) / GT_K;
     // A stored [rows, inner] (AT = false) has the reduction index contiguous; B stored
     // [inner, cols] (BT = false) has the column index contiguous.
     if (nk > 0) {
-        tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k_begin, k_end, ra);
-        tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k_begin, k_end, rb);
-        tile_store<!AT, BM>(As[0], ra);
-        tile_store<BT, GT_N>(Bs[0], rb);
+        tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k_begin, k_end, ra0);
+        tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k_begin, k_end, rb0);
+        tile_store<!AT, BM>(As[0], ra0);
+        tile_store<BT, GT_N>(Bs[0], rb0);
     }
-    if (nk > 1) {
-        tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k_begin + GT_K, k_end, ra);
-        tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k_begin + GT_K, k_end, rb);
+    if constexpr (DEEP) {
+        if (nk > 1) {
+            tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k_begin + GT_K, k_end, ra1);
+            tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k_begin + GT_K, k_end, rb1);
+        }
+        if (nk > 2) {
+            tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k_begin + 2 * GT_K, k_end, ra0);
+            tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k_begin + 2 * GT_K, k_end, rb0);
+        }
+    } else if (nk > 1) {
+        tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k_begin + GT_K, k_end, ra0);
+        tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k_begin + GT_K, k_end, rb0);
     }
     __syncthreads();
-    for (int64_t kt = 0; kt < nk; ++kt) {
+    // One step: the MFMAs of tile kt from LDS buffer kt & 1.  Behind the first of them tile kt+1, which sits in
+    // the register set (ra, rb), is parked in the other LDS buffer (free since the barrier that ended step kt-1)
+    // and the same registers take the loads of tile kt+AHEAD.
+    auto step = [&](int64_t kt, float4 (&ra)[NA], float4 (&rb)[NB]) {
         const int buf = (int)(kt & 1);
-        // Tile kt+1 sits in registers since the previous step: it is parked in the other LDS buffer (free
-        // since the barrier that ended step kt-1) and the registers are reused for the loads of tile kt+2,
-        // which get a whole step of MFMAs to arrive.
         float fa[2][2], fb[2][TN];
 #pragma unroll
         for (int i = 0; i < 2; ++i) fa[0][i] = As[buf][frag_k][wm * 64 + i * 32 + frag_c];
@@ -147,8 +163,8 @@ __device__ __forceinline__ void gemm_tile_loop(const GemmArgs &g, const float *_
                     tile_store<!AT, BM>(As[buf ^ 1], ra);
                     tile_store<BT, GT_N>(Bs[buf ^ 1], rb);
                 }
-                if (kt + 2 < nk) {
-                    const int64_t k0 = k_begin + (kt + 2) * GT_K;
+                if (kt + AHEAD < nk) {
+                    const int64_t k0 = k_begin + (kt + AHEAD) * GT_K;
                     tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k0, k_end, ra);
                     tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k0, k_end, rb);
                 }
@@ -159,6 +175,14 @@ __device__ __forceinline__ void gemm_tile_loop(const GemmArgs &g, const float *_
             __builtin_amdgcn_sched_group_barrier(0x008, 2 * TN, 0);
         }
         __syncthreads();
+    };
+    if constexpr (DEEP) {
+        for (int64_t kt = 0; kt < nk; kt += 2) {
+            step(kt, ra1, rb1);                                     // tile kt+1 (odd) travels in set 1
+            if (kt + 1 < nk) step(kt + 1, ra0, rb0);                // tile kt+2 (even) in set 0
+        }
+    } else {
+        for (int64_t kt = 0; kt < nk; ++kt) step(kt, ra0, rb0);
     }
 }
 
