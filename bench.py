@@ -208,8 +208,9 @@ def main():
         return torch.autograd.grad(out, leaves, out_grads)
 
     def pc_fresh():
-        p = lib.pc.Pointcloud.__new__(lib.pc.Pointcloud)         # same tensors, no cached grid
+        p = lib.pc.Pointcloud.__new__(lib.pc.Pointcloud)         # same tensors, nothing cached: a cold build
         p.__dict__.update(pc.__dict__)
+        p.__dict__.pop("aabb_cache_", None)
         return p
 
     def neighbor_step():
@@ -297,6 +298,7 @@ def main():
         def scene_step():
             p = lib.pc.Pointcloud.__new__(lib.pc.Pointcloud)
             p.__dict__.update(spc.__dict__)
+            p.__dict__.pop("aabb_cache_", None)             # a cold build: the box is computed again
             return lib.pc.layers.conv_base.build_neighborhood(p, p, sradii, 0)
 
         snb = scene_step()
@@ -320,6 +322,7 @@ def main():
         def scene_pdf_step():
             p = lib.pc.Pointcloud.__new__(lib.pc.Pointcloud)
             p.__dict__.update(spc.__dict__)
+            p.__dict__.pop("aabb_cache_", None)             # a cold build: the box is computed again
             p.compute_pdf(sbw)
             return p
 

@@ -1,13 +1,26 @@
+import weakref
+
 from .. import pccnn_lib_ops
 
 
 class BoundingBox(object):
     """Per-cloud axis-aligned box padded by 1e-6 (pccnn_lib/pc/BoundingBox.py:10-18):
-    ``min_`` and ``max_`` are float32 [B, D].  One native reduction replaces torch_scatter."""
+    ``min_`` and ``max_`` are float32 [B, D].  One native reduction replaces torch_scatter.
+
+    A hierarchy level asks for the box of the same cloud several times (one grid each for pooling, density and the
+    convolution's neighborhood), so the result is remembered on the cloud for as long as its coordinate and batch
+    tensors are the same objects and have not been written to (torch's version counters)."""
 
     def __init__(self, p_point_cloud):
-        self.min_, self.max_ = pccnn_lib_ops.bounding_box(
-            p_point_cloud.pts_.detach(), p_point_cloud.batch_ids_, p_point_cloud.batch_size_host())
+        pts, ids = p_point_cloud.pts_, p_point_cloud.batch_ids_
+        cached = getattr(p_point_cloud, "aabb_cache_", None)
+        if cached is not None and cached[0]() is pts and cached[1] == pts._version and cached[2]() is ids \
+                and cached[3] == ids._version:
+            self.min_, self.max_ = cached[4], cached[5]
+            return
+        self.min_, self.max_ = pccnn_lib_ops.bounding_box(pts.detach(), ids, p_point_cloud.batch_size_host())
+        # weak references: the entry neither keeps replaced tensors alive nor matches a new tensor at a reused address
+        p_point_cloud.aabb_cache_ = (weakref.ref(pts), pts._version, weakref.ref(ids), ids._version, self.min_, self.max_)
 
     def __repr__(self):
         return "### Min:\n{}\n### Max:\n{}".format(self.min_, self.max_)

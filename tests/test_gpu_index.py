@@ -282,3 +282,19 @@ def test_grid_ops_on_an_empty_cloud(ops):
     assert tuple(pdf.shape) == (0,) and tuple(normed.shape) == (0,)
     with pytest.raises(RuntimeError):
         ops.compute_pdf_grid(3, g["radii"][:2].contiguous(), g["spts"], g["skeys"], None, g["ds"], g["nc"], g["radii"])
+
+
+def test_bounding_box_is_remembered_until_the_cloud_changes(ops):
+    import pccnn_lib_amd as lib
+    pts, ids = synthetic.primitives(5, 2, 500)
+    pc = lib.pc.Pointcloud(t(pts), t(ids))
+    first = lib.pc.BoundingBox(pc)
+    again = lib.pc.BoundingBox(pc)
+    assert again.min_ is first.min_ and again.max_ is first.max_          # same cloud, untouched: not recomputed
+    pc.pts_.mul_(2.0)                                                     # written in place: computed again
+    scaled = lib.pc.BoundingBox(pc)
+    assert scaled.min_ is not first.min_
+    assert torch.allclose(scaled.max_ - scaled.min_, 2.0 * (first.max_ - first.min_), atol=1e-5)
+    pc.pts_ = pc.pts_ + 1.0                                               # replaced: computed again
+    moved = lib.pc.BoundingBox(pc)
+    assert torch.allclose(moved.min_, scaled.min_ + 1.0, atol=1e-5)
