@@ -1,0 +1,35 @@
+"""Small per-dimension constants (radii, bandwidths, cell sizes) as device tensors.
+
+The reference turns such an argument into a tensor on every call (``torch.as_tensor(p_radius, device=...)``,
+pccnn_lib/pc/layers/IConvLayer.py:129-131, pc/Pointcloud.py:89-91, pc/Grid.py:23).  From host memory that is a
+synchronous copy: the host waits until the device has finished everything queued before, which for a small level of
+a hierarchy costs more than the level's kernels.  A value that was seen before is therefore served from a table of
+the tensors already on the device; tensors that are on the device already pass through untouched."""
+import numbers
+
+import numpy as np
+import torch
+
+_table = {}
+_MAX_ENTRIES = 256
+
+
+def device_vector(value, num_dims, device):
+    """``value`` (number, sequence, numpy array or tensor) as a float32 tensor of ``num_dims`` entries on ``device``;
+    a scalar is repeated.  Treat the result as read-only: equal values share one tensor."""
+    if torch.is_tensor(value):
+        out = value.to(device=device, dtype=torch.float32)
+        return out.repeat(num_dims) if out.dim() == 0 else out
+    if isinstance(value, numbers.Real):
+        flat = (float(value),) * num_dims
+    else:
+        arr = np.asarray(value, dtype=np.float32).reshape(-1)
+        flat = tuple(float(v) for v in arr) if arr.size > 1 else (float(arr[0]),) * num_dims
+    key = (flat, str(device))
+    out = _table.get(key)
+    if out is None:
+        if len(_table) >= _MAX_ENTRIES:
+            _table.clear()
+        out = torch.tensor(flat, dtype=torch.float32, device=device)
+        _table[key] = out
+    return out

@@ -1,6 +1,7 @@
 import torch
 
 from .. import pccnn_lib_ops
+from ._consts import device_vector
 
 
 class Grid(object):
@@ -15,9 +16,7 @@ class Grid(object):
     def __init__(self, p_point_cloud, p_bounding_box, p_cell_size):
         self.pointcloud_ = p_point_cloud
         self.bounding_box_ = p_bounding_box
-        self.cell_size_ = torch.as_tensor(p_cell_size, dtype=torch.float32, device=p_point_cloud.pts_.device)
-        if self.cell_size_.dim() == 0:
-            self.cell_size_ = self.cell_size_.repeat(p_point_cloud.pts_.shape[1])
+        self.cell_size_ = device_vector(p_cell_size, p_point_cloud.pts_.shape[1], p_point_cloud.pts_.device)
         with torch.no_grad():
             # Grid.py:26-28: fp32 division, truncation, + 1, maximum over the clouds.
             self.num_cells_ = pccnn_lib_ops.num_cells(self.bounding_box_.min_, self.bounding_box_.max_,

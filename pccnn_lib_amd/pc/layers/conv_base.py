@@ -1,5 +1,7 @@
 import torch
 
+from .._consts import device_vector
+
 
 def build_neighborhood(p_pc_in, p_pc_out, p_radius, p_max_neighs):
     """Box -> grid -> keys/sort -> pillar table -> neighbor search, as every layer of the reference does when no
@@ -53,9 +55,7 @@ class IConvLayer(torch.nn.Module):
         return build_neighborhood(p_pc_in, p_pc_out, p_radius, p_max_neighs)
 
     def forward(self, p_pc_in, p_pc_out, p_in_features, p_radius, p_neighborhood=None, p_max_neighs=0):
-        radius = torch.as_tensor(p_radius, dtype=torch.float32, device=p_pc_in.pts_.device)
-        if radius.dim() == 0:
-            radius = radius.repeat(self.num_dims_)
+        radius = device_vector(p_radius, self.num_dims_, p_pc_in.pts_.device)
         neighborhood = p_neighborhood
         if neighborhood is None:
             neighborhood = self.__create_neighborhood__(p_pc_in, p_pc_out, radius, p_max_neighs)

@@ -2,6 +2,7 @@ import torch
 
 from .. import pccnn_lib_ops
 from ..op_wrappers import ComputePDF
+from ._consts import device_vector
 
 
 class Pointcloud(object):
@@ -52,9 +53,7 @@ class Pointcloud(object):
         from .bounding_box import BoundingBox
         from .grid import Grid
         from .neighborhood import Neighborhood
-        bandwidth = torch.as_tensor(p_badnwidth, dtype=torch.float32, device=self.pts_.device)
-        if bandwidth.dim() == 0:
-            bandwidth = bandwidth.repeat(self.pts_.shape[1])
+        bandwidth = device_vector(p_badnwidth, self.pts_.shape[1], self.pts_.device)
         radii = bandwidth * 4.0
         aabb = BoundingBox(self)
         grid = Grid(self, aabb, radii)
