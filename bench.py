@@ -17,6 +17,7 @@ density pipeline are timed as well and reported as extra keys of the same JSON l
                 divided by its mean launch duration, taken live with HIP events on the launch stream;
   roofline_neighbors   the same for the neighbor fill kernel against HBM bandwidth, measured on the
                 million-point room of config 4 (`scene` carries that leg's pairs / second);
+  roofline_projection_forward / _backward   the two projection kernels of the step against HBM bandwidth;
   cpu_baseline  the same step on the host cores: the vectorised torch form of the oracle on all threads over the whole
                 workload, and the scalar oracle (C + numpy, one thread) on two clouds beside it.
 
@@ -41,6 +42,8 @@ HBM_PEAK_GBPS = 8000.0            # MI355X HBM3E peak
 # of this command scaled by a copy kernel of known size (profiles/bench_mcconv_16x4096_hbm_traffic.md).  They
 # hold for the default workloads only (config 2; the scene leg at 1 000 000 points) and are reported as null otherwise.
 TRAFFIC_GEMM_BYTES = 312.7e6            # mean of the three contraction launches of a step (algorithmic: 313.5e6)
+TRAFFIC_PROJ_FWD_BYTES = 411.6e6         # conv_proj_fwd_kernel<MLP, 16, f32> (algorithmic: 294.7e6)
+TRAFFIC_PROJ_BWD_BYTES = 679.3e6         # conv_proj_bwd_kernel<MLP, 16, dF, dBasis> (algorithmic: 385.3e6)
 TRAFFIC_NB_FILL_BYTES_CONFIG2 = 17.1e6  # launches of 65 536 samples (algorithmic: 10.3e6)
 TRAFFIC_NB_FILL_BYTES_SCENE = 610.2e6   # launches of 1 000 000 samples (algorithmic: 194.6e6)
 
@@ -264,6 +267,25 @@ def main():
                 "traffic": TRAFFIC_GEMM_BYTES, "flops_per_launch": gemm_flops, "avg_launch_ms": gemm_avg_ms,
                 "launches": gemm_n}
 
+    # ---- the two projection kernels against HBM bandwidth.  Algorithmic bytes, forward: pairs 8T + offsets 4M +
+    # coordinates 12(N + M) + features 4 N Cin + density 4N in, projection 4 M Cin K out.  Backward: the projection
+    # gradient 4 M Cin K, pairs, offsets, coordinates, features and density in; feature gradient 4 N Cin, basis
+    # gradient 4 T K and the per-pair point gradients 16 T out.
+    t_pairs = float(total_pairs)
+    geo_bytes = 8.0 * t_pairs + 4.0 * m + 12.0 * 2 * m + 4.0 * m * wl["c_in"] + 4.0 * m
+    proj_bytes = 4.0 * m * kdim
+    rooflines_proj = {}
+    for key, name, alg, traffic in (
+            ("proj_fwd", "conv_proj_fwd_kernel", geo_bytes + proj_bytes, TRAFFIC_PROJ_FWD_BYTES),
+            ("proj_bwd", "conv_proj_bwd_kernel", geo_bytes + proj_bytes + 4.0 * m * wl["c_in"] +
+             4.0 * t_pairs * wl["hidden"] + 16.0 * t_pairs, TRAFFIC_PROJ_BWD_BYTES)):
+        k_n, k_ms = conv_kernels.get(key, (0, 0.0))
+        avg = k_ms / max(k_n, 1)
+        gbps = alg / (avg * 1e-3) / 1e9 if k_n else 0.0
+        rooflines_proj[key] = {"kernel": name, "bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                               "frac": gbps / HBM_PEAK_GBPS, "traffic": traffic, "bytes_per_launch": alg,
+                               "avg_launch_ms": avg, "launches": k_n}
+
     # the same three launches on the bf16 pipe (reported beside the fp32 figures; `value` is the fp32 step)
     bf_n, bf_total_ms = bf_kernels.get("gemm", (0, 0.0))
     bf_avg_ms = bf_total_ms / max(bf_n, 1)
@@ -358,7 +380,9 @@ def main():
         "density_ms": pdf_ms,
         "kernels_us": {leg: {k: round(1e3 * v[1] / v[0], 2) for k, v in ks.items()}
                        for leg, ks in (("conv", conv_kernels), ("neighborhood", nb_kernels), ("density", pdf_kernels))},
-        "bf16_contraction": bf16_leg, "scene": scene, "roofline": roofline, "roofline_neighbors": roofline_nb, "hbm_copy_ceiling_gbps": copy_gbps,
+        "bf16_contraction": bf16_leg, "scene": scene, "roofline": roofline, "roofline_neighbors": roofline_nb,
+        "roofline_projection_forward": rooflines_proj["proj_fwd"],
+        "roofline_projection_backward": rooflines_proj["proj_bwd"], "hbm_copy_ceiling_gbps": copy_gbps,
         "cpu_baseline": cpu,
     }
     print(json.dumps(result), flush=True)
