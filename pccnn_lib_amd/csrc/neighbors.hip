@@ -366,12 +366,20 @@ neighbors_group_kernel(NbArgs a)
     if (!FILL && valid && sub == 0) a.counts[s] = cnt;
 }
 
+#define NB_CHIP_LANES (256 * 32 * 64)       // lanes of one round of wavefronts at full occupancy
+
 // Lanes per sample: one when there are about as many samples as points, more when the samples are few.
 static int nb_group_size(int64_t n, int64_t m, int d)
 {
     if (d != 3 || m <= 0) return 1;
     if (n >= 16 * m) return 64;
     if (n >= 4 * m) return 16;
+    // about as many samples as points, but few of them: one sample per lane leaves the chip short of wavefronts
+    // (65 536 samples are 4 per CU), so lanes share a sample as long as the launch still fits the chip in one round
+    // of 32 wavefronts per CU (config 2: count 21 -> 17 us, fill 34 -> 23 us with 8 lanes; at 200 000 samples the
+    // one-lane walk is ahead again, 19 / 31 us against 30 / 37 us)
+    if (m * 8 <= NB_CHIP_LANES) return 8;
+    if (m * 4 <= NB_CHIP_LANES) return 4;
     return 1;
 }
 
@@ -604,6 +612,8 @@ extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t
         const unsigned blocks = (unsigned)pccnn_ceil_div(waves, NB_THREADS / 64);
         if (group == 64) neighbors_group_kernel<false, false, 64><<<blocks, NB_THREADS, 0, s>>>(a);
         else if (group == 16) neighbors_group_kernel<false, false, 16><<<blocks, NB_THREADS, 0, s>>>(a);
+        else if (group == 8) neighbors_group_kernel<false, false, 8><<<blocks, NB_THREADS, 0, s>>>(a);
+        else if (group == 4) neighbors_group_kernel<false, false, 4><<<blocks, NB_THREADS, 0, s>>>(a);
         else switch (d) {
         case 3: neighbors_kernel<false, false, NB_UNROLL_COUNT><<<blocks, NB_THREADS, 0, s>>>(a); break;
         case 2: neighbors_generic_kernel<false, false, 2><<<blocks, NB_THREADS, 0, s>>>(a); break;
@@ -658,6 +668,12 @@ extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t 
             } else if (group == 16) {
                 if (max_neighbors > 0) neighbors_group_kernel<true, true, 16><<<blocks, NB_THREADS, 0, s>>>(a);
                 else neighbors_group_kernel<true, false, 16><<<blocks, NB_THREADS, 0, s>>>(a);
+            } else if (group == 8) {
+                if (max_neighbors > 0) neighbors_group_kernel<true, true, 8><<<blocks, NB_THREADS, 0, s>>>(a);
+                else neighbors_group_kernel<true, false, 8><<<blocks, NB_THREADS, 0, s>>>(a);
+            } else if (group == 4) {
+                if (max_neighbors > 0) neighbors_group_kernel<true, true, 4><<<blocks, NB_THREADS, 0, s>>>(a);
+                else neighbors_group_kernel<true, false, 4><<<blocks, NB_THREADS, 0, s>>>(a);
             } else if (max_neighbors > 0) neighbors_kernel<true, true, NB_UNROLL_FILL><<<blocks, NB_THREADS, 0, s>>>(a);
             else neighbors_kernel<true, false, NB_UNROLL_FILL><<<blocks, NB_THREADS, 0, s>>>(a);
         } else {
