@@ -44,8 +44,8 @@ HBM_PEAK_GBPS = 8000.0            # MI355X HBM3E peak
 TRAFFIC_GEMM_BYTES = 312.7e6            # mean of the three contraction launches of a step (algorithmic: 313.5e6)
 TRAFFIC_PROJ_FWD_BYTES = 411.6e6         # conv_proj_fwd_kernel<MLP, 16, f32> (algorithmic: 294.7e6)
 TRAFFIC_PROJ_BWD_BYTES = 679.3e6         # conv_proj_bwd_kernel<MLP, 16, dF, dBasis> (algorithmic: 385.3e6)
-TRAFFIC_NB_FILL_BYTES_CONFIG2 = 17.1e6  # launches of 65 536 samples (algorithmic: 10.3e6)
-TRAFFIC_NB_FILL_BYTES_SCENE = 610.2e6   # launches of 1 000 000 samples (algorithmic: 194.6e6)
+TRAFFIC_NB_FILL_BYTES_CONFIG2 = 20.0e6  # launches of 65 536 samples (algorithmic: 10.3e6)
+TRAFFIC_NB_FILL_BYTES_SCENE = 610.5e6   # launches of 1 000 000 samples (algorithmic: 194.6e6)
 
 
 def log(*a):
@@ -303,7 +303,7 @@ def main():
     fill_n, fill_total_ms = nb_kernels.get("nb_fill", (0, 0.0))
     fill_avg_ms = fill_total_ms / max(fill_n, 1)
     fill_gbps = nb_bytes / (fill_avg_ms * 1e-3) / 1e9 if fill_n else 0.0
-    roofline_nb = {"kernel": "neighbors_kernel<fill>", "workload": "config 2", "bound": "hbm", "achieved": fill_gbps, "peak": HBM_PEAK_GBPS,
+    roofline_nb = {"kernel": "neighbors_group_kernel<fill, 8 lanes per sample>", "workload": "config 2", "bound": "hbm", "achieved": fill_gbps, "peak": HBM_PEAK_GBPS,
                    "unit": "GB/s", "frac": fill_gbps / HBM_PEAK_GBPS, "traffic": TRAFFIC_NB_FILL_BYTES_CONFIG2,
                    "bytes_per_launch": nb_bytes, "avg_launch_ms": fill_avg_ms, "launches": fill_n}
 
