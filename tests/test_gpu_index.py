@@ -298,3 +298,27 @@ def test_bounding_box_is_remembered_until_the_cloud_changes(ops):
     pc.pts_ = pc.pts_ + 1.0                                               # replaced: computed again
     moved = lib.pc.BoundingBox(pc)
     assert torch.allclose(moved.min_, scaled.min_ + 1.0, atol=1e-5)
+
+
+@pytest.mark.parametrize("num_pts", [40000, 200000])
+def test_capped_lists_are_the_ruled_subset_of_the_full_lists(ops, num_pts):
+    # With a cap, sample by sample, hit number r of raw (in walk order) is kept iff floor((r + 1) cap / raw) >
+    # floor(r cap / raw).  Checked against the uncapped search of the same grid, restated with numpy, at a size that
+    # runs 8 lanes per sample (40 000) and at one that runs the one-lane walk (200 000).
+    import pccnn_lib_amd as lib
+    cap = 6
+    pts = t(synthetic.room(8, num_pts))
+    pc = lib.pc.Pointcloud(pts, torch.zeros(num_pts, dtype=torch.int32, device=DEV))
+    radii = torch.full((3,), 0.12 if num_pts < 100000 else 0.06, device=DEV)
+    full = lib.pc.layers.conv_base.build_neighborhood(pc, pc, radii, 0)
+    capped = lib.pc.layers.conv_base.build_neighborhood(pc, pc, radii, cap)
+    f_neigh, f_ends = full.neighbors_.cpu().numpy(), full.start_ids_.cpu().numpy().astype(np.int64)
+    c_neigh, c_ends = capped.neighbors_.cpu().numpy(), capped.start_ids_.cpu().numpy().astype(np.int64)
+    raw = np.diff(f_ends, prepend=0)
+    assert raw.max() > 4 * cap                                     # the cap bites
+    assert np.array_equal(np.diff(c_ends, prepend=0), np.minimum(raw, cap))
+    starts = f_ends - raw
+    rank = np.arange(f_neigh.shape[0], dtype=np.int64) - np.repeat(starts, raw)
+    raw_of_pair = np.repeat(raw, raw)
+    keep = (raw_of_pair <= cap) | (((rank + 1) * cap) // raw_of_pair > (rank * cap) // raw_of_pair)
+    assert np.array_equal(c_neigh, f_neigh[keep])
