@@ -331,6 +331,134 @@ pdf_grid_kernel(PdfGridArgs a)
     }
 }
 
+// The same with G lanes per point, for clouds too small to fill the chip with one point per lane: the lanes of a
+// group stride over every pillar range together, one candidate per lane and step, a ballot over the group counts
+// and ranks the hits of the step (so the capped subset is the one of the one-lane walk), every lane sums its own
+// hits in double and the group's sums are added at the end.
+template <int G>
+__global__ void __launch_bounds__(256)
+pdf_grid_group_kernel(PdfGridArgs a)
+{
+    constexpr int GROUPS = 64 / G;
+    __shared__ int2 ranges[4][GROUPS][9];
+    const int lane = pccnn_lane();
+    const int wib = threadIdx.x >> 6;
+    const int grp = lane / G, sub = lane % G;
+    const int64_t wave = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 6;
+    if (wave * GROUPS >= a.n) return;                 // wave-uniform
+    const int64_t i = wave * GROUPS + grp;
+    const bool valid = i < a.n;
+    long long key = -1;
+    float sx = 0.f, sy = 0.f, sz = 0.f;
+    if (valid) {
+        key = a.keys[i];
+        sx = a.pts[i * 3 + 0];
+        sy = a.pts[i * 3 + 1];
+        sz = a.pts[i * 3 + 2];
+    }
+    const int nc0 = a.num_cells[0], nc1 = a.num_cells[1], nc2 = a.num_cells[2];
+    float ir[3], ib[3];
+    float prod = 1.0f;
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+        ir[c] = __fdiv_rn(1.0f, a.radii[c]);
+        ib[c] = __fdiv_rn(1.0f, a.bandwidth[c]);
+        prod = prod * ib[c];
+    }
+    const double scale = (double)prod * a.norm_const;
+    const bool usable = valid && key >= 0;
+    long long k = usable ? key : 0;
+    const int c2 = (int)(k % nc2); k /= nc2;
+    const int c1 = (int)(k % nc1);
+    const long long pil = k; k /= nc1;
+    const int c0 = (int)(k % nc0);
+    for (int o = sub; o < 9; o += G) {
+        int first = 0, len = 0;
+        if (usable) {
+            const int cmin = c2 > 0 ? c2 - 1 : 0, cmax = c2 + 1 < nc2 ? c2 + 1 : nc2 - 1;
+            const int dx = o / 3 - 1, dy = o % 3 - 1;
+            const int x = c0 + dx, y = c1 + dy;
+            if (x >= 0 && x < nc0 && y >= 0 && y < nc1)
+                grid_pillar_range(a.grid, pil + (long long)dx * nc1 + dy, nc2, cmin, cmax, first, len);
+        }
+        ranges[wib][grp][o] = make_int2(first, len);
+    }
+    // (a wavefront's own LDS writes are in order with its reads: no barrier between the lanes of a group)
+    const unsigned long long group_bits = (G == 64) ? ~0ull : (((1ull << (G & 63)) - 1ull) << (grp * G));
+    const unsigned long long below = group_bits & pccnn_lanemask_lt();
+
+    // walk(raw, cap): raw == 0 sums every hit, else only the capped subset; returns the hits of the point
+    auto walk = [&](bool go, long long raw, long long cap, double &sum) -> int {
+        int cnt = 0, r = 0, j0 = 0;
+        int2 cur = ranges[wib][grp][0];
+        bool active = go;
+        sum = 0.0;
+        while (__any(active)) {
+            bool hit = false;
+            float px = 0.f, py = 0.f, pz = 0.f;
+            if (active) {
+                const int j = j0 + sub;
+                if (j < cur.y) {
+                    const int64_t idx = cur.x + j;
+                    px = a.pts[idx * 3 + 0];
+                    py = a.pts[idx * 3 + 1];
+                    pz = a.pts[idx * 3 + 2];
+                    const float vx = (sx - px) * ir[0];
+                    const float vy = (sy - py) * ir[1];
+                    const float vz = (sz - pz) * ir[2];
+                    const float acc = ((0.0f + vx * vx) + vy * vy) + vz * vz;
+                    hit = acc < 1.0f;
+                }
+            }
+            const unsigned long long hits = __ballot(hit);
+            if (active) {
+                if (hit) {
+                    bool take = true;
+                    if (raw > 0) {
+                        const long long rank = cnt + __popcll(hits & below);
+                        take = (rank + 1) * cap / raw > rank * cap / raw;
+                    }
+                    if (take) {
+                        const float d0 = (px - sx) * ib[0];
+                        const float d1 = (py - sy) * ib[1];
+                        const float d2 = (pz - sz) * ib[2];
+                        const float dot = ((0.0f + d0 * d0) + d1 * d1) + d2 * d2;
+                        sum += scale * (double)expf(dot * (-0.5f));
+                    }
+                }
+                cnt += __popcll(hits & group_bits);
+                j0 += G;
+                if (j0 >= cur.y) {
+                    j0 = 0;
+                    if (++r < 9) cur = ranges[wib][grp][r];
+                    else active = false;
+                }
+            }
+        }
+        return cnt;
+    };
+    double sum;
+    const int cnt = walk(usable, 0, 0, sum);
+    const bool redo = a.max_neighbors > 0 && cnt > a.max_neighbors;
+    if (__any(redo)) {
+        double capped_sum;
+        (void)walk(redo, cnt, a.max_neighbors, capped_sum);
+        if (redo) sum = capped_sum;
+    }
+#pragma unroll
+    for (int o = G / 2; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+    if (valid && sub == 0) {
+        const int64_t at = a.order ? (int64_t)a.order[i] : i;
+        const float v = (float)sum;
+        a.out[at] = v;
+        if (a.out_norm) {
+            const long long cells = (long long)nc0 * nc1 * nc2;
+            const int count = usable ? pdf_grid_cloud_count(a, key / cells, cells) : 1;
+            a.out_norm[at] = __fdiv_rn(v, (float)count);
+        }
+    }
+}
+
 extern "C" int pccnn_compute_pdf_grid(int manifold_dims, const float *bandwidth, const float *pts_sorted,
                                       const int64_t *sorted_keys, int64_t n, const int32_t *sample_order,
                                       const int32_t *grid_ds, int64_t num_pillars, const int32_t *cell_table,
@@ -357,7 +485,12 @@ extern "C" int pccnn_compute_pdf_grid(int manifold_dims, const float *bandwidth,
     hipStream_t s = (hipStream_t)stream;
     {
         PccnnTimed timed(PCCNN_T_PDF, s);
-        pdf_grid_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(a);
+        // one point per lane, unless that leaves the chip short of wavefronts: then 8 or 4 lanes per point, as long
+        // as the launch still is one round of wavefronts (256 CUs x 32 x 64 lanes)
+        const int64_t chip_lanes = 256 * 32 * 64;
+        if (n * 8 <= chip_lanes) pdf_grid_group_kernel<8><<<(unsigned)pccnn_ceil_div(n * 8, 256), 256, 0, s>>>(a);
+        else if (n * 4 <= chip_lanes) pdf_grid_group_kernel<4><<<(unsigned)pccnn_ceil_div(n * 4, 256), 256, 0, s>>>(a);
+        else pdf_grid_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(a);
     }
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;

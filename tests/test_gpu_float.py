@@ -84,7 +84,9 @@ def test_pdf_from_the_grid_equals_the_list_route(ops, models, cap):
     import pccnn_lib_amd as lib
     pts, ids = _cloud(models, 3, 1000)
     rooms = (synthetic.room(11, 20000) / 10.0).astype(np.float32)
-    for cloud, cloud_ids, bw in ((pts, ids, 0.05), (rooms, np.zeros(rooms.shape[0], np.int32), 0.004)):
+    large = synthetic.room(12, 150000)                    # one point per lane; the smaller clouds run 8 lanes per point
+    for cloud, cloud_ids, bw in ((pts, ids, 0.05), (rooms, np.zeros(rooms.shape[0], np.int32), 0.004),
+                                 (large, np.zeros(large.shape[0], np.int32), 0.012)):
         pc = lib.pc.Pointcloud(cloud, cloud_ids, device=DEV)
         bandwidth = torch.full((3,), bw, device=DEV)
         grid = lib.pc.Grid(pc, lib.pc.BoundingBox(pc), bandwidth * 4.0)
