@@ -115,6 +115,16 @@ size_t pccnn_find_neighbors_workspace_bytes(int64_t n, int64_t m);
  * pillar table and a binary search are used.  Same results either way. */
 int pccnn_build_cell_table(const int64_t *sorted_keys, int64_t n, int64_t total_cells, int32_t *cell_table_out,
                            void *stream);
+/* Keys, sort, pillar table and (cell_table_out non-NULL) cell table of one grid in one call: the work of
+ * Grid.compute_cell_ids + Grid.build_ds (pccnn_lib/pc/Grid.py:40-72).  Arguments as for pccnn_compute_keys,
+ * pccnn_sort_keys (key_bits, workspace of pccnn_grid_build_workspace_bytes(n) bytes), pccnn_build_grid_ds
+ * (num_pillars) and pccnn_build_cell_table (total_cells); keys_out i64[n] are the unsorted keys. */
+size_t pccnn_grid_build_workspace_bytes(int64_t n);
+int pccnn_grid_build(const float *pts, const int32_t *batch_ids, const float *aabb_min, const int32_t *num_cells,
+                     const float *cell_size, int64_t n, int d, int key_bits, int64_t num_pillars,
+                     int64_t total_cells, int64_t *keys_out, int64_t *sorted_keys_out, int32_t *perm_out,
+                     float *sorted_pts_out, int32_t *grid_ds_out, int32_t *cell_table_out, void *workspace,
+                     size_t workspace_bytes, void *stream);
 int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t *pt_keys_sorted, int64_t n,
                                const float *samples, const int64_t *sample_keys, int64_t m,
                                const int32_t *sample_order, int samples_presorted,

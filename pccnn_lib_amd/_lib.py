@@ -42,6 +42,8 @@ SIGNATURES = {
     "pccnn_find_neighbors_count": (I32, [P, P, I64, P, P, I64, P, I32, P, I64, P, I64, P, P, I32, I32, P, P, SZ, P]),
     "pccnn_find_neighbors_fill": (I32, [P, P, I64, P, P, I64, P, I32, P, I64, P, I64, P, P, I32, I32, P, P, I64, P, P,
                                         SZ, P]),
+    "pccnn_grid_build_workspace_bytes": (SZ, [I64]),
+    "pccnn_grid_build": (I32, [P, P, P, P, P, I64, I32, I32, I64, I64, P, P, P, P, P, P, P, SZ, P]),
     "pccnn_compute_pdf": (I32, [I32, P, P, I64, I32, P, I64, P, P, P]),
     "pccnn_compute_pdf_sorted": (I32, [I32, P, P, P, I64, I32, P, I64, P, P, P]),
     "pccnn_compute_pdf_grads": (I32, [I32, P, P, I64, I32, P, I64, P, P, P, P]),

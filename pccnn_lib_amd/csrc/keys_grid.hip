@@ -292,3 +292,26 @@ extern "C" int pccnn_build_grid_ds(const int64_t *sorted_keys, int64_t n, const 
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
 }
+
+// ------------------------------------------------------------------- the four steps of a grid in one call
+// Keys, stable sort (with the gather of the coordinates), pillar table and, when asked for, the per-cell start
+// table: what Grid.compute_cell_ids + Grid.build_ds of the reference do (pccnn_lib/pc/Grid.py:40-72), as one entry
+// point, so that a host layer pays one call instead of four.  The launches are those of the four entry points.
+extern "C" size_t pccnn_grid_build_workspace_bytes(int64_t n) { return pccnn_sort_keys_workspace_bytes(n); }
+
+extern "C" int pccnn_grid_build(const float *pts, const int32_t *batch_ids, const float *aabb_min,
+                                const int32_t *num_cells, const float *cell_size, int64_t n, int d, int key_bits,
+                                int64_t num_pillars, int64_t total_cells, int64_t *keys_out, int64_t *sorted_keys_out,
+                                int32_t *perm_out, float *sorted_pts_out, int32_t *grid_ds_out,
+                                int32_t *cell_table_out, void *workspace, size_t workspace_bytes, void *stream)
+{
+    int rc = pccnn_compute_keys(pts, batch_ids, aabb_min, num_cells, cell_size, n, d, keys_out, stream);
+    if (rc != PCCNN_OK) return rc;
+    rc = pccnn_sort_keys(keys_out, n, key_bits, sorted_keys_out, perm_out, pts, d, sorted_pts_out, workspace,
+                         workspace_bytes, stream);
+    if (rc != PCCNN_OK) return rc;
+    rc = pccnn_build_grid_ds(sorted_keys_out, n, num_cells, d, num_pillars, grid_ds_out, stream);
+    if (rc != PCCNN_OK || cell_table_out == nullptr) return rc;
+    return pccnn_build_cell_table(sorted_keys_out, n, total_cells, cell_table_out, stream);
+}
+

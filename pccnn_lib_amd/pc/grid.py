@@ -46,13 +46,22 @@ class Grid(object):
         return pccnn_lib_ops.key_bits_for(self.num_cells_host(), self.pointcloud_.batch_size_host())
 
     def compute_cell_ids(self):
+        """Keys and their stable order (Grid.py:40-53).  The native call that computes them also builds the pillar
+        table (and the cell table of small grids), which ``build_ds`` then finds in place."""
         if self.cell_ids_ is None:
             with torch.no_grad():
                 pts = self.pointcloud_.pts_.detach()
-                self.cell_ids_ = pccnn_lib_ops.compute_keys(pts, self.pointcloud_.batch_ids_, self.bounding_box_.min_,
-                                                            self.num_cells_, self.cell_size_)
-                self.sorted_cell_ids_, self.sorted_ids_i32_, self.sorted_pts_ = pccnn_lib_ops.sort_keys(
-                    self.cell_ids_, self.key_bits(), pts)
+                batch = self.pointcloud_.batch_size_host()
+                cells = self.num_cells_host()
+                shape = [batch] + cells[0:2] + [2]
+                total = batch
+                for c in cells:
+                    total *= c
+                with_table = total if (len(cells) == 3 and total <= pccnn_lib_ops.CELL_TABLE_MAX_CELLS) else 0
+                (self.cell_ids_, self.sorted_cell_ids_, self.sorted_ids_i32_, self.sorted_pts_, self.grid_ds_,
+                 self.cell_table_) = pccnn_lib_ops.grid_build(pts, self.pointcloud_.batch_ids_,
+                                                              self.bounding_box_.min_, self.num_cells_,
+                                                              self.cell_size_, self.key_bits(), shape, with_table)
 
     def build_ds(self):
         if self.cell_ids_ is None or self.sorted_ids_i32_ is None:

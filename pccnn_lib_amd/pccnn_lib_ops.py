@@ -177,6 +177,39 @@ def build_cell_table(sorted_keys, total_cells):
     return table
 
 
+def grid_build(pts, batch_ids, aabb_min, grid_size, cell_size, key_bits, out_shape, with_cell_table):
+    """compute_keys + sort_keys + build_grid_ds (+ build_cell_table) of one grid as a single native call (what
+    pccnn_lib/pc/Grid.py:40-72 does in several).  Returns (keys i64[N], sorted keys i64[N], perm i32[N], sorted
+    points f32[N,D], grid_ds i32 of ``out_shape`` = [B, nc0, nc1, 2], cell table i32[cells + 1] or None)."""
+    name = "grid_build"
+    _chk(pts, name + ": pts", torch.float32, 2)
+    dev = pts.device
+    _chk(batch_ids, name + ": batch_ids", torch.int32, 1, dev)
+    _chk(aabb_min, name + ": aabb_min", torch.float32, 2, dev)
+    _chk(grid_size, name + ": grid_size", torch.int32, 1, dev)
+    _chk(cell_size, name + ": cell_size", torch.float32, 1, dev)
+    d = _dims(pts, name)
+    n = pts.shape[0]
+    out_shape = [int(v) for v in out_shape]
+    if batch_ids.shape[0] != n or aabb_min.shape[1] != d or grid_size.shape[0] != d or cell_size.shape[0] != d \
+            or len(out_shape) != 4 or out_shape[3] != 2 or min(out_shape) < 1:
+        raise RuntimeError(name + ": inconsistent shapes")
+    keys = torch.empty((n,), dtype=torch.int64, device=dev)
+    skeys = torch.empty_like(keys)
+    perm = torch.empty((n,), dtype=torch.int32, device=dev)
+    spts = torch.empty_like(pts)
+    ds = torch.empty(out_shape, dtype=torch.int32, device=dev)
+    total_cells, table = 0, None
+    if with_cell_table:
+        total_cells = int(with_cell_table)
+        table = torch.empty((total_cells + 1,), dtype=torch.int32, device=dev)
+    ws = _workspace(_lib.load().pccnn_grid_build_workspace_bytes(n), dev)
+    _lib.call("pccnn_grid_build", _ptr(pts), _ptr(batch_ids), _ptr(aabb_min), _ptr(grid_size), _ptr(cell_size), n, d,
+              int(key_bits), out_shape[0] * out_shape[1] * out_shape[2], total_cells, _ptr(keys), _ptr(skeys),
+              _ptr(perm), _ptr(spts), _ptr(ds), _optr(table), _ptr(ws), ws.numel(), _stream())
+    return keys, skeys, perm, spts, ds, table
+
+
 def find_neighbors_ex(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, radii, max_neighbors,
                       sample_order=None, point_remap=None, cell_table=None, samples_presorted=False):
     """find_neighbors with the native extras: ``sample_order`` (i32[M], samples listed in key order),
