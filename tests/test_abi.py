@@ -72,6 +72,14 @@ def test_argument_validation_needs_no_gpu(lib_path):
     rc = lib.pccnn_conv_weight_var(ctypes.byref(desc), None, None, None, None, None, None, 10, 10, 10, 3, 8, 0, None,
                                    None, 0, None)
     assert rc == -2 and b"k=65" in lib.pccnn_last_error()
+    rc = lib.pccnn_grid_build(None, None, None, None, None, 10, 9, 20, 4, 0, None, None, None, None, None, None, None,
+                              0, None)
+    assert rc == -2 and b"d=9" in lib.pccnn_last_error()
+    rc = lib.pccnn_compute_pdf_grid(3, None, None, None, 10, None, None, 4, None, 0, None, None, 2, 300, None, None, None)
+    assert rc == -2 and b"d=2" in lib.pccnn_last_error()
+    assert lib.pccnn_compute_pdf_grid(3, None, None, None, 0, None, None, 4, None, 0, None, None, 3, 300, None, None,
+                                      None) == 0
+    assert lib.pccnn_grid_build_workspace_bytes(1000) == lib.pccnn_sort_keys_workspace_bytes(1000)
     assert lib.pccnn_conv_workspace_bytes(1000, 5000, 32, 16, 64, 0) >= 1000 * 32 * 16 * 4
     assert lib.pccnn_find_neighbors_workspace_bytes(500, 1000) >= 4000 + 500 * 16
 
