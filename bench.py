@@ -354,6 +354,8 @@ def main():
                  "neighbor_pairs_per_sec": s_pairs / (s_ms * 1e-3),
                  "kernels_us": {k: round(1e3 * v[1] / v[0], 2) for k, v in s_kernels.items()},
                  "density_ms": sp_ms, "density_bandwidth": 0.01,
+                 # config 4 as the baseline words it: keys, grid, neighbors, then the density, per neighbor pair
+                 "neighbor_pairs_per_sec_with_density": s_pairs / ((s_ms + sp_ms) * 1e-3),
                  "density_kernels_us": {k: round(1e3 * v[1] / v[0], 2) for k, v in sp_kernels.items()}}
         log("scene: %d points, %d pairs, neighborhood %.3f ms -> %.2f G pairs/s" % (n_s, s_pairs, s_ms,
                                                                                   s_pairs / s_ms / 1e6))
