@@ -14,8 +14,10 @@
  *  - Return value: 0 on success, a negative PCCNN_ERR_* code otherwise;
  *    pccnn_last_error() then returns a thread-local description.  Arguments
  *    are validated on the host before any kernel is launched.
- *  - D (point dimensionality) is 3 in this build; other values return
- *    PCCNN_ERR_UNSUPPORTED.
+ *  - D (point dimensionality) is 2 to 6; the measured
+ *    kernels are the 3-dimensional ones, other D run slower general forms.
+ *    An entry point that is 3-dimensional only says so and returns
+ *    PCCNN_ERR_UNSUPPORTED for another D.
  *
  * Each entry point cites the reference interface it replaces (paths relative
  * to the reference repository; *.cuh lines are the host-function prototypes

@@ -7,8 +7,7 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-# PCCNN_HIP_LIB points at another build of the same library (e.g. an experimental one).
-LIB_PATH = os.environ.get("PCCNN_HIP_LIB") or os.path.join(HERE, "libpccnn_hip.so")
+LIB_PATH = os.path.join(HERE, "libpccnn_hip.so")
 
 P = ctypes.c_void_p
 I64 = ctypes.c_int64

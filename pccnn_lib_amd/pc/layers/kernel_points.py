@@ -1,11 +1,32 @@
 """Kernel-point layouts for KPConv.
 
-The reference ships hard-coded layouts for K in {8, 16, 32, 64}
-(pccnn_lib/pc/layers/kernel_points/kernel_points.py); this build generates its own, deterministically:
-one centre point plus K - 1 points on one shell (K <= 16) or on two shells of radius 0.5 and 1 (K > 16), in 2 to 6
-dimensions (the reference's table covers 2, 3 and 4).  Any K in [2, 64] is available.  A layout only has to start with the centre point:
-the layer normalises it by its largest norm (pccnn_lib/pc/layers/KPConv.py:46-57)."""
+The reference's twelve constant layouts (2, 3 and 4 dimensions, K in {8, 16, 32, 64};
+pccnn_lib/pc/layers/kernel_points/kernel_points.py:3-364) are read from ``kernel_points_tables.txt`` beside this file,
+so a layer built for one of those keys has the reference's ``kernel_pts_`` and ``sigma_``.  Any other key
+(2 to 6 dimensions, K in [2, 64], e.g. the 15 points of ``3_15``) is generated deterministically: one centre point plus
+K - 1 points on one shell (K <= 16) or on two shells of radius 0.5 and 1 (K > 16).  A layout only has to start with the
+centre point: the layer normalises it by its largest norm (pccnn_lib/pc/layers/KPConv.py:46-57)."""
+import os
+
 import numpy as np
+
+TABLES_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "kernel_points_tables.txt")
+
+
+def load_tables(path=TABLES_PATH):
+    """{'<dims>_<count>': float64 [count, dims]} from the data file: a line 'dims count', then the rows."""
+    tables = {}
+    with open(path) as handle:
+        lines = [l.split() for l in handle if l.strip() and not l.startswith("#")]
+    pos = 0
+    while pos < len(lines):
+        dims, count = int(lines[pos][0]), int(lines[pos][1])
+        block = np.array(lines[pos + 1:pos + 1 + count], dtype=np.float64)
+        if block.shape != (count, dims):
+            raise RuntimeError("kernel point table %d_%d is malformed in %s" % (dims, count, path))
+        tables["%d_%d" % (dims, count)] = block
+        pos += 1 + count
+    return tables
 
 
 def _fibonacci_sphere(count):
@@ -70,7 +91,7 @@ def kernel_points(num_dims, num_kernel_pts):
 
 
 class _Layouts(dict):
-    """Lookup by the reference's '<dims>_<count>' keys."""
+    """Lookup by the reference's '<dims>_<count>' keys: the constant tables, else a generated layout."""
 
     def __missing__(self, key):
         dims, count = key.split("_")
@@ -78,4 +99,4 @@ class _Layouts(dict):
         return self[key]
 
 
-kernel_pts_dict = _Layouts()
+kernel_pts_dict = _Layouts(load_tables())

@@ -3,6 +3,7 @@ import ctypes
 import os
 import re
 
+import numpy as np
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -127,6 +128,32 @@ def test_layers_keep_reference_parameter_names():
     assert {"proj_axis_", "proj_bias_", "conv_weights_", "pdf_mlp_.0.weight", "pdf_mlp_.2.weight"} <= set(pcv.state_dict())
 
 
+def test_kernel_point_layers_hold_the_reference_buffers():
+    """kernel_pts_ / sigma_ of a new layer, for every constant layout of the reference, against the fixture that
+    applies pccnn_lib/pc/layers/KPConv.py:46-57 to the reference's tables (tests/golden/make_kernel_point_buffers.py)."""
+    import torch
+    from pccnn_lib_amd.pc.layers import KPConv, KPConvN, PCCNN
+    from pccnn_lib_amd.pc.layers.kernel_points import kernel_pts_dict, load_tables
+    gold = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "kernel_point_buffers.npz"))
+    keys = sorted(k[len("table_"):] for k in gold.files if k.startswith("table_"))
+    assert keys == sorted(load_tables()) and len(keys) == 12
+    for key in keys:
+        dims, count = (int(v) for v in key.split("_"))
+        assert np.array_equal(kernel_pts_dict[key], gold["table_" + key]), key
+        layer = KPConv(dims, 4, 4, count)
+        assert layer.kernel_pts_.dtype == torch.float32 and layer.sigma_.dtype == torch.float32
+        assert np.array_equal(layer.kernel_pts_.numpy(), gold["kernel_pts_" + key]), key
+        assert float(layer.sigma_) == float(gold["sigma_" + key]), key
+    # KPConvN and PCCNN scale sigma by 2 and 0.4 (KPConvN.py:57, PCCNN.py:57); their rotation is seeded with the
+    # clock (KPConvN.py:53, PCCNN.py:53), so only what a rotation keeps is compared: norms and mutual distances
+    for cls, scale in ((KPConvN, 2.0), (PCCNN, 0.4)):
+        layer = cls(3, 4, 4, 16)
+        got, exp = layer.kernel_pts_.numpy().astype(np.float64), gold["kernel_pts_3_16"].astype(np.float64)
+        assert np.allclose(got @ got.T, exp @ exp.T, atol=1e-6)
+        d = float(gold["sigma_3_16"]) / (1.0 - float(gold["sigma_3_16"]))
+        assert abs(float(layer.sigma_) - scale * d / (1.0 + d)) < 1e-6
+
+
 def test_install_as_reference_resolves_the_reference_imports():
     # in a process of its own: the call registers modules under the reference's names
     import subprocess
@@ -141,4 +168,15 @@ def test_install_as_reference_resolves_the_reference_imports():
     import os
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     res = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr
+
+
+def test_the_op_module_imports_under_the_reference_name():
+    """`import pccnn_lib_ops` alone, in a fresh process, as pccnn_lib/op_wrappers/*.py do."""
+    import subprocess
+    import sys
+    code = ("import pccnn_lib_ops\n"
+            "assert len(pccnn_lib_ops.REFERENCE_NAMES) == 26\n"
+            "assert all(callable(getattr(pccnn_lib_ops, n)) for n in pccnn_lib_ops.REFERENCE_NAMES)\n")
+    res = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True, timeout=300)
     assert res.returncode == 0, res.stderr
