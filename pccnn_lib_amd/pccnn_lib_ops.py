@@ -280,9 +280,10 @@ def find_neighbors(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, radii
         cells = grid_size.tolist()
         bits = key_bits_for(cells, grid_ds.shape[0])
         skeys, order, spts = sort_keys(sample_keys, bits, samples)
-        total = grid_ds.shape[0] * cells[0] * cells[1] * cells[2]
-        if total <= CELL_TABLE_MAX_CELLS:
-            table = build_cell_table(pt_keys, total)
+        if len(cells) == 3:          # the per-cell start table belongs to the 3-dimensional walk only
+            total = grid_ds.shape[0] * cells[0] * cells[1] * cells[2]
+            if total <= CELL_TABLE_MAX_CELLS:
+                table = build_cell_table(pt_keys, total)
         return find_neighbors_ex(pts, pt_keys, spts, skeys, grid_ds, grid_size, radii, max_neighbors, order,
                                  cell_table=table, samples_presorted=True)
     return find_neighbors_ex(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, radii, max_neighbors, order,

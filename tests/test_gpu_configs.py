@@ -228,6 +228,7 @@ def test_config5_hierarchy_8x100k_properties(oracle):
         ends = p(nbh.start_ids_)
         assert ends[-1] == nbh.neighbors_.shape[0] and np.all(np.diff(ends, prepend=0) >= 1)
         if level == 0:
+            out.retain_grad()
             first = dict(pc_in=cur_pc, pc_out=out_pc, layer=layer, feats=cur_feats, out=out, nbh=nbh, radius=2 * radius)
         cur_pc, cur_feats, c_in = out_pc, torch.nn.functional.leaky_relu(out, 0.2), c_out
     out.sum().backward()
@@ -251,6 +252,19 @@ def test_config5_hierarchy_8x100k_properties(oracle):
                         (ends[sin] - p_lo).astype(np.int32), radii, p(layer.proj_axis_), p(layer.proj_bias_),
                         p(layer.conv_weights_), contraction="bf16")
     assert relerr(p(lv["out"])[sin], exp) < 3e-3
+    # Gradients of that cloud at the configuration's size.  The gradient that arrived at the first level's output
+    # through the three levels above it is the oracle's input.  Clouds do not interact, so the feature-gradient
+    # rows of the cloud in the end-to-end pass must be the oracle's; the weight gradient is summed over the batch,
+    # so the cloud's own share comes from one more call of the op on the cloud's slice (same kernels, same sizes).
+    g_out = p(lv["out"].grad)[sin]
+    host = (hp[pin], pdf, p(lv["feats"])[pin], hs[sin], local.astype(np.int32), (ends[sin] - p_lo).astype(np.int32),
+            radii, p(layer.proj_axis_), p(layer.proj_bias_), p(layer.conv_weights_))
+    exp_g = oracle.mcconv_grads(*host, g_out, contraction="bf16")
+    assert relerr(p(feats.grad)[pin], exp_g[1]) < 3e-3
+    from pccnn_lib_amd import pccnn_lib_ops as ops
+    got_g = ops.mc_conv_grads(*[t(a) for a in host], t(g_out), contraction="bf16")
+    for i, name in ((0, "dW"), (1, "dFeat"), (2, "dAxis"), (3, "dBias"), (4, "dPdf")):
+        assert relerr(p(got_g[i]), exp_g[i]) < 3e-3, name
 
 
 def test_projection_with_more_than_two_to_the_31_elements(ops):

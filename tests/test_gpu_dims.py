@@ -60,6 +60,21 @@ def test_neighborhood_bit_exact(ops, oracle, dims, batch, num_pts, radius):
         assert np.array_equal(exp["ends"], bf_ends)
 
 
+@pytest.mark.parametrize("dims,batch,num_pts,radius", [(2, 3, 2000, 0.04), (4, 2, 2500, 0.22)])
+def test_drop_in_find_neighbors_above_the_sorting_threshold(ops, oracle, dims, batch, num_pts, radius):
+    # more than 4096 samples: the reference-signature op sorts the samples by itself; the per-cell start table is a
+    # 3-dimensional structure and must stay out of it
+    pts, ids = _cloud(dims, batch, num_pts, 500 + dims)
+    assert pts.shape[0] > 4096
+    exp = oracle.neighborhood(pts, ids, pts, ids, radius)
+    g = gpu_neighborhood(ops, pts, ids, pts, ids, radius, batch)
+    d = g["dev"]
+    neigh, ends = ops.find_neighbors(d["spts"], d["skeys"], d["samples"], t(g["sample_keys"]), d["ds"], d["nc"],
+                                     d["radii"], 0)
+    assert np.array_equal(ends.cpu().numpy(), exp["ends"])
+    assert np.array_equal(oracle.canonical_pairs(neigh.cpu().numpy()), oracle.canonical_pairs(exp["neigh_sorted"]))
+
+
 @pytest.mark.parametrize("dims,batch,num_pts,radius", [(2, 3, 800, 0.1), (4, 2, 900, 0.3), (6, 2, 700, 0.6)])
 def test_distinct_samples_and_cap(ops, oracle, dims, batch, num_pts, radius):
     pts, ids = _cloud(dims, batch, num_pts, 200 + dims)

@@ -331,3 +331,28 @@ def test_capped_lists_are_the_ruled_subset_of_the_full_lists(ops, num_pts):
     raw_of_pair = np.repeat(raw, raw)
     keep = (raw_of_pair <= cap) | (((rank + 1) * cap) // raw_of_pair > (rank * cap) // raw_of_pair)
     assert np.array_equal(c_neigh, f_neigh[keep])
+
+
+@pytest.mark.parametrize("batch,num_pts,radius", [(3, 2500, 0.08), (1, 6000, 0.05)])
+def test_cell_average_pooling(ops, oracle, batch, num_pts, radius):
+    # pccnn_lib/pc/PointPooling.py:71-83 (one group per occupied cell: np.unique of the cell keys) and :97-102
+    # (scatter_mean / scatter_max over the groups)
+    import pccnn_lib_amd as lib
+    pts, ids = synthetic.primitives(31, batch, num_pts)
+    pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+    pool = lib.pc.PointPooling(pc, torch.full((3,), radius, device=DEV), "cell_average")
+    exp = oracle.neighborhood(pts, ids, pts, ids, radius)
+    uniq, inverse = np.unique(exp["keys"], return_inverse=True)
+    assert pool.num_pooling_pts_ == uniq.shape[0] and pool.pooling_ids_.dtype == torch.int64
+    assert np.array_equal(pool.pooling_ids_.cpu().numpy(), inverse.reshape(-1))
+    rng = np.random.default_rng(31)
+    vals = rng.normal(size=(pts.shape[0], 5)).astype(np.float32)
+    sums = np.zeros((uniq.shape[0], 5), np.float64)
+    np.add.at(sums, inverse.reshape(-1), vals.astype(np.float64))
+    counts = np.bincount(inverse.reshape(-1), minlength=uniq.shape[0]).astype(np.float64)
+    maxes = np.full((uniq.shape[0], 5), -np.inf, np.float32)
+    np.maximum.at(maxes, inverse.reshape(-1), vals)
+    mean = pool.pool_tensor(t(vals))
+    assert tuple(mean.shape) == (uniq.shape[0], 5)
+    assert np.abs(mean.cpu().numpy() - sums / counts[:, None]).max() < 1e-5
+    assert np.array_equal(pool.pool_tensor(t(vals), max_pool=True).cpu().numpy(), maxes)
