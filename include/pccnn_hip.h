@@ -73,6 +73,17 @@ size_t pccnn_sort_keys_workspace_bytes(int64_t n);
 int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int64_t *sorted_keys_out, int32_t *perm_out,
                     const float *pts, int d, float *sorted_pts_out,
                     void *workspace, size_t workspace_bytes, void *stream);
+/* pccnn_sort_keys without the workspace argument, for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same arguments, same results; the temporary storage is an array built into the library's device image
+ * (about 16 MiB per GPU, held until the process ends), so n is limited to PCCNN_SORT_KEYS_STATIC_MAX keys and a
+ * larger n returns PCCNN_ERR_UNSUPPORTED.  The call allocates nothing, frees nothing and creates no events; the
+ * device current at the call must be the stream's.  The first call on a device looks up the array's device
+ * address (make it outside a capture).  Every call on a GPU uses that GPU's one array: calls that overlap on
+ * one GPU (two streams, two threads) race; calls on one stream, or ordered by events, do not. */
+#define PCCNN_SORT_KEYS_STATIC_MAX (1 << 20)
+int pccnn_sort_keys_static(const int64_t *keys, int64_t n, int key_bits, int64_t *sorted_keys_out, int32_t *perm_out,
+                           const float *pts, int d, float *sorted_pts_out, void *stream);
 
 /* ---- pillar grid --------------------------------------------------------
  * Replaces build_grid_ds (pccnn_lib_ops/build_grid/build_grid_ds.cuh:25-28,

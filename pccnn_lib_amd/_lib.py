@@ -35,6 +35,7 @@ SIGNATURES = {
     "pccnn_compute_keys": (I32, [P, P, P, P, P, I64, I32, P, P]),
     "pccnn_sort_keys_workspace_bytes": (SZ, [I64]),
     "pccnn_sort_keys": (I32, [P, I64, I32, P, P, P, I32, P, P, SZ, P]),
+    "pccnn_sort_keys_static": (I32, [P, I64, I32, P, P, P, I32, P, P]),
     "pccnn_build_grid_ds": (I32, [P, I64, P, I32, I64, P, P]),
     "pccnn_find_neighbors_workspace_bytes": (SZ, [I64, I64]),
     "pccnn_build_cell_table": (I32, [P, I64, I64, P, P]),

@@ -176,6 +176,7 @@ __device__ __forceinline__ float pccnn_wave_sum(float v)
 
 // Optional per-kernel timing (off by default): a PccnnTimed object brackets the launches made
 // during its lifetime with two events on the launch stream; pccnn_timing_read sums them up.
+// A negative id never times (and so never creates an event).
 enum PccnnTimerId {
     PCCNN_T_GEMM = 0, PCCNN_T_PROJ_FWD, PCCNN_T_PROJ_BWD, PCCNN_T_BASIS_BWD, PCCNN_T_NB_COUNT, PCCNN_T_NB_FILL,
     PCCNN_T_SORT, PCCNN_T_KEYS, PCCNN_T_GRID, PCCNN_T_PDF, PCCNN_T_SCAN, PCCNN_T_COUNT

@@ -198,9 +198,11 @@ extern "C" size_t pccnn_sort_keys_workspace_bytes(int64_t n)
            pccnn_align((size_t)tiles * RS_MAX_DIGITS * sizeof(int32_t)) + pccnn_align(RS_MAX_DIGITS * sizeof(int32_t)) + 256;
 }
 
-extern "C" int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int64_t *sorted_keys_out,
-                               int32_t *perm_out, const float *pts, int d, float *sorted_pts_out,
-                               void *workspace, size_t workspace_bytes, void *stream)
+// The sort proper; `timed` = bracket the launches with the optional timing events (which are created on the fly,
+// so the entry point that must not allocate anything passes false).
+static int sort_keys_run(const int64_t *keys, int64_t n, int key_bits, int64_t *sorted_keys_out, int32_t *perm_out,
+                         const float *pts, int d, float *sorted_pts_out, void *workspace, size_t workspace_bytes,
+                         void *stream, bool timed_on)
 {
     PCCNN_REQUIRE(n >= 0 && n < (1ll << 31), PCCNN_ERR_INVALID, "pccnn_sort_keys: n=%lld", (long long)n);
     PCCNN_REQUIRE((pts == nullptr) == (sorted_pts_out == nullptr), PCCNN_ERR_INVALID,
@@ -225,7 +227,7 @@ extern "C" int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int
     int32_t *totals = arena.take<int32_t>(RS_MAX_DIGITS);
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "pccnn_sort_keys: workspace too small");
 
-    PccnnTimed timed(PCCNN_T_SORT, s);
+    PccnnTimed timed(timed_on ? PCCNN_T_SORT : -1, s);
     const int64_t *src_k = keys;
     const int32_t *src_v = nullptr;
     for (int p = 0; p < passes; ++p) {
@@ -265,4 +267,62 @@ extern "C" int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int
         src_v = dst_v;
     }
     return PCCNN_OK;
+}
+
+extern "C" int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int64_t *sorted_keys_out,
+                               int32_t *perm_out, const float *pts, int d, float *sorted_pts_out,
+                               void *workspace, size_t workspace_bytes, void *stream)
+{
+    return sort_keys_run(keys, n, key_bits, sorted_keys_out, perm_out, pts, d, sorted_pts_out, workspace,
+                         workspace_bytes, stream, true);
+}
+
+// ---- the same sort for callers that cannot allocate device memory ---------------------------------------------
+// Its workspace is a fixed array in the library's device image, one copy per GPU, held until the process ends.
+// In host code the array's name is only a handle: the device address of the current GPU's copy comes from
+// hipGetSymbolAddress, once per device, and that pointer is what the kernels, fills and copies get.
+#include <mutex>
+
+#define SORT_SCRATCH_BYTES                                                                                          \
+    ((size_t)PCCNN_SORT_KEYS_STATIC_MAX * 8 + (size_t)PCCNN_SORT_KEYS_STATIC_MAX * 4 +                              \
+     (size_t)(PCCNN_SORT_KEYS_STATIC_MAX / (RS_THREADS * RS_MAX_ITEMS)) * RS_MAX_DIGITS * 4 + RS_MAX_DIGITS * 4 + 1024)
+static __device__ __align__(256) unsigned char scratch[SORT_SCRATCH_BYTES];
+
+#define SORT_MAX_DEVICES 64
+static std::mutex g_scratch_mu;
+static void *g_scratch_ptr[SORT_MAX_DEVICES];          // device address of `scratch` on each GPU, 0 = not asked yet
+
+static int scratch_of_current_device(void **out)
+{
+    int dev = -1;
+    PCCNN_HIP_CHECK(hipGetDevice(&dev));
+    PCCNN_REQUIRE(dev >= 0 && dev < SORT_MAX_DEVICES, PCCNN_ERR_UNSUPPORTED,
+                  "pccnn_sort_keys_static: device %d is beyond the %d devices this build keeps a scratch pointer for",
+                  dev, SORT_MAX_DEVICES);
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void *p = nullptr;
+        PCCNN_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        PCCNN_REQUIRE(p != nullptr, PCCNN_ERR_HIP, "pccnn_sort_keys_static: the scratch array has no device address");
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return PCCNN_OK;
+}
+
+extern "C" int pccnn_sort_keys_static(const int64_t *keys, int64_t n, int key_bits, int64_t *sorted_keys_out,
+                                      int32_t *perm_out, const float *pts, int d, float *sorted_pts_out, void *stream)
+{
+    PCCNN_REQUIRE(n >= 0 && n <= PCCNN_SORT_KEYS_STATIC_MAX, PCCNN_ERR_UNSUPPORTED,
+                  "pccnn_sort_keys_static: n=%lld keys, the built-in scratch holds at most %d; use pccnn_sort_keys with "
+                  "a workspace for more", (long long)n, PCCNN_SORT_KEYS_STATIC_MAX);
+    PCCNN_REQUIRE(pccnn_sort_keys_workspace_bytes(n) <= SORT_SCRATCH_BYTES, PCCNN_ERR_UNSUPPORTED,
+                  "pccnn_sort_keys_static: %zu bytes of scratch needed, %zu built in",
+                  pccnn_sort_keys_workspace_bytes(n), (size_t)SORT_SCRATCH_BYTES);
+    void *ws = nullptr;
+    int rc = scratch_of_current_device(&ws);
+    if (rc != PCCNN_OK) return rc;
+    // every piece of the scratch that a pass reads is written by that pass first: nothing has to start at zero
+    return sort_keys_run(keys, n, key_bits, sorted_keys_out, perm_out, pts, d, sorted_pts_out, ws, SORT_SCRATCH_BYTES,
+                         stream, false);
 }

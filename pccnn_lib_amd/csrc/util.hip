@@ -30,7 +30,7 @@ static long long g_timing_n[PCCNN_T_COUNT];
 static const char *g_timing_names[PCCNN_T_COUNT] = {"gemm", "proj_fwd", "proj_bwd", "basis_bwd", "nb_count",
                                                     "nb_fill",  "sort",     "keys",     "grid",      "pdf", "scan"};
 
-PccnnTimed::PccnnTimed(int id_, hipStream_t s) : id(id_), stream(s), stop(nullptr), on(g_timing_on)
+PccnnTimed::PccnnTimed(int id_, hipStream_t s) : id(id_), stream(s), stop(nullptr), on(g_timing_on && id_ >= 0)
 {
     if (!on) return;
     hipEvent_t start;
