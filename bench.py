@@ -38,14 +38,24 @@ MFMA_FP32_PEAK_TFLOPS = 157.3     # MI355X dense fp32 matrix peak
 MFMA_BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 matrix peak
 HBM_PEAK_GBPS = 8000.0            # MI355X HBM3E peak
 
-# Bytes per launch that the dominant kernels move past the L2, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# of this command scaled by a copy kernel of known size (profiles/bench_mcconv_16x4096_hbm_traffic.md).  They
-# hold for the default workloads only (config 2; the scene leg at 1 000 000 points) and are reported as null otherwise.
-TRAFFIC_GEMM_BYTES = 312.7e6            # mean of the three contraction launches of a step (algorithmic: 313.5e6)
-TRAFFIC_PROJ_FWD_BYTES = 411.6e6         # conv_proj_fwd_kernel<MLP, 16, f32> (algorithmic: 294.7e6)
-TRAFFIC_PROJ_BWD_BYTES = 679.3e6         # conv_proj_bwd_kernel<MLP, 16, dF, dBasis> (algorithmic: 385.3e6)
-TRAFFIC_NB_FILL_BYTES_CONFIG2 = 20.0e6  # launches of 65 536 samples (algorithmic: 10.3e6)
-TRAFFIC_NB_FILL_BYTES_SCENE = 610.5e6   # launches of 1 000 000 samples (algorithmic: 194.6e6)
+
+
+def traffic(workload, kernel):
+    """Bytes per launch that a kernel moves past the L2 on one of the default workloads, from the table kept beside
+    the rocprofv3 counter summaries (profiles/traffic_table.json: FETCH_SIZE / WRITE_SIZE runs of this command, scaled
+    by the copy kernel of known size); None when the table has no entry (another size, a kernel not yet measured)."""
+    global _TRAFFIC
+    if _TRAFFIC is None:
+        try:
+            with open(os.path.join(ROOT, "profiles", "traffic_table.json")) as handle:
+                _TRAFFIC = json.load(handle)
+        except (OSError, ValueError):
+            _TRAFFIC = {}
+    entry = _TRAFFIC.get(workload, {}).get(kernel)
+    return float(entry["bytes"]) if entry else None
+
+
+_TRAFFIC = None
 
 
 def log(*a):
@@ -120,6 +130,144 @@ def cpu_baseline(wl, scalar_clouds=2):
     return result
 
 
+def config3_leg(lib, dev, timed, steps, warmup, with_cpu):
+    """Config 3: KPConv on 8 x 8192 surface points, radius 0.04, 15 kernel points, 128 -> 256 channels, fp32; forward
+    plus the gradients w.r.t. features, weights and point positions through the autograd wrapper."""
+    import torch
+    from pccnn_lib_amd import synthetic
+    from pccnn_lib_amd.op_wrappers import ComputeKPConv
+    batch, num_pts, c_in, c_out, k, radius = 8, 8192, 128, 256, 15, 0.04
+    pts, ids = synthetic.primitives(3, batch, num_pts)
+    rng = np.random.default_rng(3)
+    kp, sigma = synthetic.kernel_points_sphere(3, k)
+    feats = rng.normal(size=(pts.shape[0], c_in)).astype(np.float32)
+    w = rng.normal(0, np.sqrt(1.0 / (k * c_in)), (k * c_in, c_out)).astype(np.float32)
+    og = rng.normal(size=(pts.shape[0], c_out)).astype(np.float32)
+    t = lambda a: torch.as_tensor(a, device=dev)
+    pc = lib.pc.Pointcloud(t(pts), t(ids))
+    radii = torch.full((3,), radius, dtype=torch.float32, device=dev)
+    nbh = lib.pc.layers.conv_base.build_neighborhood(pc, pc, radii, 0)
+    mirror = nbh.mirror()
+    pairs = int(nbh.neighbors_.shape[0])
+    leaves = [x.clone().requires_grad_(True) for x in (t(pts), t(feats), t(w))]
+    tkp, tog = t(kp), t(og)
+
+    def step():
+        p, f, ww = leaves
+        out = ComputeKPConv.apply(p, f, p, nbh.neighbors_, nbh.start_ids_, radii, tkp, float(sigma), ww, mirror)
+        return torch.autograd.grad(out, leaves, tog)
+
+    ms, kernels = timed(step, steps, warmup)
+    m = pts.shape[0]
+    flops = 2.0 * m * (k * c_in) * c_out
+    g_n, g_ms = kernels.get("gemm", (0, 0.0))
+    g_avg = g_ms / max(g_n, 1)
+    tflops = flops / (g_avg * 1e-3) / 1e12 if g_n else 0.0
+    leg = {"workload": "config 3: KPConv fwd + dFeat, dW, dPts, 8 x 8192 points on random primitives, radius 0.04, "
+                       "15 kernel points, Cin 128 -> Cout 256, fp32",
+           "points": m, "pairs": pairs, "ms_per_step": ms, "points_per_sec": m / (ms * 1e-3),
+           "kernels_us": {kk: round(1e3 * v[1] / v[0], 2) for kk, v in kernels.items()},
+           "roofline": {"kernel": "gemm_f32_mfma_kernel", "bound": "mfma", "achieved": tflops,
+                        "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_FP32_PEAK_TFLOPS,
+                        "traffic": traffic("config3", "gemm_f32_mfma_kernel"), "flops_per_launch": flops,
+                        "avg_launch_ms": g_avg, "launches": g_n,
+                        "shapes": "P[65536,1920] W[1920,256]; P^T dOut; dOut W^T (mean of the three launches)"}}
+    log("config 3: %d pairs, step %.3f ms" % (pairs, ms),
+        {kk: "%d x %.1f us" % (v[0], 1e3 * v[1] / v[0]) for kk, v in kernels.items()})
+    if with_cpu:
+        # the same step in torch on the host cores, on the first two of the eight clouds
+        from oracle import oracle, torch_cpu
+        ns = 2 * num_pts
+        nb = oracle.neighborhood(pts[:ns], ids[:ns], pts[:ns], ids[:ns], radius)
+        run = lambda: torch_cpu.kpconv_step(pts[:ns], feats[:ns], nb["neighbors"], nb["ends"], nb["radii"], kp, sigma, w,
+                                            og[:ns])
+        run()
+        t0 = time.perf_counter()
+        reps = 0
+        while reps < 10 and (reps == 0 or time.perf_counter() - t0 < 8.0):
+            run()
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        leg["cpu_baseline"] = {"value": ns / dt, "unit": "points/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": "vectorised torch-CPU KPConv forward + weight, feature and position gradients "
+                                         "(oracle/torch_cpu.py) on 2 of the 8 clouds (%d points, %d pairs), %d "
+                                         "repetition(s)" % (ns, nb["neighbors"].shape[0], reps)}
+        log("config 3 cpu baseline: %.0f points/s" % (ns / dt))
+    return leg
+
+
+def config5_leg(lib, dev, steps, warmup):
+    """Config 5: 8 x 100 000 room points, four Poisson-disk levels (radii 0.025 / 0.05 / 0.1 / 0.2 of the room's
+    longest side), each with neighbor search (2 x the pooling radius), density and an MCConv with division by the
+    density, channels 8 -> 32 -> 64 -> 128 -> 256, bf16 contraction operands with fp32 accumulation; one forward pass
+    through the four levels and one backward pass, host-synchronised only at the end."""
+    import torch
+    from pccnn_lib_amd import synthetic
+    batch, num_pts = 8, 100000
+    pts = np.concatenate([synthetic.room(70 + b, num_pts) / 10.0 for b in range(batch)]).astype(np.float32)
+    ids = np.repeat(np.arange(batch, dtype=np.int32), num_pts)
+    tp, ti = torch.as_tensor(pts, device=dev), torch.as_tensor(ids, device=dev)
+    torch.manual_seed(5)
+    layers, c_in = [], 8
+    for c_out in (32, 64, 128, 256):
+        layer = lib.pc.layers.MCConv(3, c_in, c_out, 8).to(dev)
+        layer.contraction_ = "bf16"
+        layers.append(layer)
+        c_in = c_out
+    feats0 = torch.randn(pts.shape[0], 8, device=dev)
+    radii_levels = (0.025, 0.05, 0.1, 0.2)
+    sizes, marks = [], []
+
+    def whole(split=False):
+        pc = lib.pc.Pointcloud(tp, ti)
+        feats = feats0.clone().requires_grad_(True)
+        del sizes[:], marks[:]
+        for level, radius in enumerate(radii_levels):
+            if split:
+                torch.cuda.synchronize()
+                marks.append(time.perf_counter())
+            pool = lib.pc.PointPooling(pc, torch.full((3,), radius, device=dev))
+            out_pc = lib.pc.Pointcloud(pool.pool_tensor(pc.pts_), pool.pool_tensor(pc.batch_ids_))
+            pc.compute_pdf(0.2 * radius)
+            feats, nbh = layers[level](pc, out_pc, feats, 2.0 * radius)
+            feats = torch.nn.functional.leaky_relu(feats, 0.2)
+            sizes.append((int(pc.pts_.shape[0]), int(out_pc.pts_.shape[0]), int(nbh.neighbors_.shape[0])))
+            pc = out_pc
+        if split:
+            torch.cuda.synchronize()
+            marks.append(time.perf_counter())
+        feats.sum().backward()
+        if split:
+            torch.cuda.synchronize()
+            marks.append(time.perf_counter())
+        return feats
+
+    for _ in range(warmup):
+        whole()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        whole()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    split_ms = np.zeros(5)
+    for _ in range(steps):
+        whole(split=True)
+        split_ms += np.diff(np.array(marks)) * 1e3
+    split_ms /= steps
+    levels = [{"level": i, "radius": radii_levels[i], "points_in": sizes[i][0], "points_out": sizes[i][1],
+               "pairs": sizes[i][2], "forward_ms": float(split_ms[i])} for i in range(4)]
+    leg = {"workload": "config 5: 8 x 100000 room points, four Poisson-disk levels (0.025/0.05/0.1/0.2), neighbor "
+                       "search + density + MCConv 8->32->64->128->256 with bf16 contraction operands, forward + backward",
+           "points": int(pts.shape[0]), "ms_per_pass": ms, "points_per_sec": pts.shape[0] / (ms * 1e-3),
+           "dtype": "bf16 operands, f32 accumulate", "levels": levels, "backward_ms": float(split_ms[4]),
+           "note": "ms_per_pass is synchronised at the end only; the per-level times come from a second run with a "
+                   "host synchronisation between the levels, so they add up to more"}
+    log("config 5: pass %.3f ms" % ms, [(l["points_in"], l["points_out"], l["pairs"], round(l["forward_ms"], 3))
+                                        for l in levels], "backward %.3f ms" % split_ms[4])
+    return leg
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -128,6 +276,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-scene", action="store_true", help="skip the million-point neighbor-search leg")
     ap.add_argument("--scene-points", type=int, default=1000000)
+    ap.add_argument("--no-config3", action="store_true", help="skip the KPConv leg of config 3")
+    ap.add_argument("--no-config5", action="store_true", help="skip the four-level bf16 encoder leg of config 5")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on one GPU only; --gpus %d is not supported "
@@ -193,6 +343,9 @@ def main():
 
     mirror = nbh.mirror()        # the samples are the points: symmetric pair list (built once per neighborhood)
 
+    def mirror_step():
+        return ops.mirror_pairs(neigh, ends)
+
     def conv_step():
         p, q, f, a, b, w = leaves
         out = ComputeMCConv.apply(p, q, f, p, neigh, ends, radii, a, b, w, mirror)
@@ -249,6 +402,7 @@ def main():
     bf_ms, bf_kernels = timed(conv_step_bf16, args.steps, args.warmup)
     nb_ms, nb_kernels = timed(neighbor_step, args.steps, args.warmup)
     pdf_ms, pdf_kernels = timed(pdf_step, args.steps, args.warmup)
+    mirror_ms, _ = timed(mirror_step, args.steps, args.warmup)
     log("conv fwd+bwd %.3f ms (features+weights grads only: %.3f ms) | neighborhood %.3f ms | density %.3f ms"
         % (conv_ms, fw_ms, nb_ms, pdf_ms))
     log("conv fwd+bwd with bf16 contraction operands: %.3f ms" % bf_ms)
@@ -264,7 +418,7 @@ def main():
     gemm_tflops = gemm_flops / (gemm_avg_ms * 1e-3) / 1e12 if gemm_n else 0.0
     roofline = {"kernel": "gemm_f32_mfma_kernel", "bound": "mfma", "achieved": gemm_tflops,
                 "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": gemm_tflops / MFMA_FP32_PEAK_TFLOPS,
-                "traffic": TRAFFIC_GEMM_BYTES, "flops_per_launch": gemm_flops, "avg_launch_ms": gemm_avg_ms,
+                "traffic": traffic("config2", "gemm_f32_mfma_kernel"), "flops_per_launch": gemm_flops, "avg_launch_ms": gemm_avg_ms,
                 "launches": gemm_n}
 
     # ---- the two projection kernels against HBM bandwidth.  Algorithmic bytes, forward: pairs 8T + offsets 4M +
@@ -275,15 +429,15 @@ def main():
     geo_bytes = 8.0 * t_pairs + 4.0 * m + 12.0 * 2 * m + 4.0 * m * wl["c_in"] + 4.0 * m
     proj_bytes = 4.0 * m * kdim
     rooflines_proj = {}
-    for key, name, alg, traffic in (
-            ("proj_fwd", "conv_proj_fwd_kernel", geo_bytes + proj_bytes, TRAFFIC_PROJ_FWD_BYTES),
+    for key, name, alg, moved in (
+            ("proj_fwd", "conv_proj_fwd_kernel", geo_bytes + proj_bytes, traffic("config2", "conv_proj_fwd_kernel")),
             ("proj_bwd", "conv_proj_bwd_kernel", geo_bytes + proj_bytes + 4.0 * m * wl["c_in"] +
-             4.0 * t_pairs * wl["hidden"] + 16.0 * t_pairs, TRAFFIC_PROJ_BWD_BYTES)):
+             4.0 * t_pairs * wl["hidden"] + 16.0 * t_pairs, traffic("config2", "conv_proj_bwd_kernel"))):
         k_n, k_ms = conv_kernels.get(key, (0, 0.0))
         avg = k_ms / max(k_n, 1)
         gbps = alg / (avg * 1e-3) / 1e9 if k_n else 0.0
         rooflines_proj[key] = {"kernel": name, "bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                               "frac": gbps / HBM_PEAK_GBPS, "traffic": traffic, "bytes_per_launch": alg,
+                               "frac": gbps / HBM_PEAK_GBPS, "traffic": moved, "bytes_per_launch": alg,
                                "avg_launch_ms": avg, "launches": k_n}
 
     # the same three launches on the bf16 pipe (reported beside the fp32 figures; `value` is the fp32 step)
@@ -304,12 +458,12 @@ def main():
     fill_avg_ms = fill_total_ms / max(fill_n, 1)
     fill_gbps = nb_bytes / (fill_avg_ms * 1e-3) / 1e9 if fill_n else 0.0
     roofline_nb = {"kernel": "neighbors_group_kernel<fill, 8 lanes per sample>", "workload": "config 2", "bound": "hbm", "achieved": fill_gbps, "peak": HBM_PEAK_GBPS,
-                   "unit": "GB/s", "frac": fill_gbps / HBM_PEAK_GBPS, "traffic": TRAFFIC_NB_FILL_BYTES_CONFIG2,
+                   "unit": "GB/s", "frac": fill_gbps / HBM_PEAK_GBPS, "traffic": traffic("config2", "neighbors_fill"),
                    "bytes_per_launch": nb_bytes, "avg_launch_ms": fill_avg_ms, "launches": fill_n}
 
     # ---- scene-scale neighbor search (config 4: one room of 10^6 points, cell = radius = 0.05 m): the
     # neighbor kernels only show their throughput at this size, so their roofline entry is taken here
-    scene = None
+    scene = roofline_sort = roofline_pdf = roofline_pdf_grid = None
     if not args.no_scene:
         from pccnn_lib_amd import synthetic
         spts = t(synthetic.room(4, args.scene_points))
@@ -335,7 +489,7 @@ def main():
         roofline_nb = {"kernel": "neighbors_kernel<fill>", "workload": "config 4: %d room points, radius 0.05" % n_s,
                        "bound": "hbm", "achieved": s_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                        "frac": s_gbps / HBM_PEAK_GBPS,
-                       "traffic": TRAFFIC_NB_FILL_BYTES_SCENE if n_s == 1000000 else None, "bytes_per_launch": s_bytes,
+                       "traffic": traffic("scene_%d" % n_s, "neighbors_fill"), "bytes_per_launch": s_bytes,
                        "avg_launch_ms": f_avg, "launches": f_n}
         # the density of the same scene (Pointcloud.compute_pdf, bandwidth 0.2 x radius: its own grid of cell size
         # 4 x bandwidth, then the KDE walk on it)
@@ -350,6 +504,40 @@ def main():
 
         scene_pdf_step()
         sp_ms, sp_kernels = timed(scene_pdf_step, max(args.steps // 2, 3), 2)
+        # the key sort of the scene's grid: 44 N algorithmic bytes for one logical sort (keys 8N in, sorted keys 8N,
+        # permutation 4N and gathered coordinates 12N + 12N out), however many digit passes it takes
+        so_n, so_ms = s_kernels.get("sort", (0, 0.0))
+        so_avg = so_ms / max(so_n, 1)
+        so_gbps = 44.0 * n_s / (so_avg * 1e-3) / 1e9 if so_n else 0.0
+        roofline_sort = {"kernel": "radix_hist / radix_scan / radix_scatter (all passes of one sort)",
+                         "workload": "config 4: %d keys of %d significant bits" % (n_s, snb.grid_.key_bits()),
+                         "bound": "hbm", "achieved": so_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": so_gbps / HBM_PEAK_GBPS, "traffic": None, "bytes_per_launch": 44.0 * n_s,
+                         "avg_launch_ms": so_avg, "launches": so_n,
+                         "traffic_last_pass": traffic("scene_%d" % n_s, "radix_scatter_kernel_last_pass")}
+        # the density two ways: the walk on the grid that Pointcloud.compute_pdf runs (no pair list: sorted xyz 12N and
+        # keys 8N in, estimate and normalised estimate 8N out), and the list form of the reference's op on the
+        # radius-0.05 pair list (pairs 8T and xyz 12N in, offsets 4N in, estimate 4N out)
+        pg_n, pg_ms = sp_kernels.get("pdf", (0, 0.0))
+        pg_avg = pg_ms / max(pg_n, 1)
+        pg_gbps = 28.0 * n_s / (pg_avg * 1e-3) / 1e9 if pg_n else 0.0
+        roofline_pdf_grid = {"kernel": "pdf_grid_kernel", "workload": "config 4, bandwidth 0.01 (cell 0.04, cap 300)",
+                             "bound": "hbm", "achieved": pg_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                             "frac": pg_gbps / HBM_PEAK_GBPS, "traffic": traffic("scene_%d" % n_s, "pdf_grid_kernel"),
+                             "bytes_per_launch": 28.0 * n_s, "avg_launch_ms": pg_avg, "launches": pg_n}
+        tbw = torch.as_tensor(sbw, device=dev)
+        list_pdf_step = lambda: ops.compute_pdf(3, tbw, spts, snb.neighbors_, snb.start_ids_)
+        list_pdf_step()
+        _, pl_kernels = timed(list_pdf_step, max(args.steps // 2, 3), 2)
+        pl_n, pl_ms = pl_kernels.get("pdf", (0, 0.0))
+        pl_avg = pl_ms / max(pl_n, 1)
+        pl_bytes = 8.0 * s_pairs + 20.0 * n_s
+        pl_gbps = pl_bytes / (pl_avg * 1e-3) / 1e9 if pl_n else 0.0
+        roofline_pdf = {"kernel": "pdf_kernel", "workload": "config 4: compute_pdf on the radius-0.05 pair list "
+                                                            "(%d pairs), bandwidth 0.01" % s_pairs,
+                        "bound": "hbm", "achieved": pl_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                        "frac": pl_gbps / HBM_PEAK_GBPS, "traffic": None, "bytes_per_launch": pl_bytes,
+                        "avg_launch_ms": pl_avg, "launches": pl_n}
         scene = {"points": n_s, "pairs": s_pairs, "neighborhood_ms": s_ms,
                  "neighbor_pairs_per_sec": s_pairs / (s_ms * 1e-3),
                  "kernels_us": {k: round(1e3 * v[1] / v[0], 2) for k, v in s_kernels.items()},
@@ -361,6 +549,10 @@ def main():
                                                                                   s_pairs / s_ms / 1e6))
         log("scene", {k: "%d x %.1f us" % (v[0], 1e3 * v[1] / v[0]) for k, v in s_kernels.items()})
         log("scene density %.3f ms" % sp_ms, {k: "%d x %.1f us" % (v[0], 1e3 * v[1] / v[0]) for k, v in sp_kernels.items()})
+
+    config3 = None if args.no_config3 else config3_leg(lib, dev, timed, args.steps, args.warmup,
+                                                        not args.no_cpu_baseline)
+    config5 = None if args.no_config5 else config5_leg(lib, dev, max(args.steps // 2, 3), 2)
 
     cpu = None
     if not args.no_cpu_baseline:
@@ -378,13 +570,18 @@ def main():
                    "gradients": "all inputs (features, weights, axis, bias, density, positions); the step with the "
                                 "feature and weight gradients only is ms_per_step_feature_and_weight_grads_only"},
         "ms_per_step_feature_and_weight_grads_only": fw_ms,
+        # the symmetric-pair index that the step's point / density gradients use is built once per neighborhood
+        # (outside ms_per_step); a step on a fresh neighborhood pays it once more
+        "mirror_ms": mirror_ms, "ms_per_step_with_mirror": conv_ms + mirror_ms,
         "neighbor_pairs_per_sec": total_pairs / (nb_ms * 1e-3), "neighborhood_ms": nb_ms,
         "density_ms": pdf_ms,
         "kernels_us": {leg: {k: round(1e3 * v[1] / v[0], 2) for k, v in ks.items()}
                        for leg, ks in (("conv", conv_kernels), ("neighborhood", nb_kernels), ("density", pdf_kernels))},
         "bf16_contraction": bf16_leg, "scene": scene, "roofline": roofline, "roofline_neighbors": roofline_nb,
         "roofline_projection_forward": rooflines_proj["proj_fwd"],
-        "roofline_projection_backward": rooflines_proj["proj_bwd"], "hbm_copy_ceiling_gbps": copy_gbps,
+        "roofline_projection_backward": rooflines_proj["proj_bwd"], "roofline_sort": roofline_sort,
+        "roofline_pdf": roofline_pdf, "roofline_pdf_grid": roofline_pdf_grid, "config3": config3, "config5": config5,
+        "hbm_copy_ceiling_gbps": copy_gbps,
         "cpu_baseline": cpu,
     }
     print(json.dumps(result), flush=True)

@@ -257,6 +257,26 @@ def test_torch_cpu_step_matches_the_scalar_oracle(oracle, models):
         assert _relerr(grads[name].reshape(want.shape), want) < 1e-4, name
 
 
+def test_torch_cpu_kpconv_step_matches_the_scalar_oracle(oracle, models):
+    """The multi-threaded CPU baseline of the KPConv step (weights, features and position gradients) against the
+    scalar oracle, with an isolated point and a ragged last chunk."""
+    from oracle import torch_cpu
+    c_in, c_out = 6, 5
+    pts, ids, nb, feats, rng = _setup(oracle, models, 0.2, c_in, 23)
+    pts[-1] += 50.0
+    nb = oracle.neighborhood(pts, ids, pts, ids, 0.2)
+    neigh, ends, radii = nb["neighbors"], nb["ends"], nb["radii"]
+    kp, sigma = synthetic.kernel_points_sphere(5, 15)
+    w = rng.normal(0, 0.2, (15 * c_in, c_out)).astype(np.float32)
+    g = rng.normal(size=(pts.shape[0], c_out)).astype(np.float32)
+    out, grads = torch_cpu.kpconv_step(pts, feats, neigh, ends, radii, kp, sigma, w, g, samples_per_chunk=300)
+    ref = oracle.kpconv(pts, feats, pts, neigh, ends, radii, kp, sigma, w)
+    dw, dfeat, _, dpts, dsmp = oracle.kpconv_grads(pts, feats, pts, neigh, ends, radii, kp, sigma, w, g)
+    assert _relerr(out, ref) < 1e-5
+    for name, want in (("weights", dw), ("feats", dfeat), ("pts", dpts + dsmp)):
+        assert _relerr(grads[name].reshape(want.shape), want) < 1e-4, name
+
+
 def test_weight_variance_equals_projection_norm(oracle, models):
     # The double sum over neighbor pairs of (w_i . w_j)(F_i . F_j) (compute_variance_weights.cu:38-108) is the
     # squared Frobenius norm of the sample's projection tile; the literal O(n^2) restatement must agree with it.
