@@ -226,7 +226,7 @@ def config5_leg(lib, dev, steps, warmup):
             if split:
                 torch.cuda.synchronize()
                 marks.append(time.perf_counter())
-            pool = lib.pc.PointPooling(pc, torch.full((3,), radius, device=dev))
+            pool = lib.pc.PointPooling(pc, radius)
             out_pc = lib.pc.Pointcloud(pool.pool_tensor(pc.pts_), pool.pool_tensor(pc.batch_ids_))
             pc.compute_pdf(0.2 * radius)
             feats, nbh = layers[level](pc, out_pc, feats, 2.0 * radius)
@@ -276,6 +276,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-scene", action="store_true", help="skip the million-point neighbor-search leg")
     ap.add_argument("--scene-points", type=int, default=1000000)
+    ap.add_argument("--profile-leg", choices=["config3", "config5"], default=None,
+                    help="run this leg only (for rocprofv3 runs of one leg)")
     ap.add_argument("--no-config3", action="store_true", help="skip the KPConv leg of config 3")
     ap.add_argument("--no-config5", action="store_true", help="skip the four-level bf16 encoder leg of config 5")
     args = ap.parse_args()
@@ -297,6 +299,25 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    def timed(fn, steps, warmup):
+        """(ms per step, per-kernel timings).  The step time comes from a pass without the library's event
+        hooks (they serialise the stream around every hooked launch); a second pass of the same steps with
+        the hooks on gives the per-kernel durations."""
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        _lib.timing(enable=True, reset=True)
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        kernels = _lib.timing(enable=False)
+        return dt / steps * 1e3, kernels
+
     # what a plain float4 copy reaches on this part, as the practical ceiling beside the published 8 TB/s: 1 GiB read
     # and 1 GiB written per launch (beyond every cache), timed with events on the launch stream.  The same launches
     # are the known-size yardstick that rocprofv3's traffic counters are scaled against.
@@ -316,6 +337,13 @@ def main():
     copy_gbps = 5 * 2.0 * src.numel() * 4 / (e0.elapsed_time(e1) * 1e-3) / 1e9
     log("copy ceiling: %.0f GB/s" % copy_gbps)
     del src, dst
+
+    if args.profile_leg:
+        # one leg alone, for a profiler run of that leg (the JSON line then carries only that leg)
+        leg = config3_leg(lib, dev, timed, args.steps, args.warmup, False) if args.profile_leg == "config3" \
+            else config5_leg(lib, dev, args.steps, args.warmup)
+        print(json.dumps({"leg": args.profile_leg, "result": leg}), flush=True)
+        return 0
 
     wl = make_workload()
     t = lambda a: torch.as_tensor(a, device=dev)
@@ -377,25 +405,6 @@ def main():
         p = pc_fresh()
         p.compute_pdf(bw)
         return p
-
-    def timed(fn, steps, warmup):
-        """(ms per step, per-kernel timings).  The step time comes from a pass without the library's event
-        hooks (they serialise the stream around every hooked launch); a second pass of the same steps with
-        the hooks on gives the per-kernel durations."""
-        for _ in range(warmup):
-            fn()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            fn()
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-        _lib.timing(enable=True, reset=True)
-        for _ in range(steps):
-            fn()
-        torch.cuda.synchronize()
-        kernels = _lib.timing(enable=False)
-        return dt / steps * 1e3, kernels
 
     conv_ms, conv_kernels = timed(conv_step, args.steps, args.warmup)
     fw_ms, _ = timed(conv_step_fw_only, args.steps, args.warmup)

@@ -11,6 +11,7 @@ import numpy as np
 import torch
 
 _table = {}
+_host_values = {}        # id(tensor of the table) -> the host values it was made from
 _MAX_ENTRIES = 256
 
 
@@ -30,6 +31,15 @@ def device_vector(value, num_dims, device):
     if out is None:
         if len(_table) >= _MAX_ENTRIES:
             _table.clear()
+            _host_values.clear()
         out = torch.tensor(flat, dtype=torch.float32, device=device)
         _table[key] = out
+        _host_values[id(out)] = np.asarray(flat, dtype=np.float32)
     return out
+
+
+def host_vector(tensor):
+    """The host values (float32 numpy array) behind a tensor that ``device_vector`` made from host data, or None for
+    any other tensor: lets a caller do on the host, with the same fp32 arithmetic, what would otherwise need a
+    read-back."""
+    return _host_values.get(id(tensor)) if tensor is not None else None

@@ -1,7 +1,7 @@
 import torch
 
 from .. import pccnn_lib_ops
-from ._consts import device_vector
+from ._consts import device_vector, host_vector
 
 
 class Grid(object):
@@ -38,8 +38,19 @@ class Grid(object):
         return self.sorted_ids_i64_
 
     def num_cells_host(self):
+        """``num_cells_`` as a list of ints.  When the cell size came from host values, the same fp32 arithmetic
+        (subtract, IEEE divide, truncate, + 1, maximum over the clouds) runs in numpy on the box's host copy, which is
+        read back once per cloud, not once per grid; otherwise the device result is read back."""
         if self.num_cells_host_ is None:
-            self.num_cells_host_ = self.num_cells_.tolist()
+            cell = host_vector(self.cell_size_)
+            if cell is not None and hasattr(self.bounding_box_, "host"):
+                import numpy as np
+                mn, mx = self.bounding_box_.host()
+                with np.errstate(all="ignore"):
+                    cells = ((mx - mn) / cell.reshape(1, -1)).astype(np.int32) + np.int32(1)
+                self.num_cells_host_ = [int(v) for v in cells.max(axis=0)]
+            else:
+                self.num_cells_host_ = self.num_cells_.tolist()
         return self.num_cells_host_
 
     def key_bits(self):

@@ -1,8 +1,9 @@
+import numpy as np
 import torch
 
 from .. import pccnn_lib_ops
 from ..op_wrappers import ComputePDF
-from ._consts import device_vector
+from ._consts import device_vector, host_vector
 
 
 class Pointcloud(object):
@@ -18,18 +19,35 @@ class Pointcloud(object):
             del kwargs['requires_grad']
         self.pts_ = torch.as_tensor(p_pts, **kwargs)
         self.batch_ids_ = torch.as_tensor(p_batch_ids, **kwargs)
-        self.batch_size_ = torch.max(self.batch_ids_) + 1
-        self.batch_size_host_ = None            # int(batch_size_), read back once
+        # batch ids that PointPooling selected carry the number of clouds along (a Poisson-disk selection keeps at
+        # least one point of every cloud), which saves the read-back of their maximum
+        self.batch_size_host_ = getattr(p_batch_ids, "pccnn_batch_size_", None)
+        self.batch_size_tensor_ = None
+        if self.batch_size_host_ is None:
+            self.batch_size_tensor_ = torch.max(self.batch_ids_) + 1
         self.num_pts_per_batch_ = None          # cached result of get_num_points_per_batch()
         if self.pts_with_grads_:
             self.pts_.requires_grad = True
         self.pts_pdf_ = None
         self.pts_unnorm_pdf_ = None
 
+    @property
+    def batch_size_(self):
+        """0-d tensor max(batch_ids_) + 1 as in the reference (Pointcloud.py:38); made on first use when the number of
+        clouds was already known on the host."""
+        if self.batch_size_tensor_ is None:
+            self.batch_size_tensor_ = torch.max(self.batch_ids_) + 1
+        return self.batch_size_tensor_
+
+    @batch_size_.setter
+    def batch_size_(self, value):
+        self.batch_size_tensor_ = value
+
     def to_device(self, p_device):
         self.pts_ = self.pts_.to(p_device)
         self.batch_ids_ = self.batch_ids_.to(p_device)
-        self.batch_size_ = self.batch_size_.to(p_device)
+        if self.batch_size_tensor_ is not None:
+            self.batch_size_tensor_ = self.batch_size_tensor_.to(p_device)
         if self.pts_unnorm_pdf_ is not None:
             self.pts_unnorm_pdf_ = self.pts_unnorm_pdf_.to(p_device)
             self.pts_pdf_ = self.pts_pdf_.to(p_device)
@@ -54,7 +72,10 @@ class Pointcloud(object):
         from .grid import Grid
         from .neighborhood import Neighborhood
         bandwidth = device_vector(p_badnwidth, self.pts_.shape[1], self.pts_.device)
-        radii = bandwidth * 4.0
+        bandwidth_host = host_vector(bandwidth)
+        # four bandwidths (exact in fp32: a power of two), from the host values when they are known
+        radii = bandwidth * 4.0 if bandwidth_host is None else device_vector(bandwidth_host * np.float32(4.0),
+                                                                             self.pts_.shape[1], self.pts_.device)
         aabb = BoundingBox(self)
         grid = Grid(self, aabb, radii)
         grid.compute_cell_ids()

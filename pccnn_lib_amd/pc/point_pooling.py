@@ -45,7 +45,12 @@ class PointPooling(object):
 
     def pool_tensor(self, p_in_tensor, max_pool=False):
         if self.method_ == "poisson_disk":
-            return torch.index_select(p_in_tensor, 0, self.pooling_ids_)
+            out = torch.index_select(p_in_tensor, 0, self.pooling_ids_)
+            if p_in_tensor is self.point_cloud_.batch_ids_:
+                # the selection keeps at least one point of every cloud: a Pointcloud built from these ids need not
+                # read their maximum back
+                out.pccnn_batch_size_ = self.point_cloud_.batch_size_host()
+            return out
         index = self.pooling_ids_.to(torch.int64).reshape(-1, 1).expand(-1, p_in_tensor.shape[1])
         out = torch.zeros((self.num_pooling_pts_, p_in_tensor.shape[1]), dtype=p_in_tensor.dtype,
                           device=p_in_tensor.device)

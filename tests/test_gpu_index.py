@@ -356,3 +356,24 @@ def test_cell_average_pooling(ops, oracle, batch, num_pts, radius):
     assert tuple(mean.shape) == (uniq.shape[0], 5)
     assert np.abs(mean.cpu().numpy() - sums / counts[:, None]).max() < 1e-5
     assert np.array_equal(pool.pool_tensor(t(vals), max_pool=True).cpu().numpy(), maxes)
+
+
+def test_grid_size_on_the_host_equals_the_device_result(ops):
+    # a cell size given as host values: Grid.num_cells_host() redoes the fp32 arithmetic of Grid.py:26-28 in numpy on
+    # the box's host copy instead of reading the device result back; both must agree for every cloud and cell size
+    import pccnn_lib_amd as lib
+    rng = np.random.default_rng(77)
+    for trial in range(40):
+        batch = int(rng.integers(1, 5))
+        pts, ids = synthetic.primitives(100 + trial, batch, 700)
+        pts = (pts * rng.uniform(0.3, 7.0, (1, 3))).astype(np.float32)
+        pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+        for cell in (float(rng.uniform(0.01, 0.5)), rng.uniform(0.01, 0.5, 3).astype(np.float32), 0.05, 0.1, 0.25):
+            grid = lib.pc.Grid(pc, lib.pc.BoundingBox(pc), cell)
+            assert grid.num_cells_host() == grid.num_cells_.tolist()
+    # a cloud made from pooled batch ids knows its number of clouds without reading the ids back
+    pts, ids = synthetic.primitives(5, 3, 2000)
+    pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+    pool = lib.pc.PointPooling(pc, 0.1)
+    out = lib.pc.Pointcloud(pool.pool_tensor(pc.pts_), pool.pool_tensor(pc.batch_ids_))
+    assert out.batch_size_host_ == 3 and int(out.batch_size_) == 3 and int(torch.max(out.batch_ids_)) == 2
