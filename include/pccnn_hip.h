@@ -119,7 +119,10 @@ int pccnn_build_grid_ds(const int64_t *sorted_keys, int64_t n, const int32_t *nu
  * sorted index as in the reference op.  Pairs are grouped by ascending sample
  * index; inside a sample they are in ascending sorted-point order.
  * Both calls take the same workspace of pccnn_find_neighbors_workspace_bytes(n, m) bytes (count leaves the
- * per-sample raw counts in it; fill packs the sorted points into 16-byte records there). */
+ * per-sample raw counts in it; fill packs the sorted points into 16-byte records there).  The count call also
+ * leaves the pair total T as an int64 in the first 8 bytes of the workspace: ends_out is 32-bit like the
+ * reference's tensor and wraps beyond 2^31 - 1 pairs, that number does not, so a caller that reads it instead of
+ * ends_out[m-1] can refuse such a search. */
 size_t pccnn_find_neighbors_workspace_bytes(int64_t n, int64_t m);
 /* Optional accelerator for the search (no counterpart in the reference, which binary-searches the sorted
  * keys inside each pillar, find_ranges_grid_ds.cu:111-163): cell_table_out i32[total_cells + 1], entry c =

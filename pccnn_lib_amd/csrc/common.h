@@ -193,8 +193,9 @@ struct PccnnTimed {
 // Device-wide inclusive scan of int32 (scan.hip).  `clamp_max` > 0 clamps each input first.
 // tmp must hold pccnn_scan_tmp_elems(n) ints.
 size_t pccnn_scan_tmp_elems(int64_t n);
+// total64_out (nullable, device): the grand total without the 32-bit wrap-around.
 int pccnn_scan_inclusive_i32(const int32_t *in, int32_t *out, int64_t n, int clamp_max, int32_t *tmp,
-                             hipStream_t stream);
+                             hipStream_t stream, int64_t *total64_out = nullptr);
 
 // bf16 contraction (gemm_bf16.hip), used by conv.hip.
 extern "C" int pccnn_f32_to_bf16(const float *src, uint16_t *dst, int64_t count, void *stream);

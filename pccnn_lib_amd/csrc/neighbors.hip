@@ -546,15 +546,16 @@ extern "C" int pccnn_build_cell_table(const int64_t *sorted_keys, int64_t n, int
     return PCCNN_OK;
 }
 
-// Workspace layout, shared by the two calls: raw counts i32[m] | scan scratch (count) overlaid by the packed
-// point records float4[n] (fill).
+// Workspace layout, shared by the two calls: the pair total as int64 (written by the count call: the running
+// totals in ends_out are 32-bit and wrap, this number does not) | raw counts i32[m] | scan scratch (count)
+// overlaid by the packed point records float4[n] (fill).
 extern "C" size_t pccnn_find_neighbors_workspace_bytes(int64_t n, int64_t m)
 {
     if (m < 1) m = 1;
     if (n < 1) n = 1;
     size_t scan = pccnn_align(pccnn_scan_tmp_elems(m) * sizeof(int32_t));
     size_t rec = pccnn_align((size_t)n * sizeof(float4));
-    return pccnn_align((size_t)m * sizeof(int32_t)) + (scan > rec ? scan : rec) + 256;
+    return 256 + pccnn_align((size_t)m * sizeof(int32_t)) + (scan > rec ? scan : rec) + 256;
 }
 
 static int nb_validate(const char *who, const float *pts_sorted, const int64_t *pt_keys_sorted, int64_t n,
@@ -594,6 +595,7 @@ extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t
     PCCNN_REQUIRE(ends_out, PCCNN_ERR_INVALID, "pccnn_find_neighbors_count: null ends_out");
     hipStream_t s = (hipStream_t)stream;
     PccnnArena arena(workspace, workspace_bytes);
+    int64_t *total64 = arena.take<int64_t>(1);
     int32_t *counts = arena.take<int32_t>((size_t)m);
     int32_t *scan_tmp = arena.take<int32_t>(pccnn_scan_tmp_elems(m));
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "pccnn_find_neighbors_count: workspace too small");
@@ -624,7 +626,7 @@ extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t
     }
     PCCNN_LAUNCH_CHECK();
     PccnnTimed timed(PCCNN_T_SCAN, s);
-    return pccnn_scan_inclusive_i32(counts, ends_out, m, max_neighbors, scan_tmp, s);
+    return pccnn_scan_inclusive_i32(counts, ends_out, m, max_neighbors, scan_tmp, s, total64);
 }
 
 extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t *pt_keys_sorted, int64_t n,
@@ -644,6 +646,7 @@ extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t 
     PCCNN_REQUIRE(ends && neigh_out, PCCNN_ERR_INVALID, "pccnn_find_neighbors_fill: null pointer");
     hipStream_t s = (hipStream_t)stream;
     PccnnArena arena(workspace, workspace_bytes);
+    (void)arena.take<int64_t>(1);                              // the count call's pair total
     int32_t *counts = arena.take<int32_t>((size_t)m);
     float4 *rec = arena.take<float4>((size_t)(n > 0 ? n : 1));
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "pccnn_find_neighbors_fill: workspace too small");

@@ -155,7 +155,9 @@ extern "C" int pccnn_compute_pdf_sorted(int manifold_dims, const float *bandwidt
 // the 3 x 3 pillar ranges around its cell (the walk of the neighbor search, same order, same fp32 predicate) and adds
 // the kernel values as it goes: no pair list, no count / scan / fill, no host read-back of the pair count.  A point
 // with more hits than the cap walks a second time and keeps the subset the capped neighbor search keeps (hit number
-// r iff floor((r + 1) cap / raw) > floor(r cap / raw)), so both routes sum the same terms in the same order.
+// r iff floor((r + 1) cap / raw) > floor(r cap / raw)), so both routes sum the same terms.  The order of the
+// additions is the same only in the one-lane kernels; the kernels that share a point between several lanes add
+// strided partial sums, and the routes agree because the sums are kept in double, not bit for bit.
 struct PdfGridArgs {
     const float *pts;          // [n,3] in key order
     const int64_t *keys;       // [n] sorted

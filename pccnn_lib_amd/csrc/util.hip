@@ -145,7 +145,8 @@ extern "C" int pccnn_calibration_copy(const float *src, float *dst, int64_t coun
 #define SCAN_ITEMS 8
 #define SCAN_TILE (SCAN_THREADS * SCAN_ITEMS)
 
-size_t pccnn_scan_tmp_elems(int64_t n) { return (size_t)pccnn_ceil_div(n > 0 ? n : 1, SCAN_TILE) + 1; }
+// int32 tile sums, then (8-byte aligned) the 64-bit sums of the same tiles
+size_t pccnn_scan_tmp_elems(int64_t n) { return 3 * ((size_t)pccnn_ceil_div(n > 0 ? n : 1, SCAN_TILE) + 2); }
 
 // Inclusive scan of one value per thread across a 256-thread workgroup.
 __device__ __forceinline__ int block_inclusive_scan(int v, int *lds /* >= 4 ints */, int &total)
@@ -172,11 +173,28 @@ __device__ __forceinline__ int block_inclusive_scan(int v, int *lds /* >= 4 ints
     return v + add;
 }
 
+// Sum of one 64-bit value per thread across the workgroup, returned in every thread of wavefront 0.
+__device__ __forceinline__ long long block_sum_i64(long long v, long long *lds /* >= 4 */)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    if (pccnn_lane() == 0) lds[threadIdx.x >> 6] = v;
+    __syncthreads();
+    long long tot = 0;
+#pragma unroll
+    for (int w = 0; w < SCAN_THREADS / 64; ++w) tot += lds[w];
+    __syncthreads();
+    return tot;
+}
+
+// tile_sums64 (nullable): the same tile totals without the 32-bit wrap-around, for the caller that has to know
+// whether the running totals still fit 31 bits.
 __global__ void __launch_bounds__(SCAN_THREADS)
 scan_tiles_kernel(const int32_t *__restrict__ in, int32_t *__restrict__ out, int64_t n, int clamp_max,
-                  int32_t *__restrict__ tile_sums)
+                  int32_t *__restrict__ tile_sums, long long *__restrict__ tile_sums64)
 {
     __shared__ int lds[4];
+    __shared__ long long lds64[4];
     int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
     int v[SCAN_ITEMS];
     int sum = 0;
@@ -194,6 +212,28 @@ scan_tiles_kernel(const int32_t *__restrict__ in, int32_t *__restrict__ out, int
     for (int i = 0; i < SCAN_ITEMS; ++i)
         if (base + i < n) out[base + i] = v[i] + excl;
     if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
+    if (tile_sums64) {
+        long long wide = 0;
+#pragma unroll
+        for (int i = 0; i < SCAN_ITEMS; ++i) {
+            int x = (base + i < n) ? in[base + i] : 0;
+            if (clamp_max > 0 && x > clamp_max) x = clamp_max;
+            wide += x;
+        }
+        wide = block_sum_i64(wide, lds64);
+        if (threadIdx.x == 0) tile_sums64[blockIdx.x] = wide;
+    }
+}
+
+// total_out[0] = sum of the 64-bit tile sums (one workgroup).
+__global__ void __launch_bounds__(SCAN_THREADS)
+scan_total64_kernel(const long long *__restrict__ tile_sums64, int64_t num_tiles, long long *__restrict__ total_out)
+{
+    __shared__ long long lds64[4];
+    long long v = 0;
+    for (int64_t i = threadIdx.x; i < num_tiles; i += SCAN_THREADS) v += tile_sums64[i];
+    v = block_sum_i64(v, lds64);
+    if (threadIdx.x == 0) total_out[0] = v;
 }
 
 // Exclusive scan of the tile totals, in place, by a single workgroup.
@@ -223,12 +263,17 @@ scan_add_kernel(int32_t *__restrict__ out, int64_t n, const int32_t *__restrict_
 }
 
 int pccnn_scan_inclusive_i32(const int32_t *in, int32_t *out, int64_t n, int clamp_max, int32_t *tmp,
-                             hipStream_t stream)
+                             hipStream_t stream, int64_t *total64_out)
 {
     if (n <= 0) return PCCNN_OK;
     int64_t tiles = pccnn_ceil_div(n, SCAN_TILE);
-    scan_tiles_kernel<<<(unsigned)tiles, SCAN_THREADS, 0, stream>>>(in, out, n, clamp_max, tmp);
+    long long *sums64 = total64_out ? (long long *)(tmp + 2 * ((tiles + 2) / 2)) : nullptr;    // 8-byte aligned
+    scan_tiles_kernel<<<(unsigned)tiles, SCAN_THREADS, 0, stream>>>(in, out, n, clamp_max, tmp, sums64);
     PCCNN_LAUNCH_CHECK();
+    if (total64_out) {
+        scan_total64_kernel<<<1, SCAN_THREADS, 0, stream>>>(sums64, tiles, (long long *)total64_out);
+        PCCNN_LAUNCH_CHECK();
+    }
     if (tiles > 1) {
         scan_tile_sums_kernel<<<1, SCAN_THREADS, 0, stream>>>(tmp, tiles);
         PCCNN_LAUNCH_CHECK();

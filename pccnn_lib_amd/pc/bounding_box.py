@@ -11,7 +11,9 @@ class BoundingBox(object):
 
     A hierarchy level asks for the box of the same cloud several times (one grid each for pooling, density and the
     convolution's neighborhood), so the result is remembered on the cloud for as long as its coordinate and batch
-    tensors are the same objects and have not been written to (torch's version counters)."""
+    tensors are the same objects and have not been written to (torch's version counters).  A write through
+    ``pts_.data`` or ``.detach()`` does not move those counters: after such a write, drop the entry
+    (``del cloud.aabb_cache_``) or build a new Pointcloud, else grids keep using the old box."""
 
     def __init__(self, p_point_cloud):
         pts, ids = p_point_cloud.pts_, p_point_cloud.batch_ids_

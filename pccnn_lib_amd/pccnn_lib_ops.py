@@ -47,8 +47,13 @@ def _chk(t, name, dtype, ndim=None, device=None):
         raise RuntimeError("%s: expected %d dimensions, got shape %s" % (name, ndim, tuple(t.shape)))
     if not t.is_contiguous():
         raise RuntimeError("%s: expected a contiguous tensor" % name)
-    if device is not None and t.device != device:
-        raise RuntimeError("%s: on %s but other arguments are on %s" % (name, t.device, device))
+    if device is not None:
+        if t.device != device:
+            raise RuntimeError("%s: on %s but other arguments are on %s" % (name, t.device, device))
+    elif t.device.index != torch.cuda.current_device():
+        # the kernels are queued on the current device's stream (see _stream): the tensors must live there
+        raise RuntimeError("%s: on %s, but the current device is cuda:%d; run the call under "
+                           "`with torch.cuda.device(tensor.device):`" % (name, t.device, torch.cuda.current_device()))
     return t
 
 
@@ -256,8 +261,10 @@ def find_neighbors_ex(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, ra
     _lib.call("pccnn_find_neighbors_count", _ptr(pts), _ptr(pt_keys), n, _ptr(samples), _ptr(sample_keys), m, order_p,
               presorted, _ptr(grid_ds), pillars, table_p, total_cells, _ptr(grid_size), _ptr(radii), d, max_neighbors, _ptr(ends),
               _ptr(ws), ws.numel(), _stream())
-    total = int(ends[-1].item())                      # the one host read-back, as in the reference
-    if total < 0:
+    # the one host read-back, as in the reference; the 64-bit total from the head of the workspace rather than
+    # ends[-1], which is 32-bit and wraps (to a negative or, beyond 2^32 pairs, to a plausible positive number)
+    total = int(ws[:8].view(torch.int64).item())
+    if total < 0 or total > 0x7fffffff:
         raise RuntimeError(name + ": more than 2^31 - 1 pairs; the pair offsets are 32-bit as in the reference, "
                                   "use a smaller radius, a neighbor cap or fewer samples per call")
     neigh = torch.empty((total, 2), dtype=torch.int32, device=dev)

@@ -276,6 +276,13 @@ def test_pair_count_beyond_32_bits_is_an_error(ops):
     pc = lib.pc.Pointcloud(pts, torch.zeros(n, dtype=torch.int32, device=DEV))
     with pytest.raises(RuntimeError, match="pairs"):
         lib.pc.layers.conv_base.build_neighborhood(pc, pc, torch.full((3,), 1.0, device=DEV), 0)
+    # 70 000 such points are 4.9e9 pairs: the 32-bit running total wraps past 2^32 to a positive number
+    # (about 6e8), which only the 64-bit total that the count pass leaves in its workspace gives away
+    n = 70000
+    pts = t(np.random.default_rng(4).random((n, 3), dtype=np.float32) * 0.1)
+    pc = lib.pc.Pointcloud(pts, torch.zeros(n, dtype=torch.int32, device=DEV))
+    with pytest.raises(RuntimeError, match="pairs"):
+        lib.pc.layers.conv_base.build_neighborhood(pc, pc, torch.full((3,), 1.0, device=DEV), 0)
 
 
 def test_grid_ops_on_an_empty_cloud(ops):
