@@ -225,22 +225,20 @@ scan_tiles_kernel(const int32_t *__restrict__ in, int32_t *__restrict__ out, int
     }
 }
 
-// total_out[0] = sum of the 64-bit tile sums (one workgroup).
-__global__ void __launch_bounds__(SCAN_THREADS)
-scan_total64_kernel(const long long *__restrict__ tile_sums64, int64_t num_tiles, long long *__restrict__ total_out)
-{
-    __shared__ long long lds64[4];
-    long long v = 0;
-    for (int64_t i = threadIdx.x; i < num_tiles; i += SCAN_THREADS) v += tile_sums64[i];
-    v = block_sum_i64(v, lds64);
-    if (threadIdx.x == 0) total_out[0] = v;
-}
-
 // Exclusive scan of the tile totals, in place, by a single workgroup.
+// total_out (nullable): the sum of the 64-bit tile sums.
 __global__ void __launch_bounds__(SCAN_THREADS)
-scan_tile_sums_kernel(int32_t *__restrict__ tile_sums, int64_t num_tiles)
+scan_tile_sums_kernel(int32_t *__restrict__ tile_sums, int64_t num_tiles, const long long *__restrict__ tile_sums64,
+                      long long *__restrict__ total_out)
 {
     __shared__ int lds[4];
+    __shared__ long long lds64[4];
+    if (total_out) {
+        long long v = 0;
+        for (int64_t i = threadIdx.x; i < num_tiles; i += SCAN_THREADS) v += tile_sums64[i];
+        v = block_sum_i64(v, lds64);
+        if (threadIdx.x == 0) total_out[0] = v;
+    }
     int carry = 0;
     for (int64_t base = 0; base < num_tiles; base += SCAN_THREADS) {
         int64_t i = base + threadIdx.x;
@@ -267,15 +265,13 @@ int pccnn_scan_inclusive_i32(const int32_t *in, int32_t *out, int64_t n, int cla
 {
     if (n <= 0) return PCCNN_OK;
     int64_t tiles = pccnn_ceil_div(n, SCAN_TILE);
-    long long *sums64 = total64_out ? (long long *)(tmp + 2 * ((tiles + 2) / 2)) : nullptr;    // 8-byte aligned
+    // 64-bit tile sums behind the 32-bit ones (8-byte aligned); with a single tile its sum is the total
+    long long *sums64 = nullptr;
+    if (total64_out) sums64 = tiles > 1 ? (long long *)(tmp + 2 * ((tiles + 2) / 2)) : (long long *)total64_out;
     scan_tiles_kernel<<<(unsigned)tiles, SCAN_THREADS, 0, stream>>>(in, out, n, clamp_max, tmp, sums64);
     PCCNN_LAUNCH_CHECK();
-    if (total64_out) {
-        scan_total64_kernel<<<1, SCAN_THREADS, 0, stream>>>(sums64, tiles, (long long *)total64_out);
-        PCCNN_LAUNCH_CHECK();
-    }
     if (tiles > 1) {
-        scan_tile_sums_kernel<<<1, SCAN_THREADS, 0, stream>>>(tmp, tiles);
+        scan_tile_sums_kernel<<<1, SCAN_THREADS, 0, stream>>>(tmp, tiles, sums64, (long long *)total64_out);
         PCCNN_LAUNCH_CHECK();
         scan_add_kernel<<<(unsigned)tiles, SCAN_THREADS, 0, stream>>>(out, n, tmp);
         PCCNN_LAUNCH_CHECK();
