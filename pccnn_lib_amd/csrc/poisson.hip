@@ -31,6 +31,48 @@ cell_list_kernel(const int32_t *__restrict__ flags, const int32_t *__restrict__ 
     if (i == n - 1) *count = scan[i];
 }
 
+// Three dimensions: the non-empty cells listed per parity colour, so that a pass only touches the cells it works
+// on.  colour_list[colour * n + i] = index (into cell_first) of the i-th cell of that colour, in no particular
+// order: cells of one colour do not interact, so the selection does not depend on the order.  colour_count[8]
+// must be zero on entry.
+// COLOUR_ITEMS points per thread: 8 on large inputs, where the atomics on the eight global counters would
+// otherwise queue up, 1 on small ones, where the launch is a single round of short workgroups.
+template <int COLOUR_ITEMS>
+__global__ void __launch_bounds__(256)
+cell_colour_kernel(const int32_t *__restrict__ flags, const int32_t *__restrict__ scan, const int64_t *__restrict__ keys,
+                   int64_t n, const int32_t *__restrict__ num_cells, int32_t *__restrict__ colour_list,
+                   int32_t *__restrict__ colour_count)
+{
+    // the workgroup counts its cells per colour in LDS and reserves its share of every list with one atomic
+    __shared__ int local[8], start[8];
+    if (threadIdx.x < 8) local[threadIdx.x] = 0;
+    __syncthreads();
+    const int nc0 = num_cells[0], nc1 = num_cells[1], nc2 = num_cells[2];
+    int colour[COLOUR_ITEMS], at[COLOUR_ITEMS];
+#pragma unroll
+    for (int r = 0; r < COLOUR_ITEMS; ++r) {
+        const int64_t i = ((int64_t)blockIdx.x * COLOUR_ITEMS + r) * 256 + threadIdx.x;
+        colour[r] = -1;
+        at[r] = 0;
+        if (i < n && flags[i] != 0) {
+            long long k = keys[i];
+            const int c2 = (int)(k % nc2); k /= nc2;
+            const int c1 = (int)(k % nc1); k /= nc1;
+            const int c0 = (int)(k % nc0);
+            colour[r] = (c0 & 1) | ((c1 & 1) << 1) | ((c2 & 1) << 2);
+            at[r] = atomicAdd(&local[colour[r]], 1);
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < 8) start[threadIdx.x] = local[threadIdx.x] ? atomicAdd(&colour_count[threadIdx.x], local[threadIdx.x]) : 0;
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < COLOUR_ITEMS; ++r) {
+        const int64_t i = ((int64_t)blockIdx.x * COLOUR_ITEMS + r) * 256 + threadIdx.x;
+        if (colour[r] >= 0) colour_list[(int64_t)colour[r] * n + start[colour[r]] + at[r]] = scan[i] - 1;
+    }
+}
+
 #define POISSON_LOADS 8     // neighbor flags requested together by a lane
 
 template <int D>
@@ -120,6 +162,8 @@ struct PoissonGridArgs {
     volatile int32_t *used;      // [n] selection flags
     const int32_t *cell_first;   // compact list of the non-empty cells
     const int32_t *cell_count;
+    const int32_t *colour_list;  // [8][n] cells per parity colour (indices into cell_first)
+    const int32_t *colour_count; // [8]
 };
 
 __global__ void __launch_bounds__(256)
@@ -132,12 +176,14 @@ poisson_grid_pass_kernel(PoissonGridArgs a, int colour)
     const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     const int64_t waves = ((int64_t)gridDim.x * blockDim.x) >> 6;
     const int cells = *a.cell_count;
+    const int mine = a.colour_count[colour];                   // cells of this pass's colour
     const int32_t *settled = (const int32_t *)a.used;
     const int nc0 = a.num_cells[0], nc1 = a.num_cells[1], nc2 = a.num_cells[2];
     const float ir0 = __fdiv_rn(1.0f, a.radii[0]);
     const float ir1 = __fdiv_rn(1.0f, a.radii[1]);
     const float ir2 = __fdiv_rn(1.0f, a.radii[2]);
-    for (int64_t c = wave; c < cells; c += waves) {
+    for (int64_t ci = wave; ci < mine; ci += waves) {
+        const int c = a.colour_list[(int64_t)colour * a.grid.n + ci];
         const int first = a.cell_first[c];
         const int last = (c + 1 < cells) ? a.cell_first[c + 1] : (int)a.grid.n;
         long long k = a.grid.pt_keys[first];
@@ -145,7 +191,6 @@ poisson_grid_pass_kernel(PoissonGridArgs a, int colour)
         const int c1 = (int)(k % nc1);
         const long long pil = k; k /= nc1;
         const int c0 = (int)(k % nc0);
-        if ((c0 & 1) != (colour & 1) || (c1 & 1) != ((colour >> 1) & 1) || (c2 & 1) != ((colour >> 2) & 1)) continue;
         // the nine index ranges of the 27-cell walk (lane o looks up range o)
         if (lane < 9) {
             const int cmin = c2 > 0 ? c2 - 1 : 0, cmax = c2 + 1 < nc2 ? c2 + 1 : nc2 - 1;
@@ -220,8 +265,9 @@ compact_kernel(const int32_t *__restrict__ flags, const int32_t *__restrict__ sc
 extern "C" size_t pccnn_poisson_disk_workspace_bytes(int64_t n)
 {
     if (n < 1) n = 1;
-    // scan scratch | cell flags | first point of every cell | cell count
-    return pccnn_align(pccnn_scan_tmp_elems(n) * sizeof(int32_t)) + 2 * pccnn_align((size_t)n * sizeof(int32_t)) + 512;
+    // scan scratch | cell flags | first point of every cell | cell count, colour counts | cells per colour (3-D)
+    return pccnn_align(pccnn_scan_tmp_elems(n) * sizeof(int32_t)) + 2 * pccnn_align((size_t)n * sizeof(int32_t)) + 512 +
+           pccnn_align(8 * (size_t)n * sizeof(int32_t));
 }
 
 extern "C" int pccnn_poisson_disk_select(const int64_t *sorted_keys, int64_t n, const int32_t *neigh, int64_t t,
@@ -286,15 +332,26 @@ extern "C" int pccnn_poisson_disk_grid(const float *pts_sorted, const int64_t *s
     int32_t *scan_tmp = arena.take<int32_t>(pccnn_scan_tmp_elems(n));
     int32_t *flags = arena.take<int32_t>((size_t)n);
     int32_t *cell_first = arena.take<int32_t>((size_t)n);
-    int32_t *cell_count = arena.take<int32_t>(1);
+    int32_t *cell_count = arena.take<int32_t>(64);               // [0]: cells; [8..15]: cells per colour
+    int32_t *colour_list = arena.take<int32_t>(8 * (size_t)n);
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "pccnn_poisson_disk_grid: workspace of %zu bytes, need %zu",
                   workspace_bytes, pccnn_poisson_disk_workspace_bytes(n));
+    int32_t *colour_count = cell_count + 8;
     const unsigned blocks = (unsigned)pccnn_ceil_div(n, 256);
+    int rc = pccnn_fill_i32(cell_count, 0, 64, s);
+    if (rc != PCCNN_OK) return rc;
     cell_flag_kernel<<<blocks, 256, 0, s>>>(sorted_keys, n, flags);
     PCCNN_LAUNCH_CHECK();
-    int rc = pccnn_scan_inclusive_i32(flags, selected_scan_out, n, 0, scan_tmp, s);
+    rc = pccnn_scan_inclusive_i32(flags, selected_scan_out, n, 0, scan_tmp, s);
     if (rc != PCCNN_OK) return rc;
     cell_list_kernel<<<blocks, 256, 0, s>>>(flags, selected_scan_out, n, cell_first, cell_count);
+    PCCNN_LAUNCH_CHECK();
+    if (n > 131072)
+        cell_colour_kernel<8><<<(unsigned)pccnn_ceil_div(n, 256 * 8), 256, 0, s>>>(
+            flags, selected_scan_out, sorted_keys, n, num_cells, colour_list, colour_count);
+    else
+        cell_colour_kernel<1><<<blocks, 256, 0, s>>>(flags, selected_scan_out, sorted_keys, n, num_cells, colour_list,
+                                                     colour_count);
     PCCNN_LAUNCH_CHECK();
     if ((rc = pccnn_fill_i32(selected_out, 0, n, s)) != PCCNN_OK) return rc;
     PoissonGridArgs a;
@@ -302,6 +359,7 @@ extern "C" int pccnn_poisson_disk_grid(const float *pts_sorted, const int64_t *s
     a.grid = GridRef{cell_table, total_cells, grid_ds, num_pillars, sorted_keys, n};
     a.num_cells = num_cells; a.radii = radii; a.used = selected_out;
     a.cell_first = cell_first; a.cell_count = cell_count;
+    a.colour_list = colour_list; a.colour_count = colour_count;
     int64_t pass_blocks = pccnn_ceil_div(n, 64);
     if (pass_blocks > 2048) pass_blocks = 2048;
     for (int colour = 0; colour < 8; ++colour) {
