@@ -545,7 +545,8 @@ def main():
         roofline_pdf = {"kernel": "pdf_kernel", "workload": "config 4: compute_pdf on the radius-0.05 pair list "
                                                             "(%d pairs), bandwidth 0.01" % s_pairs,
                         "bound": "hbm", "achieved": pl_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                        "frac": pl_gbps / HBM_PEAK_GBPS, "traffic": None, "bytes_per_launch": pl_bytes,
+                        "frac": pl_gbps / HBM_PEAK_GBPS, "traffic": traffic("scene_%d" % n_s, "pdf_kernel"),
+                        "bytes_per_launch": pl_bytes,
                         "avg_launch_ms": pl_avg, "launches": pl_n}
         scene = {"points": n_s, "pairs": s_pairs, "neighborhood_ms": s_ms,
                  "neighbor_pairs_per_sec": s_pairs / (s_ms * 1e-3),
