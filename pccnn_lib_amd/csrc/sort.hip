@@ -10,6 +10,8 @@
 
 #define RS_THREADS 256
 #define RS_MAX_ITEMS 8                                  // keys per thread and tile, at most
+#define RS_STAGED_ITEMS RS_MAX_ITEMS                    // register arrays of the staged scatter kernel
+#define RS_STAGED_FROM_ITEMS 3                          // tiles of this many keys per thread or more take the staged kernel
 #define RS_WAVES (RS_THREADS / PCCNN_WAVE)
 
 // Keys per thread of a tile: small inputs get small tiles, so that the launch still has a few hundred
@@ -174,6 +176,157 @@ radix_scatter_kernel(const int64_t *__restrict__ keys_in, const int32_t *__restr
     }
 }
 
+// The scatter pass for large inputs.  Same job as radix_scatter_kernel (the slot of every key = keys with a smaller
+// digit + keys of the same digit in earlier tiles + its rank among the tile's keys of that digit), laid out
+// differently:
+//  * a wavefront owns items * 64 consecutive keys and ranks them against its own LDS counters, round after round
+//    without a workgroup barrier (a wavefront's LDS accesses execute in order); one barrier and one prefix over the
+//    waves then turn the counters into places inside the tile;
+//  * the tile is parked in LDS in sorted order and written out from there: the keys of one digit are consecutive
+//    in the tile and consecutive at their destination, so a run leaves as consecutive addresses from consecutive
+//    lanes instead of one 8-byte and one 4-byte store per lane wherever its key happens to go.
+template <int BITS, bool FIRST, bool GATHER>
+__global__ void __launch_bounds__(RS_THREADS)
+radix_scatter_staged_kernel(const int64_t *__restrict__ keys_in, const int32_t *__restrict__ vals_in, int64_t n, int shift,
+                            int items, const int32_t *__restrict__ tile_offsets, int64_t num_tiles,
+                            const int32_t *__restrict__ digit_totals, int64_t *__restrict__ keys_out,
+                            int32_t *__restrict__ vals_out, const float *__restrict__ pts, float *__restrict__ pts_out,
+                            int dims)
+{
+    constexpr int D = 1 << BITS;
+    constexpr int PER = D / RS_THREADS;                // digits per thread: tid * PER ... tid * PER + PER - 1
+    constexpr int STAGE_BYTES = RS_THREADS * RS_STAGED_ITEMS * 12;
+    constexpr int CNT_BYTES = RS_WAVES * D * 4;
+    __shared__ __align__(16) unsigned char lds[(STAGE_BYTES > CNT_BYTES ? STAGE_BYTES : CNT_BYTES) + D * 4 + 64];
+    volatile int *cnt = (volatile int *)lds;                                       // [RS_WAVES][D]; later the staging area
+    const int tile_keys = RS_THREADS * items;
+    long long *stage_keys = (long long *)lds;                                     // [tile_keys]
+    int *stage_vals = (int *)(lds + (size_t)tile_keys * 8);                       // [tile_keys]
+    int *base = (int *)(lds + (STAGE_BYTES > CNT_BYTES ? STAGE_BYTES : CNT_BYTES)); // [D] slot of the tile's j-th key = base[digit] + j
+    int *misc = base + D;                                                         // [16]
+
+    const int tid = threadIdx.x, lane = pccnn_lane(), wave = tid >> 6;
+    const int64_t tile = blockIdx.x;
+    for (int i = tid; i < RS_WAVES * D; i += RS_THREADS) cnt[i] = 0;
+    const int64_t tile_base = tile * tile_keys;
+    const int64_t wave_base = tile_base + (int64_t)wave * items * 64;
+    long long key[RS_STAGED_ITEMS];
+    int val[RS_STAGED_ITEMS], rnk[RS_STAGED_ITEMS];
+#pragma unroll
+    for (int r = 0; r < RS_STAGED_ITEMS; ++r) {
+        key[r] = 0;
+        val[r] = -1;                                                  // -1 = no key in this slot
+        if (r < items) {
+            const int64_t i = wave_base + r * 64 + lane;
+            if (i < n) {
+                key[r] = keys_in[i];
+                val[r] = FIRST ? (int)i : vals_in[i];
+            }
+        }
+    }
+    __syncthreads();                                                  // counters are zero
+    const unsigned long long lt = pccnn_lanemask_lt();
+#pragma unroll
+    for (int r = 0; r < RS_STAGED_ITEMS; ++r) {
+        rnk[r] = 0;
+        if (r < items) {
+            const bool valid = val[r] >= 0;
+            const int digit = (int)((key[r] >> shift) & (D - 1));
+            unsigned long long peers = __ballot(valid);               // lanes of this wave holding the same digit
+#pragma unroll
+            for (int b = 0; b < BITS; ++b) {
+                const unsigned long long bal = __ballot((digit >> b) & 1);
+                peers &= ((digit >> b) & 1) ? bal : ~bal;
+            }
+            const int rank_in_wave = __popcll(peers & lt);
+            // every lane reads the counter before the first of its peers moves it on
+            const int before = valid ? cnt[wave * D + digit] : 0;
+            __builtin_amdgcn_wave_barrier();
+            if (valid && rank_in_wave == 0) cnt[wave * D + digit] = before + __popcll(peers);
+            __builtin_amdgcn_wave_barrier();
+            rnk[r] = before + rank_in_wave;
+        }
+    }
+    __syncthreads();
+    // per digit: the tile's count and the waves' shares of it; prefix over the digits of both the tile's counts
+    // and the totals of all tiles
+    int tot[PER], glob[PER], wcnt[PER][RS_WAVES];
+    int sum_tot = 0, sum_glob = 0;
+#pragma unroll
+    for (int q = 0; q < PER; ++q) {
+        const int d = tid * PER + q;
+        tot[q] = 0;
+#pragma unroll
+        for (int w = 0; w < RS_WAVES; ++w) {
+            wcnt[q][w] = cnt[w * D + d];
+            tot[q] += wcnt[q][w];
+        }
+        glob[q] = digit_totals[d];
+        sum_tot += tot[q];
+        sum_glob += glob[q];
+    }
+    int local_start = sum_tot, global_start = sum_glob;
+    {
+        int ia = local_start, ib = global_start;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int ta = __shfl_up(ia, o), tb = __shfl_up(ib, o);
+            if (lane >= o) { ia += ta; ib += tb; }
+        }
+        if (lane == 63) { misc[wave] = ia; misc[RS_WAVES + wave] = ib; }
+        __syncthreads();
+        int pa = 0, pb = 0;
+#pragma unroll
+        for (int w = 0; w < RS_WAVES; ++w)
+            if (w < wave) { pa += misc[w]; pb += misc[RS_WAVES + w]; }
+        local_start = pa + ia - local_start;                          // exclusive, of this thread's first digit
+        global_start = pb + ib - global_start;
+    }
+#pragma unroll
+    for (int q = 0; q < PER; ++q) {
+        const int d = tid * PER + q;
+        base[d] = global_start + tile_offsets[(int64_t)d * num_tiles + tile] - local_start;
+        int at = local_start;
+#pragma unroll
+        for (int w = 0; w < RS_WAVES; ++w) {
+            cnt[w * D + d] = at;                                      // place of wave w's first key with digit d
+            at += wcnt[q][w];
+        }
+        local_start += tot[q];
+        global_start += glob[q];
+    }
+    __syncthreads();
+    int pos[RS_STAGED_ITEMS];
+#pragma unroll
+    for (int r = 0; r < RS_STAGED_ITEMS; ++r) {
+        pos[r] = 0;
+        if (r < items && val[r] >= 0) pos[r] = cnt[wave * D + (int)((key[r] >> shift) & (D - 1))] + rnk[r];
+    }
+    __syncthreads();                                                  // cnt is dead: its memory becomes the staging area
+#pragma unroll
+    for (int r = 0; r < RS_STAGED_ITEMS; ++r) {
+        if (r < items && val[r] >= 0) {
+            stage_keys[pos[r]] = key[r];
+            stage_vals[pos[r]] = val[r];
+        }
+    }
+    __syncthreads();
+    const int64_t left = n - tile_base;
+    const int tile_count = left < tile_keys ? (int)left : tile_keys;
+    for (int j = tid; j < tile_count; j += RS_THREADS) {
+        const long long k = stage_keys[j];
+        const int v = stage_vals[j];
+        const int64_t dst = (int64_t)base[(int)((k >> shift) & (D - 1))] + j;
+        keys_out[dst] = k;
+        vals_out[dst] = v;
+        if (GATHER) {
+#pragma unroll
+            for (int c = 0; c < PCCNN_MAX_DIMS; ++c)
+                if (c < dims) pts_out[dst * dims + c] = pts[(int64_t)v * dims + c];
+        }
+    }
+}
+
 // Passes and bits per pass for keys of `key_bits` significant bits: as few passes as the widest digit allows,
 // the bits spread evenly over them (18 bits: 2 x 9; 24: 3 x 8).  Wide digits pay where a pass is bound by its three
 // launches: up to 11 bits for at most 2^18 keys (65 536 keys of 18 bits: 26 us in 2 passes against 35 us in 3).
@@ -228,6 +381,9 @@ static int sort_keys_run(const int64_t *keys, int64_t n, int key_bits, int64_t *
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "pccnn_sort_keys: workspace too small");
 
     PccnnTimed timed(timed_on ? PCCNN_T_SORT : -1, s);
+    // measured: the staged scatter wins from about 300 000 keys on (84 against 99 us at 10^6 keys of 22 bits),
+    // the plain one below that (27 against 30 us at 65 536 keys), where a tile's fixed work outweighs its stores
+    const bool staged = items >= RS_STAGED_FROM_ITEMS;
     const int64_t *src_k = keys;
     const int32_t *src_v = nullptr;
     for (int p = 0; p < passes; ++p) {
@@ -239,9 +395,16 @@ static int sort_keys_run(const int64_t *keys, int64_t n, int key_bits, int64_t *
         bool gather = last && pts != nullptr;
         const unsigned grid = (unsigned)tiles;
 #define RS_SCATTER(B, FIRST, GATHER)                                                                            \
-    radix_scatter_kernel<B, FIRST, GATHER><<<grid, RS_THREADS, 0, s>>>(src_k, src_v, n, shift, items, hist, tiles, \
-                                                                       totals, dst_k, dst_v, GATHER ? pts : nullptr, \
-                                                                       GATHER ? sorted_pts_out : nullptr, d)
+    do {                                                                                                          \
+        if (staged)                                                                                               \
+            radix_scatter_staged_kernel<B, FIRST, GATHER><<<grid, RS_THREADS, 0, s>>>(                            \
+                src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, GATHER ? pts : nullptr,         \
+                GATHER ? sorted_pts_out : nullptr, d);                                                            \
+        else                                                                                                      \
+            radix_scatter_kernel<B, FIRST, GATHER><<<grid, RS_THREADS, 0, s>>>(                                   \
+                src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, GATHER ? pts : nullptr,         \
+                GATHER ? sorted_pts_out : nullptr, d);                                                            \
+    } while (0)
 #define RS_PASS(B)                                                                                   \
     do {                                                                                             \
         radix_hist_kernel<B><<<grid, RS_THREADS, 0, s>>>(src_k, n, shift, items, hist, tiles);       \
