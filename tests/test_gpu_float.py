@@ -28,7 +28,12 @@ def _cloud(models, batch, num_pts):
 
 @pytest.mark.parametrize("rows,cols,inner,at,bt,split", [
     (256, 128, 64, 0, 0, 1), (300, 70, 45, 0, 0, 1), (128, 256, 32, 0, 1, 1), (77, 130, 19, 0, 1, 1),
-    (128, 128, 4096, 1, 0, 8), (480, 40, 1000, 1, 0, 4), (129, 129, 17, 1, 1, 1), (1024, 128, 1024, 0, 0, 1)])
+    (128, 128, 4096, 1, 0, 8), (480, 40, 1000, 1, 0, 4), (129, 129, 17, 1, 1, 1), (1024, 128, 1024, 0, 0, 1),
+    # full tiles in every layout (64-row and 128-row tiles of the kernel without bounds checks), with and without
+    # a split of the reduction, and a reduction too short for that kernel
+    (192, 384, 208, 0, 0, 1), (192, 384, 208, 1, 0, 1), (192, 384, 208, 0, 1, 1), (192, 384, 208, 1, 1, 1),
+    (32768, 256, 192, 0, 0, 1), (32768, 128, 192, 1, 0, 1), (32768, 256, 192, 0, 1, 1), (32768, 128, 192, 1, 1, 1),
+    (256, 256, 16384, 1, 0, 8), (1024, 128, 8192, 1, 0, 32), (32768, 256, 64, 0, 1, 1)])
 def test_gemm_against_float64(rows, cols, inner, at, bt, split):
     from pccnn_lib_amd import _lib
     rng = np.random.default_rng(rows + cols + inner)
