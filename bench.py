@@ -271,8 +271,11 @@ def config5_leg(lib, dev, steps, warmup):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    # defaults: the first few milliseconds after an idle spell run at a lower shader clock and with the caching
+    # allocator still growing (about 2 ms spread over the first steps), so the warm-up is 50 steps (40 ms) and the
+    # timed region 100
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-scene", action="store_true", help="skip the million-point neighbor-search leg")
     ap.add_argument("--scene-points", type=int, default=1000000)
