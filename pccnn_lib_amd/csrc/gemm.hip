@@ -518,7 +518,9 @@ extern "C" int pccnn_gemm_f32(const float *a, const float *b, float *c, int64_t 
     // Lane offsets inside a tile are 32-bit byte offsets: 256 rows of the leading dimension must fit.
     const bool full_128 = rows % 128 == 0, full_64 = rows % 64 == 0;
     const bool full_ok = g.aligned && cols % GT_N == 0 && inner % GT_K == 0 && chunk >= 12 * GT_K && lda < (1ll << 20) &&
-                         ldb < (1ll << 20) && ldc % 4 == 0 && (uintptr_t)c % 16 == 0 && stride_c % 4 == 0;
+                         ldb < (1ll << 20) &&
+                         (split_k > 1 ? (uintptr_t)partial % 16 == 0
+                                      : ldc % 4 == 0 && (uintptr_t)c % 16 == 0 && stride_c % 4 == 0);
     // 128-row tiles unless that leaves the chip short of workgroups: the general kernel wants about four per CU,
     // the kernel for full tiles is ahead with 128-row tiles from one per CU on (65 536 x 128 x 1024: 140 against
     // 153 us with 64-row tiles; the wider tile needs fewer load instructions per MFMA)
