@@ -50,10 +50,11 @@ def test_gemm_against_float64(rows, cols, inner, at, bt, split):
     assert relerr(tc.cpu().numpy(), exp) < 1e-5
 
 
-def test_gemm_batched_strided():
+@pytest.mark.parametrize("m,mlps,inner,co", [(200, 2, 48, 24), (256, 2, 208, 128), (32768, 3, 192, 128)])
+def test_gemm_batched_strided(m, mlps, inner, co):
+    # the second and third shapes have full tiles: the kernel without bounds checks, 64-row and 128-row tiles
     from pccnn_lib_amd import _lib
     rng = np.random.default_rng(0)
-    m, mlps, inner, co = 200, 2, 48, 24
     a = rng.normal(size=(m, mlps * inner)).astype(np.float32)
     b = rng.normal(size=(mlps, inner, co)).astype(np.float32)
     ta, tb = t(a), t(b)
