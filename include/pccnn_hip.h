@@ -118,8 +118,10 @@ int pccnn_build_grid_ds(const int64_t *sorted_keys, int64_t n, const int32_t *nu
  * point_remap[sorted index] (fuses pccnn_lib/pc/Neighborhood.py:47-53), else the
  * sorted index as in the reference op.  Pairs are grouped by ascending sample
  * index; inside a sample they are in ascending sorted-point order.
- * Both calls take the same workspace of pccnn_find_neighbors_workspace_bytes(n, m) bytes (count leaves the
- * per-sample raw counts in it; fill packs the sorted points into 16-byte records there).  The count call also
+ * Both calls take the same workspace of pccnn_find_neighbors_workspace_bytes(n, m) bytes, untouched in between and
+ * with the same arguments: count leaves the per-sample raw counts in it and, for large uncapped searches, one bit
+ * per candidate it tested (neighbor or not), from which fill writes the pairs without testing again; otherwise
+ * fill packs the sorted points into 16-byte records there and repeats the walk.  The count call also
  * leaves the pair total T as an int64 in the first 8 bytes of the workspace: ends_out is 32-bit like the
  * reference's tensor and wraps beyond 2^31 - 1 pairs, that number does not, so a caller that reads it instead of
  * ends_out[m-1] can refuse such a search. */

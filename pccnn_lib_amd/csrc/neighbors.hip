@@ -20,6 +20,10 @@
 #define NB_WAVES (NB_THREADS / 64)
 #define NB_UNROLL_COUNT 4                              // candidates per lane and iteration of the walk
 #define NB_UNROLL_FILL 8
+// The count pass of the one-lane walk can leave its decisions behind: bit 4 * i + u of a sample's mask is the
+// outcome of candidate slot u of its walk iteration i (NB_UNROLL_COUNT slots per iteration).  Word w of all samples
+// is one row, so the 64 lanes of a tile, which finish a word in the same iteration, store it as one run.
+#define NB_MASK_WORDS 16                               // 256 iterations = 1024 candidate slots per sample are recorded
 
 struct NbArgs {
     const float *pts;          // sorted points [n,3]
@@ -43,6 +47,8 @@ struct NbArgs {
     int64_t t;                 // FILL: number of output pairs
     int32_t *neigh;            // FILL: [t,2]
     const float4 *rec;         // FILL: packed (x, y, z, id) of the sorted points
+    unsigned long long *masks; // nullable: hit bits of the one-lane walk, [NB_MASK_WORDS][m_pad] (count writes, fill reads)
+    int64_t m_pad;             // m rounded up to whole wavefronts
 };
 
 // Four consecutive ints at an 8-byte aligned address as one store instruction.
@@ -78,19 +84,25 @@ pack_points_kernel(const float *__restrict__ pts, const int32_t *__restrict__ re
     rec[i] = v;
 }
 
-template <bool FILL, bool CAPPED, int UNROLL>
-__global__ void __launch_bounds__(NB_THREADS)
-neighbors_kernel(NbArgs a)
-{
-    // ranges[w][r][lane] = r-th non-empty (first, len) range of the lane's sample; written and read by the
-    // same lane only, so no barrier is involved
-    __shared__ int2 ranges[NB_WAVES][9][64];
+// What a lane of the one-lane walk knows before it starts walking: its sample (index s, coordinates), and in
+// ranges[wib][0 .. nr - 1][lane] the non-empty index ranges of the sorted points it has to look at.
+struct NbLane {
+    int lane, wib;
+    int64_t base;
+    bool live, valid;          // the wavefront has samples at all; this lane has one
+    int s, nr;
+    float sx, sy, sz, ir0, ir1, ir2;
+};
 
+__device__ __forceinline__ NbLane nb_lane_setup(const NbArgs &a, int2 (*ranges)[9][64])
+{
+    NbLane L;
     const int lane = pccnn_lane();
     const int wib = threadIdx.x >> 6;
     const int64_t wave = ((int64_t)blockIdx.x * NB_THREADS + threadIdx.x) >> 6;
     const int64_t base = wave * 64;
-    if (base >= a.m) return;                                   // wave-uniform
+    L.live = base < a.m;                                       // wave-uniform
+    if (!L.live) return L;
     const bool valid = base + lane < a.m;
 
     int s = 0;
@@ -145,6 +157,26 @@ neighbors_kernel(NbArgs a)
         }
     }
 
+    L.lane = lane; L.wib = wib; L.base = base; L.valid = valid; L.s = s; L.nr = nr;
+    L.sx = sx; L.sy = sy; L.sz = sz; L.ir0 = ir0; L.ir1 = ir1; L.ir2 = ir2;
+    return L;
+}
+
+template <bool FILL, bool CAPPED, int UNROLL>
+__global__ void __launch_bounds__(NB_THREADS)
+neighbors_kernel(NbArgs a)
+{
+    // ranges[w][r][lane] = r-th non-empty (first, len) range of the lane's sample; written and read by the
+    // same lane only, so no barrier is involved
+    __shared__ int2 ranges[NB_WAVES][9][64];
+
+    const NbLane L = nb_lane_setup(a, ranges);
+    if (!L.live) return;
+    const int lane = L.lane, wib = L.wib, s = L.s, nr = L.nr;
+    const int64_t base = L.base;
+    const bool valid = L.valid;
+    const float sx = L.sx, sy = L.sy, sz = L.sz, ir0 = L.ir0, ir1 = L.ir1, ir2 = L.ir2;
+
     unsigned int my_off = 0;                                    // FILL: next output slot of this lane's sample
     int raw = 0, take_step = 0;                                 // capped: see below
     if (FILL && valid) {
@@ -162,6 +194,10 @@ neighbors_kernel(NbArgs a)
     // with every kept hit.  Samples at or below the cap use step = raw, which keeps every hit.
     int cnt = 0, err = 0;
     int r = 0, j = 0, first = 0, len = 0;
+    // count, uncapped: the outcome of every candidate slot goes into the sample's mask (see NB_MASK_WORDS)
+    const bool record = !FILL && UNROLL == NB_UNROLL_COUNT && a.masks != nullptr;
+    unsigned long long word = 0ull;
+    int it = 0;
     bool active = nr > 0;
     if (active) {
         const int2 g = ranges[wib][0][lane];
@@ -222,6 +258,7 @@ neighbors_kernel(NbArgs a)
                         }
                     }
                     ++cnt;
+                    if (!FILL) word |= 1ull << (((it & 15) << 2) + u);
                 }
             }
             j += UNROLL;
@@ -235,6 +272,15 @@ neighbors_kernel(NbArgs a)
                     active = false;
                 }
             }
+            if (!FILL) {
+                ++it;
+                // a word is complete after 16 iterations (for every lane still walking at once: one run of 8-byte
+                // stores), or when the lane's walk ends
+                if (record && ((it & 15) == 0 || !active) && ((it - 1) >> 4) < NB_MASK_WORDS) {
+                    a.masks[(size_t)((it - 1) >> 4) * a.m_pad + base + lane] = word;
+                    word = 0ull;
+                }
+            }
         }
     }
     if (FILL) {
@@ -242,6 +288,148 @@ neighbors_kernel(NbArgs a)
     } else if (valid) {
         a.counts[s] = cnt;
     }
+}
+
+// The fill pass of the one-lane walk when the count pass has left its masks.  Nothing is tested again and no
+// candidate is loaded: a lane reads its mask words (one run of 8-byte loads per word and tile), turns every set bit
+// into the index of the sorted point it stands for - bit 4 i + u is slot u of walk iteration i, and the iterations
+// of a sample are those of its ranges one after the other, ceil(len / 4) each -, fetches the ids of four neighbors
+// at a time and writes two pairs per store.  A pass over a word depends on memory once per four neighbors, where
+// the walk depended on it once per iteration.  Beyond the NB_MASK_WORDS * 16 recorded iterations (a sample with
+// more than about 1000 candidates) the lane tests the remaining candidates itself, exactly as the count pass did.
+__global__ void __launch_bounds__(NB_THREADS)
+neighbors_fill_masks_kernel(NbArgs a)
+{
+    __shared__ int2 ranges[NB_WAVES][9][64];
+    const NbLane L = nb_lane_setup(a, ranges);
+    if (!L.live) return;
+    const int lane = L.lane, wib = L.wib, s = L.s, nr = L.nr;
+    const int64_t base = L.base;
+
+    unsigned int my_off = 0;
+    if (L.valid) my_off = s > 0 ? (unsigned int)a.ends[s - 1] : 0u;
+    const unsigned int out_limit = (unsigned int)a.t;
+
+    int total_it = 0;                                           // iterations of this lane's walk
+    for (int q = 0; q < nr; ++q) total_it += (ranges[wib][q][lane].y + NB_UNROLL_COUNT - 1) / NB_UNROLL_COUNT;
+    // the range the enumeration stands in: its first iteration, its number of iterations, its first point
+    int r = 0, cum = 0, nit = 0, first = 0;
+    if (nr > 0) {
+        const int2 g = ranges[wib][0][lane];
+        first = g.x;
+        nit = (g.y + NB_UNROLL_COUNT - 1) / NB_UNROLL_COUNT;
+    }
+    const int my_words = total_it < NB_MASK_WORDS * 16 ? (total_it + 15) >> 4 : NB_MASK_WORDS;
+    int w = 0;
+    unsigned long long word = my_words > 0 ? a.masks[base + lane] : 0ull;
+    unsigned long long next_word = my_words > 1 ? a.masks[(size_t)a.m_pad + base + lane] : 0ull;
+    // Up to eight neighbors per round, and never across a 64-byte boundary of the pair list: after its first
+    // round a lane writes whole aligned 64-byte pieces of its segment, four 16-byte stores back to back, so a
+    // piece reaches memory complete instead of in quarters that leave the L2 one by one.
+    while (__any(word != 0ull || w + 1 < my_words)) {
+        const int cap = 8 - (int)(my_off & 7u);
+        int idx[8], have = 0;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            idx[q] = 0;
+            while (word == 0ull && w + 1 < my_words) {          // on to the lane's next word that has a bit set:
+                ++w;                                            // the neighbors of a round stay in slots 0 .. have - 1
+                word = next_word;
+                if (w + 1 < my_words) next_word = a.masks[(size_t)(w + 1) * a.m_pad + base + lane];
+            }
+            if (have < cap && word != 0ull) {
+                const int b = __builtin_ctzll(word);
+                word &= word - 1ull;
+                const int i = (w << 4) + (b >> 2);
+                while (i >= cum + nit && r + 1 < nr) {          // at most nr - 1 steps in the life of the lane
+                    cum += nit;
+                    ++r;
+                    const int2 g = ranges[wib][r][lane];
+                    first = g.x;
+                    nit = (g.y + NB_UNROLL_COUNT - 1) / NB_UNROLL_COUNT;
+                }
+                // (masks that no count call wrote cannot send a lane out of its ranges or out of the points)
+                const int at = first + ((i - cum) << 2) + (b & 3);
+                idx[q] = (i < cum + nit && (int64_t)at < a.n) ? at : 0;
+                have = q + 1;
+            }
+        }
+        int id[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) id[q] = (q < have && a.remap) ? a.remap[idx[q]] : idx[q];
+#pragma unroll
+        for (int q = 0; q < 8; q += 2) {
+            if (q + 1 < have) {
+                if (my_off + 1u < out_limit) nb_store4(a.neigh + 2 * (size_t)my_off, id[q], s, id[q + 1], s);
+                my_off += 2u;
+            } else if (q < have) {
+                if (my_off < out_limit) ((int2 *)a.neigh)[my_off] = make_int2(id[q], s);
+                my_off += 1u;
+            }
+        }
+    }
+    int held = -1;
+    auto emit = [&](int id) {
+        if (held < 0) {
+            held = id;
+        } else {
+            if (my_off + 1u < out_limit) nb_store4(a.neigh + 2 * (size_t)my_off, held, s, id, s);
+            my_off += 2u;
+            held = -1;
+        }
+    };
+    // the rare tail: iterations that the masks do not cover
+    if (__any(total_it > NB_MASK_WORDS * 16)) {
+        bool active = total_it > NB_MASK_WORDS * 16;
+        int j = 0, len = 0;
+        if (active) {
+            const int it0 = NB_MASK_WORDS * 16;
+            while (it0 >= cum + nit && r + 1 < nr) {
+                cum += nit;
+                ++r;
+                nit = (ranges[wib][r][lane].y + NB_UNROLL_COUNT - 1) / NB_UNROLL_COUNT;
+            }
+            const int2 g = ranges[wib][r][lane];
+            first = g.x;
+            len = g.y;
+            j = (it0 - cum) * NB_UNROLL_COUNT;
+        }
+        while (__any(active)) {
+            if (active) {
+                const int left = len - j;
+                float px[NB_UNROLL_COUNT], py[NB_UNROLL_COUNT], pz[NB_UNROLL_COUNT];
+                int id[NB_UNROLL_COUNT];
+#pragma unroll
+                for (int u = 0; u < NB_UNROLL_COUNT; ++u) {         // all loads of the iteration together
+                    const int64_t iu = first + j + (u < left ? u : 0);
+                    px[u] = a.pts[iu * 3 + 0];
+                    py[u] = a.pts[iu * 3 + 1];
+                    pz[u] = a.pts[iu * 3 + 2];
+                    id[u] = a.remap ? a.remap[iu] : (int)iu;
+                }
+#pragma unroll
+                for (int u = 0; u < NB_UNROLL_COUNT; ++u) {
+                    const float vx = (L.sx - px[u]) * L.ir0;
+                    const float vy = (L.sy - py[u]) * L.ir1;
+                    const float vz = (L.sz - pz[u]) * L.ir2;
+                    const float acc = ((0.0f + vx * vx) + vy * vy) + vz * vz;
+                    if (u < left && acc < 1.0f) emit(id[u]);
+                }
+                j += NB_UNROLL_COUNT;
+                if (j >= len) {
+                    j = 0;
+                    if (++r < nr) {
+                        const int2 g = ranges[wib][r][lane];
+                        first = g.x;
+                        len = g.y;
+                    } else {
+                        active = false;
+                    }
+                }
+            }
+        }
+    }
+    if (held >= 0 && my_off < out_limit) ((int2 *)a.neigh)[my_off] = make_int2(held, s);
 }
 
 // Few samples against many points (every pooling level of a hierarchy): with one sample per lane the launch has
@@ -555,7 +743,8 @@ extern "C" size_t pccnn_find_neighbors_workspace_bytes(int64_t n, int64_t m)
     if (n < 1) n = 1;
     size_t scan = pccnn_align(pccnn_scan_tmp_elems(m) * sizeof(int32_t));
     size_t rec = pccnn_align((size_t)n * sizeof(float4));
-    return 256 + pccnn_align((size_t)m * sizeof(int32_t)) + (scan > rec ? scan : rec) + 256;
+    size_t masks = pccnn_align((size_t)NB_MASK_WORDS * pccnn_ceil_div(m, 64) * 64 * sizeof(unsigned long long));
+    return 256 + pccnn_align((size_t)m * sizeof(int32_t)) + masks + (scan > rec ? scan : rec) + 256;
 }
 
 static int nb_validate(const char *who, const float *pts_sorted, const int64_t *pt_keys_sorted, int64_t n,
@@ -597,6 +786,8 @@ extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t
     PccnnArena arena(workspace, workspace_bytes);
     int64_t *total64 = arena.take<int64_t>(1);
     int32_t *counts = arena.take<int32_t>((size_t)m);
+    const int64_t m_pad = pccnn_ceil_div(m, 64) * 64;
+    unsigned long long *masks = arena.take<unsigned long long>((size_t)NB_MASK_WORDS * m_pad);
     int32_t *scan_tmp = arena.take<int32_t>(pccnn_scan_tmp_elems(m));
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "pccnn_find_neighbors_count: workspace too small");
     NbArgs a;
@@ -608,6 +799,9 @@ extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t
     a.num_cells = num_cells; a.radii = radii; a.max_neighbors = max_neighbors;
     a.counts = counts; a.ends = nullptr; a.remap = nullptr; a.t = 0; a.neigh = nullptr; a.rec = nullptr;
     const int group = nb_group_size(n, m, d);
+    // the uncapped one-lane walk leaves its decisions for the fill call
+    a.masks = (group == 1 && d == 3 && max_neighbors == 0) ? masks : nullptr;
+    a.m_pad = m_pad;
     int64_t waves = pccnn_ceil_div(m * group, 64);
     {
         PccnnTimed timed(PCCNN_T_NB_COUNT, s);
@@ -648,6 +842,8 @@ extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t 
     PccnnArena arena(workspace, workspace_bytes);
     (void)arena.take<int64_t>(1);                              // the count call's pair total
     int32_t *counts = arena.take<int32_t>((size_t)m);
+    const int64_t m_pad = pccnn_ceil_div(m, 64) * 64;
+    unsigned long long *masks = arena.take<unsigned long long>((size_t)NB_MASK_WORDS * m_pad);
     float4 *rec = arena.take<float4>((size_t)(n > 0 ? n : 1));
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "pccnn_find_neighbors_fill: workspace too small");
     NbArgs a;
@@ -658,12 +854,16 @@ extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t 
     a.cell_table = cell_table; a.total_cells = total_cells;
     a.num_cells = num_cells; a.radii = radii; a.max_neighbors = max_neighbors;
     a.counts = counts; a.ends = ends; a.remap = point_remap; a.t = t; a.neigh = neigh_out; a.rec = rec;
+    a.masks = masks; a.m_pad = m_pad;
     const int group = nb_group_size(n, m, d);
     int64_t waves = pccnn_ceil_div(m * group, 64);
     {
         PccnnTimed timed(PCCNN_T_NB_FILL, s);
         const unsigned blocks = (unsigned)pccnn_ceil_div(waves, NB_THREADS / 64);
-        if (d == 3) {
+        if (d == 3 && group == 1 && max_neighbors == 0) {
+            // the count call left the outcome of every candidate test in the workspace: nothing is tested again
+            neighbors_fill_masks_kernel<<<blocks, NB_THREADS, 0, s>>>(a);
+        } else if (d == 3) {
             if (n > 0) pack_points_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(pts_sorted, point_remap, n, rec);
             if (group == 64) {
                 if (max_neighbors > 0) neighbors_group_kernel<true, true, 64><<<blocks, NB_THREADS, 0, s>>>(a);
