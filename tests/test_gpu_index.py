@@ -267,6 +267,35 @@ def test_scene_scale_properties(ops, num_pts):
         assert sure <= count <= maybe, s_i
 
 
+def test_one_lane_walk_with_more_candidates_than_its_masks_hold(ops):
+    # 140 000 samples run the one-lane walk, whose count pass records 1024 candidate slots per sample for the fill
+    # pass; 1500 points inside a 4 mm cube give their samples more than that, so the fill pass tests the rest itself.
+    # Every list of the clump and of 200 other samples against a float64 count over all points (boundary cases
+    # within 1e-6 of the radius set aside), plus the properties that hold for the whole list.
+    rng = np.random.default_rng(11)
+    clump = (np.float32(0.5) + np.float32(0.004) * rng.random((1500, 3), dtype=np.float32)).astype(np.float32)
+    pts = np.concatenate([synthetic.room(6, 138500), clump])
+    pts = pts[rng.permutation(pts.shape[0])]
+    ids = np.zeros(pts.shape[0], np.int32)
+    g = gpu_neighborhood(ops, pts, ids, pts, ids, 0.05, 1, use_table=True)
+    ends, neigh = g["ends"], g["neighbors"]
+    counts = np.diff(ends, prepend=0)
+    assert ends[-1] == neigh.shape[0] and counts.max() >= 1500
+    assert np.array_equal(neigh[:, 1], np.repeat(np.arange(pts.shape[0]), counts))
+    fwd = neigh[:, 0].astype(np.int64) * pts.shape[0] + neigh[:, 1]
+    bwd = neigh[:, 1].astype(np.int64) * pts.shape[0] + neigh[:, 0]
+    assert np.array_equal(np.sort(fwd), np.sort(bwd))
+    in_clump = np.flatnonzero(np.all(np.abs(pts - np.float32(0.502)) < 0.0021, axis=1))
+    assert in_clump.size >= 1500
+    p64 = pts.astype(np.float64)
+    for s_i in np.concatenate([in_clump[:60], rng.choice(pts.shape[0], 200, replace=False)]):
+        dist = np.linalg.norm(p64 - p64[s_i], axis=1)
+        sure, maybe = dist < 0.05 * (1 - 1e-6), dist < 0.05 * (1 + 1e-6)
+        mine = neigh[(ends[s_i] - counts[s_i]):ends[s_i], 0]
+        assert np.count_nonzero(sure) <= mine.size <= np.count_nonzero(maybe), s_i
+        assert np.all(maybe[mine]) and np.all(np.isin(np.flatnonzero(sure), mine)), s_i
+
+
 def test_pair_count_beyond_32_bits_is_an_error(ops):
     # 50 000 points inside one search radius are 2.5e9 pairs: the offsets are 32-bit as in the reference, so the
     # search refuses instead of returning wrapped offsets
