@@ -498,7 +498,7 @@ def main():
         f_n, f_ms = s_kernels.get("nb_fill", (0, 0.0))
         f_avg = f_ms / max(f_n, 1)
         s_gbps = s_bytes / (f_avg * 1e-3) / 1e9 if f_n else 0.0
-        roofline_nb = {"kernel": "neighbors_kernel<fill>", "workload": "config 4: %d room points, radius 0.05" % n_s,
+        roofline_nb = {"kernel": "neighbors_fill_masks_kernel", "workload": "config 4: %d room points, radius 0.05" % n_s,
                        "bound": "hbm", "achieved": s_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                        "frac": s_gbps / HBM_PEAK_GBPS,
                        "traffic": traffic("scene_%d" % n_s, "neighbors_fill"), "bytes_per_launch": s_bytes,
