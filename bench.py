@@ -167,9 +167,9 @@ def config3_leg(lib, dev, timed, steps, warmup, with_cpu):
                        "15 kernel points, Cin 128 -> Cout 256, fp32",
            "points": m, "pairs": pairs, "ms_per_step": ms, "points_per_sec": m / (ms * 1e-3),
            "kernels_us": {kk: round(1e3 * v[1] / v[0], 2) for kk, v in kernels.items()},
-           "roofline": {"kernel": "gemm_f32_mfma_kernel", "bound": "mfma", "achieved": tflops,
+           "roofline": {"kernel": "gemm_f32_full_tiles_kernel (all three products)", "bound": "mfma", "achieved": tflops,
                         "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_FP32_PEAK_TFLOPS,
-                        "traffic": traffic("config3", "gemm_f32_mfma_kernel"), "flops_per_launch": flops,
+                        "traffic": traffic("config3", "contraction_f32"), "flops_per_launch": flops,
                         "avg_launch_ms": g_avg, "launches": g_n,
                         "shapes": "P[65536,1920] W[1920,256]; P^T dOut; dOut W^T (mean of the three launches)"}}
     log("config 3: %d pairs, step %.3f ms" % (pairs, ms),
@@ -428,9 +428,9 @@ def main():
     gemm_n, gemm_total_ms = conv_kernels.get("gemm", (0, 0.0))
     gemm_avg_ms = gemm_total_ms / max(gemm_n, 1)
     gemm_tflops = gemm_flops / (gemm_avg_ms * 1e-3) / 1e12 if gemm_n else 0.0
-    roofline = {"kernel": "gemm_f32_mfma_kernel", "bound": "mfma", "achieved": gemm_tflops,
+    roofline = {"kernel": "gemm_f32_full_tiles_kernel (P W, Pt dOut), gemm_f32_mfma_kernel (dOut Wt)", "bound": "mfma", "achieved": gemm_tflops,
                 "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": gemm_tflops / MFMA_FP32_PEAK_TFLOPS,
-                "traffic": traffic("config2", "gemm_f32_mfma_kernel"), "flops_per_launch": gemm_flops, "avg_launch_ms": gemm_avg_ms,
+                "traffic": traffic("config2", "contraction_f32"), "flops_per_launch": gemm_flops, "avg_launch_ms": gemm_avg_ms,
                 "launches": gemm_n}
 
     # ---- the two projection kernels against HBM bandwidth.  Algorithmic bytes, forward: pairs 8T + offsets 4M +
