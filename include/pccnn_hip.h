@@ -415,6 +415,14 @@ int pccnn_timing_read(int id, int64_t *h_launches, double *h_total_ms);
  * whose traffic is known (4*count bytes each way), give the scale for the same counters on the other kernels. */
 int pccnn_calibration_copy(const float *src, float *dst, int64_t count, void *stream);
 
+/* Row permutation, used where the reference's Python gathers with torch.index_select (e.g. pccnn_lib/pc/Grid.py:68-70
+ * for the sorted copies): dst f32[rows, row_floats] = src[index[i], :], index i32[rows] with values in
+ * [0, src_rows) (a row whose index is outside is left untouched).  And the inverse of a permutation of 0..n-1:
+ * inverse[perm[i]] = i. */
+int pccnn_gather_rows_f32(const float *src, const int32_t *index, float *dst, int64_t rows, int row_floats,
+                          int64_t src_rows, void *stream);
+int pccnn_invert_permutation_i32(const int32_t *perm, int32_t *inverse, int64_t n, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

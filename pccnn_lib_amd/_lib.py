@@ -83,6 +83,8 @@ SIGNATURES = {
     "pccnn_timing_name": (ctypes.c_char_p, [I32]),
     "pccnn_timing_read": (I32, [I32, P, P]),
     "pccnn_calibration_copy": (I32, [P, P, I64, P]),
+    "pccnn_gather_rows_f32": (I32, [P, P, P, I64, I32, I64, P]),
+    "pccnn_invert_permutation_i32": (I32, [P, P, I64, P]),
     "pccnn_gemm_f32": (I32, [P, P, P, I64, I64, I64, I32, I32, I64, I64, I64, I32, I64, I64, I64, I32, P, SZ, P]),
 }
 

@@ -137,6 +137,63 @@ extern "C" int pccnn_calibration_copy(const float *src, float *dst, int64_t coun
     return PCCNN_OK;
 }
 
+// ------------------------------------------------------------------- row permutation
+// dst[i, :] = src[index[i], :] for rows of `row_floats` floats: one lane per 16 bytes when the rows allow it.
+template <typename V>
+__global__ void __launch_bounds__(256)
+gather_rows_kernel(const V *__restrict__ src, const int32_t *__restrict__ index, V *__restrict__ dst, int64_t rows,
+                   int per_row, int64_t src_rows)
+{
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= rows * per_row) return;
+    const int64_t r = e / per_row;
+    const int c = (int)(e % per_row);
+    const int64_t from = index[r];
+    if (from >= 0 && from < src_rows) dst[e] = src[from * per_row + c];
+}
+
+extern "C" int pccnn_gather_rows_f32(const float *src, const int32_t *index, float *dst, int64_t rows, int row_floats,
+                                     int64_t src_rows, void *stream)
+{
+    PCCNN_REQUIRE(rows >= 0 && row_floats >= 1 && src_rows >= 0, PCCNN_ERR_INVALID,
+                  "pccnn_gather_rows_f32: rows=%lld row_floats=%d src_rows=%lld", (long long)rows, row_floats,
+                  (long long)src_rows);
+    if (rows == 0) return PCCNN_OK;
+    PCCNN_REQUIRE(src && index && dst, PCCNN_ERR_INVALID, "pccnn_gather_rows_f32: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    const bool wide = row_floats % 4 == 0 && (uintptr_t)src % 16 == 0 && (uintptr_t)dst % 16 == 0;
+    const int per_row = wide ? row_floats / 4 : row_floats;
+    const int64_t blocks = pccnn_ceil_div(rows * per_row, 256);
+    PCCNN_REQUIRE(blocks < (1ll << 31), PCCNN_ERR_UNSUPPORTED, "pccnn_gather_rows_f32: too many elements");
+    if (wide)
+        gather_rows_kernel<float4><<<(unsigned)blocks, 256, 0, s>>>((const float4 *)src, index, (float4 *)dst, rows,
+                                                                   per_row, src_rows);
+    else
+        gather_rows_kernel<float><<<(unsigned)blocks, 256, 0, s>>>(src, index, dst, rows, per_row, src_rows);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
+// inverse[perm[i]] = i
+__global__ void __launch_bounds__(256)
+invert_permutation_kernel(const int32_t *__restrict__ perm, int32_t *__restrict__ inverse, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int64_t to = perm[i];
+    if (to >= 0 && to < n) inverse[to] = (int32_t)i;
+}
+
+extern "C" int pccnn_invert_permutation_i32(const int32_t *perm, int32_t *inverse, int64_t n, void *stream)
+{
+    PCCNN_REQUIRE(n >= 0 && n < (1ll << 31), PCCNN_ERR_INVALID, "pccnn_invert_permutation_i32: n=%lld", (long long)n);
+    if (n == 0) return PCCNN_OK;
+    PCCNN_REQUIRE(perm && inverse, PCCNN_ERR_INVALID, "pccnn_invert_permutation_i32: null pointer");
+    invert_permutation_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, (hipStream_t)stream>>>(perm, inverse, n);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
 // ------------------------------------------------------------------- scan
 // Three launches: per-tile inclusive scan + tile totals, scan of the totals by one
 // workgroup, add of the tile prefix.  Tiles are SCAN_TILE consecutive elements.

@@ -37,6 +37,12 @@ class Grid(object):
             self.sorted_ids_i64_ = self.sorted_ids_i32_.to(torch.int64)
         return self.sorted_ids_i64_
 
+    def inverse_sorted_ids(self):
+        """int32 [N]: position of every point in the key order (the inverse of ``sorted_ids_``), made on first use."""
+        if getattr(self, "inverse_sorted_ids_", None) is None:
+            self.inverse_sorted_ids_ = pccnn_lib_ops.invert_permutation(self.sorted_ids_i32_)
+        return self.inverse_sorted_ids_
+
     def num_cells_host(self):
         """``num_cells_`` as a list of ints.  When the cell size came from host values, the same fp32 arithmetic
         (subtract, IEEE divide, truncate, + 1, maximum over the clouds) runs in numpy on the box's host copy, which is

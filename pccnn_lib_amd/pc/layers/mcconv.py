@@ -3,7 +3,7 @@ import math
 import torch
 
 from ...op_wrappers import ComputeMCConv, ComputeMCConvWeightVar
-from .conv_base import IConvLayer, IConvLayerFactory, mirror_if_needed
+from .conv_base import IConvLayer, IConvLayerFactory, mirror_if_needed, point_side
 
 
 class MCConv(IConvLayer):
@@ -13,6 +13,8 @@ class MCConv(IConvLayer):
     receives it multiplied by the product of the radii (MCConv.py:93-94).  ``contraction_`` ("f32" by default;
     "bf16" = bf16 operands with fp32 accumulation, a mode the reference does not have) selects the precision of the
     [M, H*Cin] x [H*Cin, Cout] products of the forward and backward pass."""
+
+    key_order_capable_ = True
 
     def __init__(self, p_dims, p_in_features, p_out_features, p_hidden_size, p_num_mlps=1,
                  p_constant_weight_var=True, p_const_var_value=1.0):
@@ -37,17 +39,21 @@ class MCConv(IConvLayer):
         if p_pc_in.pts_unnorm_pdf_ is None:
             raise RuntimeError("MCConv: the input point cloud has no density; call compute_pdf(bandwidth) first")
         cur_pdf = p_pc_in.pts_unnorm_pdf_ * torch.prod(p_radius)
+        if torch.is_grad_enabled() and cur_pdf.requires_grad:
+            pts, pairs, pdf, feats = p_pc_in.pts_, p_neighborhood.neighbors_, cur_pdf, p_in_features
+        else:
+            pts, pairs, pdf, feats = point_side(p_pc_in, p_neighborhood, cur_pdf, p_in_features)
         if self.wamup_state_ and self.use_const_variance_init_:
             variance = ComputeMCConvWeightVar.apply(
-                p_pc_in.pts_, cur_pdf, p_in_features, p_pc_out.pts_, p_neighborhood.neighbors_,
+                pts, pdf, feats, p_pc_out.pts_, pairs,
                 p_neighborhood.start_ids_, p_radius, self.proj_axis_, self.proj_bias_) * self.num_mlps_
             self.__update_weight_var__(1.0 / variance.item())
             stdv = math.sqrt(self.out_constant_variance_ / self.accum_weight_var_)
             self.conv_weights_.data.normal_(0.0, stdv)
         return ComputeMCConv.apply(
-            p_pc_in.pts_, cur_pdf, p_in_features, p_pc_out.pts_, p_neighborhood.neighbors_,
+            pts, pdf, feats, p_pc_out.pts_, pairs,
             p_neighborhood.start_ids_, p_radius, self.proj_axis_, self.proj_bias_, self.conv_weights_,
-            mirror_if_needed(p_neighborhood, p_pc_in.pts_, cur_pdf), self.contraction_)
+            mirror_if_needed(p_neighborhood, pts, pdf), self.contraction_)
 
 
 class MCConvFactory(IConvLayerFactory):

@@ -11,11 +11,16 @@ class Neighborhood(object):
     The search radius is the grid's cell size (Neighborhood.py:44).  The sorted-index -> original-index
     remap of the reference (:47-53) happens inside the native fill pass."""
 
-    def __init__(self, p_grid, p_samples, p_max_neighbors=0):
+    def __init__(self, p_grid, p_samples, p_max_neighbors=0, p_key_order=False):
+        """``p_key_order`` (not in the reference): keep the pair list with column 0 = index into the grid's sorted
+        copy of the cloud, and make ``neighbors_`` from it only if somebody asks.  For a consumer that can work on
+        the sorted copy (``layers.conv_base.point_side``)."""
         self.grid_ = p_grid
         self.samples_ = p_samples
         self.max_neighbors_ = p_max_neighbors
         self.mirror_ = False            # not computed yet; None = the neighborhood is not symmetric
+        self.neighbors_key_order_ = None
+        self.neighbors_original_ = None
         grid = p_grid
         with torch.no_grad():
             sample_pts = p_samples.pts_.detach()
@@ -27,10 +32,31 @@ class Neighborhood(object):
                 sample_keys = pccnn_lib_ops.compute_keys(sample_pts, p_samples.batch_ids_, grid.bounding_box_.min_,
                                                          grid.num_cells_, grid.cell_size_)
                 sorted_keys, order, sorted_pts = pccnn_lib_ops.sort_keys(sample_keys, grid.key_bits(), sample_pts)
-            self.neighbors_, self.start_ids_ = pccnn_lib_ops.find_neighbors_ex(
+            key_order = bool(p_key_order) and grid.sorted_pts_.shape[1] == 3
+            neighbors, self.start_ids_ = pccnn_lib_ops.find_neighbors_ex(
                 grid.sorted_pts_, grid.sorted_cell_ids_, sorted_pts, sorted_keys, grid.grid_ds_, grid.num_cells_,
-                grid.cell_size_, p_max_neighbors, sample_order=order, point_remap=grid.sorted_ids_i32_,
-                cell_table=grid.cell_table_, samples_presorted=True)
+                grid.cell_size_, p_max_neighbors, sample_order=order,
+                point_remap=None if key_order else grid.sorted_ids_i32_, cell_table=grid.cell_table_,
+                samples_presorted=True)
+            if key_order:
+                self.neighbors_key_order_ = neighbors
+            else:
+                self.neighbors_original_ = neighbors
+
+    @property
+    def neighbors_(self):
+        """int32 [T, 2] (original point index, sample index) as in the reference."""
+        if self.neighbors_original_ is None:
+            with torch.no_grad():
+                pairs = self.neighbors_key_order_
+                point = torch.index_select(self.grid_.sorted_ids_i32_, 0, pairs[:, 0].to(torch.int64))
+                self.neighbors_original_ = torch.stack((point, pairs[:, 1]), dim=1)
+        return self.neighbors_original_
+
+    @neighbors_.setter
+    def neighbors_(self, p_value):
+        self.neighbors_original_ = p_value
+        self.neighbors_key_order_ = None
 
     def mirror(self):
         """int32 [T]: for every pair (a, b) the index of pair (b, a), when the samples are the gridded cloud

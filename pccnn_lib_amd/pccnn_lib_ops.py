@@ -584,6 +584,31 @@ def _mirror_arg(name, mirror, neigh, pts, samples):
     return _ptr(mirror)
 
 
+def gather_rows(rows, index):
+    """rows[index] for float32 rows [N] or [N, C] and an int32 index [M] (no counterpart in the reference op module;
+    what its Python does with torch.index_select)."""
+    _chk(rows, "gather_rows: rows", torch.float32)
+    _chk(index, "gather_rows: index", torch.int32, 1, rows.device)
+    width = 1
+    for extent in rows.shape[1:]:
+        width *= int(extent)
+    out = torch.empty((index.shape[0],) + tuple(rows.shape[1:]), dtype=torch.float32, device=rows.device)
+    if index.shape[0] > 0 and width > 0:
+        if rows.shape[0] == 0:
+            raise RuntimeError("gather_rows: an index into an empty tensor")
+        _lib.call("pccnn_gather_rows_f32", _ptr(rows), _ptr(index), _ptr(out), index.shape[0], width, rows.shape[0],
+                  _stream())
+    return out
+
+
+def invert_permutation(perm):
+    """int32 [N] with inverse[perm[i]] = i, for a permutation of 0 .. N-1."""
+    _chk(perm, "invert_permutation: perm", torch.int32, 1)
+    inverse = torch.empty_like(perm)
+    _lib.call("pccnn_invert_permutation_i32", _ptr(perm), _ptr(inverse), perm.shape[0], _stream())
+    return inverse
+
+
 def mirror_pairs(neigh, ends):
     """Mirror index of a symmetric neighborhood (samples are the points, uncapped search): int32 [T] with the
     index of pair (b, a) for every pair (a, b), or None when some pair has no mirror.  Reads one int back."""

@@ -267,6 +267,44 @@ def test_config5_hierarchy_8x100k_properties(oracle):
         assert relerr(p(got_g[i]), exp_g[i]) < 3e-3, name
 
 
+@pytest.mark.parametrize("pooled", [True, False])
+def test_mcconv_on_the_sorted_copy_of_a_large_cloud_equals_the_plain_run(monkeypatch, pooled):
+    # From conv_base.KEY_ORDER_MIN_POINTS input points on, an MCConv layer that builds its own neighborhood keeps the
+    # pair list in key order and runs on the grid's sorted copy of the cloud (features and densities permuted once).
+    # With the threshold lowered: the same outputs (the sums run over the same pairs in the same order) and the same
+    # gradients as the plain run, and `neighbors_` of the returned neighborhood is still the reference's list.
+    import pccnn_lib_amd as lib
+    from pccnn_lib_amd.pc.layers import conv_base
+    torch.manual_seed(3)
+    pts = t(np.concatenate([synthetic.room(20 + b, 6000) / 10.0 for b in range(3)]).astype(np.float32))
+    ids = t(np.repeat(np.arange(3, dtype=np.int32), 6000))
+    layer = lib.pc.layers.MCConv(3, 8, 32, 8).to(DEV)
+    feats0 = torch.randn(pts.shape[0], 8, device=DEV)
+    out_grads = torch.randn(1, 32, device=DEV)
+
+    def run(min_points):
+        monkeypatch.setattr(conv_base, "KEY_ORDER_MIN_POINTS", min_points)
+        pc = lib.pc.Pointcloud(pts, ids)
+        pc.compute_pdf(0.01)
+        pc_out = pc
+        if pooled:
+            pool = lib.pc.PointPooling(pc, 0.05)
+            pc_out = lib.pc.Pointcloud(pool.pool_tensor(pc.pts_), pool.pool_tensor(pc.batch_ids_))
+        feats = feats0.clone().requires_grad_(True)
+        out, nbh = layer(pc, pc_out, feats, 0.1)
+        grads = torch.autograd.grad((out * out_grads).sum(), [feats, layer.conv_weights_, layer.proj_axis_,
+                                                               layer.proj_bias_])
+        return out.detach(), grads, nbh
+
+    out_a, grads_a, nbh_a = run(10 ** 9)
+    out_b, grads_b, nbh_b = run(0)
+    assert nbh_a.neighbors_key_order_ is None and nbh_b.neighbors_key_order_ is not None
+    assert torch.equal(out_a, out_b)
+    for ga, gb in zip(grads_a, grads_b):
+        assert relerr(gb.cpu().numpy(), ga.cpu().numpy()) < 1e-5
+    assert torch.equal(nbh_a.neighbors_, nbh_b.neighbors_) and torch.equal(nbh_a.start_ids_, nbh_b.start_ids_)
+
+
 def test_projection_with_more_than_two_to_the_31_elements(ops):
     # Maximum sizes: 2.2 million samples x 64 features x 16 hidden units put 2.25e9 floats (9 GB) into the projection
     # and as many into its gradient, past what 32-bit element offsets reach.  No oracle runs at this size; the check
