@@ -296,6 +296,21 @@ def test_one_lane_walk_with_more_candidates_than_its_masks_hold(ops):
         assert np.all(maybe[mine]) and np.all(np.isin(np.flatnonzero(sure), mine)), s_i
 
 
+def test_row_gather_and_permutation_inverse(ops):
+    # what the reference's Python does with torch.index_select: rows of 1, 3, 8 and 33 floats (16-byte and 4-byte
+    # paths), an index with repeats, and the inverse of a permutation
+    rng = np.random.default_rng(2)
+    for width in (None, 3, 8, 33):
+        src = rng.normal(size=(5000,) if width is None else (5000, width)).astype(np.float32)
+        index = rng.integers(0, 5000, 7001).astype(np.int32)
+        got = ops.gather_rows(t(src), t(index)).cpu().numpy()
+        assert np.array_equal(got, src[index])
+    perm = rng.permutation(100001).astype(np.int32)
+    inverse = ops.invert_permutation(t(perm)).cpu().numpy()
+    assert np.array_equal(inverse[perm], np.arange(100001))
+    assert ops.gather_rows(t(np.zeros((4, 8), np.float32)), t(np.zeros(0, np.int32))).shape == (0, 8)
+
+
 def test_pair_count_beyond_32_bits_is_an_error(ops):
     # 50 000 points inside one search radius are 2.5e9 pairs: the offsets are 32-bit as in the reference, so the
     # search refuses instead of returning wrapped offsets
