@@ -180,3 +180,29 @@ def test_the_op_module_imports_under_the_reference_name():
             "assert all(callable(getattr(pccnn_lib_ops, n)) for n in pccnn_lib_ops.REFERENCE_NAMES)\n")
     res = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True, timeout=300)
     assert res.returncode == 0, res.stderr
+
+
+def test_point_side_keeps_the_plain_route_unless_the_pairs_are_in_key_order():
+    # host logic of the layers (no GPU): a convolution reads the cloud's own tensors and the reference's pair list
+    # unless its neighborhood kept the pairs in key order, belongs to this cloud, and no gradient goes to the positions
+    import types
+    import torch
+    from pccnn_lib_amd.pc.layers import conv_base
+    feats = torch.ones(4, 2)
+    cloud = types.SimpleNamespace(pts_=torch.zeros(4, 3))
+    plain = types.SimpleNamespace(neighbors_key_order_=None, neighbors_=torch.zeros(2, 2, dtype=torch.int32),
+                                  grid_=types.SimpleNamespace(pointcloud_=cloud))
+    pts, pairs, moved = conv_base.point_side(cloud, plain, feats)
+    assert pts is cloud.pts_ and pairs is plain.neighbors_ and moved is feats
+    other = types.SimpleNamespace(pts_=torch.zeros(4, 3))
+    keyed = types.SimpleNamespace(neighbors_key_order_=torch.ones(2, 2, dtype=torch.int32),
+                                  neighbors_=torch.zeros(2, 2, dtype=torch.int32),
+                                  grid_=types.SimpleNamespace(pointcloud_=other))
+    pts, pairs, moved = conv_base.point_side(cloud, keyed, feats)             # a neighborhood of another cloud
+    assert pts is cloud.pts_ and pairs is keyed.neighbors_ and moved is feats
+    wanted = types.SimpleNamespace(pts_=torch.zeros(4, 3, requires_grad=True))
+    keyed.grid_.pointcloud_ = wanted
+    pts, pairs, moved = conv_base.point_side(wanted, keyed, feats)            # positions that want a gradient
+    assert pts is wanted.pts_ and pairs is keyed.neighbors_ and moved is feats
+    layer = conv_base.IConvLayer(3, 2, 2)
+    assert layer.key_order_capable_ is False and conv_base.KEY_ORDER_MIN_POINTS >= 100000
