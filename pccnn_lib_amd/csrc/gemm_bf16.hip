@@ -248,7 +248,15 @@ bg_splitk_reduce_kernel(const float *__restrict__ partial, GemmBf16Args g, int b
         const int64_t bi = i / per, e = i % per;
         const float *src = partial + bi * g.split_k * per + e;
         float s = 0.0f;
-        for (int k = 0; k < g.split_k; ++k) s += src[(int64_t)k * per];
+        int k = 0;
+        for (; k + 8 <= g.split_k; k += 8) {                        // eight loads in flight, added in order
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = src[(int64_t)(k + u) * per];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += v[u];
+        }
+        for (; k < g.split_k; ++k) s += src[(int64_t)k * per];
         g.c[bi * g.stride_c + (e / g.cols) * g.ldc + (e % g.cols)] = s;
     }
 }
