@@ -7,7 +7,7 @@ import time
 
 from ...op_wrappers import ComputeKPConv, ComputeKPConvWeightVar, ComputeKPConvN, ComputeKPConvNWeightVar, \
     ComputePCCNN, ComputePCCNNWeightVar
-from .conv_base import IConvLayer, IConvLayerFactory, mirror_if_needed
+from .conv_base import IConvLayer, IConvLayerFactory, mirror_if_needed, point_side
 from .kernel_points import kernel_pts_dict
 
 
@@ -41,6 +41,8 @@ class KPConv(IConvLayer):
     Buffers ``kernel_pts_`` [K, D] and ``sigma_``, parameter ``conv_weights_`` [K*Cin, Cout] keep the
     reference's names and shapes, so its state dicts load."""
 
+    key_order_capable_ = True
+
     def __init__(self, p_dims, p_in_features, p_out_features, p_num_kernel_pts, p_constant_weight_var=True,
                  p_const_var_value=1.0):
         super(KPConv, self).__init__(p_dims, p_in_features, p_out_features, p_constant_weight_var,
@@ -62,17 +64,18 @@ class KPConv(IConvLayer):
     def __compute_convolution__(self, p_pc_in, p_pc_out, p_in_features, p_radius, p_neighborhood):
         if self.sigma_cpu_ is None:
             self.sigma_cpu_ = self.sigma_.item()
+        pts, pairs, feats = point_side(p_pc_in, p_neighborhood, p_in_features)
         if self.wamup_state_ and self.use_const_variance_init_:
             variance = ComputeKPConvWeightVar.apply(
-                p_pc_in.pts_, p_in_features, p_pc_out.pts_, p_neighborhood.neighbors_, p_neighborhood.start_ids_,
+                pts, feats, p_pc_out.pts_, pairs, p_neighborhood.start_ids_,
                 p_radius, self.kernel_pts_, self.sigma_cpu_)
             self.__update_weight_var__(1.0 / variance.item())
             stdv = math.sqrt(self.out_constant_variance_ / self.accum_weight_var_)
             self.conv_weights_.data.normal_(0.0, stdv)
         return ComputeKPConv.apply(
-            p_pc_in.pts_, p_in_features, p_pc_out.pts_, p_neighborhood.neighbors_, p_neighborhood.start_ids_,
+            pts, feats, p_pc_out.pts_, pairs, p_neighborhood.start_ids_,
             p_radius, self.kernel_pts_, self.sigma_cpu_, self.conv_weights_,
-            mirror_if_needed(p_neighborhood, p_pc_in.pts_), self.contraction_)
+            mirror_if_needed(p_neighborhood, pts), self.contraction_)
 
 
 class KPConvFactory(IConvLayerFactory):
@@ -94,6 +97,7 @@ class _DensityKernelPointConv(IConvLayer):
     sigma_scale_ = 1.0
     conv_op_ = None
     weight_var_op_ = None
+    key_order_capable_ = True
 
     def __init__(self, p_dims, p_in_features, p_out_features, p_num_kernel_pts, p_constant_weight_var=True,
                  p_const_var_value=1.0):
@@ -116,17 +120,21 @@ class _DensityKernelPointConv(IConvLayer):
         cur_pdf = p_pc_in.pts_unnorm_pdf_ * torch.prod(p_radius)
         if self.sigma_cpu_ is None:
             self.sigma_cpu_ = self.sigma_.item()
+        if torch.is_grad_enabled() and cur_pdf.requires_grad:
+            pts, pairs, pdf, feats = p_pc_in.pts_, p_neighborhood.neighbors_, cur_pdf, p_in_features
+        else:
+            pts, pairs, pdf, feats = point_side(p_pc_in, p_neighborhood, cur_pdf, p_in_features)
         if self.wamup_state_ and self.use_const_variance_init_:
             variance = self.weight_var_op_.apply(
-                p_pc_in.pts_, cur_pdf, p_in_features, p_pc_out.pts_, p_neighborhood.neighbors_,
+                pts, pdf, feats, p_pc_out.pts_, pairs,
                 p_neighborhood.start_ids_, p_radius, self.kernel_pts_, self.sigma_cpu_)
             self.__update_weight_var__(1.0 / variance.item())
             stdv = math.sqrt(self.out_constant_variance_ / self.accum_weight_var_)
             self.conv_weights_.data.normal_(0.0, stdv)
         return self.conv_op_.apply(
-            p_pc_in.pts_, cur_pdf, p_in_features, p_pc_out.pts_, p_neighborhood.neighbors_, p_neighborhood.start_ids_,
+            pts, pdf, feats, p_pc_out.pts_, pairs, p_neighborhood.start_ids_,
             p_radius, self.kernel_pts_, self.sigma_cpu_, self.conv_weights_,
-            mirror_if_needed(p_neighborhood, p_pc_in.pts_, cur_pdf))
+            mirror_if_needed(p_neighborhood, pts, pdf))
 
 
 class KPConvN(_DensityKernelPointConv):

@@ -267,6 +267,36 @@ def test_config5_hierarchy_8x100k_properties(oracle):
         assert relerr(p(got_g[i]), exp_g[i]) < 3e-3, name
 
 
+@pytest.mark.parametrize("kind", ["KPConv", "KPConvN"])
+def test_kernel_point_layers_on_the_sorted_copy_equal_the_plain_run(monkeypatch, kind):
+    # the same for the kernel-point layers (with and without the density)
+    import pccnn_lib_amd as lib
+    from pccnn_lib_amd.pc.layers import conv_base
+    torch.manual_seed(4)
+    pts = t(np.concatenate([synthetic.room(30 + b, 5000) / 10.0 for b in range(2)]).astype(np.float32))
+    ids = t(np.repeat(np.arange(2, dtype=np.int32), 5000))
+    layer = getattr(lib.pc.layers, kind)(3, 8, 16, 16).to(DEV)
+    feats0 = torch.randn(pts.shape[0], 8, device=DEV)
+
+    def run(min_points):
+        monkeypatch.setattr(conv_base, "KEY_ORDER_MIN_POINTS", min_points)
+        pc = lib.pc.Pointcloud(pts, ids)
+        pc.compute_pdf(0.01)
+        pool = lib.pc.PointPooling(pc, 0.05)
+        pc_out = lib.pc.Pointcloud(pool.pool_tensor(pc.pts_), pool.pool_tensor(pc.batch_ids_))
+        feats = feats0.clone().requires_grad_(True)
+        out, nbh = layer(pc, pc_out, feats, 0.1)
+        grads = torch.autograd.grad(out.sum(), [feats, layer.conv_weights_])
+        return out.detach(), grads, nbh
+
+    out_a, grads_a, nbh_a = run(10 ** 9)
+    out_b, grads_b, nbh_b = run(0)
+    assert nbh_a.neighbors_key_order_ is None and nbh_b.neighbors_key_order_ is not None
+    assert torch.equal(out_a, out_b)
+    for ga, gb in zip(grads_a, grads_b):
+        assert relerr(gb.cpu().numpy(), ga.cpu().numpy()) < 1e-5
+
+
 @pytest.mark.parametrize("pooled", [True, False])
 def test_mcconv_on_the_sorted_copy_of_a_large_cloud_equals_the_plain_run(monkeypatch, pooled):
     # From conv_base.KEY_ORDER_MIN_POINTS input points on, an MCConv layer that builds its own neighborhood keeps the
