@@ -31,6 +31,7 @@ struct GemmArgs {
     int split_k;
     int64_t k_chunk;       // inner elements per split (multiple of GT_K)
     int aligned;           // pointers, leading dimensions and batch strides allow float4 loads
+    int whole_units;       // aligned, and no float4 unit of a tile straddles the edge of its operand
     int tiles_x, tiles_y;  // workgroup tiles along the columns / rows
     int64_t total_wg;      // tiles_x * tiles_y * batch * split_k
 };
@@ -44,8 +45,10 @@ struct GemmArgs {
 
 // Global -> registers for one 128 x 16 operand tile.  `KCONTIG`: the reduction index is the
 // contiguous one in memory (element (x, k) at p[x * ld + k]); otherwise element (x, k) at p[k * ld + x].
-// `FAST`: the tile is fully inside the matrix and 16-byte aligned, so it is read with float4 loads.
-template <bool KCONTIG, bool FAST, int TILE_X>
+// MODE 1: the tile is fully inside the matrix and 16-byte aligned, so it is read with float4 loads and no checks;
+// MODE 2: float4 loads, a unit outside the matrix reads as zeros (the host checks that no unit straddles an edge:
+// the extents along the units are multiples of 4); MODE 0: element by element.
+template <bool KCONTIG, int MODE, int TILE_X>
 __device__ __forceinline__ void tile_load(const float *__restrict__ p, int64_t ld, int64_t x0, int64_t x_end,
                                           int64_t k0, int64_t k_end, float4 (&r)[TILE_X / 64 * (GT_K / 16)])
 {
@@ -55,8 +58,12 @@ __device__ __forceinline__ void tile_load(const float *__restrict__ p, int64_t l
         int64_t x, k;
         if (KCONTIG) { x = x0 + idx / (GT_K / 4); k = k0 + (idx % (GT_K / 4)) * 4; }
         else { k = k0 + idx / (TILE_X / 4); x = x0 + (idx % (TILE_X / 4)) * 4; }
-        if (FAST) {
+        if (MODE == 1) {
             r[i] = KCONTIG ? *(const float4 *)(p + x * ld + k) : *(const float4 *)(p + k * ld + x);
+        } else if (MODE == 2) {
+            r[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (x < x_end && k < k_end)
+                r[i] = KCONTIG ? *(const float4 *)(p + x * ld + k) : *(const float4 *)(p + k * ld + x);
         } else {
             float v[4];
 #pragma unroll
@@ -93,7 +100,7 @@ __device__ __forceinline__ void tile_store(float (*lds)[GT_LD], const float4 (&r
 // The k loop of one workgroup tile.  Global loads run two or three tiles ahead of the MFMAs (one or two register
 // sets, then the free LDS buffer); inside a tile the LDS fragments of sub-step ks+1 are read before the MFMAs of
 // sub-step ks are issued, so the matrix pipe never waits on an LDS round trip.
-template <bool AT, bool BT, bool FAST, int BM>
+template <bool AT, bool BT, int MODE, int BM>
 __device__ __forceinline__ void gemm_tile_loop(const GemmArgs &g, const float *__restrict__ a,
                                                const float *__restrict__ b, int64_t bm, int64_t bn, int64_t k_begin,
                                                int64_t k_end, float (*As)[GT_K][GT_LD], float (*Bs)[GT_K][GT_LD],
@@ -110,30 +117,30 @@ __device__ __forceinline__ void gemm_tile_loop(const GemmArgs &g, const float *_
     // two whole steps of MFMAs to arrive (3 - 4 % on the products of 65 536 x 1024 x 128).  The 128-row tiles keep
     // one set (AHEAD = 2): with two they pass 128 registers, which halves the waves per SIMD and costs 9 %; so does
     // the bounds-checked path of edge tiles.
-    constexpr bool DEEP = FAST && BM == 64;
+    constexpr bool DEEP = MODE == 1 && BM == 64;
     constexpr int AHEAD = DEEP ? 3 : 2;
     float4 ra0[NA], rb0[NB], ra1[DEEP ? NA : 1], rb1[DEEP ? NB : 1];
     const int64_t nk = (k_end - k_begin + GT_K - 1) / GT_K;
     // A stored [rows, inner] (AT = false) has the reduction index contiguous; B stored
     // [inner, cols] (BT = false) has the column index contiguous.
     if (nk > 0) {
-        tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k_begin, k_end, ra0);
-        tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k_begin, k_end, rb0);
+        tile_load<!AT, MODE, BM>(a, g.lda, bm, g.rows, k_begin, k_end, ra0);
+        tile_load<BT, MODE, GT_N>(b, g.ldb, bn, g.cols, k_begin, k_end, rb0);
         tile_store<!AT, BM>(As[0], ra0);
         tile_store<BT, GT_N>(Bs[0], rb0);
     }
     if constexpr (DEEP) {
         if (nk > 1) {
-            tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k_begin + GT_K, k_end, ra1);
-            tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k_begin + GT_K, k_end, rb1);
+            tile_load<!AT, MODE, BM>(a, g.lda, bm, g.rows, k_begin + GT_K, k_end, ra1);
+            tile_load<BT, MODE, GT_N>(b, g.ldb, bn, g.cols, k_begin + GT_K, k_end, rb1);
         }
         if (nk > 2) {
-            tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k_begin + 2 * GT_K, k_end, ra0);
-            tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k_begin + 2 * GT_K, k_end, rb0);
+            tile_load<!AT, MODE, BM>(a, g.lda, bm, g.rows, k_begin + 2 * GT_K, k_end, ra0);
+            tile_load<BT, MODE, GT_N>(b, g.ldb, bn, g.cols, k_begin + 2 * GT_K, k_end, rb0);
         }
     } else if (nk > 1) {
-        tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k_begin + GT_K, k_end, ra0);
-        tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k_begin + GT_K, k_end, rb0);
+        tile_load<!AT, MODE, BM>(a, g.lda, bm, g.rows, k_begin + GT_K, k_end, ra0);
+        tile_load<BT, MODE, GT_N>(b, g.ldb, bn, g.cols, k_begin + GT_K, k_end, rb0);
     }
     __syncthreads();
     // One step: the MFMAs of tile kt from LDS buffer kt & 1.  Behind the first of them tile kt+1, which sits in
@@ -169,8 +176,8 @@ __device__ __forceinline__ void gemm_tile_loop(const GemmArgs &g, const float *_
                 }
                 if (kt + AHEAD < nk) {
                     const int64_t k0 = k_begin + (kt + AHEAD) * GT_K;
-                    tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k0, k_end, ra);
-                    tile_load<BT, FAST, GT_N>(b, g.ldb, bn, g.cols, k0, k_end, rb);
+                    tile_load<!AT, MODE, BM>(a, g.lda, bm, g.rows, k0, k_end, ra);
+                    tile_load<BT, MODE, GT_N>(b, g.ldb, bn, g.cols, k0, k_end, rb);
                 }
             }
             // keep the order written above in the instruction stream: the fragment reads of the next sub-step go
@@ -226,8 +233,9 @@ gemm_f32_mfma_kernel(GemmArgs g, float *__restrict__ partial)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    if (fast) gemm_tile_loop<AT, BT, true, BM>(g, a, b, bm, bn, k_begin, k_end, As, Bs, acc);
-    else gemm_tile_loop<AT, BT, false, BM>(g, a, b, bm, bn, k_begin, k_end, As, Bs, acc);
+    if (fast) gemm_tile_loop<AT, BT, 1, BM>(g, a, b, bm, bn, k_begin, k_end, As, Bs, acc);
+    else if (g.whole_units) gemm_tile_loop<AT, BT, 2, BM>(g, a, b, bm, bn, k_begin, k_end, As, Bs, acc);
+    else gemm_tile_loop<AT, BT, 0, BM>(g, a, b, bm, bn, k_begin, k_end, As, Bs, acc);
 
     // Accumulator layout of the 32x32 MFMA: register v of lane l holds
     // row 8*(v/4) + 4*(l/32) + v%4, column l%32 of the tile.
@@ -512,6 +520,8 @@ extern "C" int pccnn_gemm_f32(const float *a, const float *b, float *c, int64_t 
     g.k_chunk = chunk;
     g.aligned = ((uintptr_t)a % 16 == 0) && ((uintptr_t)b % 16 == 0) && (lda % 4 == 0) && (ldb % 4 == 0) &&
                 (stride_a % 4 == 0) && (stride_b % 4 == 0);
+    // units run along the reduction index where that is contiguous in memory, else along the rows / columns
+    g.whole_units = g.aligned && ((a_trans ? rows : inner) % 4 == 0) && ((b_trans ? inner : cols) % 4 == 0);
     float *partial = nullptr;
     if (split_k > 1) {
         size_t need = (size_t)batch * split_k * rows * cols * sizeof(float);

@@ -28,15 +28,18 @@ struct GemmBf16Args {
     int split_k;
     int64_t k_chunk;       // inner elements per split (multiple of BG_K)
     int aligned;           // pointers, leading dimensions and batch strides allow 16-byte loads
+    int whole_units;       // aligned, and no 16-byte unit of a tile straddles the edge of its operand
     int tiles_x, tiles_y;
     int64_t total_wg;
 };
 
-// Global -> registers for one TILE_X x 32 operand tile.
+// Global -> registers for one TILE_X x 32 operand tile.  MODE 1: 16-byte loads, nothing checked (tile inside the
+// operand); MODE 2: 16-byte loads, a unit outside the operand reads as zeros (units are never cut: the host checks
+// that the operand's extents along the units are multiples of 8); MODE 0: element by element.
 // KCONTIG (element (x, k) at p[x * ld + k]): unit u = (x = u / 4, 8 consecutive k); TILE_X / 64 units per thread.
 // otherwise (element (x, k) at p[k * ld + x]): unit u = (k-pair u / (TILE_X / 8), 8 consecutive x), both rows of
 // the pair; one unit per thread, threads beyond the tile idle.
-template <bool KCONTIG, bool FAST, int TILE_X>
+template <bool KCONTIG, int MODE, int TILE_X>
 __device__ __forceinline__ void bg_tile_load(const uint16_t *__restrict__ p, int64_t ld, int64_t x0, int64_t x_end,
                                              int64_t k0, int64_t k_end, uint4 (&r)[2])
 {
@@ -45,8 +48,11 @@ __device__ __forceinline__ void bg_tile_load(const uint16_t *__restrict__ p, int
         for (int i = 0; i < TILE_X / 64; ++i) {
             const int u = threadIdx.x + 256 * i;
             const int64_t x = x0 + u / 4, k = k0 + (u % 4) * 8;
-            if (FAST) {
+            if (MODE == 1) {
                 r[i] = *(const uint4 *)(p + x * ld + k);
+            } else if (MODE == 2) {
+                r[i] = make_uint4(0, 0, 0, 0);
+                if (x < x_end && k < k_end) r[i] = *(const uint4 *)(p + x * ld + k);
             } else {
                 uint16_t v[8];
 #pragma unroll
@@ -61,8 +67,11 @@ __device__ __forceinline__ void bg_tile_load(const uint16_t *__restrict__ p, int
             const int64_t k = k0 + 2 * (u / (TILE_X / 8)), x = x0 + (u % (TILE_X / 8)) * 8;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                if (FAST) {
+                if (MODE == 1) {
                     r[h] = *(const uint4 *)(p + (k + h) * ld + x);
+                } else if (MODE == 2) {
+                    r[h] = make_uint4(0, 0, 0, 0);
+                    if (x < x_end && k + h < k_end) r[h] = *(const uint4 *)(p + (k + h) * ld + x);
                 } else {
                     uint16_t v[8];
 #pragma unroll
@@ -107,7 +116,7 @@ __device__ __forceinline__ void bg_tile_store(uint32_t (*lds)[BG_LD], const uint
     }
 }
 
-template <bool AT, bool BT, bool FAST, int BM>
+template <bool AT, bool BT, int MODE, int BM>
 __device__ __forceinline__ void bg_tile_loop(const GemmBf16Args &g, const uint16_t *__restrict__ a,
                                              const uint16_t *__restrict__ b, int64_t bm, int64_t bn, int64_t k_begin,
                                              int64_t k_end, uint32_t (*As)[BG_KP][BG_LD], uint32_t (*Bs)[BG_KP][BG_LD],
@@ -123,14 +132,14 @@ __device__ __forceinline__ void bg_tile_loop(const GemmBf16Args &g, const uint16
     const int64_t nk = (k_end - k_begin + BG_K - 1) / BG_K;
     // A stored [rows, inner] (AT = false) and B stored [cols, inner] (BT = true) have the reduction index contiguous.
     if (nk > 0) {
-        bg_tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k_begin, k_end, ra);
-        bg_tile_load<BT, FAST, BG_N>(b, g.ldb, bn, g.cols, k_begin, k_end, rb);
+        bg_tile_load<!AT, MODE, BM>(a, g.lda, bm, g.rows, k_begin, k_end, ra);
+        bg_tile_load<BT, MODE, BG_N>(b, g.ldb, bn, g.cols, k_begin, k_end, rb);
         bg_tile_store<!AT, BM>(As[0], ra);
         bg_tile_store<BT, BG_N>(Bs[0], rb);
     }
     if (nk > 1) {
-        bg_tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k_begin + BG_K, k_end, ra);
-        bg_tile_load<BT, FAST, BG_N>(b, g.ldb, bn, g.cols, k_begin + BG_K, k_end, rb);
+        bg_tile_load<!AT, MODE, BM>(a, g.lda, bm, g.rows, k_begin + BG_K, k_end, ra);
+        bg_tile_load<BT, MODE, BG_N>(b, g.ldb, bn, g.cols, k_begin + BG_K, k_end, rb);
     }
     __syncthreads();
     for (int64_t kt = 0; kt < nk; ++kt) {
@@ -166,8 +175,8 @@ __device__ __forceinline__ void bg_tile_loop(const GemmBf16Args &g, const uint16
                 }
                 if (kt + 2 < nk) {
                     const int64_t k0 = k_begin + (kt + 2) * BG_K;
-                    bg_tile_load<!AT, FAST, BM>(a, g.lda, bm, g.rows, k0, k_end, ra);
-                    bg_tile_load<BT, FAST, BG_N>(b, g.ldb, bn, g.cols, k0, k_end, rb);
+                    bg_tile_load<!AT, MODE, BM>(a, g.lda, bm, g.rows, k0, k_end, ra);
+                    bg_tile_load<BT, MODE, BG_N>(b, g.ldb, bn, g.cols, k0, k_end, rb);
                 }
             }
         }
@@ -212,8 +221,9 @@ gemm_bf16_mfma_kernel(GemmBf16Args g, float *__restrict__ partial)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    if (fast) bg_tile_loop<AT, BT, true, BM>(g, a, b, bm, bn, k_begin, k_end, As, Bs, acc);
-    else bg_tile_loop<AT, BT, false, BM>(g, a, b, bm, bn, k_begin, k_end, As, Bs, acc);
+    if (fast) bg_tile_loop<AT, BT, 1, BM>(g, a, b, bm, bn, k_begin, k_end, As, Bs, acc);
+    else if (g.whole_units) bg_tile_loop<AT, BT, 2, BM>(g, a, b, bm, bn, k_begin, k_end, As, Bs, acc);
+    else bg_tile_loop<AT, BT, 0, BM>(g, a, b, bm, bn, k_begin, k_end, As, Bs, acc);
 
     // Accumulator layout of the 32x32 MFMA: register v of lane l holds
     // row 8*(v/4) + 4*(l/32) + v%4, column l%32 of the tile.
@@ -306,6 +316,8 @@ extern "C" int pccnn_gemm_bf16(const uint16_t *a, const uint16_t *b, float *c, i
     g.k_chunk = chunk;
     g.aligned = ((uintptr_t)a % 16 == 0) && ((uintptr_t)b % 16 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) &&
                 (stride_a % 8 == 0) && (stride_b % 8 == 0);
+    // units run along the reduction index where that is contiguous in memory, else along the rows / columns
+    g.whole_units = g.aligned && ((a_trans ? rows : inner) % 8 == 0) && ((b_trans ? inner : cols) % 8 == 0);
     float *partial = nullptr;
     if (split_k > 1) {
         size_t need = (size_t)batch * split_k * rows * cols * sizeof(float);

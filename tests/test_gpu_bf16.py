@@ -76,7 +76,10 @@ def test_rounding_matches_oracle_bit_for_bit(oracle):
 @pytest.mark.parametrize("rows,cols,inner,at,bt,split", [
     (256, 128, 64, 0, 0, 1), (256, 128, 64, 0, 1, 1), (256, 128, 64, 1, 0, 1), (256, 128, 64, 1, 1, 1),
     (300, 70, 45, 0, 0, 1), (77, 130, 19, 0, 1, 1), (129, 129, 17, 1, 1, 1), (480, 40, 1000, 1, 0, 4),
-    (128, 128, 4096, 1, 0, 8), (2048, 128, 1024, 0, 0, 1), (4096, 1024, 128, 0, 1, 1), (1024, 128, 8192, 1, 0, 64)])
+    (128, 128, 4096, 1, 0, 8), (2048, 128, 1024, 0, 0, 1), (4096, 1024, 128, 0, 1, 1), (1024, 128, 8192, 1, 0, 64),
+    # edge tiles read with whole 16-byte units: the three products of a small hierarchy level
+    (346, 256, 1024, 0, 0, 1), (1024, 256, 346, 1, 0, 1), (346, 1024, 256, 0, 1, 1), (512, 128, 6844, 1, 0, 64),
+    (200, 72, 104, 0, 0, 1), (200, 72, 104, 1, 1, 1), (40, 8, 24, 1, 0, 1)])
 def test_gemm_bf16_against_float64(oracle, rows, cols, inner, at, bt, split):
     from pccnn_lib_amd import _lib
     rng = np.random.default_rng(rows + cols + inner + at + 2 * bt)

@@ -33,7 +33,11 @@ def _cloud(models, batch, num_pts):
     # a split of the reduction, and a reduction too short for that kernel
     (192, 384, 208, 0, 0, 1), (192, 384, 208, 1, 0, 1), (192, 384, 208, 0, 1, 1), (192, 384, 208, 1, 1, 1),
     (32768, 256, 192, 0, 0, 1), (32768, 128, 192, 1, 0, 1), (32768, 256, 192, 0, 1, 1), (32768, 128, 192, 1, 1, 1),
-    (256, 256, 16384, 1, 0, 8), (1024, 128, 8192, 1, 0, 32), (32768, 256, 64, 0, 1, 1)])
+    (256, 256, 16384, 1, 0, 8), (1024, 128, 8192, 1, 0, 32), (32768, 256, 64, 0, 1, 1),
+    # edge tiles read with whole 16-byte units (extents are multiples of the unit, not of the tile): the three
+    # products of a small hierarchy level, forward, weight gradient (with a cut last split) and projection gradient
+    (346, 256, 1024, 0, 0, 1), (1024, 256, 346, 1, 0, 1), (346, 1024, 256, 0, 1, 1), (512, 128, 6844, 1, 0, 64),
+    (200, 72, 104, 0, 0, 1), (200, 72, 104, 1, 1, 1), (36, 8, 12, 1, 0, 1)])
 def test_gemm_against_float64(rows, cols, inner, at, bt, split):
     from pccnn_lib_amd import _lib
     rng = np.random.default_rng(rows + cols + inner)
