@@ -217,6 +217,58 @@ int pccnn_poisson_disk_grid(const float *pts_sorted, const int64_t *sorted_keys,
                             int32_t *selected_out, int32_t *selected_scan_out,
                             void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- host sequences with one read-back -----------------------------------
+ * Chains of the entry points above for the steps whose output size depends on the data; each ends with one small
+ * device-to-host copy on `stream` and returns after it (the calls are synchronous).  The launches are those of the
+ * entry points named.
+ *
+ * pccnn_bounding_box, and the box on the host as well (host_min_out / host_max_out: host memory, f32[batch_size,d]):
+ * what pccnn_lib/pc/Grid.py:26-28 reads when it sizes a grid. */
+int pccnn_bounding_box_host(const float *pts, const int32_t *batch_ids, int64_t n, int d, int batch_size,
+                            float *aabb_min_out, float *aabb_max_out, float *host_min_out, float *host_max_out,
+                            void *stream);
+/* Poisson-disk pooling of a 3-D cloud up to the number of selected points: the grid of cell size `cell_size` over
+ * the cloud (pccnn_grid_build, into the workspace), then pccnn_poisson_disk_grid, i.e. what
+ * pccnn_lib/pc/PointPooling.py:38-65 does between the bounding box and the selected ids.  num_cells_host: the grid
+ * size as three host ints (pccnn_num_cells' arithmetic on the host copy of the box); key_bits as pccnn_sort_keys;
+ * with_cell_table != 0 builds the per-cell table for the walk.  Outputs: perm_out i32[n] (original index of sorted
+ * point i), selected_out / selected_scan_out i32[n] as pccnn_poisson_disk_grid (sorted-index space), *count_out
+ * (host) = number of selected points.  pccnn_compact_selected_remap then writes remap[i] of the selected i,
+ * ascending in i, as i64: with remap = perm_out these are PointPooling's pooling_ids_ (PointPooling.py:66-69). */
+size_t pccnn_pool_poisson_workspace_bytes(int64_t n, int64_t num_pillars, int64_t total_cells);
+int pccnn_pool_poisson_select(const float *pts, const int32_t *batch_ids, int64_t n, int batch_size,
+                              const float *aabb_min, const float *cell_size, const int32_t *num_cells_host,
+                              int key_bits, int with_cell_table, int32_t *perm_out, int32_t *selected_out,
+                              int32_t *selected_scan_out, int64_t *count_out, void *workspace,
+                              size_t workspace_bytes, void *stream);
+int pccnn_compact_selected_remap(const int32_t *selected, const int32_t *selected_scan, const int32_t *remap,
+                                 int64_t n, int64_t *ids_out, void *stream);
+/* pccnn_grid_build for a grid whose size is known on the host (num_cells_host: d host ints): writes that size to
+ * num_cells_out i32[d] on the device, where the kernels read it, instead of computing it there with pccnn_num_cells;
+ * the numbers of pillars and cells follow from it.  with_cell_table != 0 (d == 3 only) fills cell_table_out
+ * i32[cells + 1]. */
+int pccnn_grid_build_sized(const float *pts, const int32_t *batch_ids, const float *aabb_min,
+                           const int32_t *num_cells_host, const float *cell_size, int64_t n, int d, int batch_size,
+                           int key_bits, int with_cell_table, int32_t *num_cells_out, int64_t *keys_out,
+                           int64_t *sorted_keys_out, int32_t *perm_out, float *sorted_pts_out, int32_t *grid_ds_out,
+                           int32_t *cell_table_out, void *workspace, size_t workspace_bytes, void *stream);
+/* A layer's neighborhood up to the pair count (d == 3): pccnn_grid_build_sized over the cloud, keys and key order
+ * of the samples (pccnn_compute_keys + pccnn_sort_keys into sample_keys_tmp i64[m] and sample_keys_out i64[m] /
+ * sample_order_out i32[m] / sample_pts_out f32[m,3]; samples == NULL: the cloud itself, m == n, those four unused),
+ * pccnn_find_neighbors_count, and the pair total in *total_out (host): what pccnn_lib/pc/layers/MCConv.py:136-140
+ * and pccnn_lib/pc/Neighborhood.py:27-45 do up to the allocation of the pair list.  sort_workspace as
+ * pccnn_grid_build for max(n, m) keys, workspace as pccnn_find_neighbors_count; pccnn_find_neighbors_fill then takes
+ * the same sorted points, sample buffers, tables and workspace. */
+int pccnn_neighborhood_count(const float *pts, const int32_t *batch_ids, int64_t n, int batch_size,
+                             const float *aabb_min, const float *cell_size, const int32_t *num_cells_host,
+                             int key_bits, int with_cell_table, int32_t *num_cells_out, int64_t *keys_out,
+                             int64_t *sorted_keys_out, int32_t *perm_out, float *sorted_pts_out, int32_t *grid_ds_out,
+                             int32_t *cell_table_out, const float *samples, const int32_t *sample_batch_ids, int64_t m,
+                             int64_t *sample_keys_tmp, int64_t *sample_keys_out, int32_t *sample_order_out,
+                             float *sample_pts_out, int max_neighbors, int32_t *ends_out, int64_t *total_out,
+                             void *sort_workspace, size_t sort_workspace_bytes, void *workspace, size_t workspace_bytes,
+                             void *stream);
+
 /* ---- convolutions -------------------------------------------------------
  * Shapes: pts f32[n,d], feats f32[n,c_in], samples f32[m,d], neigh i32[t,2]
  * (point, sample), ends i32[m], radii f32[d] (device), out f32[m,c_out].

@@ -1,0 +1,259 @@
+// Host-side sequences for the steps of a hierarchy level whose sizes depend on data: the box of a cloud, the
+// Poisson-disk pooling of a cloud, and the pair count of a neighborhood.  Each is a fixed chain of the library's
+// own launches with one small read-back at its end; run from Python, such a chain of 10 - 30 launches over a cloud
+// of a few thousand points costs several times more in interpreter and binding overhead than on the GPU.  Nothing
+// here computes: the kernels are those of the entry points that are called.
+//
+// The read-backs go through a small pinned host buffer (one per host thread, allocated on first use and kept):
+// an asynchronous copy into it on the caller's stream, then a wait for that stream.
+#include "common.h"
+#include <string.h>
+
+namespace {
+
+struct PinnedSlot {
+    void *p = nullptr;
+    size_t bytes = 0;
+};
+thread_local PinnedSlot g_slot;
+
+int pinned_slot(size_t bytes, void **out)
+{
+    if (g_slot.bytes < bytes) {
+        if (g_slot.p) PCCNN_HIP_CHECK(hipHostFree(g_slot.p));
+        g_slot.p = nullptr;
+        g_slot.bytes = 0;
+        const size_t want = bytes < 4096 ? 4096 : bytes;
+        PCCNN_HIP_CHECK(hipHostMalloc(&g_slot.p, want, hipHostMallocPortable));
+        g_slot.bytes = want;
+    }
+    *out = g_slot.p;
+    return PCCNN_OK;
+}
+
+// device -> caller's host memory, through the pinned buffer; returns when the values are there
+int read_back(void *host_out, const void *dev, size_t bytes, hipStream_t s)
+{
+    void *slot;
+    int rc = pinned_slot(bytes, &slot);
+    if (rc != PCCNN_OK) return rc;
+    PCCNN_HIP_CHECK(hipMemcpyAsync(slot, dev, bytes, hipMemcpyDeviceToHost, s));
+    PCCNN_HIP_CHECK(hipStreamSynchronize(s));
+    memcpy(host_out, slot, bytes);
+    return PCCNN_OK;
+}
+
+struct GridDims {
+    int v[PCCNN_MAX_DIMS];
+};
+
+__global__ void set_dims_kernel(int32_t *dst, GridDims dims, int d)
+{
+    if ((int)threadIdx.x < d) dst[threadIdx.x] = dims.v[threadIdx.x];
+}
+
+// the grid size, known on the host, as the device vector the kernels read; also checks it
+int put_grid_dims(const char *who, const int32_t *num_cells_host, int d, int batch_size, int32_t *dst, hipStream_t s,
+                  int64_t *num_pillars, int64_t *total_cells)
+{
+    GridDims dims;
+    int64_t total = batch_size;
+    for (int k = 0; k < d; ++k) {
+        dims.v[k] = num_cells_host[k];
+        PCCNN_REQUIRE(dims.v[k] > 0, PCCNN_ERR_INVALID, "%s: %d cells along axis %d", who, dims.v[k], k);
+        PCCNN_REQUIRE(total <= INT64_MAX / dims.v[k], PCCNN_ERR_INVALID, "%s: the cell count overflows 64 bits", who);
+        total *= dims.v[k];
+    }
+    *num_pillars = (int64_t)batch_size * dims.v[0] * dims.v[1];
+    *total_cells = total;
+    set_dims_kernel<<<1, 64, 0, s>>>(dst, dims, d);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
+__global__ void __launch_bounds__(256)
+compact_remap_kernel(const int32_t *__restrict__ flags, const int32_t *__restrict__ scan,
+                     const int32_t *__restrict__ remap, int64_t n, int64_t *__restrict__ ids)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n && flags[i] != 0) ids[scan[i] - 1] = remap[i];
+}
+
+struct PoolLayout {
+    int64_t *keys, *sorted_keys;
+    float *sorted_pts;
+    int32_t *grid_ds, *cell_table, *num_cells;
+    void *sort_ws, *poisson_ws;
+    size_t sort_bytes, poisson_bytes;
+};
+
+bool pool_layout(PccnnArena &arena, int64_t n, int64_t num_pillars, int64_t total_cells, PoolLayout &l)
+{
+    l.keys = arena.take<int64_t>((size_t)n);
+    l.sorted_keys = arena.take<int64_t>((size_t)n);
+    l.sorted_pts = arena.take<float>((size_t)n * 3);
+    l.grid_ds = arena.take<int32_t>((size_t)num_pillars * 2);
+    l.cell_table = total_cells > 0 ? arena.take<int32_t>((size_t)total_cells + 1) : nullptr;
+    l.num_cells = arena.take<int32_t>(64);
+    l.sort_bytes = pccnn_grid_build_workspace_bytes(n);
+    l.sort_ws = arena.take<char>(l.sort_bytes);
+    l.poisson_bytes = pccnn_poisson_disk_workspace_bytes(n);
+    l.poisson_ws = arena.take<char>(l.poisson_bytes);
+    return arena.ok();
+}
+
+}  // namespace
+
+extern "C" int pccnn_bounding_box_host(const float *pts, const int32_t *batch_ids, int64_t n, int d, int batch_size,
+                                       float *aabb_min_out, float *aabb_max_out, float *host_min_out,
+                                       float *host_max_out, void *stream)
+{
+    PCCNN_REQUIRE(host_min_out && host_max_out, PCCNN_ERR_INVALID, "pccnn_bounding_box_host: null host pointer");
+    int rc = pccnn_bounding_box(pts, batch_ids, n, d, batch_size, aabb_min_out, aabb_max_out, stream);
+    if (rc != PCCNN_OK) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    const size_t bytes = (size_t)batch_size * d * sizeof(float);
+    void *slot;
+    if ((rc = pinned_slot(2 * bytes, &slot)) != PCCNN_OK) return rc;
+    PCCNN_HIP_CHECK(hipMemcpyAsync(slot, aabb_min_out, bytes, hipMemcpyDeviceToHost, s));
+    PCCNN_HIP_CHECK(hipMemcpyAsync((char *)slot + bytes, aabb_max_out, bytes, hipMemcpyDeviceToHost, s));
+    PCCNN_HIP_CHECK(hipStreamSynchronize(s));
+    memcpy(host_min_out, slot, bytes);
+    memcpy(host_max_out, (char *)slot + bytes, bytes);
+    return PCCNN_OK;
+}
+
+extern "C" size_t pccnn_pool_poisson_workspace_bytes(int64_t n, int64_t num_pillars, int64_t total_cells)
+{
+    if (n < 1) n = 1;
+    if (num_pillars < 1) num_pillars = 1;
+    return 2 * pccnn_align((size_t)n * sizeof(int64_t)) + pccnn_align((size_t)n * 3 * sizeof(float)) +
+           pccnn_align((size_t)num_pillars * 2 * sizeof(int32_t)) +
+           (total_cells > 0 ? pccnn_align(((size_t)total_cells + 1) * sizeof(int32_t)) : 0) + 256 +
+           pccnn_align(pccnn_grid_build_workspace_bytes(n)) + pccnn_align(pccnn_poisson_disk_workspace_bytes(n));
+}
+
+extern "C" int pccnn_pool_poisson_select(const float *pts, const int32_t *batch_ids, int64_t n, int batch_size,
+                                         const float *aabb_min, const float *cell_size,
+                                         const int32_t *num_cells_host, int key_bits, int with_cell_table,
+                                         int32_t *perm_out, int32_t *selected_out, int32_t *selected_scan_out,
+                                         int64_t *count_out, void *workspace, size_t workspace_bytes, void *stream)
+{
+    PCCNN_REQUIRE(n >= 0 && n < (1ll << 31) && batch_size > 0, PCCNN_ERR_INVALID,
+                  "pccnn_pool_poisson_select: n=%lld batch_size=%d", (long long)n, batch_size);
+    PCCNN_REQUIRE(count_out && num_cells_host, PCCNN_ERR_INVALID, "pccnn_pool_poisson_select: null host pointer");
+    *count_out = 0;
+    if (n == 0) return PCCNN_OK;
+    PCCNN_REQUIRE(pts && batch_ids && aabb_min && cell_size && perm_out && selected_out && selected_scan_out,
+                  PCCNN_ERR_INVALID, "pccnn_pool_poisson_select: null pointer");
+    for (int k = 0; k < 3; ++k)
+        PCCNN_REQUIRE(num_cells_host[k] > 0, PCCNN_ERR_INVALID, "pccnn_pool_poisson_select: %d cells along axis %d",
+                      num_cells_host[k], k);
+    int64_t num_pillars = (int64_t)batch_size * num_cells_host[0] * num_cells_host[1];
+    int64_t total_cells = with_cell_table ? num_pillars * num_cells_host[2] : 0;
+    PccnnArena arena(workspace, workspace_bytes);
+    PoolLayout l;
+    PCCNN_REQUIRE(pool_layout(arena, n, num_pillars, total_cells, l), PCCNN_ERR_WORKSPACE,
+                  "pccnn_pool_poisson_select: workspace of %zu bytes, need %zu", workspace_bytes,
+                  pccnn_pool_poisson_workspace_bytes(n, num_pillars, total_cells));
+    hipStream_t s = (hipStream_t)stream;
+    int64_t all_cells;
+    int rc = put_grid_dims("pccnn_pool_poisson_select", num_cells_host, 3, batch_size, l.num_cells, s, &num_pillars,
+                           &all_cells);
+    if (rc != PCCNN_OK) return rc;
+    rc = pccnn_grid_build(pts, batch_ids, aabb_min, l.num_cells, cell_size, n, 3, key_bits, num_pillars, total_cells,
+                              l.keys, l.sorted_keys, perm_out, l.sorted_pts, l.grid_ds, l.cell_table, l.sort_ws,
+                              l.sort_bytes, stream);
+    if (rc != PCCNN_OK) return rc;
+    rc = pccnn_poisson_disk_grid(l.sorted_pts, l.sorted_keys, n, l.grid_ds, num_pillars, l.cell_table, total_cells,
+                                 l.num_cells, cell_size, 3, selected_out, selected_scan_out, l.poisson_ws,
+                                 l.poisson_bytes, stream);
+    if (rc != PCCNN_OK) return rc;
+    int32_t count = 0;
+    if ((rc = read_back(&count, selected_scan_out + (n - 1), sizeof(int32_t), s)) != PCCNN_OK) return rc;
+    *count_out = count;
+    return PCCNN_OK;
+}
+
+extern "C" int pccnn_compact_selected_remap(const int32_t *selected, const int32_t *selected_scan,
+                                            const int32_t *remap, int64_t n, int64_t *ids_out, void *stream)
+{
+    PCCNN_REQUIRE(n >= 0, PCCNN_ERR_INVALID, "pccnn_compact_selected_remap: n=%lld", (long long)n);
+    if (n == 0) return PCCNN_OK;
+    PCCNN_REQUIRE(selected && selected_scan && remap && ids_out, PCCNN_ERR_INVALID,
+                  "pccnn_compact_selected_remap: null pointer");
+    compact_remap_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, (hipStream_t)stream>>>(selected, selected_scan,
+                                                                                           remap, n, ids_out);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
+extern "C" int pccnn_grid_build_sized(const float *pts, const int32_t *batch_ids, const float *aabb_min,
+                                      const int32_t *num_cells_host, const float *cell_size, int64_t n, int d,
+                                      int batch_size, int key_bits, int with_cell_table, int32_t *num_cells_out,
+                                      int64_t *keys_out, int64_t *sorted_keys_out, int32_t *perm_out,
+                                      float *sorted_pts_out, int32_t *grid_ds_out, int32_t *cell_table_out,
+                                      void *workspace, size_t workspace_bytes, void *stream)
+{
+    PCCNN_REQUIRE(d >= 2 && d <= PCCNN_MAX_DIMS, PCCNN_ERR_UNSUPPORTED,
+                  "pccnn_grid_build_sized: d=%d is not supported (2 <= d <= 6)", d);
+    PCCNN_REQUIRE(num_cells_host && num_cells_out && batch_size > 0, PCCNN_ERR_INVALID,
+                  "pccnn_grid_build_sized: null grid size or batch_size=%d", batch_size);
+    PCCNN_REQUIRE(!with_cell_table || (cell_table_out && d == 3), PCCNN_ERR_INVALID,
+                  "pccnn_grid_build_sized: the cell table needs its output and d == 3");
+    int64_t num_pillars, total_cells;
+    int rc = put_grid_dims("pccnn_grid_build_sized", num_cells_host, d, batch_size, num_cells_out, (hipStream_t)stream,
+                           &num_pillars, &total_cells);
+    if (rc != PCCNN_OK) return rc;
+    return pccnn_grid_build(pts, batch_ids, aabb_min, num_cells_out, cell_size, n, d, key_bits, num_pillars,
+                            with_cell_table ? total_cells : 0, keys_out, sorted_keys_out, perm_out, sorted_pts_out,
+                            grid_ds_out, with_cell_table ? cell_table_out : nullptr, workspace, workspace_bytes, stream);
+}
+
+extern "C" int pccnn_neighborhood_count(const float *pts, const int32_t *batch_ids, int64_t n, int batch_size,
+                                        const float *aabb_min, const float *cell_size,
+                                        const int32_t *num_cells_host, int key_bits, int with_cell_table,
+                                        int32_t *num_cells_out, int64_t *keys_out, int64_t *sorted_keys_out,
+                                        int32_t *perm_out, float *sorted_pts_out, int32_t *grid_ds_out,
+                                        int32_t *cell_table_out, const float *samples,
+                                        const int32_t *sample_batch_ids, int64_t m, int64_t *sample_keys_tmp,
+                                        int64_t *sample_keys_out, int32_t *sample_order_out, float *sample_pts_out,
+                                        int max_neighbors, int32_t *ends_out, int64_t *total_out,
+                                        void *sort_workspace, size_t sort_workspace_bytes, void *workspace,
+                                        size_t workspace_bytes, void *stream)
+{
+    PCCNN_REQUIRE(total_out, PCCNN_ERR_INVALID, "pccnn_neighborhood_count: null host pointer");
+    *total_out = 0;
+    PCCNN_REQUIRE(n > 0 && m > 0, PCCNN_ERR_INVALID, "pccnn_neighborhood_count: n=%lld m=%lld (both must be positive)",
+                  (long long)n, (long long)m);
+    int rc = pccnn_grid_build_sized(pts, batch_ids, aabb_min, num_cells_host, cell_size, n, 3, batch_size, key_bits,
+                                    with_cell_table, num_cells_out, keys_out, sorted_keys_out, perm_out, sorted_pts_out,
+                                    grid_ds_out, cell_table_out, sort_workspace, sort_workspace_bytes, stream);
+    if (rc != PCCNN_OK) return rc;
+    const int64_t num_pillars = (int64_t)batch_size * num_cells_host[0] * num_cells_host[1];
+    const int64_t total_cells = with_cell_table ? num_pillars * num_cells_host[2] : 0;
+    const float *s_pts = sorted_pts_out;
+    const int64_t *s_keys = sorted_keys_out;
+    const int32_t *s_order = perm_out;
+    if (samples != nullptr) {
+        PCCNN_REQUIRE(sample_batch_ids && sample_keys_tmp && sample_keys_out && sample_order_out && sample_pts_out,
+                      PCCNN_ERR_INVALID, "pccnn_neighborhood_count: null sample buffer");
+        rc = pccnn_compute_keys(samples, sample_batch_ids, aabb_min, num_cells_out, cell_size, m, 3, sample_keys_tmp,
+                                stream);
+        if (rc != PCCNN_OK) return rc;
+        rc = pccnn_sort_keys(sample_keys_tmp, m, key_bits, sample_keys_out, sample_order_out, samples, 3, sample_pts_out,
+                             sort_workspace, sort_workspace_bytes, stream);
+        if (rc != PCCNN_OK) return rc;
+        s_pts = sample_pts_out;
+        s_keys = sample_keys_out;
+        s_order = sample_order_out;
+    } else {
+        PCCNN_REQUIRE(m == n, PCCNN_ERR_INVALID, "pccnn_neighborhood_count: without samples m must equal n");
+    }
+    rc = pccnn_find_neighbors_count(sorted_pts_out, sorted_keys_out, n, s_pts, s_keys, m, s_order, 1, grid_ds_out,
+                                    num_pillars, with_cell_table ? cell_table_out : nullptr, total_cells, num_cells_out,
+                                    cell_size, 3, max_neighbors, ends_out, workspace, workspace_bytes, stream);
+    if (rc != PCCNN_OK) return rc;
+    // the 64-bit pair total sits at the head of the search's workspace
+    return read_back(total_out, workspace, sizeof(int64_t), (hipStream_t)stream);
+}

@@ -207,14 +207,48 @@ poisson_grid_pass_kernel(PoissonGridArgs a, int colour)
             float sx = 0.f, sy = 0.f, sz = 0.f;
             if (valid) { sx = a.pts[(int64_t)p * 3 + 0]; sy = a.pts[(int64_t)p * 3 + 1]; sz = a.pts[(int64_t)p * 3 + 2]; }
             bool cand = valid;
-            // selected points around the cell: flags first, positions only where a flag is set
+            // Selected points around the cell: flags first, positions only where a flag is set.  The first 64 flags of
+            // all nine ranges are requested together, then every lane that found a flag fetches that point's position
+            // itself, so the tests below read registers: two memory round trips per round of 64 points, not one or
+            // two per range.
+            int flag[9];
+            float fx[9], fy[9], fz[9];
+#pragma unroll
             for (int r = 0; r < 9; ++r) {
                 const int2 g = rng[wib][r];
-                for (int j0 = 0; j0 < g.y; j0 += 64) {
+                const int q = g.x + lane;
+                flag[r] = 0;
+                if (lane < g.y) flag[r] = (q >= first && q < base) ? a.used[q] : settled[q];
+            }
+#pragma unroll
+            for (int r = 0; r < 9; ++r) {
+                fx[r] = fy[r] = fz[r] = 0.f;
+                if (flag[r] != 0) {
+                    const int64_t q = (int64_t)rng[wib][r].x + lane;
+                    fx[r] = a.pts[q * 3 + 0]; fy[r] = a.pts[q * 3 + 1]; fz[r] = a.pts[q * 3 + 2];
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 9; ++r) {
+                unsigned long long set = __ballot(flag[r] != 0);
+                while (set != 0ull) {
+                    const int src = __builtin_ctzll(set);
+                    set &= set - 1ull;
+                    const float vx = (sx - pccnn_bcast_f(fx[r], src)) * ir0;
+                    const float vy = (sy - pccnn_bcast_f(fy[r], src)) * ir1;
+                    const float vz = (sz - pccnn_bcast_f(fz[r], src)) * ir2;
+                    const float acc = ((0.0f + vx * vx) + vy * vy) + vz * vz;
+                    if (acc < 1.0f) cand = false;
+                }
+            }
+            // ranges of more than 64 points: the rest, range by range
+            for (int r = 0; r < 9; ++r) {
+                const int2 g = rng[wib][r];
+                for (int j0 = 64; j0 < g.y; j0 += 64) {
                     const int q = g.x + j0 + lane;
-                    int flag = 0;
-                    if (j0 + lane < g.y) flag = (q >= first && q < base) ? a.used[q] : settled[q];
-                    unsigned long long set = __ballot(flag != 0);
+                    int more = 0;
+                    if (j0 + lane < g.y) more = (q >= first && q < base) ? a.used[q] : settled[q];
+                    unsigned long long set = __ballot(more != 0);
                     while (set != 0ull) {
                         const int qi = g.x + j0 + __builtin_ctzll(set);
                         set &= set - 1ull;

@@ -43,3 +43,12 @@ def host_vector(tensor):
     any other tensor: lets a caller do on the host, with the same fp32 arithmetic, what would otherwise need a
     read-back."""
     return _host_values.get(id(tensor)) if tensor is not None else None
+
+
+def host_num_cells(box_host, cell_host):
+    """Grid size as a list of ints from the box and the cell size on the host: the fp32 arithmetic of
+    pccnn_lib/pc/Grid.py:26-28 (subtract, IEEE divide, truncate, + 1, maximum over the clouds) in numpy."""
+    mn, mx = box_host
+    with np.errstate(all="ignore"):
+        cells = ((mx - mn) / cell_host.reshape(1, -1)).astype(np.int32) + np.int32(1)
+    return [int(v) for v in cells.max(axis=0)]

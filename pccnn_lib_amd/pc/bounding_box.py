@@ -22,14 +22,16 @@ class BoundingBox(object):
                 and cached[3] == ids._version:
             self.min_, self.max_, self.host_ = cached[4], cached[5], cached[6]
             return
-        self.min_, self.max_ = pccnn_lib_ops.bounding_box(pts.detach(), ids, p_point_cloud.batch_size_host())
-        self.host_ = [None]      # the box on the host, read back at most once and shared by every user of the cache entry
+        # every grid over the cloud sizes itself from the box on the host: it comes back with the same native call
+        self.min_, self.max_, host = pccnn_lib_ops.bounding_box_host(pts.detach(), ids,
+                                                                    p_point_cloud.batch_size_host())
+        self.host_ = [host]      # shared by every user of the cache entry
         # weak references: the entry neither keeps replaced tensors alive nor matches a new tensor at a reused address
         p_point_cloud.aabb_cache_ = (weakref.ref(pts), pts._version, weakref.ref(ids), ids._version, self.min_,
                                      self.max_, self.host_)
 
     def host(self):
-        """(min, max) as float32 numpy arrays [B, D]: one read-back per box, however many grids are laid over it."""
+        """(min, max) as float32 numpy arrays [B, D]: read back once per box, however many grids are laid over it."""
         if self.host_[0] is None:
             both = torch.stack([self.min_, self.max_]).cpu().numpy()
             self.host_[0] = (both[0], both[1])

@@ -1,7 +1,7 @@
 import torch
 
 from .. import pccnn_lib_ops
-from ._consts import device_vector, host_vector
+from ._consts import device_vector, host_num_cells, host_vector
 
 
 class Grid(object):
@@ -17,10 +17,7 @@ class Grid(object):
         self.pointcloud_ = p_point_cloud
         self.bounding_box_ = p_bounding_box
         self.cell_size_ = device_vector(p_cell_size, p_point_cloud.pts_.shape[1], p_point_cloud.pts_.device)
-        with torch.no_grad():
-            # Grid.py:26-28: fp32 division, truncation, + 1, maximum over the clouds.
-            self.num_cells_ = pccnn_lib_ops.num_cells(self.bounding_box_.min_, self.bounding_box_.max_,
-                                                      self.cell_size_.contiguous())
+        self.num_cells_device_ = None
         self.num_cells_host_ = None
         self.cell_ids_ = None
         self.sorted_ids_i64_ = None
@@ -29,6 +26,31 @@ class Grid(object):
         self.sorted_pts_ = None
         self.grid_ds_ = None
         self.cell_table_ = None
+
+    @property
+    def num_cells_(self):
+        """int32 [D] on the device (Grid.py:26-28: fp32 division, truncation, + 1, maximum over the clouds): computed
+        there on first use, unless the grid was built from the host copy of the same numbers before."""
+        if self.num_cells_device_ is None:
+            with torch.no_grad():
+                self.num_cells_device_ = pccnn_lib_ops.num_cells(self.bounding_box_.min_, self.bounding_box_.max_,
+                                                                 self.cell_size_.contiguous())
+        return self.num_cells_device_
+
+    @num_cells_.setter
+    def num_cells_(self, p_value):
+        self.num_cells_device_ = p_value
+
+    def sized_on_host(self):
+        """True when the grid size can be had without a read-back of its own: the cell size came from host values
+        and the box keeps a host copy."""
+        return self.num_cells_host_ is not None or (host_vector(self.cell_size_) is not None
+                                                    and hasattr(self.bounding_box_, "host"))
+
+    def adopt(self, p_built):
+        """Takes the tensors of ``pccnn_lib_ops.grid_build_sized`` as this grid's."""
+        (self.num_cells_device_, self.cell_ids_, self.sorted_cell_ids_, self.sorted_ids_i32_, self.sorted_pts_,
+         self.grid_ds_, self.cell_table_) = p_built
 
     @property
     def sorted_ids_(self):
@@ -50,11 +72,7 @@ class Grid(object):
         if self.num_cells_host_ is None:
             cell = host_vector(self.cell_size_)
             if cell is not None and hasattr(self.bounding_box_, "host"):
-                import numpy as np
-                mn, mx = self.bounding_box_.host()
-                with np.errstate(all="ignore"):
-                    cells = ((mx - mn) / cell.reshape(1, -1)).astype(np.int32) + np.int32(1)
-                self.num_cells_host_ = [int(v) for v in cells.max(axis=0)]
+                self.num_cells_host_ = host_num_cells(self.bounding_box_.host(), cell)
             else:
                 self.num_cells_host_ = self.num_cells_.tolist()
         return self.num_cells_host_
@@ -69,6 +87,10 @@ class Grid(object):
             with torch.no_grad():
                 pts = self.pointcloud_.pts_.detach()
                 batch = self.pointcloud_.batch_size_host()
+                if self.num_cells_device_ is None and self.sized_on_host():
+                    self.adopt(pccnn_lib_ops.grid_build_sized(pts, self.pointcloud_.batch_ids_, self.bounding_box_.min_,
+                                                              self.num_cells_host(), self.cell_size_, batch))
+                    return
                 cells = self.num_cells_host()
                 shape = [batch] + cells[0:2] + [2]
                 total = batch

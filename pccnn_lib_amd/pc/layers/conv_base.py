@@ -19,9 +19,7 @@ def build_neighborhood(p_pc_in, p_pc_out, p_radius, p_max_neighs, p_key_order=Fa
     from ..neighborhood import Neighborhood
     bb = BoundingBox(p_pc_in)
     grid = Grid(p_pc_in, bb, p_radius)
-    grid.compute_cell_ids()
-    grid.build_ds()
-    return Neighborhood(grid, p_pc_out, p_max_neighs, p_key_order)
+    return Neighborhood(grid, p_pc_out, p_max_neighs, p_key_order)     # builds the grid
 
 
 class _PermuteRows(torch.autograd.Function):

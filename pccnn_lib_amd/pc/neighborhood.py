@@ -3,6 +3,11 @@ import torch
 from .. import pccnn_lib_ops
 
 
+# A neighborhood over a grid that is not built yet (three dimensions, grid size known on the host) builds the grid and
+# searches it in one native call (False: grid first, then the search, step by step; the result is the same).
+ONE_CALL = True
+
+
 class Neighborhood(object):
     """Radius neighborhood of the samples in a gridded cloud (pccnn_lib/pc/Neighborhood.py:10-53).
 
@@ -24,6 +29,27 @@ class Neighborhood(object):
         grid = p_grid
         with torch.no_grad():
             sample_pts = p_samples.pts_.detach()
+            cloud = grid.pointcloud_
+            if ONE_CALL and grid.cell_ids_ is None and grid.num_cells_device_ is None and cloud.pts_.shape[1] == 3 \
+                    and sample_pts.shape[1] == 3 and cloud.pts_.shape[0] > 0 and sample_pts.shape[0] > 0 \
+                    and grid.sized_on_host():
+                # a grid that is not built yet, in three dimensions, sized from host values: grid, sample order,
+                # count pass and pair total in one native call
+                own = p_samples is cloud
+                key_order = bool(p_key_order)
+                built, neighbors, self.start_ids_ = pccnn_lib_ops.neighborhood_build(
+                    cloud.pts_.detach(), cloud.batch_ids_, grid.bounding_box_.min_, grid.num_cells_host(),
+                    grid.cell_size_, cloud.batch_size_host(), None if own else sample_pts,
+                    None if own else p_samples.batch_ids_, p_max_neighbors, not key_order)
+                grid.adopt(built)
+                if key_order:
+                    self.neighbors_key_order_ = neighbors
+                else:
+                    self.neighbors_original_ = neighbors
+                return
+            if grid.cell_ids_ is None:
+                grid.compute_cell_ids()
+            grid.build_ds()
             # the samples go to the search in key order (a wavefront's 64 samples then share their cell walk and
             # read their coordinates as one run): the gridded cloud itself is sorted already
             if p_samples is grid.pointcloud_:

@@ -3,6 +3,12 @@ import torch
 from .. import pccnn_lib_ops
 from .bounding_box import BoundingBox
 from .grid import Grid
+from ._consts import device_vector, host_num_cells, host_vector
+
+
+# Three-dimensional Poisson-disk pooling with a cell size known on the host runs as one native call (False: the
+# same steps one by one through Grid, as for every other case; the result is the same).
+ONE_CALL = True
 
 
 class PointPooling(object):
@@ -18,6 +24,15 @@ class PointPooling(object):
         self.method_ = p_method
         with torch.no_grad():
             bb = BoundingBox(p_point_cloud)
+            if ONE_CALL and p_method == "poisson_disk" and p_point_cloud.pts_.shape[1] == 3:
+                cell = device_vector(p_radii, 3, p_point_cloud.pts_.device)
+                cell_host = host_vector(cell)
+                if cell_host is not None:
+                    # three dimensions, cell size known on the host: grid, selection and its size in one native call
+                    self.pooling_ids_ = pccnn_lib_ops.pool_poisson(
+                        p_point_cloud.pts_.detach(), p_point_cloud.batch_ids_, bb.min_, cell,
+                        host_num_cells(bb.host(), cell_host), p_point_cloud.batch_size_host())
+                    return
             grid = Grid(p_point_cloud, bb, p_radii)
             grid.compute_cell_ids()
             if p_method == "poisson_disk":

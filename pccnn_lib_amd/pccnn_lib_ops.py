@@ -88,6 +88,22 @@ def bounding_box(pts, batch_ids, batch_size):
     return mn, mx
 
 
+def bounding_box_host(pts, batch_ids, batch_size):
+    """``bounding_box`` and the same box on the host, from one native call that ends with its one read-back:
+    -> (f32[B,D], f32[B,D], (numpy f32[B,D], numpy f32[B,D]))."""
+    import numpy as np
+    _chk(pts, "bounding_box: pts", torch.float32, 2)
+    _chk(batch_ids, "bounding_box: batch_ids", torch.int32, 1, pts.device)
+    d = _dims(pts, "bounding_box")
+    batch_size = int(batch_size)
+    mn = torch.empty((batch_size, d), dtype=torch.float32, device=pts.device)
+    mx = torch.empty_like(mn)
+    host = np.empty((2, batch_size, d), dtype=np.float32)
+    _lib.call("pccnn_bounding_box_host", _ptr(pts), _ptr(batch_ids), pts.shape[0], d, batch_size, _ptr(mn), _ptr(mx),
+              _P(host.ctypes.data), _P(host.ctypes.data + host[0].nbytes), _stream())
+    return mn, mx, (host[0], host[1])
+
+
 def num_cells(aabb_min, aabb_max, cell_size):
     """Grid size i32[D] = max over the clouds of int32((max - min) / cell_size) + 1 (pccnn_lib/pc/Grid.py:26-28)."""
     name = "num_cells"
@@ -297,6 +313,110 @@ def find_neighbors(pts, pt_keys, samples, sample_keys, grid_ds, grid_size, radii
                              cell_table=table)
 
 
+def grid_build_sized(pts, batch_ids, aabb_min, num_cells_host, cell_size, batch_size):
+    """``grid_build`` for a grid whose size is known on the host (a list of D ints): the device copy of that size
+    is written by the same native call.  Returns (num_cells i32[D], keys, sorted keys, perm, sorted points, grid_ds
+    [B, nc0, nc1, 2], cell table or None)."""
+    name = "grid_build"
+    _chk(pts, name + ": pts", torch.float32, 2)
+    dev = pts.device
+    _chk(batch_ids, name + ": batch_ids", torch.int32, 1, dev)
+    _chk(aabb_min, name + ": aabb_min", torch.float32, 2, dev)
+    _chk(cell_size, name + ": cell_size", torch.float32, 1, dev)
+    d = _dims(pts, name)
+    n = pts.shape[0]
+    batch_size = int(batch_size)
+    cells = [int(v) for v in num_cells_host]
+    if batch_ids.shape[0] != n or tuple(aabb_min.shape) != (batch_size, d) or cell_size.shape[0] != d \
+            or len(cells) != d or min(cells) < 1:
+        raise RuntimeError(name + ": inconsistent shapes")
+    total = batch_size
+    for c in cells:
+        total *= c
+    with_table = 1 if (d == 3 and total <= CELL_TABLE_MAX_CELLS) else 0
+    num = torch.empty((d,), dtype=torch.int32, device=dev)
+    keys = torch.empty((n,), dtype=torch.int64, device=dev)
+    skeys = torch.empty_like(keys)
+    perm = torch.empty((n,), dtype=torch.int32, device=dev)
+    spts = torch.empty_like(pts)
+    ds = torch.empty((batch_size, cells[0], cells[1], 2), dtype=torch.int32, device=dev)
+    table = torch.empty((total + 1,), dtype=torch.int32, device=dev) if with_table else None
+    ws = _workspace(_lib.load().pccnn_grid_build_workspace_bytes(n), dev)
+    _lib.call("pccnn_grid_build_sized", _ptr(pts), _ptr(batch_ids), _ptr(aabb_min), (ctypes.c_int32 * d)(*cells),
+              _ptr(cell_size), n, d, batch_size, key_bits_for(cells, batch_size), with_table, _ptr(num), _ptr(keys),
+              _ptr(skeys), _ptr(perm), _ptr(spts), _ptr(ds), _optr(table), _ptr(ws), ws.numel(), _stream())
+    return num, keys, skeys, perm, spts, ds, table
+
+
+def neighborhood_build(pts, batch_ids, aabb_min, num_cells_host, cell_size, batch_size, samples, sample_batch_ids,
+                       max_neighbors, remap_points):
+    """A 3-D layer's neighborhood from the cloud's box: the grid over ``pts`` (as ``grid_build_sized``), the samples
+    in key order, the count pass and the pair total in one native call, the pair list in a second one (what
+    pccnn_lib/pc/layers/MCConv.py:136-140 with pccnn_lib/pc/Neighborhood.py:27-53 does).  ``samples`` None: the
+    cloud's own points.  ``remap_points``: column 0 of the pairs holds original point indices, else indices into
+    the sorted copy.  Returns (grid tuple of ``grid_build_sized``, pairs i32[T,2], ends i32[M])."""
+    name = "neighborhood_build"
+    _chk(pts, name + ": pts", torch.float32, 2)
+    dev = pts.device
+    _chk(batch_ids, name + ": batch_ids", torch.int32, 1, dev)
+    _chk(aabb_min, name + ": aabb_min", torch.float32, 2, dev)
+    _chk(cell_size, name + ": cell_size", torch.float32, 1, dev)
+    n = pts.shape[0]
+    batch_size = int(batch_size)
+    cells = [int(v) for v in num_cells_host]
+    max_neighbors = int(max_neighbors)
+    if pts.shape[1] != 3 or batch_ids.shape[0] != n or tuple(aabb_min.shape) != (batch_size, 3) \
+            or cell_size.shape[0] != 3 or len(cells) != 3 or min(cells) < 1 or n < 1 or max_neighbors < 0:
+        raise RuntimeError(name + ": 3-D points [N,3] (N > 0), batch_ids [N], aabb_min [B,3], cell_size [3], three "
+                                  "grid sizes, max_neighbors >= 0")
+    m = n
+    if samples is not None:
+        _chk(samples, name + ": samples", torch.float32, 2, dev)
+        _chk(sample_batch_ids, name + ": sample batch_ids", torch.int32, 1, dev)
+        m = samples.shape[0]
+        if samples.shape[1] != 3 or sample_batch_ids.shape[0] != m or m < 1:
+            raise RuntimeError(name + ": samples [M,3] (M > 0) with batch_ids [M]")
+    pillars = batch_size * cells[0] * cells[1]
+    total_cells = pillars * cells[2]
+    with_table = 1 if total_cells <= CELL_TABLE_MAX_CELLS else 0
+    lib = _lib.load()
+    num = torch.empty((3,), dtype=torch.int32, device=dev)
+    keys = torch.empty((n,), dtype=torch.int64, device=dev)
+    skeys = torch.empty_like(keys)
+    perm = torch.empty((n,), dtype=torch.int32, device=dev)
+    spts = torch.empty_like(pts)
+    ds = torch.empty((batch_size, cells[0], cells[1], 2), dtype=torch.int32, device=dev)
+    table = torch.empty((total_cells + 1,), dtype=torch.int32, device=dev) if with_table else None
+    ends = torch.empty((m,), dtype=torch.int32, device=dev)
+    sort_ws = _workspace(lib.pccnn_grid_build_workspace_bytes(max(n, m)), dev)
+    ws = _workspace(lib.pccnn_find_neighbors_workspace_bytes(n, m), dev)
+    if samples is not None:
+        # unsorted keys | sorted keys (i64 each) | sorted points (3 f32) | order (i32): 32 bytes per sample
+        sbuf = torch.empty((4 * m,), dtype=torch.int64, device=dev)
+        sb = sbuf.data_ptr()
+        s_tmp, s_keys, s_pts, s_order = _P(sb), _P(sb + 8 * m), _P(sb + 16 * m), _P(sb + 28 * m)
+        f_pts, f_keys, f_order = s_pts, s_keys, s_order
+        samples_p, sample_ids_p = _ptr(samples), _ptr(sample_batch_ids)
+    else:
+        s_tmp = s_keys = s_pts = s_order = samples_p = sample_ids_p = _P(0)
+        f_pts, f_keys, f_order = _ptr(spts), _ptr(skeys), _ptr(perm)
+    bits = key_bits_for(cells, batch_size)
+    total = ctypes.c_int64(0)
+    _lib.call("pccnn_neighborhood_count", _ptr(pts), _ptr(batch_ids), n, batch_size, _ptr(aabb_min), _ptr(cell_size),
+              (ctypes.c_int32 * 3)(*cells), bits, with_table, _ptr(num), _ptr(keys), _ptr(skeys), _ptr(perm), _ptr(spts),
+              _ptr(ds), _optr(table), samples_p, sample_ids_p, m, s_tmp, s_keys, s_order, s_pts, max_neighbors,
+              _ptr(ends), ctypes.byref(total), _ptr(sort_ws), sort_ws.numel(), _ptr(ws), ws.numel(), _stream())
+    total = total.value
+    if total < 0 or total > 0x7fffffff:
+        raise RuntimeError(name + ": more than 2^31 - 1 pairs; the pair offsets are 32-bit as in the reference, "
+                                  "use a smaller radius, a neighbor cap or fewer samples per call")
+    neigh = torch.empty((total, 2), dtype=torch.int32, device=dev)
+    _lib.call("pccnn_find_neighbors_fill", _ptr(spts), _ptr(skeys), n, f_pts, f_keys, m, f_order, 1, _ptr(ds), pillars,
+              _optr(table), total_cells if with_table else 0, _ptr(num), _ptr(cell_size), 3, max_neighbors, _ptr(ends),
+              _ptr(perm) if remap_points else _P(0), total, _ptr(neigh), _ptr(ws), ws.numel(), _stream())
+    return (num, keys, skeys, perm, spts, ds, table), neigh, ends
+
+
 # ------------------------------------------------------------------------------ pdf
 
 
@@ -449,6 +569,41 @@ def poisson_disk_sampling_grid(sorted_pts, sorted_keys, grid_ds, grid_size, radi
     count = int(scan[-1].item())
     ids = torch.empty((count, 1), dtype=torch.int64, device=dev)
     _lib.call("pccnn_compact_selected", _ptr(sel), _ptr(scan), n, _ptr(ids), _stream())
+    return ids
+
+
+def pool_poisson(pts, batch_ids, aabb_min, cell_size, num_cells_host, batch_size):
+    """Poisson-disk pooling of a 3-D cloud from its box and the grid size on the host (what
+    pccnn_lib/pc/PointPooling.py:38-69 does after the bounding box): the grid, the selection and its size in one
+    native call, the selected points' ORIGINAL indices in a second one -> i64[S], in key order.  No counterpart in
+    the reference's module; the kernels are those of grid_build and poisson_disk_sampling_grid."""
+    name = "pool_poisson"
+    _chk(pts, name + ": pts", torch.float32, 2)
+    dev = pts.device
+    _chk(batch_ids, name + ": batch_ids", torch.int32, 1, dev)
+    _chk(aabb_min, name + ": aabb_min", torch.float32, 2, dev)
+    _chk(cell_size, name + ": cell_size", torch.float32, 1, dev)
+    n = pts.shape[0]
+    batch_size = int(batch_size)
+    cells = [int(v) for v in num_cells_host]
+    if pts.shape[1] != 3 or batch_ids.shape[0] != n or tuple(aabb_min.shape) != (batch_size, 3) \
+            or cell_size.shape[0] != 3 or len(cells) != 3 or min(cells) < 1:
+        raise RuntimeError(name + ": 3-D points [N,3], batch_ids [N], aabb_min [B,3], cell_size [3], three grid sizes")
+    if n == 0:
+        return torch.empty((0,), dtype=torch.int64, device=dev)
+    pillars = batch_size * cells[0] * cells[1]
+    total = pillars * cells[2]
+    with_table = 1 if total <= CELL_TABLE_MAX_CELLS else 0
+    lib = _lib.load()
+    ws = _workspace(lib.pccnn_pool_poisson_workspace_bytes(n, pillars, total if with_table else 0), dev)
+    rows = torch.empty((3 * n,), dtype=torch.int32, device=dev)      # permutation | selection flags | their scan
+    base = rows.data_ptr()
+    count = ctypes.c_int64(0)
+    _lib.call("pccnn_pool_poisson_select", _ptr(pts), _ptr(batch_ids), n, batch_size, _ptr(aabb_min), _ptr(cell_size),
+              (ctypes.c_int32 * 3)(*cells), key_bits_for(cells, batch_size), with_table, _P(base), _P(base + 4 * n),
+              _P(base + 8 * n), ctypes.byref(count), _ptr(ws), ws.numel(), _stream())
+    ids = torch.empty((count.value,), dtype=torch.int64, device=dev)
+    _lib.call("pccnn_compact_selected_remap", _P(base + 4 * n), _P(base + 8 * n), _P(base), n, _ptr(ids), _stream())
     return ids
 
 

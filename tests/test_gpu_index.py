@@ -428,3 +428,44 @@ def test_grid_size_on_the_host_equals_the_device_result(ops):
     pool = lib.pc.PointPooling(pc, 0.1)
     out = lib.pc.Pointcloud(pool.pool_tensor(pc.pts_), pool.pool_tensor(pc.batch_ids_))
     assert out.batch_size_host_ == 3 and int(out.batch_size_) == 3 and int(torch.max(out.batch_ids_)) == 2
+
+
+@pytest.mark.parametrize("batch,num_pts,radius", [(3, 3000, 0.08), (1, 500, 0.3), (4, 20000, 0.04)])
+def test_one_call_pooling_and_neighborhood_equal_the_step_by_step_routes(ops, monkeypatch, batch, num_pts, radius):
+    # PointPooling and Neighborhood run their chain of launches as one native call when the grid size is known on
+    # the host; the same launches step by step (the route of every other case) must give the same tensors
+    import pccnn_lib_amd as lib
+    from pccnn_lib_amd.pc import neighborhood, point_pooling
+    pts, ids = synthetic.primitives(31 + batch, batch, num_pts)
+
+    def run(one_call):
+        monkeypatch.setattr(point_pooling, "ONE_CALL", one_call)
+        monkeypatch.setattr(neighborhood, "ONE_CALL", one_call)
+        pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+        pool = lib.pc.PointPooling(pc, radius)
+        out_pc = lib.pc.Pointcloud(pool.pool_tensor(pc.pts_), pool.pool_tensor(pc.batch_ids_))
+        got = [pool.pooling_ids_]
+        for samples, cap, key_order in ((out_pc, 0, False), (pc, 0, False), (out_pc, 5, False), (out_pc, 0, True)):
+            grid = lib.pc.Grid(pc, lib.pc.BoundingBox(pc), 2.0 * radius)
+            if not one_call:
+                grid.compute_cell_ids()
+                grid.build_ds()
+            nbh = lib.pc.Neighborhood(grid, samples, cap, key_order)
+            got += [nbh.neighbors_key_order_ if key_order else nbh.neighbors_original_, nbh.neighbors_,
+                    nbh.start_ids_, grid.num_cells_, grid.cell_ids_, grid.sorted_cell_ids_, grid.sorted_ids_,
+                    grid.sorted_pts_, grid.grid_ds_, grid.cell_table_]
+        return got
+
+    a, b = run(False), run(True)
+    assert len(a) == len(b) and a[0].dtype == torch.int64 and a[0].shape[0] > 0
+    for x, y in zip(a, b):
+        assert x.dtype == y.dtype and tuple(x.shape) == tuple(y.shape) and torch.equal(x, y)
+
+
+def test_bounding_box_comes_back_on_the_host_with_the_same_call(ops):
+    pts, ids = synthetic.primitives(3, 5, 800)
+    mn, mx, (host_mn, host_mx) = ops.bounding_box_host(t(pts), t(ids), 5)
+    mn2, mx2 = ops.bounding_box(t(pts), t(ids), 5)
+    assert torch.equal(mn, mn2) and torch.equal(mx, mx2)
+    assert np.array_equal(host_mn, mn.cpu().numpy()) and np.array_equal(host_mx, mx.cpu().numpy())
+    assert host_mn.dtype == np.float32 and host_mn.shape == (5, 3)
