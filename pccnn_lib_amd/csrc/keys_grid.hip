@@ -293,6 +293,98 @@ extern "C" int pccnn_build_grid_ds(const int64_t *sorted_keys, int64_t n, const 
     return PCCNN_OK;
 }
 
+// Pillar table and per-cell table of a sorted key array in one launch (the results of pccnn_build_grid_ds, its zero
+// fill included, and of pccnn_build_cell_table).  One lane per point plus one for the tail: the lane of a point that
+// starts a new key owns the table entries between the previous key and its own, the lane of a point that starts a
+// new pillar owns the empty pillars in between (they are zeroed) and writes the pillar's start, the pillar's last
+// point writes its end; the lanes of a wavefront fill each other's runs together with coalesced stores.
+template <int D, bool TABLE>
+__global__ void __launch_bounds__(256)
+grid_tables_kernel(const int64_t *__restrict__ keys, int64_t n, const int32_t *__restrict__ num_cells,
+                   int64_t num_pillars, int64_t total_cells, int32_t *__restrict__ ds, int32_t *__restrict__ table)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    long long div = 1;
+#pragma unroll
+    for (int k = 2; k < D; ++k) div *= num_cells[k];
+    long long from = 0, to = -1;                                    // table[from..to] = i (empty when to < from)
+    long long zfrom = 0, zto = -1;                                  // pillars zfrom..zto are empty
+    if (i == n) {
+        const long long last = n > 0 ? keys[n - 1] : -1;
+        from = last + 1;
+        to = total_cells;
+        zfrom = last >= 0 ? last / div + 1 : 0;
+        zto = num_pillars - 1;
+    } else if (i < n) {
+        const long long key = keys[i];
+        const long long prev = i > 0 ? keys[i - 1] : -1;
+        if (key != prev) { from = prev + 1; to = key; }
+        const long long cur = key / div;
+        const long long prev_p = prev >= 0 ? prev / div : -1;
+        const long long next_p = (i + 1 < n) ? keys[i + 1] / div : -1;
+        if (cur >= 0 && cur < num_pillars) {                        // a key outside the table is never written
+            if (prev_p != cur) ds[2 * cur] = (int32_t)i;
+            if (i + 1 == n || next_p != cur) ds[2 * cur + 1] = (int32_t)(i + 1);
+        }
+        if (prev_p != cur) { zfrom = prev_p + 1; zto = cur - 1; }
+    }
+    if (zfrom < 0) zfrom = 0;
+    if (zto > num_pillars - 1) zto = num_pillars - 1;
+    const int lane = pccnn_lane();
+    unsigned long long todo = __ballot(zto >= zfrom);
+    while (todo) {
+        const int src = __builtin_ctzll(todo);
+        todo &= todo - 1;
+        const long long f = pccnn_bcast_ll(zfrom, src) * 2, t = pccnn_bcast_ll(zto, src) * 2 + 1;
+        for (long long c = f + lane; c <= t; c += 64) ds[c] = 0;
+    }
+    if (!TABLE) return;
+    if (from < 0) from = 0;
+    if (to > total_cells) to = total_cells;
+    todo = __ballot(to >= from);
+    while (todo) {
+        const int src = __builtin_ctzll(todo);
+        todo &= todo - 1;
+        const long long f = pccnn_bcast_ll(from, src), t = pccnn_bcast_ll(to, src);
+        const int32_t v = (int32_t)pccnn_bcast_ll((long long)i, src);
+        for (long long c = f + lane; c <= t; c += 64) table[c] = v;
+    }
+}
+
+static int grid_tables(const int64_t *sorted_keys, int64_t n, const int32_t *num_cells, int d, int64_t num_pillars,
+                       int64_t total_cells, int32_t *grid_ds_out, int32_t *cell_table_out, hipStream_t s)
+{
+    PCCNN_REQUIRE(d >= 2 && d <= PCCNN_MAX_DIMS, PCCNN_ERR_UNSUPPORTED,
+                  "pccnn_grid_build: d=%d is not supported (2 <= d <= 6)", d);
+    PCCNN_REQUIRE(n >= 0 && n < (1ll << 31) && num_pillars > 0 && num_pillars < (1ll << 30), PCCNN_ERR_INVALID,
+                  "pccnn_grid_build: n=%lld num_pillars=%lld", (long long)n, (long long)num_pillars);
+    PCCNN_REQUIRE(grid_ds_out && num_cells && (n == 0 || sorted_keys), PCCNN_ERR_INVALID,
+                  "pccnn_grid_build: null pointer");
+    PCCNN_REQUIRE(cell_table_out == nullptr || (total_cells > 0 && total_cells < (1ll << 40)), PCCNN_ERR_INVALID,
+                  "pccnn_grid_build: total_cells=%lld", (long long)total_cells);
+    PccnnTimed timed(PCCNN_T_GRID, s);
+    const unsigned blocks = (unsigned)pccnn_ceil_div(n + 1, 256);
+#define GRID_TABLES_GO(D)                                                                                        \
+    do {                                                                                                         \
+        if (cell_table_out != nullptr)                                                                           \
+            grid_tables_kernel<D, true><<<blocks, 256, 0, s>>>(sorted_keys, n, num_cells, num_pillars, total_cells, \
+                                                               grid_ds_out, cell_table_out);                     \
+        else                                                                                                     \
+            grid_tables_kernel<D, false><<<blocks, 256, 0, s>>>(sorted_keys, n, num_cells, num_pillars, 0,         \
+                                                                grid_ds_out, nullptr);                           \
+    } while (0)
+    switch (d) {
+    case 2: GRID_TABLES_GO(2); break;
+    case 3: GRID_TABLES_GO(3); break;
+    case 4: GRID_TABLES_GO(4); break;
+    case 5: GRID_TABLES_GO(5); break;
+    default: GRID_TABLES_GO(6); break;
+    }
+#undef GRID_TABLES_GO
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
 // ------------------------------------------------------------------- the four steps of a grid in one call
 // Keys, stable sort (with the gather of the coordinates), pillar table and, when asked for, the per-cell start
 // table: what Grid.compute_cell_ids + Grid.build_ds of the reference do (pccnn_lib/pc/Grid.py:40-72), as one entry
@@ -310,8 +402,8 @@ extern "C" int pccnn_grid_build(const float *pts, const int32_t *batch_ids, cons
     rc = pccnn_sort_keys(keys_out, n, key_bits, sorted_keys_out, perm_out, pts, d, sorted_pts_out, workspace,
                          workspace_bytes, stream);
     if (rc != PCCNN_OK) return rc;
-    rc = pccnn_build_grid_ds(sorted_keys_out, n, num_cells, d, num_pillars, grid_ds_out, stream);
-    if (rc != PCCNN_OK || cell_table_out == nullptr) return rc;
-    return pccnn_build_cell_table(sorted_keys_out, n, total_cells, cell_table_out, stream);
+    // pillar table and cell table from one launch
+    return grid_tables(sorted_keys_out, n, num_cells, d, num_pillars, total_cells, grid_ds_out, cell_table_out,
+                       (hipStream_t)stream);
 }
 

@@ -13,11 +13,17 @@
 #include "common.h"
 #include "grid_walk.h"
 
+// Also clears what the passes start from: the selection flags and (when given) the 64 counters.
 __global__ void __launch_bounds__(256)
-cell_flag_kernel(const int64_t *__restrict__ keys, int64_t n, int32_t *__restrict__ flags)
+cell_flag_kernel(const int64_t *__restrict__ keys, int64_t n, int32_t *__restrict__ flags,
+                 int32_t *__restrict__ selected, int32_t *__restrict__ counters)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) flags[i] = (i == 0 || keys[i - 1] != keys[i]) ? 1 : 0;
+    if (counters != nullptr && i < 64) counters[i] = 0;
+    if (i < n) {
+        flags[i] = (i == 0 || keys[i - 1] != keys[i]) ? 1 : 0;
+        selected[i] = 0;
+    }
 }
 
 // cell_first[c] = index of the first point of the c-th non-empty cell; *count = number of such cells.
@@ -329,13 +335,12 @@ extern "C" int pccnn_poisson_disk_select(const int64_t *sorted_keys, int64_t n, 
                   workspace_bytes, pccnn_poisson_disk_workspace_bytes(n));
     // the list of non-empty cells (selected_scan_out is free until the end and holds the scan of the flags)
     const unsigned blocks = (unsigned)pccnn_ceil_div(n, 256);
-    cell_flag_kernel<<<blocks, 256, 0, s>>>(sorted_keys, n, flags);
+    cell_flag_kernel<<<blocks, 256, 0, s>>>(sorted_keys, n, flags, selected_out, nullptr);
     PCCNN_LAUNCH_CHECK();
     int rc = pccnn_scan_inclusive_i32(flags, selected_scan_out, n, 0, scan_tmp, s);
     if (rc != PCCNN_OK) return rc;
     cell_list_kernel<<<blocks, 256, 0, s>>>(flags, selected_scan_out, n, cell_first, cell_count);
     PCCNN_LAUNCH_CHECK();
-    if ((rc = pccnn_fill_i32(selected_out, 0, n, s)) != PCCNN_OK) return rc;
     // a fixed number of wavefronts takes the cells in turn: the cell count stays on the device
     int64_t pass_blocks = pccnn_ceil_div(n, 64);
     if (pass_blocks > 2048) pass_blocks = 2048;
@@ -372,11 +377,9 @@ extern "C" int pccnn_poisson_disk_grid(const float *pts_sorted, const int64_t *s
                   workspace_bytes, pccnn_poisson_disk_workspace_bytes(n));
     int32_t *colour_count = cell_count + 8;
     const unsigned blocks = (unsigned)pccnn_ceil_div(n, 256);
-    int rc = pccnn_fill_i32(cell_count, 0, 64, s);
-    if (rc != PCCNN_OK) return rc;
-    cell_flag_kernel<<<blocks, 256, 0, s>>>(sorted_keys, n, flags);
+    cell_flag_kernel<<<blocks, 256, 0, s>>>(sorted_keys, n, flags, selected_out, cell_count);
     PCCNN_LAUNCH_CHECK();
-    rc = pccnn_scan_inclusive_i32(flags, selected_scan_out, n, 0, scan_tmp, s);
+    int rc = pccnn_scan_inclusive_i32(flags, selected_scan_out, n, 0, scan_tmp, s);
     if (rc != PCCNN_OK) return rc;
     cell_list_kernel<<<blocks, 256, 0, s>>>(flags, selected_scan_out, n, cell_first, cell_count);
     PCCNN_LAUNCH_CHECK();
@@ -387,7 +390,6 @@ extern "C" int pccnn_poisson_disk_grid(const float *pts_sorted, const int64_t *s
         cell_colour_kernel<1><<<blocks, 256, 0, s>>>(flags, selected_scan_out, sorted_keys, n, num_cells, colour_list,
                                                      colour_count);
     PCCNN_LAUNCH_CHECK();
-    if ((rc = pccnn_fill_i32(selected_out, 0, n, s)) != PCCNN_OK) return rc;
     PoissonGridArgs a;
     a.pts = pts_sorted;
     a.grid = GridRef{cell_table, total_cells, grid_ds, num_pillars, sorted_keys, n};
