@@ -252,6 +252,15 @@ int pccnn_grid_build_sized(const float *pts, const int32_t *batch_ids, const flo
                            int key_bits, int with_cell_table, int32_t *num_cells_out, int64_t *keys_out,
                            int64_t *sorted_keys_out, int32_t *perm_out, float *sorted_pts_out, int32_t *grid_ds_out,
                            int32_t *cell_table_out, void *workspace, size_t workspace_bytes, void *stream);
+/* The density of every point of a 3-D cloud from its box: pccnn_grid_build_sized (cell size = 4 x bandwidth, into
+ * the workspace) and pccnn_compute_pdf_grid on it, i.e. the whole of pccnn_lib/pc/Pointcloud.py:81-109 after the
+ * bounding box when no gradient is wanted.  No read-back: the call only queues work.  pdf_out / pdf_norm_out
+ * (nullable) f32[n] in the cloud's own order. */
+size_t pccnn_pdf_cloud_workspace_bytes(int64_t n, int64_t num_pillars, int64_t total_cells);
+int pccnn_pdf_cloud(int manifold_dims, const float *bandwidth, const float *pts, const int32_t *batch_ids, int64_t n,
+                    int batch_size, const float *aabb_min, const float *cell_size, const int32_t *num_cells_host,
+                    int key_bits, int with_cell_table, int max_neighbors, float *pdf_out, float *pdf_norm_out,
+                    void *workspace, size_t workspace_bytes, void *stream);
 /* A layer's neighborhood up to the pair count (d == 3): pccnn_grid_build_sized over the cloud, keys and key order
  * of the samples (pccnn_compute_keys + pccnn_sort_keys into sample_keys_tmp i64[m] and sample_keys_out i64[m] /
  * sample_order_out i32[m] / sample_pts_out f32[m,3]; samples == NULL: the cloud itself, m == n, those four unused),

@@ -188,6 +188,52 @@ extern "C" int pccnn_compact_selected_remap(const int32_t *selected, const int32
     return PCCNN_OK;
 }
 
+extern "C" size_t pccnn_pdf_cloud_workspace_bytes(int64_t n, int64_t num_pillars, int64_t total_cells)
+{
+    if (n < 1) n = 1;
+    if (num_pillars < 1) num_pillars = 1;
+    // keys, sorted keys | sorted points | permutation | pillar table | cell table | grid size | sort scratch
+    return 2 * pccnn_align((size_t)n * sizeof(int64_t)) + pccnn_align((size_t)n * 3 * sizeof(float)) +
+           pccnn_align((size_t)n * sizeof(int32_t)) + pccnn_align((size_t)num_pillars * 2 * sizeof(int32_t)) +
+           (total_cells > 0 ? pccnn_align(((size_t)total_cells + 1) * sizeof(int32_t)) : 0) + 256 +
+           pccnn_align(pccnn_grid_build_workspace_bytes(n));
+}
+
+extern "C" int pccnn_pdf_cloud(int manifold_dims, const float *bandwidth, const float *pts, const int32_t *batch_ids,
+                               int64_t n, int batch_size, const float *aabb_min, const float *cell_size,
+                               const int32_t *num_cells_host, int key_bits, int with_cell_table, int max_neighbors,
+                               float *pdf_out, float *pdf_norm_out, void *workspace, size_t workspace_bytes,
+                               void *stream)
+{
+    PCCNN_REQUIRE(n >= 0 && n < (1ll << 31) && batch_size > 0 && num_cells_host, PCCNN_ERR_INVALID,
+                  "pccnn_pdf_cloud: n=%lld batch_size=%d", (long long)n, batch_size);
+    if (n == 0) return PCCNN_OK;
+    for (int k = 0; k < 3; ++k)
+        PCCNN_REQUIRE(num_cells_host[k] > 0, PCCNN_ERR_INVALID, "pccnn_pdf_cloud: %d cells along axis %d",
+                      num_cells_host[k], k);
+    const int64_t num_pillars = (int64_t)batch_size * num_cells_host[0] * num_cells_host[1];
+    const int64_t total_cells = with_cell_table ? num_pillars * num_cells_host[2] : 0;
+    PccnnArena arena(workspace, workspace_bytes);
+    int64_t *keys = arena.take<int64_t>((size_t)n);
+    int64_t *sorted_keys = arena.take<int64_t>((size_t)n);
+    float *sorted_pts = arena.take<float>((size_t)n * 3);
+    int32_t *perm = arena.take<int32_t>((size_t)n);
+    int32_t *grid_ds = arena.take<int32_t>((size_t)num_pillars * 2);
+    int32_t *cell_table = total_cells > 0 ? arena.take<int32_t>((size_t)total_cells + 1) : nullptr;
+    int32_t *num_cells = arena.take<int32_t>(64);
+    const size_t sort_bytes = pccnn_grid_build_workspace_bytes(n);
+    void *sort_ws = arena.take<char>(sort_bytes);
+    PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "pccnn_pdf_cloud: workspace of %zu bytes, need %zu", workspace_bytes,
+                  pccnn_pdf_cloud_workspace_bytes(n, num_pillars, total_cells));
+    int rc = pccnn_grid_build_sized(pts, batch_ids, aabb_min, num_cells_host, cell_size, n, 3, batch_size, key_bits,
+                                    with_cell_table, num_cells, keys, sorted_keys, perm, sorted_pts, grid_ds, cell_table,
+                                    sort_ws, sort_bytes, stream);
+    if (rc != PCCNN_OK) return rc;
+    return pccnn_compute_pdf_grid(manifold_dims, bandwidth, sorted_pts, sorted_keys, n, perm, grid_ds, num_pillars,
+                                  cell_table, total_cells, num_cells, cell_size, 3, max_neighbors, pdf_out, pdf_norm_out,
+                                  stream);
+}
+
 extern "C" int pccnn_grid_build_sized(const float *pts, const int32_t *batch_ids, const float *aabb_min,
                                       const int32_t *num_cells_host, const float *cell_size, int64_t n, int d,
                                       int batch_size, int key_bits, int with_cell_table, int32_t *num_cells_out,

@@ -3,7 +3,12 @@ import torch
 
 from .. import pccnn_lib_ops
 from ..op_wrappers import ComputePDF
-from ._consts import device_vector, host_vector
+from ._consts import device_vector, host_num_cells, host_vector
+
+
+# compute_pdf without gradients (three dimensions, bandwidth known on the host) builds its grid and sums over it in
+# one native call (False: Grid first, then the sum; the result is the same).
+ONE_CALL = True
 
 
 class Pointcloud(object):
@@ -77,6 +82,14 @@ class Pointcloud(object):
         radii = bandwidth * 4.0 if bandwidth_host is None else device_vector(bandwidth_host * np.float32(4.0),
                                                                              self.pts_.shape[1], self.pts_.device)
         aabb = BoundingBox(self)
+        radii_host = host_vector(radii)
+        if ONE_CALL and not self.pts_.requires_grad and self.pts_.shape[1] == 3 and radii_host is not None:
+            # no gradient wanted, three dimensions, bandwidth known on the host: grid and sum in one native call
+            with torch.no_grad():
+                self.pts_unnorm_pdf_, self.pts_pdf_ = pccnn_lib_ops.pdf_cloud(
+                    self.dim_manifold_, bandwidth, self.pts_.detach(), self.batch_ids_, aabb.min_, radii,
+                    host_num_cells(aabb.host(), radii_host), self.batch_size_host(), 300)
+            return
         grid = Grid(self, aabb, radii)
         grid.compute_cell_ids()
         grid.build_ds()

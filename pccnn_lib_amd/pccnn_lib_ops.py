@@ -496,6 +496,42 @@ def compute_pdf_grid(manifold_dims, bandwidth, sorted_pts, sorted_keys, sample_o
     return (out, norm) if with_normalized else out
 
 
+def pdf_cloud(manifold_dims, bandwidth, pts, batch_ids, aabb_min, cell_size, num_cells_host, batch_size,
+              max_neighbors=0):
+    """The density of every point of a 3-D cloud from its box and the grid size on the host: the grid of
+    ``cell_size`` (the search radii) and the sum over it in one native call that only queues work (what
+    pccnn_lib/pc/Pointcloud.py:81-109 computes; the kernels are those of ``grid_build`` and ``compute_pdf_grid``)
+    -> (estimate f32[N], estimate / number of points of the point's cloud f32[N])."""
+    name = "pdf_cloud"
+    _chk(pts, name + ": pts", torch.float32, 2)
+    dev = pts.device
+    _chk(bandwidth, name + ": bandwidth", torch.float32, 1, dev)
+    _chk(batch_ids, name + ": batch_ids", torch.int32, 1, dev)
+    _chk(aabb_min, name + ": aabb_min", torch.float32, 2, dev)
+    _chk(cell_size, name + ": cell_size", torch.float32, 1, dev)
+    n = pts.shape[0]
+    batch_size = int(batch_size)
+    cells = [int(v) for v in num_cells_host]
+    max_neighbors = int(max_neighbors)
+    if pts.shape[1] != 3 or batch_ids.shape[0] != n or tuple(aabb_min.shape) != (batch_size, 3) \
+            or cell_size.shape[0] != 3 or bandwidth.shape[0] != 3 or len(cells) != 3 or min(cells) < 1 \
+            or max_neighbors < 0:
+        raise RuntimeError(name + ": 3-D points [N,3], batch_ids [N], aabb_min [B,3], cell_size / bandwidth [3], "
+                                  "three grid sizes, max_neighbors >= 0")
+    out = torch.empty((2, n), dtype=torch.float32, device=dev)
+    if n == 0:
+        return out[0], out[1]
+    pillars = batch_size * cells[0] * cells[1]
+    total = pillars * cells[2]
+    with_table = 1 if total <= CELL_TABLE_MAX_CELLS else 0
+    ws = _workspace(_lib.load().pccnn_pdf_cloud_workspace_bytes(n, pillars, total if with_table else 0), dev)
+    base = out.data_ptr()
+    _lib.call("pccnn_pdf_cloud", int(manifold_dims), _ptr(bandwidth), _ptr(pts), _ptr(batch_ids), n, batch_size,
+              _ptr(aabb_min), _ptr(cell_size), (ctypes.c_int32 * 3)(*cells), key_bits_for(cells, batch_size), with_table,
+              max_neighbors, _P(base), _P(base + 4 * n), _ptr(ws), ws.numel(), _stream())
+    return out[0], out[1]
+
+
 def compute_pdf_grads(manifold_dims, bandwidth, pts, neigh, ends, in_grads):
     """compute_pdf_grads(..., in_grads f32[N]) -> f32[N,D] (pccnn_lib_ops/compute_pdf/compute_pdf.cuh:45-51)."""
     d = _pdf_args("compute_pdf_grads", bandwidth, pts, neigh, ends)

@@ -431,20 +431,22 @@ def test_grid_size_on_the_host_equals_the_device_result(ops):
 
 
 @pytest.mark.parametrize("batch,num_pts,radius", [(3, 3000, 0.08), (1, 500, 0.3), (4, 20000, 0.04)])
-def test_one_call_pooling_and_neighborhood_equal_the_step_by_step_routes(ops, monkeypatch, batch, num_pts, radius):
-    # PointPooling and Neighborhood run their chain of launches as one native call when the grid size is known on
+def test_one_call_pooling_density_and_neighborhood_equal_the_step_by_step_routes(ops, monkeypatch, batch, num_pts, radius):
+    # PointPooling, Pointcloud.compute_pdf and Neighborhood run their chain of launches as one native call when the grid size is known on
     # the host; the same launches step by step (the route of every other case) must give the same tensors
     import pccnn_lib_amd as lib
-    from pccnn_lib_amd.pc import neighborhood, point_pooling
+    from pccnn_lib_amd.pc import neighborhood, point_cloud, point_pooling
     pts, ids = synthetic.primitives(31 + batch, batch, num_pts)
 
     def run(one_call):
         monkeypatch.setattr(point_pooling, "ONE_CALL", one_call)
         monkeypatch.setattr(neighborhood, "ONE_CALL", one_call)
+        monkeypatch.setattr(point_cloud, "ONE_CALL", one_call)
         pc = lib.pc.Pointcloud(pts, ids, device=DEV)
         pool = lib.pc.PointPooling(pc, radius)
         out_pc = lib.pc.Pointcloud(pool.pool_tensor(pc.pts_), pool.pool_tensor(pc.batch_ids_))
-        got = [pool.pooling_ids_]
+        pc.compute_pdf(0.25 * radius)
+        got = [pool.pooling_ids_, pc.pts_unnorm_pdf_, pc.pts_pdf_]
         for samples, cap, key_order in ((out_pc, 0, False), (pc, 0, False), (out_pc, 5, False), (out_pc, 0, True)):
             grid = lib.pc.Grid(pc, lib.pc.BoundingBox(pc), 2.0 * radius)
             if not one_call:
