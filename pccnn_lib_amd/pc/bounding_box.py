@@ -15,17 +15,22 @@ class BoundingBox(object):
     ``pts_.data`` or ``.detach()`` does not move those counters: after such a write, drop the entry
     (``del cloud.aabb_cache_``) or build a new Pointcloud, else grids keep using the old box."""
 
-    def __init__(self, p_point_cloud):
+    def __init__(self, p_point_cloud, p_with_host=False):
+        """``p_with_host`` (not in the reference): also bring the box to the host, with the same native call, for a
+        caller that is about to size a grid from it on the host; otherwise ``host()`` reads it back when asked."""
         pts, ids = p_point_cloud.pts_, p_point_cloud.batch_ids_
         cached = getattr(p_point_cloud, "aabb_cache_", None)
         if cached is not None and cached[0]() is pts and cached[1] == pts._version and cached[2]() is ids \
                 and cached[3] == ids._version:
             self.min_, self.max_, self.host_ = cached[4], cached[5], cached[6]
             return
-        # every grid over the cloud sizes itself from the box on the host: it comes back with the same native call
-        self.min_, self.max_, host = pccnn_lib_ops.bounding_box_host(pts.detach(), ids,
-                                                                    p_point_cloud.batch_size_host())
-        self.host_ = [host]      # shared by every user of the cache entry
+        if p_with_host:
+            self.min_, self.max_, host = pccnn_lib_ops.bounding_box_host(pts.detach(), ids,
+                                                                        p_point_cloud.batch_size_host())
+        else:
+            self.min_, self.max_ = pccnn_lib_ops.bounding_box(pts.detach(), ids, p_point_cloud.batch_size_host())
+            host = None
+        self.host_ = [host]      # the box on the host, read back at most once and shared by every user of the cache entry
         # weak references: the entry neither keeps replaced tensors alive nor matches a new tensor at a reused address
         p_point_cloud.aabb_cache_ = (weakref.ref(pts), pts._version, weakref.ref(ids), ids._version, self.min_,
                                      self.max_, self.host_)

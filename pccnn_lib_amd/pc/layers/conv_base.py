@@ -1,7 +1,7 @@
 import torch
 
 from ... import pccnn_lib_ops
-from .._consts import device_vector
+from .._consts import device_vector, host_vector
 
 
 # A layer that can run on the grid's sorted copy of its input cloud (``point_side``) builds its own neighborhood in
@@ -17,8 +17,9 @@ def build_neighborhood(p_pc_in, p_pc_out, p_radius, p_max_neighs, p_key_order=Fa
     from ..bounding_box import BoundingBox
     from ..grid import Grid
     from ..neighborhood import Neighborhood
-    bb = BoundingBox(p_pc_in)
-    grid = Grid(p_pc_in, bb, p_radius)
+    radius = device_vector(p_radius, p_pc_in.pts_.shape[1], p_pc_in.pts_.device)
+    bb = BoundingBox(p_pc_in, host_vector(radius) is not None)
+    grid = Grid(p_pc_in, bb, radius)
     return Neighborhood(grid, p_pc_out, p_max_neighs, p_key_order)     # builds the grid
 
 

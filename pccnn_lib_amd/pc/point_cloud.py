@@ -81,8 +81,8 @@ class Pointcloud(object):
         # four bandwidths (exact in fp32: a power of two), from the host values when they are known
         radii = bandwidth * 4.0 if bandwidth_host is None else device_vector(bandwidth_host * np.float32(4.0),
                                                                              self.pts_.shape[1], self.pts_.device)
-        aabb = BoundingBox(self)
         radii_host = host_vector(radii)
+        aabb = BoundingBox(self, radii_host is not None)
         if ONE_CALL and not self.pts_.requires_grad and self.pts_.shape[1] == 3 and radii_host is not None:
             # no gradient wanted, three dimensions, bandwidth known on the host: grid and sum in one native call
             with torch.no_grad():

@@ -23,10 +23,10 @@ class PointPooling(object):
         self.radii_ = p_radii
         self.method_ = p_method
         with torch.no_grad():
-            bb = BoundingBox(p_point_cloud)
+            cell = device_vector(p_radii, p_point_cloud.pts_.shape[1], p_point_cloud.pts_.device)
+            cell_host = host_vector(cell)
+            bb = BoundingBox(p_point_cloud, cell_host is not None)
             if ONE_CALL and p_method == "poisson_disk" and p_point_cloud.pts_.shape[1] == 3:
-                cell = device_vector(p_radii, 3, p_point_cloud.pts_.device)
-                cell_host = host_vector(cell)
                 if cell_host is not None:
                     # three dimensions, cell size known on the host: grid, selection and its size in one native call
                     self.pooling_ids_ = pccnn_lib_ops.pool_poisson(
