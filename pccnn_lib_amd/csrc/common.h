@@ -204,6 +204,19 @@ extern "C" int pccnn_gemm_bf16(const uint16_t *a, const uint16_t *b, float *c, i
                                int batch, int64_t stride_a, int64_t stride_b, int64_t stride_c, int split_k,
                                void *workspace, size_t workspace_bytes, void *stream);
 
+// A grid size by value (kernel argument), and the key computation that takes it that way (keys_grid.hip).
+struct PccnnGridDims {
+    int v[PCCNN_MAX_DIMS];
+};
+int pccnn_compute_keys_sized(const float *pts, const int32_t *batch_ids, const float *aabb_min,
+                             const int32_t *num_cells_host, const float *cell_size, int64_t n, int d,
+                             int32_t *num_cells_out, int64_t *keys_out, hipStream_t stream);
+// The rest of pccnn_grid_build after the keys: sort, pillar table, cell table (keys_grid.hip).
+int pccnn_grid_build_from_keys(const int64_t *keys, const float *pts, const int32_t *num_cells, int64_t n, int d,
+                               int key_bits, int64_t num_pillars, int64_t total_cells, int64_t *sorted_keys_out,
+                               int32_t *perm_out, float *sorted_pts_out, int32_t *grid_ds_out, int32_t *cell_table_out,
+                               void *workspace, size_t workspace_bytes, void *stream);
+
 // Internal sort entry used by other translation units.
 int pccnn_fill_i32(int32_t *p, int32_t value, int64_t count, hipStream_t stream);
 int pccnn_fill_f32(float *p, float value, int64_t count, hipStream_t stream);

@@ -211,13 +211,17 @@ extern "C" int pccnn_num_cells(const float *aabb_min, const float *aabb_max, con
 
 // ------------------------------------------------------------------- keys
 
-template <int D>
+// SIZED: the grid size arrives by value (`sized`), and the first workgroup also writes it to num_cells_out, where the
+// kernels after this one read it; otherwise it is read from num_cells.
+template <int D, bool SIZED>
 __global__ void __launch_bounds__(256)
 compute_keys_kernel(const float *__restrict__ pts, const int32_t *__restrict__ batch_ids,
                     const float *__restrict__ aabb_min, const int32_t *__restrict__ num_cells,
-                    const float *__restrict__ cell_size, int64_t n, int64_t *__restrict__ keys)
+                    const float *__restrict__ cell_size, int64_t n, int64_t *__restrict__ keys, PccnnGridDims sized,
+                    int32_t *__restrict__ num_cells_out)
 {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (SIZED && blockIdx.x == 0 && threadIdx.x < D) num_cells_out[threadIdx.x] = sized.v[threadIdx.x];
     if (i >= n) return;
     int b = batch_ids[i];
     long long key = 0, accum = 1;
@@ -227,7 +231,7 @@ compute_keys_kernel(const float *__restrict__ pts, const int32_t *__restrict__ b
         // reciprocal of the cell size, floor, clamp.
         float inv = __fdiv_rn(1.0f, cell_size[k]);
         float rel = (pts[i * D + k] - aabb_min[(int64_t)b * D + k]) * inv;
-        int nc = num_cells[k];
+        int nc = SIZED ? sized.v[k] : num_cells[k];
         int c = (int)floorf(rel);
         c = max(0, min(c, nc - 1));
         key += (long long)c * accum;
@@ -247,8 +251,48 @@ extern "C" int pccnn_compute_keys(const float *pts, const int32_t *batch_ids, co
     PCCNN_REQUIRE(pts && batch_ids && aabb_min && num_cells && cell_size && keys_out, PCCNN_ERR_INVALID,
                   "pccnn_compute_keys: null pointer");
     PccnnTimed timed(PCCNN_T_KEYS, (hipStream_t)stream);
-    PCCNN_DIM_DISPATCH(d, compute_keys_kernel, <<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, (hipStream_t)stream>>>(
-        pts, batch_ids, aabb_min, num_cells, cell_size, n, (int64_t *)keys_out));
+    const unsigned blocks = (unsigned)pccnn_ceil_div(n, 256);
+    hipStream_t s = (hipStream_t)stream;
+    const PccnnGridDims none = {};
+#define KEYS_GO(D) compute_keys_kernel<D, false><<<blocks, 256, 0, s>>>(pts, batch_ids, aabb_min, num_cells, cell_size, n, \
+                                                                       (int64_t *)keys_out, none, nullptr)
+    switch (d) {
+    case 2: KEYS_GO(2); break;
+    case 3: KEYS_GO(3); break;
+    case 4: KEYS_GO(4); break;
+    case 5: KEYS_GO(5); break;
+    default: KEYS_GO(6); break;
+    }
+#undef KEYS_GO
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
+// pccnn_compute_keys for a grid size known on the host (d ints): the keys are computed from those numbers, and the
+// same launch writes them to num_cells_out i32[d] on the device for the kernels that follow.
+int pccnn_compute_keys_sized(const float *pts, const int32_t *batch_ids, const float *aabb_min,
+                             const int32_t *num_cells_host, const float *cell_size, int64_t n, int d,
+                             int32_t *num_cells_out, int64_t *keys_out, hipStream_t s)
+{
+    PCCNN_REQUIRE(d >= 2 && d <= PCCNN_MAX_DIMS, PCCNN_ERR_UNSUPPORTED,
+                  "pccnn_compute_keys: d=%d is not supported (2 <= d <= 6)", d);
+    PCCNN_REQUIRE(n >= 0, PCCNN_ERR_INVALID, "pccnn_compute_keys: n=%lld", (long long)n);
+    PCCNN_REQUIRE(num_cells_host && num_cells_out && cell_size && aabb_min && (n == 0 || (pts && batch_ids && keys_out)),
+                  PCCNN_ERR_INVALID, "pccnn_compute_keys: null pointer");
+    PccnnGridDims dims = {};
+    for (int k = 0; k < d; ++k) dims.v[k] = num_cells_host[k];
+    PccnnTimed timed(PCCNN_T_KEYS, s);
+    const unsigned blocks = (unsigned)pccnn_ceil_div(n > 0 ? n : 1, 256);       // n == 0: the size is still written
+#define KEYS_GO(D) compute_keys_kernel<D, true><<<blocks, 256, 0, s>>>(pts, batch_ids, aabb_min, nullptr, cell_size, n, \
+                                                                      keys_out, dims, num_cells_out)
+    switch (d) {
+    case 2: KEYS_GO(2); break;
+    case 3: KEYS_GO(3); break;
+    case 4: KEYS_GO(4); break;
+    case 5: KEYS_GO(5); break;
+    default: KEYS_GO(6); break;
+    }
+#undef KEYS_GO
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
 }
@@ -399,8 +443,18 @@ extern "C" int pccnn_grid_build(const float *pts, const int32_t *batch_ids, cons
 {
     int rc = pccnn_compute_keys(pts, batch_ids, aabb_min, num_cells, cell_size, n, d, keys_out, stream);
     if (rc != PCCNN_OK) return rc;
-    rc = pccnn_sort_keys(keys_out, n, key_bits, sorted_keys_out, perm_out, pts, d, sorted_pts_out, workspace,
-                         workspace_bytes, stream);
+    return pccnn_grid_build_from_keys(keys_out, pts, num_cells, n, d, key_bits, num_pillars, total_cells,
+                                      sorted_keys_out, perm_out, sorted_pts_out, grid_ds_out, cell_table_out, workspace,
+                                      workspace_bytes, stream);
+}
+
+int pccnn_grid_build_from_keys(const int64_t *keys, const float *pts, const int32_t *num_cells, int64_t n, int d,
+                               int key_bits, int64_t num_pillars, int64_t total_cells, int64_t *sorted_keys_out,
+                               int32_t *perm_out, float *sorted_pts_out, int32_t *grid_ds_out, int32_t *cell_table_out,
+                               void *workspace, size_t workspace_bytes, void *stream)
+{
+    int rc = pccnn_sort_keys(keys, n, key_bits, sorted_keys_out, perm_out, pts, d, sorted_pts_out, workspace,
+                             workspace_bytes, stream);
     if (rc != PCCNN_OK) return rc;
     // pillar table and cell table from one launch
     return grid_tables(sorted_keys_out, n, num_cells, d, num_pillars, total_cells, grid_ds_out, cell_table_out,

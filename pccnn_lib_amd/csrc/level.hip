@@ -43,31 +43,19 @@ int read_back(void *host_out, const void *dev, size_t bytes, hipStream_t s)
     return PCCNN_OK;
 }
 
-struct GridDims {
-    int v[PCCNN_MAX_DIMS];
-};
-
-__global__ void set_dims_kernel(int32_t *dst, GridDims dims, int d)
+// checks a grid size given on the host and derives the numbers of pillars and cells
+int grid_extent(const char *who, const int32_t *num_cells_host, int d, int batch_size, int64_t *num_pillars,
+                int64_t *total_cells)
 {
-    if ((int)threadIdx.x < d) dst[threadIdx.x] = dims.v[threadIdx.x];
-}
-
-// the grid size, known on the host, as the device vector the kernels read; also checks it
-int put_grid_dims(const char *who, const int32_t *num_cells_host, int d, int batch_size, int32_t *dst, hipStream_t s,
-                  int64_t *num_pillars, int64_t *total_cells)
-{
-    GridDims dims;
     int64_t total = batch_size;
     for (int k = 0; k < d; ++k) {
-        dims.v[k] = num_cells_host[k];
-        PCCNN_REQUIRE(dims.v[k] > 0, PCCNN_ERR_INVALID, "%s: %d cells along axis %d", who, dims.v[k], k);
-        PCCNN_REQUIRE(total <= INT64_MAX / dims.v[k], PCCNN_ERR_INVALID, "%s: the cell count overflows 64 bits", who);
-        total *= dims.v[k];
+        const int c = num_cells_host[k];
+        PCCNN_REQUIRE(c > 0, PCCNN_ERR_INVALID, "%s: %d cells along axis %d", who, c, k);
+        PCCNN_REQUIRE(total <= INT64_MAX / c, PCCNN_ERR_INVALID, "%s: the cell count overflows 64 bits", who);
+        total *= c;
     }
-    *num_pillars = (int64_t)batch_size * dims.v[0] * dims.v[1];
+    *num_pillars = (int64_t)batch_size * num_cells_host[0] * num_cells_host[1];
     *total_cells = total;
-    set_dims_kernel<<<1, 64, 0, s>>>(dst, dims, d);
-    PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
 }
 
@@ -157,13 +145,9 @@ extern "C" int pccnn_pool_poisson_select(const float *pts, const int32_t *batch_
                   "pccnn_pool_poisson_select: workspace of %zu bytes, need %zu", workspace_bytes,
                   pccnn_pool_poisson_workspace_bytes(n, num_pillars, total_cells));
     hipStream_t s = (hipStream_t)stream;
-    int64_t all_cells;
-    int rc = put_grid_dims("pccnn_pool_poisson_select", num_cells_host, 3, batch_size, l.num_cells, s, &num_pillars,
-                           &all_cells);
-    if (rc != PCCNN_OK) return rc;
-    rc = pccnn_grid_build(pts, batch_ids, aabb_min, l.num_cells, cell_size, n, 3, key_bits, num_pillars, total_cells,
-                              l.keys, l.sorted_keys, perm_out, l.sorted_pts, l.grid_ds, l.cell_table, l.sort_ws,
-                              l.sort_bytes, stream);
+    int rc = pccnn_grid_build_sized(pts, batch_ids, aabb_min, num_cells_host, cell_size, n, 3, batch_size, key_bits,
+                                    with_cell_table, l.num_cells, l.keys, l.sorted_keys, perm_out, l.sorted_pts,
+                                    l.grid_ds, l.cell_table, l.sort_ws, l.sort_bytes, stream);
     if (rc != PCCNN_OK) return rc;
     rc = pccnn_poisson_disk_grid(l.sorted_pts, l.sorted_keys, n, l.grid_ds, num_pillars, l.cell_table, total_cells,
                                  l.num_cells, cell_size, 3, selected_out, selected_scan_out, l.poisson_ws,
@@ -248,12 +232,15 @@ extern "C" int pccnn_grid_build_sized(const float *pts, const int32_t *batch_ids
     PCCNN_REQUIRE(!with_cell_table || (cell_table_out && d == 3), PCCNN_ERR_INVALID,
                   "pccnn_grid_build_sized: the cell table needs its output and d == 3");
     int64_t num_pillars, total_cells;
-    int rc = put_grid_dims("pccnn_grid_build_sized", num_cells_host, d, batch_size, num_cells_out, (hipStream_t)stream,
-                           &num_pillars, &total_cells);
+    int rc = grid_extent("pccnn_grid_build_sized", num_cells_host, d, batch_size, &num_pillars, &total_cells);
     if (rc != PCCNN_OK) return rc;
-    return pccnn_grid_build(pts, batch_ids, aabb_min, num_cells_out, cell_size, n, d, key_bits, num_pillars,
-                            with_cell_table ? total_cells : 0, keys_out, sorted_keys_out, perm_out, sorted_pts_out,
-                            grid_ds_out, with_cell_table ? cell_table_out : nullptr, workspace, workspace_bytes, stream);
+    rc = pccnn_compute_keys_sized(pts, batch_ids, aabb_min, num_cells_host, cell_size, n, d, num_cells_out, keys_out,
+                                  (hipStream_t)stream);
+    if (rc != PCCNN_OK) return rc;
+    return pccnn_grid_build_from_keys(keys_out, pts, num_cells_out, n, d, key_bits, num_pillars,
+                                      with_cell_table ? total_cells : 0, sorted_keys_out, perm_out, sorted_pts_out,
+                                      grid_ds_out, with_cell_table ? cell_table_out : nullptr, workspace,
+                                      workspace_bytes, stream);
 }
 
 extern "C" int pccnn_neighborhood_count(const float *pts, const int32_t *batch_ids, int64_t n, int batch_size,
