@@ -156,6 +156,53 @@ __global__ void bbox_pad_kernel(float *mn, float *mx, int count)
     if (i < count) { mn[i] = mn[i] - 1e-6f; mx[i] = mx[i] + 1e-6f; }
 }
 
+// A small cloud (up to BBOX_SMALL_POINTS points, up to BBOX_SMALL_CLOUDS clouds): one workgroup, the boxes in LDS,
+// initial values, reduction and padding in one launch instead of three.  Same minima and maxima (they do not depend
+// on the order of the comparisons), same padding.
+#define BBOX_SMALL_POINTS 16384
+#define BBOX_SMALL_CLOUDS 64
+template <int D>
+__global__ void __launch_bounds__(1024)
+bbox_small_kernel(const float *__restrict__ pts, const int32_t *__restrict__ batch_ids, int64_t n, int batch_size,
+                  float *__restrict__ mn, float *__restrict__ mx)
+{
+    __shared__ float box_lo[BBOX_SMALL_CLOUDS * D], box_hi[BBOX_SMALL_CLOUDS * D];
+    const float inf = __int_as_float(0x7f800000);
+    const int count = batch_size * D;
+    for (int i = threadIdx.x; i < count; i += blockDim.x) { box_lo[i] = inf; box_hi[i] = -inf; }
+    __syncthreads();
+    int cur = -1;
+    float lo[D], hi[D];
+#pragma unroll
+    for (int k = 0; k < D; ++k) { lo[k] = inf; hi[k] = -inf; }
+    // the same trip count for every thread: the wavefront-wide flush sits in uniform control flow
+    for (int64_t w0 = 0; w0 < n; w0 += blockDim.x) {
+        const int64_t i = w0 + threadIdx.x;
+        int b = -1;
+        float v[D];
+        if (i < n) {
+            b = batch_ids[i];
+            if (b < 0 || b >= batch_size) b = -1;                      // ids outside the table are ignored
+#pragma unroll
+            for (int k = 0; k < D; ++k) v[k] = pts[i * D + k];
+        }
+        if (__any(b >= 0 && cur >= 0 && b != cur)) {
+            bbox_flush_wave<D>(cur, lo, hi, box_lo, box_hi);
+            cur = -1;
+#pragma unroll
+            for (int k = 0; k < D; ++k) { lo[k] = inf; hi[k] = -inf; }
+        }
+        if (b >= 0) {
+            cur = b;
+#pragma unroll
+            for (int k = 0; k < D; ++k) { lo[k] = fminf(lo[k], v[k]); hi[k] = fmaxf(hi[k], v[k]); }
+        }
+    }
+    bbox_flush_wave<D>(cur, lo, hi, box_lo, box_hi);
+    __syncthreads();
+    for (int i = threadIdx.x; i < count; i += blockDim.x) { mn[i] = box_lo[i] - 1e-6f; mx[i] = box_hi[i] + 1e-6f; }
+}
+
 extern "C" int pccnn_bounding_box(const float *pts, const int32_t *batch_ids, int64_t n, int d, int batch_size,
                                   float *aabb_min_out, float *aabb_max_out, void *stream)
 {
@@ -167,6 +214,12 @@ extern "C" int pccnn_bounding_box(const float *pts, const int32_t *batch_ids, in
                   "pccnn_bounding_box: null pointer");
     hipStream_t s = (hipStream_t)stream;
     int count = batch_size * d;
+    if (n > 0 && n <= BBOX_SMALL_POINTS && batch_size <= BBOX_SMALL_CLOUDS) {
+        PCCNN_DIM_DISPATCH(d, bbox_small_kernel, <<<1, 1024, 0, s>>>(pts, batch_ids, n, batch_size, aabb_min_out,
+                                                                    aabb_max_out));
+        PCCNN_LAUNCH_CHECK();
+        return PCCNN_OK;
+    }
     bbox_init_kernel<<<(unsigned)pccnn_ceil_div(count, 256), 256, 0, s>>>(aabb_min_out, aabb_max_out, count);
     PCCNN_LAUNCH_CHECK();
     if (n > 0) {

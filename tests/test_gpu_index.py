@@ -471,3 +471,21 @@ def test_bounding_box_comes_back_on_the_host_with_the_same_call(ops):
     assert torch.equal(mn, mn2) and torch.equal(mx, mx2)
     assert np.array_equal(host_mn, mn.cpu().numpy()) and np.array_equal(host_mx, mx.cpu().numpy())
     assert host_mn.dtype == np.float32 and host_mn.shape == (5, 3)
+
+
+@pytest.mark.parametrize("num_pts,batch", [(1000, 7), (16384, 64), (16385, 3), (40000, 70)])
+def test_bounding_box_with_interleaved_clouds_and_an_empty_one(ops, num_pts, batch):
+    # the one-workgroup kernel of small inputs and the chunked one, on batch ids in no order, with one cloud that has
+    # no points: minima and maxima equal numpy's, padded by 1e-6 in fp32 (BoundingBox.py:17-18)
+    rng = np.random.default_rng(num_pts + batch)
+    pts = rng.normal(size=(num_pts, 3)).astype(np.float32)
+    ids = rng.integers(0, batch - 1, num_pts).astype(np.int32)          # cloud batch - 1 stays empty
+    mn, mx = ops.bounding_box(t(pts), t(ids), batch)
+    mn, mx = mn.cpu().numpy(), mx.cpu().numpy()
+    for b in range(batch - 1):
+        sel = pts[ids == b]
+        if sel.shape[0] == 0:
+            continue
+        assert np.array_equal(mn[b], sel.min(axis=0) - np.float32(1e-6))
+        assert np.array_equal(mx[b], sel.max(axis=0) + np.float32(1e-6))
+    assert np.all(np.isposinf(mn[batch - 1])) and np.all(np.isneginf(mx[batch - 1]))
