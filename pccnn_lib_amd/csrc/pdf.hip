@@ -194,7 +194,11 @@ __device__ __forceinline__ int pdf_grid_cloud_count(const PdfGridArgs &a, long l
 
 #define PDF_GRID_UNROLL 4
 
-template <bool CAPPED>
+// QUARTER: the search radius is exactly four bandwidths on every axis (what Pointcloud.compute_pdf asks for), i.e.
+// 1 / radius == (1 / bandwidth) / 4 bit for bit.  Scaling by a power of two is exact, so the kernel's argument
+// ((p - s) / bandwidth)^2 is then 16 x the predicate's ((s - p) / radius)^2, rounding included, and is not computed
+// a second time.
+template <bool CAPPED, bool QUARTER>
 __device__ __forceinline__ void pdf_grid_walk(const PdfGridArgs &a, const int2 (*ranges)[64], int lane, int nr, bool go,
                                               float sx, float sy, float sz, const float (&ir)[3], const float (&ib)[3],
                                               double scale, int raw, int step, double &sum, int &cnt)
@@ -234,10 +238,15 @@ __device__ __forceinline__ void pdf_grid_walk(const PdfGridArgs &a, const int2 (
                     }
                     if (take) {
                         // the term of pdf_kernel: ((p - s) / bandwidth)^2 summed in fp32, exp in fp32, scaled in double
-                        const float d0 = (px[u] - sx) * ib[0];
-                        const float d1 = (py[u] - sy) * ib[1];
-                        const float d2 = (pz[u] - sz) * ib[2];
-                        const float dot = ((0.0f + d0 * d0) + d1 * d1) + d2 * d2;
+                        float dot;
+                        if (QUARTER) {
+                            dot = acc * 16.0f;
+                        } else {
+                            const float d0 = (px[u] - sx) * ib[0];
+                            const float d1 = (py[u] - sy) * ib[1];
+                            const float d2 = (pz[u] - sz) * ib[2];
+                            dot = ((0.0f + d0 * d0) + d1 * d1) + d2 * d2;
+                        }
                         sum += scale * (double)expf(dot * (-0.5f));
                     }
                     ++cnt;
@@ -311,13 +320,15 @@ pdf_grid_kernel(PdfGridArgs a)
     }
     double sum = 0.0;
     int cnt = 0;
-    pdf_grid_walk<false>(a, ranges[wib], lane, nr, usable, sx, sy, sz, ir, ib, scale, 0, 0, sum, cnt);
+    const bool quarter = ir[0] * 4.0f == ib[0] && ir[1] * 4.0f == ib[1] && ir[2] * 4.0f == ib[2];     // uniform
+    if (quarter) pdf_grid_walk<false, true>(a, ranges[wib], lane, nr, usable, sx, sy, sz, ir, ib, scale, 0, 0, sum, cnt);
+    else pdf_grid_walk<false, false>(a, ranges[wib], lane, nr, usable, sx, sy, sz, ir, ib, scale, 0, 0, sum, cnt);
     const bool redo = a.max_neighbors > 0 && cnt > a.max_neighbors;
     if (__any(redo)) {
         double capped_sum = 0.0;
         int again = 0;
-        pdf_grid_walk<true>(a, ranges[wib], lane, nr, redo, sx, sy, sz, ir, ib, scale, cnt, a.max_neighbors, capped_sum,
-                            again);
+        pdf_grid_walk<true, false>(a, ranges[wib], lane, nr, redo, sx, sy, sz, ir, ib, scale, cnt, a.max_neighbors,
+                                   capped_sum, again);
         if (redo) sum = capped_sum;
     }
     if (valid) {
