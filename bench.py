@@ -231,7 +231,10 @@ def config5_leg(lib, dev, steps, warmup):
             pc.compute_pdf(0.2 * radius)
             feats, nbh = layers[level](pc, out_pc, feats, 2.0 * radius)
             feats = torch.nn.functional.leaky_relu(feats, 0.2)
-            sizes.append((int(pc.pts_.shape[0]), int(out_pc.pts_.shape[0]), int(nbh.neighbors_.shape[0])))
+            # (the pair count from the list the search kept: reading neighbors_ of a key-order list would make the
+            # original-index copy just for its shape)
+            kept = nbh.neighbors_original_ if nbh.neighbors_original_ is not None else nbh.neighbors_key_order_
+            sizes.append((int(pc.pts_.shape[0]), int(out_pc.pts_.shape[0]), int(kept.shape[0])))
             pc = out_pc
         if split:
             torch.cuda.synchronize()
