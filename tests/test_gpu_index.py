@@ -489,3 +489,36 @@ def test_bounding_box_with_interleaved_clouds_and_an_empty_one(ops, num_pts, bat
         assert np.array_equal(mn[b], sel.min(axis=0) - np.float32(1e-6))
         assert np.array_equal(mx[b], sel.max(axis=0) + np.float32(1e-6))
     assert np.all(np.isposinf(mn[batch - 1])) and np.all(np.isneginf(mx[batch - 1]))
+
+
+@pytest.mark.parametrize("use_table", [True, False])
+def test_poisson_disk_from_the_grid_on_a_large_cloud_equals_the_list_version(ops, use_table):
+    # The list-free selection at the size of a hierarchy's first level: a room plus two tight clusters, so that most
+    # cells hold a few points and some hold hundreds (several rounds of 64 per cell, index ranges longer than the 64
+    # flags a wavefront requests at once).  The neighbor-list version (itself checked against the oracle at small
+    # sizes) must pick the same points.
+    rng = np.random.default_rng(8)
+    room = (synthetic.room(21, 230000) / 10.0).astype(np.float32)
+    blobs = np.concatenate([rng.normal((0.3, 0.4, 0.1), 0.004, (9000, 3)),
+                            rng.normal((0.71, 0.22, 0.05), 0.002, (6000, 3))]).astype(np.float32)
+    pts = np.concatenate([room, blobs])[rng.permutation(room.shape[0] + blobs.shape[0])]
+    ids = np.zeros(pts.shape[0], np.int32)
+    ids[pts.shape[0] // 2:] = 1
+    radius = 0.012
+    g = gpu_neighborhood(ops, pts, ids, pts, ids, radius, 2)["dev"]
+    table = ops.build_cell_table(g["skeys"], 2 * int(np.prod(g["nc"].tolist()))) if use_table else None
+    sel = ops.poisson_disk_sampling_grid(g["spts"], g["skeys"], g["ds"], g["nc"], g["radii"], cell_table=table)
+    neigh, ends = ops.find_neighbors_ex(g["spts"], g["skeys"], g["spts"], g["skeys"], g["ds"], g["nc"], g["radii"], 0)
+    counts = torch.diff(ends, prepend=ends.new_zeros(1))
+    assert int(counts.max()) > 200                       # the clusters are there
+    want = ops.poisson_disk_sampling(g["skeys"], neigh, ends, g["nc"])
+    assert sel.shape[0] > 1000 and torch.equal(sel, want)
+    # the selection is a maximal independent set: no two selected points are neighbors, every other point has one
+    chosen = torch.zeros(pts.shape[0], dtype=torch.bool, device=DEV)
+    chosen[sel.reshape(-1)] = True
+    pair_pt, pair_sample = neigh[:, 0].to(torch.int64), neigh[:, 1].to(torch.int64)
+    both = chosen[pair_pt] & chosen[pair_sample] & (pair_pt != pair_sample)
+    assert not bool(both.any())
+    covered = torch.zeros(pts.shape[0], dtype=torch.bool, device=DEV)
+    covered[pair_sample[chosen[pair_pt]]] = True
+    assert bool(covered.all())
