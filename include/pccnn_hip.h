@@ -233,14 +233,19 @@ int pccnn_bounding_box_host(const float *pts, const int32_t *batch_ids, int64_t 
  * size as three host ints (pccnn_num_cells' arithmetic on the host copy of the box); key_bits as pccnn_sort_keys;
  * with_cell_table != 0 builds the per-cell table for the walk.  Outputs: perm_out i32[n] (original index of sorted
  * point i), selected_out / selected_scan_out i32[n] as pccnn_poisson_disk_grid (sorted-index space), *count_out
- * (host) = number of selected points.  pccnn_compact_selected_remap then writes remap[i] of the selected i,
- * ascending in i, as i64: with remap = perm_out these are PointPooling's pooling_ids_ (PointPooling.py:66-69). */
+ * (host) = number of selected points.  pooled_min_out / pooled_max_out (device, f32[batch_size,3]; all four NULL to
+ * skip) receive the bounding box of the selected points per cloud, i.e. pccnn_bounding_box of the pooled cloud a
+ * caller is about to build from them (pccnn_lib/pc/BoundingBox.py:17-18 on PointPooling's output), and
+ * pooled_host_min_out / pooled_host_max_out (host) the same values, read back together with the count.
+ * pccnn_compact_selected_remap then writes remap[i] of the selected i, ascending in i, as i64: with
+ * remap = perm_out these are PointPooling's pooling_ids_ (PointPooling.py:66-69). */
 size_t pccnn_pool_poisson_workspace_bytes(int64_t n, int64_t num_pillars, int64_t total_cells);
 int pccnn_pool_poisson_select(const float *pts, const int32_t *batch_ids, int64_t n, int batch_size,
                               const float *aabb_min, const float *cell_size, const int32_t *num_cells_host,
                               int key_bits, int with_cell_table, int32_t *perm_out, int32_t *selected_out,
-                              int32_t *selected_scan_out, int64_t *count_out, void *workspace,
-                              size_t workspace_bytes, void *stream);
+                              int32_t *selected_scan_out, int64_t *count_out, float *pooled_min_out,
+                              float *pooled_max_out, float *pooled_host_min_out, float *pooled_host_max_out,
+                              void *workspace, size_t workspace_bytes, void *stream);
 int pccnn_compact_selected_remap(const int32_t *selected, const int32_t *selected_scan, const int32_t *remap,
                                  int64_t n, int64_t *ids_out, void *stream);
 /* pccnn_grid_build for a grid whose size is known on the host (num_cells_host: d host ints): writes that size to

@@ -54,7 +54,7 @@ SIGNATURES = {
     "pccnn_poisson_disk_grid": (I32, [P, P, I64, P, I64, P, I64, P, P, I32, P, P, P, SZ, P]),
     "pccnn_bounding_box_host": (I32, [P, P, I64, I32, I32, P, P, P, P, P]),
     "pccnn_pool_poisson_workspace_bytes": (SZ, [I64, I64, I64]),
-    "pccnn_pool_poisson_select": (I32, [P, P, I64, I32, P, P, P, I32, I32, P, P, P, P, P, SZ, P]),
+    "pccnn_pool_poisson_select": (I32, [P, P, I64, I32, P, P, P, I32, I32, P, P, P, P, P, P, P, P, P, SZ, P]),
     "pccnn_compact_selected_remap": (I32, [P, P, P, I64, P, P]),
     "pccnn_grid_build_sized": (I32, [P, P, P, P, P, I64, I32, I32, I32, I32, P, P, P, P, P, P, P, P, SZ, P]),
     "pccnn_pdf_cloud_workspace_bytes": (SZ, [I64, I64, I64]),

@@ -67,6 +67,15 @@ compact_remap_kernel(const int32_t *__restrict__ flags, const int32_t *__restric
     if (i < n && flags[i] != 0) ids[scan[i] - 1] = remap[i];
 }
 
+// ids[i] = cloud of sorted point i if it is selected, else -1 (which the bounding box ignores)
+__global__ void __launch_bounds__(256)
+selected_cloud_kernel(const int32_t *__restrict__ selected, const int32_t *__restrict__ perm,
+                      const int32_t *__restrict__ batch_ids, int64_t n, int32_t *__restrict__ ids)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) ids[i] = selected[i] != 0 ? batch_ids[perm[i]] : -1;
+}
+
 struct PoolLayout {
     int64_t *keys, *sorted_keys;
     float *sorted_pts;
@@ -125,11 +134,16 @@ extern "C" int pccnn_pool_poisson_select(const float *pts, const int32_t *batch_
                                          const float *aabb_min, const float *cell_size,
                                          const int32_t *num_cells_host, int key_bits, int with_cell_table,
                                          int32_t *perm_out, int32_t *selected_out, int32_t *selected_scan_out,
-                                         int64_t *count_out, void *workspace, size_t workspace_bytes, void *stream)
+                                         int64_t *count_out, float *pooled_min_out, float *pooled_max_out,
+                                         float *pooled_host_min_out, float *pooled_host_max_out, void *workspace,
+                                         size_t workspace_bytes, void *stream)
 {
     PCCNN_REQUIRE(n >= 0 && n < (1ll << 31) && batch_size > 0, PCCNN_ERR_INVALID,
                   "pccnn_pool_poisson_select: n=%lld batch_size=%d", (long long)n, batch_size);
     PCCNN_REQUIRE(count_out && num_cells_host, PCCNN_ERR_INVALID, "pccnn_pool_poisson_select: null host pointer");
+    const bool with_box = pooled_min_out != nullptr;
+    PCCNN_REQUIRE(!with_box || (pooled_max_out && pooled_host_min_out && pooled_host_max_out), PCCNN_ERR_INVALID,
+                  "pccnn_pool_poisson_select: the box of the selection needs all four of its outputs");
     *count_out = 0;
     if (n == 0) return PCCNN_OK;
     PCCNN_REQUIRE(pts && batch_ids && aabb_min && cell_size && perm_out && selected_out && selected_scan_out,
@@ -153,8 +167,30 @@ extern "C" int pccnn_pool_poisson_select(const float *pts, const int32_t *batch_
                                  l.num_cells, cell_size, 3, selected_out, selected_scan_out, l.poisson_ws,
                                  l.poisson_bytes, stream);
     if (rc != PCCNN_OK) return rc;
-    int32_t count = 0;
-    if ((rc = read_back(&count, selected_scan_out + (n - 1), sizeof(int32_t), s)) != PCCNN_OK) return rc;
+    if (!with_box) {
+        int32_t count = 0;
+        if ((rc = read_back(&count, selected_scan_out + (n - 1), sizeof(int32_t), s)) != PCCNN_OK) return rc;
+        *count_out = count;
+        return PCCNN_OK;
+    }
+    // the box of the selected points (the unsorted keys are not needed any more: their memory takes the masked ids)
+    int32_t *masked = (int32_t *)l.keys;
+    selected_cloud_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(selected_out, perm_out, batch_ids, n, masked);
+    PCCNN_LAUNCH_CHECK();
+    rc = pccnn_bounding_box(l.sorted_pts, masked, n, 3, batch_size, pooled_min_out, pooled_max_out, stream);
+    if (rc != PCCNN_OK) return rc;
+    // count and box come back together: one wait
+    const size_t box = (size_t)batch_size * 3 * sizeof(float);
+    void *slot;
+    if ((rc = pinned_slot(256 + 2 * box, &slot)) != PCCNN_OK) return rc;
+    PCCNN_HIP_CHECK(hipMemcpyAsync(slot, selected_scan_out + (n - 1), sizeof(int32_t), hipMemcpyDeviceToHost, s));
+    PCCNN_HIP_CHECK(hipMemcpyAsync((char *)slot + 256, pooled_min_out, box, hipMemcpyDeviceToHost, s));
+    PCCNN_HIP_CHECK(hipMemcpyAsync((char *)slot + 256 + box, pooled_max_out, box, hipMemcpyDeviceToHost, s));
+    PCCNN_HIP_CHECK(hipStreamSynchronize(s));
+    int32_t count;
+    memcpy(&count, slot, sizeof(int32_t));
+    memcpy(pooled_host_min_out, (char *)slot + 256, box);
+    memcpy(pooled_host_max_out, (char *)slot + 256 + box, box);
     *count_out = count;
     return PCCNN_OK;
 }

@@ -1,3 +1,5 @@
+import weakref
+
 import numpy as np
 import torch
 
@@ -30,6 +32,14 @@ class Pointcloud(object):
         self.batch_size_tensor_ = None
         if self.batch_size_host_ is None:
             self.batch_size_tensor_ = torch.max(self.batch_ids_) + 1
+        # coordinates and batch ids that one PointPooling selected carry the box of the selection along (it came back
+        # with the selection's size): the cloud starts with its bounding box known, as BoundingBox remembers it
+        pooled = getattr(p_pts, "pccnn_pooled_box_", None)
+        if pooled is not None and pooled is getattr(p_batch_ids, "pccnn_pooled_box_", None) \
+                and self.pts_ is p_pts and self.batch_ids_ is p_batch_ids and p_pts._version == 0 \
+                and p_batch_ids._version == 0:
+            mn, mx, host = pooled.box
+            self.aabb_cache_ = (weakref.ref(self.pts_), 0, weakref.ref(self.batch_ids_), 0, mn, mx, [host])
         self.num_pts_per_batch_ = None          # cached result of get_num_points_per_batch()
         if self.pts_with_grads_:
             self.pts_.requires_grad = True

@@ -11,6 +11,16 @@ from ._consts import device_vector, host_num_cells, host_vector
 ONE_CALL = True
 
 
+class PooledBox(object):
+    """What the pooled coordinates and the pooled batch ids of one Poisson-disk pooling carry along: the bounding
+    box of the selected points (device tensors and host copy), which came back with the selection's size.  A
+    Pointcloud built from exactly these two tensors starts with its box known."""
+    __slots__ = ("box",)
+
+    def __init__(self, p_box):
+        self.box = p_box
+
+
 class PointPooling(object):
     """Point-cloud pooling (pccnn_lib/pc/PointPooling.py:16-102).
 
@@ -22,6 +32,7 @@ class PointPooling(object):
         self.point_cloud_ = p_point_cloud
         self.radii_ = p_radii
         self.method_ = p_method
+        self.pooled_box_ = None
         with torch.no_grad():
             cell = device_vector(p_radii, p_point_cloud.pts_.shape[1], p_point_cloud.pts_.device)
             cell_host = host_vector(cell)
@@ -29,9 +40,11 @@ class PointPooling(object):
             if ONE_CALL and p_method == "poisson_disk" and p_point_cloud.pts_.shape[1] == 3:
                 if cell_host is not None:
                     # three dimensions, cell size known on the host: grid, selection and its size in one native call
-                    self.pooling_ids_ = pccnn_lib_ops.pool_poisson(
+                    self.pooling_ids_, box = pccnn_lib_ops.pool_poisson(
                         p_point_cloud.pts_.detach(), p_point_cloud.batch_ids_, bb.min_, cell,
                         host_num_cells(bb.host(), cell_host), p_point_cloud.batch_size_host())
+                    if box is not None:
+                        self.pooled_box_ = PooledBox(box)
                     return
             grid = Grid(p_point_cloud, bb, p_radii)
             grid.compute_cell_ids()
@@ -65,6 +78,9 @@ class PointPooling(object):
                 # the selection keeps at least one point of every cloud: a Pointcloud built from these ids need not
                 # read their maximum back
                 out.pccnn_batch_size_ = self.point_cloud_.batch_size_host()
+                out.pccnn_pooled_box_ = self.pooled_box_
+            elif p_in_tensor is self.point_cloud_.pts_:
+                out.pccnn_pooled_box_ = self.pooled_box_
             return out
         index = self.pooling_ids_.to(torch.int64).reshape(-1, 1).expand(-1, p_in_tensor.shape[1])
         out = torch.zeros((self.num_pooling_pts_, p_in_tensor.shape[1]), dtype=p_in_tensor.dtype,

@@ -611,8 +611,12 @@ def poisson_disk_sampling_grid(sorted_pts, sorted_keys, grid_ds, grid_size, radi
 def pool_poisson(pts, batch_ids, aabb_min, cell_size, num_cells_host, batch_size):
     """Poisson-disk pooling of a 3-D cloud from its box and the grid size on the host (what
     pccnn_lib/pc/PointPooling.py:38-69 does after the bounding box): the grid, the selection and its size in one
-    native call, the selected points' ORIGINAL indices in a second one -> i64[S], in key order.  No counterpart in
-    the reference's module; the kernels are those of grid_build and poisson_disk_sampling_grid."""
+    native call, the selected points' ORIGINAL indices in a second one -> (i64[S] in key order, box), where box =
+    (min f32[B,3], max f32[B,3], (numpy min, numpy max)) is the bounding box of the selected points per cloud, as
+    ``bounding_box_host`` of the pooled cloud would return it (it comes back with the count, in the same read).
+    No counterpart in the reference's module; the kernels are those of grid_build, poisson_disk_sampling_grid and
+    bounding_box."""
+    import numpy as np
     name = "pool_poisson"
     _chk(pts, name + ": pts", torch.float32, 2)
     dev = pts.device
@@ -626,7 +630,7 @@ def pool_poisson(pts, batch_ids, aabb_min, cell_size, num_cells_host, batch_size
             or cell_size.shape[0] != 3 or len(cells) != 3 or min(cells) < 1:
         raise RuntimeError(name + ": 3-D points [N,3], batch_ids [N], aabb_min [B,3], cell_size [3], three grid sizes")
     if n == 0:
-        return torch.empty((0,), dtype=torch.int64, device=dev)
+        return torch.empty((0,), dtype=torch.int64, device=dev), None
     pillars = batch_size * cells[0] * cells[1]
     total = pillars * cells[2]
     with_table = 1 if total <= CELL_TABLE_MAX_CELLS else 0
@@ -635,12 +639,16 @@ def pool_poisson(pts, batch_ids, aabb_min, cell_size, num_cells_host, batch_size
     rows = torch.empty((3 * n,), dtype=torch.int32, device=dev)      # permutation | selection flags | their scan
     base = rows.data_ptr()
     count = ctypes.c_int64(0)
+    mn = torch.empty((batch_size, 3), dtype=torch.float32, device=dev)
+    mx = torch.empty_like(mn)
+    host = np.empty((2, batch_size, 3), dtype=np.float32)
     _lib.call("pccnn_pool_poisson_select", _ptr(pts), _ptr(batch_ids), n, batch_size, _ptr(aabb_min), _ptr(cell_size),
               (ctypes.c_int32 * 3)(*cells), key_bits_for(cells, batch_size), with_table, _P(base), _P(base + 4 * n),
-              _P(base + 8 * n), ctypes.byref(count), _ptr(ws), ws.numel(), _stream())
+              _P(base + 8 * n), ctypes.byref(count), _ptr(mn), _ptr(mx), _P(host.ctypes.data),
+              _P(host.ctypes.data + host[0].nbytes), _ptr(ws), ws.numel(), _stream())
     ids = torch.empty((count.value,), dtype=torch.int64, device=dev)
     _lib.call("pccnn_compact_selected_remap", _P(base + 4 * n), _P(base + 8 * n), _P(base), n, _ptr(ids), _stream())
-    return ids
+    return ids, (mn, mx, (host[0], host[1]))
 
 
 # ----------------------------------------------------------------------------- conv

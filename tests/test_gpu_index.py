@@ -446,7 +446,13 @@ def test_one_call_pooling_density_and_neighborhood_equal_the_step_by_step_routes
         pool = lib.pc.PointPooling(pc, radius)
         out_pc = lib.pc.Pointcloud(pool.pool_tensor(pc.pts_), pool.pool_tensor(pc.batch_ids_))
         pc.compute_pdf(0.25 * radius)
-        got = [pool.pooling_ids_, pc.pts_unnorm_pdf_, pc.pts_pdf_]
+        # the pooled cloud's box: computed on request (step by step), or come back with the selection (one call)
+        assert (getattr(out_pc, "aabb_cache_", None) is not None) == one_call
+        box = lib.pc.BoundingBox(out_pc)
+        fresh_min, fresh_max = ops.bounding_box(out_pc.pts_, out_pc.batch_ids_, batch)
+        assert torch.equal(box.min_, fresh_min) and torch.equal(box.max_, fresh_max)
+        assert np.array_equal(box.host()[0], fresh_min.cpu().numpy()) and np.array_equal(box.host()[1], fresh_max.cpu().numpy())
+        got = [pool.pooling_ids_, pc.pts_unnorm_pdf_, pc.pts_pdf_, box.min_, box.max_]
         for samples, cap, key_order in ((out_pc, 0, False), (pc, 0, False), (out_pc, 5, False), (out_pc, 0, True)):
             grid = lib.pc.Grid(pc, lib.pc.BoundingBox(pc), 2.0 * radius)
             if not one_call:
