@@ -248,6 +248,12 @@ int pccnn_pool_poisson_select(const float *pts, const int32_t *batch_ids, int64_
                               void *workspace, size_t workspace_bytes, void *stream);
 int pccnn_compact_selected_remap(const int32_t *selected, const int32_t *selected_scan, const int32_t *remap,
                                  int64_t n, int64_t *ids_out, void *stream);
+/* pccnn_compact_selected_remap with remap = perm, plus the rows a pooled cloud is made of: pooled_pts_out f32[S,d] =
+ * pts[ids], pooled_batch_ids_out i32[S] = batch_ids[ids] (what PointPooling.pool_tensor returns for the cloud's own
+ * coordinates and batch ids, pccnn_lib/pc/PointPooling.py:91-95). */
+int pccnn_compact_pooled(const int32_t *selected, const int32_t *selected_scan, const int32_t *perm, const float *pts,
+                         const int32_t *batch_ids, int64_t n, int d, int64_t *ids_out, float *pooled_pts_out,
+                         int32_t *pooled_batch_ids_out, void *stream);
 /* pccnn_grid_build for a grid whose size is known on the host (num_cells_host: d host ints): writes that size to
  * num_cells_out i32[d] on the device, where the kernels read it, instead of computing it there with pccnn_num_cells;
  * the numbers of pillars and cells follow from it.  with_cell_table != 0 (d == 3 only) fills cell_table_out

@@ -67,6 +67,21 @@ compact_remap_kernel(const int32_t *__restrict__ flags, const int32_t *__restric
     if (i < n && flags[i] != 0) ids[scan[i] - 1] = remap[i];
 }
 
+// the selected points' original indices, coordinates and batch ids, in the order of the selection
+__global__ void __launch_bounds__(256)
+compact_pooled_kernel(const int32_t *__restrict__ flags, const int32_t *__restrict__ scan,
+                      const int32_t *__restrict__ perm, const float *__restrict__ pts,
+                      const int32_t *__restrict__ batch_ids, int64_t n, int d, int64_t *__restrict__ ids,
+                      float *__restrict__ pts_out, int32_t *__restrict__ batch_out)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n || flags[i] == 0) return;
+    const int64_t j = scan[i] - 1, o = perm[i];
+    ids[j] = o;
+    for (int k = 0; k < d; ++k) pts_out[j * d + k] = pts[o * d + k];
+    batch_out[j] = batch_ids[o];
+}
+
 // ids[i] = cloud of sorted point i if it is selected, else -1 (which the bounding box ignores)
 __global__ void __launch_bounds__(256)
 selected_cloud_kernel(const int32_t *__restrict__ selected, const int32_t *__restrict__ perm,
@@ -204,6 +219,22 @@ extern "C" int pccnn_compact_selected_remap(const int32_t *selected, const int32
                   "pccnn_compact_selected_remap: null pointer");
     compact_remap_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, (hipStream_t)stream>>>(selected, selected_scan,
                                                                                            remap, n, ids_out);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
+extern "C" int pccnn_compact_pooled(const int32_t *selected, const int32_t *selected_scan, const int32_t *perm,
+                                    const float *pts, const int32_t *batch_ids, int64_t n, int d, int64_t *ids_out,
+                                    float *pooled_pts_out, int32_t *pooled_batch_ids_out, void *stream)
+{
+    PCCNN_REQUIRE(n >= 0 && d >= 2 && d <= PCCNN_MAX_DIMS, PCCNN_ERR_INVALID, "pccnn_compact_pooled: n=%lld d=%d",
+                  (long long)n, d);
+    if (n == 0) return PCCNN_OK;
+    PCCNN_REQUIRE(selected && selected_scan && perm && pts && batch_ids && ids_out && pooled_pts_out &&
+                      pooled_batch_ids_out,
+                  PCCNN_ERR_INVALID, "pccnn_compact_pooled: null pointer");
+    compact_pooled_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, (hipStream_t)stream>>>(
+        selected, selected_scan, perm, pts, batch_ids, n, d, ids_out, pooled_pts_out, pooled_batch_ids_out);
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
 }

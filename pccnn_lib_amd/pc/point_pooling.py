@@ -33,6 +33,7 @@ class PointPooling(object):
         self.radii_ = p_radii
         self.method_ = p_method
         self.pooled_box_ = None
+        self.pooled_pts_ = self.pooled_batch_ids_ = None      # the cloud's own rows, when the pooling call gathered them
         with torch.no_grad():
             cell = device_vector(p_radii, p_point_cloud.pts_.shape[1], p_point_cloud.pts_.device)
             cell_host = host_vector(cell)
@@ -40,7 +41,7 @@ class PointPooling(object):
             if ONE_CALL and p_method == "poisson_disk" and p_point_cloud.pts_.shape[1] == 3:
                 if cell_host is not None:
                     # three dimensions, cell size known on the host: grid, selection and its size in one native call
-                    self.pooling_ids_, box = pccnn_lib_ops.pool_poisson(
+                    self.pooling_ids_, box, self.pooled_pts_, self.pooled_batch_ids_ = pccnn_lib_ops.pool_poisson(
                         p_point_cloud.pts_.detach(), p_point_cloud.batch_ids_, bb.min_, cell,
                         host_num_cells(bb.host(), cell_host), p_point_cloud.batch_size_host())
                     if box is not None:
@@ -73,7 +74,13 @@ class PointPooling(object):
 
     def pool_tensor(self, p_in_tensor, max_pool=False):
         if self.method_ == "poisson_disk":
-            out = torch.index_select(p_in_tensor, 0, self.pooling_ids_)
+            if p_in_tensor is self.point_cloud_.batch_ids_ and self.pooled_batch_ids_ is not None:
+                out, self.pooled_batch_ids_ = self.pooled_batch_ids_, None          # handed out once
+            elif p_in_tensor is self.point_cloud_.pts_ and self.pooled_pts_ is not None \
+                    and not (torch.is_grad_enabled() and p_in_tensor.requires_grad):
+                out, self.pooled_pts_ = self.pooled_pts_, None
+            else:
+                out = torch.index_select(p_in_tensor, 0, self.pooling_ids_)
             if p_in_tensor is self.point_cloud_.batch_ids_:
                 # the selection keeps at least one point of every cloud: a Pointcloud built from these ids need not
                 # read their maximum back

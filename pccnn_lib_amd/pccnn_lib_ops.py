@@ -611,7 +611,8 @@ def poisson_disk_sampling_grid(sorted_pts, sorted_keys, grid_ds, grid_size, radi
 def pool_poisson(pts, batch_ids, aabb_min, cell_size, num_cells_host, batch_size):
     """Poisson-disk pooling of a 3-D cloud from its box and the grid size on the host (what
     pccnn_lib/pc/PointPooling.py:38-69 does after the bounding box): the grid, the selection and its size in one
-    native call, the selected points' ORIGINAL indices in a second one -> (i64[S] in key order, box), where box =
+    native call, the selected points' ORIGINAL indices, coordinates and batch ids in a second one -> (i64[S] in key
+    order, box, f32[S,3], i32[S]), where box =
     (min f32[B,3], max f32[B,3], (numpy min, numpy max)) is the bounding box of the selected points per cloud, as
     ``bounding_box_host`` of the pooled cloud would return it (it comes back with the count, in the same read).
     No counterpart in the reference's module; the kernels are those of grid_build, poisson_disk_sampling_grid and
@@ -630,7 +631,7 @@ def pool_poisson(pts, batch_ids, aabb_min, cell_size, num_cells_host, batch_size
             or cell_size.shape[0] != 3 or len(cells) != 3 or min(cells) < 1:
         raise RuntimeError(name + ": 3-D points [N,3], batch_ids [N], aabb_min [B,3], cell_size [3], three grid sizes")
     if n == 0:
-        return torch.empty((0,), dtype=torch.int64, device=dev), None
+        return torch.empty((0,), dtype=torch.int64, device=dev), None, torch.empty_like(pts), torch.empty_like(batch_ids)
     pillars = batch_size * cells[0] * cells[1]
     total = pillars * cells[2]
     with_table = 1 if total <= CELL_TABLE_MAX_CELLS else 0
@@ -647,8 +648,11 @@ def pool_poisson(pts, batch_ids, aabb_min, cell_size, num_cells_host, batch_size
               _P(base + 8 * n), ctypes.byref(count), _ptr(mn), _ptr(mx), _P(host.ctypes.data),
               _P(host.ctypes.data + host[0].nbytes), _ptr(ws), ws.numel(), _stream())
     ids = torch.empty((count.value,), dtype=torch.int64, device=dev)
-    _lib.call("pccnn_compact_selected_remap", _P(base + 4 * n), _P(base + 8 * n), _P(base), n, _ptr(ids), _stream())
-    return ids, (mn, mx, (host[0], host[1]))
+    pooled_pts = torch.empty((count.value, 3), dtype=torch.float32, device=dev)
+    pooled_ids = torch.empty((count.value,), dtype=torch.int32, device=dev)
+    _lib.call("pccnn_compact_pooled", _P(base + 4 * n), _P(base + 8 * n), _P(base), _ptr(pts), _ptr(batch_ids), n, 3,
+              _ptr(ids), _ptr(pooled_pts), _ptr(pooled_ids), _stream())
+    return ids, (mn, mx, (host[0], host[1])), pooled_pts, pooled_ids
 
 
 # ----------------------------------------------------------------------------- conv

@@ -452,7 +452,9 @@ def test_one_call_pooling_density_and_neighborhood_equal_the_step_by_step_routes
         fresh_min, fresh_max = ops.bounding_box(out_pc.pts_, out_pc.batch_ids_, batch)
         assert torch.equal(box.min_, fresh_min) and torch.equal(box.max_, fresh_max)
         assert np.array_equal(box.host()[0], fresh_min.cpu().numpy()) and np.array_equal(box.host()[1], fresh_max.cpu().numpy())
-        got = [pool.pooling_ids_, pc.pts_unnorm_pdf_, pc.pts_pdf_, box.min_, box.max_]
+        got = [pool.pooling_ids_, pc.pts_unnorm_pdf_, pc.pts_pdf_, box.min_, box.max_, out_pc.pts_, out_pc.batch_ids_,
+               pool.pool_tensor(pc.pts_), pool.pool_tensor(pc.batch_ids_)]       # (a second request: gathered anew)
+        assert torch.equal(got[-2], pc.pts_[pool.pooling_ids_]) and got[-2] is not out_pc.pts_
         for samples, cap, key_order in ((out_pc, 0, False), (pc, 0, False), (out_pc, 5, False), (out_pc, 0, True)):
             grid = lib.pc.Grid(pc, lib.pc.BoundingBox(pc), 2.0 * radius)
             if not one_call:
