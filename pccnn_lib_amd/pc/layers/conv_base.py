@@ -64,6 +64,20 @@ def point_side(p_pc_in, p_neighborhood, *p_per_point):
     return (grid.sorted_pts_, pairs) + tuple(moved)
 
 
+def density_times_volume(p_pdf, p_radius):
+    """``p_pdf * prod(p_radius)`` (pccnn_lib/pc/layers/MCConv.py:101-102).  For an isotropic radius given as a host
+    value the product is taken on the host in fp32, (r * r) * r, which is what the device reduction of three equal
+    numbers gives in any order, and multiplies the densities as a scalar: one launch instead of two."""
+    import numpy as np
+    host = host_vector(p_radius)
+    if host is not None and host.size > 0 and bool(np.all(host == host[0])):
+        prod = np.float32(1.0)
+        for v in host:
+            prod = np.float32(prod * v)
+        return p_pdf * float(prod)
+    return p_pdf * torch.prod(p_radius)
+
+
 def mirror_if_needed(p_neighborhood, *p_geometry):
     """The neighborhood's mirror index when one of the tensors that receive point-side gradients (positions,
     densities) requires a gradient; None otherwise, or for a neighborhood object that has none."""

@@ -7,7 +7,7 @@ import time
 
 from ...op_wrappers import ComputeKPConv, ComputeKPConvWeightVar, ComputeKPConvN, ComputeKPConvNWeightVar, \
     ComputePCCNN, ComputePCCNNWeightVar
-from .conv_base import IConvLayer, IConvLayerFactory, mirror_if_needed, point_side
+from .conv_base import IConvLayer, IConvLayerFactory, mirror_if_needed, point_side, density_times_volume
 from .kernel_points import kernel_pts_dict
 
 
@@ -117,7 +117,7 @@ class _DensityKernelPointConv(IConvLayer):
         self.conv_weights_.data.normal_(0.0, stdv)
 
     def __compute_convolution__(self, p_pc_in, p_pc_out, p_in_features, p_radius, p_neighborhood):
-        cur_pdf = p_pc_in.pts_unnorm_pdf_ * torch.prod(p_radius)
+        cur_pdf = density_times_volume(p_pc_in.pts_unnorm_pdf_, p_radius)
         if self.sigma_cpu_ is None:
             self.sigma_cpu_ = self.sigma_.item()
         if torch.is_grad_enabled() and cur_pdf.requires_grad:

@@ -3,7 +3,7 @@ import math
 import torch
 
 from ...op_wrappers import ComputeMCConv, ComputeMCConvWeightVar
-from .conv_base import IConvLayer, IConvLayerFactory, mirror_if_needed, point_side
+from .conv_base import IConvLayer, IConvLayerFactory, mirror_if_needed, point_side, density_times_volume
 
 
 class MCConv(IConvLayer):
@@ -38,7 +38,7 @@ class MCConv(IConvLayer):
     def __compute_convolution__(self, p_pc_in, p_pc_out, p_in_features, p_radius, p_neighborhood):
         if p_pc_in.pts_unnorm_pdf_ is None:
             raise RuntimeError("MCConv: the input point cloud has no density; call compute_pdf(bandwidth) first")
-        cur_pdf = p_pc_in.pts_unnorm_pdf_ * torch.prod(p_radius)
+        cur_pdf = density_times_volume(p_pc_in.pts_unnorm_pdf_, p_radius)
         if torch.is_grad_enabled() and cur_pdf.requires_grad:
             pts, pairs, pdf, feats = p_pc_in.pts_, p_neighborhood.neighbors_, cur_pdf, p_in_features
         else:

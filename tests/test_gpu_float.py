@@ -456,3 +456,19 @@ def test_ops_run_on_torch_current_stream(ops, models):
     assert torch.equal(nbh_side.neighbors_, nbh.neighbors_)
     assert torch.equal(got, want)
     torch.cuda.synchronize()
+
+
+def test_density_times_volume_on_the_host_equals_the_device_product():
+    # an isotropic radius given as a host value: prod(radius) is taken on the host in fp32 and multiplies the densities
+    # as a scalar; it must be the number the device reduction gives, bit for bit, for any radius
+    from pccnn_lib_amd.pc._consts import device_vector, host_vector
+    from pccnn_lib_amd.pc.layers.conv_base import density_times_volume
+    rng = np.random.default_rng(3)
+    pdf = t(rng.uniform(0.0, 50.0, 4096).astype(np.float32))
+    for r in [0.05, 0.1, 0.025, 0.4, 1.0, 3.0] + [float(v) for v in rng.uniform(1e-3, 10.0, 40)]:
+        radius = device_vector(r, 3, DEV)
+        assert host_vector(radius) is not None
+        want = pdf * torch.prod(radius.clone())                # a tensor the host knows nothing about
+        assert torch.equal(density_times_volume(pdf, radius), want)
+    mixed = device_vector([0.1, 0.2, 0.05], 3, DEV)             # not isotropic: the device product as before
+    assert torch.equal(density_times_volume(pdf, mixed), pdf * torch.prod(mixed))
