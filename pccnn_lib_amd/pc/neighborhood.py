@@ -38,7 +38,7 @@ class Neighborhood(object):
                 own = p_samples is cloud
                 key_order = bool(p_key_order)
                 built, neighbors, self.start_ids_ = pccnn_lib_ops.neighborhood_build(
-                    cloud.pts_.detach(), cloud.batch_ids_, grid.bounding_box_.min_, grid.num_cells_host(),
+                    cloud.pts_.detach(), cloud.batch_ids_, grid.bounding_box_.min_, grid.num_cells_host,
                     grid.cell_size_, cloud.batch_size_host(), None if own else sample_pts,
                     None if own else p_samples.batch_ids_, p_max_neighbors, not key_order)
                 grid.adopt(built)

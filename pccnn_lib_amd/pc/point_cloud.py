@@ -98,7 +98,7 @@ class Pointcloud(object):
             with torch.no_grad():
                 self.pts_unnorm_pdf_, self.pts_pdf_ = pccnn_lib_ops.pdf_cloud(
                     self.dim_manifold_, bandwidth, self.pts_.detach(), self.batch_ids_, aabb.min_, radii,
-                    host_num_cells(aabb.host(), radii_host), self.batch_size_host(), 300)
+                    lambda: host_num_cells(aabb.host(), radii_host), self.batch_size_host(), 300)
             return
         grid = Grid(self, aabb, radii)
         grid.compute_cell_ids()

@@ -43,7 +43,7 @@ class PointPooling(object):
                     # three dimensions, cell size known on the host: grid, selection and its size in one native call
                     self.pooling_ids_, box, self.pooled_pts_, self.pooled_batch_ids_ = pccnn_lib_ops.pool_poisson(
                         p_point_cloud.pts_.detach(), p_point_cloud.batch_ids_, bb.min_, cell,
-                        host_num_cells(bb.host(), cell_host), p_point_cloud.batch_size_host())
+                        lambda: host_num_cells(bb.host(), cell_host), p_point_cloud.batch_size_host())
                     if box is not None:
                         self.pooled_box_ = PooledBox(box)
                     return

@@ -104,6 +104,30 @@ def bounding_box_host(pts, batch_ids, batch_size):
     return mn, mx, (host[0], host[1])
 
 
+def bounding_box_host_later(pts, batch_ids, batch_size):
+    """``bounding_box`` with the host copy on its way: -> (f32[B,D], f32[B,D], fetch), where ``fetch()`` waits for
+    an asynchronous copy into pinned memory that was queued behind the box kernels and returns the two numpy arrays.
+    Whatever the caller does before it calls ``fetch`` runs beside the device's work."""
+    _chk(pts, "bounding_box: pts", torch.float32, 2)
+    _chk(batch_ids, "bounding_box: batch_ids", torch.int32, 1, pts.device)
+    d = _dims(pts, "bounding_box")
+    batch_size = int(batch_size)
+    box = torch.empty((2, batch_size, d), dtype=torch.float32, device=pts.device)
+    base = box.data_ptr()
+    _lib.call("pccnn_bounding_box", _ptr(pts), _ptr(batch_ids), pts.shape[0], d, batch_size, _P(base),
+              _P(base + 4 * batch_size * d), _stream())
+    pinned = torch.empty((2, batch_size, d), dtype=torch.float32, pin_memory=True)
+    pinned.copy_(box, non_blocking=True)
+    done = torch.cuda.Event()
+    done.record()
+
+    def fetch():
+        done.synchronize()
+        host = pinned.numpy()
+        return host[0], host[1]
+    return box[0], box[1], fetch
+
+
 def num_cells(aabb_min, aabb_max, cell_size):
     """Grid size i32[D] = max over the clouds of int32((max - min) / cell_size) + 1 (pccnn_lib/pc/Grid.py:26-28)."""
     name = "num_cells"
@@ -363,10 +387,9 @@ def neighborhood_build(pts, batch_ids, aabb_min, num_cells_host, cell_size, batc
     _chk(cell_size, name + ": cell_size", torch.float32, 1, dev)
     n = pts.shape[0]
     batch_size = int(batch_size)
-    cells = [int(v) for v in num_cells_host]
     max_neighbors = int(max_neighbors)
     if pts.shape[1] != 3 or batch_ids.shape[0] != n or tuple(aabb_min.shape) != (batch_size, 3) \
-            or cell_size.shape[0] != 3 or len(cells) != 3 or min(cells) < 1 or n < 1 or max_neighbors < 0:
+            or cell_size.shape[0] != 3 or n < 1 or max_neighbors < 0:
         raise RuntimeError(name + ": 3-D points [N,3] (N > 0), batch_ids [N], aabb_min [B,3], cell_size [3], three "
                                   "grid sizes, max_neighbors >= 0")
     m = n
@@ -376,17 +399,12 @@ def neighborhood_build(pts, batch_ids, aabb_min, num_cells_host, cell_size, batc
         m = samples.shape[0]
         if samples.shape[1] != 3 or sample_batch_ids.shape[0] != m or m < 1:
             raise RuntimeError(name + ": samples [M,3] (M > 0) with batch_ids [M]")
-    pillars = batch_size * cells[0] * cells[1]
-    total_cells = pillars * cells[2]
-    with_table = 1 if total_cells <= CELL_TABLE_MAX_CELLS else 0
     lib = _lib.load()
     num = torch.empty((3,), dtype=torch.int32, device=dev)
     keys = torch.empty((n,), dtype=torch.int64, device=dev)
     skeys = torch.empty_like(keys)
     perm = torch.empty((n,), dtype=torch.int32, device=dev)
     spts = torch.empty_like(pts)
-    ds = torch.empty((batch_size, cells[0], cells[1], 2), dtype=torch.int32, device=dev)
-    table = torch.empty((total_cells + 1,), dtype=torch.int32, device=dev) if with_table else None
     ends = torch.empty((m,), dtype=torch.int32, device=dev)
     sort_ws = _workspace(lib.pccnn_grid_build_workspace_bytes(max(n, m)), dev)
     ws = _workspace(lib.pccnn_find_neighbors_workspace_bytes(n, m), dev)
@@ -400,6 +418,15 @@ def neighborhood_build(pts, batch_ids, aabb_min, num_cells_host, cell_size, batc
     else:
         s_tmp = s_keys = s_pts = s_order = samples_p = sample_ids_p = _P(0)
         f_pts, f_keys, f_order = _ptr(spts), _ptr(skeys), _ptr(perm)
+    # (the grid size last: when it is a callable it may have to wait for the cloud's box to arrive on the host)
+    cells = [int(v) for v in (num_cells_host() if callable(num_cells_host) else num_cells_host)]
+    if len(cells) != 3 or min(cells) < 1:
+        raise RuntimeError(name + ": three positive grid sizes")
+    pillars = batch_size * cells[0] * cells[1]
+    total_cells = pillars * cells[2]
+    with_table = 1 if total_cells <= CELL_TABLE_MAX_CELLS else 0
+    ds = torch.empty((batch_size, cells[0], cells[1], 2), dtype=torch.int32, device=dev)
+    table = torch.empty((total_cells + 1,), dtype=torch.int32, device=dev) if with_table else None
     bits = key_bits_for(cells, batch_size)
     total = ctypes.c_int64(0)
     _lib.call("pccnn_neighborhood_count", _ptr(pts), _ptr(batch_ids), n, batch_size, _ptr(aabb_min), _ptr(cell_size),
@@ -511,16 +538,17 @@ def pdf_cloud(manifold_dims, bandwidth, pts, batch_ids, aabb_min, cell_size, num
     _chk(cell_size, name + ": cell_size", torch.float32, 1, dev)
     n = pts.shape[0]
     batch_size = int(batch_size)
-    cells = [int(v) for v in num_cells_host]
     max_neighbors = int(max_neighbors)
     if pts.shape[1] != 3 or batch_ids.shape[0] != n or tuple(aabb_min.shape) != (batch_size, 3) \
-            or cell_size.shape[0] != 3 or bandwidth.shape[0] != 3 or len(cells) != 3 or min(cells) < 1 \
-            or max_neighbors < 0:
+            or cell_size.shape[0] != 3 or bandwidth.shape[0] != 3 or max_neighbors < 0:
         raise RuntimeError(name + ": 3-D points [N,3], batch_ids [N], aabb_min [B,3], cell_size / bandwidth [3], "
                                   "three grid sizes, max_neighbors >= 0")
     out = torch.empty((2, n), dtype=torch.float32, device=dev)
     if n == 0:
         return out[0], out[1]
+    cells = [int(v) for v in (num_cells_host() if callable(num_cells_host) else num_cells_host)]
+    if len(cells) != 3 or min(cells) < 1:
+        raise RuntimeError(name + ": three positive grid sizes")
     pillars = batch_size * cells[0] * cells[1]
     total = pillars * cells[2]
     with_table = 1 if total <= CELL_TABLE_MAX_CELLS else 0
@@ -626,23 +654,26 @@ def pool_poisson(pts, batch_ids, aabb_min, cell_size, num_cells_host, batch_size
     _chk(cell_size, name + ": cell_size", torch.float32, 1, dev)
     n = pts.shape[0]
     batch_size = int(batch_size)
-    cells = [int(v) for v in num_cells_host]
     if pts.shape[1] != 3 or batch_ids.shape[0] != n or tuple(aabb_min.shape) != (batch_size, 3) \
-            or cell_size.shape[0] != 3 or len(cells) != 3 or min(cells) < 1:
+            or cell_size.shape[0] != 3:
         raise RuntimeError(name + ": 3-D points [N,3], batch_ids [N], aabb_min [B,3], cell_size [3], three grid sizes")
     if n == 0:
         return torch.empty((0,), dtype=torch.int64, device=dev), None, torch.empty_like(pts), torch.empty_like(batch_ids)
-    pillars = batch_size * cells[0] * cells[1]
-    total = pillars * cells[2]
-    with_table = 1 if total <= CELL_TABLE_MAX_CELLS else 0
     lib = _lib.load()
-    ws = _workspace(lib.pccnn_pool_poisson_workspace_bytes(n, pillars, total if with_table else 0), dev)
     rows = torch.empty((3 * n,), dtype=torch.int32, device=dev)      # permutation | selection flags | their scan
     base = rows.data_ptr()
     count = ctypes.c_int64(0)
     mn = torch.empty((batch_size, 3), dtype=torch.float32, device=dev)
     mx = torch.empty_like(mn)
     host = np.empty((2, batch_size, 3), dtype=np.float32)
+    # (the grid size last: when it is a callable it may have to wait for the cloud's box to arrive on the host)
+    cells = [int(v) for v in (num_cells_host() if callable(num_cells_host) else num_cells_host)]
+    if len(cells) != 3 or min(cells) < 1:
+        raise RuntimeError(name + ": three positive grid sizes")
+    pillars = batch_size * cells[0] * cells[1]
+    total = pillars * cells[2]
+    with_table = 1 if total <= CELL_TABLE_MAX_CELLS else 0
+    ws = _workspace(lib.pccnn_pool_poisson_workspace_bytes(n, pillars, total if with_table else 0), dev)
     _lib.call("pccnn_pool_poisson_select", _ptr(pts), _ptr(batch_ids), n, batch_size, _ptr(aabb_min), _ptr(cell_size),
               (ctypes.c_int32 * 3)(*cells), key_bits_for(cells, batch_size), with_table, _P(base), _P(base + 4 * n),
               _P(base + 8 * n), ctypes.byref(count), _ptr(mn), _ptr(mx), _P(host.ctypes.data),
