@@ -162,7 +162,10 @@ __device__ __forceinline__ NbLane nb_lane_setup(const NbArgs &a, int2 (*ranges)[
     return L;
 }
 
-template <bool FILL, bool CAPPED, int UNROLL>
+// OFF32 (count pass): the coordinate array is below 4 GiB, so a candidate's byte offset is a 32-bit number kept up
+// to date with additions (one multiplication per range, none per candidate) and the loads take it beside a scalar
+// base, instead of a 64-bit multiply-add per candidate.
+template <bool FILL, bool CAPPED, int UNROLL, bool OFF32 = false>
 __global__ void __launch_bounds__(NB_THREADS)
 neighbors_kernel(NbArgs a)
 {
@@ -199,10 +202,13 @@ neighbors_kernel(NbArgs a)
     unsigned long long word = 0ull;
     int it = 0;
     bool active = nr > 0;
+    unsigned int byte_off = 0u;                                 // OFF32: 12 * (first + j)
+    const char *const pts_bytes = (const char *)a.pts;
     if (active) {
         const int2 g = ranges[wib][0][lane];
         first = g.x;
         len = g.y;
+        byte_off = 12u * (unsigned int)first;
     }
     while (__any(active)) {
         if (active) {
@@ -219,6 +225,12 @@ neighbors_kernel(NbArgs a)
                     const float4 v = a.rec[iu];
                     px[u] = v.x; py[u] = v.y; pz[u] = v.z;
                     id[u] = __float_as_int(v.w);
+                } else if (OFF32) {
+                    const float *q = (const float *)(pts_bytes + (byte_off + (u < left ? 12u * u : 0u)));
+                    px[u] = q[0];
+                    py[u] = q[1];
+                    pz[u] = q[2];
+                    id[u] = 0;
                 } else {
                     px[u] = a.pts[(int64_t)iu * 3 + 0];
                     py[u] = a.pts[(int64_t)iu * 3 + 1];
@@ -226,6 +238,7 @@ neighbors_kernel(NbArgs a)
                     id[u] = 0;
                 }
             }
+            unsigned int nibble = 0u;                               // count: the outcome of this iteration's slots
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 // fp32, no contraction: ((s - p) * (1/r)) squared, summed x, y, z; the reference tests
@@ -257,17 +270,24 @@ neighbors_kernel(NbArgs a)
                             }
                         }
                     }
-                    ++cnt;
-                    if (!FILL) word |= 1ull << (((it & 15) << 2) + u);
+                    if (FILL) ++cnt;
+                    else nibble |= 1u << u;
                 }
             }
+            // one 64-bit shift and one population count per iteration, not one per slot
+            if (!FILL) {
+                word |= (unsigned long long)nibble << ((it & 15) << 2);
+                cnt += __popc(nibble);
+            }
             j += UNROLL;
+            byte_off += 12u * UNROLL;
             if (j >= len) {
                 j = 0;
                 if (++r < nr) {
                     const int2 g = ranges[wib][r][lane];
                     first = g.x;
                     len = g.y;
+                    byte_off = 12u * (unsigned int)first;
                 } else {
                     active = false;
                 }
@@ -823,7 +843,10 @@ extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t
         else if (group == 8) neighbors_group_kernel<false, false, 8><<<blocks, NB_THREADS, 0, s>>>(a);
         else if (group == 4) neighbors_group_kernel<false, false, 4><<<blocks, NB_THREADS, 0, s>>>(a);
         else switch (d) {
-        case 3: neighbors_kernel<false, false, NB_UNROLL_COUNT><<<blocks, NB_THREADS, 0, s>>>(a); break;
+        case 3:
+            if (n < (1ll << 28)) neighbors_kernel<false, false, NB_UNROLL_COUNT, true><<<blocks, NB_THREADS, 0, s>>>(a);
+            else neighbors_kernel<false, false, NB_UNROLL_COUNT><<<blocks, NB_THREADS, 0, s>>>(a);
+            break;
         case 2: neighbors_generic_kernel<false, false, 2><<<blocks, NB_THREADS, 0, s>>>(a); break;
         case 4: neighbors_generic_kernel<false, false, 4><<<blocks, NB_THREADS, 0, s>>>(a); break;
         case 5: neighbors_generic_kernel<false, false, 5><<<blocks, NB_THREADS, 0, s>>>(a); break;
