@@ -211,6 +211,50 @@ struct PccnnGridDims {
 int pccnn_compute_keys_sized(const float *pts, const int32_t *batch_ids, const float *aabb_min,
                              const int32_t *num_cells_host, const float *cell_size, int64_t n, int d,
                              int32_t *num_cells_out, int64_t *keys_out, hipStream_t stream);
+// Where the keys of a sort come from when they are made on the way in (3-D points): the arguments of the key
+// computation.  The grid size is read from `num_cells` (device) or, with `use_sized`, taken from `sized` and written
+// to `num_cells_out` for the kernels that follow.
+struct PccnnKeySource {
+    const float *pts;
+    const int32_t *batch_ids;
+    const float *aabb_min;
+    const float *cell_size;
+    const int32_t *num_cells;
+    PccnnGridDims sized;
+    int32_t *num_cells_out;
+    int use_sized;
+};
+// pccnn_compute_keys (3-D) and pccnn_sort_keys in one: the first histogram pass computes the keys (sort.hip).
+int pccnn_sort_keys_from_points(const PccnnKeySource &source, int64_t *keys_out, int64_t n, int key_bits,
+                                int64_t *sorted_keys_out, int32_t *perm_out, float *sorted_pts_out, void *workspace,
+                                size_t workspace_bytes, void *stream);
+#ifdef __HIPCC__
+// The cell key of 3-D point i: fp32, exactly in this order - subtract the box corner, multiply by the fp32
+// reciprocal of the cell size, floor, clamp (no fused multiply-add).
+__device__ __forceinline__ long long pccnn_point_key3(const float *__restrict__ pts, const int32_t *__restrict__ batch_ids,
+                                                      const float *__restrict__ aabb_min,
+                                                      const float *__restrict__ cell_size, const int (&nc)[3], int64_t i)
+{
+#pragma clang fp contract(off)
+    const int b = batch_ids[i];
+    long long key = 0, accum = 1;
+#pragma unroll
+    for (int k = 2; k >= 0; --k) {
+        const float inv = __fdiv_rn(1.0f, cell_size[k]);
+        const float rel = (pts[i * 3 + k] - aabb_min[(int64_t)b * 3 + k]) * inv;
+        int c = (int)floorf(rel);
+        c = max(0, min(c, nc[k] - 1));
+        key += (long long)c * accum;
+        accum *= nc[k];
+    }
+    return key + accum * (long long)b;
+}
+#endif
+int pccnn_grid_build_sized3(const float *pts, const int32_t *batch_ids, const float *aabb_min,
+                            const int32_t *num_cells_host, const float *cell_size, int64_t n, int key_bits,
+                            int64_t num_pillars, int64_t total_cells, int32_t *num_cells_out, int64_t *keys_out,
+                            int64_t *sorted_keys_out, int32_t *perm_out, float *sorted_pts_out, int32_t *grid_ds_out,
+                            int32_t *cell_table_out, void *workspace, size_t workspace_bytes, void *stream);
 // The rest of pccnn_grid_build after the keys: sort, pillar table, cell table (keys_grid.hip).
 int pccnn_grid_build_from_keys(const int64_t *keys, const float *pts, const int32_t *num_cells, int64_t n, int d,
                                int key_bits, int64_t num_pillars, int64_t total_cells, int64_t *sorted_keys_out,

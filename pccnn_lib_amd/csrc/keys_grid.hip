@@ -494,11 +494,39 @@ extern "C" int pccnn_grid_build(const float *pts, const int32_t *batch_ids, cons
                                 int32_t *perm_out, float *sorted_pts_out, int32_t *grid_ds_out,
                                 int32_t *cell_table_out, void *workspace, size_t workspace_bytes, void *stream)
 {
+    if (d == 3 && n > 0 && pts && batch_ids && aabb_min && num_cells && cell_size && keys_out && sorted_pts_out) {
+        // three dimensions: the keys are computed by the sort's first histogram pass
+        PccnnKeySource src = {pts, batch_ids, aabb_min, cell_size, num_cells, {}, nullptr, 0};
+        int rc = pccnn_sort_keys_from_points(src, keys_out, n, key_bits, sorted_keys_out, perm_out, sorted_pts_out,
+                                             workspace, workspace_bytes, stream);
+        if (rc != PCCNN_OK) return rc;
+        return grid_tables(sorted_keys_out, n, num_cells, d, num_pillars, total_cells, grid_ds_out, cell_table_out,
+                           (hipStream_t)stream);
+    }
     int rc = pccnn_compute_keys(pts, batch_ids, aabb_min, num_cells, cell_size, n, d, keys_out, stream);
     if (rc != PCCNN_OK) return rc;
     return pccnn_grid_build_from_keys(keys_out, pts, num_cells, n, d, key_bits, num_pillars, total_cells,
                                       sorted_keys_out, perm_out, sorted_pts_out, grid_ds_out, cell_table_out, workspace,
                                       workspace_bytes, stream);
+}
+
+// pccnn_grid_build for three dimensions and a grid size known on the host: the sort's first pass computes the keys
+// from that size and writes the device copy.
+int pccnn_grid_build_sized3(const float *pts, const int32_t *batch_ids, const float *aabb_min,
+                            const int32_t *num_cells_host, const float *cell_size, int64_t n, int key_bits,
+                            int64_t num_pillars, int64_t total_cells, int32_t *num_cells_out, int64_t *keys_out,
+                            int64_t *sorted_keys_out, int32_t *perm_out, float *sorted_pts_out, int32_t *grid_ds_out,
+                            int32_t *cell_table_out, void *workspace, size_t workspace_bytes, void *stream)
+{
+    PCCNN_REQUIRE(n > 0 && num_cells_host && num_cells_out && keys_out && sorted_pts_out, PCCNN_ERR_INVALID,
+                  "pccnn_grid_build_sized: null pointer or n=%lld", (long long)n);
+    PccnnKeySource src = {pts, batch_ids, aabb_min, cell_size, nullptr, {}, num_cells_out, 1};
+    for (int k = 0; k < 3; ++k) src.sized.v[k] = num_cells_host[k];
+    int rc = pccnn_sort_keys_from_points(src, keys_out, n, key_bits, sorted_keys_out, perm_out, sorted_pts_out,
+                                         workspace, workspace_bytes, stream);
+    if (rc != PCCNN_OK) return rc;
+    return grid_tables(sorted_keys_out, n, num_cells_out, 3, num_pillars, total_cells, grid_ds_out, cell_table_out,
+                       (hipStream_t)stream);
 }
 
 int pccnn_grid_build_from_keys(const int64_t *keys, const float *pts, const int32_t *num_cells, int64_t n, int d,

@@ -301,6 +301,11 @@ extern "C" int pccnn_grid_build_sized(const float *pts, const int32_t *batch_ids
     int64_t num_pillars, total_cells;
     int rc = grid_extent("pccnn_grid_build_sized", num_cells_host, d, batch_size, &num_pillars, &total_cells);
     if (rc != PCCNN_OK) return rc;
+    if (d == 3 && n > 0)
+        return pccnn_grid_build_sized3(pts, batch_ids, aabb_min, num_cells_host, cell_size, n, key_bits, num_pillars,
+                                       with_cell_table ? total_cells : 0, num_cells_out, keys_out, sorted_keys_out,
+                                       perm_out, sorted_pts_out, grid_ds_out, with_cell_table ? cell_table_out : nullptr,
+                                       workspace, workspace_bytes, stream);
     rc = pccnn_compute_keys_sized(pts, batch_ids, aabb_min, num_cells_host, cell_size, n, d, num_cells_out, keys_out,
                                   (hipStream_t)stream);
     if (rc != PCCNN_OK) return rc;

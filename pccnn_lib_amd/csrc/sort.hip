@@ -47,6 +47,39 @@ radix_hist_kernel(const int64_t *__restrict__ keys, int64_t n, int shift, int it
     }
 }
 
+// The first pass's histogram for keys that do not exist yet: the tile computes the cell keys of its points (the
+// arithmetic of compute_keys_kernel), stores them for the scatter that follows, and counts their lowest digit.
+template <int BITS>
+__global__ void __launch_bounds__(RS_THREADS)
+radix_hist_keys_kernel(PccnnKeySource src, int64_t *__restrict__ keys, int64_t n, int items,
+                       int32_t *__restrict__ tile_hist, int64_t num_tiles)
+{
+    constexpr int D = 1 << BITS;
+    __shared__ int hist[D];
+#pragma unroll
+    for (int q = 0; q < D / RS_THREADS; ++q) hist[threadIdx.x + q * RS_THREADS] = 0;
+    int nc[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) nc[k] = src.use_sized ? src.sized.v[k] : src.num_cells[k];
+    if (src.use_sized && blockIdx.x == 0 && threadIdx.x < 3) src.num_cells_out[threadIdx.x] = src.sized.v[threadIdx.x];
+    __syncthreads();
+    int64_t base = (int64_t)blockIdx.x * RS_THREADS * items;
+    for (int r = 0; r < items; ++r) {
+        int64_t i = base + r * RS_THREADS + threadIdx.x;
+        if (i < n) {
+            const long long key = pccnn_point_key3(src.pts, src.batch_ids, src.aabb_min, src.cell_size, nc, i);
+            keys[i] = key;
+            atomicAdd(&hist[(int)(key & (D - 1))], 1);
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < D / RS_THREADS; ++q) {
+        const int d = threadIdx.x + q * RS_THREADS;
+        tile_hist[(int64_t)d * num_tiles + blockIdx.x] = hist[d];
+    }
+}
+
 // One workgroup per digit: exclusive scan of that digit's per-tile counts (contiguous in the digit-major
 // table), in place; the digit's total goes to digit_totals[digit].
 __global__ void __launch_bounds__(256)
@@ -353,9 +386,10 @@ extern "C" size_t pccnn_sort_keys_workspace_bytes(int64_t n)
 
 // The sort proper; `timed` = bracket the launches with the optional timing events (which are created on the fly,
 // so the entry point that must not allocate anything passes false).
+// `make_keys` (nullable): the keys do not exist yet; the first histogram pass computes them into `keys`.
 static int sort_keys_run(const int64_t *keys, int64_t n, int key_bits, int64_t *sorted_keys_out, int32_t *perm_out,
                          const float *pts, int d, float *sorted_pts_out, void *workspace, size_t workspace_bytes,
-                         void *stream, bool timed_on)
+                         void *stream, bool timed_on, const PccnnKeySource *make_keys = nullptr)
 {
     PCCNN_REQUIRE(n >= 0 && n < (1ll << 31), PCCNN_ERR_INVALID, "pccnn_sort_keys: n=%lld", (long long)n);
     PCCNN_REQUIRE((pts == nullptr) == (sorted_pts_out == nullptr), PCCNN_ERR_INVALID,
@@ -407,7 +441,10 @@ static int sort_keys_run(const int64_t *keys, int64_t n, int key_bits, int64_t *
     } while (0)
 #define RS_PASS(B)                                                                                   \
     do {                                                                                             \
-        radix_hist_kernel<B><<<grid, RS_THREADS, 0, s>>>(src_k, n, shift, items, hist, tiles);       \
+        if (p == 0 && make_keys != nullptr)                                                          \
+            radix_hist_keys_kernel<B><<<grid, RS_THREADS, 0, s>>>(*make_keys, (int64_t *)keys, n, items, hist, tiles); \
+        else                                                                                         \
+            radix_hist_kernel<B><<<grid, RS_THREADS, 0, s>>>(src_k, n, shift, items, hist, tiles);   \
         PCCNN_LAUNCH_CHECK();                                                                        \
         radix_scan_kernel<<<1 << B, 256, 0, s>>>(hist, tiles, totals);                               \
         PCCNN_LAUNCH_CHECK();                                                                        \
@@ -438,6 +475,17 @@ extern "C" int pccnn_sort_keys(const int64_t *keys, int64_t n, int key_bits, int
 {
     return sort_keys_run(keys, n, key_bits, sorted_keys_out, perm_out, pts, d, sorted_pts_out, workspace,
                          workspace_bytes, stream, true);
+}
+
+int pccnn_sort_keys_from_points(const PccnnKeySource &source, int64_t *keys_out, int64_t n, int key_bits,
+                                int64_t *sorted_keys_out, int32_t *perm_out, float *sorted_pts_out, void *workspace,
+                                size_t workspace_bytes, void *stream)
+{
+    PCCNN_REQUIRE(source.pts && source.batch_ids && source.aabb_min && source.cell_size &&
+                      (source.use_sized ? source.num_cells_out != nullptr : source.num_cells != nullptr),
+                  PCCNN_ERR_INVALID, "pccnn_grid_build: null pointer");
+    return sort_keys_run(keys_out, n, key_bits, sorted_keys_out, perm_out, source.pts, 3, sorted_pts_out, workspace,
+                         workspace_bytes, stream, true, &source);
 }
 
 // ---- the same sort for callers that cannot allocate device memory ---------------------------------------------
