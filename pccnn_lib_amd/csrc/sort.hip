@@ -129,12 +129,28 @@ radix_scatter_kernel(const int64_t *__restrict__ keys_in, const int32_t *__restr
     int wave = threadIdx.x >> 6;
     // first output slot of digit d for this tile = (keys with a smaller digit) + (same digit in earlier tiles);
     // for this prefix thread t takes the PER consecutive digits t * PER ...
+    // digit_totals == nullptr (few tiles): tile_offsets is the histogram pass's table as it stands, and every
+    // workgroup adds up its digits' rows itself - the row's total and the part before its own tile - instead of a
+    // scan launch in between.
     {
-        int tot[PER];
+        int tot[PER], before[PER];
         int sum = 0;
 #pragma unroll
         for (int q = 0; q < PER; ++q) {
-            tot[q] = digit_totals[threadIdx.x * PER + q];
+            const int d = threadIdx.x * PER + q;
+            if (digit_totals != nullptr) {
+                tot[q] = digit_totals[d];
+                before[q] = tile_offsets[(int64_t)d * num_tiles + blockIdx.x];
+            } else {
+                int all = 0, mine = 0;
+                for (int64_t t = 0; t < num_tiles; ++t) {
+                    const int v = tile_offsets[(int64_t)d * num_tiles + t];
+                    all += v;
+                    if (t < (int64_t)blockIdx.x) mine += v;
+                }
+                tot[q] = all;
+                before[q] = mine;
+            }
             sum += tot[q];
         }
         int incl = sum;
@@ -153,7 +169,7 @@ radix_scatter_kernel(const int64_t *__restrict__ keys_in, const int32_t *__restr
 #pragma unroll
         for (int q = 0; q < PER; ++q) {
             const int d = threadIdx.x * PER + q;
-            running[d] = excl + tile_offsets[(int64_t)d * num_tiles + blockIdx.x];
+            running[d] = excl + before[q];
             excl += tot[q];
         }
     }
@@ -366,6 +382,7 @@ radix_scatter_staged_kernel(const int64_t *__restrict__ keys_in, const int32_t *
 // On a million keys a pass with 2^11 digits leaves two keys per digit and tile, its scattered stores and the
 // larger table cost more than the saved pass (22 bits: 116 us in 2 passes against 99 us in 3), and 9 bits are the
 // widest digit that still wins (800 000 keys of 18 bits: 72 us against 80 us).
+#define RS_SELF_SCAN_TILES 64           // tiles up to which the scatter does the scan's job itself
 #define RS_MAX_BITS 11
 #define RS_MAX_DIGITS (1 << RS_MAX_BITS)
 static void rs_plan(int key_bits, int64_t n, int &passes, int &bits)
@@ -418,6 +435,8 @@ static int sort_keys_run(const int64_t *keys, int64_t n, int key_bits, int64_t *
     // measured: the staged scatter wins from about 300 000 keys on (84 against 99 us at 10^6 keys of 22 bits),
     // the plain one below that (27 against 30 us at 65 536 keys), where a tile's fixed work outweighs its stores
     const bool staged = items >= RS_STAGED_FROM_ITEMS;
+    // few tiles: the scatter's workgroups add up the histogram rows themselves, no scan launch
+    const bool self_scan = !staged && tiles <= RS_SELF_SCAN_TILES;
     const int64_t *src_k = keys;
     const int32_t *src_v = nullptr;
     for (int p = 0; p < passes; ++p) {
@@ -436,8 +455,8 @@ static int sort_keys_run(const int64_t *keys, int64_t n, int key_bits, int64_t *
                 GATHER ? sorted_pts_out : nullptr, d);                                                            \
         else                                                                                                      \
             radix_scatter_kernel<B, FIRST, GATHER><<<grid, RS_THREADS, 0, s>>>(                                   \
-                src_k, src_v, n, shift, items, hist, tiles, totals, dst_k, dst_v, GATHER ? pts : nullptr,         \
-                GATHER ? sorted_pts_out : nullptr, d);                                                            \
+                src_k, src_v, n, shift, items, hist, tiles, self_scan ? nullptr : totals, dst_k, dst_v,           \
+                GATHER ? pts : nullptr, GATHER ? sorted_pts_out : nullptr, d);                                    \
     } while (0)
 #define RS_PASS(B)                                                                                   \
     do {                                                                                             \
@@ -446,7 +465,7 @@ static int sort_keys_run(const int64_t *keys, int64_t n, int key_bits, int64_t *
         else                                                                                         \
             radix_hist_kernel<B><<<grid, RS_THREADS, 0, s>>>(src_k, n, shift, items, hist, tiles);   \
         PCCNN_LAUNCH_CHECK();                                                                        \
-        radix_scan_kernel<<<1 << B, 256, 0, s>>>(hist, tiles, totals);                               \
+        if (!self_scan) radix_scan_kernel<<<1 << B, 256, 0, s>>>(hist, tiles, totals);               \
         PCCNN_LAUNCH_CHECK();                                                                        \
         if (p == 0) {                                                                                \
             if (gather) RS_SCATTER(B, true, true); else RS_SCATTER(B, true, false);                  \
