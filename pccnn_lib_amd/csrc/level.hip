@@ -343,11 +343,10 @@ extern "C" int pccnn_neighborhood_count(const float *pts, const int32_t *batch_i
     if (samples != nullptr) {
         PCCNN_REQUIRE(sample_batch_ids && sample_keys_tmp && sample_keys_out && sample_order_out && sample_pts_out,
                       PCCNN_ERR_INVALID, "pccnn_neighborhood_count: null sample buffer");
-        rc = pccnn_compute_keys(samples, sample_batch_ids, aabb_min, num_cells_out, cell_size, m, 3, sample_keys_tmp,
-                                stream);
-        if (rc != PCCNN_OK) return rc;
-        rc = pccnn_sort_keys(sample_keys_tmp, m, key_bits, sample_keys_out, sample_order_out, samples, 3, sample_pts_out,
-                             sort_workspace, sort_workspace_bytes, stream);
+        // (the keys of the samples are computed by their sort's first histogram pass)
+        PccnnKeySource src = {samples, sample_batch_ids, aabb_min, cell_size, num_cells_out, {}, nullptr, 0};
+        rc = pccnn_sort_keys_from_points(src, sample_keys_tmp, m, key_bits, sample_keys_out, sample_order_out,
+                                         sample_pts_out, sort_workspace, sort_workspace_bytes, stream);
         if (rc != PCCNN_OK) return rc;
         s_pts = sample_pts_out;
         s_keys = sample_keys_out;

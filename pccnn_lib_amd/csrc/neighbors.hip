@@ -23,6 +23,7 @@
 // The count pass of the one-lane walk can leave its decisions behind: bit 4 * i + u of a sample's mask is the
 // outcome of candidate slot u of its walk iteration i (NB_UNROLL_COUNT slots per iteration).  Word w of all samples
 // is one row, so the 64 lanes of a tile, which finish a word in the same iteration, store it as one run.
+#define NB_PACK_FROM_PAIRS 1000000    // pairs from which the grouped fill packs its point records first
 #define NB_MASK_WORDS 16                               // 256 iterations = 1024 candidate slots per sample are recorded
 
 struct NbArgs {
@@ -544,14 +545,16 @@ neighbors_group_kernel(NbArgs a)
             if (j < cur.y) {
                 const int idx = cur.x + j;
                 float px, py, pz;
-                if (FILL) {
+                if (FILL && a.rec != nullptr) {
                     const float4 v = a.rec[idx];
                     px = v.x; py = v.y; pz = v.z;
                     id = __float_as_int(v.w);
                 } else {
+                    // (count, and the fill of a small search, where packing the records would be one more launch)
                     px = a.pts[(int64_t)idx * 3 + 0];
                     py = a.pts[(int64_t)idx * 3 + 1];
                     pz = a.pts[(int64_t)idx * 3 + 2];
+                    if (FILL) id = a.remap ? a.remap[idx] : idx;
                 }
                 // fp32, no contraction: the predicate of the one-lane walk
                 const float vx = (sx - px) * ir0;
@@ -899,7 +902,12 @@ extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t 
             // the count call left the outcome of every candidate test in the workspace: nothing is tested again
             neighbors_fill_masks_kernel<<<blocks, NB_THREADS, 0, s>>>(a);
         } else if (d == 3) {
-            if (n > 0) pack_points_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(pts_sorted, point_remap, n, rec);
+            // the packed (x, y, z, id) records pay for their launch from a few ten thousand pairs on; the grouped walk
+            // of a small search reads the coordinate array and the id table instead
+            const bool packed = group == 1 || t >= NB_PACK_FROM_PAIRS;
+            if (!packed) a.rec = nullptr;
+            if (n > 0 && packed)
+                pack_points_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(pts_sorted, point_remap, n, rec);
             if (group == 64) {
                 if (max_neighbors > 0) neighbors_group_kernel<true, true, 64><<<blocks, NB_THREADS, 0, s>>>(a);
                 else neighbors_group_kernel<true, false, 64><<<blocks, NB_THREADS, 0, s>>>(a);
