@@ -211,6 +211,33 @@ struct PccnnGridDims {
 int pccnn_compute_keys_sized(const float *pts, const int32_t *batch_ids, const float *aabb_min,
                              const int32_t *num_cells_host, const float *cell_size, int64_t n, int d,
                              int32_t *num_cells_out, int64_t *keys_out, hipStream_t stream);
+// The bounding box of a subset of a sorted cloud, and a second copy of the result for one read-back.  With
+// `selected`, point i counts only when selected[i] != 0; with `perm`, its cloud is batch_ids[perm[i]] (the points
+// are a sorted copy, the cloud ids are not).  With `tail`, the padded boxes are also written there as
+// [minima | maxima] followed by the 32-bit word at `count_src`, so that one copy brings box and count to the host.
+struct PccnnBoxMask {
+    const int32_t *selected = nullptr;
+    const int32_t *perm = nullptr;
+    float *tail = nullptr;
+    const int32_t *count_src = nullptr;
+#ifdef __HIPCC__
+    __device__ __forceinline__ int cloud_of(const int32_t *__restrict__ batch_ids, int64_t i) const
+    {
+        if (selected != nullptr && selected[i] == 0) return -1;
+        return batch_ids[perm != nullptr ? (int64_t)perm[i] : i];
+    }
+    __device__ __forceinline__ void second_copy(int i, int count, float lo, float hi) const
+    {
+        if (tail == nullptr) return;
+        tail[i] = lo;
+        tail[count + i] = hi;
+        if (i == 0 && count_src != nullptr) ((int32_t *)tail)[2 * count] = *count_src;
+    }
+#endif
+};
+int pccnn_bounding_box_masked(const float *pts, const int32_t *batch_ids, int64_t n, int d, int batch_size,
+                              float *aabb_min_out, float *aabb_max_out, const PccnnBoxMask &mask, void *stream);
+
 // Where the keys of a sort come from when they are made on the way in (3-D points): the arguments of the key
 // computation.  The grid size is read from `num_cells` (device) or, with `use_sized`, taken from `sized` and written
 // to `num_cells_out` for the kernels that follow.

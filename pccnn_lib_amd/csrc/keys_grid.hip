@@ -63,7 +63,7 @@ __device__ __forceinline__ void bbox_flush_wave(int cur, const float (&lo)[D], c
 template <int D>
 __global__ void __launch_bounds__(256)
 bbox_reduce_kernel(const float *__restrict__ pts, const int32_t *__restrict__ batch_ids, int64_t n, int batch_size,
-                   float *mn, float *mx)
+                   float *mn, float *mx, PccnnBoxMask mask)
 {
     __shared__ float lds_lo[4][D], lds_hi[4][D];
     __shared__ int lds_b[4];
@@ -85,7 +85,7 @@ bbox_reduce_kernel(const float *__restrict__ pts, const int32_t *__restrict__ ba
             const int64_t i = w0 + (int64_t)u * blockDim.x + threadIdx.x;
             bs[u] = -1;
             if (i < chunk_end) {
-                const int b = batch_ids[i];
+                const int b = mask.cloud_of(batch_ids, i);
                 bs[u] = (b >= 0 && b < batch_size) ? b : -1;          // ids outside the table are ignored
 #pragma unroll
                 for (int k = 0; k < D; ++k) vs[u][k] = pts[i * D + k];
@@ -150,10 +150,14 @@ bbox_reduce_kernel(const float *__restrict__ pts, const int32_t *__restrict__ ba
     }
 }
 
-__global__ void bbox_pad_kernel(float *mn, float *mx, int count)
+__global__ void bbox_pad_kernel(float *mn, float *mx, int count, PccnnBoxMask mask)
 {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < count) { mn[i] = mn[i] - 1e-6f; mx[i] = mx[i] + 1e-6f; }
+    if (i < count) {
+        const float l = mn[i] - 1e-6f, h = mx[i] + 1e-6f;
+        mn[i] = l; mx[i] = h;
+        mask.second_copy(i, count, l, h);
+    }
 }
 
 // A small cloud (up to BBOX_SMALL_POINTS points, up to BBOX_SMALL_CLOUDS clouds): one workgroup, the boxes in LDS,
@@ -164,7 +168,7 @@ __global__ void bbox_pad_kernel(float *mn, float *mx, int count)
 template <int D>
 __global__ void __launch_bounds__(1024)
 bbox_small_kernel(const float *__restrict__ pts, const int32_t *__restrict__ batch_ids, int64_t n, int batch_size,
-                  float *__restrict__ mn, float *__restrict__ mx)
+                  float *__restrict__ mn, float *__restrict__ mx, PccnnBoxMask mask)
 {
     __shared__ float box_lo[BBOX_SMALL_CLOUDS * D], box_hi[BBOX_SMALL_CLOUDS * D];
     const float inf = __int_as_float(0x7f800000);
@@ -181,7 +185,7 @@ bbox_small_kernel(const float *__restrict__ pts, const int32_t *__restrict__ bat
         int b = -1;
         float v[D];
         if (i < n) {
-            b = batch_ids[i];
+            b = mask.cloud_of(batch_ids, i);
             if (b < 0 || b >= batch_size) b = -1;                      // ids outside the table are ignored
 #pragma unroll
             for (int k = 0; k < D; ++k) v[k] = pts[i * D + k];
@@ -200,11 +204,22 @@ bbox_small_kernel(const float *__restrict__ pts, const int32_t *__restrict__ bat
     }
     bbox_flush_wave<D>(cur, lo, hi, box_lo, box_hi);
     __syncthreads();
-    for (int i = threadIdx.x; i < count; i += blockDim.x) { mn[i] = box_lo[i] - 1e-6f; mx[i] = box_hi[i] + 1e-6f; }
+    for (int i = threadIdx.x; i < count; i += blockDim.x) {
+        const float l = box_lo[i] - 1e-6f, h = box_hi[i] + 1e-6f;
+        mn[i] = l; mx[i] = h;
+        mask.second_copy(i, count, l, h);
+    }
 }
 
 extern "C" int pccnn_bounding_box(const float *pts, const int32_t *batch_ids, int64_t n, int d, int batch_size,
                                   float *aabb_min_out, float *aabb_max_out, void *stream)
+{
+    return pccnn_bounding_box_masked(pts, batch_ids, n, d, batch_size, aabb_min_out, aabb_max_out, PccnnBoxMask{},
+                                     stream);
+}
+
+int pccnn_bounding_box_masked(const float *pts, const int32_t *batch_ids, int64_t n, int d, int batch_size,
+                              float *aabb_min_out, float *aabb_max_out, const PccnnBoxMask &mask, void *stream)
 {
     PCCNN_REQUIRE(d >= 2 && d <= PCCNN_MAX_DIMS, PCCNN_ERR_UNSUPPORTED,
                   "pccnn_bounding_box: d=%d is not supported (2 <= d <= 6)", d);
@@ -216,7 +231,7 @@ extern "C" int pccnn_bounding_box(const float *pts, const int32_t *batch_ids, in
     int count = batch_size * d;
     if (n > 0 && n <= BBOX_SMALL_POINTS && batch_size <= BBOX_SMALL_CLOUDS) {
         PCCNN_DIM_DISPATCH(d, bbox_small_kernel, <<<1, 1024, 0, s>>>(pts, batch_ids, n, batch_size, aabb_min_out,
-                                                                    aabb_max_out));
+                                                                    aabb_max_out, mask));
         PCCNN_LAUNCH_CHECK();
         return PCCNN_OK;
     }
@@ -228,10 +243,10 @@ extern "C" int pccnn_bounding_box(const float *pts, const int32_t *batch_ids, in
         int64_t blocks = pccnn_ceil_div(n, 256 * 4);
         if (blocks > 256) blocks = 256;
         PCCNN_DIM_DISPATCH(d, bbox_reduce_kernel, <<<(unsigned)blocks, 256, 0, s>>>(pts, batch_ids, n, batch_size,
-                                                                                    aabb_min_out, aabb_max_out));
+                                                                                    aabb_min_out, aabb_max_out, mask));
         PCCNN_LAUNCH_CHECK();
     }
-    bbox_pad_kernel<<<(unsigned)pccnn_ceil_div(count, 256), 256, 0, s>>>(aabb_min_out, aabb_max_out, count);
+    bbox_pad_kernel<<<(unsigned)pccnn_ceil_div(count, 256), 256, 0, s>>>(aabb_min_out, aabb_max_out, count, mask);
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
 }

@@ -82,15 +82,6 @@ compact_pooled_kernel(const int32_t *__restrict__ flags, const int32_t *__restri
     batch_out[j] = batch_ids[o];
 }
 
-// ids[i] = cloud of sorted point i if it is selected, else -1 (which the bounding box ignores)
-__global__ void __launch_bounds__(256)
-selected_cloud_kernel(const int32_t *__restrict__ selected, const int32_t *__restrict__ perm,
-                      const int32_t *__restrict__ batch_ids, int64_t n, int32_t *__restrict__ ids)
-{
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) ids[i] = selected[i] != 0 ? batch_ids[perm[i]] : -1;
-}
-
 struct PoolLayout {
     int64_t *keys, *sorted_keys;
     float *sorted_pts;
@@ -188,24 +179,37 @@ extern "C" int pccnn_pool_poisson_select(const float *pts, const int32_t *batch_
         *count_out = count;
         return PCCNN_OK;
     }
-    // the box of the selected points (the unsorted keys are not needed any more: their memory takes the masked ids)
-    int32_t *masked = (int32_t *)l.keys;
-    selected_cloud_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(selected_out, perm_out, batch_ids, n, masked);
-    PCCNN_LAUNCH_CHECK();
-    rc = pccnn_bounding_box(l.sorted_pts, masked, n, 3, batch_size, pooled_min_out, pooled_max_out, stream);
-    if (rc != PCCNN_OK) return rc;
-    // count and box come back together: one wait
+    // The box of the selected points, from the sorted copy and the selection flags.  The kernel that pads the boxes
+    // also writes them, and the count, into one stretch of the workspace (the unsorted keys are not needed any
+    // more), so count and box come back with one copy and one wait; with so many clouds that the stretch is too
+    // short for that, they come back with three copies.
     const size_t box = (size_t)batch_size * 3 * sizeof(float);
+    const bool one_copy = 2 * box + sizeof(int32_t) <= pccnn_align((size_t)n * sizeof(int64_t));
+    PccnnBoxMask mask;
+    mask.selected = selected_out;
+    mask.perm = perm_out;
+    if (one_copy) {
+        mask.tail = (float *)l.keys;
+        mask.count_src = selected_scan_out + (n - 1);
+    }
+    rc = pccnn_bounding_box_masked(l.sorted_pts, batch_ids, n, 3, batch_size, pooled_min_out, pooled_max_out, mask,
+                                   stream);
+    if (rc != PCCNN_OK) return rc;
     void *slot;
-    if ((rc = pinned_slot(256 + 2 * box, &slot)) != PCCNN_OK) return rc;
-    PCCNN_HIP_CHECK(hipMemcpyAsync(slot, selected_scan_out + (n - 1), sizeof(int32_t), hipMemcpyDeviceToHost, s));
-    PCCNN_HIP_CHECK(hipMemcpyAsync((char *)slot + 256, pooled_min_out, box, hipMemcpyDeviceToHost, s));
-    PCCNN_HIP_CHECK(hipMemcpyAsync((char *)slot + 256 + box, pooled_max_out, box, hipMemcpyDeviceToHost, s));
+    if ((rc = pinned_slot(2 * box + sizeof(int32_t), &slot)) != PCCNN_OK) return rc;
+    if (one_copy) {
+        PCCNN_HIP_CHECK(hipMemcpyAsync(slot, mask.tail, 2 * box + sizeof(int32_t), hipMemcpyDeviceToHost, s));
+    } else {
+        PCCNN_HIP_CHECK(hipMemcpyAsync(slot, pooled_min_out, box, hipMemcpyDeviceToHost, s));
+        PCCNN_HIP_CHECK(hipMemcpyAsync((char *)slot + box, pooled_max_out, box, hipMemcpyDeviceToHost, s));
+        PCCNN_HIP_CHECK(hipMemcpyAsync((char *)slot + 2 * box, selected_scan_out + (n - 1), sizeof(int32_t),
+                                       hipMemcpyDeviceToHost, s));
+    }
     PCCNN_HIP_CHECK(hipStreamSynchronize(s));
     int32_t count;
-    memcpy(&count, slot, sizeof(int32_t));
-    memcpy(pooled_host_min_out, (char *)slot + 256, box);
-    memcpy(pooled_host_max_out, (char *)slot + 256 + box, box);
+    memcpy(pooled_host_min_out, slot, box);
+    memcpy(pooled_host_max_out, (char *)slot + box, box);
+    memcpy(&count, (char *)slot + 2 * box, sizeof(int32_t));
     *count_out = count;
     return PCCNN_OK;
 }

@@ -40,14 +40,15 @@ cell_list_kernel(const int32_t *__restrict__ flags, const int32_t *__restrict__ 
 // Three dimensions: the non-empty cells listed per parity colour, so that a pass only touches the cells it works
 // on.  colour_list[colour * n + i] = index (into cell_first) of the i-th cell of that colour, in no particular
 // order: cells of one colour do not interact, so the selection does not depend on the order.  colour_count[8]
-// must be zero on entry.
+// must be zero on entry.  The kernel writes the list of first points and the number of cells as well (what
+// cell_list_kernel does for the other dimensions).
 // COLOUR_ITEMS points per thread: 8 on large inputs, where the atomics on the eight global counters would
 // otherwise queue up, 1 on small ones, where the launch is a single round of short workgroups.
 template <int COLOUR_ITEMS>
 __global__ void __launch_bounds__(256)
 cell_colour_kernel(const int32_t *__restrict__ flags, const int32_t *__restrict__ scan, const int64_t *__restrict__ keys,
                    int64_t n, const int32_t *__restrict__ num_cells, int32_t *__restrict__ colour_list,
-                   int32_t *__restrict__ colour_count)
+                   int32_t *__restrict__ colour_count, int32_t *__restrict__ cell_first, int32_t *__restrict__ count)
 {
     // the workgroup counts its cells per colour in LDS and reserves its share of every list with one atomic
     __shared__ int local[8], start[8];
@@ -60,7 +61,9 @@ cell_colour_kernel(const int32_t *__restrict__ flags, const int32_t *__restrict_
         const int64_t i = ((int64_t)blockIdx.x * COLOUR_ITEMS + r) * 256 + threadIdx.x;
         colour[r] = -1;
         at[r] = 0;
+        if (i == n - 1) *count = scan[i];
         if (i < n && flags[i] != 0) {
+            cell_first[scan[i] - 1] = (int32_t)i;
             long long k = keys[i];
             const int c2 = (int)(k % nc2); k /= nc2;
             const int c1 = (int)(k % nc1); k /= nc1;
@@ -381,14 +384,12 @@ extern "C" int pccnn_poisson_disk_grid(const float *pts_sorted, const int64_t *s
     PCCNN_LAUNCH_CHECK();
     int rc = pccnn_scan_inclusive_i32(flags, selected_scan_out, n, 0, scan_tmp, s);
     if (rc != PCCNN_OK) return rc;
-    cell_list_kernel<<<blocks, 256, 0, s>>>(flags, selected_scan_out, n, cell_first, cell_count);
-    PCCNN_LAUNCH_CHECK();
     if (n > 131072)
         cell_colour_kernel<8><<<(unsigned)pccnn_ceil_div(n, 256 * 8), 256, 0, s>>>(
-            flags, selected_scan_out, sorted_keys, n, num_cells, colour_list, colour_count);
+            flags, selected_scan_out, sorted_keys, n, num_cells, colour_list, colour_count, cell_first, cell_count);
     else
         cell_colour_kernel<1><<<blocks, 256, 0, s>>>(flags, selected_scan_out, sorted_keys, n, num_cells, colour_list,
-                                                     colour_count);
+                                                     colour_count, cell_first, cell_count);
     PCCNN_LAUNCH_CHECK();
     PoissonGridArgs a;
     a.pts = pts_sorted;
