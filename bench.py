@@ -200,7 +200,9 @@ def config5_leg(lib, dev, steps, warmup):
     """Config 5: 8 x 100 000 room points, four Poisson-disk levels (radii 0.025 / 0.05 / 0.1 / 0.2 of the room's
     longest side), each with neighbor search (2 x the pooling radius), density and an MCConv with division by the
     density, channels 8 -> 32 -> 64 -> 128 -> 256, bf16 contraction operands with fp32 accumulation; one forward pass
-    through the four levels and one backward pass, host-synchronised only at the end."""
+    through the four levels and one backward pass, host-synchronised only at the end.  As in a training step, the
+    parameters' gradients are reset to none before the pass (what ``optimizer.zero_grad()`` does), and the backward
+    pass starts from a gradient of ones on the last level's features (the gradient of their sum)."""
     import torch
     from pccnn_lib_amd import synthetic
     batch, num_pts = 8, 100000
@@ -217,8 +219,12 @@ def config5_leg(lib, dev, steps, warmup):
     feats0 = torch.randn(pts.shape[0], 8, device=dev)
     radii_levels = (0.025, 0.05, 0.1, 0.2)
     sizes, marks = [], []
+    params = [p for layer in layers for p in layer.parameters()]
+    ones = {}
 
     def whole(split=False):
+        for p in params:
+            p.grad = None
         pc = lib.pc.Pointcloud(tp, ti)
         feats = feats0.clone().requires_grad_(True)
         del sizes[:], marks[:]
@@ -239,7 +245,10 @@ def config5_leg(lib, dev, steps, warmup):
         if split:
             torch.cuda.synchronize()
             marks.append(time.perf_counter())
-        feats.sum().backward()
+        shape = tuple(feats.shape)
+        if shape not in ones:
+            ones[shape] = torch.ones(shape, dtype=feats.dtype, device=dev)
+        feats.backward(ones[shape])
         if split:
             torch.cuda.synchronize()
             marks.append(time.perf_counter())

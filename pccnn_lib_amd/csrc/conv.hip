@@ -457,6 +457,9 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
     LaneBasis<BASIS> lb;
     lb.load(g, k);
     const int fblocks = (g.c_in + 63) / 64;
+    // gradients towards positions or densities wanted (uniform): otherwise the per-pair sums over the basis index
+    // and their hand-over through LDS are skipped
+    const bool geometry = d_pts != nullptr || d_samples != nullptr || d_pdf != nullptr || pair_grads != nullptr;
     float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;       // parameter gradients of this lane's k (FUSED)
     float sg = 0.f;                                     // component (lane & 3) of the sample's gradient, unsigned
 
@@ -615,6 +618,7 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
                 float gx = 0.f, gy = 0.f, gz = 0.f, gpdf = 0.f;
                 if (j < cnt && lb.active)
                     basis_derivative<BASIS>(g, lb, ge.x, ge.y, ge.z, ge.w, db_lds[j][k], gx, gy, gz, gpdf, p0, p1, p2, p3);
+                if (!geometry) continue;                // only the parameters' gradients are asked for
                 // summed over the basis index: the KPAD lanes of this pair
                 gx = pccnn_group_sum<KPAD>(gx);
                 gy = pccnn_group_sum<KPAD>(gy);
@@ -623,7 +627,7 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
                 if (k < 4) g_lds[j][k] = (k == 0) ? gx * ir0 : (k == 1) ? gy * ir1 : (k == 2) ? gz * ir2 : gpdf;
             }
             __syncthreads();
-            for (int i = 0; i * 16 < cnt; ++i) {
+            for (int i = 0; geometry && i * 16 < cnt; ++i) {
                 const int j = i * 16 + (lane >> 2), comp = lane & 3;
                 if (j < cnt) {
                     const int jn = nidx_lds[j];
@@ -678,7 +682,9 @@ conv_proj_bwd_narrow_kernel(ConvGeom g, const float *__restrict__ feats, const f
                             float *__restrict__ param_partials, float *__restrict__ pair_grads)
 {
     constexpr bool FUSED = want_db && BasisTraits<BASIS>::differentiable;   // basis derivative applied here
-    constexpr int CH = 32;                                          // pairs staged in LDS at a time
+    // pairs staged in LDS at a time: with the feature gradients' atomics in the chunk, 64 (8 x 10^5 points, 8 M pairs,
+    // 8 features: 400 -> 377 us); without them 32, where 64 costs occupancy and gains nothing (221 -> 257 us)
+    constexpr int CH = want_df ? 64 : 32;
     constexpr int PARTS = 64 / KPAD;                                // pairs per step of the dw / derivative stages
     constexpr int GF = 64 / FPAD;                                   // pairs per step of the dF stage
     constexpr bool GEOM = BASIS != BASIS_EXPLICIT;
@@ -702,6 +708,9 @@ conv_proj_bwd_narrow_kernel(ConvGeom g, const float *__restrict__ feats, const f
     }
     LaneBasis<BASIS> lb;
     lb.load(g, k);
+    // gradients towards positions or densities wanted (uniform): otherwise the per-pair sums over the basis index
+    // and their hand-over through LDS are skipped
+    const bool geometry = d_pts != nullptr || d_samples != nullptr || d_pdf != nullptr || pair_grads != nullptr;
     float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;       // parameter gradients of this lane's k (FUSED)
     float sg = 0.f;                                     // component (lane & 3) of the sample's gradient, unsigned
     // the sample's gradient tile: row f (dF stage) and column k (dw stage)
@@ -794,6 +803,7 @@ conv_proj_bwd_narrow_kernel(ConvGeom g, const float *__restrict__ feats, const f
                 float gx = 0.f, gy = 0.f, gz = 0.f, gpdf = 0.f;
                 if (j < cnt && lb.active)
                     basis_derivative<BASIS>(g, lb, ge.x, ge.y, ge.z, ge.w, db_lds[j][k], gx, gy, gz, gpdf, p0, p1, p2, p3);
+                if (!geometry) continue;                // only the parameters' gradients are asked for
                 // summed over the basis index: the KPAD lanes of this pair
                 gx = pccnn_group_sum<KPAD>(gx);
                 gy = pccnn_group_sum<KPAD>(gy);
@@ -802,7 +812,7 @@ conv_proj_bwd_narrow_kernel(ConvGeom g, const float *__restrict__ feats, const f
                 if (k < 4) g_lds[j][k] = (k == 0) ? gx * ir0 : (k == 1) ? gy * ir1 : (k == 2) ? gz * ir2 : gpdf;
             }
             __syncthreads();
-            for (int i = 0; i * 16 < cnt; ++i) {
+            for (int i = 0; geometry && i * 16 < cnt; ++i) {
                 const int j = i * 16 + (lane >> 2), comp = lane & 3;
                 if (j < cnt) {
                     const int jn = nidx_lds[j];

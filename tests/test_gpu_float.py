@@ -318,6 +318,30 @@ def test_cached_projection_and_gradient_masks(ops, oracle):
     assert torch.equal(gw, cached[0]) and relerr(gf.cpu().numpy(), full[1].cpu().numpy()) < 1e-6
 
 
+@pytest.mark.parametrize("c_in", [8, 32, 64])
+def test_parameter_gradients_alone_equal_the_full_call(ops, oracle, c_in):
+    # with no gradient towards positions, samples or densities asked for, the backward projection leaves out the
+    # per-pair geometry sums; the features' and the basis parameters' gradients are those of the full call
+    pts, ids, smp, nb, rng = _conv_case(oracle, ops, 92, 2, 1500, 0.12, True)
+    d = nb["dev"]
+    c_out, k = 16, 8
+    feats = t(rng.normal(size=(pts.shape[0], c_in)).astype(np.float32))
+    pdf = t(rng.uniform(0.5, 2.0, pts.shape[0]).astype(np.float32))
+    axis = t(rng.normal(0, 0.6, (3, k)).astype(np.float32))
+    bias = t(rng.normal(0, 0.1, (1, k)).astype(np.float32))
+    w = t(rng.normal(0, 0.1, (1, k * c_in, c_out)).astype(np.float32))
+    g = t(rng.normal(size=(smp.shape[0], c_out)).astype(np.float32))
+    args = (d["pts"], pdf, feats, d["samples"], d["neigh"], d["ends"], d["radii"], axis, bias, w)
+    full = ops.mc_conv_grads(*args, g)
+    for mask in (ops.GRAD_BASIS_PARAMS, ops.GRAD_BASIS_PARAMS | ops.GRAD_FEATS | ops.GRAD_WEIGHTS):
+        some = ops.mc_conv_grads(*args, g, grad_mask=mask)
+        assert some[4] is None and some[5] is None and some[6] is None       # density, positions, samples
+        assert relerr(some[2].cpu().numpy(), full[2].cpu().numpy()) < 1e-5      # axes
+        assert relerr(some[3].cpu().numpy(), full[3].cpu().numpy()) < 1e-5      # biases
+        if mask & ops.GRAD_FEATS:
+            assert relerr(some[1].cpu().numpy(), full[1].cpu().numpy()) < 1e-6
+
+
 def test_weight_variance_ops_and_layer_warmup(ops, oracle):
     import pccnn_lib_amd as lib
     pts, ids, smp, nb, rng = _conv_case(oracle, ops, 77, 2, 1500, 0.12, True)
