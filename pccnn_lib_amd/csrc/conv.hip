@@ -1285,6 +1285,64 @@ static int conv_forward(ConvGeom g, const float *feats, const float *weights, in
     return PCCNN_OK;
 }
 
+// What the backward call does before its contractions, in one launch: the accumulators that the projection kernel
+// adds into are cleared and the bf16 copies of the output gradients and of the weights are made (up to four
+// arrays to clear and two to convert; unused entries have a count of zero).  One thread per four elements of the
+// jobs laid end to end.
+struct ConvPrepJobs {
+    float *zero[4];
+    int64_t zero_count[4];
+    const float *src[2];
+    uint16_t *dst[2];
+    int64_t convert_count[2];
+};
+
+__global__ void __launch_bounds__(256) conv_prep_kernel(ConvPrepJobs jobs, int64_t quads)
+{
+    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += (int64_t)gridDim.x * blockDim.x) {
+        int64_t at = q;
+        bool done = false;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t job_quads = (jobs.zero_count[j] + 3) / 4;
+            if (!done && at < job_quads) {
+                float *p = jobs.zero[j] + at * 4;
+                const int64_t left = jobs.zero_count[j] - at * 4;
+                if (left >= 4 && (((uintptr_t)p) & 15) == 0) {
+                    *(float4 *)p = make_float4(0.f, 0.f, 0.f, 0.f);
+                } else {
+                    for (int e = 0; e < 4 && e < left; ++e) p[e] = 0.0f;
+                }
+                done = true;
+            }
+            if (!done) at -= job_quads;
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int64_t job_quads = (jobs.convert_count[j] + 3) / 4;
+            if (!done && at < job_quads) {
+                const int64_t left = jobs.convert_count[j] - at * 4;
+                for (int e = 0; e < 4 && e < left; ++e) jobs.dst[j][at * 4 + e] = pccnn_bf16_bits(jobs.src[j][at * 4 + e]);
+                done = true;
+            }
+            if (!done) at -= job_quads;
+        }
+    }
+}
+
+static int conv_prep(const ConvPrepJobs &jobs, hipStream_t s)
+{
+    int64_t quads = 0;
+    for (int j = 0; j < 4; ++j) quads += (jobs.zero_count[j] + 3) / 4;
+    for (int j = 0; j < 2; ++j) quads += (jobs.convert_count[j] + 3) / 4;
+    if (quads == 0) return PCCNN_OK;
+    int64_t blocks = pccnn_ceil_div(quads, 256);
+    if (blocks > 16384) blocks = 16384;
+    conv_prep_kernel<<<(unsigned)blocks, 256, 0, s>>>(jobs, quads);
+    PCCNN_LAUNCH_CHECK();
+    return PCCNN_OK;
+}
+
 // Gradients are produced only for the groups named in `mask`; pointers of groups not requested may be null.
 template <int BASIS>
 static int conv_backward(ConvGeom g, const float *feats, const float *weights, const float *in_grads, int num_mlps,
@@ -1312,12 +1370,15 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     float *stage = partials + partial_rows * 256;
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv backward: workspace of %zu bytes, need %zu", workspace_bytes,
                   pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 1));
-    if (want_f && (rc = pccnn_fill_f32(d_feats, 0.0f, g.n * g.c_in, s)) != PCCNN_OK) return rc;
     // with a mirror index the point-side gradients are written once per point, not accumulated
     const bool gather = mirror != nullptr && Tr::differentiable && (want_pts || want_pdf) && g.m > 0 && g.t > 0;
-    if (want_pts && !gather && (rc = pccnn_fill_f32(d_pts, 0.0f, g.n * 3, s)) != PCCNN_OK) return rc;
-    if (want_pdf && !gather && (rc = pccnn_fill_f32(d_pdf, 0.0f, g.n, s)) != PCCNN_OK) return rc;
+    // the accumulators to clear; the launch follows below, together with the bf16 copies
+    ConvPrepJobs prep = {};
+    if (want_f) { prep.zero[0] = d_feats; prep.zero_count[0] = g.n * g.c_in; }
+    if (want_pts && !gather) { prep.zero[1] = d_pts; prep.zero_count[1] = g.n * 3; }
+    if (want_pdf && !gather) { prep.zero[2] = d_pdf; prep.zero_count[2] = g.n; }
     if (g.m == 0 || g.t == 0) {
+        if ((rc = conv_prep(prep, s)) != PCCNN_OK) return rc;
         if (want_pts && (rc = pccnn_fill_f32(d_samples, 0.0f, g.m * 3, s)) != PCCNN_OK) return rc;
         if (want_par && (rc = pccnn_fill_f32(d_param_a, 0.0f, count_a, s)) != PCCNN_OK) return rc;
         if (want_par && count_b && (rc = pccnn_fill_f32(d_param_b, 0.0f, count_b, s)) != PCCNN_OK) return rc;
@@ -1347,7 +1408,14 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
         PCCNN_LAUNCH_CHECK();
         in_grads = scaled_grads;
     }
-    if (bf16 && (rc = pccnn_f32_to_bf16(in_grads, g16, g.m * c_out, s)) != PCCNN_OK) return rc;
+    const bool with_projection_pass = want_f || want_basis;
+    const bool with_partials = with_projection_pass && want_par && Tr::differentiable;
+    if (with_partials) { prep.zero[3] = partials; prep.zero_count[3] = partial_rows * 256; }
+    if (bf16) {
+        prep.src[0] = in_grads; prep.dst[0] = g16; prep.convert_count[0] = g.m * c_out;
+        if (with_projection_pass) { prep.src[1] = weights; prep.dst[1] = w16; prep.convert_count[1] = w_count; }
+    }
+    if ((rc = conv_prep(prep, s)) != PCCNN_OK) return rc;
     if (want_w) {
         // d_weights = P^T x dOut; P comes from the caller (kept from the forward call) or is rebuilt here
         const void *proj = proj_in;
@@ -1369,7 +1437,6 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     if (!want_f && !want_basis) return PCCNN_OK;
     // d_proj = dOut x W^T
     if (bf16) {
-        if ((rc = pccnn_f32_to_bf16(weights, w16, w_count, s)) != PCCNN_OK) return rc;
         rc = pccnn_gemm_bf16(g16, w16, d_proj, g.m, inner, co, 0, 1, c_out, co, (int64_t)g.c_in * g.k, num_mlps, co,
                              inner * co, inner, 1, nullptr, 0, s);
     } else {
@@ -1379,7 +1446,6 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     if (rc != PCCNN_OK) return rc;
     BasisGradOut o = {basis_g, want_pts ? d_pts : nullptr, want_pts ? d_samples : nullptr, want_pdf ? d_pdf : nullptr,
                       (want_par && Tr::differentiable) ? partials : nullptr, gather ? pair_grads : nullptr};
-    if (o.partials && (rc = pccnn_fill_f32(partials, 0.0f, partial_rows * 256, s)) != PCCNN_OK) return rc;
     if ((rc = launch_proj_bwd<BASIS>(g, feats, d_proj, want_f ? d_feats : nullptr, want_basis, o, s)) != PCCNN_OK)
         return rc;
     if (gather) {
