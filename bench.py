@@ -232,9 +232,11 @@ def config5_leg(lib, dev, steps, warmup):
             if split:
                 torch.cuda.synchronize()
                 marks.append(time.perf_counter())
+            # (the density is queued between the pooling and the first use of its result: the device computes it
+            # while the host waits for the size of the selection)
             pool = lib.pc.PointPooling(pc, radius)
-            out_pc = lib.pc.Pointcloud(pool.pool_tensor(pc.pts_), pool.pool_tensor(pc.batch_ids_))
             pc.compute_pdf(0.2 * radius)
+            out_pc = lib.pc.Pointcloud(pool.pool_tensor(pc.pts_), pool.pool_tensor(pc.batch_ids_))
             feats, nbh = layers[level](pc, out_pc, feats, 2.0 * radius)
             feats = torch.nn.functional.leaky_relu(feats, 0.2)
             # (the pair count from the list the search kept: reading neighbors_ of a key-order list would make the

@@ -246,6 +246,17 @@ int pccnn_pool_poisson_select(const float *pts, const int32_t *batch_ids, int64_
                               int32_t *selected_scan_out, int64_t *count_out, float *pooled_min_out,
                               float *pooled_max_out, float *pooled_host_min_out, float *pooled_host_max_out,
                               void *workspace, size_t workspace_bytes, void *stream);
+/* pccnn_pool_poisson_select without the wait (n > 0, the boxes always): everything is queued on `stream`, ending
+ * with the copy of the results to host_out - host memory of 6 * batch_size floats and one int32, best page-locked,
+ * laid out as [minima f32[batch_size,3] | maxima f32[batch_size,3] | count i32] - and the call returns.  The caller
+ * reads host_out once the work queued up to here has finished (an event recorded after the call, or a stream
+ * synchronisation), and may queue other work on the stream in between; workspace and outputs stay untouched by
+ * others until then.  No counterpart in the reference, whose PointPooling waits where it reads the sizes. */
+int pccnn_pool_poisson_select_queued(const float *pts, const int32_t *batch_ids, int64_t n, int batch_size,
+                                     const float *aabb_min, const float *cell_size, const int32_t *num_cells_host,
+                                     int key_bits, int with_cell_table, int32_t *perm_out, int32_t *selected_out,
+                                     int32_t *selected_scan_out, float *pooled_min_out, float *pooled_max_out,
+                                     void *host_out, void *workspace, size_t workspace_bytes, void *stream);
 int pccnn_compact_selected_remap(const int32_t *selected, const int32_t *selected_scan, const int32_t *remap,
                                  int64_t n, int64_t *ids_out, void *stream);
 /* pccnn_compact_selected_remap with remap = perm, plus the rows a pooled cloud is made of: pooled_pts_out f32[S,d] =

@@ -136,6 +136,67 @@ extern "C" size_t pccnn_pool_poisson_workspace_bytes(int64_t n, int64_t num_pill
            pccnn_align(pccnn_grid_build_workspace_bytes(n)) + pccnn_align(pccnn_poisson_disk_workspace_bytes(n));
 }
 
+// Grid, Poisson-disk selection, the selection's size and (with_box) the selected points' boxes, all queued on the
+// stream and ending with the copies that bring the results to `host_dst`: [minima | maxima | count (int32)] with
+// the boxes, the count alone without.  Nothing waits here.
+static int pool_select_queue(const float *pts, const int32_t *batch_ids, int64_t n, int batch_size,
+                             const float *aabb_min, const float *cell_size, const int32_t *num_cells_host,
+                             int key_bits, int with_cell_table, int32_t *perm_out, int32_t *selected_out,
+                             int32_t *selected_scan_out, float *pooled_min_out, float *pooled_max_out, bool with_box,
+                             void *host_dst, void *workspace, size_t workspace_bytes, hipStream_t s)
+{
+    const char *who = "pccnn_pool_poisson_select";
+    PCCNN_REQUIRE(pts && batch_ids && aabb_min && cell_size && perm_out && selected_out && selected_scan_out,
+                  PCCNN_ERR_INVALID, "%s: null pointer", who);
+    for (int k = 0; k < 3; ++k)
+        PCCNN_REQUIRE(num_cells_host[k] > 0, PCCNN_ERR_INVALID, "%s: %d cells along axis %d", who, num_cells_host[k], k);
+    int64_t num_pillars = (int64_t)batch_size * num_cells_host[0] * num_cells_host[1];
+    int64_t total_cells = with_cell_table ? num_pillars * num_cells_host[2] : 0;
+    PccnnArena arena(workspace, workspace_bytes);
+    PoolLayout l;
+    PCCNN_REQUIRE(pool_layout(arena, n, num_pillars, total_cells, l), PCCNN_ERR_WORKSPACE,
+                  "%s: workspace of %zu bytes, need %zu", who, workspace_bytes,
+                  pccnn_pool_poisson_workspace_bytes(n, num_pillars, total_cells));
+    void *stream = (void *)s;
+    int rc = pccnn_grid_build_sized(pts, batch_ids, aabb_min, num_cells_host, cell_size, n, 3, batch_size, key_bits,
+                                    with_cell_table, l.num_cells, l.keys, l.sorted_keys, perm_out, l.sorted_pts,
+                                    l.grid_ds, l.cell_table, l.sort_ws, l.sort_bytes, stream);
+    if (rc != PCCNN_OK) return rc;
+    rc = pccnn_poisson_disk_grid(l.sorted_pts, l.sorted_keys, n, l.grid_ds, num_pillars, l.cell_table, total_cells,
+                                 l.num_cells, cell_size, 3, selected_out, selected_scan_out, l.poisson_ws,
+                                 l.poisson_bytes, stream);
+    if (rc != PCCNN_OK) return rc;
+    if (!with_box) {
+        PCCNN_HIP_CHECK(hipMemcpyAsync(host_dst, selected_scan_out + (n - 1), sizeof(int32_t), hipMemcpyDeviceToHost, s));
+        return PCCNN_OK;
+    }
+    // The box of the selected points, from the sorted copy and the selection flags.  The kernel that pads the boxes
+    // also writes them, and the count, into one stretch of the workspace (the unsorted keys are not needed any
+    // more), so count and box travel with one copy; with so many clouds that the stretch is too short for that,
+    // with three.
+    const size_t box = (size_t)batch_size * 3 * sizeof(float);
+    const bool one_copy = 2 * box + sizeof(int32_t) <= pccnn_align((size_t)n * sizeof(int64_t));
+    PccnnBoxMask mask;
+    mask.selected = selected_out;
+    mask.perm = perm_out;
+    if (one_copy) {
+        mask.tail = (float *)l.keys;
+        mask.count_src = selected_scan_out + (n - 1);
+    }
+    rc = pccnn_bounding_box_masked(l.sorted_pts, batch_ids, n, 3, batch_size, pooled_min_out, pooled_max_out, mask,
+                                   stream);
+    if (rc != PCCNN_OK) return rc;
+    if (one_copy) {
+        PCCNN_HIP_CHECK(hipMemcpyAsync(host_dst, mask.tail, 2 * box + sizeof(int32_t), hipMemcpyDeviceToHost, s));
+    } else {
+        PCCNN_HIP_CHECK(hipMemcpyAsync(host_dst, pooled_min_out, box, hipMemcpyDeviceToHost, s));
+        PCCNN_HIP_CHECK(hipMemcpyAsync((char *)host_dst + box, pooled_max_out, box, hipMemcpyDeviceToHost, s));
+        PCCNN_HIP_CHECK(hipMemcpyAsync((char *)host_dst + 2 * box, selected_scan_out + (n - 1), sizeof(int32_t),
+                                       hipMemcpyDeviceToHost, s));
+    }
+    return PCCNN_OK;
+}
+
 extern "C" int pccnn_pool_poisson_select(const float *pts, const int32_t *batch_ids, int64_t n, int batch_size,
                                          const float *aabb_min, const float *cell_size,
                                          const int32_t *num_cells_host, int key_bits, int with_cell_table,
@@ -152,66 +213,40 @@ extern "C" int pccnn_pool_poisson_select(const float *pts, const int32_t *batch_
                   "pccnn_pool_poisson_select: the box of the selection needs all four of its outputs");
     *count_out = 0;
     if (n == 0) return PCCNN_OK;
-    PCCNN_REQUIRE(pts && batch_ids && aabb_min && cell_size && perm_out && selected_out && selected_scan_out,
-                  PCCNN_ERR_INVALID, "pccnn_pool_poisson_select: null pointer");
-    for (int k = 0; k < 3; ++k)
-        PCCNN_REQUIRE(num_cells_host[k] > 0, PCCNN_ERR_INVALID, "pccnn_pool_poisson_select: %d cells along axis %d",
-                      num_cells_host[k], k);
-    int64_t num_pillars = (int64_t)batch_size * num_cells_host[0] * num_cells_host[1];
-    int64_t total_cells = with_cell_table ? num_pillars * num_cells_host[2] : 0;
-    PccnnArena arena(workspace, workspace_bytes);
-    PoolLayout l;
-    PCCNN_REQUIRE(pool_layout(arena, n, num_pillars, total_cells, l), PCCNN_ERR_WORKSPACE,
-                  "pccnn_pool_poisson_select: workspace of %zu bytes, need %zu", workspace_bytes,
-                  pccnn_pool_poisson_workspace_bytes(n, num_pillars, total_cells));
     hipStream_t s = (hipStream_t)stream;
-    int rc = pccnn_grid_build_sized(pts, batch_ids, aabb_min, num_cells_host, cell_size, n, 3, batch_size, key_bits,
-                                    with_cell_table, l.num_cells, l.keys, l.sorted_keys, perm_out, l.sorted_pts,
-                                    l.grid_ds, l.cell_table, l.sort_ws, l.sort_bytes, stream);
-    if (rc != PCCNN_OK) return rc;
-    rc = pccnn_poisson_disk_grid(l.sorted_pts, l.sorted_keys, n, l.grid_ds, num_pillars, l.cell_table, total_cells,
-                                 l.num_cells, cell_size, 3, selected_out, selected_scan_out, l.poisson_ws,
-                                 l.poisson_bytes, stream);
-    if (rc != PCCNN_OK) return rc;
-    if (!with_box) {
-        int32_t count = 0;
-        if ((rc = read_back(&count, selected_scan_out + (n - 1), sizeof(int32_t), s)) != PCCNN_OK) return rc;
-        *count_out = count;
-        return PCCNN_OK;
-    }
-    // The box of the selected points, from the sorted copy and the selection flags.  The kernel that pads the boxes
-    // also writes them, and the count, into one stretch of the workspace (the unsorted keys are not needed any
-    // more), so count and box come back with one copy and one wait; with so many clouds that the stretch is too
-    // short for that, they come back with three copies.
-    const size_t box = (size_t)batch_size * 3 * sizeof(float);
-    const bool one_copy = 2 * box + sizeof(int32_t) <= pccnn_align((size_t)n * sizeof(int64_t));
-    PccnnBoxMask mask;
-    mask.selected = selected_out;
-    mask.perm = perm_out;
-    if (one_copy) {
-        mask.tail = (float *)l.keys;
-        mask.count_src = selected_scan_out + (n - 1);
-    }
-    rc = pccnn_bounding_box_masked(l.sorted_pts, batch_ids, n, 3, batch_size, pooled_min_out, pooled_max_out, mask,
-                                   stream);
-    if (rc != PCCNN_OK) return rc;
+    const size_t box = with_box ? (size_t)batch_size * 3 * sizeof(float) : 0;
     void *slot;
+    int rc;
     if ((rc = pinned_slot(2 * box + sizeof(int32_t), &slot)) != PCCNN_OK) return rc;
-    if (one_copy) {
-        PCCNN_HIP_CHECK(hipMemcpyAsync(slot, mask.tail, 2 * box + sizeof(int32_t), hipMemcpyDeviceToHost, s));
-    } else {
-        PCCNN_HIP_CHECK(hipMemcpyAsync(slot, pooled_min_out, box, hipMemcpyDeviceToHost, s));
-        PCCNN_HIP_CHECK(hipMemcpyAsync((char *)slot + box, pooled_max_out, box, hipMemcpyDeviceToHost, s));
-        PCCNN_HIP_CHECK(hipMemcpyAsync((char *)slot + 2 * box, selected_scan_out + (n - 1), sizeof(int32_t),
-                                       hipMemcpyDeviceToHost, s));
-    }
-    PCCNN_HIP_CHECK(hipStreamSynchronize(s));
+    rc = pool_select_queue(pts, batch_ids, n, batch_size, aabb_min, cell_size, num_cells_host, key_bits,
+                           with_cell_table, perm_out, selected_out, selected_scan_out, pooled_min_out, pooled_max_out,
+                           with_box, slot, workspace, workspace_bytes, s);
+    if (rc != PCCNN_OK) return rc;
+    PCCNN_HIP_CHECK(hipStreamSynchronize(s));           // count and box: one wait
     int32_t count;
-    memcpy(pooled_host_min_out, slot, box);
-    memcpy(pooled_host_max_out, (char *)slot + box, box);
+    if (with_box) {
+        memcpy(pooled_host_min_out, slot, box);
+        memcpy(pooled_host_max_out, (char *)slot + box, box);
+    }
     memcpy(&count, (char *)slot + 2 * box, sizeof(int32_t));
     *count_out = count;
     return PCCNN_OK;
+}
+
+extern "C" int pccnn_pool_poisson_select_queued(const float *pts, const int32_t *batch_ids, int64_t n, int batch_size,
+                                                const float *aabb_min, const float *cell_size,
+                                                const int32_t *num_cells_host, int key_bits, int with_cell_table,
+                                                int32_t *perm_out, int32_t *selected_out, int32_t *selected_scan_out,
+                                                float *pooled_min_out, float *pooled_max_out, void *host_out,
+                                                void *workspace, size_t workspace_bytes, void *stream)
+{
+    PCCNN_REQUIRE(n > 0 && n < (1ll << 31) && batch_size > 0, PCCNN_ERR_INVALID,
+                  "pccnn_pool_poisson_select_queued: n=%lld batch_size=%d", (long long)n, batch_size);
+    PCCNN_REQUIRE(host_out && num_cells_host && pooled_min_out && pooled_max_out, PCCNN_ERR_INVALID,
+                  "pccnn_pool_poisson_select_queued: null pointer");
+    return pool_select_queue(pts, batch_ids, n, batch_size, aabb_min, cell_size, num_cells_host, key_bits,
+                             with_cell_table, perm_out, selected_out, selected_scan_out, pooled_min_out, pooled_max_out,
+                             true, host_out, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 extern "C" int pccnn_compact_selected_remap(const int32_t *selected, const int32_t *selected_scan,

@@ -28,10 +28,33 @@ class PointPooling(object):
     greedily in cell order; ``pooling_ids_`` holds the selected ORIGINAL point indices (int64).
     ``cell_average``: points are grouped by grid cell; ``pooling_ids_`` maps a point to its group."""
 
+    # The one-call route queues its work and leaves the wait for the selection's size to the first use of one of
+    # these four (LATER = False: waits in the constructor).  Whatever the caller queues in between - the cloud's
+    # density, typically - runs on the device while the host waits for the count.
+    LATER = True
+    pooling_ids_ = property(lambda self: self._settled("ids"), lambda self, v: self._store("ids", v))
+    pooled_box_ = property(lambda self: self._settled("box"), lambda self, v: self._store("box", v))
+    pooled_pts_ = property(lambda self: self._settled("pts"), lambda self, v: self._store("pts", v))
+    pooled_batch_ids_ = property(lambda self: self._settled("batch_ids"),
+                                 lambda self, v: self._store("batch_ids", v))
+
+    def _store(self, p_name, p_value):
+        self.values_[p_name] = p_value
+
+    def _settled(self, p_name):
+        if self.pending_ is not None:
+            finish, self.pending_ = self.pending_, None
+            ids, box, pts, batch_ids = finish()
+            self.values_.update(ids=ids, box=PooledBox(box) if box is not None else None, pts=pts,
+                                batch_ids=batch_ids)
+        return self.values_.get(p_name)
+
     def __init__(self, p_point_cloud, p_radii, p_method="poisson_disk"):
         self.point_cloud_ = p_point_cloud
         self.radii_ = p_radii
         self.method_ = p_method
+        self.pending_ = None
+        self.values_ = {}
         self.pooled_box_ = None
         self.pooled_pts_ = self.pooled_batch_ids_ = None      # the cloud's own rows, when the pooling call gathered them
         with torch.no_grad():
@@ -41,11 +64,11 @@ class PointPooling(object):
             if ONE_CALL and p_method == "poisson_disk" and p_point_cloud.pts_.shape[1] == 3:
                 if cell_host is not None:
                     # three dimensions, cell size known on the host: grid, selection and its size in one native call
-                    self.pooling_ids_, box, self.pooled_pts_, self.pooled_batch_ids_ = pccnn_lib_ops.pool_poisson(
+                    self.pending_ = pccnn_lib_ops.pool_poisson_later(
                         p_point_cloud.pts_.detach(), p_point_cloud.batch_ids_, bb.min_, cell,
                         lambda: host_num_cells(bb.host(), cell_host), p_point_cloud.batch_size_host())
-                    if box is not None:
-                        self.pooled_box_ = PooledBox(box)
+                    if not self.LATER:
+                        self._settled("ids")
                     return
             grid = Grid(p_point_cloud, bb, p_radii)
             grid.compute_cell_ids()

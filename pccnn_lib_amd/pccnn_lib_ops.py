@@ -645,6 +645,14 @@ def pool_poisson(pts, batch_ids, aabb_min, cell_size, num_cells_host, batch_size
     ``bounding_box_host`` of the pooled cloud would return it (it comes back with the count, in the same read).
     No counterpart in the reference's module; the kernels are those of grid_build, poisson_disk_sampling_grid and
     bounding_box."""
+    return pool_poisson_later(pts, batch_ids, aabb_min, cell_size, num_cells_host, batch_size)()
+
+
+def pool_poisson_later(pts, batch_ids, aabb_min, cell_size, num_cells_host, batch_size):
+    """``pool_poisson`` in two halves: the call queues grid, selection, box and the copy of count and box to pinned
+    memory and returns ``finish``; ``finish()`` waits for that copy, gathers the selected rows and returns what
+    ``pool_poisson`` returns.  Work the caller queues between the two (the cloud's density, say) runs on the device
+    while the host waits for the count."""
     import numpy as np
     name = "pool_poisson"
     _chk(pts, name + ": pts", torch.float32, 2)
@@ -658,14 +666,14 @@ def pool_poisson(pts, batch_ids, aabb_min, cell_size, num_cells_host, batch_size
             or cell_size.shape[0] != 3:
         raise RuntimeError(name + ": 3-D points [N,3], batch_ids [N], aabb_min [B,3], cell_size [3], three grid sizes")
     if n == 0:
-        return torch.empty((0,), dtype=torch.int64, device=dev), None, torch.empty_like(pts), torch.empty_like(batch_ids)
+        empty = (torch.empty((0,), dtype=torch.int64, device=dev), None, torch.empty_like(pts),
+                 torch.empty_like(batch_ids))
+        return lambda: empty
     lib = _lib.load()
     rows = torch.empty((3 * n,), dtype=torch.int32, device=dev)      # permutation | selection flags | their scan
     base = rows.data_ptr()
-    count = ctypes.c_int64(0)
-    mn = torch.empty((batch_size, 3), dtype=torch.float32, device=dev)
-    mx = torch.empty_like(mn)
-    host = np.empty((2, batch_size, 3), dtype=np.float32)
+    box = torch.empty((2, batch_size, 3), dtype=torch.float32, device=dev)
+    landing = torch.empty((6 * batch_size + 1,), dtype=torch.float32, pin_memory=True)
     # (the grid size last: when it is a callable it may have to wait for the cloud's box to arrive on the host)
     cells = [int(v) for v in (num_cells_host() if callable(num_cells_host) else num_cells_host)]
     if len(cells) != 3 or min(cells) < 1:
@@ -674,16 +682,27 @@ def pool_poisson(pts, batch_ids, aabb_min, cell_size, num_cells_host, batch_size
     total = pillars * cells[2]
     with_table = 1 if total <= CELL_TABLE_MAX_CELLS else 0
     ws = _workspace(lib.pccnn_pool_poisson_workspace_bytes(n, pillars, total if with_table else 0), dev)
-    _lib.call("pccnn_pool_poisson_select", _ptr(pts), _ptr(batch_ids), n, batch_size, _ptr(aabb_min), _ptr(cell_size),
-              (ctypes.c_int32 * 3)(*cells), key_bits_for(cells, batch_size), with_table, _P(base), _P(base + 4 * n),
-              _P(base + 8 * n), ctypes.byref(count), _ptr(mn), _ptr(mx), _P(host.ctypes.data),
-              _P(host.ctypes.data + host[0].nbytes), _ptr(ws), ws.numel(), _stream())
-    ids = torch.empty((count.value,), dtype=torch.int64, device=dev)
-    pooled_pts = torch.empty((count.value, 3), dtype=torch.float32, device=dev)
-    pooled_ids = torch.empty((count.value,), dtype=torch.int32, device=dev)
-    _lib.call("pccnn_compact_pooled", _P(base + 4 * n), _P(base + 8 * n), _P(base), _ptr(pts), _ptr(batch_ids), n, 3,
-              _ptr(ids), _ptr(pooled_pts), _ptr(pooled_ids), _stream())
-    return ids, (mn, mx, (host[0], host[1])), pooled_pts, pooled_ids
+    _lib.call("pccnn_pool_poisson_select_queued", _ptr(pts), _ptr(batch_ids), n, batch_size, _ptr(aabb_min),
+              _ptr(cell_size), (ctypes.c_int32 * 3)(*cells), key_bits_for(cells, batch_size), with_table, _P(base),
+              _P(base + 4 * n), _P(base + 8 * n), _P(box.data_ptr()), _P(box.data_ptr() + 12 * batch_size),
+              _P(landing.data_ptr()), _ptr(ws), ws.numel(), _stream())
+    done = torch.cuda.Event()
+    done.record()
+
+    def finish():
+        done.synchronize()
+        host = landing.numpy()
+        count = int(host[6 * batch_size:].view(np.int32)[0])
+        host_box = host[:6 * batch_size].reshape(2, batch_size, 3)
+        ids = torch.empty((count,), dtype=torch.int64, device=dev)
+        pooled_pts = torch.empty((count, 3), dtype=torch.float32, device=dev)
+        pooled_ids = torch.empty((count,), dtype=torch.int32, device=dev)
+        # (`rows` through the tensor itself: the closure keeps permutation, flags and scan alive until they are read)
+        at = rows.data_ptr()
+        _lib.call("pccnn_compact_pooled", _P(at + 4 * n), _P(at + 8 * n), _P(at), _ptr(pts), _ptr(batch_ids), n,
+                  3, _ptr(ids), _ptr(pooled_pts), _ptr(pooled_ids), _stream())
+        return ids, (box[0], box[1], (host_box[0], host_box[1])), pooled_pts, pooled_ids
+    return finish
 
 
 # ----------------------------------------------------------------------------- conv

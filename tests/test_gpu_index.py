@@ -472,6 +472,38 @@ def test_one_call_pooling_density_and_neighborhood_equal_the_step_by_step_routes
         assert x.dtype == y.dtype and tuple(x.shape) == tuple(y.shape) and torch.equal(x, y)
 
 
+@pytest.mark.parametrize("num_pts", [900, 30000])
+def test_pooling_settles_on_first_use_with_other_work_queued_in_between(ops, monkeypatch, num_pts):
+    # the one-call pooling queues its work and waits for the selection's size only when a result is asked for;
+    # density, allocations of every size and a second pooling queued in between change nothing, and the result is
+    # that of the pooling that waits in its constructor
+    import pccnn_lib_amd as lib
+    from pccnn_lib_amd.pc.point_pooling import PointPooling
+    pts, ids = synthetic.primitives(57, 3, num_pts)
+    radius = 0.06
+
+    def run(later):
+        monkeypatch.setattr(PointPooling, "LATER", later)
+        pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+        pool = PointPooling(pc, radius)
+        assert (pool.pending_ is not None) == later
+        other = PointPooling(pc, 2.0 * radius)
+        pc.compute_pdf(0.25 * radius)
+        junk = [torch.full((size,), 7, dtype=torch.int32, device=DEV) for size in (64, 5000, 3 * num_pts, 400000)]
+        out_pts, out_ids = pool.pool_tensor(pc.pts_), pool.pool_tensor(pc.batch_ids_)
+        assert pool.pending_ is None and all(int(j[0]) == 7 for j in junk)
+        box = out_pts.pccnn_pooled_box_.box
+        return [pool.pooling_ids_, out_pts, out_ids, box[0], box[1], torch.as_tensor(box[2][0]),
+                torch.as_tensor(box[2][1]), other.pooling_ids_, pc.pts_unnorm_pdf_]
+
+    a, b = run(False), run(True)
+    assert a[0].shape[0] > 0 and torch.equal(a[1], t(pts)[a[0]])
+    mn, mx = ops.bounding_box(a[1], a[2], 3)
+    assert torch.equal(a[3], mn) and torch.equal(a[4], mx) and torch.equal(a[5], mn.cpu()) and torch.equal(a[6], mx.cpu())
+    for x, y in zip(a, b):
+        assert x.dtype == y.dtype and tuple(x.shape) == tuple(y.shape) and torch.equal(x, y)
+
+
 def test_bounding_box_comes_back_on_the_host_with_the_same_call(ops):
     pts, ids = synthetic.primitives(3, 5, 800)
     mn, mx, (host_mn, host_mx) = ops.bounding_box_host(t(pts), t(ids), 5)
