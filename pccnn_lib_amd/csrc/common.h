@@ -211,6 +211,32 @@ struct PccnnGridDims {
 int pccnn_compute_keys_sized(const float *pts, const int32_t *batch_ids, const float *aabb_min,
                              const int32_t *num_cells_host, const float *cell_size, int64_t n, int d,
                              int32_t *num_cells_out, int64_t *keys_out, hipStream_t stream);
+// Workgroups are handed to the 8 XCDs round-robin by their linear id, and each XCD has its own L2.  A kernel whose
+// consecutive workgroups work on neighboring parts of space (sorted samples sharing their neighbors) launches
+// pccnn_xcd_grid(blocks, chunk) workgroups and lets workgroup b do the work of logical block
+// pccnn_xcd_block(b, grid, chunk): runs of `chunk` consecutive logical blocks go to one XCD, so that what
+// neighbors share stays in its L2, and the runs are dealt to the XCDs in turn, so that all of them sweep through
+// the same part of space at a time and a dense region does not land on one XCD alone.  A grid of fewer than
+// 8 * chunk blocks is cut into eight runs.  Logical blocks past the real count must return at once.
+#define PCCNN_XCDS 8
+static inline unsigned pccnn_xcd_grid(int64_t blocks, int chunk)
+{
+    int64_t per = (blocks + PCCNN_XCDS - 1) / PCCNN_XCDS;
+    if (per > chunk) per = chunk;
+    if (per < 1) per = 1;
+    const int64_t super = per * PCCNN_XCDS;
+    return (unsigned)(((blocks + super - 1) / super) * super);
+}
+#ifdef __HIPCC__
+__device__ __forceinline__ int64_t pccnn_xcd_block(unsigned block, unsigned grid, int chunk)
+{
+    const unsigned per = grid / PCCNN_XCDS < (unsigned)chunk ? grid / PCCNN_XCDS : (unsigned)chunk;
+    const unsigned super = per * PCCNN_XCDS;
+    const unsigned within = block % super;
+    return (int64_t)(block - within) + (int64_t)(within % PCCNN_XCDS) * per + within / PCCNN_XCDS;
+}
+#endif
+
 // The bounding box of a subset of a sorted cloud, and a second copy of the result for one read-back.  With
 // `selected`, point i counts only when selected[i] != 0; with `perm`, its cloud is batch_ids[perm[i]] (the points
 // are a sorted copy, the cloud ids are not).  With `tail`, the padded boxes are also written there as

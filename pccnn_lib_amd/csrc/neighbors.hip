@@ -24,6 +24,9 @@
 // outcome of candidate slot u of its walk iteration i (NB_UNROLL_COUNT slots per iteration).  Word w of all samples
 // is one row, so the 64 lanes of a tile, which finish a word in the same iteration, store it as one run.
 #define NB_PACK_FROM_PAIRS 1000000    // pairs from which the grouped fill packs its point records first
+#ifndef NB_XCD_CHUNK
+#define NB_XCD_CHUNK 64                    // consecutive workgroups of the walk kernels that share an XCD
+#endif
 #define NB_MASK_WORDS 16                               // 256 iterations = 1024 candidate slots per sample are recorded
 
 struct NbArgs {
@@ -100,7 +103,8 @@ __device__ __forceinline__ NbLane nb_lane_setup(const NbArgs &a, int2 (*ranges)[
     NbLane L;
     const int lane = pccnn_lane();
     const int wib = threadIdx.x >> 6;
-    const int64_t wave = ((int64_t)blockIdx.x * NB_THREADS + threadIdx.x) >> 6;
+    // (samples are walked in key order: an XCD gets one contiguous run of them)
+    const int64_t wave = (pccnn_xcd_block(blockIdx.x, gridDim.x, NB_XCD_CHUNK) * NB_THREADS + threadIdx.x) >> 6;
     const int64_t base = wave * 64;
     L.live = base < a.m;                                       // wave-uniform
     if (!L.live) return L;
@@ -480,7 +484,8 @@ neighbors_group_kernel(NbArgs a)
     const int lane = pccnn_lane();
     const int wib = threadIdx.x >> 6;
     const int grp = lane / G, sub = lane % G;
-    const int64_t wave = ((int64_t)blockIdx.x * NB_THREADS + threadIdx.x) >> 6;
+    // (samples are walked in key order: an XCD gets one contiguous run of them)
+    const int64_t wave = (pccnn_xcd_block(blockIdx.x, gridDim.x, NB_XCD_CHUNK) * NB_THREADS + threadIdx.x) >> 6;
     const int64_t at0 = wave * GROUPS + grp;                    // place of the group's sample in the walk order
     if (wave * GROUPS >= a.m) return;                           // wave-uniform
     const bool valid = at0 < a.m;
@@ -841,14 +846,14 @@ extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t
     {
         PccnnTimed timed(PCCNN_T_NB_COUNT, s);
         const unsigned blocks = (unsigned)pccnn_ceil_div(waves, NB_THREADS / 64);
-        if (group == 64) neighbors_group_kernel<false, false, 64><<<blocks, NB_THREADS, 0, s>>>(a);
-        else if (group == 16) neighbors_group_kernel<false, false, 16><<<blocks, NB_THREADS, 0, s>>>(a);
-        else if (group == 8) neighbors_group_kernel<false, false, 8><<<blocks, NB_THREADS, 0, s>>>(a);
-        else if (group == 4) neighbors_group_kernel<false, false, 4><<<blocks, NB_THREADS, 0, s>>>(a);
+        if (group == 64) neighbors_group_kernel<false, false, 64><<<pccnn_xcd_grid(blocks, NB_XCD_CHUNK), NB_THREADS, 0, s>>>(a);
+        else if (group == 16) neighbors_group_kernel<false, false, 16><<<pccnn_xcd_grid(blocks, NB_XCD_CHUNK), NB_THREADS, 0, s>>>(a);
+        else if (group == 8) neighbors_group_kernel<false, false, 8><<<pccnn_xcd_grid(blocks, NB_XCD_CHUNK), NB_THREADS, 0, s>>>(a);
+        else if (group == 4) neighbors_group_kernel<false, false, 4><<<pccnn_xcd_grid(blocks, NB_XCD_CHUNK), NB_THREADS, 0, s>>>(a);
         else switch (d) {
         case 3:
-            if (n < (1ll << 28)) neighbors_kernel<false, false, NB_UNROLL_COUNT, true><<<blocks, NB_THREADS, 0, s>>>(a);
-            else neighbors_kernel<false, false, NB_UNROLL_COUNT><<<blocks, NB_THREADS, 0, s>>>(a);
+            if (n < (1ll << 28)) neighbors_kernel<false, false, NB_UNROLL_COUNT, true><<<pccnn_xcd_grid(blocks, NB_XCD_CHUNK), NB_THREADS, 0, s>>>(a);
+            else neighbors_kernel<false, false, NB_UNROLL_COUNT><<<pccnn_xcd_grid(blocks, NB_XCD_CHUNK), NB_THREADS, 0, s>>>(a);
             break;
         case 2: neighbors_generic_kernel<false, false, 2><<<blocks, NB_THREADS, 0, s>>>(a); break;
         case 4: neighbors_generic_kernel<false, false, 4><<<blocks, NB_THREADS, 0, s>>>(a); break;
@@ -900,7 +905,7 @@ extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t 
         const unsigned blocks = (unsigned)pccnn_ceil_div(waves, NB_THREADS / 64);
         if (d == 3 && group == 1 && max_neighbors == 0) {
             // the count call left the outcome of every candidate test in the workspace: nothing is tested again
-            neighbors_fill_masks_kernel<<<blocks, NB_THREADS, 0, s>>>(a);
+            neighbors_fill_masks_kernel<<<pccnn_xcd_grid(blocks, NB_XCD_CHUNK), NB_THREADS, 0, s>>>(a);
         } else if (d == 3) {
             // the packed (x, y, z, id) records pay for their launch from a few ten thousand pairs on; the grouped walk
             // of a small search reads the coordinate array and the id table instead
@@ -909,19 +914,19 @@ extern "C" int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t 
             if (n > 0 && packed)
                 pack_points_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(pts_sorted, point_remap, n, rec);
             if (group == 64) {
-                if (max_neighbors > 0) neighbors_group_kernel<true, true, 64><<<blocks, NB_THREADS, 0, s>>>(a);
-                else neighbors_group_kernel<true, false, 64><<<blocks, NB_THREADS, 0, s>>>(a);
+                if (max_neighbors > 0) neighbors_group_kernel<true, true, 64><<<pccnn_xcd_grid(blocks, NB_XCD_CHUNK), NB_THREADS, 0, s>>>(a);
+                else neighbors_group_kernel<true, false, 64><<<pccnn_xcd_grid(blocks, NB_XCD_CHUNK), NB_THREADS, 0, s>>>(a);
             } else if (group == 16) {
-                if (max_neighbors > 0) neighbors_group_kernel<true, true, 16><<<blocks, NB_THREADS, 0, s>>>(a);
-                else neighbors_group_kernel<true, false, 16><<<blocks, NB_THREADS, 0, s>>>(a);
+                if (max_neighbors > 0) neighbors_group_kernel<true, true, 16><<<pccnn_xcd_grid(blocks, NB_XCD_CHUNK), NB_THREADS, 0, s>>>(a);
+                else neighbors_group_kernel<true, false, 16><<<pccnn_xcd_grid(blocks, NB_XCD_CHUNK), NB_THREADS, 0, s>>>(a);
             } else if (group == 8) {
-                if (max_neighbors > 0) neighbors_group_kernel<true, true, 8><<<blocks, NB_THREADS, 0, s>>>(a);
-                else neighbors_group_kernel<true, false, 8><<<blocks, NB_THREADS, 0, s>>>(a);
+                if (max_neighbors > 0) neighbors_group_kernel<true, true, 8><<<pccnn_xcd_grid(blocks, NB_XCD_CHUNK), NB_THREADS, 0, s>>>(a);
+                else neighbors_group_kernel<true, false, 8><<<pccnn_xcd_grid(blocks, NB_XCD_CHUNK), NB_THREADS, 0, s>>>(a);
             } else if (group == 4) {
-                if (max_neighbors > 0) neighbors_group_kernel<true, true, 4><<<blocks, NB_THREADS, 0, s>>>(a);
-                else neighbors_group_kernel<true, false, 4><<<blocks, NB_THREADS, 0, s>>>(a);
-            } else if (max_neighbors > 0) neighbors_kernel<true, true, NB_UNROLL_FILL><<<blocks, NB_THREADS, 0, s>>>(a);
-            else neighbors_kernel<true, false, NB_UNROLL_FILL><<<blocks, NB_THREADS, 0, s>>>(a);
+                if (max_neighbors > 0) neighbors_group_kernel<true, true, 4><<<pccnn_xcd_grid(blocks, NB_XCD_CHUNK), NB_THREADS, 0, s>>>(a);
+                else neighbors_group_kernel<true, false, 4><<<pccnn_xcd_grid(blocks, NB_XCD_CHUNK), NB_THREADS, 0, s>>>(a);
+            } else if (max_neighbors > 0) neighbors_kernel<true, true, NB_UNROLL_FILL><<<pccnn_xcd_grid(blocks, NB_XCD_CHUNK), NB_THREADS, 0, s>>>(a);
+            else neighbors_kernel<true, false, NB_UNROLL_FILL><<<pccnn_xcd_grid(blocks, NB_XCD_CHUNK), NB_THREADS, 0, s>>>(a);
         } else {
 #define NB_GENERIC(D)                                                                            \
     do {                                                                                         \

@@ -10,6 +10,10 @@
 // fp32 expressions in this file must round exactly as written (no fused multiply-add).
 #pragma clang fp contract(off)
 
+#ifndef PDF_XCD_CHUNK
+#define PDF_XCD_CHUNK 64                   // consecutive workgroups of the grid walk that share an XCD
+#endif
+
 template <int G, bool GRADS, int D>
 __global__ void __launch_bounds__(256)
 pdf_kernel(double norm_const, const float *__restrict__ bandwidth, const float *__restrict__ pts,
@@ -273,7 +277,8 @@ pdf_grid_kernel(PdfGridArgs a)
     __shared__ int2 ranges[4][9][64];          // written and read by the same lane only
     const int lane = pccnn_lane();
     const int wib = threadIdx.x >> 6;
-    const int64_t base = (((int64_t)blockIdx.x * 256 + threadIdx.x) >> 6) * 64;
+    // (the points are in key order: an XCD gets one contiguous run of them)
+    const int64_t base = ((pccnn_xcd_block(blockIdx.x, gridDim.x, PDF_XCD_CHUNK) * 256 + threadIdx.x) >> 6) * 64;
     if (base >= a.n) return;                   // wave-uniform
     const int64_t i = base + lane;
     const bool valid = i < a.n;
@@ -357,7 +362,7 @@ pdf_grid_group_kernel(PdfGridArgs a)
     const int lane = pccnn_lane();
     const int wib = threadIdx.x >> 6;
     const int grp = lane / G, sub = lane % G;
-    const int64_t wave = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 6;
+    const int64_t wave = (pccnn_xcd_block(blockIdx.x, gridDim.x, PDF_XCD_CHUNK) * 256 + threadIdx.x) >> 6;
     if (wave * GROUPS >= a.n) return;                 // wave-uniform
     const int64_t i = wave * GROUPS + grp;
     const bool valid = i < a.n;
@@ -501,9 +506,9 @@ extern "C" int pccnn_compute_pdf_grid(int manifold_dims, const float *bandwidth,
         // one point per lane, unless that leaves the chip short of wavefronts: then 8 or 4 lanes per point, as long
         // as the launch still is one round of wavefronts (256 CUs x 32 x 64 lanes)
         const int64_t chip_lanes = 256 * 32 * 64;
-        if (n * 8 <= chip_lanes) pdf_grid_group_kernel<8><<<(unsigned)pccnn_ceil_div(n * 8, 256), 256, 0, s>>>(a);
-        else if (n * 4 <= chip_lanes) pdf_grid_group_kernel<4><<<(unsigned)pccnn_ceil_div(n * 4, 256), 256, 0, s>>>(a);
-        else pdf_grid_kernel<<<(unsigned)pccnn_ceil_div(n, 256), 256, 0, s>>>(a);
+        if (n * 8 <= chip_lanes) pdf_grid_group_kernel<8><<<pccnn_xcd_grid(pccnn_ceil_div(n * 8, 256), PDF_XCD_CHUNK), 256, 0, s>>>(a);
+        else if (n * 4 <= chip_lanes) pdf_grid_group_kernel<4><<<pccnn_xcd_grid(pccnn_ceil_div(n * 4, 256), PDF_XCD_CHUNK), 256, 0, s>>>(a);
+        else pdf_grid_kernel<<<pccnn_xcd_grid(pccnn_ceil_div(n, 256), PDF_XCD_CHUNK), 256, 0, s>>>(a);
     }
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
