@@ -49,6 +49,15 @@ class PointPooling(object):
                                 batch_ids=batch_ids)
         return self.values_.get(p_name)
 
+    def __del__(self):
+        # a pooling nobody asked for: its queued copy to pinned memory has to land before that memory is released
+        pending = getattr(self, "pending_", None)
+        if pending is not None:
+            try:
+                pending.wait()
+            except Exception:       # interpreter shutdown
+                pass
+
     def __init__(self, p_point_cloud, p_radii, p_method="poisson_disk"):
         self.point_cloud_ = p_point_cloud
         self.radii_ = p_radii

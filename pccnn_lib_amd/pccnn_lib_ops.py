@@ -668,7 +668,9 @@ def pool_poisson_later(pts, batch_ids, aabb_min, cell_size, num_cells_host, batc
     if n == 0:
         empty = (torch.empty((0,), dtype=torch.int64, device=dev), None, torch.empty_like(pts),
                  torch.empty_like(batch_ids))
-        return lambda: empty
+        finish = lambda: empty
+        finish.wait = lambda: None
+        return finish
     lib = _lib.load()
     rows = torch.empty((3 * n,), dtype=torch.int32, device=dev)      # permutation | selection flags | their scan
     base = rows.data_ptr()
@@ -702,6 +704,9 @@ def pool_poisson_later(pts, batch_ids, aabb_min, cell_size, num_cells_host, batc
         _lib.call("pccnn_compact_pooled", _P(at + 4 * n), _P(at + 8 * n), _P(at), _ptr(pts), _ptr(batch_ids), n,
                   3, _ptr(ids), _ptr(pooled_pts), _ptr(pooled_ids), _stream())
         return ids, (box[0], box[1], (host_box[0], host_box[1])), pooled_pts, pooled_ids
+    # a caller that drops `finish` unused waits with this before it lets go of it: the copy into the pinned block
+    # must have landed before the block can be handed out again
+    finish.wait = done.synchronize
     return finish
 
 

@@ -488,6 +488,8 @@ def test_pooling_settles_on_first_use_with_other_work_queued_in_between(ops, mon
         pool = PointPooling(pc, radius)
         assert (pool.pending_ is not None) == later
         other = PointPooling(pc, 2.0 * radius)
+        unused = PointPooling(pc, 3.0 * radius)
+        del unused                                  # never asked for: waits for its queued copy, then lets go
         pc.compute_pdf(0.25 * radius)
         junk = [torch.full((size,), 7, dtype=torch.int32, device=DEV) for size in (64, 5000, 3 * num_pts, 400000)]
         out_pts, out_ids = pool.pool_tensor(pc.pts_), pool.pool_tensor(pc.batch_ids_)
