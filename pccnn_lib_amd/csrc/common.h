@@ -102,6 +102,21 @@ __device__ __forceinline__ float pccnn_dpp(float v)
 #define PCCNN_DPP_ROW_MIRROR 0x140
 #define PCCNN_DPP_ROW_HALF_MIRROR 0x141
 
+// Inclusive prefix sum over the 64 lanes of a wavefront, all of them active: shifts by 1, 2, 4 and 8 inside the
+// rows of sixteen (a lane whose source falls outside its row adds zero), then lane 15 of a row broadcast into the
+// next row (rows 1 and 3), then lane 31 into the upper half - six adds whose second operand comes with the
+// instruction, where six __shfl_up go through the LDS crossbar one after the other.
+__device__ __forceinline__ int pccnn_wave_inclusive_scan_i(int v)
+{
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);     // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);     // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);     // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);     // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);     // row_bcast:15, rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);     // row_bcast:31, rows 2 and 3
+    return v;
+}
+
 // v + (v of the row 16 lanes away), in every lane: rows {0,1} and {2,3} are paired.
 __device__ __forceinline__ float pccnn_add_row_xor16(float v)
 {

@@ -92,12 +92,7 @@ radix_scan_kernel(int32_t *__restrict__ tile_hist, int64_t num_tiles, int32_t *_
     for (int64_t base = 0; base < num_tiles; base += 256) {
         const int64_t i = base + threadIdx.x;
         const int x = i < num_tiles ? row[i] : 0;
-        int incl = x;
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            const int t = __shfl_up(incl, o);
-            if (lane >= o) incl += t;
-        }
+        const int incl = pccnn_wave_inclusive_scan_i(x);
         if (lane == 63) wave_tot[wave] = incl;
         __syncthreads();
         int add = carry, tot = 0;
@@ -153,12 +148,7 @@ radix_scatter_kernel(const int64_t *__restrict__ keys_in, const int32_t *__restr
             }
             sum += tot[q];
         }
-        int incl = sum;
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            const int t = __shfl_up(incl, o);
-            if (lane >= o) incl += t;
-        }
+        const int incl = pccnn_wave_inclusive_scan_i(sum);
         if (lane == 63) wave_cnt[0][wave] = incl;
         __syncthreads();
         int excl = incl - sum;
@@ -316,12 +306,7 @@ radix_scatter_staged_kernel(const int64_t *__restrict__ keys_in, const int32_t *
     }
     int local_start = sum_tot, global_start = sum_glob;
     {
-        int ia = local_start, ib = global_start;
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            const int ta = __shfl_up(ia, o), tb = __shfl_up(ib, o);
-            if (lane >= o) { ia += ta; ib += tb; }
-        }
+        const int ia = pccnn_wave_inclusive_scan_i(local_start), ib = pccnn_wave_inclusive_scan_i(global_start);
         if (lane == 63) { misc[wave] = ia; misc[RS_WAVES + wave] = ib; }
         __syncthreads();
         int pa = 0, pb = 0;

@@ -210,11 +210,7 @@ __device__ __forceinline__ int block_inclusive_scan(int v, int *lds /* >= 4 ints
 {
     int lane = pccnn_lane();
     int wave = threadIdx.x >> 6;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        int t = __shfl_up(v, o);
-        if (lane >= o) v += t;
-    }
+    v = pccnn_wave_inclusive_scan_i(v);
     if (lane == 63) lds[wave] = v;
     __syncthreads();
     int add = 0;
@@ -318,11 +314,12 @@ scan_add_kernel(int32_t *__restrict__ out, int64_t n, const int32_t *__restrict_
 }
 
 // Up to SCAN_SMALL_MAX elements: one workgroup of 1024 threads, one launch instead of three (each of which runs for
-// 4 to 6 us whatever its size).  Every thread owns ITEMS consecutive elements and requests them all before it adds
-// anything, so the launch costs one memory round trip, one scan over the 16 wavefronts' totals and the stores
-// (6 844 elements: 10 -> 8 us against a loop over tiles of 2048 that waits for its loads tile after tile).
+// 4 to 6 us whatever its size).  Every wavefront owns ITEMS (4 to 48) consecutive rows of 64 elements and requests
+// them all before it adds anything (lane = column: every load and store is one contiguous 256-byte row), scans row
+// after row (pccnn_wave_inclusive_scan_i) with a running total, and the 16 wavefronts' totals meet in LDS: one memory round
+// trip, ITEMS row scans, one exchange, the stores.
 #define SCAN_SMALL_THREADS 1024
-#define SCAN_SMALL_MAX (32 * SCAN_SMALL_THREADS)
+#define SCAN_SMALL_MAX (48 * SCAN_SMALL_THREADS)
 
 template <int ITEMS>
 __global__ void __launch_bounds__(SCAN_SMALL_THREADS)
@@ -333,30 +330,24 @@ scan_small_kernel(const int32_t *__restrict__ in, int32_t *__restrict__ out, int
     __shared__ int wave_sum[WAVES];
     __shared__ long long wave_wide[WAVES];
     const int lane = pccnn_lane(), wave = threadIdx.x >> 6;
-    const int64_t base = (int64_t)threadIdx.x * ITEMS;
+    const int64_t base = (int64_t)wave * ITEMS * 64 + lane;
     int v[ITEMS];
 #pragma unroll
-    for (int i = 0; i < ITEMS; ++i) v[i] = (base + i < n) ? in[base + i] : 0;
-    int sum = 0;
+    for (int i = 0; i < ITEMS; ++i) v[i] = (base + i * 64 < n) ? in[base + i * 64] : 0;
+    int carry = 0;
     long long wide = 0;
 #pragma unroll
     for (int i = 0; i < ITEMS; ++i) {
         int x = v[i];
         if (clamp_max > 0 && x > clamp_max) x = clamp_max;
-        sum += x;
         wide += x;
-        v[i] = sum;
-    }
-    int incl = sum;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        const int t = __shfl_up(incl, o);
-        if (lane >= o) incl += t;
+        x = pccnn_wave_inclusive_scan_i(x);
+        v[i] = x + carry;
+        carry += pccnn_bcast_i(x, 63);
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) wide += __shfl_xor(wide, o);
-    if (lane == 63) wave_sum[wave] = incl;
-    if (lane == 0) wave_wide[wave] = wide;
+    if (lane == 0) { wave_sum[wave] = carry; wave_wide[wave] = wide; }
     __syncthreads();
     int before = 0;
     long long total = 0;
@@ -365,10 +356,9 @@ scan_small_kernel(const int32_t *__restrict__ in, int32_t *__restrict__ out, int
         if (w < wave) before += wave_sum[w];
         total += wave_wide[w];
     }
-    const int excl = before + incl - sum;
 #pragma unroll
     for (int i = 0; i < ITEMS; ++i)
-        if (base + i < n) out[base + i] = v[i] + excl;
+        if (base + i * 64 < n) out[base + i * 64] = v[i] + before;
     if (total_out && threadIdx.x == 0) total_out[0] = total;
 }
 
@@ -381,7 +371,8 @@ int pccnn_scan_inclusive_i32(const int32_t *in, int32_t *out, int64_t n, int cla
         if (n <= 4 * SCAN_SMALL_THREADS) scan_small_kernel<4><<<1, SCAN_SMALL_THREADS, 0, stream>>>(in, out, n, clamp_max, total);
         else if (n <= 8 * SCAN_SMALL_THREADS) scan_small_kernel<8><<<1, SCAN_SMALL_THREADS, 0, stream>>>(in, out, n, clamp_max, total);
         else if (n <= 16 * SCAN_SMALL_THREADS) scan_small_kernel<16><<<1, SCAN_SMALL_THREADS, 0, stream>>>(in, out, n, clamp_max, total);
-        else scan_small_kernel<32><<<1, SCAN_SMALL_THREADS, 0, stream>>>(in, out, n, clamp_max, total);
+        else if (n <= 32 * SCAN_SMALL_THREADS) scan_small_kernel<32><<<1, SCAN_SMALL_THREADS, 0, stream>>>(in, out, n, clamp_max, total);
+        else scan_small_kernel<48><<<1, SCAN_SMALL_THREADS, 0, stream>>>(in, out, n, clamp_max, total);
         PCCNN_LAUNCH_CHECK();
         return PCCNN_OK;
     }

@@ -506,6 +506,20 @@ def test_pooling_settles_on_first_use_with_other_work_queued_in_between(ops, mon
         assert x.dtype == y.dtype and tuple(x.shape) == tuple(y.shape) and torch.equal(x, y)
 
 
+@pytest.mark.parametrize("m", [4096, 4097, 8193, 16385, 32768, 32769, 49152, 49153, 70000])
+def test_start_ids_are_the_running_sum_of_the_counts_at_every_scan_size(ops, m):
+    # the scan behind start_ids_ runs as one workgroup with 4, 8, 16, 32 or 48 elements per thread, or as three
+    # launches: sample counts on either side of every limit, start_ids_ against numpy's cumulative sum of the
+    # per-sample pair counts
+    rng = np.random.default_rng(m)
+    pts = rng.random((20000, 3), dtype=np.float32)
+    samples = rng.random((m, 3), dtype=np.float32)
+    nb = gpu_neighborhood(ops, pts, np.zeros(20000, np.int32), samples, np.zeros(m, np.int32), 0.03, 1)
+    counts = np.bincount(nb["neighbors"][:, 1], minlength=m)
+    assert nb["ends"].shape == (m,) and nb["neighbors"].shape[0] > m
+    assert np.array_equal(nb["ends"], np.cumsum(counts))
+
+
 def test_bounding_box_comes_back_on_the_host_with_the_same_call(ops):
     pts, ids = synthetic.primitives(3, 5, 800)
     mn, mx, (host_mn, host_mx) = ops.bounding_box_host(t(pts), t(ids), 5)
