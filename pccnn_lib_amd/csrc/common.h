@@ -144,6 +144,22 @@ __device__ __forceinline__ float pccnn_group_sum(float v)
     return v;
 }
 
+// Minimum (MAX = false) or maximum over the 64 lanes of a wavefront, left in every lane; the exchanges of
+// pccnn_group_sum<64>.  All lanes must be active.
+template <bool MAX>
+__device__ __forceinline__ float pccnn_wave_minmax(float v)
+{
+    auto pick = [](float a, float b) { return MAX ? fmaxf(a, b) : fminf(a, b); };
+    v = pick(v, pccnn_dpp<PCCNN_DPP_QUAD_XOR1>(v));
+    v = pick(v, pccnn_dpp<PCCNN_DPP_QUAD_XOR2>(v));
+    v = pick(v, pccnn_dpp<PCCNN_DPP_ROW_HALF_MIRROR>(v));
+    v = pick(v, pccnn_dpp<PCCNN_DPP_ROW_MIRROR>(v));
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = pick(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    const auto q = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return pick(__uint_as_float(q[0]), __uint_as_float(q[1]));
+}
+
 // Sum over the lanes that share (lane % STRIDE) (STRIDE a power of two, 1..64), left in every one of them.
 // Inside a row the cosets are closed under rotation, so rotations by STRIDE, 2 STRIDE, ... add them up.
 template <int STRIDE>

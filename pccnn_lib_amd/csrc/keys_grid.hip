@@ -40,12 +40,8 @@ __device__ __forceinline__ void bbox_flush_wave(int cur, const float (&lo)[D], c
         const bool mine = cur == b;
 #pragma unroll
         for (int k = 0; k < D; ++k) {
-            float l = mine ? lo[k] : inf, h = mine ? hi[k] : -inf;
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) {
-                l = fminf(l, __shfl_xor(l, o));
-                h = fmaxf(h, __shfl_xor(h, o));
-            }
+            const float l = pccnn_wave_minmax<false>(mine ? lo[k] : inf);
+            const float h = pccnn_wave_minmax<true>(mine ? hi[k] : -inf);
             if (pccnn_lane() == 0) {
                 atomic_min_f32(&mn[b * D + k], l);
                 atomic_max_f32(&mx[b * D + k], h);
@@ -117,11 +113,8 @@ bbox_reduce_kernel(const float *__restrict__ pts, const int32_t *__restrict__ ba
     if (wave_uniform) {
 #pragma unroll
         for (int k = 0; k < D; ++k) {
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) {
-                lo[k] = fminf(lo[k], __shfl_xor(lo[k], o));
-                hi[k] = fmaxf(hi[k], __shfl_xor(hi[k], o));
-            }
+            lo[k] = pccnn_wave_minmax<false>(lo[k]);
+            hi[k] = pccnn_wave_minmax<true>(hi[k]);
         }
         if (lane == 0) {
             lds_b[wave] = b0;
