@@ -38,7 +38,8 @@ cell_list_kernel(const int32_t *__restrict__ flags, const int32_t *__restrict__ 
 }
 
 // Three dimensions: the non-empty cells listed per parity colour, so that a pass only touches the cells it works
-// on.  colour_list[colour * n + i] = index (into cell_first) of the i-th cell of that colour, in no particular
+// on.  colour_list[colour * n + i] = (index into cell_first, first point, key) of the i-th cell of that colour - what
+// a pass needs to start on a cell, in one 16-byte load instead of three dependent ones -, in no particular
 // order: cells of one colour do not interact, so the selection does not depend on the order.  colour_count[8]
 // must be zero on entry.  The kernel writes the list of first points and the number of cells as well (what
 // cell_list_kernel does for the other dimensions).
@@ -47,7 +48,7 @@ cell_list_kernel(const int32_t *__restrict__ flags, const int32_t *__restrict__ 
 template <int COLOUR_ITEMS>
 __global__ void __launch_bounds__(256)
 cell_colour_kernel(const int32_t *__restrict__ flags, const int32_t *__restrict__ scan, const int64_t *__restrict__ keys,
-                   int64_t n, const int32_t *__restrict__ num_cells, int32_t *__restrict__ colour_list,
+                   int64_t n, const int32_t *__restrict__ num_cells, int4 *__restrict__ colour_list,
                    int32_t *__restrict__ colour_count, int32_t *__restrict__ cell_first, int32_t *__restrict__ count)
 {
     // the workgroup counts its cells per colour in LDS and reserves its share of every list with one atomic
@@ -78,7 +79,11 @@ cell_colour_kernel(const int32_t *__restrict__ flags, const int32_t *__restrict_
 #pragma unroll
     for (int r = 0; r < COLOUR_ITEMS; ++r) {
         const int64_t i = ((int64_t)blockIdx.x * COLOUR_ITEMS + r) * 256 + threadIdx.x;
-        if (colour[r] >= 0) colour_list[(int64_t)colour[r] * n + start[colour[r]] + at[r]] = scan[i] - 1;
+        if (colour[r] >= 0) {
+            const long long k = keys[i];
+            colour_list[(int64_t)colour[r] * n + start[colour[r]] + at[r]] =
+                make_int4(scan[i] - 1, (int)i, (int)(k & 0xffffffffll), (int)(k >> 32));
+        }
     }
 }
 
@@ -171,7 +176,7 @@ struct PoissonGridArgs {
     volatile int32_t *used;      // [n] selection flags
     const int32_t *cell_first;   // compact list of the non-empty cells
     const int32_t *cell_count;
-    const int32_t *colour_list;  // [8][n] cells per parity colour (indices into cell_first)
+    const int4 *colour_list;     // [8][n] cells per parity colour: (index into cell_first, first point, key lo, key hi)
     const int32_t *colour_count; // [8]
 };
 
@@ -192,10 +197,10 @@ poisson_grid_pass_kernel(PoissonGridArgs a, int colour)
     const float ir1 = __fdiv_rn(1.0f, a.radii[1]);
     const float ir2 = __fdiv_rn(1.0f, a.radii[2]);
     for (int64_t ci = wave; ci < mine; ci += waves) {
-        const int c = a.colour_list[(int64_t)colour * a.grid.n + ci];
-        const int first = a.cell_first[c];
+        const int4 rec = a.colour_list[(int64_t)colour * a.grid.n + ci];
+        const int c = rec.x, first = rec.y;
         const int last = (c + 1 < cells) ? a.cell_first[c + 1] : (int)a.grid.n;
-        long long k = a.grid.pt_keys[first];
+        long long k = ((long long)rec.w << 32) | (unsigned int)rec.z;
         const int c2 = (int)(k % nc2); k /= nc2;
         const int c1 = (int)(k % nc1);
         const long long pil = k; k /= nc1;
@@ -308,9 +313,9 @@ compact_kernel(const int32_t *__restrict__ flags, const int32_t *__restrict__ sc
 extern "C" size_t pccnn_poisson_disk_workspace_bytes(int64_t n)
 {
     if (n < 1) n = 1;
-    // scan scratch | cell flags | first point of every cell | cell count, colour counts | cells per colour (3-D)
+    // scan scratch | cell flags | first point of every cell | cell count, colour counts | 16-byte cell records per colour (3-D)
     return pccnn_align(pccnn_scan_tmp_elems(n) * sizeof(int32_t)) + 2 * pccnn_align((size_t)n * sizeof(int32_t)) + 512 +
-           pccnn_align(8 * (size_t)n * sizeof(int32_t));
+           pccnn_align(8 * (size_t)n * 4 * sizeof(int32_t));
 }
 
 extern "C" int pccnn_poisson_disk_select(const int64_t *sorted_keys, int64_t n, const int32_t *neigh, int64_t t,
@@ -375,7 +380,7 @@ extern "C" int pccnn_poisson_disk_grid(const float *pts_sorted, const int64_t *s
     int32_t *flags = arena.take<int32_t>((size_t)n);
     int32_t *cell_first = arena.take<int32_t>((size_t)n);
     int32_t *cell_count = arena.take<int32_t>(64);               // [0]: cells; [8..15]: cells per colour
-    int32_t *colour_list = arena.take<int32_t>(8 * (size_t)n);
+    int4 *colour_list = arena.take<int4>(8 * (size_t)n);
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "pccnn_poisson_disk_grid: workspace of %zu bytes, need %zu",
                   workspace_bytes, pccnn_poisson_disk_workspace_bytes(n));
     int32_t *colour_count = cell_count + 8;
