@@ -295,6 +295,10 @@ struct PccnnBoxMask {
 int pccnn_bounding_box_masked(const float *pts, const int32_t *batch_ids, int64_t n, int d, int batch_size,
                               float *aabb_min_out, float *aabb_max_out, const PccnnBoxMask &mask, void *stream);
 
+// Where the next pccnn_find_neighbors_count of this host thread writes its 64-bit pair total instead of the head of
+// its workspace (device-visible memory, e.g. mapped host memory; nullptr: the workspace again).
+void pccnn_redirect_pair_total(int64_t *destination);
+
 // Where the keys of a sort come from when they are made on the way in (3-D points): the arguments of the key
 // computation.  The grid size is read from `num_cells` (device) or, with `use_sized`, taken from `sized` and written
 // to `num_cells_out` for the kernels that follow.

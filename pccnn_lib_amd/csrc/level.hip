@@ -8,6 +8,7 @@
 // an asynchronous copy into it on the caller's stream, then a wait for that stream.
 #include "common.h"
 #include <string.h>
+#include <chrono>
 
 namespace {
 
@@ -393,10 +394,31 @@ extern "C" int pccnn_neighborhood_count(const float *pts, const int32_t *batch_i
     } else {
         PCCNN_REQUIRE(m == n, PCCNN_ERR_INVALID, "pccnn_neighborhood_count: without samples m must equal n");
     }
+    // The scan that ends the count writes the 64-bit pair total straight into the pinned host buffer (mapped into
+    // the device's address space), and the host polls that word: no copy launch behind the scan and no wake-up
+    // through the runtime.  Should the word not arrive (it always has), the stream is waited for as before.
+    void *slot, *slot_on_device;
+    if ((rc = pinned_slot(sizeof(int64_t), &slot)) != PCCNN_OK) return rc;
+    PCCNN_HIP_CHECK(hipHostGetDevicePointer(&slot_on_device, slot, 0));
+    volatile int64_t *word = (volatile int64_t *)slot;
+    const int64_t pending = INT64_MIN;
+    *word = pending;
+    pccnn_redirect_pair_total((int64_t *)slot_on_device);
     rc = pccnn_find_neighbors_count(sorted_pts_out, sorted_keys_out, n, s_pts, s_keys, m, s_order, 1, grid_ds_out,
                                     num_pillars, with_cell_table ? cell_table_out : nullptr, total_cells, num_cells_out,
                                     cell_size, 3, max_neighbors, ends_out, workspace, workspace_bytes, stream);
+    pccnn_redirect_pair_total(nullptr);
     if (rc != PCCNN_OK) return rc;
-    // the 64-bit pair total sits at the head of the search's workspace
-    return read_back(total_out, workspace, sizeof(int64_t), (hipStream_t)stream);
+    const auto start = std::chrono::steady_clock::now();
+    unsigned spins = 0;
+    while (*word == pending) {
+        if ((++spins & 1023u) == 0 && std::chrono::steady_clock::now() - start > std::chrono::milliseconds(20)) {
+            PCCNN_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+            break;
+        }
+    }
+    const int64_t total = *word;
+    PCCNN_REQUIRE(total != pending, PCCNN_ERR_INVALID, "pccnn_neighborhood_count: the pair total did not arrive");
+    *total_out = total;
+    return PCCNN_OK;
 }

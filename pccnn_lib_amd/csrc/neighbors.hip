@@ -808,6 +808,9 @@ static int nb_validate(const char *who, const float *pts_sorted, const int64_t *
     return PCCNN_OK;
 }
 
+static thread_local int64_t *g_pair_total_destination = nullptr;
+void pccnn_redirect_pair_total(int64_t *destination) { g_pair_total_destination = destination; }
+
 extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t *pt_keys_sorted, int64_t n,
                                           const float *samples, const int64_t *sample_keys, int64_t m,
                                           const int32_t *sample_order, int samples_presorted,
@@ -825,6 +828,7 @@ extern "C" int pccnn_find_neighbors_count(const float *pts_sorted, const int64_t
     hipStream_t s = (hipStream_t)stream;
     PccnnArena arena(workspace, workspace_bytes);
     int64_t *total64 = arena.take<int64_t>(1);
+    if (g_pair_total_destination != nullptr) total64 = g_pair_total_destination;
     int32_t *counts = arena.take<int32_t>((size_t)m);
     const int64_t m_pad = pccnn_ceil_div(m, 64) * 64;
     unsigned long long *masks = arena.take<unsigned long long>((size_t)NB_MASK_WORDS * m_pad);
