@@ -251,7 +251,11 @@ int pccnn_pool_poisson_select(const float *pts, const int32_t *batch_ids, int64_
  * laid out as [minima f32[batch_size,3] | maxima f32[batch_size,3] | count i32] - and the call returns.  The caller
  * reads host_out once the work queued up to here has finished (an event recorded after the call, or a stream
  * synchronisation), and may queue other work on the stream in between; workspace and outputs stay untouched by
- * others until then.  No counterpart in the reference, whose PointPooling waits where it reads the sizes. */
+ * others until then.  The count is the last word to arrive (with page-locked host_out and up to 85 clouds the
+ * kernels write host_out themselves, through its device address, the count behind a system-scope fence; otherwise
+ * it travels in a copy of its own behind the boxes), so a caller that stored a negative value there before the call
+ * may poll that word instead of waiting for an event.  No counterpart in the reference, whose PointPooling waits
+ * where it reads the sizes. */
 int pccnn_pool_poisson_select_queued(const float *pts, const int32_t *batch_ids, int64_t n, int batch_size,
                                      const float *aabb_min, const float *cell_size, const int32_t *num_cells_host,
                                      int key_bits, int with_cell_table, int32_t *perm_out, int32_t *selected_out,

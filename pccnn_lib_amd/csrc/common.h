@@ -271,7 +271,9 @@ __device__ __forceinline__ int64_t pccnn_xcd_block(unsigned block, unsigned grid
 // The bounding box of a subset of a sorted cloud, and a second copy of the result for one read-back.  With
 // `selected`, point i counts only when selected[i] != 0; with `perm`, its cloud is batch_ids[perm[i]] (the points
 // are a sorted copy, the cloud ids are not).  With `tail`, the padded boxes are also written there as
-// [minima | maxima] followed by the 32-bit word at `count_src`, so that one copy brings box and count to the host.
+// [minima | maxima] followed by the 32-bit word at `count_src` (or 1), so that one copy brings box and count to the
+// host - or none, when `tail` is host memory mapped into the device's address space: the word is written last, so
+// the host can poll it (at most 256 box values then: the kernel that pads the boxes must be one workgroup).
 struct PccnnBoxMask {
     const int32_t *selected = nullptr;
     const int32_t *perm = nullptr;
@@ -288,7 +290,13 @@ struct PccnnBoxMask {
         if (tail == nullptr) return;
         tail[i] = lo;
         tail[count + i] = hi;
-        if (i == 0 && count_src != nullptr) ((int32_t *)tail)[2 * count] = *count_src;
+    }
+    // The word behind the boxes, written by one thread after every box value of `tail` has left (the kernels call
+    // this behind a system-scope fence and a workgroup barrier, so a host that polls the word in mapped memory
+    // finds the boxes complete): the 32-bit word at `count_src`, or 1 without one.
+    __device__ __forceinline__ void publish(int count) const
+    {
+        if (tail != nullptr) ((volatile int32_t *)tail)[2 * count] = count_src != nullptr ? *count_src : 1;
     }
 #endif
 };

@@ -151,6 +151,12 @@ __global__ void bbox_pad_kernel(float *mn, float *mx, int count, PccnnBoxMask ma
         mn[i] = l; mx[i] = h;
         mask.second_copy(i, count, l, h);
     }
+    if (mask.tail != nullptr) {
+        // (the word is behind all the box values only when this is the launch's one workgroup)
+        __threadfence_system();
+        __syncthreads();
+        if (i == 0) mask.publish(count);
+    }
 }
 
 // A small cloud (up to BBOX_SMALL_POINTS points, up to BBOX_SMALL_CLOUDS clouds): one workgroup, the boxes in LDS,
@@ -201,6 +207,11 @@ bbox_small_kernel(const float *__restrict__ pts, const int32_t *__restrict__ bat
         const float l = box_lo[i] - 1e-6f, h = box_hi[i] + 1e-6f;
         mn[i] = l; mx[i] = h;
         mask.second_copy(i, count, l, h);
+    }
+    if (mask.tail != nullptr) {
+        __threadfence_system();
+        __syncthreads();
+        if (threadIdx.x == 0) mask.publish(count);
     }
 }
 

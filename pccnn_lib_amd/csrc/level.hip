@@ -172,29 +172,41 @@ static int pool_select_queue(const float *pts, const int32_t *batch_ids, int64_t
         return PCCNN_OK;
     }
     // The box of the selected points, from the sorted copy and the selection flags.  The kernel that pads the boxes
-    // also writes them, and the count, into one stretch of the workspace (the unsorted keys are not needed any
-    // more), so count and box travel with one copy; with so many clouds that the stretch is too short for that,
-    // with three.
+    // also writes them, and behind them the count, to a second place.  With page-locked `host_dst` that place is
+    // host_dst itself, through its address on the device: nothing is copied, and because the count is written last,
+    // behind a system-scope fence, the caller may poll that word.  Otherwise (or with more than 256 box values, which
+    // the padding kernel writes from several workgroups) the second place is a stretch of the workspace (the
+    // unsorted keys are not needed any more) that one copy brings over, and the count follows in a copy of its own,
+    // so that it still arrives last.
     const size_t box = (size_t)batch_size * 3 * sizeof(float);
-    const bool one_copy = 2 * box + sizeof(int32_t) <= pccnn_align((size_t)n * sizeof(int64_t));
+    void *host_on_device = nullptr;
+    bool direct = batch_size * 3 <= 256;
+    if (direct && hipHostGetDevicePointer(&host_on_device, host_dst, 0) != hipSuccess) {
+        (void)hipGetLastError();                        // pageable memory: not an error, the copies do it
+        direct = false;
+    }
+    const bool staged = !direct && 2 * box + sizeof(int32_t) <= pccnn_align((size_t)n * sizeof(int64_t));
     PccnnBoxMask mask;
     mask.selected = selected_out;
     mask.perm = perm_out;
-    if (one_copy) {
-        mask.tail = (float *)l.keys;
+    if (direct) {
+        mask.tail = (float *)host_on_device;
         mask.count_src = selected_scan_out + (n - 1);
+    } else if (staged) {
+        mask.tail = (float *)l.keys;
     }
     rc = pccnn_bounding_box_masked(l.sorted_pts, batch_ids, n, 3, batch_size, pooled_min_out, pooled_max_out, mask,
                                    stream);
     if (rc != PCCNN_OK) return rc;
-    if (one_copy) {
-        PCCNN_HIP_CHECK(hipMemcpyAsync(host_dst, mask.tail, 2 * box + sizeof(int32_t), hipMemcpyDeviceToHost, s));
+    if (direct) return PCCNN_OK;
+    if (staged) {
+        PCCNN_HIP_CHECK(hipMemcpyAsync(host_dst, mask.tail, 2 * box, hipMemcpyDeviceToHost, s));
     } else {
         PCCNN_HIP_CHECK(hipMemcpyAsync(host_dst, pooled_min_out, box, hipMemcpyDeviceToHost, s));
         PCCNN_HIP_CHECK(hipMemcpyAsync((char *)host_dst + box, pooled_max_out, box, hipMemcpyDeviceToHost, s));
-        PCCNN_HIP_CHECK(hipMemcpyAsync((char *)host_dst + 2 * box, selected_scan_out + (n - 1), sizeof(int32_t),
-                                       hipMemcpyDeviceToHost, s));
     }
+    PCCNN_HIP_CHECK(hipMemcpyAsync((char *)host_dst + 2 * box, selected_scan_out + (n - 1), sizeof(int32_t),
+                                   hipMemcpyDeviceToHost, s));
     return PCCNN_OK;
 }
 

@@ -676,6 +676,8 @@ def pool_poisson_later(pts, batch_ids, aabb_min, cell_size, num_cells_host, batc
     base = rows.data_ptr()
     box = torch.empty((2, batch_size, 3), dtype=torch.float32, device=dev)
     landing = torch.empty((6 * batch_size + 1,), dtype=torch.float32, pin_memory=True)
+    words = landing.numpy().view(np.int32)
+    words[6 * batch_size] = -1                                     # the count arrives last: polled below
     # (the grid size last: when it is a callable it may have to wait for the cloud's box to arrive on the host)
     cells = [int(v) for v in (num_cells_host() if callable(num_cells_host) else num_cells_host)]
     if len(cells) != 3 or min(cells) < 1:
@@ -692,9 +694,17 @@ def pool_poisson_later(pts, batch_ids, aabb_min, cell_size, num_cells_host, batc
     done.record()
 
     def finish():
-        done.synchronize()
+        # the count is the last word to arrive: a short poll of the pinned word, then the event if it takes long
+        spins = 0
+        while words[6 * batch_size] < 0:
+            spins += 1
+            if spins > 100000:
+                done.synchronize()
+                break
         host = landing.numpy()
-        count = int(host[6 * batch_size:].view(np.int32)[0])
+        count = int(words[6 * batch_size])
+        if count < 0:
+            raise RuntimeError(name + ": the selection's size did not arrive")
         host_box = host[:6 * batch_size].reshape(2, batch_size, 3)
         ids = torch.empty((count,), dtype=torch.int64, device=dev)
         pooled_pts = torch.empty((count, 3), dtype=torch.float32, device=dev)
