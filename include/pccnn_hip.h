@@ -227,6 +227,14 @@ int pccnn_poisson_disk_grid(const float *pts_sorted, const int64_t *sorted_keys,
 int pccnn_bounding_box_host(const float *pts, const int32_t *batch_ids, int64_t n, int d, int batch_size,
                             float *aabb_min_out, float *aabb_max_out, float *host_min_out, float *host_max_out,
                             void *stream);
+/* pccnn_bounding_box with the host copy queued, not waited for: host_out is host memory of 2 * batch_size * d floats
+ * and one int32, laid out as [minima | maxima | word].  With page-locked host_out and at most 256 box values the
+ * kernels write host_out themselves (through its device address), the word - a 1 - last and behind a system-scope
+ * fence, and *polled_out is 1: a caller that stored a negative value in the word before the call polls it.  Otherwise
+ * *polled_out is 0, the boxes travel in two copies on `stream` and the caller waits for the stream (or an event). */
+int pccnn_bounding_box_queued(const float *pts, const int32_t *batch_ids, int64_t n, int d, int batch_size,
+                              float *aabb_min_out, float *aabb_max_out, void *host_out, int *polled_out,
+                              void *stream);
 /* Poisson-disk pooling of a 3-D cloud up to the number of selected points: the grid of cell size `cell_size` over
  * the cloud (pccnn_grid_build, into the workspace), then pccnn_poisson_disk_grid, i.e. what
  * pccnn_lib/pc/PointPooling.py:38-65 does between the bounding box and the selected ids.  num_cells_host: the grid

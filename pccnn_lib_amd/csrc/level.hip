@@ -127,6 +127,36 @@ extern "C" int pccnn_bounding_box_host(const float *pts, const int32_t *batch_id
     return PCCNN_OK;
 }
 
+extern "C" int pccnn_bounding_box_queued(const float *pts, const int32_t *batch_ids, int64_t n, int d, int batch_size,
+                                         float *aabb_min_out, float *aabb_max_out, void *host_out, int *polled_out,
+                                         void *stream)
+{
+    PCCNN_REQUIRE(host_out && polled_out, PCCNN_ERR_INVALID, "pccnn_bounding_box_queued: null host pointer");
+    PCCNN_REQUIRE(d >= 2 && d <= PCCNN_MAX_DIMS && batch_size > 0, PCCNN_ERR_INVALID,
+                  "pccnn_bounding_box_queued: d=%d batch_size=%d", d, batch_size);
+    *polled_out = 0;
+    hipStream_t s = (hipStream_t)stream;
+    const size_t bytes = (size_t)batch_size * d * sizeof(float);
+    // page-locked host memory and one workgroup's worth of box values: the kernel that pads the boxes writes them
+    // to host_out itself and a 1 behind them, last; otherwise two copies, and the caller waits for the stream
+    void *host_on_device = nullptr;
+    bool direct = batch_size * d <= 256;
+    if (direct && hipHostGetDevicePointer(&host_on_device, host_out, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        direct = false;
+    }
+    PccnnBoxMask mask;
+    if (direct) mask.tail = (float *)host_on_device;
+    int rc = pccnn_bounding_box_masked(pts, batch_ids, n, d, batch_size, aabb_min_out, aabb_max_out, mask, stream);
+    if (rc != PCCNN_OK) return rc;
+    if (!direct) {
+        PCCNN_HIP_CHECK(hipMemcpyAsync(host_out, aabb_min_out, bytes, hipMemcpyDeviceToHost, s));
+        PCCNN_HIP_CHECK(hipMemcpyAsync((char *)host_out + bytes, aabb_max_out, bytes, hipMemcpyDeviceToHost, s));
+    }
+    *polled_out = direct ? 1 : 0;
+    return PCCNN_OK;
+}
+
 extern "C" size_t pccnn_pool_poisson_workspace_bytes(int64_t n, int64_t num_pillars, int64_t total_cells)
 {
     if (n < 1) n = 1;

@@ -104,26 +104,53 @@ def bounding_box_host(pts, batch_ids, batch_size):
     return mn, mx, (host[0], host[1])
 
 
+# Pinned blocks that kernels write into by themselves (torch's host allocator does not know about those writes):
+# the last few are kept, each with an event recorded behind its kernels, and a block is let go only after its event
+# has passed, so that it cannot be handed out again while a write into it is still on its way.
+_LANDINGS = []
+
+
+def _keep_until_written(landing, done):
+    _LANDINGS.append((landing, done))
+    if len(_LANDINGS) > 8:
+        _, oldest = _LANDINGS.pop(0)
+        oldest.synchronize()
+
+
 def bounding_box_host_later(pts, batch_ids, batch_size):
-    """``bounding_box`` with the host copy on its way: -> (f32[B,D], f32[B,D], fetch), where ``fetch()`` waits for
-    an asynchronous copy into pinned memory that was queued behind the box kernels and returns the two numpy arrays.
-    Whatever the caller does before it calls ``fetch`` runs beside the device's work."""
+    """``bounding_box`` with the host copy on its way: -> (f32[B,D], f32[B,D], fetch), where ``fetch()`` returns the
+    two numpy arrays once they are there.  The box kernels write them into pinned memory themselves, a flag word
+    last, and ``fetch`` polls that word (with many clouds: two copies and an event).  Whatever the caller does
+    before it calls ``fetch`` runs beside the device's work."""
+    import numpy as np
     _chk(pts, "bounding_box: pts", torch.float32, 2)
     _chk(batch_ids, "bounding_box: batch_ids", torch.int32, 1, pts.device)
     d = _dims(pts, "bounding_box")
     batch_size = int(batch_size)
+    count = batch_size * d
     box = torch.empty((2, batch_size, d), dtype=torch.float32, device=pts.device)
     base = box.data_ptr()
-    _lib.call("pccnn_bounding_box", _ptr(pts), _ptr(batch_ids), pts.shape[0], d, batch_size, _P(base),
-              _P(base + 4 * batch_size * d), _stream())
-    pinned = torch.empty((2, batch_size, d), dtype=torch.float32, pin_memory=True)
-    pinned.copy_(box, non_blocking=True)
+    landing = torch.empty((2 * count + 1,), dtype=torch.float32, pin_memory=True)
+    words = landing.numpy().view(np.int32)
+    words[2 * count] = -1
+    polled = ctypes.c_int(0)
+    _lib.call("pccnn_bounding_box_queued", _ptr(pts), _ptr(batch_ids), pts.shape[0], d, batch_size, _P(base),
+              _P(base + 4 * count), _P(landing.data_ptr()), ctypes.byref(polled), _stream())
     done = torch.cuda.Event()
     done.record()
+    _keep_until_written(landing, done)
 
     def fetch():
-        done.synchronize()
-        host = pinned.numpy()
+        if polled.value:
+            spins = 0
+            while words[2 * count] < 0:
+                spins += 1
+                if spins > 100000:
+                    done.synchronize()
+                    break
+        else:
+            done.synchronize()
+        host = landing.numpy()[:2 * count].reshape(2, batch_size, d)
         return host[0], host[1]
     return box[0], box[1], fetch
 
@@ -692,6 +719,7 @@ def pool_poisson_later(pts, batch_ids, aabb_min, cell_size, num_cells_host, batc
               _P(landing.data_ptr()), _ptr(ws), ws.numel(), _stream())
     done = torch.cuda.Event()
     done.record()
+    _keep_until_written(landing, done)
 
     def finish():
         # the count is the last word to arrive: a short poll of the pinned word, then the event if it takes long
