@@ -219,8 +219,8 @@ int pccnn_poisson_disk_grid(const float *pts_sorted, const int64_t *sorted_keys,
 
 /* ---- host sequences with one read-back -----------------------------------
  * Chains of the entry points above for the steps whose output size depends on the data; each ends with one small
- * device-to-host copy on `stream` and returns after it (the calls are synchronous).  The launches are those of the
- * entry points named.
+ * read-back and returns after it (the calls without "queued" in their name are synchronous).  The launches are those
+ * of the entry points named.
  *
  * pccnn_bounding_box, and the box on the host as well (host_min_out / host_max_out: host memory, f32[batch_size,d]):
  * what pccnn_lib/pc/Grid.py:26-28 reads when it sizes a grid. */

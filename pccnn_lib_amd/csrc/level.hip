@@ -5,7 +5,9 @@
 // here computes: the kernels are those of the entry points that are called.
 //
 // The read-backs go through a small pinned host buffer (one per host thread, allocated on first use and kept):
-// an asynchronous copy into it on the caller's stream, then a wait for that stream.
+// an asynchronous copy into it on the caller's stream, then a wait for that stream - or, where the last kernel of
+// the chain can write the result itself (the pair total, the pooled boxes and their count, a cloud's box), a store
+// into page-locked host memory through its device address and a host that polls the word written last.
 #include "common.h"
 #include <string.h>
 #include <chrono>
