@@ -222,6 +222,14 @@ def config5_leg(lib, dev, steps, warmup):
     params = [p for layer in layers for p in layer.parameters()]
     ones = {}
 
+    def drained():
+        # the device has finished what was queued (a spin on an event query: torch.cuda.synchronize() returns some
+        # tens of microseconds late, which would be charged to every level of the split run)
+        mark = torch.cuda.Event()
+        mark.record()
+        while not mark.query():
+            pass
+
     def whole(split=False):
         for p in params:
             p.grad = None
@@ -230,7 +238,7 @@ def config5_leg(lib, dev, steps, warmup):
         del sizes[:], marks[:]
         for level, radius in enumerate(radii_levels):
             if split:
-                torch.cuda.synchronize()
+                drained()
                 marks.append(time.perf_counter())
             # (the density is queued between the pooling and the first use of its result: the device computes it
             # while the host waits for the size of the selection)
@@ -245,14 +253,14 @@ def config5_leg(lib, dev, steps, warmup):
             sizes.append((int(pc.pts_.shape[0]), int(out_pc.pts_.shape[0]), int(kept.shape[0])))
             pc = out_pc
         if split:
-            torch.cuda.synchronize()
+            drained()
             marks.append(time.perf_counter())
         shape = tuple(feats.shape)
         if shape not in ones:
             ones[shape] = torch.ones(shape, dtype=feats.dtype, device=dev)
         feats.backward(ones[shape])
         if split:
-            torch.cuda.synchronize()
+            drained()
             marks.append(time.perf_counter())
         return feats
 
