@@ -175,6 +175,17 @@ def test_poisson_disk_matches_oracle(ops, oracle, models):
         assert np.array_equal(sel.cpu().numpy(), e_sel)
 
 
+@pytest.mark.parametrize("case", ["3d", "2d", "4d"])
+def test_poisson_disk_hand_worked_known_answers(ops, case):
+    # the same hand-derived selections that pin the oracle (tests/golden/poisson_known_answers.py), asked of the
+    # HIP path directly: colour order, bit <-> dimension, sorted order inside a cell
+    from tests.golden import poisson_known_answers as kat
+    (keys, neigh, ends, ncells), expect = kat.CASES[case]()
+    sel = ops.poisson_disk_sampling(t(keys), t(neigh), t(ends), t(ncells))
+    assert sel.dtype == torch.int64 and tuple(sel.shape) == (expect.shape[0], 1)
+    assert sel.cpu().numpy().reshape(-1).tolist() == expect.tolist()
+
+
 @pytest.mark.parametrize("batch,num_pts,radius,use_table", [(4, 1000, 0.1, True), (3, 4000, 0.05, False),
                                                             (1, 3000, 0.45, True), (2, 2500, 0.3, False),
                                                             (1, 40, 5.0, True)])

@@ -183,3 +183,16 @@ def test_poisson_disk(oracle, models, num_pts, radius):
         if not chosen[s]:
             lo = ends[s - 1] if s > 0 else 0
             assert chosen[neigh[lo:ends[s], 0]].any()
+
+
+@pytest.mark.parametrize("case", ["3d", "2d", "4d"])
+def test_poisson_disk_hand_worked_known_answers(oracle, case):
+    # Expected ids are derived by hand from poisson_disk_sampling.cu:66-72,:82-104,:158-170 in
+    # tests/golden/poisson_known_answers.py: launch (colour) order, which bit belongs to which dimension,
+    # sorted order inside a cell.  A reversed colour order, the reversed bit order, both at once, or a plain
+    # walk in sorted order each give another selection on these inputs.
+    from tests.golden import poisson_known_answers as kat
+    (keys, neigh, ends, ncells), expect = kat.CASES[case]()
+    got = oracle.poisson_disk_sampling(keys, neigh, ends, ncells)
+    assert got.shape == (expect.shape[0], 1)
+    assert got.reshape(-1).tolist() == expect.tolist()
