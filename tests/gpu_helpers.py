@@ -45,3 +45,11 @@ def gpu_neighborhood(ops, pts, ids, samples, sample_ids, radius, batch_size, max
 def relerr(a, b):
     a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
     return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
+
+
+def mixed_close(a, b, rtol=1e-3, atol_frac=1e-5):
+    """Element-wise check beside the norm-wise relerr(): every entry within rtol of its own magnitude plus
+    atol_frac of the tensor's largest magnitude (the floor that fp32 sums of terms of that size leave), so an entry a
+    hundred times smaller than the largest one must still be right to about a percent of itself, not merely small."""
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return bool(np.all(np.abs(a - b) <= rtol * np.abs(b) + atol_frac * max(np.abs(b).max(), 1e-30)))

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from pccnn_lib_amd import synthetic
-from tests.gpu_helpers import DEV, gpu_neighborhood, relerr, t
+from tests.gpu_helpers import DEV, gpu_neighborhood, mixed_close, relerr, t
 
 pytestmark = pytest.mark.gpu
 
@@ -175,6 +175,7 @@ def test_kpconv_forward_and_grads(ops, oracle, k, c_in, c_out, distinct):
     for got, e, name in zip(grads, exp_g, ("dW", "dFeat", "dKernelPts", "dPts", "dSamples")):
         assert tuple(got.shape) == e.shape, name
         assert relerr(got.cpu().numpy(), e) < GRAD_TOL, name
+        assert mixed_close(got.cpu().numpy(), e), name
 
 
 @pytest.mark.parametrize("hidden,mlps,c_in,c_out,distinct", [(16, 1, 64, 128, False), (8, 2, 32, 24, True),
@@ -199,6 +200,7 @@ def test_mcconv_forward_and_grads(ops, oracle, hidden, mlps, c_in, c_out, distin
     for got, e, name in zip(grads, exp_g, ("dW", "dFeat", "dAxis", "dBias", "dPdf", "dPts", "dSamples")):
         assert tuple(got.shape) == e.shape, name
         assert relerr(got.cpu().numpy(), e) < GRAD_TOL, name
+        assert mixed_close(got.cpu().numpy(), e), name
 
 
 def test_config1_plumbing_kpconv_layer(oracle):
@@ -249,6 +251,49 @@ def test_mcconv_layer_autograd_routing(oracle):
     assert relerr(p(tf.grad), exp_g[1]) < GRAD_TOL
     assert relerr(p(layer.proj_axis_.grad), exp_g[2]) < GRAD_TOL
     assert relerr(p(layer.proj_bias_.grad), exp_g[3]) < GRAD_TOL
+
+
+def test_point_gradient_through_density_and_mcconv_equals_the_composed_oracle(oracle):
+    # unit_test/test_mcconv_pt_grads.py:92-103: points -> Pointcloud.compute_pdf -> pdf * prod(radius) -> MCConv with
+    # the same tensor as points and samples; pts.grad = dPts + dSamples + compute_pdf_grads(dPdf * prod(radius)).
+    # The three terms come from two different ops and are added by autograd; here the sum is compared with the
+    # oracle's mcconv_grads and compute_pdf_grads composed by hand (3-D, full kernels).
+    import pccnn_lib_amd as lib
+    from pccnn_lib_amd.op_wrappers import ComputeMCConv
+    pts, ids = synthetic.primitives(17, 2, 1200)
+    rng = np.random.default_rng(17)
+    c_in, c_out, hidden, radius = 16, 24, 8, 0.1
+    bw = np.full(3, 0.025, np.float32)
+    feats = rng.normal(size=(pts.shape[0], c_in)).astype(np.float32)
+    axis = rng.normal(0, np.sqrt(1 / 3), (3, hidden)).astype(np.float32)
+    bias = rng.normal(0, 0.1, (1, hidden)).astype(np.float32)
+    w = rng.normal(0, np.sqrt(1.0 / (c_in * hidden)), (1, hidden * c_in, c_out)).astype(np.float32)
+    g = rng.normal(size=(pts.shape[0], c_out)).astype(np.float32)
+    radii = np.full(3, radius, np.float32)
+
+    pc = lib.pc.Pointcloud(pts, ids, device=DEV, requires_grad=True)
+    pc.compute_pdf(bw)
+    assert pc.pts_unnorm_pdf_.requires_grad
+    nbh = lib.pc.layers.conv_base.build_neighborhood(pc, pc, t(radii), 0)
+    cur_pdf = pc.pts_unnorm_pdf_ * torch.prod(t(radii))
+    out = ComputeMCConv.apply(pc.pts_, cur_pdf, t(feats), pc.pts_, nbh.neighbors_, nbh.start_ids_, t(radii), t(axis),
+                              t(bias), t(w))
+    (out * t(g)).sum().backward()
+    got = pc.pts_.grad.cpu().numpy()
+
+    unnorm, _, nb_pdf = oracle.pointcloud_pdf(pts, ids, bw)
+    nb = oracle.neighborhood(pts, ids, pts, ids, radius)
+    pdf = (unnorm * np.prod(radii)).astype(np.float32)
+    assert relerr(cur_pdf.detach().cpu().numpy(), pdf) < FWD_TOL
+    eg = oracle.mcconv_grads(pts, pdf, feats, pts, nb["neighbors"], nb["ends"], radii, axis, bias, w, g)
+    through_pdf = oracle.compute_pdf_grads(3, bw, pts, nb_pdf["neighbors"], nb_pdf["ends"],
+                                           (eg[4] * np.prod(radii)).astype(np.float32))
+    direct = eg[5] + eg[6]
+    exp = direct + through_pdf
+    # both routes carry weight: neither term alone satisfies the tolerance
+    assert relerr(direct, exp) > 100 * GRAD_TOL and relerr(through_pdf, exp) > 100 * GRAD_TOL
+    assert relerr(got, exp) < GRAD_TOL
+    assert mixed_close(got, exp)
 
 
 def test_hierarchy_level_with_pooling(oracle):
