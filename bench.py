@@ -172,6 +172,20 @@ def config3_leg(lib, dev, timed, steps, warmup, with_cpu):
                         "traffic": traffic("config3", "contraction_f32"), "flops_per_launch": flops,
                         "avg_launch_ms": g_avg, "launches": g_n,
                         "shapes": "P[65536,1920] W[1920,256]; P^T dOut; dOut W^T (mean of the three launches)"}}
+    # the two projection kernels of this step against HBM (bytes as for config 2: pairs, offsets, coordinates and
+    # features in, the projection out; backward: the projection gradient in, feature gradient, basis gradient and
+    # per-pair point gradients out)
+    geo = 8.0 * pairs + 4.0 * m + 12.0 * 2 * m + 4.0 * m * c_in
+    proj = 4.0 * m * c_in * k
+    for key, name, alg in (("proj_fwd", "conv_proj_fwd_kernel", geo + proj),
+                           ("proj_bwd", "conv_proj_bwd_kernel", geo + proj + 4.0 * m * c_in + 4.0 * pairs * k + 16.0 * pairs)):
+        k_n, k_ms = kernels.get(key, (0, 0.0))
+        avg = k_ms / max(k_n, 1)
+        gbps = alg / (avg * 1e-3) / 1e9 if k_n else 0.0
+        leg["roofline_projection_" + ("forward" if key == "proj_fwd" else "backward")] = {
+            "kernel": name, "bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": gbps / HBM_PEAK_GBPS, "traffic": traffic("config3", name), "bytes_per_launch": alg,
+            "avg_launch_ms": avg, "launches": k_n}
     log("config 3: %d pairs, step %.3f ms" % (pairs, ms),
         {kk: "%d x %.1f us" % (v[0], 1e3 * v[1] / v[0]) for kk, v in kernels.items()})
     if with_cpu:
@@ -266,12 +280,17 @@ def config5_leg(lib, dev, steps, warmup):
 
     for _ in range(warmup):
         whole()
+    stream = torch.cuda.current_stream()
+    passes = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
+    for i in range(steps):
+        passes[i].record(stream)
         whole()
+    passes[steps].record(stream)
     torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) / steps * 1e3
+    mean_ms = (time.perf_counter() - t0) / steps * 1e3
+    ms = float(np.median([passes[i].elapsed_time(passes[i + 1]) for i in range(steps)]))
     split_ms = np.zeros(5)
     for _ in range(steps):
         whole(split=True)
@@ -281,9 +300,9 @@ def config5_leg(lib, dev, steps, warmup):
                "pairs": sizes[i][2], "forward_ms": float(split_ms[i])} for i in range(4)]
     leg = {"workload": "config 5: 8 x 100000 room points, four Poisson-disk levels (0.025/0.05/0.1/0.2), neighbor "
                        "search + density + MCConv 8->32->64->128->256 with bf16 contraction operands, forward + backward",
-           "points": int(pts.shape[0]), "ms_per_pass": ms, "points_per_sec": pts.shape[0] / (ms * 1e-3),
+           "points": int(pts.shape[0]), "ms_per_pass": ms, "ms_per_pass_mean_wall": mean_ms, "points_per_sec": pts.shape[0] / (ms * 1e-3),
            "dtype": "bf16 operands, f32 accumulate", "levels": levels, "backward_ms": float(split_ms[4]),
-           "note": "ms_per_pass is synchronised at the end only; the per-level times come from a second run with a "
+           "note": "ms_per_pass is the median over the passes (HIP events around each), synchronised at the end only; the per-level times come from a second run with a "
                    "host synchronisation between the levels, so they add up to more"}
     log("config 5: pass %.3f ms" % ms, [(l["points_in"], l["points_out"], l["pairs"], round(l["forward_ms"], 3))
                                         for l in levels], "backward %.3f ms" % split_ms[4])
@@ -324,24 +343,48 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    def timed(fn, steps, warmup):
-        """(ms per step, per-kernel timings).  The step time comes from a pass without the library's event
-        hooks (they serialise the stream around every hooked launch); a second pass of the same steps with
-        the hooks on gives the per-kernel durations."""
+    def timed(fn, steps, warmup, stats=None):
+        """(ms per step, per-kernel timings).  After the warm-up exactly `steps` steps run between two device
+        synchronisations, each bracketed by HIP events on the launch stream; the step time reported is the MEDIAN of
+        those per-step durations, and `stats` (a dict, optional) also receives the wall-clock mean over the same
+        steps, the fastest and the slowest step.  That pass runs without the library's event hooks (they serialise
+        the stream around every hooked launch); a second pass of the same steps with the hooks on gives the
+        per-kernel durations."""
         for _ in range(warmup):
             fn()
+        stream = torch.cuda.current_stream()
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(steps):
+        for i in range(steps):
+            marks[i].record(stream)
             fn()
+        marks[steps].record(stream)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
+        per_step = np.array([marks[i].elapsed_time(marks[i + 1]) for i in range(steps)])
+        if stats is not None:
+            stats.update(median_ms=float(np.median(per_step)), mean_wall_ms=dt / steps * 1e3,
+                         min_ms=float(per_step.min()), max_ms=float(per_step.max()), steps=steps)
         _lib.timing(enable=True, reset=True)
         for _ in range(steps):
             fn()
         torch.cuda.synchronize()
         kernels = _lib.timing(enable=False)
-        return dt / steps * 1e3, kernels
+        if stats is not None and stats.get("sustained"):
+            # the same step once the device has been under this load for a while: after an idle spell the part's clock
+            # management takes 30 - 40 ms of continuous work to settle (the first steps run up to 20 % slower), which
+            # a short warm-up does not cover; 60 more untimed steps, then the median of 100
+            for _ in range(60):
+                fn()
+            marks = [torch.cuda.Event(enable_timing=True) for _ in range(101)]
+            for i in range(100):
+                marks[i].record(stream)
+                fn()
+            marks[100].record(stream)
+            torch.cuda.synchronize()
+            stats["sustained_ms"] = float(np.median([marks[i].elapsed_time(marks[i + 1]) for i in range(100)]))
+        return float(np.median(per_step)), kernels
 
     # what a plain float4 copy reaches on this part, as the practical ceiling beside the published 8 TB/s: 1 GiB read
     # and 1 GiB written per launch (beyond every cache), timed with events on the launch stream.  The same launches
@@ -431,14 +474,16 @@ def main():
         p.compute_pdf(bw)
         return p
 
-    conv_ms, conv_kernels = timed(conv_step, args.steps, args.warmup)
-    fw_ms, _ = timed(conv_step_fw_only, args.steps, args.warmup)
+    conv_stats, fw_stats = {"sustained": True}, {"sustained": True}
+    conv_ms, conv_kernels = timed(conv_step, args.steps, args.warmup, conv_stats)
+    fw_ms, _ = timed(conv_step_fw_only, args.steps, args.warmup, fw_stats)
     bf_ms, bf_kernels = timed(conv_step_bf16, args.steps, args.warmup)
     nb_ms, nb_kernels = timed(neighbor_step, args.steps, args.warmup)
     pdf_ms, pdf_kernels = timed(pdf_step, args.steps, args.warmup)
     mirror_ms, _ = timed(mirror_step, args.steps, args.warmup)
-    log("conv fwd+bwd %.3f ms (features+weights grads only: %.3f ms) | neighborhood %.3f ms | density %.3f ms"
-        % (conv_ms, fw_ms, nb_ms, pdf_ms))
+    log("conv fwd+bwd %.3f ms median, %.3f ms wall-clock mean (features+weights grads only: %.3f ms) | neighborhood "
+        "%.3f ms | density %.3f ms | sustained %.3f / %.3f ms" % (conv_ms, conv_stats["mean_wall_ms"], fw_ms, nb_ms, pdf_ms,
+                                                                  conv_stats["sustained_ms"], fw_stats["sustained_ms"]))
     log("conv fwd+bwd with bf16 contraction operands: %.3f ms" % bf_ms)
     for name, ks in (("conv", conv_kernels), ("conv bf16", bf_kernels), ("neighbors", nb_kernels),
                      ("pdf", pdf_kernels)):
@@ -497,7 +542,7 @@ def main():
 
     # ---- scene-scale neighbor search (config 4: one room of 10^6 points, cell = radius = 0.05 m): the
     # neighbor kernels only show their throughput at this size, so their roofline entry is taken here
-    scene = roofline_sort = roofline_pdf = roofline_pdf_grid = None
+    scene = roofline_sort = roofline_pdf = roofline_pdf_grid = roofline_nb_count = roofline_nb_search = None
     if not args.no_scene:
         from pccnn_lib_amd import synthetic
         spts = t(synthetic.room(4, args.scene_points))
@@ -525,6 +570,24 @@ def main():
                        "frac": s_gbps / HBM_PEAK_GBPS,
                        "traffic": traffic("scene_%d" % n_s, "neighbors_fill"), "bytes_per_launch": s_bytes,
                        "avg_launch_ms": f_avg, "launches": f_n}
+        # the count pass of the same search: the fill's inputs (24M + 20N + pillar table), per-sample counts 4M out
+        c_n, c_ms = s_kernels.get("nb_count", (0, 0.0))
+        c_avg = c_ms / max(c_n, 1)
+        c_bytes = 24.0 * n_s + 20.0 * n_s + s_grid + 4.0 * n_s
+        c_gbps = c_bytes / (c_avg * 1e-3) / 1e9 if c_n else 0.0
+        roofline_nb_count = {"kernel": "neighbors_kernel<count>", "workload": roofline_nb["workload"], "bound": "hbm",
+                             "achieved": c_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": c_gbps / HBM_PEAK_GBPS,
+                             "traffic": traffic("scene_%d" % n_s, "neighbors_count"), "bytes_per_launch": c_bytes,
+                             "avg_launch_ms": c_avg, "launches": c_n}
+        # the whole search as a caller sees it (box, keys, sort, pillar table, count, scan, fill, the two read-backs
+        # of sizes): the algorithmic bytes of its stages (keys 24N, sort 44N, table 8N + 8 B nc0 nc1, search
+        # 8T + 24M + 20N + 8 B nc0 nc1) over the time of one neighborhood build
+        e2e_bytes = 24.0 * n_s + 44.0 * n_s + 8.0 * n_s + s_grid + s_bytes
+        e2e_gbps = e2e_bytes / (s_ms * 1e-3) / 1e9
+        roofline_nb_search = {"kernel": "neighborhood build end to end (box, keys, sort, table, count, scan, fill)",
+                              "workload": roofline_nb["workload"], "bound": "hbm", "achieved": e2e_gbps,
+                              "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": e2e_gbps / HBM_PEAK_GBPS, "traffic": None,
+                              "bytes_per_launch": e2e_bytes, "avg_launch_ms": s_ms, "launches": max(args.steps // 2, 3)}
         # the density of the same scene (Pointcloud.compute_pdf, bandwidth 0.2 x radius: its own grid of cell size
         # 4 x bandwidth, then the KDE walk on it)
         sbw = np.full(3, 0.2 * 0.05, np.float32)
@@ -604,7 +667,16 @@ def main():
                    "points": m, "pairs": total_pairs, "seed": 2,
                    "gradients": "all inputs (features, weights, axis, bias, density, positions); the step with the "
                                 "feature and weight gradients only is ms_per_step_feature_and_weight_grads_only"},
+        "timing": "ms_per_step is the median of the per-step durations of the timed steps (HIP events on the launch "
+                  "stream around every step); ms_per_step_mean_wall is the wall-clock mean over the same steps",
+        "ms_per_step_mean_wall": conv_stats["mean_wall_ms"], "ms_per_step_min": conv_stats["min_ms"],
+        "ms_per_step_max": conv_stats["max_ms"],
+        # (not `value`: the same step after 60 more untimed steps, median of 100 - what a training loop sees once the
+        # part's clock management has settled under the load)
+        "ms_per_step_sustained": conv_stats["sustained_ms"],
         "ms_per_step_feature_and_weight_grads_only": fw_ms,
+        "ms_per_step_feature_and_weight_grads_only_mean_wall": fw_stats["mean_wall_ms"],
+        "ms_per_step_feature_and_weight_grads_only_sustained": fw_stats["sustained_ms"],
         # the symmetric-pair index that the step's point / density gradients use is built once per neighborhood
         # (outside ms_per_step); a step on a fresh neighborhood pays it once more
         "mirror_ms": mirror_ms, "ms_per_step_with_mirror": conv_ms + mirror_ms,
@@ -613,6 +685,7 @@ def main():
         "kernels_us": {leg: {k: round(1e3 * v[1] / v[0], 2) for k, v in ks.items()}
                        for leg, ks in (("conv", conv_kernels), ("neighborhood", nb_kernels), ("density", pdf_kernels))},
         "bf16_contraction": bf16_leg, "scene": scene, "roofline": roofline, "roofline_neighbors": roofline_nb,
+        "roofline_neighbors_count": roofline_nb_count, "roofline_neighbor_search": roofline_nb_search,
         "roofline_projection_forward": rooflines_proj["proj_fwd"],
         "roofline_projection_backward": rooflines_proj["proj_bwd"], "roofline_sort": roofline_sort,
         "roofline_pdf": roofline_pdf, "roofline_pdf_grid": roofline_pdf_grid, "config3": config3, "config5": config5,
