@@ -8,9 +8,16 @@
  *  - Every pointer is a DEVICE pointer unless its name starts with `h_`.
  *  - Tensors are dense, row-major, of exactly the stated element type.
  *  - `stream` is a hipStream_t passed as void* (NULL = the null stream).  All
- *    work is enqueued on it; no entry point synchronises or allocates device
- *    memory.  Temporary storage comes in through `workspace` arguments whose
- *    minimum size the matching *_workspace_bytes function reports.
+ *    work is enqueued on it.  The operator entry points neither synchronise
+ *    nor allocate: temporary storage comes in through `workspace` arguments
+ *    whose minimum size the matching *_workspace_bytes function reports.
+ *    Three groups are the exception, and each says so where it is declared:
+ *    the "host sequences" (they end with a read-back: the synchronous ones
+ *    wait for `stream` with hipStreamSynchronize, and every one keeps a small
+ *    page-locked staging block per host thread, allocated with hipHostMalloc
+ *    on first use and kept until the process ends); pccnn_sort_keys_static
+ *    (its storage is a static device array); and the optional timing hooks
+ *    (pccnn_timing_*: they create events while switched on).
  *  - Return value: 0 on success, a negative PCCNN_ERR_* code otherwise;
  *    pccnn_last_error() then returns a thread-local description.  Arguments
  *    are validated on the host before any kernel is launched.
@@ -262,13 +269,15 @@ int pccnn_pool_poisson_select(const float *pts, const int32_t *batch_ids, int64_
  * others until then.  The count is the last word to arrive (with page-locked host_out and up to 85 clouds the
  * kernels write host_out themselves, through its device address, the count behind a system-scope fence; otherwise
  * it travels in a copy of its own behind the boxes), so a caller that stored a negative value there before the call
- * may poll that word instead of waiting for an event.  No counterpart in the reference, whose PointPooling waits
- * where it reads the sizes. */
+ * may poll that word instead of waiting for an event.  *polled_out (host int, may be NULL) says which way the
+ * results travel: 1 = written by the kernels, poll the count; 0 = copies, wait for the stream or an event.  No
+ * counterpart in the reference, whose PointPooling waits where it reads the sizes. */
 int pccnn_pool_poisson_select_queued(const float *pts, const int32_t *batch_ids, int64_t n, int batch_size,
                                      const float *aabb_min, const float *cell_size, const int32_t *num_cells_host,
                                      int key_bits, int with_cell_table, int32_t *perm_out, int32_t *selected_out,
                                      int32_t *selected_scan_out, float *pooled_min_out, float *pooled_max_out,
-                                     void *host_out, void *workspace, size_t workspace_bytes, void *stream);
+                                     void *host_out, int *polled_out, void *workspace, size_t workspace_bytes,
+                                     void *stream);
 int pccnn_compact_selected_remap(const int32_t *selected, const int32_t *selected_scan, const int32_t *remap,
                                  int64_t n, int64_t *ids_out, void *stream);
 /* pccnn_compact_selected_remap with remap = perm, plus the rows a pooled cloud is made of: pooled_pts_out f32[S,d] =

@@ -56,7 +56,7 @@ SIGNATURES = {
     "pccnn_pool_poisson_workspace_bytes": (SZ, [I64, I64, I64]),
     "pccnn_pool_poisson_select": (I32, [P, P, I64, I32, P, P, P, I32, I32, P, P, P, P, P, P, P, P, P, SZ, P]),
     "pccnn_bounding_box_queued": (I32, [P, P, I64, I32, I32, P, P, P, P, P]),
-    "pccnn_pool_poisson_select_queued": (I32, [P, P, I64, I32, P, P, P, I32, I32, P, P, P, P, P, P, P, SZ, P]),
+    "pccnn_pool_poisson_select_queued": (I32, [P, P, I64, I32, P, P, P, I32, I32, P, P, P, P, P, P, P, P, SZ, P]),
     "pccnn_compact_selected_remap": (I32, [P, P, P, I64, P, P]),
     "pccnn_compact_pooled": (I32, [P, P, P, P, P, I64, I32, P, P, P, P]),
     "pccnn_grid_build_sized": (I32, [P, P, P, P, P, I64, I32, I32, I32, I32, P, P, P, P, P, P, P, P, SZ, P]),

@@ -25,17 +25,25 @@ def sources():
     return sorted(glob.glob(os.path.join(CSRC, "*.hip")))
 
 
-def build(verbose=True, jobs=8):
+def _up_to_date(obj, src):
+    """True if the object file is newer than its source and every header beside it."""
+    if not os.path.exists(obj):
+        return False
+    deps = [src] + glob.glob(os.path.join(CSRC, "*.h")) + glob.glob(os.path.join(HERE, "..", "include", "*.h"))
+    return os.path.getmtime(obj) > max(os.path.getmtime(d) for d in deps)
+
+
+def build(verbose=True, jobs=8, incremental=False):
+    """Compiles every source (``incremental``: only those changed since their object file was written) and links."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     obj_dir = os.path.join(HERE, "build")
     os.makedirs(obj_dir, exist_ok=True)
-    procs, objs = [], []
-    srcs = sources()
+    objs = [os.path.join(obj_dir, os.path.basename(src) + ".o") for src in sources()]
+    srcs = [src for src, obj in zip(sources(), objs) if not (incremental and _up_to_date(obj, src))]
     for i in range(0, len(srcs), jobs):
         batch = []
         for src in srcs[i:i + jobs]:
             obj = os.path.join(obj_dir, os.path.basename(src) + ".o")
-            objs.append(obj)
             cmd = [hipcc] + HIPCC_FLAGS + ["-c", src, "-o", obj]
             if verbose:
                 print(" ".join(cmd), flush=True)
@@ -55,6 +63,6 @@ def build(verbose=True, jobs=8):
 
 
 if __name__ == "__main__":
-    build()
+    build(incremental="--incremental" in sys.argv)
     print("built", LIB_PATH)
     sys.exit(0)

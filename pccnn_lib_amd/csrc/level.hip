@@ -176,9 +176,10 @@ static int pool_select_queue(const float *pts, const int32_t *batch_ids, int64_t
                              const float *aabb_min, const float *cell_size, const int32_t *num_cells_host,
                              int key_bits, int with_cell_table, int32_t *perm_out, int32_t *selected_out,
                              int32_t *selected_scan_out, float *pooled_min_out, float *pooled_max_out, bool with_box,
-                             void *host_dst, void *workspace, size_t workspace_bytes, hipStream_t s)
+                             void *host_dst, int *polled_out, void *workspace, size_t workspace_bytes, hipStream_t s)
 {
     const char *who = "pccnn_pool_poisson_select";
+    if (polled_out) *polled_out = 0;
     PCCNN_REQUIRE(pts && batch_ids && aabb_min && cell_size && perm_out && selected_out && selected_scan_out,
                   PCCNN_ERR_INVALID, "%s: null pointer", who);
     for (int k = 0; k < 3; ++k)
@@ -229,8 +230,16 @@ static int pool_select_queue(const float *pts, const int32_t *batch_ids, int64_t
     }
     rc = pccnn_bounding_box_masked(l.sorted_pts, batch_ids, n, 3, batch_size, pooled_min_out, pooled_max_out, mask,
                                    stream);
-    if (rc != PCCNN_OK) return rc;
-    if (direct) return PCCNN_OK;
+    if (rc != PCCNN_OK) {
+        // a launch that writes into the caller's host block may already be queued: let it land before the caller
+        // hears of the error and reuses the block
+        if (direct) (void)hipStreamSynchronize(s);
+        return rc;
+    }
+    if (direct) {
+        if (polled_out) *polled_out = 1;
+        return PCCNN_OK;
+    }
     if (staged) {
         PCCNN_HIP_CHECK(hipMemcpyAsync(host_dst, mask.tail, 2 * box, hipMemcpyDeviceToHost, s));
     } else {
@@ -265,7 +274,7 @@ extern "C" int pccnn_pool_poisson_select(const float *pts, const int32_t *batch_
     if ((rc = pinned_slot(2 * box + sizeof(int32_t), &slot)) != PCCNN_OK) return rc;
     rc = pool_select_queue(pts, batch_ids, n, batch_size, aabb_min, cell_size, num_cells_host, key_bits,
                            with_cell_table, perm_out, selected_out, selected_scan_out, pooled_min_out, pooled_max_out,
-                           with_box, slot, workspace, workspace_bytes, s);
+                           with_box, slot, nullptr, workspace, workspace_bytes, s);
     if (rc != PCCNN_OK) return rc;
     PCCNN_HIP_CHECK(hipStreamSynchronize(s));           // count and box: one wait
     int32_t count;
@@ -283,7 +292,8 @@ extern "C" int pccnn_pool_poisson_select_queued(const float *pts, const int32_t 
                                                 const int32_t *num_cells_host, int key_bits, int with_cell_table,
                                                 int32_t *perm_out, int32_t *selected_out, int32_t *selected_scan_out,
                                                 float *pooled_min_out, float *pooled_max_out, void *host_out,
-                                                void *workspace, size_t workspace_bytes, void *stream)
+                                                int *polled_out, void *workspace, size_t workspace_bytes,
+                                                void *stream)
 {
     PCCNN_REQUIRE(n > 0 && n < (1ll << 31) && batch_size > 0, PCCNN_ERR_INVALID,
                   "pccnn_pool_poisson_select_queued: n=%lld batch_size=%d", (long long)n, batch_size);
@@ -291,7 +301,7 @@ extern "C" int pccnn_pool_poisson_select_queued(const float *pts, const int32_t 
                   "pccnn_pool_poisson_select_queued: null pointer");
     return pool_select_queue(pts, batch_ids, n, batch_size, aabb_min, cell_size, num_cells_host, key_bits,
                              with_cell_table, perm_out, selected_out, selected_scan_out, pooled_min_out, pooled_max_out,
-                             true, host_out, workspace, workspace_bytes, (hipStream_t)stream);
+                             true, host_out, polled_out, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 extern "C" int pccnn_compact_selected_remap(const int32_t *selected, const int32_t *selected_scan,
@@ -452,7 +462,12 @@ extern "C" int pccnn_neighborhood_count(const float *pts, const int32_t *batch_i
                                     num_pillars, with_cell_table ? cell_table_out : nullptr, total_cells, num_cells_out,
                                     cell_size, 3, max_neighbors, ends_out, workspace, workspace_bytes, stream);
     pccnn_redirect_pair_total(nullptr);
-    if (rc != PCCNN_OK) return rc;
+    if (rc != PCCNN_OK) {
+        // a launch that writes the total into this thread's pinned word may already be queued: let it land before
+        // the next call arms the word again
+        (void)hipStreamSynchronize((hipStream_t)stream);
+        return rc;
+    }
     const auto start = std::chrono::steady_clock::now();
     unsigned spins = 0;
     while (*word == pending) {

@@ -251,10 +251,12 @@ scan_tiles_kernel(const int32_t *__restrict__ in, int32_t *__restrict__ out, int
     int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
     int v[SCAN_ITEMS];
     int sum = 0;
+    long long wide = 0;                 // the tile's sum in 64 bits, from the same loads (in may alias out)
 #pragma unroll
     for (int i = 0; i < SCAN_ITEMS; ++i) {
         int x = (base + i < n) ? in[base + i] : 0;
         if (clamp_max > 0 && x > clamp_max) x = clamp_max;
+        wide += x;
         sum += x;
         v[i] = sum;
     }
@@ -266,13 +268,6 @@ scan_tiles_kernel(const int32_t *__restrict__ in, int32_t *__restrict__ out, int
         if (base + i < n) out[base + i] = v[i] + excl;
     if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
     if (tile_sums64) {
-        long long wide = 0;
-#pragma unroll
-        for (int i = 0; i < SCAN_ITEMS; ++i) {
-            int x = (base + i < n) ? in[base + i] : 0;
-            if (clamp_max > 0 && x > clamp_max) x = clamp_max;
-            wide += x;
-        }
         wide = block_sum_i64(wide, lds64);
         if (threadIdx.x == 0) tile_sums64[blockIdx.x] = wide;
     }

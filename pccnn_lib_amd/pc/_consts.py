@@ -11,7 +11,7 @@ import numpy as np
 import torch
 
 _table = {}
-_host_values = {}        # id(tensor of the table) -> the host values it was made from
+_host_values = {}        # id(tensor of the table) -> (the tensor, the host values it was made from)
 _MAX_ENTRIES = 256
 
 
@@ -34,15 +34,19 @@ def device_vector(value, num_dims, device):
             _host_values.clear()
         out = torch.tensor(flat, dtype=torch.float32, device=device)
         _table[key] = out
-        _host_values[id(out)] = np.asarray(flat, dtype=np.float32)
+        _host_values[id(out)] = (out, np.asarray(flat, dtype=np.float32))
     return out
 
 
 def host_vector(tensor):
     """The host values (float32 numpy array) behind a tensor that ``device_vector`` made from host data, or None for
     any other tensor: lets a caller do on the host, with the same fp32 arithmetic, what would otherwise need a
-    read-back."""
-    return _host_values.get(id(tensor)) if tensor is not None else None
+    read-back.  A table tensor that somebody wrote to in place (its version counter moved) no longer counts: the
+    kernels would read the new values while the host sized grids from the old ones."""
+    entry = _host_values.get(id(tensor)) if tensor is not None else None
+    if entry is None or entry[0] is not tensor or tensor._version != 0:
+        return None
+    return entry[1]
 
 
 def host_num_cells(box_host, cell_host):

@@ -29,6 +29,8 @@ class Pointcloud(object):
         # batch ids that PointPooling selected carry the number of clouds along (a Poisson-disk selection keeps at
         # least one point of every cloud), which saves the read-back of their maximum
         self.batch_size_host_ = getattr(p_batch_ids, "pccnn_batch_size_", None)
+        if self.batch_size_host_ is not None and (self.batch_ids_ is not p_batch_ids or p_batch_ids._version != 0):
+            self.batch_size_host_ = None        # converted, moved or written to since the pooling made it
         self.batch_size_tensor_ = None
         if self.batch_size_host_ is None:
             self.batch_size_tensor_ = torch.max(self.batch_ids_) + 1

@@ -109,6 +109,10 @@ def bounding_box_host(pts, batch_ids, batch_size):
 # has passed, so that it cannot be handed out again while a write into it is still on its way.
 _LANDINGS = []
 
+# Reads of a polled pinned word before the host falls back to waiting for the event recorded behind the kernels
+# (tests lower it to exercise that fall-back).
+SPIN_LIMIT = 100000
+
 
 def _keep_until_written(landing, done):
     _LANDINGS.append((landing, done))
@@ -141,17 +145,16 @@ def bounding_box_host_later(pts, batch_ids, batch_size):
     _keep_until_written(landing, done)
 
     def fetch():
-        if polled.value:
-            spins = 0
-            while words[2 * count] < 0:
-                spins += 1
-                if spins > 100000:
-                    done.synchronize()
-                    break
-        else:
+        spins = 0
+        while polled.value and words[2 * count] < 0:
+            spins += 1
+            if spins > SPIN_LIMIT:
+                break
+        if not polled.value or words[2 * count] < 0:
             done.synchronize()
         host = landing.numpy()[:2 * count].reshape(2, batch_size, d)
         return host[0], host[1]
+    fetch.polled = bool(polled.value)
     return box[0], box[1], fetch
 
 
@@ -713,22 +716,25 @@ def pool_poisson_later(pts, batch_ids, aabb_min, cell_size, num_cells_host, batc
     total = pillars * cells[2]
     with_table = 1 if total <= CELL_TABLE_MAX_CELLS else 0
     ws = _workspace(lib.pccnn_pool_poisson_workspace_bytes(n, pillars, total if with_table else 0), dev)
+    polled = ctypes.c_int(0)
     _lib.call("pccnn_pool_poisson_select_queued", _ptr(pts), _ptr(batch_ids), n, batch_size, _ptr(aabb_min),
               _ptr(cell_size), (ctypes.c_int32 * 3)(*cells), key_bits_for(cells, batch_size), with_table, _P(base),
               _P(base + 4 * n), _P(base + 8 * n), _P(box.data_ptr()), _P(box.data_ptr() + 12 * batch_size),
-              _P(landing.data_ptr()), _ptr(ws), ws.numel(), _stream())
+              _P(landing.data_ptr()), ctypes.byref(polled), _ptr(ws), ws.numel(), _stream())
     done = torch.cuda.Event()
     done.record()
     _keep_until_written(landing, done)
 
     def finish():
-        # the count is the last word to arrive: a short poll of the pinned word, then the event if it takes long
+        # written by the kernels: the count is the last word to arrive, so a short poll of the pinned word, then
+        # the event if it takes long; brought over by copies (many clouds): the event right away
         spins = 0
-        while words[6 * batch_size] < 0:
+        while polled.value and words[6 * batch_size] < 0:
             spins += 1
-            if spins > 100000:
-                done.synchronize()
+            if spins > SPIN_LIMIT:
                 break
+        if words[6 * batch_size] < 0:
+            done.synchronize()
         host = landing.numpy()
         count = int(words[6 * batch_size])
         if count < 0:
@@ -745,6 +751,7 @@ def pool_poisson_later(pts, batch_ids, aabb_min, cell_size, num_cells_host, batc
     # a caller that drops `finish` unused waits with this before it lets go of it: the copy into the pinned block
     # must have landed before the block can be handed out again
     finish.wait = done.synchronize
+    finish.polled = bool(polled.value)
     return finish
 
 

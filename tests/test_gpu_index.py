@@ -589,3 +589,77 @@ def test_poisson_disk_from_the_grid_on_a_large_cloud_equals_the_list_version(ops
     covered = torch.zeros(pts.shape[0], dtype=torch.bool, device=DEV)
     covered[pair_sample[chosen[pair_pt]]] = True
     assert bool(covered.all())
+
+
+@pytest.mark.parametrize("pts_per_cloud,staged", [(2, False), (60, True)])
+def test_one_call_pooling_with_more_clouds_than_the_kernels_write_to_the_host_themselves(ops, monkeypatch, pts_per_cloud,
+                                                                                        staged):
+    # 90 clouds are 270 box values, more than the one workgroup that may write them into the pinned block itself: the
+    # one-call pooling then brings box and count over in copies (one staged copy of the boxes when the workspace has
+    # room for them - not with two points per cloud -, else two) and the host waits for the event instead of polling.
+    # Same tensors as the step-by-step route.
+    import pccnn_lib_amd as lib
+    from pccnn_lib_amd.pc import neighborhood, point_cloud, point_pooling
+    batch = 90
+    rng = np.random.default_rng(batch + pts_per_cloud)
+    pts = rng.random((batch * pts_per_cloud, 3), dtype=np.float32)
+    ids = np.repeat(np.arange(batch, dtype=np.int32), pts_per_cloud)
+    n = pts.shape[0]
+    assert (2 * batch * 12 + 4 <= 8 * n) == staged          # the library's own rule for the staged copy
+
+    def run(one_call):
+        for mod in (point_pooling, neighborhood, point_cloud):
+            monkeypatch.setattr(mod, "ONE_CALL", one_call)
+        pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+        pool = lib.pc.PointPooling(pc, 0.3)
+        if one_call:
+            assert pool.pending_ is not None and pool.pending_.polled is False
+        out_pc = lib.pc.Pointcloud(pool.pool_tensor(pc.pts_), pool.pool_tensor(pc.batch_ids_))
+        box = lib.pc.BoundingBox(out_pc)
+        fresh_min, fresh_max = ops.bounding_box(out_pc.pts_, out_pc.batch_ids_, batch)
+        assert torch.equal(box.min_, fresh_min) and torch.equal(box.max_, fresh_max)
+        assert np.array_equal(box.host()[0], fresh_min.cpu().numpy())
+        assert np.array_equal(box.host()[1], fresh_max.cpu().numpy())
+        return [pool.pooling_ids_, out_pc.pts_, out_pc.batch_ids_, box.min_, box.max_]
+
+    a, b = run(False), run(True)
+    assert a[0].shape[0] >= batch
+    for x, y in zip(a, b):
+        assert x.dtype == y.dtype and torch.equal(x, y)
+
+
+def test_box_of_many_clouds_in_six_dimensions_travels_in_copies(ops):
+    # 50 clouds x 6 dimensions = 300 box values: the queued box does not write the pinned block from its kernels
+    # (polled_out = 0); the copies and the event bring the same numbers as a read-back of the device tensors
+    import pccnn_lib_amd as lib
+    batch, per = 50, 40
+    rng = np.random.default_rng(6)
+    pts = rng.normal(size=(batch * per, 6)).astype(np.float32)
+    ids = np.repeat(np.arange(batch, dtype=np.int32), per)
+    mn, mx, fetch = ops.bounding_box_host_later(t(pts), t(ids), batch)
+    assert fetch.polled is False
+    host_min, host_max = fetch()
+    assert np.array_equal(host_min, mn.cpu().numpy()) and np.array_equal(host_max, mx.cpu().numpy())
+    exp_min = np.stack([pts[ids == b].min(axis=0) for b in range(batch)]) - np.float32(1e-6)
+    assert np.array_equal(host_min, exp_min.astype(np.float32))
+    box = lib.pc.BoundingBox(lib.pc.Pointcloud(pts, ids, device=DEV), p_with_host=True)
+    assert np.array_equal(box.host()[0], box.min_.cpu().numpy()) and np.array_equal(box.host()[1], box.max_.cpu().numpy())
+    # the small case for contrast: written by the kernels, polled
+    small = ops.bounding_box_host_later(t(pts[:, :3].copy()), t(ids), batch)
+    assert small[2].polled is True
+    assert np.array_equal(small[2]()[0], small[0].cpu().numpy())
+
+
+def test_polled_read_backs_fall_back_to_the_event_when_the_spin_limit_is_reached(ops, monkeypatch):
+    # with a spin limit of zero the host gives up polling at once and waits for the event recorded behind the
+    # kernels: same results
+    import pccnn_lib_amd as lib
+    pts, ids = synthetic.primitives(77, 3, 4000)
+    pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+    want = lib.pc.PointPooling(pc, 0.07).pooling_ids_
+    monkeypatch.setattr(ops, "SPIN_LIMIT", 0)
+    pool = lib.pc.PointPooling(lib.pc.Pointcloud(pts, ids, device=DEV), 0.07)
+    assert pool.pending_ is not None and pool.pending_.polled is True
+    assert torch.equal(pool.pooling_ids_, want)
+    mn, mx, fetch = ops.bounding_box_host_later(t(pts), t(ids), 3)
+    assert np.array_equal(fetch()[0], mn.cpu().numpy()) and np.array_equal(fetch()[1], mx.cpu().numpy())

@@ -44,6 +44,30 @@ def _both(lib, n, key_bits, seed, with_pts):
         assert np.array_equal(x1, x0) and np.array_equal(x0, pts.cpu().numpy()[p0])
 
 
+def test_static_sort_leaves_the_free_device_memory_unchanged():
+    # what the entry point is for: once the first call on the device has looked up the scratch array's address, a
+    # call neither allocates nor frees device memory (hipMemGetInfo before and after, inputs and outputs made first)
+    from pccnn_lib_amd import _lib
+    lib = _lib.load()
+    ptr = lambda x: ctypes.c_void_p(0 if x is None else x.data_ptr())
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    gen = torch.Generator(device=DEV).manual_seed(9)
+    n = 200_000
+    keys = torch.randint(0, 1 << 20, (n,), dtype=torch.int64, device=DEV, generator=gen)
+    pts = torch.rand((n, 3), device=DEV, generator=gen)
+    skeys, perm, spts = torch.empty_like(keys), torch.empty((n,), dtype=torch.int32, device=DEV), torch.empty_like(pts)
+    call = lambda count: lib.pccnn_sort_keys_static(ptr(keys), count, 20, ptr(skeys), ptr(perm), ptr(pts), 3, ptr(spts),
+                                                   stream)
+    assert call(n) == 0, lib.pccnn_last_error()
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for count in (n, 50_000, n):
+        assert call(count) == 0, lib.pccnn_last_error()
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
+    assert torch.equal(skeys, torch.sort(keys, stable=True)[0])
+
+
 def test_static_sort_equals_the_workspace_sort_on_two_calls_in_a_row():
     from pccnn_lib_amd import _lib
     lib = _lib.load()
