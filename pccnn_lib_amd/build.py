@@ -62,7 +62,47 @@ def build(verbose=True, jobs=8, incremental=False):
     return LIB_PATH
 
 
+EXT_SOURCE = os.path.join(CSRC, "ops_module.cpp")
+
+
+def extension_path():
+    """Where the compiled ``pccnn_lib_ops`` module goes: the repository root, beside the package, so that
+    ``import pccnn_lib_ops`` finds it (an extension module takes precedence over the .py of the same name there)."""
+    import sysconfig
+    return os.path.join(os.path.dirname(HERE), "pccnn_lib_ops" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_extension(verbose=True):
+    """Compiles csrc/ops_module.cpp - the ``pccnn_lib_ops`` PyTorch extension (pybind11, host code only) - against
+    this interpreter's torch and links it to libpccnn_hip.so (found at run time relative to the module)."""
+    import sysconfig
+    import torch
+    from torch.utils import cpp_extension
+    cxx = os.environ.get("CXX", "g++")
+    out = extension_path()
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wno-attributes",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=pccnn_lib_ops",
+           "-DTORCH_API_INCLUDE_EXTENSION_H", "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI)]
+    for inc in cpp_extension.include_paths("cuda") + [sysconfig.get_paths()["include"],
+                                                       os.path.join(os.path.dirname(HERE), "include")]:
+        cmd += ["-isystem" if "torch" in inc or "rocm" in inc else "-I", inc]
+    cmd += [EXT_SOURCE, "-o", out, "-L" + torch_lib, "-L" + HERE, "-l:libpccnn_hip.so", "-ltorch", "-ltorch_cpu",
+            "-ltorch_python", "-lc10", "-lc10_hip", "-ltorch_hip", "-Wl,-rpath,$ORIGIN/pccnn_lib_amd",
+            "-Wl,-rpath," + torch_lib]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("compiling the pccnn_lib_ops extension failed:\n%s" % res.stdout)
+    if verbose and res.stdout.strip():
+        print(res.stdout)
+    return out
+
+
 if __name__ == "__main__":
     build(incremental="--incremental" in sys.argv)
+    if "--no-extension" not in sys.argv:
+        print("built", build_extension())
     print("built", LIB_PATH)
     sys.exit(0)

@@ -1392,3 +1392,67 @@ REFERENCE_NAMES = (
     "point_conv_grads", "point_conv_weight_var", "kp_conv", "kp_conv_grads", "kp_conv_weight_var", "kp_conv_n",
     "kp_conv_n_grads", "kp_conv_n_weight_var", "sph_conv", "sph_conv_grads", "sph_conv_weight_var", "pccnn",
     "pccnn_grads", "pccnn_weight_variance")
+
+
+# ----------------------------------------------------------------------------- bindings
+#
+# Two bindings of the same C ABI serve the 26 reference names: the compiled extension module ``pccnn_lib_ops`` (what
+# the reference builds from setup.py:7-31; csrc/ops_module.cpp here: pybind11, TORCH_CHECK contracts, at::empty
+# outputs, torch's current HIP stream) and the ctypes functions above, which need no compiler.  The compiled one is
+# used when it has been built; ``use_binding`` switches.  Functions beyond the 26 names exist only in this module.
+
+BINDINGS = {"ctypes": {name: globals()[name] for name in REFERENCE_NAMES}}
+binding = "ctypes"
+
+
+def _load_compiled():
+    import importlib.util
+    import os
+    import sys
+    mod = sys.modules.get("pccnn_lib_ops")
+    if mod is not None and getattr(mod, "binding", None) == "compiled":
+        return mod
+    from .build import extension_path
+    path = extension_path()
+    if not os.path.exists(path):
+        return None
+    _lib.load()                                   # libpccnn_hip.so first, by its path
+    spec = importlib.util.spec_from_file_location("pccnn_lib_ops", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    sys.modules.setdefault("pccnn_lib_ops", mod)    # a later ``import pccnn_lib_ops`` gets this very module
+    return mod
+
+
+def use_binding(which):
+    """Route the 26 reference names through the "compiled" extension or through "ctypes"; returns the name of the
+    binding in use before the call.  Raises if the compiled module has not been built."""
+    global binding
+    if which not in BINDINGS:
+        if which != "compiled":
+            raise RuntimeError("use_binding: 'compiled' or 'ctypes', got %r" % (which,))
+        mod = _load_compiled()
+        if mod is None:
+            raise RuntimeError("use_binding: the compiled pccnn_lib_ops extension has not been built "
+                               "(python -m pccnn_lib_amd.build)")
+        BINDINGS["compiled"] = {name: getattr(mod, name) for name in REFERENCE_NAMES}
+    before, binding = binding, which
+    globals().update(BINDINGS[which])
+    return before
+
+
+def _initial_binding():
+    """The compiled binding when it has been built, unless the environment asks for the other
+    (PCCNN_LIB_OPS_BINDING=ctypes|compiled; asking for a compiled module that is not there is an error)."""
+    import os
+    asked = os.environ.get("PCCNN_LIB_OPS_BINDING", "")
+    if asked:
+        use_binding(asked)
+        return
+    try:
+        use_binding("compiled")
+    except (RuntimeError, ImportError, OSError):      # not built (or built for another torch): ctypes it is
+        pass
+
+
+_initial_binding()

@@ -206,3 +206,66 @@ def test_point_side_keeps_the_plain_route_unless_the_pairs_are_in_key_order():
     assert pts is wanted.pts_ and pairs is keyed.neighbors_ and moved is feats
     layer = conv_base.IConvLayer(3, 2, 2)
     assert layer.key_order_capable_ is False and conv_base.KEY_ORDER_MIN_POINTS >= 100000
+
+
+@pytest.fixture(scope="module")
+def compiled_module(lib_path):
+    from pccnn_lib_amd import build
+    if not os.path.exists(build.extension_path()):
+        build.build_extension(verbose=False)
+    from pccnn_lib_amd import pccnn_lib_ops as ops
+    before = ops.use_binding("compiled")
+    ops.use_binding(before)
+    import sys
+    return sys.modules["pccnn_lib_ops"]
+
+
+def test_import_of_the_reference_name_resolves_to_the_compiled_extension(compiled_module):
+    # setup.py:7-8 of the reference builds an extension module named pccnn_lib_ops; so does this build, and a plain
+    # `import pccnn_lib_ops` from the repository root finds the shared object rather than the Python stand-in
+    import subprocess
+    import sys
+    code = ("import pccnn_lib_ops as m\n"
+            "assert m.__file__.endswith('.so'), m.__file__\n"
+            "assert m.binding == 'compiled' and len(m.REFERENCE_NAMES) == 26\n"
+            "assert all(callable(getattr(m, n)) for n in m.REFERENCE_NAMES)\n")
+    res = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr
+
+
+@pytest.mark.parametrize("which", ["compiled", "ctypes"])
+def test_both_bindings_export_the_reference_names_and_validate_on_the_host(compiled_module, which):
+    import torch
+    from pccnn_lib_amd import pccnn_lib_ops as ops
+    before = ops.use_binding(which)
+    try:
+        assert ops.binding == which
+        for name in ops.REFERENCE_NAMES:
+            assert callable(getattr(ops, name)) and getattr(ops, name) is ops.BINDINGS[which][name]
+        z, zi = torch.zeros(4, 3), torch.zeros(4, dtype=torch.int32)
+        with pytest.raises(RuntimeError, match="GPU tensor"):
+            ops.compute_keys(z, zi, torch.zeros(1, 3), torch.ones(3, dtype=torch.int32), torch.ones(3))
+        with pytest.raises(RuntimeError, match="GPU tensor"):
+            ops.sph_conv(z, z, z, z, z, z, z, z, z, z)
+        with pytest.raises(RuntimeError, match="GPU tensor"):
+            ops.point_conv(z, z, z, z, z)
+        with pytest.raises(RuntimeError, match="GPU tensor"):
+            ops.mc_conv_grads(z, z, z, z, z, z, z, z, z, z, z, grad_mask=ops.GRAD_FEATS, contraction="bf16")
+    finally:
+        ops.use_binding(before)
+
+
+def test_compiled_functions_take_the_arguments_of_the_ctypes_functions(compiled_module):
+    # same parameter count and the same keyword additions (return_proj, proj, grad_mask, mirror, contraction), read
+    # from the signature line pybind11 writes into each docstring
+    import inspect
+    from pccnn_lib_amd import pccnn_lib_ops as ops
+    for name in ops.REFERENCE_NAMES:
+        py_params = list(inspect.signature(ops.BINDINGS["ctypes"][name]).parameters.values())
+        line = getattr(compiled_module, name).__doc__.splitlines()[0]
+        inner = line[line.index("(") + 1:line.rindex(")")]
+        c_params = [p for p in re.split(r",\s*(?![^\[]*\])", inner) if p]
+        assert len(c_params) == len(py_params), (name, line)
+        for cp, pp in zip(c_params, py_params):
+            if pp.default is not inspect.Parameter.empty:
+                assert cp.split(":")[0].strip() == pp.name and "=" in cp, (name, cp, pp.name)
