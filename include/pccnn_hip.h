@@ -386,6 +386,15 @@ int pccnn_mcconv_backward(const float *pts, const float *pdf, const float *feats
                           float *d_pts, float *d_samples,
                           void *workspace, size_t workspace_bytes, void *stream);
 
+/* An optional forward path that keeps the projection on chip: with pccnn_set_fused_forward(1), forward calls that are
+ * not asked for the projection (proj_out == NULL) and whose shape allows it (3-D or caller-given basis, k <= 16,
+ * num_mlps == 1, c_in > 32, c_out 64, 128 or 256) run as one kernel that gathers a 64-sample x 256-column slice of P
+ * into LDS and multiplies it with the matching rows of the weights right away, where the reference writes P out and
+ * reads it back for torch::matmul (pccnn_lib_ops/pcconvs/kpconv.cu:52-57, mcconv.cu:58-68).  Same results to rounding.
+ * Off by default: on MI355X the two-kernel path is faster (csrc/conv_fused.hip has the figures).  Returns the
+ * previous setting.  Process-wide. */
+int pccnn_set_fused_forward(int on);
+
 /* ---- the other convolution families -----------------------------------------
  * One descriptor-driven triple covers KPConvN, PCCNN, PointConv and SPHConv (and, redundantly, KPConv and
  * MCConv).  It replaces kp_conv_n* (pccnn_lib_ops/pcconvs/kpconvn.cuh:32-93), pccnn* (pccnn.cuh:32-93),

@@ -66,6 +66,7 @@ SIGNATURES = {
                                        I32, P, P, P, SZ, P, SZ, P]),
     "pccnn_conv_workspace_bytes": (SZ, [I64, I64, I32, I32, I32, I32]),
     "pccnn_kpconv_forward": (I32, [P, P, P, P, P, P, P, F32, P, I64, I64, I64, I32, I32, I32, I32, P, P, P, SZ, P]),
+    "pccnn_set_fused_forward": (I32, [I32]),
     "pccnn_mirror_pairs": (I32, [P, P, I64, I64, P, P, P]),
     "pccnn_kpconv_backward": (I32, [P, P, P, P, P, P, P, F32, P, P, P, P, I32, I64, I64, I64, I32, I32, I32, I32,
                                     P, P, P, P, P, P, SZ, P]),
@@ -114,7 +115,10 @@ def load():
             "(needs hipcc; there is no fallback implementation)" % LIB_PATH)
     lib = ctypes.CDLL(LIB_PATH)
     for name, (res, args) in SIGNATURES.items():
-        fn = getattr(lib, name)
+        fn = getattr(lib, name, None)
+        if fn is None:
+            raise RuntimeError("pccnn_lib_amd: %s does not export %s: it was built from older sources; rebuild it "
+                               "with `python -m pccnn_lib_amd.build`" % (LIB_PATH, name))
         fn.restype = res
         fn.argtypes = args
     _lib = lib

@@ -210,7 +210,7 @@ __device__ __forceinline__ float pccnn_wave_sum(float v)
 // A negative id never times (and so never creates an event).
 enum PccnnTimerId {
     PCCNN_T_GEMM = 0, PCCNN_T_PROJ_FWD, PCCNN_T_PROJ_BWD, PCCNN_T_BASIS_BWD, PCCNN_T_NB_COUNT, PCCNN_T_NB_FILL,
-    PCCNN_T_SORT, PCCNN_T_KEYS, PCCNN_T_GRID, PCCNN_T_PDF, PCCNN_T_SCAN, PCCNN_T_COUNT
+    PCCNN_T_SORT, PCCNN_T_KEYS, PCCNN_T_GRID, PCCNN_T_PDF, PCCNN_T_SCAN, PCCNN_T_FUSED_FWD, PCCNN_T_COUNT
 };
 struct PccnnTimed {
     int id;

@@ -14,41 +14,7 @@
 // (feature rows staged in LDS, K-lane partial sums); a per-sample kernel then applies the basis
 // derivative and accumulates point, sample, density and basis-parameter gradients.
 #include "common.h"
-
-// Basis families (values = PCCNN_BASIS_* of the C header).
-//   KP     clamp(1 - |kp_k - d| / sigma, 0, 1)                      (KPConv)
-//   MLP    leaky_relu(d . A_k + b_k, 0.2) / pdf                     (MCConv)
-//   KPN    the KP value / pdf                                       (KPConvN)
-//   GAUSS  exp(-|kp_k - d|^2 / (2 sigma^2)) / pdf                   (PCCNN)
-//   EXPLICIT  values given per pair in a [T, K] tensor              (PointConv)
-//   SPH    one-hot spherical bin of d, bin 0 = the centre           (SPHConv)
-//   LINEAR d . A_k + b_k                                            (PointConv's own basis op)
-enum { BASIS_KP = 0, BASIS_MLP = 1, BASIS_KPN = 2, BASIS_GAUSS = 3, BASIS_EXPLICIT = 4, BASIS_SPH = 5,
-       BASIS_LINEAR = 6 };
-
-template <int BASIS> struct BasisTraits {
-    static constexpr bool kernel_pts = BASIS == BASIS_KP || BASIS == BASIS_KPN || BASIS == BASIS_GAUSS;
-    static constexpr bool axis = BASIS == BASIS_MLP || BASIS == BASIS_LINEAR;
-    static constexpr bool uses_pdf = BASIS == BASIS_MLP || BASIS == BASIS_KPN || BASIS == BASIS_GAUSS;
-    static constexpr bool pdf_grad = BASIS == BASIS_MLP || BASIS == BASIS_GAUSS;
-    static constexpr bool differentiable = kernel_pts || axis;       // has a basis_bwd stage
-};
-
-struct ConvGeom {
-    const float *pts;       // [n,3]
-    const float *samples;   // [m,3]
-    const int2 *neigh;      // [t] (point, sample)
-    const int32_t *ends;    // [m]
-    const float *radii;     // [3]
-    const float *pdf;       // [n] or null
-    const float *basis_a;   // kernel points [K,3] | axis [3,K] | explicit basis [T,K] | radial bin edges
-    const float *basis_b;   // bias [K] | azimuth bin edges
-    float sigma;
-    int64_t n, m, t;
-    int c_in, k;
-    const float *basis_c;   // polar bin edges
-    int nb0, nb1, nb2;      // spherical bin counts
-};
+#include "conv_basis.h"
 
 // Sample lists usually come in a spatial order (pooled points and sorted clouds are in cell order), and neighboring
 // samples share most of their neighbors: runs of CONV_XCD_CHUNK consecutive samples go to one XCD (see
@@ -66,74 +32,6 @@ __device__ __forceinline__ int64_t conv_sample_of_block(unsigned block, int64_t 
     return pccnn_xcd_block(block, gridDim.x, CONV_XCD_CHUNK);
 }
 static inline unsigned conv_sample_blocks(int64_t m) { return pccnn_xcd_grid(m, CONV_XCD_CHUNK); }
-
-// First bin whose upper edge is >= v, the last bin when there is none.
-__device__ __forceinline__ int sph_bin(float v, const float *__restrict__ edges, int count)
-{
-    int id = -1;
-    for (int i = 0; i < count; ++i)
-        if (v <= edges[i] && id < 0) id = i;
-    return id < 0 ? count - 1 : id;
-}
-
-template <int BASIS> struct LaneBasis {
-    float c0, c1, c2, c3;
-    int kk;
-    bool active;
-    __device__ __forceinline__ void load(const ConvGeom &g, int k)
-    {
-        active = k < g.k;
-        kk = k;
-        c0 = c1 = c2 = c3 = 0.0f;
-        if (active) {
-            if (BasisTraits<BASIS>::kernel_pts) {
-                c0 = g.basis_a[k * 3 + 0]; c1 = g.basis_a[k * 3 + 1]; c2 = g.basis_a[k * 3 + 2];
-            } else if (BasisTraits<BASIS>::axis) {
-                c0 = g.basis_a[k]; c1 = g.basis_a[g.k + k]; c2 = g.basis_a[2 * g.k + k]; c3 = g.basis_b[k];
-            }
-        }
-    }
-    // Basis value of this lane's k for a pair with normalised offset (dx,dy,dz).
-    __device__ __forceinline__ float eval(const ConvGeom &g, float dx, float dy, float dz, float pdf) const
-    {
-        float w = 0.0f;
-        if (BASIS == BASIS_KP || BASIS == BASIS_KPN) {
-            const float vx = c0 - dx, vy = c1 - dy, vz = c2 - dz;
-            const float d2 = fmaxf(vx * vx + vy * vy + vz * vz, 0.0f);
-            const float r = 1.0f - sqrtf(d2) / g.sigma;
-            w = fminf(fmaxf(r, 0.0f), 1.0f);
-            if (BASIS == BASIS_KPN) w = w / pdf;
-        } else if (BASIS == BASIS_GAUSS) {
-            const float vx = c0 - dx, vy = c1 - dy, vz = c2 - dz;
-            const float d2 = vx * vx + vy * vy + vz * vz;
-            w = expf(-(d2 / (2.0f * g.sigma * g.sigma))) / pdf;
-        } else if (BASIS == BASIS_MLP) {
-            float a = dx * c0 + dy * c1 + dz * c2 + c3;
-            a = a > 0.0f ? a : a * 0.2f;
-            w = a / pdf;
-        } else if (BASIS == BASIS_LINEAR) {
-            w = dx * c0 + dy * c1 + dz * c2 + c3;
-        } else if (BASIS == BASIS_SPH) {
-            const float dist = sqrtf(dx * dx + dy * dy + dz * dz);
-            const float azimuth = atanf(dy / (dx + 1e-6f));
-            const float polar = acosf(fminf(fmaxf(dz / (dist + 1e-6f), -0.99999f), 0.99999f));
-            int id = sph_bin(dist, g.basis_a, g.nb0) * g.nb1 * g.nb2 + sph_bin(azimuth, g.basis_b, g.nb1) * g.nb2 +
-                     sph_bin(polar, g.basis_c, g.nb2) + 1;
-            if (dist < 1e-4f) id = 0;
-            w = (id == kk) ? 1.0f : 0.0f;
-        }
-        return active ? w : 0.0f;
-    }
-};
-
-// Basis value for pair `pair` (global pair index) of the chunk: evaluated, or read when given explicitly.
-template <int BASIS>
-__device__ __forceinline__ float pair_basis(const ConvGeom &g, const LaneBasis<BASIS> &lb, int64_t pair, float dx,
-                                            float dy, float dz, float pdf)
-{
-    if (BASIS == BASIS_EXPLICIT) return lb.active ? g.basis_a[pair * g.k + lb.kk] : 0.0f;
-    return lb.eval(g, dx, dy, dz, pdf);
-}
 
 // ------------------------------------------------------------------------------- forward
 
@@ -1239,7 +1137,8 @@ extern "C" size_t pccnn_conv_workspace_bytes(int64_t m, int64_t t, int c_in, int
     size_t proj = pccnn_align((size_t)m * c_in * k * sizeof(float));
     size_t w16 = pccnn_align((size_t)c_in * k * c_out * sizeof(uint16_t));       // bf16 copy of the weights
     size_t pair_b = 2 * pccnn_align((size_t)t * k * sizeof(float));              // basis (+ its gradient) when d != 3
-    if (!backward) return proj + w16 + pair_b + 256;
+    // (a forward call that keeps no projection may run fused and then needs room for the repacked weights only)
+    if (!backward) return proj + w16 + pair_b + pccnn_conv_fused_workspace_bytes(c_in, k, c_out) + 256;
     size_t basis_g = pccnn_align((size_t)t * k * sizeof(float));
     size_t splitk = pccnn_align((size_t)CONV_SPLIT_K * c_in * k * c_out * sizeof(float));
     size_t partials = pccnn_align(((size_t)PARAM_ROWS + PARAM_REDUCE_GROUPS) * 256 * sizeof(float));
@@ -1282,6 +1181,15 @@ static int conv_forward(ConvGeom g, const float *feats, const float *weights, in
                         bool divide_by_count = false, bool bf16 = false)
 {
     if (g.m == 0) return PCCNN_OK;
+    if constexpr (BASIS != BASIS_SPH) {
+        // nobody wants the projection: it stays on chip, slice by slice, between the gather and the matrix cores
+        if (proj_out == nullptr && pccnn_conv_fused_eligible(BASIS, g.c_in, g.k, num_mlps, c_out)) {
+            PCCNN_REQUIRE(workspace && workspace_bytes >= pccnn_conv_fused_workspace_bytes(g.c_in, g.k, c_out),
+                          PCCNN_ERR_WORKSPACE, "conv forward: workspace of %zu bytes, need %zu", workspace_bytes,
+                          pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 0));
+            return pccnn_conv_fused_forward<BASIS>(g, feats, weights, c_out, out, workspace, divide_by_count, bf16, s);
+        }
+    }
     PccnnArena arena(workspace, workspace_bytes);
     void *proj = proj_out;
     if (proj == nullptr) proj = arena.take<float>((size_t)g.m * g.c_in * g.k);

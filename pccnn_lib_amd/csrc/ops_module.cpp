@@ -359,11 +359,13 @@ py::object generic_forward(const std::string &name, const Generic &g, const Tens
     const int64_t n = g.feats.size(0), m = g.ends.size(0), t = g.neigh.size(0);
     const int c_in = (int)g.feats.size(1);
     Tensor out = at::empty({m, c_out}, g.feats.options());
-    Tensor proj = at::empty({m, c_in, g.k}, g.feats.options().dtype(bf16 ? at::kBFloat16 : at::kFloat));
+    // a call that does not hand the projection back lets the library build it in the workspace - or keep it on chip
+    Tensor proj;
+    if (return_proj) proj = at::empty({m, c_in, g.k}, g.feats.options().dtype(bf16 ? at::kBFloat16 : at::kFloat));
     Tensor ws;
     void *ws_p = nullptr;
     size_t ws_n = 0;
-    if (bf16 || (g.pts && g.pts->size(1) != 3)) {
+    if (bf16 || !return_proj || (g.pts && g.pts->size(1) != 3)) {
         ws = workspace(pccnn_conv_workspace_bytes(m, t, c_in, g.k, (int)c_out, 0), g.feats);
         ws_p = ws.data_ptr();
         ws_n = (size_t)ws.numel();
@@ -373,13 +375,14 @@ py::object generic_forward(const std::string &name, const Generic &g, const Tens
     if (bf16)
         rc_check(pccnn_conv_forward_bf16(&g.desc, pts, fptr(g.feats), smp, iptr(g.neigh), iptr(g.ends), rad,
                                          fptr(weights), n, m, t, g.dims(), c_in, num_mlps, (int)c_out,
-                                         g.divide_by_count, out.data_ptr<float>(), (uint16_t *)proj.data_ptr(), ws_p,
-                                         ws_n, cur_stream()),
+                                         g.divide_by_count, out.data_ptr<float>(),
+                                         return_proj ? (uint16_t *)proj.data_ptr() : nullptr, ws_p, ws_n, cur_stream()),
                  "pccnn_conv_forward_bf16");
     else
         rc_check(pccnn_conv_forward(&g.desc, pts, fptr(g.feats), smp, iptr(g.neigh), iptr(g.ends), rad, fptr(weights), n,
                                     m, t, g.dims(), c_in, num_mlps, (int)c_out, g.divide_by_count,
-                                    out.data_ptr<float>(), proj.data_ptr<float>(), ws_p, ws_n, cur_stream()),
+                                    out.data_ptr<float>(), return_proj ? proj.data_ptr<float>() : nullptr, ws_p, ws_n,
+                                    cur_stream()),
                  "pccnn_conv_forward");
     return out_and_proj(out, proj, return_proj);
 }

@@ -28,7 +28,8 @@ static std::vector<TimedPair> g_timing_pending[PCCNN_T_COUNT];
 static double g_timing_ms[PCCNN_T_COUNT];
 static long long g_timing_n[PCCNN_T_COUNT];
 static const char *g_timing_names[PCCNN_T_COUNT] = {"gemm", "proj_fwd", "proj_bwd", "basis_bwd", "nb_count",
-                                                    "nb_fill",  "sort",     "keys",     "grid",      "pdf", "scan"};
+                                                    "nb_fill",  "sort",     "keys",     "grid",      "pdf", "scan",
+                                                    "fused_fwd"};
 
 PccnnTimed::PccnnTimed(int id_, hipStream_t s) : id(id_), stream(s), stop(nullptr), on(g_timing_on && id_ >= 0)
 {

@@ -1,9 +1,10 @@
 import torch
 
 from .. import pccnn_lib_ops
+from ._forward_only import ConvFunction, keeps_projection
 
 
-class ComputeKPConv(torch.autograd.Function):
+class ComputeKPConv(ConvFunction):
     """apply(pts, features, samples, neighbors, start_ids, radii, kernel_pts, sigma, conv_weights) -> [M, Cout].
     Gradients are routed to (pts, features, samples, -, -, -, kernel_pts, -, conv_weights)
     (pccnn_lib/op_wrappers/compute_kpconv.py:14-73).  The projection built by the forward pass is kept for the
@@ -15,9 +16,11 @@ class ComputeKPConv(torch.autograd.Function):
     @staticmethod
     def forward(ctx, p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_kernel_pts, p_sigma,
                 p_conv_weights, p_mirror=None, p_contraction="f32"):
-        out, proj = pccnn_lib_ops.kp_conv(p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii,
-                                          p_kernel_pts, p_sigma, p_conv_weights, return_proj=True,
-                                          contraction=p_contraction)
+        keep = keeps_projection(ctx)          # no backward pass can follow: nothing is kept
+        out = pccnn_lib_ops.kp_conv(p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii,
+                                    p_kernel_pts, p_sigma, p_conv_weights, return_proj=keep,
+                                    contraction=p_contraction)
+        out, proj = out if keep else (out, None)
         ctx.contraction_ = p_contraction
         ctx.save_for_backward(p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_kernel_pts,
                               p_conv_weights, proj)

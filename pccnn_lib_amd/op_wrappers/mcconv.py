@@ -1,9 +1,10 @@
 import torch
 
 from .. import pccnn_lib_ops
+from ._forward_only import ConvFunction, keeps_projection
 
 
-class ComputeMCConv(torch.autograd.Function):
+class ComputeMCConv(ConvFunction):
     """apply(pts, pdf, features, samples, neighbors, start_ids, radii, proj_axis, proj_bias, conv_weights)
     -> [M, Cout].  Gradients are routed to (pts, pdf, features, samples, -, -, -, proj_axis, proj_bias,
     conv_weights) (pccnn_lib/op_wrappers/compute_mcconv.py:14-75).  The projection built by the forward pass is
@@ -15,9 +16,11 @@ class ComputeMCConv(torch.autograd.Function):
     @staticmethod
     def forward(ctx, p_pts, p_pdf, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_proj_axis,
                 p_proj_bias, p_conv_weights, p_mirror=None, p_contraction="f32"):
-        out, proj = pccnn_lib_ops.mc_conv(p_pts, p_pdf, p_features, p_samples, p_neighbors, p_start_ids, p_radii,
-                                          p_proj_axis, p_proj_bias, p_conv_weights, return_proj=True,
-                                          contraction=p_contraction)
+        keep = keeps_projection(ctx)          # no backward pass can follow: nothing is kept
+        out = pccnn_lib_ops.mc_conv(p_pts, p_pdf, p_features, p_samples, p_neighbors, p_start_ids, p_radii,
+                                    p_proj_axis, p_proj_bias, p_conv_weights, return_proj=keep,
+                                    contraction=p_contraction)
+        out, proj = out if keep else (out, None)
         ctx.contraction_ = p_contraction
         ctx.save_for_backward(p_pts, p_pdf, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_proj_axis,
                               p_proj_bias, p_conv_weights, proj)

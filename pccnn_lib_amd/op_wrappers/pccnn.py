@@ -1,9 +1,10 @@
 import torch
 
 from .. import pccnn_lib_ops
+from ._forward_only import ConvFunction, keeps_projection
 
 
-class ComputePCCNN(torch.autograd.Function):
+class ComputePCCNN(ConvFunction):
     """apply(pts, pdf, features, samples, neighbors, start_ids, radii, kernel_pts, sigma, conv_weights) -> [M, Cout]:
     gaussian kernel-point correlation divided by the density of each neighbor.  Gradients go to
     (pts, pdf, features, samples, -, -, -, kernel_pts, -, conv_weights)
@@ -12,8 +13,10 @@ class ComputePCCNN(torch.autograd.Function):
     @staticmethod
     def forward(ctx, p_pts, p_pt_pdf, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_kernel_pts, p_sigma,
                 p_conv_weights, p_mirror=None):
-        out, proj = pccnn_lib_ops.pccnn(p_pts, p_features, p_pt_pdf, p_samples, p_neighbors, p_start_ids, p_radii,
-                                        p_kernel_pts, p_sigma, p_conv_weights, return_proj=True)
+        keep = keeps_projection(ctx)          # no backward pass can follow: nothing is kept
+        out = pccnn_lib_ops.pccnn(p_pts, p_features, p_pt_pdf, p_samples, p_neighbors, p_start_ids, p_radii,
+                                  p_kernel_pts, p_sigma, p_conv_weights, return_proj=keep)
+        out, proj = out if keep else (out, None)
         ctx.save_for_backward(p_pts, p_pt_pdf, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_kernel_pts,
                               p_conv_weights, proj)
         ctx.sigma_ = p_sigma

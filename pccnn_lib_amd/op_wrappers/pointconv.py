@@ -1,6 +1,7 @@
 import torch
 
 from .. import pccnn_lib_ops
+from ._forward_only import ConvFunction, keeps_projection
 
 
 class ComputePointConvBasis(torch.autograd.Function):
@@ -21,15 +22,17 @@ class ComputePointConvBasis(torch.autograd.Function):
         return pt_grads, sample_grads, None, None, axis_grad, bias_grad.reshape(axis_bias.shape)
 
 
-class ComputePointConv(torch.autograd.Function):
+class ComputePointConv(ConvFunction):
     """apply(basis_proj [T, K], features, neighbors, start_ids, conv_weights) -> [M, Cout]; gradients go to
     (basis_proj, features, -, -, conv_weights) (pccnn_lib/op_wrappers/compute_pointconv.py:61-107)."""
 
     @staticmethod
     def forward(ctx, p_basis_proj, p_features, p_neighbors, p_start_ids, p_conv_weights):
         p_basis_proj = p_basis_proj.contiguous()
-        out, proj = pccnn_lib_ops.point_conv(p_basis_proj, p_features, p_neighbors, p_start_ids, p_conv_weights,
-                                             return_proj=True)
+        keep = keeps_projection(ctx)          # no backward pass can follow: nothing is kept
+        out = pccnn_lib_ops.point_conv(p_basis_proj, p_features, p_neighbors, p_start_ids, p_conv_weights,
+                                       return_proj=keep)
+        out, proj = out if keep else (out, None)
         ctx.save_for_backward(p_basis_proj, p_features, p_neighbors, p_start_ids, p_conv_weights, proj)
         return out
 

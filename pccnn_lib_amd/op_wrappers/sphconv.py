@@ -1,9 +1,10 @@
 import torch
 
 from .. import pccnn_lib_ops
+from ._forward_only import ConvFunction, keeps_projection
 
 
-class ComputeSPHConv(torch.autograd.Function):
+class ComputeSPHConv(ConvFunction):
     """apply(pts, features, samples, neighbors, start_ids, radii, radial_bins, azimuz_bins, polar_bins, conv_weights)
     -> [M, Cout]: one-hot spherical-bin correlation divided by the neighbor count.  Only the features and the
     weights get gradients (pccnn_lib/op_wrappers/compute_sphconv.py:5-66)."""
@@ -11,9 +12,11 @@ class ComputeSPHConv(torch.autograd.Function):
     @staticmethod
     def forward(ctx, p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_radial_bins, p_azimuz_bins,
                 p_polar_bins, p_conv_weights):
-        out, proj = pccnn_lib_ops.sph_conv(p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii,
-                                           p_radial_bins, p_azimuz_bins, p_polar_bins, p_conv_weights,
-                                           return_proj=True)
+        keep = keeps_projection(ctx)          # no backward pass can follow: nothing is kept
+        out = pccnn_lib_ops.sph_conv(p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii,
+                                     p_radial_bins, p_azimuz_bins, p_polar_bins, p_conv_weights,
+                                     return_proj=keep)
+        out, proj = out if keep else (out, None)
         ctx.save_for_backward(p_pts, p_features, p_samples, p_neighbors, p_start_ids, p_radii, p_radial_bins,
                               p_azimuz_bins, p_polar_bins, p_conv_weights, proj)
         return out

@@ -114,6 +114,13 @@ _LANDINGS = []
 SPIN_LIMIT = 100000
 
 
+def set_fused_forward(on):
+    """``set_fused_forward(True)``: forward convolutions that do not return their projection keep it on chip when the
+    shape allows it (one kernel from the gather to the output).  Off by default - the two-kernel path is the faster
+    one on MI355X.  Returns the previous setting.  Process-wide."""
+    return bool(_lib.load().pccnn_set_fused_forward(1 if on else 0))
+
+
 def _keep_until_written(landing, done):
     _LANDINGS.append((landing, done))
     if len(_LANDINGS) > 8:
@@ -770,10 +777,11 @@ def _conv_dims(pts, name, only_3d=False):
     return d
 
 
-def _forward_workspace(pts, m, t, c_in, k, c_out, dev):
-    """(pointer, bytes) of the forward call's workspace: only clouds that are not 3-D need one, for the per-pair
-    basis (the projection is an output tensor here).  Returns the tensor too, to keep it alive over the call."""
-    if pts is None or pts.shape[1] == 3:
+def _forward_workspace(pts, m, t, c_in, k, c_out, dev, keep_proj=True):
+    """(pointer, bytes) of the forward call's workspace: clouds that are not 3-D need one for the per-pair basis, and
+    a call that does not keep the projection needs one for it (or, when the library keeps the projection on chip,
+    for the repacked weights).  Returns the tensor too, to keep it alive over the call."""
+    if keep_proj and (pts is None or pts.shape[1] == 3):
         return _P(0), 0, None
     ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 0), dev)
     return _ptr(ws), ws.numel(), ws
@@ -841,27 +849,28 @@ def kp_conv(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, weights,
         raise RuntimeError(name + ": weights must be [K*Cin, Cout] and kernel_pts [K, D]")
     if bf16:
         desc = _basis(BASIS_KP, k, a=kernel_pts, sigma=sigma)
-        out, proj = _bf16_forward(name, desc, pts, feats, samples, neigh, ends, radii, weights, k, 1, c_out)
+        out, proj = _bf16_forward(name, desc, pts, feats, samples, neigh, ends, radii, weights, k, 1, c_out,
+                                  return_proj)
         return (out, proj) if return_proj else out
     out = torch.empty((m, c_out), dtype=torch.float32, device=dev)
-    proj = torch.empty((m, c_in, k), dtype=torch.float32, device=dev)
-    ws_p, ws_n, _ws = _forward_workspace(pts, m, t, c_in, k, c_out, dev)
+    proj = torch.empty((m, c_in, k), dtype=torch.float32, device=dev) if return_proj else None
+    ws_p, ws_n, _ws = _forward_workspace(pts, m, t, c_in, k, c_out, dev, return_proj)
     _lib.call("pccnn_kpconv_forward", _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends), _ptr(radii),
-              _ptr(kernel_pts), float(sigma), _ptr(weights), n, m, t, d, c_in, k, c_out, _ptr(out), _ptr(proj),
+              _ptr(kernel_pts), float(sigma), _ptr(weights), n, m, t, d, c_in, k, c_out, _ptr(out), _optr(proj),
               ws_p, ws_n, _stream())
     return (out, proj) if return_proj else out
 
 
-def _bf16_forward(name, desc, pts, feats, samples, neigh, ends, radii, weights, k, num_mlps, c_out):
-    """Forward call with the contraction operands in bf16; returns (out f32[M,Cout], proj bf16[M,Cin,K])."""
+def _bf16_forward(name, desc, pts, feats, samples, neigh, ends, radii, weights, k, num_mlps, c_out, keep_proj=True):
+    """Forward call with the contraction operands in bf16; returns (out f32[M,Cout], proj bf16[M,Cin,K] or None)."""
     dev = feats.device
     n, m, t, c_in = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1]
     out = torch.empty((m, c_out), dtype=torch.float32, device=dev)
-    proj = torch.empty((m, c_in, k), dtype=torch.bfloat16, device=dev)
+    proj = torch.empty((m, c_in, k), dtype=torch.bfloat16, device=dev) if keep_proj else None
     ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 0), dev)
     _lib.call("pccnn_conv_forward_bf16", ctypes.byref(desc), _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh),
               _ptr(ends), _ptr(radii), _ptr(weights), n, m, t, _dims_of(pts), c_in, num_mlps, c_out, 0, _ptr(out),
-              _ptr(proj), _ptr(ws), ws.numel(), _stream())
+              _optr(proj), _ptr(ws), ws.numel(), _stream())
     return out, proj
 
 
@@ -1014,14 +1023,15 @@ def mc_conv(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weights, r
     k, num_mlps, c_out = _mc_args(name, pts, pdf, axis, bias, weights, c_in, d, dev)
     if bf16:
         desc = _basis(BASIS_MLP, k, a=axis, b=bias, pdf=pdf)
-        out, proj = _bf16_forward(name, desc, pts, feats, samples, neigh, ends, radii, weights, k, num_mlps, c_out)
+        out, proj = _bf16_forward(name, desc, pts, feats, samples, neigh, ends, radii, weights, k, num_mlps, c_out,
+                                  return_proj)
         return (out, proj) if return_proj else out
     out = torch.empty((m, c_out), dtype=torch.float32, device=dev)
-    proj = torch.empty((m, c_in, k), dtype=torch.float32, device=dev)
-    ws_p, ws_n, _ws = _forward_workspace(pts, m, t, c_in, k, c_out, dev)
+    proj = torch.empty((m, c_in, k), dtype=torch.float32, device=dev) if return_proj else None
+    ws_p, ws_n, _ws = _forward_workspace(pts, m, t, c_in, k, c_out, dev, return_proj)
     _lib.call("pccnn_mcconv_forward", _ptr(pts), _ptr(pdf), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends),
               _ptr(radii), _ptr(axis), _ptr(bias), _ptr(weights), n, m, t, d, c_in, k, num_mlps, c_out, _ptr(out),
-              _ptr(proj), ws_p, ws_n, _stream())
+              _optr(proj), ws_p, ws_n, _stream())
     return (out, proj) if return_proj else out
 
 
@@ -1122,11 +1132,11 @@ def _generic_forward(name, desc, k, pts, feats, samples, neigh, ends, radii, wei
     if weights.shape[0] != k * c_in:
         raise RuntimeError(name + ": weights must be [K*Cin, Cout]")
     out = torch.empty((m, c_out), dtype=torch.float32, device=dev)
-    proj = torch.empty((m, c_in, k), dtype=torch.float32, device=dev)
-    ws_p, ws_n, _ws = _forward_workspace(pts, m, t, c_in, k, c_out, dev)
+    proj = torch.empty((m, c_in, k), dtype=torch.float32, device=dev) if return_proj else None
+    ws_p, ws_n, _ws = _forward_workspace(pts, m, t, c_in, k, c_out, dev, return_proj)
     _lib.call("pccnn_conv_forward", ctypes.byref(desc), _optr(pts), _ptr(feats), _optr(samples), _ptr(neigh),
               _ptr(ends), _optr(radii), _ptr(weights), n, m, t, _dims_of(pts), c_in, 1, c_out, int(divide_by_count),
-              _ptr(out), _ptr(proj), ws_p, ws_n, _stream())
+              _ptr(out), _optr(proj), ws_p, ws_n, _stream())
     return (out, proj) if return_proj else out
 
 
