@@ -357,7 +357,17 @@ int pccnn_neighborhood_count(const float *pts, const int32_t *batch_ids, int64_t
 #define PCCNN_GRAD_PDF 8
 #define PCCNN_GRAD_PTS 16         /* d_pts and d_samples */
 #define PCCNN_GRAD_ALL 31
+/* A flag beside the groups (not part of PCCNN_GRAD_ALL): run the backward pass without float atomics, so that every
+ * result is bit-identical from run to run.  The reference accumulates with atomics (gpuAtomicAdd,
+ * pccnn_lib_ops/pcconvs/shared/feat_basis_proj_grads.cu:132,146; index_add_, pt_diff.cu:51-80); so does this library
+ * by default, because it is faster.  With the flag, the feature gradient of every pair is stored as a row of its own
+ * and the rows of a point are summed in a fixed order: through `mirror` when it is given, else through a by-point
+ * index of the pair list that the call builds in its workspace (a key sort of the t pairs); d_pts / d_pdf take the
+ * same route, and the basis-parameter partial sums are kept per sample.  3-D (or caller-given basis) only; the
+ * workspace must hold pccnn_conv_workspace_bytes_deterministic(...) bytes. */
+#define PCCNN_GRAD_DETERMINISTIC 32
 size_t pccnn_conv_workspace_bytes(int64_t m, int64_t t, int c_in, int k, int c_out, int backward);
+size_t pccnn_conv_workspace_bytes_deterministic(int64_t n, int64_t m, int64_t t, int c_in, int k, int c_out);
 /* mirror_out i32[t]: index of the pair (point b, sample a) for pair t = (point a, sample b), -1 when absent;
  * *missing_out i32 = number of pairs without a mirror (0 for a symmetric neighborhood). */
 int pccnn_mirror_pairs(const int32_t *neigh, const int32_t *ends, int64_t t, int64_t m, int32_t *mirror_out,

@@ -65,6 +65,7 @@ SIGNATURES = {
     "pccnn_neighborhood_count": (I32, [P, P, I64, I32, P, P, P, I32, I32, P, P, P, P, P, P, P, P, P, I64, P, P, P, P,
                                        I32, P, P, P, SZ, P, SZ, P]),
     "pccnn_conv_workspace_bytes": (SZ, [I64, I64, I32, I32, I32, I32]),
+    "pccnn_conv_workspace_bytes_deterministic": (SZ, [I64, I64, I64, I32, I32, I32]),
     "pccnn_kpconv_forward": (I32, [P, P, P, P, P, P, P, F32, P, I64, I64, I64, I32, I32, I32, I32, P, P, P, SZ, P]),
     "pccnn_set_fused_forward": (I32, [I32]),
     "pccnn_mirror_pairs": (I32, [P, P, I64, I64, P, P, P]),

@@ -489,7 +489,10 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
                                 const float4 wv = *(const float4 *)&w_lds[j][q];
                                 gf += gp[q] * wv.x + gp[q + 1] * wv.y + gp[q + 2] * wv.z + gp[q + 3] * wv.w;
                             }
-                            if (fvalid) unsafeAtomicAdd(&feat_grads[(int64_t)bn[u] * g.c_in + f], gf);
+                            if (fvalid) {
+                                if (g.deterministic) __builtin_nontemporal_store(gf, &feat_grads[(int64_t)(cb + j) * g.c_in + f]);
+                                else unsafeAtomicAdd(&feat_grads[(int64_t)bn[u] * g.c_in + f], gf);
+                            }
                         }
                     }
                 }
@@ -577,11 +580,18 @@ conv_proj_bwd_kernel(ConvGeom g, const float *__restrict__ feats, const float *_
             p1 = pccnn_strided_sum<KPAD>(p1);
             p2 = pccnn_strided_sum<KPAD>(p2);
             if (BasisTraits<BASIS>::axis) p3 = pccnn_strided_sum<KPAD>(p3);
-            float *row = param_partials + (int64_t)(blockIdx.x % PARAM_ROWS) * 256;
             constexpr int COMPS = BasisTraits<BASIS>::axis ? 4 : 3;
-            for (int c = part; c < COMPS; c += PARTS) {
-                const float v = (c == 0) ? p0 : (c == 1) ? p1 : (c == 2) ? p2 : p3;
-                unsafeAtomicAdd(&row[c * 64 + k], v);
+            if (g.deterministic) {
+                // a compact row [component][KPAD] per sample, summed in a fixed order afterwards
+                float *row = param_partials + s * (4 * KPAD);
+                for (int c = part; c < 4; c += PARTS)
+                    row[c * KPAD + k] = (c == 0) ? p0 : (c == 1) ? p1 : (c == 2) ? p2 : (COMPS == 4 ? p3 : 0.0f);
+            } else {
+                float *row = param_partials + (int64_t)(blockIdx.x % PARAM_ROWS) * 256;
+                for (int c = part; c < COMPS; c += PARTS) {
+                    const float v = (c == 0) ? p0 : (c == 1) ? p1 : (c == 2) ? p2 : p3;
+                    unsafeAtomicAdd(&row[c * 64 + k], v);
+                }
             }
         }
     }
@@ -696,7 +706,8 @@ conv_proj_bwd_narrow_kernel(ConvGeom g, const float *__restrict__ feats, const f
                         const float4 wv = *(const float4 *)&w_lds[j][q];
                         gf += gp[q] * wv.x + gp[q + 1] * wv.y + gp[q + 2] * wv.z + gp[q + 3] * wv.w;
                     }
-                    unsafeAtomicAdd(&feat_grads[(int64_t)nidx_lds[j] * g.c_in + f], gf);
+                    if (g.deterministic) feat_grads[(int64_t)(cb + j) * g.c_in + f] = gf;
+                    else unsafeAtomicAdd(&feat_grads[(int64_t)nidx_lds[j] * g.c_in + f], gf);
                 }
             }
         }
@@ -763,11 +774,17 @@ conv_proj_bwd_narrow_kernel(ConvGeom g, const float *__restrict__ feats, const f
             p1 = pccnn_strided_sum<KPAD>(p1);
             p2 = pccnn_strided_sum<KPAD>(p2);
             if (BasisTraits<BASIS>::axis) p3 = pccnn_strided_sum<KPAD>(p3);
-            float *prow = param_partials + (int64_t)(blockIdx.x % PARAM_ROWS) * 256;
             constexpr int COMPS = BasisTraits<BASIS>::axis ? 4 : 3;
-            for (int c = part; c < COMPS; c += PARTS) {
-                const float v = (c == 0) ? p0 : (c == 1) ? p1 : (c == 2) ? p2 : p3;
-                unsafeAtomicAdd(&prow[c * 64 + k], v);
+            if (g.deterministic) {
+                float *prow = param_partials + s * (4 * KPAD);
+                for (int c = part; c < 4; c += PARTS)
+                    prow[c * KPAD + k] = (c == 0) ? p0 : (c == 1) ? p1 : (c == 2) ? p2 : (COMPS == 4 ? p3 : 0.0f);
+            } else {
+                float *prow = param_partials + (int64_t)(blockIdx.x % PARAM_ROWS) * 256;
+                for (int c = part; c < COMPS; c += PARTS) {
+                    const float v = (c == 0) ? p0 : (c == 1) ? p1 : (c == 2) ? p2 : p3;
+                    unsafeAtomicAdd(&prow[c * 64 + k], v);
+                }
             }
         }
     }
@@ -797,9 +814,18 @@ mirror_pairs_kernel(const int2 *__restrict__ neigh, const int32_t *__restrict__ 
 // the pairs of sample n.  Four lanes per point: lane q adds the (x, y, z, density) records of the pairs
 // q, q + 4, ... of the segment (16-byte loads, independent between the lanes), two exchanges add the four
 // partial sums in a fixed order, and lane q stores component q.
+// The pairs of point n are listed in index[lo .. hi): with `starts` == 0 the bounds are the segment of sample n in
+// `bounds` (running totals, the layout of `ends`: the index is the mirror index of a symmetric neighborhood); with
+// `starts` != 0 they are bounds[n] and bounds[n + 1] (the by-point index of conv_by_point_index).
+__device__ __forceinline__ void point_segment(const int32_t *__restrict__ bounds, int starts, int64_t n, int &lo, int &hi)
+{
+    if (starts) { lo = bounds[n]; hi = bounds[n + 1]; }
+    else { lo = n > 0 ? bounds[n - 1] : 0; hi = bounds[n]; }
+}
+
 __global__ void __launch_bounds__(256)
 conv_point_gather_kernel(const float *__restrict__ pair_grads, const int32_t *__restrict__ mirror,
-                         const int32_t *__restrict__ ends, int64_t m, float *__restrict__ d_pts,
+                         const int32_t *__restrict__ ends, int starts, int64_t m, float *__restrict__ d_pts,
                          float *__restrict__ d_pdf)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -807,7 +833,8 @@ conv_point_gather_kernel(const float *__restrict__ pair_grads, const int32_t *__
     const int q = (int)(i & 3);
     float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     if (n < m) {
-        const int lo = n > 0 ? ends[n - 1] : 0, hi = ends[n];
+        int lo, hi;
+        point_segment(ends, starts, n, lo, hi);
         const float4 *rec = (const float4 *)pair_grads;
         for (int j = lo + q; j < hi; j += 4) {
             const float4 v = rec[mirror[j]];
@@ -830,27 +857,134 @@ conv_point_gather_kernel(const float *__restrict__ pair_grads, const int32_t *__
     }
 }
 
+// d_feats[n][:] = sum of the per-pair rows rows[index[j]][:] over the pairs j of point n (bounds as in
+// conv_point_gather_kernel), in the order of the index: the feature gradients without atomics.  LANES lanes per
+// point (the row width rounded up to a power of two, at most 64); wider rows in blocks of 64 features.
+template <int LANES>
+__global__ void __launch_bounds__(256)
+conv_rows_gather_kernel(const float *__restrict__ rows, const int32_t *__restrict__ index,
+                        const int32_t *__restrict__ bounds, int starts, int64_t n_points, int c_in,
+                        float *__restrict__ d_feats)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t n = i / LANES;
+    const int l = (int)(i % LANES);
+    if (n >= n_points) return;
+    int lo, hi;
+    point_segment(bounds, starts, n, lo, hi);
+    for (int f = l; f < c_in; f += LANES) {
+        float acc = 0.0f;
+        int j = lo;
+        for (; j + 4 <= hi; j += 4) {
+            const float v0 = rows[(int64_t)index[j] * c_in + f], v1 = rows[(int64_t)index[j + 1] * c_in + f];
+            const float v2 = rows[(int64_t)index[j + 2] * c_in + f], v3 = rows[(int64_t)index[j + 3] * c_in + f];
+            acc += v0;
+            acc += v1;
+            acc += v2;
+            acc += v3;
+        }
+        for (; j < hi; ++j) acc += rows[(int64_t)index[j] * c_in + f];
+        d_feats[n * c_in + f] = acc;
+    }
+}
+
+__global__ void __launch_bounds__(256)
+pair_point_keys_kernel(const int2 *__restrict__ neigh, int64_t t, int64_t *__restrict__ keys)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < t) keys[i] = neigh[i].x;
+}
+
+// The pair list by point, for a neighborhood without a mirror index: order_out i32[t] lists the pairs sorted by
+// their point (pairs of one point in ascending pair index: the sort is stable), starts_out i32[n + 1] the first
+// entry of every point.  Workspace: two i64[t] key arrays and the sort's own.
+static size_t by_point_index_bytes(int64_t n, int64_t t)
+{
+    return 2 * pccnn_align((size_t)t * sizeof(int64_t)) + pccnn_align(pccnn_sort_keys_workspace_bytes(t)) +
+           pccnn_align((size_t)t * sizeof(int32_t)) + pccnn_align(((size_t)n + 1) * sizeof(int32_t));
+}
+
+static int conv_by_point_index(const int2 *neigh, int64_t n, int64_t t, int32_t *order_out, int32_t *starts_out,
+                               PccnnArena &arena, hipStream_t s)
+{
+    int64_t *keys = arena.take<int64_t>((size_t)t);
+    int64_t *sorted = arena.take<int64_t>((size_t)t);
+    const size_t sort_bytes = pccnn_sort_keys_workspace_bytes(t);
+    void *sort_ws = arena.take<char>(sort_bytes);
+    PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv backward: workspace too small for the by-point pair index");
+    pair_point_keys_kernel<<<(unsigned)pccnn_ceil_div(t, 256), 256, 0, s>>>(neigh, t, keys);
+    PCCNN_LAUNCH_CHECK();
+    int bits = 1;
+    while (bits < 62 && (1ll << bits) < n) ++bits;
+    int rc = pccnn_sort_keys(keys, t, bits, sorted, order_out, nullptr, 3, nullptr, sort_ws, sort_bytes, s);
+    if (rc != PCCNN_OK) return rc;
+    return pccnn_build_cell_table(sorted, t, n, starts_out, s);
+}
+
 // Sums partial rows ([rows][256], column = component * 64 + basis index) in a fixed order.
 // Stage 1: workgroup b adds the rows b, b + G, b + 2G, ... (thread = column, coalesced); stage 2: one
 // workgroup adds the G stage-1 rows and writes every value to its place in the parameter gradient tensors.
 #define PARAM_REDUCE_GROUPS 64
+#define PARAM_REDUCE_GROUPS_PER_SAMPLE 128      // first-stage groups when every sample wrote a partial row
 
 __global__ void __launch_bounds__(256)
 conv_param_reduce1_kernel(const float *__restrict__ partials, int64_t rows, float *__restrict__ stage)
 {
     float acc = 0.0f;
-    for (int64_t r = blockIdx.x; r < rows; r += PARAM_REDUCE_GROUPS) acc += partials[r * 256 + threadIdx.x];
+    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) acc += partials[r * 256 + threadIdx.x];
     stage[(int64_t)blockIdx.x * 256 + threadIdx.x] = acc;
+}
+
+// The same first stage over compact per-sample rows [4][kpad] (the pass without atomics): column c * 64 + k of the
+// stage row comes from entry c * kpad + k.  Workgroup b sums a contiguous run of rows; its 256 threads cover
+// 256 / (4 kpad) rows at a time (thread = (row lane, entry)), eight loads in flight each, and the row lanes meet in
+// LDS - a fixed order throughout.
+__global__ void __launch_bounds__(256)
+conv_param_reduce1_compact_kernel(const float *__restrict__ partials, int64_t rows, int kpad, float *__restrict__ stage)
+{
+    __shared__ float part[256];
+    const int width = 4 * kpad;                         // 32 .. 256 entries per row
+    const int lanes = 256 / width;
+    const int col = threadIdx.x % width, lane = threadIdx.x / width;
+    const int64_t per = (rows + gridDim.x - 1) / gridDim.x;
+    const int64_t r0 = (int64_t)blockIdx.x * per;
+    const int64_t r1 = r0 + per < rows ? r0 + per : rows;
+    float acc = 0.0f;
+    int64_t r = r0 + lane;
+    for (; r + 7 * lanes < r1; r += 8 * lanes) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = partials[(r + (int64_t)u * lanes) * width + col];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc += v[u];
+    }
+    for (; r < r1; r += lanes) acc += partials[r * width + col];
+    part[threadIdx.x] = acc;
+    __syncthreads();
+    // thread t writes stage column t = c * 64 + k
+    const int c = threadIdx.x >> 6, k = threadIdx.x & 63;
+    float total = 0.0f;
+    if (k < kpad)
+        for (int l = 0; l < lanes; ++l) total += part[l * width + c * kpad + k];
+    stage[(int64_t)blockIdx.x * 256 + threadIdx.x] = total;
 }
 
 template <int BASIS>
 __global__ void __launch_bounds__(256)
-conv_param_reduce2_kernel(const float *__restrict__ stage, int k_basis, float *__restrict__ dst_a,
+conv_param_reduce2_kernel(const float *__restrict__ stage, int groups, int k_basis, float *__restrict__ dst_a,
                           float *__restrict__ dst_b)
 {
     const int comp = threadIdx.x >> 6, kk = threadIdx.x & 63;
     float acc = 0.0f;
-    for (int r = 0; r < PARAM_REDUCE_GROUPS; ++r) acc += stage[r * 256 + threadIdx.x];
+    int r = 0;
+    for (; r + 8 <= groups; r += 8) {                   // eight loads in flight, added in order
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = stage[(r + u) * 256 + threadIdx.x];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc += v[u];
+    }
+    for (; r < groups; ++r) acc += stage[r * 256 + threadIdx.x];
     if (kk < k_basis && dst_a) {
         if (BasisTraits<BASIS>::kernel_pts) {
             if (comp < 3) dst_a[kk * 3 + comp] = acc;               // d_kernel_pts [K,3]
@@ -1148,6 +1282,16 @@ extern "C" size_t pccnn_conv_workspace_bytes(int64_t m, int64_t t, int c_in, int
     return 2 * proj + basis_g + splitk + partials + scaled + pair_g + w16 + g16 + pair_b + 256;
 }
 
+extern "C" size_t pccnn_conv_workspace_bytes_deterministic(int64_t n, int64_t m, int64_t t, int c_in, int k, int c_out)
+{
+    if (n < 1) n = 1;
+    if (m < 1) m = 1;
+    if (t < 1) t = 1;
+    return pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1) +
+           pccnn_align(((size_t)m + PARAM_REDUCE_GROUPS_PER_SAMPLE) * 256 * sizeof(float)) +
+           pccnn_align((size_t)t * c_in * sizeof(float)) + by_point_index_bytes(n, t) + 256;
+}
+
 // out[m, c_out] = P[m, c_in*k] x W, with the feature axis split over num_mlps independent
 // weight blocks (num_mlps == 1 is the plain product).
 // Split of the sample dimension for d_weights = P^T x dOut, whose output ([K*Cin, Cout]) has few tiles: enough
@@ -1293,17 +1437,32 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     const bool want_pdf = (mask & PCCNN_GRAD_PDF) && Tr::pdf_grad;
     const bool want_basis = want_par || want_pts || want_pdf;
     int rc;
+    // PCCNN_GRAD_DETERMINISTIC: no float atomics anywhere in the pass.  Feature gradients go to one row per pair
+    // and are summed per point in the order of the mirror index (symmetric neighborhoods) or of a by-point index of
+    // the pair list built here; the point-side gradients take the same route; every sample writes its own
+    // basis-parameter partial row.
+    const bool det = (mask & PCCNN_GRAD_DETERMINISTIC) != 0 && g.m > 0 && g.t > 0;
+    // The per-pair rows and their gather are also the faster way to the feature gradients when they are all the
+    // projection pass has to produce, the rows are wide and a mirror index is at hand (65 536 samples, 0.92 M pairs,
+    // 64 features: feature + weight gradients in 480 instead of 512 us); taken when the workspace has the room.
+    const bool rows_auto = !det && mirror != nullptr && want_f && !want_basis && g.c_in > 32 && g.m > 0 && g.t > 0 &&
+                           workspace_bytes >= pccnn_conv_workspace_bytes_deterministic(g.n, g.m, g.t, g.c_in, g.k, c_out);
+    const bool rows_route = det || rows_auto;
+    g.deterministic = rows_route ? 1 : 0;
     PccnnArena arena(workspace, workspace_bytes);
-    const int64_t partial_rows = PARAM_ROWS;
-    float *partials = arena.take<float>((size_t)(partial_rows + PARAM_REDUCE_GROUPS) * 256);
+    const int64_t partial_rows = det ? g.m : PARAM_ROWS;
+    const int reduce_groups = det ? PARAM_REDUCE_GROUPS_PER_SAMPLE : PARAM_REDUCE_GROUPS;
+    float *partials = arena.take<float>((size_t)(partial_rows + reduce_groups) * 256);
     float *stage = partials + partial_rows * 256;
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv backward: workspace of %zu bytes, need %zu", workspace_bytes,
-                  pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 1));
-    // with a mirror index the point-side gradients are written once per point, not accumulated
-    const bool gather = mirror != nullptr && Tr::differentiable && (want_pts || want_pdf) && g.m > 0 && g.t > 0;
+                  det ? pccnn_conv_workspace_bytes_deterministic(g.n, g.m, g.t, g.c_in, g.k, c_out)
+                      : pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 1));
+    // with a mirror index (or, in the deterministic pass, the by-point index) the point-side gradients are
+    // written once per point, not accumulated
+    const bool gather = (mirror != nullptr || det) && Tr::differentiable && (want_pts || want_pdf) && g.m > 0 && g.t > 0;
     // the accumulators to clear; the launch follows below, together with the bf16 copies
     ConvPrepJobs prep = {};
-    if (want_f) { prep.zero[0] = d_feats; prep.zero_count[0] = g.n * g.c_in; }
+    if (want_f && !rows_route) { prep.zero[0] = d_feats; prep.zero_count[0] = g.n * g.c_in; }
     if (want_pts && !gather) { prep.zero[1] = d_pts; prep.zero_count[1] = g.n * 3; }
     if (want_pdf && !gather) { prep.zero[2] = d_pdf; prep.zero_count[2] = g.n; }
     if (g.m == 0 || g.t == 0) {
@@ -1327,8 +1486,22 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     uint16_t *w16 = bf16 ? arena.take<uint16_t>((size_t)w_count) : nullptr;
     uint16_t *g16 = bf16 ? arena.take<uint16_t>((size_t)g.m * c_out) : nullptr;
     if (BASIS == BASIS_EXPLICIT && want_par) basis_g = d_param_a;    // the basis gradient is itself an output
+    // deterministic pass: per-pair feature-gradient rows, and the pairs listed by point
+    float *df_rows = (rows_route && want_f) ? arena.take<float>((size_t)g.t * g.c_in) : nullptr;
+    const int32_t *by_point = mirror, *by_point_bounds = g.ends;
+    int by_point_starts = 0;
+    const bool need_index = det && mirror == nullptr && (want_f || gather);
+    int32_t *order = need_index ? arena.take<int32_t>((size_t)g.t) : nullptr;
+    int32_t *starts = need_index ? arena.take<int32_t>((size_t)g.n + 1) : nullptr;
     PCCNN_REQUIRE(arena.ok(), PCCNN_ERR_WORKSPACE, "conv backward: workspace of %zu bytes, need %zu", workspace_bytes,
-                  pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 1));
+                  det ? pccnn_conv_workspace_bytes_deterministic(g.n, g.m, g.t, g.c_in, g.k, c_out)
+                      : pccnn_conv_workspace_bytes(g.m, g.t, g.c_in, g.k, c_out, 1));
+    if (need_index) {
+        if ((rc = conv_by_point_index(g.neigh, g.n, g.t, order, starts, arena, s)) != PCCNN_OK) return rc;
+        by_point = order;
+        by_point_bounds = starts;
+        by_point_starts = 1;
+    }
     const int64_t inner = (int64_t)g.c_in * g.k / num_mlps;
     const int64_t co = c_out / num_mlps;
     if (divide_by_count) {
@@ -1339,7 +1512,8 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     }
     const bool with_projection_pass = want_f || want_basis;
     const bool with_partials = with_projection_pass && want_par && Tr::differentiable;
-    if (with_partials) { prep.zero[3] = partials; prep.zero_count[3] = partial_rows * 256; }
+    // (the deterministic pass stores a partial row per sample instead of adding into shared ones)
+    if (with_partials && !det) { prep.zero[3] = partials; prep.zero_count[3] = partial_rows * 256; }
     if (bf16) {
         prep.src[0] = in_grads; prep.dst[0] = g16; prep.convert_count[0] = g.m * c_out;
         if (with_projection_pass) { prep.src[1] = weights; prep.dst[1] = w16; prep.convert_count[1] = w_count; }
@@ -1375,17 +1549,31 @@ static int conv_backward(ConvGeom g, const float *feats, const float *weights, c
     if (rc != PCCNN_OK) return rc;
     BasisGradOut o = {basis_g, want_pts ? d_pts : nullptr, want_pts ? d_samples : nullptr, want_pdf ? d_pdf : nullptr,
                       (want_par && Tr::differentiable) ? partials : nullptr, gather ? pair_grads : nullptr};
-    if ((rc = launch_proj_bwd<BASIS>(g, feats, d_proj, want_f ? d_feats : nullptr, want_basis, o, s)) != PCCNN_OK)
+    if ((rc = launch_proj_bwd<BASIS>(g, feats, d_proj, want_f ? (rows_route ? df_rows : d_feats) : nullptr, want_basis, o,
+                                     s)) != PCCNN_OK)
         return rc;
+    if (rows_route && want_f) {
+        const int lanes = g.c_in <= 8 ? 8 : (g.c_in <= 16 ? 16 : (g.c_in <= 32 ? 32 : 64));
+        const unsigned blocks = (unsigned)pccnn_ceil_div(g.n * lanes, 256);
+#define ROWS_GO(L) conv_rows_gather_kernel<L><<<blocks, 256, 0, s>>>(df_rows, by_point, by_point_bounds, \
+                                                                     by_point_starts, g.n, g.c_in, d_feats)
+        if (lanes == 8) ROWS_GO(8);
+        else if (lanes == 16) ROWS_GO(16);
+        else if (lanes == 32) ROWS_GO(32);
+        else ROWS_GO(64);
+#undef ROWS_GO
+        PCCNN_LAUNCH_CHECK();
+    }
     if (gather) {
-        conv_point_gather_kernel<<<(unsigned)pccnn_ceil_div(g.m * 4, 256), 256, 0, s>>>(pair_grads, mirror, g.ends, g.m,
-                                                                                        o.d_pts, o.d_pdf);
+        conv_point_gather_kernel<<<(unsigned)pccnn_ceil_div(g.n * 4, 256), 256, 0, s>>>(
+            pair_grads, by_point, by_point_bounds, by_point_starts, g.n, o.d_pts, o.d_pdf);
         PCCNN_LAUNCH_CHECK();
     }
     if (o.partials) {
-        conv_param_reduce1_kernel<<<PARAM_REDUCE_GROUPS, 256, 0, s>>>(partials, partial_rows, stage);
+        if (det) conv_param_reduce1_compact_kernel<<<reduce_groups, 256, 0, s>>>(partials, partial_rows, kpad_of(g.k), stage);
+        else conv_param_reduce1_kernel<<<reduce_groups, 256, 0, s>>>(partials, partial_rows, stage);
         PCCNN_LAUNCH_CHECK();
-        conv_param_reduce2_kernel<BASIS><<<1, 256, 0, s>>>(stage, g.k, d_param_a, d_param_b);
+        conv_param_reduce2_kernel<BASIS><<<1, 256, 0, s>>>(stage, reduce_groups, g.k, d_param_a, d_param_b);
         PCCNN_LAUNCH_CHECK();
     }
     return PCCNN_OK;
@@ -1913,6 +2101,8 @@ static int conv_backward_entry(const char *who, bool bf16, const pccnn_basis *ba
     if (d != 3 && geom) {
         PCCNN_REQUIRE(pair_basis_kind(kind), PCCNN_ERR_UNSUPPORTED, "%s: basis kind %d needs 3 dimensions (d=%d)", who,
                       kind, d);
+        PCCNN_REQUIRE(!(grad_mask & PCCNN_GRAD_DETERMINISTIC), PCCNN_ERR_UNSUPPORTED,
+                      "%s: the pass without atomics (PCCNN_GRAD_DETERMINISTIC) is three-dimensional, d=%d", who, d);
         hipStream_t s = (hipStream_t)stream;
         const bool want_par = grad_mask & PCCNN_GRAD_BASIS_PARAMS, want_pts = grad_mask & PCCNN_GRAD_PTS;
         const bool want_pdf = (grad_mask & PCCNN_GRAD_PDF) && has_pdf;
@@ -2075,7 +2265,7 @@ extern "C" int pccnn_linear_basis_backward(const float *pts, const float *sample
     PCCNN_LAUNCH_CHECK();
     conv_param_reduce1_kernel<<<PARAM_REDUCE_GROUPS, 256, 0, s>>>(partials, blocks, stage);
     PCCNN_LAUNCH_CHECK();
-    conv_param_reduce2_kernel<BASIS_MLP><<<1, 256, 0, s>>>(stage, k, d_axis, d_bias);
+    conv_param_reduce2_kernel<BASIS_MLP><<<1, 256, 0, s>>>(stage, PARAM_REDUCE_GROUPS, k, d_axis, d_bias);
     PCCNN_LAUNCH_CHECK();
     return PCCNN_OK;
 }

@@ -38,6 +38,9 @@ struct ConvGeom {
     int c_in, k;
     const float *basis_c;   // polar bin edges
     int nb0, nb1, nb2;      // spherical bin counts
+    // Backward pass without float atomics: the feature-gradient row of a pair is stored at the pair's index (and
+    // summed per point afterwards), and every sample writes a basis-parameter partial row of its own.
+    int deterministic;
 };
 
 // First bin whose upper edge is >= v, the last bin when there is none.

@@ -402,7 +402,14 @@ void generic_backward(const std::string &name, const Generic &g, const Tensor &w
     TORCH_CHECK(in_grads.size(0) == m && in_grads.size(1) == c_out, name, ": in_grads must be [M, Cout]");
     const void *proj_p = proj_arg(name, proj, m, c_in, g.k, g.feats, bf16);
     const int32_t *mirror_p = g.pts ? mirror_arg(name, mirror, g.neigh, n, m) : nullptr;
-    Tensor ws = workspace(pccnn_conv_workspace_bytes(m, t, c_in, g.k, (int)c_out, 1), g.feats);
+    // the larger workspace when the pass without atomics is asked for, and when the library may take the per-pair
+    // rows by itself (a mirror index, wide rows, no basis / position / density gradients)
+    const bool rows_route = mirror_p != nullptr && c_in > 32 && (grad_mask & PCCNN_GRAD_FEATS) &&
+                            !(grad_mask & (PCCNN_GRAD_BASIS_PARAMS | PCCNN_GRAD_PDF | PCCNN_GRAD_PTS));
+    Tensor ws = workspace(((grad_mask & PCCNN_GRAD_DETERMINISTIC) || rows_route)
+                              ? pccnn_conv_workspace_bytes_deterministic(n, m, t, c_in, g.k, (int)c_out)
+                              : pccnn_conv_workspace_bytes(m, t, c_in, g.k, (int)c_out, 1),
+                          g.feats);
     const float *pts = g.pts ? fptr(*g.pts) : nullptr, *smp = g.samples ? fptr(*g.samples) : nullptr,
                 *rad = g.radii ? fptr(*g.radii) : nullptr;
     if (bf16)
@@ -653,7 +660,7 @@ py::list sph_conv_grads(const Tensor &pts, const Tensor &feats, const Tensor &sa
     Generic g = sph_args("sph_conv_grads", pts, feats, samples, neigh, ends, radii, radial, azimuth, polar);
     chk(weights, "sph_conv_grads: weights", at::kFloat, 2, &pts);
     TORCH_CHECK(weights.size(0) == (int64_t)g.k * feats.size(1), "sph_conv_grads: inconsistent shapes");
-    const int mask = (int)grad_mask & (PCCNN_GRAD_WEIGHTS | PCCNN_GRAD_FEATS);
+    const int mask = (int)grad_mask & (PCCNN_GRAD_WEIGHTS | PCCNN_GRAD_FEATS | PCCNN_GRAD_DETERMINISTIC);
     Grads gr;
     gr.d_w = like_if(weights, mask, PCCNN_GRAD_WEIGHTS);
     gr.d_f = like_if(feats, mask, PCCNN_GRAD_FEATS);
@@ -765,7 +772,8 @@ py::list point_conv_grads(const Tensor &basis, const Tensor &feats, const Tensor
     Generic g = explicit_args("point_conv_grads", basis, feats, neigh, ends);
     chk(weights, "point_conv_grads: weights", at::kFloat, 2, &basis);
     TORCH_CHECK(weights.size(0) == (int64_t)g.k * feats.size(1), "point_conv_grads: inconsistent shapes");
-    const int mask = (int)grad_mask & (PCCNN_GRAD_WEIGHTS | PCCNN_GRAD_FEATS | PCCNN_GRAD_BASIS_PARAMS);
+    const int mask = (int)grad_mask & (PCCNN_GRAD_WEIGHTS | PCCNN_GRAD_FEATS | PCCNN_GRAD_BASIS_PARAMS |
+                                      PCCNN_GRAD_DETERMINISTIC);
     Grads gr;
     gr.d_w = like_if(weights, mask, PCCNN_GRAD_WEIGHTS);
     gr.d_f = like_if(feats, mask, PCCNN_GRAD_FEATS);
@@ -916,6 +924,7 @@ PYBIND11_MODULE(pccnn_lib_ops, mod)
     mod.attr("GRAD_PDF") = PCCNN_GRAD_PDF;
     mod.attr("GRAD_PTS") = PCCNN_GRAD_PTS;
     mod.attr("GRAD_ALL") = PCCNN_GRAD_ALL;
+    mod.attr("GRAD_DETERMINISTIC") = PCCNN_GRAD_DETERMINISTIC;
     mod.attr("REFERENCE_NAMES") = py::make_tuple(
         "build_grid_ds", "compute_keys", "find_neighbors", "compute_pdf", "compute_pdf_grads", "poisson_disk_sampling",
         "mc_conv", "mc_conv_grads", "mc_conv_weight_var", "point_conv_basis", "point_conv_basis_grads", "point_conv",

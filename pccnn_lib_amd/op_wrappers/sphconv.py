@@ -30,7 +30,7 @@ class ComputeSPHConv(ConvFunction):
         mask = (ops.GRAD_FEATS if need[1] else 0) | (ops.GRAD_WEIGHTS if need[9] else 0)
         weight_grads, feat_grads = ops.sph_conv_grads(
             pts, features, samples, neighbors, start_ids, radii, radial_bins, azimuz_bins, polar_bins, conv_weights,
-            p_grads, proj=proj, grad_mask=mask)
+            p_grads, proj=proj, grad_mask=mask | pccnn_lib_ops.deterministic_flag())
         return None, feat_grads, None, None, None, None, None, None, None, weight_grads
 
 

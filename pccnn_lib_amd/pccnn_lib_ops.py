@@ -766,6 +766,33 @@ def pool_poisson_later(pts, batch_ids, aabb_min, cell_size, num_cells_host, batc
 
 # Gradient groups of the backward entry points (PCCNN_GRAD_* in include/pccnn_hip.h).
 GRAD_WEIGHTS, GRAD_FEATS, GRAD_BASIS_PARAMS, GRAD_PDF, GRAD_PTS, GRAD_ALL = 1, 2, 4, 8, 16, 31
+# Flag beside the groups: the backward pass without float atomics (bit-identical results from run to run, slower).
+GRAD_DETERMINISTIC = 32
+
+_deterministic = False
+
+
+def set_deterministic(on):
+    """``set_deterministic(True)``: the autograd wrappers ask the backward calls for the pass without float atomics
+    (``GRAD_DETERMINISTIC``), so gradients are bit-identical from run to run.  Returns the previous setting."""
+    global _deterministic
+    before, _deterministic = _deterministic, bool(on)
+    return before
+
+
+def deterministic_flag():
+    """``GRAD_DETERMINISTIC`` while ``set_deterministic(True)`` is in force, else 0: OR it into a grad_mask."""
+    return GRAD_DETERMINISTIC if _deterministic else 0
+
+
+def _backward_workspace(n, m, t, c_in, k, c_out, grad_mask, dev, mirror=None):
+    """Workspace of a backward call: the larger one when the pass without atomics is asked for, and when the library
+    may take the per-pair rows by itself (a mirror index, wide rows, no basis / position / density gradients)."""
+    lib = _lib.load()
+    rows_route = mirror is not None and c_in > 32 and not (grad_mask & (GRAD_BASIS_PARAMS | GRAD_PDF | GRAD_PTS))
+    if grad_mask & GRAD_DETERMINISTIC or (rows_route and grad_mask & GRAD_FEATS):
+        return _workspace(lib.pccnn_conv_workspace_bytes_deterministic(n, m, t, c_in, k, c_out), dev)
+    return _workspace(lib.pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
 
 
 
@@ -879,7 +906,7 @@ def _bf16_backward(name, desc, pts, feats, samples, neigh, ends, radii, weights,
     dev = feats.device
     n, m, t, c_in = pts.shape[0], samples.shape[0], neigh.shape[0], feats.shape[1]
     proj_p = _conv_proj_arg(name, proj, m, c_in, k, dev, bf16=True)
-    ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
+    ws = _backward_workspace(n, m, t, c_in, k, c_out, grad_mask, dev, mirror)
     _lib.call("pccnn_conv_backward_bf16", ctypes.byref(desc), _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh),
               _ptr(ends), _ptr(radii), _ptr(weights), _ptr(in_grads), proj_p,
               _mirror_arg(name, mirror, neigh, pts, samples), grad_mask, n, m, t, _dims_of(pts), c_in, num_mlps, c_out, 0,
@@ -964,7 +991,7 @@ def kp_conv_grads(pts, feats, samples, neigh, ends, radii, kernel_pts, sigma, we
                        k, 1, c_out, d_w, d_f, d_kp, None, None, d_p, d_s)
         return [d_w, d_f, d_kp, d_p, d_s]
     proj_p = _conv_proj_arg(name, proj, m, c_in, k, dev)
-    ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
+    ws = _backward_workspace(n, m, t, c_in, k, c_out, grad_mask, dev, mirror)
     _lib.call("pccnn_kpconv_backward", _ptr(pts), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends), _ptr(radii),
               _ptr(kernel_pts), float(sigma), _ptr(weights), _ptr(in_grads), proj_p,
               _mirror_arg(name, mirror, neigh, pts, samples), grad_mask, n, m, t, d, c_in, k,
@@ -1062,7 +1089,7 @@ def mc_conv_grads(pts, pdf, feats, samples, neigh, ends, radii, axis, bias, weig
                        k, num_mlps, c_out, d_w, d_f, d_axis, d_bias, d_pdf, d_p, d_s)
         return [d_w, d_f, d_axis, d_bias, d_pdf, d_p, d_s]
     proj_p = _conv_proj_arg(name, proj, m, c_in, k, dev)
-    ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
+    ws = _backward_workspace(n, m, t, c_in, k, c_out, grad_mask, dev, mirror)
     _lib.call("pccnn_mcconv_backward", _ptr(pts), _ptr(pdf), _ptr(feats), _ptr(samples), _ptr(neigh), _ptr(ends),
               _ptr(radii), _ptr(axis), _ptr(bias), _ptr(weights), _ptr(in_grads), proj_p,
               _mirror_arg(name, mirror, neigh, pts, samples), grad_mask, n, m, t, d, c_in, k, num_mlps, c_out, _optr(d_w), _optr(d_f), _optr(d_axis), _optr(d_bias), _optr(d_pdf), _optr(d_p),
@@ -1154,7 +1181,7 @@ def _generic_backward(name, desc, k, pts, feats, samples, neigh, ends, radii, we
     d_p = torch.empty_like(pts) if with_pts and grad_mask & GRAD_PTS else None
     d_s = torch.empty_like(samples) if with_pts and grad_mask & GRAD_PTS else None
     proj_p = _conv_proj_arg(name, proj, m, c_in, k, dev)
-    ws = _workspace(_lib.load().pccnn_conv_workspace_bytes(m, t, c_in, k, c_out, 1), dev)
+    ws = _backward_workspace(n, m, t, c_in, k, c_out, grad_mask, dev, mirror)
     _lib.call("pccnn_conv_backward", ctypes.byref(desc), _optr(pts), _ptr(feats), _optr(samples), _ptr(neigh),
               _ptr(ends), _optr(radii), _ptr(weights), _ptr(in_grads), proj_p,
               _mirror_arg(name, mirror, neigh, pts, samples) if with_pts else _P(0), grad_mask, n, m, t, _dims_of(pts), c_in, 1,
@@ -1294,7 +1321,7 @@ def sph_conv_grads(pts, feats, samples, neigh, ends, radii, radial_bins, azimuth
     name = "sph_conv_grads"
     k, desc = _sph_args(name, pts, feats, samples, neigh, ends, radii, radial_bins, azimuth_bins, polar_bins)
     d_w, d_f, _, _ = _generic_backward(name, desc, k, pts, feats, samples, neigh, ends, radii, weights, in_grads,
-                                       proj, int(grad_mask) & (GRAD_WEIGHTS | GRAD_FEATS), True, with_pts=False)
+                                       proj, int(grad_mask) & (GRAD_WEIGHTS | GRAD_FEATS | GRAD_DETERMINISTIC), True, with_pts=False)
     return [d_w, d_f]
 
 
@@ -1383,7 +1410,7 @@ def point_conv_grads(basis, feats, neigh, ends, weights, in_grads, proj=None, gr
     k, desc = _explicit_args(name, basis, feats, neigh, ends)
     d_b = torch.empty_like(basis) if int(grad_mask) & GRAD_BASIS_PARAMS else None
     d_w, d_f, _, _ = _generic_backward(name, desc, k, None, feats, None, neigh, ends, None, weights, in_grads, proj,
-                                       int(grad_mask) & (GRAD_WEIGHTS | GRAD_FEATS | GRAD_BASIS_PARAMS), False,
+                                       int(grad_mask) & (GRAD_WEIGHTS | GRAD_FEATS | GRAD_BASIS_PARAMS | GRAD_DETERMINISTIC), False,
                                        d_param_a=d_b, with_pts=False)
     return [d_w, d_f, d_b]
 
