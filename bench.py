@@ -448,10 +448,31 @@ def main():
         return torch.autograd.grad(out, leaves, out_grads)
 
     def conv_step_fw_only():
-        # gradients w.r.t. features and weights only (the gradient set config 2 names)
+        # gradients w.r.t. features and weights only (the gradient set config 2 names); with the neighborhood's
+        # mirror index at hand the feature gradients go through per-pair rows and a gather instead of atomics
         f, w = leaves[2], leaves[5]
-        out = ComputeMCConv.apply(pts, pdf, f, pts, neigh, ends, radii, axis, bias, w)
+        out = ComputeMCConv.apply(pts, pdf, f, pts, neigh, ends, radii, axis, bias, w, mirror)
         return torch.autograd.grad(out, [f, w], out_grads)
+
+    def conv_step_deterministic():
+        # the headline step with the backward pass that uses no float atomics (bit-identical from run to run)
+        before = ops.set_deterministic(True)
+        try:
+            return conv_step()
+        finally:
+            ops.set_deterministic(before)
+
+    def forward_only():
+        # inference: no projection is kept
+        with torch.no_grad():
+            return ComputeMCConv.apply(pts, pdf, feats, pts, neigh, ends, radii, axis, bias, weights)
+
+    def forward_only_fused():
+        before = ops.set_fused_forward(True)
+        try:
+            return forward_only()
+        finally:
+            ops.set_fused_forward(before)
 
     def conv_step_bf16():
         # the same step with the three contractions on the bf16 matrix pipe (bf16 operands, fp32 accumulation)
@@ -478,13 +499,17 @@ def main():
     conv_ms, conv_kernels = timed(conv_step, args.steps, args.warmup, conv_stats)
     fw_ms, _ = timed(conv_step_fw_only, args.steps, args.warmup, fw_stats)
     bf_ms, bf_kernels = timed(conv_step_bf16, args.steps, args.warmup)
+    det_ms, _ = timed(conv_step_deterministic, args.steps, args.warmup)
+    fwd_ms, _ = timed(forward_only, args.steps, args.warmup)
+    fwd_fused_ms, _ = timed(forward_only_fused, args.steps, args.warmup)
     nb_ms, nb_kernels = timed(neighbor_step, args.steps, args.warmup)
     pdf_ms, pdf_kernels = timed(pdf_step, args.steps, args.warmup)
     mirror_ms, _ = timed(mirror_step, args.steps, args.warmup)
     log("conv fwd+bwd %.3f ms median, %.3f ms wall-clock mean (features+weights grads only: %.3f ms) | neighborhood "
         "%.3f ms | density %.3f ms | sustained %.3f / %.3f ms" % (conv_ms, conv_stats["mean_wall_ms"], fw_ms, nb_ms, pdf_ms,
                                                                   conv_stats["sustained_ms"], fw_stats["sustained_ms"]))
-    log("conv fwd+bwd with bf16 contraction operands: %.3f ms" % bf_ms)
+    log("conv fwd+bwd with bf16 contraction operands: %.3f ms | without atomics: %.3f ms | forward only %.3f ms "
+        "(fused %.3f ms)" % (bf_ms, det_ms, fwd_ms, fwd_fused_ms))
     for name, ks in (("conv", conv_kernels), ("conv bf16", bf_kernels), ("neighbors", nb_kernels),
                      ("pdf", pdf_kernels)):
         log(name, {k: "%d x %.1f us" % (v[0], 1e3 * v[1] / v[0]) for k, v in ks.items()})
@@ -677,6 +702,11 @@ def main():
         "ms_per_step_feature_and_weight_grads_only": fw_ms,
         "ms_per_step_feature_and_weight_grads_only_mean_wall": fw_stats["mean_wall_ms"],
         "ms_per_step_feature_and_weight_grads_only_sustained": fw_stats["sustained_ms"],
+        # the same step with the backward pass without float atomics (GRAD_DETERMINISTIC)
+        "ms_per_step_deterministic": det_ms,
+        # the forward pass alone under no_grad (no projection kept): the two-kernel path that is the default, and the
+        # optional kernel that keeps the projection on chip
+        "forward_only_ms": fwd_ms, "forward_only_fused_ms": fwd_fused_ms,
         # the symmetric-pair index that the step's point / density gradients use is built once per neighborhood
         # (outside ms_per_step); a step on a fresh neighborhood pays it once more
         "mirror_ms": mirror_ms, "ms_per_step_with_mirror": conv_ms + mirror_ms,
