@@ -172,7 +172,12 @@ int pccnn_find_neighbors_fill(const float *pts_sorted, const int64_t *pt_keys_so
  * Replaces compute_pdf / compute_pdf_grads (pccnn_lib_ops/compute_pdf/compute_pdf.cuh:28-51,
  * compute_pdf.cu:153-257).  neigh i32[t,2] = (point, sample) in original point
  * ids, ends i32[n]; samples are the points themselves.  pdf_out f32[n];
- * pt_grads_out f32[n,d]. */
+ * pt_grads_out f32[n,d].  Coordinates are gathered by original index, one
+ * cache line per pair when the points are in no spatial order;
+ * pccnn_compute_pdf_sorted and pccnn_compute_pdf_grid below work on the
+ * grid's sorted copy and read whole lines.  pccnn_compute_pdf_grads adds
+ * into pt_grads_out with float atomics (pccnn_lib_ops/compute_pdf/compute_pdf.cu:153-257
+ * does the same), so its sums depend on the order of arrival in the last bit. */
 int pccnn_compute_pdf(int manifold_dims, const float *bandwidth, const float *pts, int64_t n, int d,
                       const int32_t *neigh, int64_t t, const int32_t *ends, float *pdf_out, void *stream);
 /* Same estimate for a pair list left in sorted-index space (pccnn_find_neighbors_fill without point_remap):

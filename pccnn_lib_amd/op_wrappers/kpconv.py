@@ -34,9 +34,10 @@ class ComputeKPConv(ConvFunction):
         need = ctx.needs_input_grad
         mask = (pccnn_lib_ops.GRAD_PTS if (need[0] or need[2]) else 0) | (pccnn_lib_ops.GRAD_FEATS if need[1] else 0) \
             | (pccnn_lib_ops.GRAD_BASIS_PARAMS if need[6] else 0) | (pccnn_lib_ops.GRAD_WEIGHTS if need[8] else 0)
+        mask |= pccnn_lib_ops.deterministic_flag()
         weight_grads, feat_grads, kernel_pts_grads, pt_grads, sample_grads = pccnn_lib_ops.kp_conv_grads(
             pts, features, samples, neighbors, start_ids, radii, kernel_pts, ctx.sigma_, conv_weights, p_grads,
-            proj=proj, grad_mask=mask | pccnn_lib_ops.deterministic_flag(), mirror=ctx.mirror_, contraction=ctx.contraction_)
+            proj=proj, grad_mask=mask, mirror=ctx.mirror_, contraction=ctx.contraction_)
         return pt_grads if need[0] else None, feat_grads, sample_grads if need[2] else None, None, None, None, \
             kernel_pts_grads, None, weight_grads, None, None
 

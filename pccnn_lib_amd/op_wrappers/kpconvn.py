@@ -32,9 +32,10 @@ class ComputeKPConvN(ConvFunction):
         ops = pccnn_lib_ops
         mask = (ops.GRAD_PTS if (need[0] or need[3]) else 0) | (ops.GRAD_FEATS if need[2] else 0) \
             | (ops.GRAD_BASIS_PARAMS if need[7] else 0) | (ops.GRAD_WEIGHTS if need[9] else 0)
+        mask |= pccnn_lib_ops.deterministic_flag()
         weight_grads, feat_grads, kernel_pts_grads, pt_grads, sample_grads = ops.kp_conv_n_grads(
             pts, pdfs, features, samples, neighbors, start_ids, radii, kernel_pts, ctx.sigma_, conv_weights, p_grads,
-            proj=proj, grad_mask=mask | pccnn_lib_ops.deterministic_flag(), mirror=ctx.mirror_)
+            proj=proj, grad_mask=mask, mirror=ctx.mirror_)
         return pt_grads if need[0] else None, None, feat_grads, sample_grads if need[3] else None, None, None, \
             None, kernel_pts_grads, None, weight_grads, None
 

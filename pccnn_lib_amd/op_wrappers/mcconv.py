@@ -35,9 +35,10 @@ class ComputeMCConv(ConvFunction):
         mask = (ops.GRAD_PTS if (need[0] or need[3]) else 0) | (ops.GRAD_PDF if need[1] else 0) \
             | (ops.GRAD_FEATS if need[2] else 0) | (ops.GRAD_BASIS_PARAMS if (need[7] or need[8]) else 0) \
             | (ops.GRAD_WEIGHTS if need[9] else 0)
+        mask |= pccnn_lib_ops.deterministic_flag()
         weight_grads, feat_grads, axis_grads, bias_grads, pdf_grads, pt_grads, sample_grads = \
             ops.mc_conv_grads(pts, pdf, features, samples, neighbors, start_ids, radii, axis, bias, conv_weights,
-                              p_grads, proj=proj, grad_mask=mask | pccnn_lib_ops.deterministic_flag(), mirror=ctx.mirror_,
+                              p_grads, proj=proj, grad_mask=mask, mirror=ctx.mirror_,
                               contraction=ctx.contraction_)
         return pt_grads if need[0] else None, pdf_grads, feat_grads, sample_grads if need[3] else None, None, None, \
             None, axis_grads if need[7] else None, bias_grads if need[8] else None, weight_grads, None, None

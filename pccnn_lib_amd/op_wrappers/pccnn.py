@@ -31,9 +31,10 @@ class ComputePCCNN(ConvFunction):
         mask = (ops.GRAD_PTS if (need[0] or need[3]) else 0) | (ops.GRAD_PDF if need[1] else 0) \
             | (ops.GRAD_FEATS if need[2] else 0) | (ops.GRAD_BASIS_PARAMS if need[7] else 0) \
             | (ops.GRAD_WEIGHTS if need[9] else 0)
+        mask |= pccnn_lib_ops.deterministic_flag()
         weight_grads, feat_grads, kernel_pts_grads, pt_pdf_grads, pt_grads, sample_grads = ops.pccnn_grads(
             pts, features, pt_pdf, samples, neighbors, start_ids, radii, kernel_pts, ctx.sigma_, conv_weights, p_grads,
-            proj=proj, grad_mask=mask | pccnn_lib_ops.deterministic_flag(), mirror=ctx.mirror_)
+            proj=proj, grad_mask=mask, mirror=ctx.mirror_)
         return pt_grads if need[0] else None, pt_pdf_grads, feat_grads, sample_grads if need[3] else None, None, \
             None, None, kernel_pts_grads, None, weight_grads, None
 

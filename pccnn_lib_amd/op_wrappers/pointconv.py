@@ -43,8 +43,9 @@ class ComputePointConv(ConvFunction):
         ops = pccnn_lib_ops
         mask = (ops.GRAD_BASIS_PARAMS if need[0] else 0) | (ops.GRAD_FEATS if need[1] else 0) \
             | (ops.GRAD_WEIGHTS if need[4] else 0)
+        mask |= pccnn_lib_ops.deterministic_flag()
         weights_grads, feat_grads, basis_grads = ops.point_conv_grads(
-            basis_proj, features, neighbors, start_ids, conv_weights, p_grads, proj=proj, grad_mask=mask | pccnn_lib_ops.deterministic_flag())
+            basis_proj, features, neighbors, start_ids, conv_weights, p_grads, proj=proj, grad_mask=mask)
         return basis_grads, feat_grads, None, None, weights_grads
 
 

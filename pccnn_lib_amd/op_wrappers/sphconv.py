@@ -28,9 +28,10 @@ class ComputeSPHConv(ConvFunction):
         need = ctx.needs_input_grad
         ops = pccnn_lib_ops
         mask = (ops.GRAD_FEATS if need[1] else 0) | (ops.GRAD_WEIGHTS if need[9] else 0)
+        mask |= pccnn_lib_ops.deterministic_flag()
         weight_grads, feat_grads = ops.sph_conv_grads(
             pts, features, samples, neighbors, start_ids, radii, radial_bins, azimuz_bins, polar_bins, conv_weights,
-            p_grads, proj=proj, grad_mask=mask | pccnn_lib_ops.deterministic_flag())
+            p_grads, proj=proj, grad_mask=mask)
         return None, feat_grads, None, None, None, None, None, None, None, weight_grads
 
 
