@@ -18,6 +18,7 @@
 //    the weights are first repacked (conv_pack_weights_kernel) so that the four (eight) values a lane feeds to
 //    consecutive MFMAs are one 16-byte load, and so that rows for padded basis functions / features read as zeros.
 //  * 64 KB (32 KB) of tile + 15 KB of staging: two (three) workgroups per CU, one gathering while another multiplies.
+#include <atomic>
 #include <type_traits>
 
 #include "conv_basis.h"
@@ -342,19 +343,17 @@ conv_fused_fwd_kernel(ConvGeom g, FusedArgs a)
 // kernel hides its dependent loads (offsets -> pairs -> positions and feature rows) behind eight; every slice also
 // walks the pair list again and pays a cross-row reduction per sample.  What the fusion saves - writing P and
 // reading it back, 2 x 268 MB at the first of these shapes - costs the two-kernel path about 50 us.
-static int g_fused_forward = 0;
+static std::atomic<int> g_fused_forward{0};
 
 // 1 lets eligible forward calls take the fused kernel, 0 (the default) sends every call down the two-kernel path.
 extern "C" int pccnn_set_fused_forward(int on)
 {
-    const int before = g_fused_forward;
-    g_fused_forward = on != 0;
-    return before;
+    return g_fused_forward.exchange(on != 0 ? 1 : 0);
 }
 
 bool pccnn_conv_fused_eligible(int basis, int c_in, int k, int num_mlps, int c_out)
 {
-    if (!g_fused_forward || num_mlps != 1 || basis == BASIS_SPH || basis == BASIS_LINEAR) return false;
+    if (!g_fused_forward.load(std::memory_order_relaxed) || num_mlps != 1 || basis == BASIS_SPH || basis == BASIS_LINEAR) return false;
     if (k > 16) return false;                           // a slice holds 16 basis functions
     if (c_in < 33) return false;                        // few features: the pair-parallel narrow kernels
     return c_out == 64 || c_out == 128 || c_out == 256;
