@@ -500,7 +500,7 @@ def main():
     # continuous load to settle, so a short run from idle reads up to 10 % slow), and again behind the other
     # forward + backward legs of this workload, when the device has been under the same kind of load without a break
     # (`ms_per_step`, `value`): the state a training loop is in after its first few dozen steps.  (The forward-only
-    # legs follow it: their steps leave the device partly idle, and a measurement behind them reads 0.83 ms again.)
+    # legs follow it: their kernels load the device less, and a measurement behind them reads 0.83 ms again.)
     idle_stats, conv_stats, fw_stats = {}, {"sustained": True}, {"sustained": True}
     idle_ms, _ = timed(conv_step, args.steps, args.warmup, idle_stats)
     fw_ms, _ = timed(conv_step_fw_only, args.steps, args.warmup, fw_stats)
