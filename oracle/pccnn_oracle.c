@@ -12,7 +12,15 @@
  * to the reference repository root).  Compile with contraction disabled
  * (-ffp-contract=off) so that fp32 expressions round exactly as written.
  *
- * Parity status of each function (what pins it) is listed in oracle/README.md.
+ * PARITY UNPINNED: one piece only.  When a sample has more neighbors than
+ * max_neighbors, orc_store_neighbors keeps an evenly spaced subset; the
+ * reference keeps a random one seeded with time(NULL)
+ * (pccnn_lib_ops/find_neighbors/store_neighbors.cu:66-99, find_neighbors.cu),
+ * so which members survive cannot be compared, only the contract of its unit
+ * test (count == cap, every member a distinct true neighbor).  Every other
+ * function is pinned in tests/ by the formulas of the reference's own unit
+ * tests, brute force, closed forms or hand-worked cases (the Poisson-disk
+ * colour order and bit-to-dimension mapping: tests/golden/poisson_known_answers.py).
  */
 #include <math.h>
 #include <stdint.h>
