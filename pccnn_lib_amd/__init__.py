@@ -27,4 +27,5 @@ def install_as_reference():
     sys.modules.setdefault("pccnn_lib.op_wrappers", op_wrappers)
     sys.modules.setdefault("pccnn_lib.pc", pc)
     sys.modules.setdefault("pccnn_lib.pc.layers", pc.layers)
+    sys.modules.setdefault("pccnn_lib.pc.models", pc.models)
     return me

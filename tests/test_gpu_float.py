@@ -418,6 +418,37 @@ def test_weight_variance_ops_and_layer_warmup(ops, oracle):
     assert 0.5 < float(out.detach().var()) < 2.0
 
 
+def test_model_base_class_runs_the_warmup_of_its_layers(ops, oracle):
+    # the loop a trainer built on the reference runs (IModel.py:19-27 with KPConv.py:103-116): layer after layer is
+    # switched into its warm-up state, fed a batch so that it measures its statistic and redraws its weights, and
+    # switched back; afterwards every layer's output variance is about the constant asked for
+    import pccnn_lib_amd as lib
+    pts, ids = synthetic.primitives(5, 2, 2000)
+    rng = np.random.default_rng(5)
+    feats = t(rng.normal(size=(pts.shape[0], 16)).astype(np.float32))
+    pc = lib.pc.Pointcloud(pts, ids, device=DEV)
+    pc.compute_pdf(np.full(3, 0.02, np.float32))
+    torch.manual_seed(11)
+    model = lib.pc.models.IModel()
+    model.add_conv(lib.pc.layers.KPConv(3, 16, 32, 15, True, 1.0).to(DEV))
+    model.add_conv(lib.pc.layers.MCConv(3, 32, 32, 8, 1, True, 1.0).to(DEV))
+    assert model.get_num_convs() == 2
+
+    def forward():
+        first, nbh = model.conv_list_[0](pc, pc, feats, 0.12)
+        return first, model.conv_list_[1](pc, pc, torch.nn.functional.leaky_relu(first, 0.2), 0.12, nbh)
+
+    with torch.no_grad():
+        for i in range(model.get_num_convs()):
+            model.init_variance(i, 1.0)
+            model.set_init_warmup_state(i, True)
+            forward()
+            model.set_init_warmup_state(i, False)
+            assert model.conv_list_[i].accum_weight_var_ > 0.0
+        mid, out = forward()
+    assert 0.4 < float(mid.var()) < 2.5 and 0.4 < float(out.var()) < 2.5
+
+
 def test_error_paths(ops):
     pts, ids = synthetic.primitives(1, 1, 128)
     tp, ti = t(pts), t(ids)
