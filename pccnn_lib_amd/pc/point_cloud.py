@@ -141,6 +141,15 @@ class Pointcloud(object):
     def global_upsample(self, p_in_tensor):
         return torch.index_select(p_in_tensor, 0, self.batch_ids_.to(torch.int64))
 
+    @classmethod
+    def __torch_function__(cls, func, types, args=(), kwargs=None):
+        """torch functions take a Pointcloud where they take a tensor (pccnn_lib/pc/Pointcloud.py:158-165): the call
+        runs on the coordinates, and its result comes back as a new Pointcloud with the batch ids of the first cloud
+        among the arguments, so ``torch.add(cloud, offset)`` or ``torch.mul(cloud, 2.0)`` move or scale a batch."""
+        first = next(a for a in args if isinstance(a, Pointcloud))
+        plain = [a.pts_ if hasattr(a, "pts_") else a for a in args]
+        return Pointcloud(func(*plain, **(kwargs or {})), first.batch_ids_)
+
     def __repr__(self):
         return "### Points:\n{}\n### Batch Ids:\n{}\n### Batch Size:\n{}\n### Pdf:\n{}".format(
             self.pts_, self.batch_ids_, self.batch_size_, self.pts_pdf_)

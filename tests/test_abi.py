@@ -179,6 +179,22 @@ def test_model_base_class_drives_the_layers_initialisation():
     assert point.init_proj_axis_ is True            # a PointConv layer redraws its axes on the next warm-up pass
 
 
+def test_torch_functions_apply_to_a_clouds_coordinates():
+    # pccnn_lib/pc/Pointcloud.py:158-165
+    import torch
+    import pccnn_lib_amd as lib
+    pts = torch.arange(12, dtype=torch.float32).reshape(4, 3)
+    ids = torch.tensor([0, 0, 1, 1], dtype=torch.int32)
+    cloud = lib.pc.Pointcloud(pts, ids)
+    moved = torch.add(cloud, 1.5)
+    assert isinstance(moved, lib.pc.Pointcloud) and torch.equal(moved.pts_, pts + 1.5)
+    assert moved.batch_ids_ is cloud.batch_ids_ and int(moved.batch_size_) == 2
+    scaled = torch.mul(cloud, torch.tensor([2.0, 1.0, 0.5]))
+    assert torch.equal(scaled.pts_, pts * torch.tensor([2.0, 1.0, 0.5]))
+    both = torch.sub(moved, cloud)
+    assert torch.equal(both.pts_, torch.full((4, 3), 1.5))
+
+
 def test_install_as_reference_resolves_the_reference_imports():
     # in a process of its own: the call registers modules under the reference's names
     import subprocess
