@@ -446,7 +446,7 @@ def test_model_base_class_runs_the_warmup_of_its_layers(ops, oracle):
             model.set_init_warmup_state(i, False)
             assert model.conv_list_[i].accum_weight_var_ > 0.0
         mid, out = forward()
-    assert 0.4 < float(mid.var()) < 2.5 and 0.4 < float(out.var()) < 2.5
+    assert 0.5 < float(mid.var()) < 2.0 and 0.5 < float(out.var()) < 2.0   # (measured: 0.94 - 1.05)
 
 
 def test_error_paths(ops):
