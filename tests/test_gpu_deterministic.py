@@ -110,6 +110,44 @@ def test_pointconv_gradients_without_atomics(ops, oracle):
         assert relerr(got.cpu().numpy(), e) < GRAD_TOL, name
 
 
+@pytest.mark.parametrize("c_in", [40, 12])
+def test_the_other_families_without_atomics(ops, oracle, c_in):
+    # KPConvN, PCCNN (both divide by the density) and SPHConv (bins, no geometry gradients): same bar, same bits
+    # from run to run; 12 features take the pair-parallel kernels
+    pts, smp, nb, rng = _case(ops, 950 + c_in, 1000, 0.12, True)
+    d = nb["dev"]
+    n, k, c_out = pts.shape[0], 16, 24
+    kp, sigma = synthetic.kernel_points_sphere(2, k)
+    pdf = rng.uniform(0.5, 2.0, n).astype(np.float32)
+    feats = rng.normal(size=(n, c_in)).astype(np.float32)
+    w = rng.normal(0, np.sqrt(1.0 / (k * c_in)), (k * c_in, c_out)).astype(np.float32)
+    g = rng.normal(size=(smp.shape[0], c_out)).astype(np.float32)
+    geo = (d["samples"], d["neigh"], d["ends"], d["radii"])
+    host = (smp, nb["neighbors"], nb["ends"], nb["radii"])
+    mask = ops.GRAD_ALL | ops.GRAD_DETERMINISTIC
+    got = _identical_runs(lambda: ops.kp_conv_n_grads(d["pts"], t(pdf), t(feats), *geo, t(kp), sigma, t(w), t(g),
+                                                      grad_mask=mask))
+    exp = oracle.kpconvn_grads(pts, pdf, feats, *host, kp, sigma, w, g)
+    for a, e, name in zip(got, exp, ("dW", "dFeat", "dKernelPts", "dPts", "dSamples")):
+        assert relerr(a.cpu().numpy(), e) < GRAD_TOL, name
+    got = _identical_runs(lambda: ops.pccnn_grads(d["pts"], t(feats), t(pdf), *geo, t(kp), sigma, t(w), t(g),
+                                                  grad_mask=mask))
+    exp = oracle.pccnn_grads(pts, feats, pdf, *host, kp, sigma, w, g)
+    for a, e, name in zip(got, exp, ("dW", "dFeat", "dKernelPts", "dPdf", "dPts", "dSamples")):
+        assert relerr(a.cpu().numpy(), e) < GRAD_TOL, name
+    radial = np.linspace(0, 1, 4)[1:].astype(np.float32)
+    azimuth = np.linspace(-np.pi / 2, np.pi / 2, 5)[1:].astype(np.float32)
+    polar = np.linspace(0, np.pi, 4)[1:].astype(np.float32)
+    ks = 3 * 4 * 3 + 1
+    ws = rng.normal(0, np.sqrt(1.0 / (ks * c_in)), (ks * c_in, c_out)).astype(np.float32)
+    got = _identical_runs(lambda: ops.sph_conv_grads(d["pts"], t(feats), *geo, t(radial), t(azimuth), t(polar), t(ws),
+                                                     t(g), grad_mask=ops.GRAD_WEIGHTS | ops.GRAD_FEATS
+                                                     | ops.GRAD_DETERMINISTIC))
+    exp = oracle.sphconv_grads(pts, feats, *host, radial, azimuth, polar, ws, g)
+    for a, e, name in zip(got, exp, ("dW", "dFeat")):
+        assert relerr(a.cpu().numpy(), e) < GRAD_TOL, name
+
+
 def test_layers_give_identical_gradients_from_run_to_run_when_asked(ops, oracle):
     # set_deterministic(True): the autograd wrappers ask for the pass without atomics; two passes over a level of a
     # hierarchy (pooled samples: no mirror index) and over a symmetric neighborhood give the same bits
