@@ -110,6 +110,18 @@ def test_shapes_outside_the_fused_kernel_take_the_two_kernel_path(ops):
             torch.cuda.synchronize()
             timers = _lib.timing(enable=False)
             assert "fused_fwd" not in timers and "proj_fwd" in timers, (k, c_in, c_out)
+        # two MLPs (MCConv with the feature axis split over two weight blocks)
+        n, c_in, hidden, c_out = pts.shape[0], 64, 8, 128
+        feats = t(rng.normal(size=(n, c_in)).astype(np.float32))
+        pdf = t(rng.uniform(0.5, 2.0, n).astype(np.float32))
+        axis = t(rng.normal(0, 0.6, (3, 2 * hidden)).astype(np.float32))
+        bias = t(rng.normal(0, 0.1, (1, 2 * hidden)).astype(np.float32))
+        w = t(rng.normal(0, 0.05, (2, hidden * c_in, c_out // 2)).astype(np.float32))
+        _lib.timing(enable=True, reset=True)
+        out = ops.mc_conv(d["pts"], pdf, feats, d["samples"], d["neigh"], d["ends"], d["radii"], axis, bias, w)
+        torch.cuda.synchronize()
+        timers = _lib.timing(enable=False)
+        assert "fused_fwd" not in timers and "proj_fwd" in timers and tuple(out.shape) == (n, c_out)
     finally:
         ops.set_fused_forward(before)
 
