@@ -1,3 +1,5 @@
+import math
+
 import torch
 
 from ... import pccnn_lib_ops
@@ -110,6 +112,22 @@ class IConvLayer(torch.nn.Module):
         self.accum_weight_var_ += (p_new_var - self.accum_weight_var_) / self.accum_weight_var_counter_
         self.accum_weight_var_counter_ += 1.0
 
+    def _new_parameters(self, **p_shapes):
+        """Register one uninitialised float32 parameter per keyword, in the order given (the order of the state dict
+        and of ``parameters()``)."""
+        for name, shape in p_shapes.items():
+            setattr(self, name, torch.nn.Parameter(torch.empty(*shape)))
+
+    def _warm_up(self, p_measure):
+        """The variance-aware initialisation every layer shares (e.g. pccnn_lib/pc/layers/KPConv.py:103-116): in the
+        warm-up state ``p_measure()`` returns this batch's weight-variance statistic, its reciprocal goes into the
+        running mean, and the weights are redrawn with the variance that mean asks for.  Returns whether it ran."""
+        if not (self.wamup_state_ and self.use_const_variance_init_):
+            return False
+        self.__update_weight_var__(1.0 / float(p_measure()))
+        self.conv_weights_.data.normal_(0.0, math.sqrt(self.out_constant_variance_ / self.accum_weight_var_))
+        return True
+
     def __compute_convolution__(self, p_pc_in, p_pc_out, p_in_features, p_radius, p_neighborhood):
         raise NotImplementedError
 
@@ -146,6 +164,10 @@ class IConvLayerFactory(object):
 
     def define_num_basis(self, p_num_basis):
         self.num_basis_ = p_num_basis
+
+    def _remember(self, p_layer):
+        self.conv_list_.append(p_layer)
+        return p_layer
 
     def create_conv_layer(self, p_dims, p_in_features, p_out_features):
         raise NotImplementedError

@@ -53,8 +53,7 @@ class KPConv(IConvLayer):
         self.register_buffer('kernel_pts_', kernel_pts)
         self.register_buffer('sigma_', sigma)
         self.sigma_cpu_ = None
-        self.conv_weights_ = torch.nn.Parameter(
-            torch.empty(self.num_kernel_pts_ * self.feat_input_size_, self.feat_output_size_))
+        self._new_parameters(conv_weights_=(p_num_kernel_pts * p_in_features, p_out_features))
         self.reset_parameters()
 
     def reset_parameters(self):
@@ -65,17 +64,11 @@ class KPConv(IConvLayer):
         if self.sigma_cpu_ is None:
             self.sigma_cpu_ = self.sigma_.item()
         pts, pairs, feats = point_side(p_pc_in, p_neighborhood, p_in_features)
-        if self.wamup_state_ and self.use_const_variance_init_:
-            variance = ComputeKPConvWeightVar.apply(
-                pts, feats, p_pc_out.pts_, pairs, p_neighborhood.start_ids_,
-                p_radius, self.kernel_pts_, self.sigma_cpu_)
-            self.__update_weight_var__(1.0 / variance.item())
-            stdv = math.sqrt(self.out_constant_variance_ / self.accum_weight_var_)
-            self.conv_weights_.data.normal_(0.0, stdv)
-        return ComputeKPConv.apply(
-            pts, feats, p_pc_out.pts_, pairs, p_neighborhood.start_ids_,
-            p_radius, self.kernel_pts_, self.sigma_cpu_, self.conv_weights_,
-            mirror_if_needed(p_neighborhood, pts), self.contraction_)
+        geometry = (pts, feats, p_pc_out.pts_, pairs, p_neighborhood.start_ids_, p_radius, self.kernel_pts_,
+                    self.sigma_cpu_)
+        self._warm_up(lambda: ComputeKPConvWeightVar.apply(*geometry))
+        return ComputeKPConv.apply(*geometry, self.conv_weights_, mirror_if_needed(p_neighborhood, pts),
+                                   self.contraction_)
 
 
 class KPConvFactory(IConvLayerFactory):
@@ -83,10 +76,8 @@ class KPConvFactory(IConvLayerFactory):
         super(KPConvFactory, self).__init__(p_num_kernel_pts, p_const_var_w_init, p_const_var_value)
 
     def create_conv_layer(self, p_dims, p_in_features, p_out_features):
-        cur_conv = KPConv(p_dims, p_in_features, p_out_features, self.num_basis_, self.conv_var_w_init_,
-                          self.const_var_value_)
-        self.conv_list_.append(cur_conv)
-        return cur_conv
+        return self._remember(KPConv(p_dims, p_in_features, p_out_features, self.num_basis_, self.conv_var_w_init_,
+                                     self.const_var_value_))
 
 
 class _DensityKernelPointConv(IConvLayer):
@@ -108,8 +99,7 @@ class _DensityKernelPointConv(IConvLayer):
         self.register_buffer('kernel_pts_', kernel_pts)
         self.register_buffer('sigma_', sigma)
         self.sigma_cpu_ = None
-        self.conv_weights_ = torch.nn.Parameter(
-            torch.empty(self.num_kernel_pts_ * self.feat_input_size_, self.feat_output_size_))
+        self._new_parameters(conv_weights_=(p_num_kernel_pts * p_in_features, p_out_features))
         self.reset_parameters()
 
     def reset_parameters(self):
@@ -124,17 +114,10 @@ class _DensityKernelPointConv(IConvLayer):
             pts, pairs, pdf, feats = p_pc_in.pts_, p_neighborhood.neighbors_, cur_pdf, p_in_features
         else:
             pts, pairs, pdf, feats = point_side(p_pc_in, p_neighborhood, cur_pdf, p_in_features)
-        if self.wamup_state_ and self.use_const_variance_init_:
-            variance = self.weight_var_op_.apply(
-                pts, pdf, feats, p_pc_out.pts_, pairs,
-                p_neighborhood.start_ids_, p_radius, self.kernel_pts_, self.sigma_cpu_)
-            self.__update_weight_var__(1.0 / variance.item())
-            stdv = math.sqrt(self.out_constant_variance_ / self.accum_weight_var_)
-            self.conv_weights_.data.normal_(0.0, stdv)
-        return self.conv_op_.apply(
-            pts, pdf, feats, p_pc_out.pts_, pairs, p_neighborhood.start_ids_,
-            p_radius, self.kernel_pts_, self.sigma_cpu_, self.conv_weights_,
-            mirror_if_needed(p_neighborhood, pts, pdf))
+        geometry = (pts, pdf, feats, p_pc_out.pts_, pairs, p_neighborhood.start_ids_, p_radius, self.kernel_pts_,
+                    self.sigma_cpu_)
+        self._warm_up(lambda: self.weight_var_op_.apply(*geometry))
+        return self.conv_op_.apply(*geometry, self.conv_weights_, mirror_if_needed(p_neighborhood, pts, pdf))
 
 
 class KPConvN(_DensityKernelPointConv):
@@ -157,10 +140,8 @@ class KPConvNFactory(IConvLayerFactory):
         super(KPConvNFactory, self).__init__(p_num_kernel_pts, p_const_var_w_init, p_const_var_value)
 
     def create_conv_layer(self, p_dims, p_in_features, p_out_features):
-        cur_conv = KPConvN(p_dims, p_in_features, p_out_features, self.num_basis_, self.conv_var_w_init_,
-                           self.const_var_value_)
-        self.conv_list_.append(cur_conv)
-        return cur_conv
+        return self._remember(KPConvN(p_dims, p_in_features, p_out_features, self.num_basis_, self.conv_var_w_init_,
+                                      self.const_var_value_))
 
 
 class PCCNNFactory(IConvLayerFactory):
@@ -168,7 +149,5 @@ class PCCNNFactory(IConvLayerFactory):
         super(PCCNNFactory, self).__init__(p_num_kernel_pts, p_const_var_w_init, p_const_var_value)
 
     def create_conv_layer(self, p_dims, p_in_features, p_out_features):
-        cur_conv = PCCNN(p_dims, p_in_features, p_out_features, self.num_basis_, self.conv_var_w_init_,
-                         self.const_var_value_)
-        self.conv_list_.append(cur_conv)
-        return cur_conv
+        return self._remember(PCCNN(p_dims, p_in_features, p_out_features, self.num_basis_, self.conv_var_w_init_,
+                                    self.const_var_value_))

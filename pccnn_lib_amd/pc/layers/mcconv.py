@@ -18,16 +18,11 @@ class MCConv(IConvLayer):
 
     def __init__(self, p_dims, p_in_features, p_out_features, p_hidden_size, p_num_mlps=1,
                  p_constant_weight_var=True, p_const_var_value=1.0):
-        super(MCConv, self).__init__(p_dims, p_in_features, p_out_features, p_constant_weight_var,
-                                     p_const_var_value)
-        self.hidden_size_ = p_hidden_size
-        self.num_mlps_ = p_num_mlps
-        self.contraction_ = "f32"
-        self.proj_axis_ = torch.nn.Parameter(torch.empty(self.num_dims_, self.hidden_size_ * self.num_mlps_))
-        self.proj_bias_ = torch.nn.Parameter(torch.empty(1, self.hidden_size_ * self.num_mlps_))
-        self.conv_weights_ = torch.nn.Parameter(
-            torch.empty(self.num_mlps_, self.hidden_size_ * self.feat_input_size_,
-                        self.feat_output_size_ // p_num_mlps))
+        IConvLayer.__init__(self, p_dims, p_in_features, p_out_features, p_constant_weight_var, p_const_var_value)
+        self.hidden_size_, self.num_mlps_, self.contraction_ = p_hidden_size, p_num_mlps, "f32"
+        hidden_total = p_hidden_size * p_num_mlps
+        self._new_parameters(proj_axis_=(p_dims, hidden_total), proj_bias_=(1, hidden_total),
+                             conv_weights_=(p_num_mlps, p_hidden_size * p_in_features, p_out_features // p_num_mlps))
         self.reset_parameters()
 
     def reset_parameters(self):
@@ -43,17 +38,11 @@ class MCConv(IConvLayer):
             pts, pairs, pdf, feats = p_pc_in.pts_, p_neighborhood.neighbors_, cur_pdf, p_in_features
         else:
             pts, pairs, pdf, feats = point_side(p_pc_in, p_neighborhood, cur_pdf, p_in_features)
-        if self.wamup_state_ and self.use_const_variance_init_:
-            variance = ComputeMCConvWeightVar.apply(
-                pts, pdf, feats, p_pc_out.pts_, pairs,
-                p_neighborhood.start_ids_, p_radius, self.proj_axis_, self.proj_bias_) * self.num_mlps_
-            self.__update_weight_var__(1.0 / variance.item())
-            stdv = math.sqrt(self.out_constant_variance_ / self.accum_weight_var_)
-            self.conv_weights_.data.normal_(0.0, stdv)
-        return ComputeMCConv.apply(
-            pts, pdf, feats, p_pc_out.pts_, pairs,
-            p_neighborhood.start_ids_, p_radius, self.proj_axis_, self.proj_bias_, self.conv_weights_,
-            mirror_if_needed(p_neighborhood, pts, pdf), self.contraction_)
+        geometry = (pts, pdf, feats, p_pc_out.pts_, pairs, p_neighborhood.start_ids_, p_radius, self.proj_axis_,
+                    self.proj_bias_)
+        self._warm_up(lambda: ComputeMCConvWeightVar.apply(*geometry) * self.num_mlps_)
+        return ComputeMCConv.apply(*geometry, self.conv_weights_, mirror_if_needed(p_neighborhood, pts, pdf),
+                                   self.contraction_)
 
 
 class MCConvFactory(IConvLayerFactory):
@@ -62,7 +51,5 @@ class MCConvFactory(IConvLayerFactory):
         self.num_mlps_ = p_num_mlps
 
     def create_conv_layer(self, p_dims, p_in_features, p_out_features):
-        cur_conv = MCConv(p_dims, p_in_features, p_out_features, self.num_basis_, self.num_mlps_,
-                          self.conv_var_w_init_, self.const_var_value_)
-        self.conv_list_.append(cur_conv)
-        return cur_conv
+        return self._remember(MCConv(p_dims, p_in_features, p_out_features, self.num_basis_, self.num_mlps_,
+                                     self.conv_var_w_init_, self.const_var_value_))

@@ -22,10 +22,8 @@ class PointConv(IConvLayer):
         self.gn_size_ = p_gn_size
         self.hidden_size_ = p_hidden_size
         self.init_proj_axis_ = False
-        self.proj_axis_ = torch.nn.Parameter(torch.empty(self.num_dims_, self.hidden_size_))
-        self.proj_bias_ = torch.nn.Parameter(torch.empty(1, self.hidden_size_))
-        self.conv_weights_ = torch.nn.Parameter(
-            torch.empty(self.hidden_size_ * self.feat_input_size_, self.feat_output_size_))
+        self._new_parameters(proj_axis_=(p_dims, p_hidden_size), proj_bias_=(1, p_hidden_size),
+                             conv_weights_=(p_hidden_size * p_in_features, p_out_features))
         norm = self.use_bn_ or self.use_gn_
         stages = [torch.nn.Linear(1, 16)] + ([torch.nn.BatchNorm1d(16)] if norm else []) + [torch.nn.ReLU()]
         stages += [torch.nn.Linear(16, 1)] + ([torch.nn.BatchNorm1d(1)] if norm else []) + [torch.nn.Sigmoid()]
@@ -65,21 +63,15 @@ class PointConv(IConvLayer):
     def __compute_convolution__(self, p_pc_in, p_pc_out, p_in_features, p_radius, p_neighborhood):
         cur_pdf = self.__density_scale__(p_pc_in, p_neighborhood)
         axis_stdv = torch.sqrt(1.0 / (self.num_dims_ * p_radius[0] * p_radius[0]))
-        if self.wamup_state_ and self.use_const_variance_init_:
+        pairs, offsets = p_neighborhood.neighbors_, p_neighborhood.start_ids_
+        warming = self.wamup_state_ and self.use_const_variance_init_
+        if warming or self.init_proj_axis_:
+            # the axes are redrawn for the radius at hand on every warm-up pass, and once after init_variance asked
             self.proj_axis_.data.normal_(0.0, float(axis_stdv))
-            basis_proj = self.__basis__(p_pc_in, p_pc_out, p_neighborhood, p_radius, True) * cur_pdf
-            variance = ComputePointConvWeightVar.apply(basis_proj, p_in_features, p_neighborhood.neighbors_,
-                                                       p_neighborhood.start_ids_)
-            self.__update_weight_var__(1.0 / variance.item())
-            stdv = math.sqrt(self.out_constant_variance_ / self.accum_weight_var_)
-            self.conv_weights_.data.normal_(0.0, stdv)
-        else:
-            if self.init_proj_axis_:
-                self.proj_axis_.data.normal_(0.0, float(axis_stdv))
-                self.init_proj_axis_ = False
-            basis_proj = self.__basis__(p_pc_in, p_pc_out, p_neighborhood, p_radius, False) * cur_pdf
-        return ComputePointConv.apply(basis_proj, p_in_features, p_neighborhood.neighbors_,
-                                      p_neighborhood.start_ids_, self.conv_weights_)
+            self.init_proj_axis_ = self.init_proj_axis_ and warming
+        basis_proj = self.__basis__(p_pc_in, p_pc_out, p_neighborhood, p_radius, warming) * cur_pdf
+        self._warm_up(lambda: ComputePointConvWeightVar.apply(basis_proj, p_in_features, pairs, offsets))
+        return ComputePointConv.apply(basis_proj, p_in_features, pairs, offsets, self.conv_weights_)
 
 
 class PointConvFactory(IConvLayerFactory):
@@ -91,7 +83,5 @@ class PointConvFactory(IConvLayerFactory):
         super(PointConvFactory, self).__init__(p_num_basis, p_const_var_w_init, p_const_var_value)
 
     def create_conv_layer(self, p_dims, p_in_features, p_out_features):
-        cur_conv = PointConv(p_dims, p_in_features, p_out_features, self.num_basis_, self.conv_var_w_init_,
-                             self.const_var_value_, self.use_bn_, self.use_gn_, self.gn_size_)
-        self.conv_list_.append(cur_conv)
-        return cur_conv
+        return self._remember(PointConv(p_dims, p_in_features, p_out_features, self.num_basis_, self.conv_var_w_init_,
+                                        self.const_var_value_, self.use_bn_, self.use_gn_, self.gn_size_))

@@ -28,8 +28,7 @@ class SPHConv(IConvLayer):
         self.register_buffer('azimuz_bins_', _upper_edges(2.0 * math.pi, p_num_azimuz_bins))
         self.register_buffer('polar_bins_', _upper_edges(math.pi, p_num_polar_bins))
         self.sigma_cpu_ = None
-        self.conv_weights_ = torch.nn.Parameter(
-            torch.empty(self.num_basis_ * self.feat_input_size_, self.feat_output_size_))
+        self._new_parameters(conv_weights_=(self.num_basis_ * p_in_features, p_out_features))
         self.reset_parameters()
 
     def reset_parameters(self):
@@ -39,11 +38,7 @@ class SPHConv(IConvLayer):
     def __compute_convolution__(self, p_pc_in, p_pc_out, p_in_features, p_radius, p_neighborhood):
         geometry = (p_pc_in.pts_, p_in_features, p_pc_out.pts_, p_neighborhood.neighbors_, p_neighborhood.start_ids_,
                     p_radius, self.radial_bins_, self.azimuz_bins_, self.polar_bins_)
-        if self.wamup_state_ and self.use_const_variance_init_:
-            variance = ComputeSPHConvWeightVar.apply(*geometry)
-            self.__update_weight_var__(1.0 / variance.item())
-            stdv = math.sqrt(self.out_constant_variance_ / self.accum_weight_var_)
-            self.conv_weights_.data.normal_(0.0, stdv)
+        self._warm_up(lambda: ComputeSPHConvWeightVar.apply(*geometry))
         return ComputeSPHConv.apply(*geometry, self.conv_weights_)
 
 
@@ -57,7 +52,5 @@ class SPHConvFactory(IConvLayerFactory):
                                              p_const_var_w_init, p_const_var_value)
 
     def create_conv_layer(self, p_dims, p_in_features, p_out_features):
-        cur_conv = SPHConv(p_dims, p_in_features, p_out_features, self.radial_bins_, self.azimuz_bins_,
-                           self.polar_bins_, self.conv_var_w_init_, self.const_var_value_)
-        self.conv_list_.append(cur_conv)
-        return cur_conv
+        return self._remember(SPHConv(p_dims, p_in_features, p_out_features, self.radial_bins_, self.azimuz_bins_,
+                                      self.polar_bins_, self.conv_var_w_init_, self.const_var_value_))
