@@ -17,22 +17,24 @@ class PointConv(IConvLayer):
                  p_const_var_value=1.0, p_use_bn=False, p_use_gn=False, p_gn_size=32):
         super(PointConv, self).__init__(p_dims, p_in_features, p_out_features, p_constant_weight_var,
                                         p_const_var_value)
-        self.use_bn_ = p_use_bn
-        self.use_gn_ = p_use_gn
-        self.gn_size_ = p_gn_size
-        self.hidden_size_ = p_hidden_size
-        self.init_proj_axis_ = False
+        self.use_bn_, self.use_gn_, self.gn_size_ = p_use_bn, p_use_gn, p_gn_size
+        self.hidden_size_, self.init_proj_axis_ = p_hidden_size, False
         self._new_parameters(proj_axis_=(p_dims, p_hidden_size), proj_bias_=(1, p_hidden_size),
                              conv_weights_=(p_hidden_size * p_in_features, p_out_features))
-        norm = self.use_bn_ or self.use_gn_
-        stages = [torch.nn.Linear(1, 16)] + ([torch.nn.BatchNorm1d(16)] if norm else []) + [torch.nn.ReLU()]
-        stages += [torch.nn.Linear(16, 1)] + ([torch.nn.BatchNorm1d(1)] if norm else []) + [torch.nn.Sigmoid()]
-        self.pdf_mlp_ = torch.nn.Sequential(*stages)
-        if self.use_bn_:
+        self.pdf_mlp_ = self._density_network(16, p_use_bn or p_use_gn)
+        if p_use_bn:
             self.basis_bn_ = torch.nn.BatchNorm1d(p_hidden_size)
-        elif self.use_gn_:
-            self.basis_gn_ = GroupNormalization(p_hidden_size, self.gn_size_)
+        elif p_use_gn:
+            self.basis_gn_ = GroupNormalization(p_hidden_size, p_gn_size)
         self.reset_parameters()
+
+    @staticmethod
+    def _density_network(p_width, p_normalised):
+        """1 -> width -> 1 with a sigmoid at the end; a batch norm behind each linear map when the layer normalises
+        its basis (module indices as in the reference, so its state dicts load)."""
+        def block(n_in, n_out, activation):
+            return [torch.nn.Linear(n_in, n_out)] + ([torch.nn.BatchNorm1d(n_out)] if p_normalised else []) + [activation]
+        return torch.nn.Sequential(*(block(1, p_width, torch.nn.ReLU()) + block(p_width, 1, torch.nn.Sigmoid())))
 
     def reset_parameters(self):
         self.conv_weights_.data.normal_(0.0, math.sqrt(2.0 / (self.feat_input_size_ * self.hidden_size_)))

@@ -20,20 +20,20 @@ class SPHConv(IConvLayer):
                  p_num_polar_bins=3, p_constant_weight_var=True, p_const_var_value=1.0):
         super(SPHConv, self).__init__(p_dims, p_in_features, p_out_features, p_constant_weight_var,
                                       p_const_var_value)
-        self.num_radial_bins_ = p_num_radial_bins
-        self.num_azimuz_bins_ = p_num_azimuz_bins
-        self.num_polar_bins_ = p_num_polar_bins
-        self.num_basis_ = p_num_radial_bins * p_num_azimuz_bins * p_num_polar_bins + 1
-        self.register_buffer('radial_bins_', _upper_edges(1.0, p_num_radial_bins))
-        self.register_buffer('azimuz_bins_', _upper_edges(2.0 * math.pi, p_num_azimuz_bins))
-        self.register_buffer('polar_bins_', _upper_edges(math.pi, p_num_polar_bins))
+        counts = {"radial": (1.0, p_num_radial_bins), "azimuz": (2.0 * math.pi, p_num_azimuz_bins),
+                  "polar": (math.pi, p_num_polar_bins)}
+        self.num_basis_ = 1
+        for label, (extent, count) in counts.items():
+            setattr(self, "num_%s_bins_" % label, count)
+            self.register_buffer("%s_bins_" % label, _upper_edges(extent, count))
+            self.num_basis_ *= count
+        self.num_basis_ += 1                    # one more bin for the sample itself
         self.sigma_cpu_ = None
         self._new_parameters(conv_weights_=(self.num_basis_ * p_in_features, p_out_features))
         self.reset_parameters()
 
     def reset_parameters(self):
-        stdv = math.sqrt(1.0 / (self.feat_input_size_ * self.num_basis_))
-        self.conv_weights_.data.normal_(0.0, stdv)
+        self.conv_weights_.data.normal_(0.0, math.sqrt(1.0 / (self.feat_input_size_ * self.num_basis_)))
 
     def __compute_convolution__(self, p_pc_in, p_pc_out, p_in_features, p_radius, p_neighborhood):
         geometry = (p_pc_in.pts_, p_in_features, p_pc_out.pts_, p_neighborhood.neighbors_, p_neighborhood.start_ids_,
@@ -45,11 +45,9 @@ class SPHConv(IConvLayer):
 class SPHConvFactory(IConvLayerFactory):
     def __init__(self, p_num_radial_bins, p_num_azimuz_bins, p_num_polar_bins, p_const_var_w_init=False,
                  p_const_var_value=1.0):
-        self.radial_bins_ = p_num_radial_bins
-        self.azimuz_bins_ = p_num_azimuz_bins
-        self.polar_bins_ = p_num_polar_bins
-        super(SPHConvFactory, self).__init__(p_num_radial_bins * p_num_azimuz_bins * p_num_polar_bins + 1,
-                                             p_const_var_w_init, p_const_var_value)
+        self.radial_bins_, self.azimuz_bins_, self.polar_bins_ = p_num_radial_bins, p_num_azimuz_bins, p_num_polar_bins
+        IConvLayerFactory.__init__(self, p_num_radial_bins * p_num_azimuz_bins * p_num_polar_bins + 1,
+                                   p_const_var_w_init, p_const_var_value)
 
     def create_conv_layer(self, p_dims, p_in_features, p_out_features):
         return self._remember(SPHConv(p_dims, p_in_features, p_out_features, self.radial_bins_, self.azimuz_bins_,
