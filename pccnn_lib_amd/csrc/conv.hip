@@ -158,8 +158,8 @@ conv_proj_fwd_kernel(ConvGeom g, const float *__restrict__ feats, void *__restri
     } else {
         float *dst = (float *)proj_out + dst_at;
         if (g.k == KPAD) {
-            // whole lines that nothing reads before the next kernel: stored past the L2, which keeps the feature rows
-            // the gathers share (65 536 samples x 64 features x 16: 85 -> 80 us, the contraction behind it 2 us slower).
+            // whole lines that nothing reads before the next kernel: stored past the L2 (65 536 samples x 64 features
+            // x 16: 85 -> 80 us, the contraction behind it 2 us slower).
             // Not for the bf16 tile: half the size, much of it is still in cache when the contraction reads it
             // (40 -> 49 us with such stores).
             for (int i = lane; i < nf * (KPAD / 4); i += 64) {
